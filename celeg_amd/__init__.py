@@ -1,0 +1,6 @@
+"""celeg_amd: a single-GPU inference engine for MI355X (gfx950), built from parts."""
+from . import parts  # registers the built-in parts  # noqa: F401
+from .config import (Lfm2Config, ModelSpec, PartSpec, LayerSpec, RunStep, register_architecture,
+                     registered_architectures, spec_from_config)
+
+__version__ = "0.1.0"

@@ -1,0 +1,292 @@
+"""The kernels as Python calls: shapes are checked on the host, then the extern "C"
+entry points of the built libraries are called through ``ctypes`` with raw device
+pointers and the current HIP stream (so a stream that is capturing a graph captures
+them too).  There is no fallback: if a library cannot be built or loaded, or a tensor
+is not on the GPU, the call fails loudly.
+
+Matrix products in bfloat16 go to the library behind ``torch.mm`` (hipBLASLt /
+rocBLAS), as the reference sends its products to cuBLAS
+(src/backend/cuda/runtime/gemm_dispatcher.cpp); products in 32-bit go to our own
+kernel, which uses no reduced-precision matrix mode.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from . import build
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+_c_int, _c_float, _c_void_p, _c_size_t = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return _c_void_p(0 if t is None else t.data_ptr())
+
+
+class HipOps:
+    def __init__(self, device="cuda:0"):
+        if not torch.cuda.is_available():
+            raise KernelError("celeg_amd needs a GPU: torch.cuda.is_available() is False and "
+                              "there is no CPU path")
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise KernelError(f"celeg_amd runs on a GPU only, not on '{device}'")
+        self._libs: Dict[str, ctypes.CDLL] = {}
+        self.loaded_libraries: Dict[str, str] = {}
+
+    # ------------------------------------------------------------------ plumbing
+    def _lib(self, module: str) -> ctypes.CDLL:
+        lib = self._libs.get(module)
+        if lib is None:
+            path = build.ensure_built(module)
+            try:
+                lib = ctypes.CDLL(path)
+            except OSError as err:
+                raise KernelError(f"cannot load the built kernels {path}: {err}") from err
+            self._libs[module] = lib
+            self.loaded_libraries[module] = path
+        return lib
+
+    def _stream(self):
+        return _c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _check(self, code: int, what: str) -> None:
+        if code != 0:
+            raise KernelError(f"{what}: HIP error {code}")
+
+    def _dev(self, t: torch.Tensor, name: str, dtype=None, contiguous=True):
+        if not isinstance(t, torch.Tensor) or t.device.type != "cuda":
+            raise KernelError(f"{name} must be a GPU tensor")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+        if contiguous and not t.is_contiguous():
+            raise KernelError(f"{name} must be contiguous")
+        return t
+
+    @staticmethod
+    def _rows(t: torch.Tensor, name: str) -> int:
+        """Row stride of a 2-D tensor whose rows are dense."""
+        if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+            raise KernelError(f"{name} must be 2-D with dense rows")
+        return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+    def _dtype(self, t: torch.Tensor, name: str) -> int:
+        if t.dtype not in _DT:
+            raise KernelError(f"{name}: dtype {t.dtype} is not supported (float32, bfloat16)")
+        return _DT[t.dtype]
+
+    # ------------------------------------------------------------------ row-wise
+    def embed(self, table, token_ids, out):
+        self._dev(table, "table"); self._dev(token_ids, "token_ids", torch.int32)
+        self._dev(out, "out", torch.float32)
+        rows, width = out.shape
+        if table.dim() != 2 or table.shape[1] != width or token_ids.numel() != rows:
+            raise KernelError("embed: shapes do not fit")
+        code = self._lib("elementwise").celeg_embed(
+            _ptr(table), _c_int(self._dtype(table, "table")), _ptr(token_ids), _ptr(out),
+            _c_int(rows), _c_int(width), _c_int(table.shape[0]), self._stream())
+        self._check(code, "embed")
+
+    def rmsnorm(self, x, weight, eps, out, delta=None, rows=None):
+        self._dev(x, "x"); self._dev(weight, "weight", torch.float32); self._dev(out, "out")
+        width = x.shape[-1]
+        n_rows = out.shape[0]
+        if x.dim() != 2 or out.dim() != 2 or out.shape[1] != width or weight.numel() != width:
+            raise KernelError("rmsnorm: shapes do not fit")
+        if delta is not None:
+            self._dev(delta, "delta")
+            if delta.shape != x.shape:
+                raise KernelError("rmsnorm: delta must have the shape of x")
+        if rows is not None:
+            self._dev(rows, "rows", torch.int32)
+            if rows.numel() != n_rows:
+                raise KernelError("rmsnorm: one output row per listed row is needed")
+        elif n_rows != x.shape[0]:
+            raise KernelError("rmsnorm: out must have the rows of x")
+        write_back = 1 if (delta is not None and rows is None) else 0
+        if write_back and x.dtype != torch.float32:
+            raise KernelError("rmsnorm: the sum can only be written back to a 32-bit x")
+        code = self._lib("elementwise").celeg_rmsnorm(
+            _ptr(x), _c_int(self._dtype(x, "x")), _ptr(delta),
+            _c_int(self._dtype(delta, "delta") if delta is not None else 0), _ptr(weight),
+            _ptr(out), _c_int(self._dtype(out, "out")), _ptr(rows), _c_int(n_rows),
+            _c_int(width), _c_float(eps), _c_int(write_back), self._stream())
+        self._check(code, "rmsnorm")
+
+    def swiglu(self, gate_up, out):
+        self._dev(gate_up, "gate_up"); self._dev(out, "out", gate_up.dtype)
+        rows, ff = out.shape
+        if gate_up.shape != (rows, 2 * ff):
+            raise KernelError("swiglu: gate_up must be [rows, 2*ff]")
+        code = self._lib("elementwise").celeg_swiglu(
+            _ptr(gate_up), _ptr(out), _c_int(self._dtype(out, "out")), _c_int(rows), _c_int(ff),
+            self._stream())
+        self._check(code, "swiglu")
+
+    def add_bias(self, x, bias):
+        self._dev(x, "x"); self._dev(bias, "bias", torch.float32)
+        rows, width = x.shape
+        if bias.numel() != width:
+            raise KernelError("add_bias: bias must have the width of x")
+        code = self._lib("elementwise").celeg_add_bias(
+            _ptr(x), _c_int(self._dtype(x, "x")), _ptr(bias), _c_int(rows), _c_int(width),
+            self._stream())
+        self._check(code, "add_bias")
+
+    def cast(self, src, dst):
+        self._dev(src, "src"); self._dev(dst, "dst")
+        if src.numel() != dst.numel():
+            raise KernelError("cast: sizes differ")
+        code = self._lib("elementwise").celeg_cast(
+            _ptr(src), _c_int(self._dtype(src, "src")), _ptr(dst),
+            _c_int(self._dtype(dst, "dst")), _c_size_t(src.numel()), self._stream())
+        self._check(code, "cast")
+
+    def apply_table_updates(self, table, updates, capacity):
+        self._dev(table, "table", torch.int32); self._dev(updates, "updates", torch.int32)
+        if updates.numel() < 1 + 3 * capacity:
+            raise KernelError("apply_table_updates: the update list is shorter than its capacity")
+        code = self._lib("elementwise").celeg_table_update(
+            _ptr(table), _c_int(table.shape[1]), _c_int(table.shape[0]), _ptr(updates),
+            _c_int(capacity), self._stream())
+        self._check(code, "apply_table_updates")
+
+    # ------------------------------------------------------------------ matrix products
+    def linear(self, x, w, out, bias=None):
+        """out = x w^T (+ bias).  x [M,K] (rows may be strided), w [N,K], out [M,N] in the
+        dtype of x or in 32-bit."""
+        self._dev(x, "x", contiguous=False); self._dev(w, "w"); self._dev(out, "out")
+        M, K = x.shape
+        N = w.shape[0]
+        if w.shape[1] != K or out.shape != (M, N):
+            raise KernelError(f"linear: shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, "
+                              f"out {tuple(out.shape)}")
+        if bias is not None:
+            self._dev(bias, "bias", torch.float32)
+            if bias.numel() != N:
+                raise KernelError("linear: bias must have one entry per output column")
+        if x.dtype == torch.float32 and w.dtype == torch.float32:
+            if out.dtype != torch.float32:
+                raise KernelError("linear: a 32-bit product needs a 32-bit output")
+            code = self._lib("gemm_f32").celeg_gemm_f32(
+                _ptr(x), _c_int(self._rows(x, "x")), _ptr(w), _c_int(K), _ptr(bias), _ptr(out),
+                _c_int(N), _c_int(M), _c_int(N), _c_int(K), self._stream())
+            self._check(code, "linear (32-bit)")
+            return out
+        if x.dtype == torch.bfloat16 and w.dtype == torch.float32:
+            # a matrix stored in 32-bit stays 32-bit: widen the rows and use the 32-bit product
+            xf = torch.empty((M, K), dtype=torch.float32, device=x.device)
+            self.cast(x.contiguous(), xf)
+            yf = out if out.dtype == torch.float32 else torch.empty((M, N), dtype=torch.float32,
+                                                                    device=x.device)
+            self.linear(xf, w, yf, bias)
+            if yf is not out:
+                self.cast(yf, out)
+            return out
+        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+            raise KernelError(f"linear: unsupported dtypes {x.dtype} x {w.dtype}")
+        if out.dtype == torch.bfloat16:
+            torch.mm(x, w.t(), out=out)
+            if bias is not None:
+                self.add_bias(out, bias)
+        elif out.dtype == torch.float32:
+            tmp = torch.mm(x, w.t())
+            self.cast(tmp, out)
+            if bias is not None:
+                self.add_bias(out, bias)
+        else:
+            raise KernelError("linear: out must be bfloat16 or float32")
+        return out
+
+    # ------------------------------------------------------------------ short convolution
+    def short_conv(self, bcx, weight, bias, state, out, batch):
+        self._dev(bcx, "bcx"); self._dev(weight, "weight", torch.float32)
+        self._dev(state, "state", torch.float32, contiguous=False); self._dev(out, "out", bcx.dtype)
+        T, width = out.shape
+        taps = weight.shape[1]
+        if bcx.shape != (T, 3 * width) or weight.shape[0] != width or T != batch.n_tokens:
+            raise KernelError("short_conv: shapes do not fit")
+        if state.dim() != 3 or state.shape[1:] != (taps, width) or state.stride(2) != 1 \
+                or state.stride(1) != width:
+            raise KernelError("short_conv: state must be [slots, taps, width] with dense slots")
+        if bias is not None:
+            self._dev(bias, "bias", torch.float32)
+        code = self._lib("short_conv").celeg_short_conv(
+            _ptr(bcx), _c_int(3 * width), _c_int(self._dtype(bcx, "bcx")), _ptr(weight), _ptr(bias),
+            _ptr(state), _c_size_t(state.stride(0)), _ptr(out), _ptr(batch.positions),
+            _ptr(batch.token_seq), _ptr(batch.seq_start), _ptr(batch.seq_slot),
+            _ptr(batch.cu_seqlens), _c_int(batch.n_tokens), _c_int(batch.n_seqs), _c_int(width),
+            _c_int(taps), self._stream())
+        self._check(code, "short_conv")
+
+    # ------------------------------------------------------------------ attention
+    def _check_kv(self, kv, kv_heads, head_dim, dtype):
+        if kv.kv_heads != kv_heads or kv.head_dim != head_dim:
+            raise KernelError("attention: the cache has other head sizes than the mixer")
+        for name, pool in (("k", kv.k), ("v", kv.v)):
+            self._dev(pool, f"{name} cache", dtype)
+            if pool.shape[1:] != (kv.n_layers, kv_heads, kv.page_tokens, head_dim):
+                raise KernelError("attention: unexpected cache shape")
+        self._dev(kv.table, "block table", torch.int32)
+        if not 0 <= kv.layer < kv.n_layers:
+            raise KernelError("attention: layer index outside the cache")
+
+    def qk_norm_rope_store(self, q, k, v, q_weight, k_weight, eps, inv_freq, rotary_dim,
+                           heads, kv_heads, head_dim, batch, kv):
+        self._dev(q, "q", contiguous=False)
+        T = q.shape[0]
+        dtype = q.dtype
+        if T != batch.n_tokens or q.shape[1] != heads * head_dim:
+            raise KernelError("qk_norm_rope_store: q must be [rows, heads*head_dim]")
+        if head_dim % 2 or head_dim > 1024:
+            raise KernelError(f"qk_norm_rope_store: head_dim {head_dim} must be even and <= 1024")
+        self._check_kv(kv, kv_heads, head_dim, dtype)
+        store = k is not None
+        if store:
+            self._dev(k, "k", dtype, contiguous=False); self._dev(v, "v", dtype, contiguous=False)
+            if k.shape != (T, kv_heads * head_dim) or v.shape != k.shape:
+                raise KernelError("qk_norm_rope_store: k and v must be [rows, kv_heads*head_dim]")
+        for name, wt in (("q_weight", q_weight), ("k_weight", k_weight)):
+            if wt is not None:
+                self._dev(wt, name, torch.float32)
+                if wt.numel() != head_dim:
+                    raise KernelError(f"qk_norm_rope_store: {name} must have head_dim entries")
+        if inv_freq is not None:
+            self._dev(inv_freq, "inv_freq", torch.float32)
+            if rotary_dim % 2 or rotary_dim > head_dim or inv_freq.numel() != rotary_dim // 2:
+                raise KernelError("qk_norm_rope_store: rotary_dim and the frequency table disagree")
+        code = self._lib("attention").celeg_qk_norm_rope_store(
+            _ptr(q), _c_int(self._rows(q, "q")), _ptr(k), _c_int(self._rows(k, "k") if store else 0),
+            _ptr(v), _c_int(self._rows(v, "v") if store else 0), _c_int(self._dtype(q, "q")),
+            _ptr(q_weight), _ptr(k_weight if store else None), _c_float(eps), _ptr(inv_freq),
+            _c_int(rotary_dim), _ptr(batch.positions), _ptr(batch.token_slot), _ptr(kv.table),
+            _c_int(kv.table.shape[1]), _ptr(kv.k), _ptr(kv.v), _c_int(kv.n_layers),
+            _c_int(kv.layer), _c_int(kv.page_tokens), _c_int(T), _c_int(heads), _c_int(kv_heads),
+            _c_int(head_dim), _c_int(1 if store else 0), self._stream())
+        self._check(code, "qk_norm_rope_store")
+
+    def paged_attention(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv):
+        self._dev(q, "q", contiguous=False); self._dev(out, "out", q.dtype)
+        T = q.shape[0]
+        if T != batch.n_tokens or q.shape[1] != heads * head_dim or out.shape != (T, heads * head_dim):
+            raise KernelError("paged_attention: q and out must be [rows, heads*head_dim]")
+        if head_dim > 256:
+            raise KernelError(f"paged_attention: head_dim {head_dim} exceeds 256")
+        if heads % kv_heads:
+            raise KernelError("paged_attention: heads must be a multiple of kv_heads")
+        self._check_kv(kv, kv_heads, head_dim, q.dtype)
+        code = self._lib("attention").celeg_paged_attention(
+            _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v),
+            _c_int(self._dtype(q, "q")), _ptr(kv.table), _c_int(kv.table.shape[1]),
+            _ptr(batch.token_slot), _ptr(batch.positions), _ptr(out), _c_int(heads * head_dim),
+            _c_int(T), _c_int(heads), _c_int(kv_heads), _c_int(head_dim), _c_int(kv.page_tokens),
+            _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
+            _c_int(window if window else 0), self._stream())
+        self._check(code, "paged_attention")

@@ -1,0 +1,177 @@
+"""One step's batch: the rows, and the per-row and per-request numbers kernels need.
+
+A step takes a list of entries, one per request: the request's next tokens (a
+portion of its prompt, or one decoded token) and the places among them whose
+logits are wanted.  The tokens of all entries are laid side by side into T rows.
+The reference builds the same arrays for its packed passes, separately for a
+prefill pass and a decode pass (src/backend/cuda/packed/batch_planner.cu:38-87);
+here one batch holds both kinds.
+
+All integer metadata travels to the device in ONE copy of one packed buffer.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    slot: int                 # the request's slot in the cache manager
+    start_pos: int            # position of tokens[0] in the request's sequence
+    tokens: Sequence[int]
+    want: Sequence[int] = ()  # indices into ``tokens`` whose logits are wanted
+
+
+class StepBatch:
+    """Device views (int32) into the packed buffer, plus host-side facts.
+
+    token_ids[T], positions[T], token_seq[T] (which entry a row belongs to),
+    token_slot[T] (that entry's cache slot), cu_seqlens[S+1] (row offsets of the
+    entries), seq_slot[S], seq_start[S] (position of the entry's first row),
+    logit_rows[R] (rows whose logits are wanted), table_updates[g] ([1 + 3*cap]:
+    a count, then (slot, logical page, physical page) triples) per cache group.
+    """
+
+    def __init__(self):
+        self.n_tokens = 0
+        self.n_seqs = 0
+        self.n_logit_rows = 0
+        self.max_seg_len = 0
+        self.max_context_len = 0
+        self.decode_only = False
+        self.token_ids = self.positions = self.token_seq = self.token_slot = None
+        self.cu_seqlens = self.seq_slot = self.seq_start = self.logit_rows = None
+        self.table_updates: List[Optional[torch.Tensor]] = []
+        self.table_update_caps: List[int] = []
+        # host copies, for parts that plan on the host
+        self.host: Dict[str, np.ndarray] = {}
+
+
+def packed_layout(T: int, S: int, R: int, update_caps: Sequence[int]) -> Tuple[Dict[str, Tuple[int, int]], int]:
+    """Offsets (in int32 elements) of every array in the packed buffer; each array
+    starts at a multiple of 4 elements.  The layout depends only on the counts, so a
+    captured graph of a fixed (T, S, R, caps) always finds its arrays in place."""
+    fields = [("token_ids", T), ("positions", T), ("token_seq", T), ("token_slot", T),
+              ("cu_seqlens", S + 1), ("seq_slot", S), ("seq_start", S), ("logit_rows", R)]
+    for g, cap in enumerate(update_caps):
+        fields.append((f"updates{g}", 1 + 3 * cap))
+    layout = {}
+    offset = 0
+    for name, count in fields:
+        layout[name] = (offset, count)
+        offset += (count + 3) // 4 * 4
+    return layout, offset
+
+
+class BatchBuilder:
+    """Packs entries on the host and ships them with one copy.  Two pinned staging
+    buffers alternate, each guarded by an event, so a step's arrays are never
+    overwritten while their copy is still in flight."""
+
+    def __init__(self, device, capacity_ints: int, n_groups: int, pin: bool):
+        self.device = torch.device(device)
+        self.capacity = capacity_ints
+        self.n_groups = n_groups
+        self._stage = [torch.empty(capacity_ints, dtype=torch.int32, pin_memory=pin)
+                       for _ in range(2)]
+        self._events = [None, None]
+        self._turn = 0
+        self.device_buffer = torch.zeros(capacity_ints, dtype=torch.int32, device=self.device)
+
+    def build(self, entries: Sequence[StepEntry], updates: Sequence[Sequence[Tuple[int, int, int]]],
+              pad_to: Optional[int] = None, null_slot: int = 0,
+              update_caps: Optional[Sequence[int]] = None) -> StepBatch:
+        """``pad_to``: for decode-only batches, the fixed number of rows of a captured
+        graph; missing rows are filled with the null slot at position 0."""
+        seg_lens = [len(e.tokens) for e in entries]
+        S_real = len(entries)
+        T_real = int(sum(seg_lens))
+        S = S_real if pad_to is None else pad_to
+        T = T_real if pad_to is None else pad_to
+        want_rows: List[int] = []
+        row = 0
+        for e, n in zip(entries, seg_lens):
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise ValueError(f"wanted place {w} is outside the entry's {n} tokens")
+                want_rows.append(row + int(w))
+            row += n
+        R = len(want_rows)
+        if update_caps is None:
+            update_caps = [len(u) for u in updates]
+        for u, cap in zip(updates, update_caps):
+            if len(u) > cap:
+                raise ValueError("more block-table updates than the step has room for")
+        layout, total = packed_layout(T, S, R, update_caps)
+        if total > self.capacity:
+            raise ValueError(f"step metadata ({total} ints) exceeds the staging buffer "
+                             f"({self.capacity} ints)")
+        turn = self._turn
+        self._turn ^= 1
+        if self._events[turn] is not None:
+            self._events[turn].synchronize()
+        stage = self._stage[turn].numpy()
+
+        def arr(name):
+            off, count = layout[name]
+            return stage[off:off + count]
+
+        token_ids, positions = arr("token_ids"), arr("positions")
+        token_seq, token_slot = arr("token_seq"), arr("token_slot")
+        cu, seq_slot, seq_start = arr("cu_seqlens"), arr("seq_slot"), arr("seq_start")
+        row = 0
+        cu[0] = 0
+        for i, (e, n) in enumerate(zip(entries, seg_lens)):
+            token_ids[row:row + n] = np.asarray(e.tokens, dtype=np.int32)
+            positions[row:row + n] = np.arange(e.start_pos, e.start_pos + n, dtype=np.int32)
+            token_seq[row:row + n] = i
+            token_slot[row:row + n] = e.slot
+            seq_slot[i] = e.slot
+            seq_start[i] = e.start_pos
+            row += n
+            cu[i + 1] = row
+        for i in range(S_real, S):          # padding rows of a fixed-size decode batch
+            token_ids[row] = 0
+            positions[row] = 0
+            token_seq[row] = i
+            token_slot[row] = null_slot
+            seq_slot[i] = null_slot
+            seq_start[i] = 0
+            row += 1
+            cu[i + 1] = row
+        arr("logit_rows")[:] = np.asarray(want_rows, dtype=np.int32)
+        for g, u in enumerate(updates):
+            a = arr(f"updates{g}")
+            a[0] = len(u)
+            if u:
+                a[1:1 + 3 * len(u)] = np.asarray(u, dtype=np.int32).reshape(-1)
+        self.device_buffer[:total].copy_(self._stage[turn][:total], non_blocking=True)
+        if self.device.type == "cuda":
+            ev = torch.cuda.Event()
+            ev.record()
+            self._events[turn] = ev
+
+        b = StepBatch()
+        b.n_tokens, b.n_seqs, b.n_logit_rows = T, S, R
+        b.max_seg_len = max(seg_lens) if seg_lens else 0
+        b.max_context_len = max((e.start_pos + n for e, n in zip(entries, seg_lens)), default=0)
+        b.decode_only = all(n == 1 for n in seg_lens)
+
+        def dev(name):
+            off, count = layout[name]
+            return self.device_buffer[off:off + count]
+
+        b.token_ids, b.positions = dev("token_ids"), dev("positions")
+        b.token_seq, b.token_slot = dev("token_seq"), dev("token_slot")
+        b.cu_seqlens, b.seq_slot, b.seq_start = dev("cu_seqlens"), dev("seq_slot"), dev("seq_start")
+        b.logit_rows = dev("logit_rows")
+        b.table_updates = [dev(f"updates{g}") for g in range(len(updates))]
+        b.table_update_caps = list(update_caps)
+        b.host = {"seg_lens": np.asarray(seg_lens + [1] * (S - S_real), dtype=np.int32),
+                  "seq_slot": seq_slot.copy(), "seq_start": seq_start.copy(),
+                  "cu_seqlens": cu.copy(), "want_rows": np.asarray(want_rows, dtype=np.int32)}
+        return b

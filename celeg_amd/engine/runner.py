@@ -1,0 +1,116 @@
+"""The step function: runs one batch of (request, its next tokens) through the model,
+from the cache, and returns the logits at the wanted places.
+
+The reference runs prompt portions and decode tokens in separate passes
+(src/backend/cuda/runtime/engine_control.cpp:4-23;
+src/backend/cuda/packed/execution.cu:141-224 and 234-384); here one function takes
+both in one batch.  Positions are the caller's to keep: ``start_pos`` is an input,
+so the scheduler and the trace replay drive the same function.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..parts.base import Runtime
+from .batch import BatchBuilder, StepBatch, StepEntry, packed_layout
+from .model import Model
+
+
+class Workspace:
+    """Reusable buffers by name, sized for the largest use so far.  ``generation``
+    changes whenever a buffer moves, which invalidates captured graphs."""
+
+    def __init__(self, device):
+        self.device = device
+        self._flat: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self.generation = 0
+        self.frozen = False
+
+    def buf(self, name: str, shape, dtype) -> torch.Tensor:
+        count = 1
+        for s in shape:
+            count *= int(s)
+        key = (name, dtype)
+        flat = self._flat.get(key)
+        if flat is None or flat.numel() < count:
+            if self.frozen:
+                raise RuntimeError(f"workspace buffer '{name}' would move while a graph is "
+                                   "being captured")
+            flat = torch.empty(max(count, 1), dtype=dtype, device=self.device)
+            self._flat[key] = flat
+            self.generation += 1
+        return flat[:count].view(tuple(int(s) for s in shape))
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self._flat.values())
+
+
+class ModelRunner:
+    def __init__(self, model: Model, cache: CacheManager, rt: Runtime, *,
+                 max_batched_tokens: int):
+        self.model = model
+        self.cache = cache
+        self.rt = rt
+        self.max_batched_tokens = max_batched_tokens
+        model.bind_cache(cache)
+        n_groups = len(cache.groups)
+        S = cache.max_requests
+        # room for the largest step, with as many table updates as rows plus requests
+        _, ints = packed_layout(max_batched_tokens, S, max_batched_tokens,
+                                [max_batched_tokens // cache.page_tokens + 2 * S + 8] * n_groups)
+        self.builder = BatchBuilder(rt.device, ints, n_groups,
+                                    pin=torch.device(rt.device).type == "cuda")
+        self.steps_run = 0
+
+    # ------------------------------------------------------------------ checks
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise ValueError("step: no entries")
+        if len(entries) > self.cache.max_requests:
+            raise ValueError(f"step: {len(entries)} requests exceed max_requests "
+                             f"{self.cache.max_requests}")
+        seen = set()
+        total = 0
+        vocab = self.model.spec.vocab_size
+        for e in entries:
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError("step: an entry has no tokens")
+            if e.slot in seen:
+                raise ValueError(f"step: slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            if e.start_pos < 0 or e.start_pos + n > self.cache.max_context:
+                raise ValueError(f"context limit reached: position {e.start_pos + n} exceeds "
+                                 f"{self.cache.max_context}")
+            toks = np.asarray(e.tokens)
+            if toks.min() < 0 or toks.max() >= vocab:
+                raise ValueError(f"step: token id out of range [0, {vocab})")
+            if not self.cache.covers(e.slot, e.start_pos, n):
+                raise ValueError(f"step: the pages of slot {e.slot} do not cover positions "
+                                 f"[{e.start_pos}, {e.start_pos + n})")
+            total += n
+        if total > self.max_batched_tokens:
+            raise ValueError(f"step: {total} tokens exceed max_batched_tokens "
+                             f"{self.max_batched_tokens}")
+
+    # ------------------------------------------------------------------ the step
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Logits, 32-bit [number of wanted places, vocab], in the order of the entries
+        and of each entry's ``want``.  The tensor is a view of a reused buffer: it holds
+        until the next step."""
+        self._validate(entries)
+        updates = self.cache.drain_table_updates()
+        batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
+        self._apply_table_updates(batch)
+        logits = self.model.forward(batch, self.rt)
+        self.steps_run += 1
+        return logits
+
+    def _apply_table_updates(self, batch: StepBatch) -> None:
+        for g, (upd, cap) in enumerate(zip(batch.table_updates, batch.table_update_caps)):
+            if cap > 0:
+                self.rt.ops.apply_table_updates(self.cache.groups[g].table, upd, cap)
