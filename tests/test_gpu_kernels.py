@@ -1,0 +1,291 @@
+"""Each HIP kernel alone against a plain torch / plain-implementation reference, at sizes
+other than the engine's tiny configurations (widths and vocabularies that are no power
+of two, head sizes in steps of 16, odd head counts and groups)."""
+import math
+
+import pytest
+import torch
+
+import plain_lfm2 as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from celeg_amd.csrc.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+def randn(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1.6e-2)
+
+
+# ---------------------------------------------------------------- row-wise kernels
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("vocab,width,rows", [(331, 96, 7), (1000, 1030, 33)])
+def test_embed(ops, dtype, vocab, width, rows):
+    table = randn(vocab, width, seed=1, dtype=dtype)
+    ids = torch.randint(0, vocab, (rows,), generator=torch.Generator().manual_seed(2),
+                        dtype=torch.int32).to(DEV)
+    out = torch.empty(rows, width, device=DEV)
+    ops.embed(table, ids, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(5, 96), (3, 1000), (9, 4100)])
+def test_rmsnorm_with_delta_and_rows(ops, dtype, rows, width):
+    x = randn(rows, width, seed=3)
+    delta = randn(rows, width, seed=4, dtype=dtype)
+    w = 1 + randn(width, seed=5, scale=0.1)
+    eps = 3e-5
+    ref_sum = x.double() + delta.double()
+    ref = plain.rmsnorm(ref_sum.cpu(), w.cpu(), eps)
+    # all rows, sum written back
+    x1 = x.clone()
+    out = torch.empty(rows, width, dtype=dtype, device=DEV)
+    ops.rmsnorm(x1, w, eps, out, delta=delta)
+    torch.testing.assert_close(x1.double().cpu(), ref_sum.cpu(), rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(out.double().cpu(), ref, **tol(dtype))
+    # listed rows only, x untouched
+    x2 = x.clone()
+    idx = torch.tensor([rows - 1, 0, rows // 2], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(3, width, dtype=dtype, device=DEV)
+    ops.rmsnorm(x2, w, eps, out2, delta=delta, rows=idx)
+    assert torch.equal(x2, x)
+    torch.testing.assert_close(out2.double().cpu(), ref[idx.long().cpu()], **tol(dtype))
+    # no delta
+    out3 = torch.empty(rows, width, dtype=dtype, device=DEV)
+    ops.rmsnorm(x2, w, eps, out3)
+    torch.testing.assert_close(out3.double().cpu(), plain.rmsnorm(x.cpu(), w.cpu(), eps), **tol(dtype))
+
+
+def test_rmsnorm_reference_vector(ops):
+    # tests/reference_test.cpp:29-31: {1,2,3,4}, w = 1, eps 1e-5 -> y0 = 1/sqrt(7.5 + 1e-5)
+    x = torch.tensor([[1., 2., 3., 4.]], device=DEV)
+    out = torch.empty_like(x)
+    ops.rmsnorm(x, torch.ones(4, device=DEV), 1e-5, out)
+    assert abs(float(out[0, 0]) - 1 / math.sqrt(7.5 + 1e-5)) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(ops, dtype):
+    rows, ff = 11, 352
+    gu = randn(rows, 2 * ff, seed=6, scale=2.0, dtype=dtype)
+    out = torch.empty(rows, ff, dtype=dtype, device=DEV)
+    ops.swiglu(gu, out)
+    g, u = gu[:, :ff].double().cpu(), gu[:, ff:].double().cpu()
+    torch.testing.assert_close(out.double().cpu(), plain.silu(g) * u, **tol(dtype))
+    zero = torch.zeros(2, 2 * ff, dtype=dtype, device=DEV)
+    zero[:, ff:] = 3.0
+    out0 = torch.empty(2, ff, dtype=dtype, device=DEV)
+    ops.swiglu(zero, out0)   # gate 0 -> 0
+    assert float(out0.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 331, 96), (67, 130, 77), (200, 65, 1030), (5, 1000, 64)])
+def test_gemm_f32_is_true_32bit_and_row_independent(ops, M, N, K):
+    x, w, b = randn(M, K, seed=7), randn(N, K, seed=8), randn(N, seed=9)
+    out = torch.empty(M, N, device=DEV)
+    ops.linear(x, w, out, bias=b)
+    ref = x.double().cpu() @ w.double().cpu().T + b.double().cpu()
+    torch.testing.assert_close(out.double().cpu(), ref, rtol=1e-5, atol=1e-5 * math.sqrt(K))
+    # a row gives the same bits alone as inside the batch
+    one = torch.empty(1, N, device=DEV)
+    ops.linear(x[M // 2:M // 2 + 1], w, one, bias=b)
+    assert torch.equal(one[0], out[M // 2])
+
+
+def test_linear_bf16_and_stored_f32_matrix(ops):
+    M, N, K = 9, 200, 96
+    x = randn(M, K, seed=10, dtype=torch.bfloat16)
+    w = randn(N, K, seed=11, scale=0.1, dtype=torch.bfloat16)
+    ref = x.double().cpu() @ w.double().cpu().T
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, w, out)
+    torch.testing.assert_close(out.double().cpu(), ref, rtol=1.6e-2, atol=1.6e-2)
+    out32 = torch.empty(M, N, device=DEV)
+    ops.linear(x, w.float(), out32)     # matrix kept in 32-bit
+    torch.testing.assert_close(out32.double().cpu(), ref, rtol=1e-5, atol=1e-5)
+
+
+# ---------------------------------------------------------------- cache-backed kernels
+def make_cache(kv_heads, head_dim, n_layers, dtype, n_pages=64, page_tokens=16, slots=4,
+               states=(), max_context=512):
+    from celeg_amd.cache import CacheLayout, CacheManager
+    from celeg_amd.parts.base import KVNeed
+    layout = CacheLayout()
+    if kv_heads:
+        layout.kv_groups = [KVNeed(kv_heads, head_dim)]
+        layout.group_layers = [n_layers]
+        layout.kv_of_step = {i: (0, i, True) for i in range(n_layers)}
+    layout.states = list(states)
+    return CacheManager(layout, page_tokens=page_tokens, n_pages=n_pages, max_requests=slots,
+                        max_context=max_context, device=DEV, dtype=dtype)
+
+
+def build_batch(ops, cache, entries):
+    from celeg_amd.engine.batch import BatchBuilder
+    builder = BatchBuilder(DEV, 1 << 16, len(cache.groups), pin=True)
+    batch = builder.build(entries, cache.drain_table_updates(), null_slot=cache.null_slot)
+    for g, (upd, cap) in enumerate(zip(batch.table_updates, batch.table_update_caps)):
+        if cap:
+            ops.apply_table_updates(cache.groups[g].table, upd, cap)
+    return batch, builder
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,taps,bias", [(2, 3, False), (96, 5, True), (1030, 4, False), (64, 1, True)])
+def test_short_conv_whole_chunked_and_token_by_token(ops, dtype, width, taps, bias):
+    from celeg_amd.engine import StepEntry
+    from celeg_amd.parts.base import StateNeed
+    T = 23
+    bcx = randn(T, 3 * width, seed=12, dtype=dtype)
+    w = randn(width, taps, seed=13)
+    b = randn(width, seed=14) if bias else None
+    ref = plain.short_conv(bcx.cpu(), w.cpu(), b.cpu() if bias else None)
+    for cuts in ([T], [1] * T, [7, 2, 1, 9, 4]):
+        cache = make_cache(0, 0, 0, dtype, states=[(0, StateNeed("bx", (taps, width)))])
+        slot_other = cache.open()     # a neighbour slot whose state must stay zero
+        slot = cache.open()
+        state = cache.layer_cache(0).states["bx"]
+        outs, pos = [], 0
+        for n in cuts:
+            batch, keep = build_batch(ops, cache, [StepEntry(slot, pos, [0] * n)])
+            out = torch.empty(n, width, dtype=dtype, device=DEV)
+            ops.short_conv(bcx[pos:pos + n].contiguous(), w, b, state, out, batch)
+            torch.cuda.synchronize()
+            outs.append(out)
+            pos += n
+        got = torch.cat(outs).double().cpu()
+        torch.testing.assert_close(got, ref, **tol(dtype))
+        assert float(state[slot_other].abs().max()) == 0.0
+        bx = (bcx[:, :width].float() * bcx[:, 2 * width:].float())
+        want_state = torch.zeros(taps, width, device=DEV)
+        want_state[max(0, taps - T):] = bx[max(0, T - taps):]
+        torch.testing.assert_close(state[slot], want_state, rtol=0, atol=0)
+
+
+def test_short_conv_reference_vector(ops):
+    # tests/reference_test.cpp:68-73: hidden 2, L 3, bcx {1,1 | 1,1 | 2,4}, weights
+    # {1,2,3 ; 1,2,3} channel-major, position 0, zero state -> {6, 12}
+    from celeg_amd.engine import StepEntry
+    from celeg_amd.parts.base import StateNeed
+    cache = make_cache(0, 0, 0, torch.float32, states=[(0, StateNeed("bx", (3, 2)))])
+    slot = cache.open()
+    batch, keep = build_batch(ops, cache, [StepEntry(slot, 0, [0])])
+    bcx = torch.tensor([[1., 1., 1., 1., 2., 4.]], device=DEV)
+    w = torch.tensor([[1., 2., 3.], [1., 2., 3.]], device=DEV)
+    out = torch.empty(1, 2, device=DEV)
+    ops.short_conv(bcx, w, None, cache.layer_cache(0).states["bx"], out, batch)
+    assert out.cpu().tolist() == [[6.0, 12.0]]
+
+
+def attention_case(ops, dtype, heads, kv_heads, head_dim, lengths, cuts, window=None,
+                   qk_norm=True, theta=10000.0, rotary_dim=None, boost=None, page_tokens=16):
+    """Runs norm+rope+store and attention for several requests cut into steps (one step
+    holds the next cut of every request) and compares with the plain whole-sequence
+    functions."""
+    from celeg_amd.engine import StepEntry
+    rotary_dim = head_dim if rotary_dim is None else rotary_dim
+    n_layers, layer = 3, 1
+    total = sum(lengths)
+    cache = make_cache(kv_heads, head_dim, n_layers, dtype, page_tokens=page_tokens,
+                       n_pages=(total + page_tokens * len(lengths)) // page_tokens + 2,
+                       max_context=max(lengths) + 16)
+    kv = cache.layer_cache(layer).kv
+    qw = 1 + randn(head_dim, seed=20, scale=0.1) if qk_norm else None
+    kw = 1 + randn(head_dim, seed=21, scale=0.1) if qk_norm else None
+    inv_freq = torch.tensor(plain.rope_inverse_frequencies(theta, rotary_dim),
+                            dtype=torch.float64).float().to(DEV) if rotary_dim else None
+    scale = 1 / math.sqrt(head_dim)
+    reqs = []
+    for i, n in enumerate(lengths):
+        q = randn(n, heads * head_dim, seed=30 + i, dtype=dtype)
+        k = randn(n, kv_heads * head_dim, seed=40 + i, dtype=dtype)
+        v = randn(n, kv_heads * head_dim, seed=50 + i, dtype=dtype)
+        if boost is not None and n > boost[1]:   # one far key stands out for one query
+            far, row = boost
+            k[far] *= 6.0
+            q[row] = (k[far].float().reshape(kv_heads, 1, head_dim) *
+                      torch.ones(1, heads // kv_heads, 1, device=DEV)).reshape(-1).to(dtype) * 2
+        reqs.append((q, k, v, cache.open()))
+    got = [[] for _ in lengths]
+    pos = [0] * len(lengths)
+    step = 0
+    while any(p < n for p, n in zip(pos, lengths)):
+        entries, parts = [], []
+        for i, n in enumerate(lengths):
+            if pos[i] >= n:
+                continue
+            c = min(cuts[(step + i) % len(cuts)], n - pos[i])
+            assert cache.prepare(reqs[i][3], pos[i], c)
+            entries.append(StepEntry(reqs[i][3], pos[i], [0] * c))
+            parts.append((i, pos[i], c))
+            pos[i] += c
+        batch, keep = build_batch(ops, cache, entries)
+        q = torch.cat([reqs[i][0][p:p + c] for i, p, c in parts]).contiguous()
+        k = torch.cat([reqs[i][1][p:p + c] for i, p, c in parts]).contiguous()
+        v = torch.cat([reqs[i][2][p:p + c] for i, p, c in parts]).contiguous()
+        ops.qk_norm_rope_store(q, k, v, qw, kw, 1e-5, inv_freq, rotary_dim, heads, kv_heads,
+                               head_dim, batch, kv)
+        out = torch.empty_like(q)
+        ops.paged_attention(q, out, heads, kv_heads, head_dim, scale, window, batch, kv)
+        torch.cuda.synchronize()
+        row = 0
+        for i, p, c in parts:
+            got[i].append(out[row:row + c].double().cpu())
+            row += c
+        step += 1
+    for i, n in enumerate(lengths):
+        q, k, v, _ = reqs[i]
+        qf = q.double().cpu().reshape(n, heads, head_dim)
+        kf = k.double().cpu().reshape(n, kv_heads, head_dim)
+        vf = v.double().cpu().reshape(n, kv_heads, head_dim)
+        if qk_norm:
+            qf = plain.head_rmsnorm(qf, qw.cpu(), 1e-5)
+            kf = plain.head_rmsnorm(kf, kw.cpu(), 1e-5)
+        if rotary_dim:
+            cos, sin = plain.rope_cos_sin(range(n), theta, rotary_dim)
+            qf, kf = plain.rope_apply(qf, cos, sin), plain.rope_apply(kf, cos, sin)
+        if dtype == torch.bfloat16:   # the kernels store q and k rounded
+            qf, kf = qf.bfloat16().double(), kf.bfloat16().double()
+        ref = plain.causal_attention(qf, kf, vf, window=window).reshape(n, -1)
+        torch.testing.assert_close(torch.cat(got[i]), ref, **tol(dtype),
+                                   msg=lambda m: f"request {i}: {m}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(6, 3, 48), (5, 5, 16), (8, 1, 128), (4, 2, 80)])
+def test_attention_mixed_steps(ops, dtype, heads, kv_heads, head_dim):
+    attention_case(ops, dtype, heads, kv_heads, head_dim, lengths=[70, 33, 150],
+                   cuts=[7, 1, 2, 30, 1, 16, 5])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_far_key_stands_out(ops, dtype):
+    # query 299 is built to look at key 3, hundreds of keys back and in the first page
+    attention_case(ops, dtype, 4, 2, 64, lengths=[300], cuts=[64, 1, 1, 50], boost=(3, 299),
+                   qk_norm=False, rotary_dim=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_window_edge(ops, dtype):
+    # with a window of 20 the boosted key 3 is visible to row 22 and not to row 23
+    attention_case(ops, dtype, 4, 2, 32, lengths=[90], cuts=[5, 1, 13, 2], window=20,
+                   boost=(3, 22), qk_norm=False, rotary_dim=0)
+    attention_case(ops, dtype, 4, 2, 32, lengths=[90], cuts=[5, 1, 13, 2], window=20,
+                   boost=(3, 23), qk_norm=False, rotary_dim=0)
+
+
+def test_attention_partial_rotary_and_other_page_size(ops):
+    attention_case(ops, torch.float32, 4, 4, 64, lengths=[45, 80], cuts=[9, 1, 3],
+                   rotary_dim=32, theta=1e6, page_tokens=32)
