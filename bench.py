@@ -1,0 +1,150 @@
+"""Headline benchmark: decode tokens/s of an LFM2-350M-shaped model (bfloat16, random
+weights, synthetic tokens) at batch 8 on ONE MI355X, with prefill throughput at 2,048
+tokens, decode at batch 1 and 64, and roofline fractions.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one decode step of the whole batch (greedy sampling on the device included).
+Prints ONE JSON line.  Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA
+2.5 PFLOP/s.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+# The layer sizes of the LFM2-350M shape: 16 layers, attention at {2,5,8,10,12,14}.
+LFM2_350M = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "vocab_size": 65536, "hidden_size": 1024, "num_hidden_layers": 16,
+    "layer_types": ["conv", "conv", "full_attention", "conv", "conv", "full_attention", "conv",
+                    "conv", "full_attention", "conv", "full_attention", "conv", "full_attention",
+                    "conv", "full_attention", "conv"],
+    "num_attention_heads": 16, "num_key_value_heads": 8, "head_dim": 64,
+    "intermediate_size": 6656, "block_auto_adjust_ff_dim": True, "block_multiple_of": 256,
+    "block_ffn_dim_multiplier": 1.0, "rope_theta": 1000000.0, "conv_L_cache": 3,
+    "conv_bias": False, "tie_word_embeddings": True, "norm_eps": 1e-5,
+    "max_position_embeddings": 4096, "bos_token_id": 1, "eos_token_id": 7, "pad_token_id": 0,
+}
+PROMPT_TOKENS = 2048
+BATCH = 8
+
+
+def weight_bytes(model) -> int:
+    seen = {}
+    for _, part in model.named_parts():
+        for value in vars(part).values():
+            if hasattr(value, "data_ptr") and hasattr(value, "element_size"):
+                key = value.untyped_storage().data_ptr() if hasattr(value, "untyped_storage") \
+                    else value.data_ptr()
+                size = value.untyped_storage().nbytes() if hasattr(value, "untyped_storage") \
+                    else value.numel() * value.element_size()
+                seen[key] = size
+    return sum(seen.values())
+
+
+def prefill_flops(cfg, tokens: int, ff: int) -> float:
+    H, hq, hkv, hd = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    per_token = 0
+    attention = 0.0
+    for kind in cfg["layer_types"]:
+        if kind == "conv":
+            per_token += 2 * (3 * H * H + H * H)
+        else:
+            per_token += 2 * ((hq + 2 * hkv) * hd * H + hq * hd * H)
+            attention += 4.0 * hq * hd * tokens * (tokens + 1) / 2     # QK^T and PV, causal
+        per_token += 2 * 3 * H * ff
+    return per_token * tokens + attention + 2.0 * H * cfg["vocab_size"]   # head for one row
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported "
+              "(this engine runs on a single MI355X)")
+        return 2
+
+    import torch
+    import celeg_amd  # noqa: F401
+    from celeg_amd.engine import load_model
+    from celeg_amd.engine.benchmark import DecodeBench, measure_prefill
+    from celeg_amd.weights import write_random_model
+
+    cfg = dict(LFM2_350M)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers and args.layers < full_layers:
+        cfg["num_hidden_layers"] = args.layers
+        cfg["layer_types"] = cfg["layer_types"][:args.layers]
+    context = cfg["max_position_embeddings"]
+    max_batch = BATCH if args.no_points else 64
+    need = PROMPT_TOKENS + args.steps + args.warmup + 1
+    if need > context:
+        raise SystemExit(f"--steps + --warmup exceed the context of {context}")
+    with tempfile.TemporaryDirectory(prefix="celeg_bench_") as folder:
+        write_random_model(cfg, folder, seed=0, dtype=torch.bfloat16, std=0.02)
+        pages_per_request = (need + 15) // 16 + 1
+        lm = load_model(folder, dtype="bfloat16", device="cuda:0", page_tokens=16,
+                        n_pages=pages_per_request * max_batch, max_requests=max_batch,
+                        max_context=context, max_batched_tokens=PROMPT_TOKENS)
+    ff = lm.config.ff_dim
+    w_bytes = weight_bytes(lm.model)
+    kv_per_token = lm.cache.layout.kv_bytes_per_token(2)
+
+    prefill = measure_prefill(lm, PROMPT_TOKENS, repeats=7, warmup=3)
+    flops = prefill_flops(cfg, PROMPT_TOKENS, ff)
+
+    def decode(batch: int):
+        bench = DecodeBench(lm, batch, PROMPT_TOKENS, seed=batch, prefill_chunk=PROMPT_TOKENS)
+        result = bench.run(args.steps, args.warmup)
+        bench.close()
+        return result
+
+    main_run = decode(BATCH)
+    points = {}
+    if not args.no_points:
+        points = {"decode_b1": round(decode(1)["tokens_per_second"], 1),
+                  "decode_b64": round(decode(64)["tokens_per_second"], 1)}
+    mean_context = PROMPT_TOKENS + args.warmup + (args.steps + 1) / 2.0
+    step_bytes = w_bytes + kv_per_token * mean_context * BATCH
+    achieved = step_bytes / (main_run["ms_per_step"] * 1e-3) / 1e9
+    line = {
+        "metric": "decode tok/s @ batch 8 (LFM2-350M shape, bf16, context 2048+)",
+        "value": round(main_run["tokens_per_second"], 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms_per_step"], 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"model": "LFM2-350M shape, random weights", "global_batch": BATCH,
+                   "seq_len": context, "prompt_tokens": PROMPT_TOKENS, "parallelism": "single GPU",
+                   "layers": cfg["num_hidden_layers"], "layers_of_shape": full_layers,
+                   "attention_layers": cfg["layer_types"].count("full_attention"),
+                   "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+                   "ff": ff, "vocab_size": cfg["vocab_size"], "conv_L_cache": cfg["conv_L_cache"],
+                   "rope_theta": cfg["rope_theta"], "tied_embeddings": True, "page_tokens": 16},
+        "prefill": {"value": round(prefill["tokens_per_second"], 1), "tokens": PROMPT_TOKENS,
+                    "ms": round(prefill["ms"], 4),
+                    "frac": round(flops / (prefill["ms"] * 1e-3) / PEAK_FLOPS["bf16"], 5)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -290,3 +290,31 @@ class HipOps:
             _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
             _c_int(window if window else 0), self._stream())
         self._check(code, "paged_attention")
+
+    # ------------------------------------------------------------------ sampling
+    def sample(self, logits, fparams, iparams, seen, out_tokens):
+        self._dev(logits, "logits", torch.float32, contiguous=False)
+        self._dev(fparams, "fparams", torch.float32); self._dev(iparams, "iparams", torch.int32)
+        self._dev(out_tokens, "out_tokens", torch.int32)
+        R, V = logits.shape
+        if out_tokens.numel() != R or fparams.numel() < 4 * R or iparams.numel() < 2 * R:
+            raise KernelError("sample: parameter arrays do not fit the rows")
+        if seen is not None:
+            self._dev(seen, "seen", torch.uint8)
+            if seen.shape[1] != V:
+                raise KernelError("sample: the seen table must be [slots, vocab]")
+        code = self._lib("sampling").celeg_sample(
+            _ptr(logits), _c_int(self._rows(logits, "logits")), _c_int(R), _c_int(V),
+            _ptr(fparams), _ptr(iparams), _ptr(seen),
+            _c_size_t(seen.stride(0) if seen is not None else 0), _ptr(out_tokens), self._stream())
+        self._check(code, "sample")
+
+    def mark_seen(self, seen, token_ids, token_slot, n):
+        self._dev(seen, "seen", torch.uint8); self._dev(token_ids, "token_ids", torch.int32)
+        self._dev(token_slot, "token_slot", torch.int32)
+        if token_ids.numel() < n or token_slot.numel() < n:
+            raise KernelError("mark_seen: fewer rows than n")
+        code = self._lib("sampling").celeg_mark_seen(
+            _ptr(seen), _c_size_t(seen.stride(0)), _c_int(seen.shape[0]), _c_int(seen.shape[1]),
+            _ptr(token_ids), _ptr(token_slot), _c_int(n), self._stream())
+        self._check(code, "mark_seen")

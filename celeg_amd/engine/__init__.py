@@ -2,6 +2,10 @@ from .batch import StepEntry, StepBatch
 from .model import Model
 from .runner import ModelRunner, Workspace
 from .loading import load_model, LoadedModel, make_runtime, parse_dtype
+from .scheduler import (Scheduler, SchedulerOptions, RequestOptions, RequestStatus, Request,
+                        PlannedEntry)
+from .engine import Engine
 
 __all__ = ["StepEntry", "StepBatch", "Model", "ModelRunner", "Workspace", "load_model",
-           "LoadedModel", "make_runtime", "parse_dtype"]
+           "LoadedModel", "make_runtime", "parse_dtype", "Scheduler", "SchedulerOptions",
+           "RequestOptions", "RequestStatus", "Request", "PlannedEntry", "Engine"]

@@ -65,6 +65,8 @@ class ModelRunner:
         self.builder = BatchBuilder(rt.device, ints, n_groups,
                                     pin=torch.device(rt.device).type == "cuda")
         self.steps_run = 0
+        self.use_graphs = True
+        self.last_batch: Optional[StepBatch] = None
 
     # ------------------------------------------------------------------ checks
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -106,6 +108,7 @@ class ModelRunner:
         updates = self.cache.drain_table_updates()
         batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
         self._apply_table_updates(batch)
+        self.last_batch = batch
         logits = self.model.forward(batch, self.rt)
         self.steps_run += 1
         return logits

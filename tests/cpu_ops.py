@@ -133,3 +133,27 @@ class CpuOps:
                 s = (keys[:, g] @ qf[t, h]) * scale
                 pr = torch.softmax(s, dim=0)
                 out[t, h * head_dim:(h + 1) * head_dim] = (pr @ vals[:, g]).to(out.dtype)
+
+    def sample(self, logits, fparams, iparams, seen, out_tokens):
+        import plain_lfm2 as plain   # the double may lean on the plain sampler
+        R, V = logits.shape
+        for r in range(R):
+            t, top_p, pen, u = (float(x) for x in fparams[4 * r: 4 * r + 4])
+            k, row = int(iparams[2 * r]), int(iparams[2 * r + 1])
+            s = seen[row].bool().tolist() if (seen is not None and row >= 0) else [False] * V
+            # the draw comes from the host: walk with it instead of a generator state
+            out_tokens[r] = _sample_with_draw(plain, logits[r].tolist(), t, k, top_p, pen, s, u)
+
+    def mark_seen(self, seen, token_ids, token_slot, n):
+        for t, s in zip(token_ids[:n].tolist(), token_slot[:n].tolist()):
+            if 0 <= s < seen.shape[0]:
+                seen[s, t] = 1
+
+
+def _sample_with_draw(plain, logits, temperature, top_k, top_p, penalty, seen, u):
+    orig = plain.random_unit
+    plain.random_unit = lambda state: (state, u)
+    try:
+        return plain.sample(logits, temperature, top_k, top_p, penalty, seen, 1)[0]
+    finally:
+        plain.random_unit = orig

@@ -1,0 +1,271 @@
+"""Configuration, registry, safetensors reading and writing, weight errors, random weights."""
+import json
+import os
+import struct
+
+import pytest
+import torch
+
+import plain_lfm2 as plain
+from conftest import TINY, TINY_A, TINY_B
+
+from celeg_amd.config import (ConfigError, Lfm2Config, ModelSpec, PartSpec, RunStep,
+                              registered_architectures, spec_from_config)
+from celeg_amd.engine.model import Model
+from celeg_amd.weights import (Checkpoint, SafetensorsError, SafetensorsFile, WeightError,
+                               check_tensors, load_tensors, write_random_model,
+                               write_safetensors)
+
+
+# ---------------------------------------------------------------- configuration
+def test_config_reads_every_key():
+    a, b = Lfm2Config.from_dict(TINY_A), Lfm2Config.from_dict(TINY_B)
+    assert (a.hidden_size, a.num_attention_heads, a.num_key_value_heads, a.head_dim) == (64, 4, 2, 16)
+    assert a.ff_dim == 192 and b.ff_dim == 352
+    assert a.conv_L_cache == 3 and b.conv_L_cache == 4 and b.conv_bias and not a.conv_bias
+    assert a.tie_word_embeddings and not b.tie_word_embeddings
+    assert a.norm_eps == 1e-5 and b.norm_eps == 1e-6
+    assert a.eos_token_ids == (7,) and b.eos_token_ids == (2, 3)
+    assert b.rope_theta == 1e6 and a.max_position_embeddings == 128
+
+
+def test_ff_arithmetic_of_the_published_shapes():
+    def ff(inter, mult):
+        cfg = dict(TINY_B, intermediate_size=inter, block_multiple_of=mult)
+        return Lfm2Config.from_dict(cfg).ff_dim
+    assert ff(6656, 256) == 4608 and ff(12288, 256) == 8192 and ff(10752, 256) == 7168
+    assert ff(512, 32) == 352
+    for inter, mult in [(6656, 256), (512, 32), (1000, 7)]:
+        assert ff(inter, mult) == plain.ff_dim(inter, True, mult, 1.0)
+
+
+def test_config_defaults_and_aliases():
+    cfg = {k: v for k, v in TINY_A.items() if k not in ("num_key_value_heads", "head_dim", "norm_eps")}
+    c = Lfm2Config.from_dict(dict(cfg, rms_norm_eps=2e-5))
+    assert c.num_key_value_heads == 4 and c.head_dim == 16 and c.norm_eps == 2e-5
+    assert Lfm2Config.from_dict(cfg).norm_eps == 1e-6
+    with pytest.raises(ConfigError, match="disagree"):
+        Lfm2Config.from_dict(dict(TINY_A, rms_norm_eps=1e-3))
+
+
+@pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers",
+                                 "num_attention_heads", "rope_theta", "conv_L_cache",
+                                 "layer_types", "intermediate_size", "max_position_embeddings"])
+def test_missing_key_is_named(key):
+    cfg = {k: v for k, v in TINY_A.items() if k != key}
+    with pytest.raises(ConfigError, match=key):
+        Lfm2Config.from_dict(cfg)
+
+
+@pytest.mark.parametrize("change,word", [
+    ({"num_key_value_heads": 3}, "multiple"), ({"head_dim": 15}, "even"),
+    ({"layer_types": ["conv"]}, "layer_types"), ({"layer_types": ["conv", "mamba", "conv", "conv"]}, "mamba"),
+    ({"conv_L_cache": 0}, "conv_L_cache"), ({"hidden_size": "64"}, "integer"),
+    ({"num_key_value_heads": 4, "head_dim": 32}, "exceeds"), ({"norm_eps": 0.0}, "norm_eps")])
+def test_invalid_config_is_refused(change, word):
+    with pytest.raises(ConfigError, match=word):
+        Lfm2Config.from_dict(dict(TINY_A, **change))
+
+
+def test_registry_chooses_by_name_and_lists_names_on_a_miss():
+    assert "Lfm2ForCausalLM" in registered_architectures()
+    config, spec = spec_from_config(TINY_B)
+    assert isinstance(config, Lfm2Config) and isinstance(spec, ModelSpec)
+    assert [l.mixer.kind for l in spec.layers] == ["short_conv", "short_conv", "gqa_attention",
+                                                   "short_conv", "gqa_attention", "short_conv"]
+    assert spec.head.kind == "linear_head" and spec_from_config(TINY_A)[1].head.kind == "tied_head"
+    with pytest.raises(ValueError, match="Lfm2ForCausalLM"):
+        spec_from_config(dict(TINY_A, architectures=["NopeForCausalLM"]))
+    only_type = {k: v for k, v in TINY_A.items() if k != "architectures"}
+    assert spec_from_config(only_type)[1].architecture == "Lfm2ForCausalLM"
+
+
+def test_spec_sizes_come_from_the_config_only():
+    _, spec = spec_from_config(TINY_B)
+    att = spec.layers[2].mixer.params
+    assert (att["heads"], att["kv_heads"], att["head_dim"], att["eps"]) == (4, 1, 32, 1e-6)
+    assert att["position"].params["theta"] == 1e6
+    assert spec.layers[0].mixer.params == {"width": 128, "taps": 4, "bias": True}
+    assert spec.layers[0].ffn.params == {"width": 128, "ff": 352}
+    assert spec.layers[0].mixer.tensors["conv_bias"] == "model.layers.0.conv.conv.bias"
+
+
+def test_run_order_validation():
+    _, spec = spec_from_config(TINY_A)
+    import dataclasses
+    bad = dataclasses.replace(spec, order=(RunStep(0), RunStep(1, kv_from=1)))
+    with pytest.raises(ValueError, match="does not run before"):
+        bad.validate()
+    with pytest.raises(ValueError, match="names layer 9"):
+        dataclasses.replace(spec, order=(RunStep(9),)).validate()
+    conv_reads = dataclasses.replace(spec, order=(RunStep(0), RunStep(1), RunStep(2, kv_from=1)))
+    with pytest.raises(ValueError, match="keys and values"):
+        Model(conv_reads)
+    # a layer named twice and one that reads another's cache
+    shared = dataclasses.replace(spec, order=(RunStep(0), RunStep(1), RunStep(1), RunStep(3, kv_from=1)))
+    layout = Model(shared).cache_layout()
+    assert layout.group_layers == [2]
+    assert layout.kv_of_step == {1: (0, 0, True), 2: (0, 1, True), 3: (0, 0, False)}
+    assert [s for s, _ in layout.states] == [0]
+    assert "model.layers.3.self_attn.k_proj.weight" not in Model(shared).expected_tensors()
+
+
+# ---------------------------------------------------------------- safetensors
+def test_safetensors_round_trip_and_agreement_with_the_library(tmp_path):
+    from safetensors import safe_open
+    tensors = {"a": torch.randn(3, 5), "b": torch.randn(7).bfloat16(),
+               "c": torch.arange(6, dtype=torch.int64).reshape(2, 3), "d": torch.randn(2, 2).half()}
+    path = str(tmp_path / "x.safetensors")
+    write_safetensors(path, tensors, metadata={"format": "pt"})
+    f = SafetensorsFile(path)
+    assert sorted(f.names()) == ["a", "b", "c", "d"]
+    for name, t in tensors.items():
+        assert torch.equal(f.tensor(name), t)
+    with safe_open(path, framework="pt") as lib:       # the library reads what we wrote
+        for name, t in tensors.items():
+            assert torch.equal(lib.get_tensor(name), t)
+    with pytest.raises(SafetensorsError, match="missing tensor: zz"):
+        f.tensor("zz")
+    f.close()
+
+
+def _raw(path, header: dict, data: bytes):
+    text = json.dumps(header).encode()
+    with open(path, "wb") as fh:
+        fh.write(struct.pack("<Q", len(text)) + text + data)
+
+
+def test_malformed_safetensors_files(tmp_path):
+    p = str(tmp_path / "m.safetensors")
+    with open(p, "wb") as fh:
+        fh.write(b"abc")
+    with pytest.raises(SafetensorsError, match="too small"):
+        SafetensorsFile(p)
+    with open(p, "wb") as fh:
+        fh.write(struct.pack("<Q", 1 << 40) + b"{}")
+    with pytest.raises(SafetensorsError, match="header length"):
+        SafetensorsFile(p)
+    _raw(p, {"a": {"dtype": "F8_E4M3", "shape": [1], "data_offsets": [0, 1]}}, b"\0")
+    with pytest.raises(SafetensorsError, match="unsupported dtype"):
+        SafetensorsFile(p)
+    _raw(p, {"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 16]}}, b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="out-of-range"):
+        SafetensorsFile(p)
+    _raw(p, {"a": {"dtype": "F32", "shape": [3], "data_offsets": [0, 8]}}, b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="byte count"):
+        SafetensorsFile(p)
+    _raw(p, {"a": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]},
+             "b": {"dtype": "F32", "shape": [2], "data_offsets": [4, 12]}}, b"\0" * 12)
+    with pytest.raises(SafetensorsError, match="overlapping"):
+        SafetensorsFile(p)
+    text = b'{"a":{"dtype":"F32","shape":[1],"data_offsets":[0,4]},"a":{"dtype":"F32","shape":[1],"data_offsets":[4,8]}}'
+    with open(p, "wb") as fh:
+        fh.write(struct.pack("<Q", len(text)) + text + b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="duplicate"):
+        SafetensorsFile(p)
+
+
+# ---------------------------------------------------------------- weights against a model
+def _expected(cfg):
+    return Model(spec_from_config(cfg)[1]).expected_tensors()
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    folder = write_random_model(TINY_B, str(tmp_path / "m"), seed=3, dtype=torch.float32)
+    f = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    f.close()
+    del tensors["model.layers.2.self_attn.q_layernorm.weight"]
+    del tensors["lm_head.weight"]
+    tensors["model.layers.0.conv.in_proj.weight"] = torch.zeros(5, 5)
+    tensors["model.layers.9.extra.weight"] = torch.zeros(1)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    with pytest.raises(WeightError) as info:
+        check_tensors(Checkpoint(folder), _expected(TINY_B))
+    err = info.value
+    assert err.missing == ["lm_head.weight", "model.layers.2.self_attn.q_layernorm.weight"]
+    assert err.unexpected == ["model.layers.9.extra.weight"]
+    assert err.wrong_shape == [("model.layers.0.conv.in_proj.weight", (5, 5), (384, 128))]
+    text = str(err)
+    for word in ("missing tensors (2)", "unexpected tensors (1)", "wrong shape",
+                 "model.layers.9.extra.weight", "(5, 5)", "(384, 128)"):
+        assert word in text
+
+
+def test_conv_filter_is_accepted_in_both_shapes_and_bias_is_required(tmp_path):
+    folder = write_random_model(TINY_B, str(tmp_path / "m"), seed=3, dtype=torch.float32)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    f.close()
+    tensors["model.layers.0.conv.conv.weight"] = tensors["model.layers.0.conv.conv.weight"].reshape(128, 4)
+    write_safetensors(path, tensors)
+    check_tensors(Checkpoint(folder), _expected(TINY_B))
+    del tensors["model.layers.1.conv.conv.bias"]
+    write_safetensors(path, tensors)
+    with pytest.raises(WeightError, match="model.layers.1.conv.conv.bias"):
+        check_tensors(Checkpoint(folder), _expected(TINY_B))
+
+
+def test_dtype_policy(tmp_path):
+    folder = write_random_model(TINY_A, str(tmp_path / "m"), seed=0, dtype=torch.bfloat16)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    f.close()
+    kept32 = "model.layers.1.self_attn.out_proj.weight"
+    tensors[kept32] = tensors[kept32].float()
+    write_safetensors(path, tensors)
+    exp = _expected(TINY_A)
+    bf = load_tensors(Checkpoint(folder), exp, torch.bfloat16, "cpu")
+    assert bf["model.embed_tokens.weight"].dtype == torch.bfloat16
+    assert bf[kept32].dtype == torch.float32                       # stored in 32-bit: stays so
+    assert bf["model.layers.0.operator_norm.weight"].dtype == torch.float32   # vectors widen exactly
+    assert bf["model.layers.0.conv.conv.weight"].dtype == torch.float32
+    f32 = load_tensors(Checkpoint(folder), exp, torch.float32, "cpu")
+    assert all(t.dtype == torch.float32 for t in f32.values())
+    assert torch.equal(f32["model.embed_tokens.weight"], tensors["model.embed_tokens.weight"].float())
+
+
+def test_random_weights_are_keyed_by_seed_and_name(tmp_path):
+    a = write_random_model(TINY_A, str(tmp_path / "a"), seed=0, dtype=torch.float32)
+    b = write_random_model(TINY_A, str(tmp_path / "b"), seed=0, dtype=torch.float32)
+    c = write_random_model(TINY_A, str(tmp_path / "c"), seed=1, dtype=torch.float32)
+    fa, fb, fc = (SafetensorsFile(os.path.join(d, "model.safetensors")) for d in (a, b, c))
+    name = "model.layers.1.self_attn.q_proj.weight"
+    assert torch.equal(fa.tensor(name), fb.tensor(name))
+    assert not torch.equal(fa.tensor(name), fc.tensor(name))
+    assert abs(float(fa.tensor(name).std()) - 0.02) < 0.002
+    assert abs(float(fa.tensor("model.layers.0.ffn_norm.weight").mean()) - 1.0) < 0.02
+    assert sorted(fa.names()) == sorted(_expected(TINY_A))
+    assert json.load(open(os.path.join(a, "config.json")))["hidden_size"] == 64
+    # a folder without weights, a folder without config
+    os.remove(os.path.join(a, "model.safetensors"))
+    with pytest.raises(FileNotFoundError, match="model.safetensors"):
+        Checkpoint(a)
+    from celeg_amd.config import read_config_file
+    os.remove(os.path.join(b, "config.json"))
+    with pytest.raises(FileNotFoundError, match="config.json"):
+        read_config_file(b)
+
+
+def test_sharded_checkpoint(tmp_path):
+    folder = write_random_model(TINY_A, str(tmp_path / "m"), seed=0, dtype=torch.float32)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    names = f.names()
+    half = len(names) // 2
+    write_safetensors(os.path.join(folder, "s1.safetensors"), {n: f.tensor(n).clone() for n in names[:half]})
+    write_safetensors(os.path.join(folder, "s2.safetensors"), {n: f.tensor(n).clone() for n in names[half:]})
+    whole = {n: f.tensor(n).clone() for n in names}
+    f.close()
+    os.remove(path)
+    index = {"weight_map": {n: ("s1.safetensors" if i < half else "s2.safetensors")
+                            for i, n in enumerate(names)}}
+    json.dump(index, open(os.path.join(folder, "model.safetensors.index.json"), "w"))
+    ck = Checkpoint(folder)
+    check_tensors(ck, _expected(TINY_A))
+    assert all(torch.equal(ck.tensor(n), whole[n]) for n in names)
+    os.remove(os.path.join(folder, "s2.safetensors"))
+    with pytest.raises(SafetensorsError, match="missing safetensors shard"):
+        Checkpoint(folder)

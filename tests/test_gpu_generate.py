@@ -1,0 +1,184 @@
+"""Generation through the Python entry point and the command line, and the sampling
+kernels alone, against the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import plain_lfm2 as plain
+from conftest import TINY
+from helpers import ROOT, WEIGHT_STD, random_tokens
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def plain_generate(cfg, W, prompt, n, generation=None, eos=()):
+    """Greedy (or sampled) continuation with the plain model and the plain sampler."""
+    seq = list(prompt)
+    out = []
+    state = generation.seed if generation else 1
+    seen = [False] * cfg["vocab_size"]
+    for t in seq:
+        seen[t] = True
+    for _ in range(n):
+        logits = plain.model_logits(cfg, W, seq)[-1].float().tolist()
+        if generation is None:
+            token, state = plain.sample(logits, 0.0, 1, 1.0, 1.0, seen, state)
+        else:
+            token, state = plain.sample(logits, generation.temperature, generation.top_k,
+                                        generation.top_p, generation.repetition_penalty, seen, state)
+        seq.append(token); out.append(token); seen[token] = True
+        if token in eos:
+            break
+    return out
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("A", "bfloat16")])
+def test_greedy_generation_through_the_entry_point(model_folders, name, dtype):
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders(name, storage, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    vocab = cfg["vocab_size"]
+    prompts = [random_tokens(vocab, n, seed=50 + n) for n in (5, 17, 33)]
+    engine = Engine.from_folder(folder, dtype=dtype, max_active_requests=3, n_pages=12,
+                                max_batched_tokens=32, prefill_chunk_tokens=8)
+    outs = engine.generate(prompts, max_new_tokens=16, generation=GREEDY, eos_token_ids=[])
+    for prompt, out in zip(prompts, outs):
+        want = plain_generate(cfg, W, prompt, 16)
+        if dtype == "float32":
+            assert out == want
+        else:   # rounding may flip a near-tie; the first tokens must agree
+            assert out[:4] == want[:4]
+    assert engine.loaded.cache.free_pages() == [12] and engine.loaded.cache.n_free_slots == 3
+    # the same requests one at a time give the same tokens: no dependence on batch mates
+    alone = [engine.generate([p], max_new_tokens=16, generation=GREEDY, eos_token_ids=[])[0]
+             for p in prompts]
+    if dtype == "float32":
+        assert alone == outs
+
+
+def test_sampled_generation_mixed_batch_equals_plain_sampler(model_folders):
+    """Tiny B's workload: prompts 1, 9, 64, 100, 200 in portions of 32 beside decoding,
+    temperature 0.8, seed 7; every request's tokens equal the plain model + plain sampler,
+    whatever its batch mates (one generator per request)."""
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GenerationConfig
+    folder = model_folders("B", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    gen = GenerationConfig(temperature=0.8, top_k=40, top_p=0.9, repetition_penalty=1.3, seed=7)
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=70 + n) for n in (1, 9, 64, 100, 200)]
+    engine = Engine.from_folder(folder, dtype="float32", max_active_requests=4, n_pages=40,
+                                max_batched_tokens=64, prefill_chunk_tokens=32)
+    outs = engine.generate(prompts, max_new_tokens=6, generation=gen, eos_token_ids=[])
+    for prompt, out in zip(prompts, outs):
+        assert out == plain_generate(cfg, W, prompt, 6, generation=gen)
+
+
+def test_generation_with_few_pages_preempts_and_keeps_the_tokens(model_folders):
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY
+    folder = model_folders("A", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], 30, seed=90 + i) for i in range(3)]
+    engine = Engine.from_folder(folder, dtype="float32", max_active_requests=3, n_pages=6,
+                                max_batched_tokens=64, prefill_chunk_tokens=32)
+    outs = engine.generate(prompts, max_new_tokens=40, generation=GREEDY, eos_token_ids=[])
+    assert engine.scheduler.stats["preemptions"] > 0
+    for prompt, out in zip(prompts, outs):
+        assert out == plain_generate(cfg, W, prompt, 40)
+
+
+def test_command_line(model_folders, tmp_path):
+    folder = model_folders("A", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    prompt = random_tokens(cfg["vocab_size"], 12, seed=5)
+    dump = str(tmp_path / "logits.f32")
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "celeg-run"), "--model", folder, "--dtype",
+         "float32", "--prompt", ",".join(map(str, prompt)), "--max-new-tokens", "8",
+         "--repetition-penalty", "1.0", "--runtime-tokens", "--dump-logits", dump, "--print-top", "2"],
+        capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    line = [l for l in proc.stdout.splitlines() if l.startswith("CELEG_GENERATED_TOKEN_IDS=")][0]
+    got = json.loads(line.split("=", 1)[1])
+    want = plain_generate(cfg, W, prompt, 8, eos=[7])
+    assert got == want
+    import numpy as np
+    logits = np.fromfile(dump, dtype="<f4")
+    ref = plain.model_logits(cfg, W, prompt)[-1]
+    assert logits.shape == (cfg["vocab_size"],)
+    assert float(np.abs(logits - ref.numpy()).max()) < 1e-4
+    assert "top[0] token=" in proc.stderr
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "celeg-run"), "--model", folder,
+                          "--prompt", "1 2 3", "--max-new-tokens", "500"],
+                         capture_output=True, text=True, timeout=300)
+    assert bad.returncode == 1 and "prompt plus output exceeds --context" in bad.stderr
+
+
+# ---------------------------------------------------------------- the sampling kernels alone
+@pytest.fixture(scope="module")
+def ops():
+    from celeg_amd.csrc.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+def run_sample(ops, logits, rows):
+    """rows: list of (temperature, top_k, top_p, penalty, u, seen list or None)"""
+    R, V = logits.shape
+    f = torch.tensor([[t, p, pen, u] for t, k, p, pen, u, s in rows], dtype=torch.float32)
+    seen = torch.zeros(R, V, dtype=torch.uint8)
+    i = []
+    for r, (t, k, p, pen, u, s) in enumerate(rows):
+        if s is not None:
+            seen[r, torch.tensor(s, dtype=torch.long)] = 1
+        i.append([k, r if s is not None else -1])
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), f.reshape(-1).to(DEV), torch.tensor(i, dtype=torch.int32).reshape(-1).to(DEV),
+               seen.to(DEV), out)
+    return out.tolist()
+
+
+def test_sampling_kernel_reference_vectors(ops):
+    # tests/cpu_sampler_test.cpp:8-43; tests/cuda/sampling_tests.cu:16-60
+    logits = torch.tensor([[1., 4., 2., 3.], [2., 5., 5., 1.], [5., 4., 3., 2.], [1., 4., 2., 3.]])
+    got = run_sample(ops, logits, [(0.0, 1, 1.0, 1.0, 0.0, None), (0.0, 1, 1.0, 1.0, 0.0, None),
+                                   (0.0, 50, 1.0, 2.0, 0.0, [0]), (0.7, 1, 1.0, 1.0, 0.3, None)])
+    assert got == [1, 1, 1, 1]
+    for u in (0.01, 0.3, 0.6, 0.99):
+        assert run_sample(ops, logits[:1], [(1.5, 2, 1.0, 1.0, u, None)])[0] in (1, 3)
+        assert run_sample(ops, logits[:1], [(1.5, 4, 0.01, 1.0, u, None)])[0] == 1
+
+
+@pytest.mark.parametrize("vocab", [331, 4096, 65536, 70001])
+def test_sampling_kernel_equals_plain_sampler(ops, vocab):
+    g = torch.Generator().manual_seed(vocab)
+    R = 6
+    logits = torch.randn(R, vocab, generator=g) * 3
+    logits[1, 100:140] = logits[1, 7]            # many ties at one value, also at the threshold
+    logits[2] = torch.round(logits[2])           # heavy ties everywhere
+    seen = [torch.randint(0, vocab, (50,), generator=g).tolist() for _ in range(R)]
+    rows = [(0.8, 40, 0.9, 1.3, 0.37, seen[0]), (1.0, 128, 1.0, 1.0, 0.81, None),
+            (0.5, 17, 0.5, 1.0, 0.999, None), (0.0, 50, 1.0, 1.7, 0.0, seen[3]),
+            (2.0, 128, 0.95, 1.1, 0.05, seen[4]), (1.3, 2, 1.0, 1.0, 0.5, None)]
+    got = run_sample(ops, logits, rows)
+    import cpu_ops
+    for r, (t, k, p, pen, u, s) in enumerate(rows):
+        flags = [False] * vocab
+        for tok in (s or []):
+            flags[tok] = True
+        want = cpu_ops._sample_with_draw(plain, logits[r].tolist(), t, k, p, pen, flags, u)
+        assert got[r] == want, f"row {r}"
+
+
+def test_mark_seen(ops):
+    seen = torch.zeros(3, 100, dtype=torch.uint8, device=DEV)
+    toks = torch.tensor([5, 99, 5, 17], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([0, 2, 2, 3], dtype=torch.int32, device=DEV)   # slot 3 is outside: ignored
+    ops.mark_seen(seen, toks, slots, 4)
+    assert seen.sum().item() == 3 and seen[0, 5] == 1 and seen[2, 99] == 1 and seen[2, 5] == 1

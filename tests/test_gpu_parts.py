@@ -1,0 +1,274 @@
+"""Each part of a layer alone against its plain function, and the generality of the
+assembly: a toy mixer with state of its own and a toy architecture, defined here, are
+registered, built and stepped without touching the framework's files; a run order that
+names a layer twice and lets a layer read another layer's cache."""
+import dataclasses
+import os
+
+import pytest
+import torch
+
+import plain_lfm2 as plain
+from conftest import TINY
+from helpers import WEIGHT_STD, EngineDriver, assert_close_f32, portions_schedule, random_tokens
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def runtime(dtype=torch.float32):
+    from celeg_amd.engine import make_runtime
+    return make_runtime(DEV, dtype)
+
+
+def one_request_batch(rt, cache, slot, start, n):
+    from celeg_amd.engine.batch import BatchBuilder
+    from celeg_amd.engine import StepEntry
+    assert cache.prepare(slot, start, n)
+    builder = BatchBuilder(DEV, 1 << 14, len(cache.groups), pin=True)
+    batch = builder.build([StepEntry(slot, start, [0] * n)], cache.drain_table_updates(),
+                          null_slot=cache.null_slot)
+    for g, (upd, cap) in enumerate(zip(batch.table_updates, batch.table_update_caps)):
+        if cap:
+            rt.ops.apply_table_updates(cache.groups[g].table, upd, cap)
+    return batch
+
+
+def build_mixer(spec, rt, seed=0):
+    """A mixer alone: built from its PartSpec, random tensors, and a cache of its own."""
+    from celeg_amd.cache import CacheLayout, CacheManager
+    from celeg_amd.parts import build_part
+    from celeg_amd.weights import random_tensor
+    mixer = build_part("mixer", spec)
+    tensors = {role: random_tensor(seed, role, w.shape, w.init, 0.2).to(DEV)
+               for role, w in mixer.weight_specs().items()}
+    mixer.load(dict(tensors), rt)
+    layout = CacheLayout()
+    if mixer.kv_need() is not None:
+        layout.kv_groups, layout.group_layers = [mixer.kv_need()], [1]
+        layout.kv_of_step = {0: (0, 0, True)}
+    layout.states = [(0, s) for s in mixer.state_needs()]
+    cache = CacheManager(layout, page_tokens=16, n_pages=16, max_requests=2, max_context=256,
+                         device=DEV, dtype=rt.dtype)
+    return mixer, tensors, cache
+
+
+def run_mixer_in_cuts(mixer, cache, rt, x, cuts):
+    slot = cache.open()
+    outs, pos = [], 0
+    for n in cuts:
+        batch = one_request_batch(rt, cache, slot, pos, n)
+        outs.append(mixer.forward(x[pos:pos + n].contiguous(), batch, cache.layer_cache(0), rt).clone())
+        pos += n
+    cache.close(slot)
+    return torch.cat(outs).double().cpu()
+
+
+def test_short_conv_mixer_alone():
+    from celeg_amd.config import PartSpec
+    rt = runtime()
+    spec = PartSpec("short_conv", {"width": 40, "taps": 4, "bias": True})
+    mixer, t, cache = build_mixer(spec, rt)
+    x = torch.randn(29, 40, generator=torch.Generator().manual_seed(1)).to(DEV)
+    W = {"conv.in_proj.weight": t["in_proj"], "conv.in_proj.bias": t["in_proj_bias"],
+         "conv.conv.weight": t["conv"], "conv.conv.bias": t["conv_bias"],
+         "conv.out_proj.weight": t["out_proj"], "conv.out_proj.bias": t["out_proj_bias"]}
+    ref = plain.conv_mixer(x.cpu(), {k: v.cpu() for k, v in W.items()}, "", True)
+    for cuts in ([29], [5, 1, 2, 21]):
+        torch.testing.assert_close(run_mixer_in_cuts(mixer, cache, rt, x, cuts), ref, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("window", [None, 7])
+def test_attention_mixer_alone(window):
+    from celeg_amd.config import PartSpec
+    rt = runtime()
+    cfg = {"num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 16, "norm_eps": 1e-5,
+           "rope_theta": 1e4}
+    spec = PartSpec("gqa_attention", {
+        "width": 40, "heads": 6, "kv_heads": 2, "head_dim": 16, "qk_norm": True, "eps": 1e-5,
+        "window": window, "position": PartSpec("rope", {"theta": 1e4, "head_dim": 16})})
+    mixer, t, cache = build_mixer(spec, rt)
+    x = torch.randn(37, 40, generator=torch.Generator().manual_seed(2)).to(DEV)
+    W = {"self_attn.q_proj.weight": t["q_proj"], "self_attn.k_proj.weight": t["k_proj"],
+         "self_attn.v_proj.weight": t["v_proj"], "self_attn.out_proj.weight": t["out_proj"],
+         "self_attn.q_layernorm.weight": t["q_norm"], "self_attn.k_layernorm.weight": t["k_norm"]}
+    ref, _ = plain.attention_mixer(x.cpu(), {k: v.cpu() for k, v in W.items()}, "", cfg,
+                                   list(range(37)), window=window)
+    for cuts in ([37], [9, 1, 1, 20, 6]):
+        torch.testing.assert_close(run_mixer_in_cuts(mixer, cache, rt, x, cuts), ref, rtol=1e-4, atol=1e-5)
+
+
+def test_attention_without_norm_or_rotation_is_library_attention():
+    import torch.nn.functional as F
+    from celeg_amd.config import PartSpec
+    rt = runtime()
+    spec = PartSpec("gqa_attention", {"width": 32, "heads": 2, "kv_heads": 2, "head_dim": 16,
+                                      "qk_norm": False, "position": PartSpec("none")})
+    mixer, t, cache = build_mixer(spec, rt)
+    x = torch.randn(21, 32, generator=torch.Generator().manual_seed(3)).to(DEV)
+    xd = x.double().cpu()
+    q, k, v = (F.linear(xd, t[n].double().cpu()).reshape(21, 2, 16).transpose(0, 1)[None]
+               for n in ("q_proj", "k_proj", "v_proj"))
+    att = F.scaled_dot_product_attention(q, k, v, is_causal=True)[0].transpose(0, 1).reshape(21, 32)
+    ref = F.linear(att, t["out_proj"].double().cpu())
+    torch.testing.assert_close(run_mixer_in_cuts(mixer, cache, rt, x, [4, 17]), ref, rtol=1e-4, atol=1e-5)
+
+
+def test_feed_forward_and_norm_alone():
+    from celeg_amd.config import PartSpec
+    from celeg_amd.parts import build_part
+    from celeg_amd.weights import random_tensor
+    rt = runtime()
+    ffn = build_part("ffn", PartSpec("swiglu", {"width": 24, "ff": 50}))
+    t = {r: random_tensor(0, r, w.shape, w.init, 0.3).to(DEV) for r, w in ffn.weight_specs().items()}
+    ffn.load(dict(t), rt)
+    x = torch.randn(9, 24, generator=torch.Generator().manual_seed(4)).to(DEV)
+    ref = plain.swiglu_ffn(x.cpu(), t["gate"].cpu(), t["up"].cpu(), t["down"].cpu())
+    torch.testing.assert_close(ffn.forward(x, None, rt).double().cpu(), ref, rtol=1e-4, atol=1e-5)
+    norm = build_part("norm", PartSpec("rmsnorm", {"width": 24, "eps": 1e-3}))
+    w = (1 + 0.1 * torch.randn(24)).to(DEV)
+    norm.load({"weight": w}, rt)
+    out = torch.empty_like(x)
+    norm.forward(x.clone(), out, rt)
+    torch.testing.assert_close(out.double().cpu(), plain.rmsnorm(x.cpu(), w.cpu(), 1e-3), rtol=1e-5, atol=1e-6)
+
+
+# ---------------------------------------------------------------- a toy mixer and architecture
+def register_toy():
+    """A mixer whose state is its own: the running sum of its inputs and their count.
+    out[t] = (sum of x[0..t]) / (t+1) @ W^T.  It is written with torch (a toy may be) and
+    plans on the host from the batch's host arrays."""
+    from celeg_amd.config import (Architecture, LayerSpec, ModelSpec, PartSpec, RunStep,
+                                  register_architecture, registered_architectures)
+    from celeg_amd.parts import Mixer, StateNeed, WeightSpec, register_part, registered_parts
+
+    class RunningMean(Mixer):
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.width = int(self.params["width"])
+            self.w = None
+
+        def state_needs(self):
+            return [StateNeed("sum", (self.width,), torch.float32),
+                    StateNeed("count", (1,), torch.float32)]
+
+        def weight_specs(self):
+            return {"proj": WeightSpec((self.width, self.width))}
+
+        def load(self, tensors, rt):
+            self.w = tensors["proj"]
+
+        def forward(self, x, batch, cache, rt):
+            out = rt.ws.buf("toy_out", (x.shape[0], self.width), rt.dtype)
+            total, count = cache.states["sum"], cache.states["count"]
+            cu = batch.host["cu_seqlens"]
+            for s in range(batch.n_seqs):
+                slot = int(batch.host["seq_slot"][s])
+                rows = x[cu[s]:cu[s + 1]].float()
+                running = total[slot] + torch.cumsum(rows, dim=0)
+                n = count[slot] + torch.arange(1, rows.shape[0] + 1, device=x.device)[:, None]
+                out[cu[s]:cu[s + 1]] = ((running / n) @ self.w.float().t()).to(rt.dtype)
+                total[slot] = running[-1]
+                count[slot] = n[-1]
+            return out
+
+    if "running_mean" not in registered_parts("mixer"):
+        register_part("mixer", "running_mean", RunningMean)
+
+    def build_spec(cfg):
+        H = cfg["width"]
+        norm = lambda name: PartSpec("rmsnorm", {"width": H, "eps": 1e-5}, {"weight": name})
+        layers = []
+        for i, kind in enumerate(cfg["layers"]):
+            p = f"blocks.{i}."
+            if kind == "mean":
+                mixer = PartSpec("running_mean", {"width": H}, {"proj": p + "mean.proj"})
+            else:
+                mixer = PartSpec("gqa_attention",
+                                 {"width": H, "heads": 2, "kv_heads": 1, "head_dim": 16,
+                                  "qk_norm": False, "position": PartSpec("rope", {"theta": 100.0, "head_dim": 16})},
+                                 {"q_proj": p + "att.q", "k_proj": p + "att.k", "v_proj": p + "att.v",
+                                  "out_proj": p + "att.o"})
+            layers.append(LayerSpec(mixer, norm(p + "n1"),
+                                    PartSpec("swiglu", {"width": H, "ff": 2 * H},
+                                             {"gate": p + "ff.g", "up": p + "ff.u", "down": p + "ff.d"}),
+                                    norm(p + "n2")))
+        return ModelSpec("ToyForCausalLM", cfg["vocab"], H, 128,
+                         PartSpec("embedding", {"vocab": cfg["vocab"], "width": H}, {"table": "emb"}),
+                         tuple(layers), tuple(RunStep(i) for i in range(len(layers))),
+                         norm("final"), PartSpec("tied_head", {"vocab": cfg["vocab"], "width": H}))
+
+    if "ToyForCausalLM" not in registered_architectures():
+        register_architecture(Architecture("ToyForCausalLM", lambda d: d, build_spec))
+
+
+def toy_plain_logits(cfg, W, tokens):
+    """Whole-sequence reference of the toy model, from the plain parts."""
+    h = plain.embedding(W["emb"], tokens)
+    T = len(tokens)
+    for i, kind in enumerate(cfg["layers"]):
+        p = f"blocks.{i}."
+        n = plain.rmsnorm(h, W[p + "n1"], 1e-5)
+        if kind == "mean":
+            mean = torch.cumsum(n, dim=0) / torch.arange(1, T + 1, dtype=torch.float64)[:, None]
+            m = plain.linear(mean, W[p + "mean.proj"])
+        else:
+            q = plain.linear(n, W[p + "att.q"]).reshape(T, 2, 16)
+            k = plain.linear(n, W[p + "att.k"]).reshape(T, 1, 16)
+            v = plain.linear(n, W[p + "att.v"]).reshape(T, 1, 16)
+            cos, sin = plain.rope_cos_sin(range(T), 100.0, 16)
+            o = plain.causal_attention(plain.rope_apply(q, cos, sin), plain.rope_apply(k, cos, sin), v)
+            m = plain.linear(o.reshape(T, -1), W[p + "att.o"])
+        h = h + m
+        h = h + plain.swiglu_ffn(plain.rmsnorm(h, W[p + "n2"], 1e-5), W[p + "ff.g"], W[p + "ff.u"], W[p + "ff.d"])
+    return plain.linear(plain.rmsnorm(h, W["final"], 1e-5), W["emb"])
+
+
+def test_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path):
+    from celeg_amd.engine import load_model
+    from celeg_amd.weights import write_random_model
+    register_toy()
+    cfg = {"architectures": ["ToyForCausalLM"], "width": 32, "vocab": 77,
+           "layers": ["mean", "attention", "mean"]}
+    folder = write_random_model(cfg, str(tmp_path / "toy"), seed=4, dtype=torch.float32, std=0.2)
+    _, W = plain.load_model_folder(folder)
+    reqs = {"x": random_tokens(77, 45, 1), "y": random_tokens(77, 30, 2)}
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2,
+                    max_batched_tokens=64)
+    assert [n.name for _, n in lm.cache.layout.states] == ["sum", "count", "sum", "count"]
+    got = EngineDriver(lm).run(portions_schedule(reqs))
+    got2 = EngineDriver(lm).run(portions_schedule(dict(reversed(list(reqs.items())))))   # slots reused
+    for rid, toks in reqs.items():
+        ref = toy_plain_logits(cfg, W, toks)
+        assert_close_f32(got[rid], ref, f"toy/{rid}")
+        assert_close_f32(got2[rid], ref, f"toy again/{rid}")
+
+
+def test_run_order_with_a_layer_twice_and_a_shared_cache(model_folders, tmp_path):
+    """LFM2 parts under another run order: layer 1 runs twice (own cache each time) and
+    layer 3 reads the keys and values the first run of layer 1 wrote."""
+    from celeg_amd.cache import CacheManager
+    from celeg_amd.config import RunStep, spec_from_config
+    from celeg_amd.engine import Model, ModelRunner, make_runtime
+    from celeg_amd.engine.loading import LoadedModel
+    from celeg_amd.weights import Checkpoint, load_tensors
+    folder = model_folders("A", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    config, spec = spec_from_config(TINY["A"][0])
+    order = (RunStep(0), RunStep(1), RunStep(2), RunStep(1), RunStep(3, kv_from=1))
+    spec = dataclasses.replace(spec, order=order)
+    model = Model(spec)
+    rt = make_runtime(DEV, torch.float32)
+    expected = model.expected_tensors()
+    assert "model.layers.3.self_attn.k_proj.weight" not in expected
+    ck = Checkpoint(folder)
+    tensors = {n: ck.tensor(n).float().to(DEV) for n in expected}
+    model.load(tensors, rt)
+    cache = CacheManager(model.cache_layout(), page_tokens=16, n_pages=8, max_requests=2,
+                         max_context=128, device=DEV, dtype=torch.float32)
+    lm = LoadedModel(config, spec, model, cache, ModelRunner(model, cache, rt, max_batched_tokens=64), rt)
+    reqs = {"a": random_tokens(256, 50, 8), "b": random_tokens(256, 37, 9)}
+    got = EngineDriver(lm).run(portions_schedule(reqs))
+    for rid, toks in reqs.items():
+        ref = plain.model_logits(cfg, W, toks, order=[0, 1, 2, 1, 3], kv_from={4: 1})
+        assert_close_f32(got[rid], ref, f"order/{rid}")
