@@ -10,8 +10,9 @@ state per lane (include/celeg/detail/model/layer_state.hpp:180-187); here state 
 fixed size per request lives in *slots*: one row of one buffer per request, zeroed
 when the request starts, with a region for every layer that declared a need.
 
-Storage of a group: K and V each ``[pages + 1, layers, kv_heads, page_tokens,
-head_dim]``.  The extra last page is never handed out: rows that pad a batch to a
+Storage of a group: K ``[pages + 1, layers, kv_heads, page_tokens, head_dim]`` and V
+``[pages + 1, layers, kv_heads, head_dim, page_tokens]`` (transposed inside a page: the
+layout the matrix-core attention kernel reads without shuffling).  The extra last page is never handed out: rows that pad a batch to a
 fixed size write there.  Likewise the last slot (``null_slot``) is never given to a
 request.
 
@@ -70,9 +71,10 @@ class _Group:
         self.need = need
         self.n_layers = n_layers
         self.pool = PagePool(n_pages, page_tokens)
-        shape = (n_pages + 1, n_layers, need.kv_heads, page_tokens, need.head_dim)
-        self.k = torch.zeros(shape, dtype=dtype, device=device)
-        self.v = torch.zeros(shape, dtype=dtype, device=device)
+        self.k = torch.zeros((n_pages + 1, n_layers, need.kv_heads, page_tokens, need.head_dim),
+                             dtype=dtype, device=device)
+        self.v = torch.zeros((n_pages + 1, n_layers, need.kv_heads, need.head_dim, page_tokens),
+                             dtype=dtype, device=device)
         self.trash_page = n_pages
         # block tables: row = slot, column = logical page (position // page_tokens)
         self.table_host = np.full((n_slots + 1, max_pages_per_request), -1, dtype=np.int32)

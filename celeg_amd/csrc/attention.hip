@@ -2,7 +2,9 @@
 // with k and v written into their pages; (2) a general attention kernel that serves
 // every kind of row (prompt portions and decode tokens) in both dtypes.
 //
-// Cache layout of a group: K and V each [pages, layers, kv_heads, page_tokens, head_dim].
+// Cache layout of a group: K [pages, layers, kv_heads, page_tokens, head_dim] and
+// V [pages, layers, kv_heads, head_dim, page_tokens] (transposed inside the page, which
+// is what the matrix-core kernel of attention_fast.hip wants).
 // A row at position p of the request in slot s lives in page table[s, p / page_tokens]
 // at place p % page_tokens.  (The reference's layout and addressing:
 // src/backend/cuda/kernels/kv_cache.cuh:1-7, 215-240.)
@@ -43,14 +45,16 @@ __global__ void qk_norm_rope_store_kernel(
         dst = q + static_cast<size_t>(t) * ldq + static_cast<size_t>(head) * head_dim;
     } else {
         const int page = table[static_cast<size_t>(token_slot[t]) * table_stride + pos / page_tokens];
-        dst = (is_k ? k_pool : v_pool) +
-              cache_offset(page, n_layers, layer, kv_heads, kv_head, page_tokens,
-                           pos % page_tokens, head_dim);
-    }
-    if (!is_q && !is_k) {  // v: copy
-        const T* src = v + static_cast<size_t>(t) * ldv + static_cast<size_t>(kv_head) * head_dim;
-        for (int d = lane; d < head_dim; d += CELEG_WAVE) dst[d] = src[d];
-        return;
+        if (!is_k) {  // v: copy, transposed inside the page
+            T* vdst = v_pool + cache_offset(page, n_layers, layer, kv_heads, kv_head, page_tokens,
+                                            0, head_dim) + pos % page_tokens;
+            const T* src = v + static_cast<size_t>(t) * ldv + static_cast<size_t>(kv_head) * head_dim;
+            for (int d = lane; d < head_dim; d += CELEG_WAVE)
+                vdst[static_cast<size_t>(d) * page_tokens] = src[d];
+            return;
+        }
+        dst = k_pool + cache_offset(page, n_layers, layer, kv_heads, kv_head, page_tokens,
+                                    pos % page_tokens, head_dim);
     }
     const T* src = is_q ? q + static_cast<size_t>(t) * ldq + static_cast<size_t>(head) * head_dim
                         : k + static_cast<size_t>(t) * ldk + static_cast<size_t>(kv_head) * head_dim;
@@ -166,13 +170,14 @@ __global__ void paged_attention_kernel(
         for (int kk = 0; kk < n_keys; ++kk) {
             const int key2 = base + kk;
             const T* vp = v_pool + cache_offset(pages[key2 / page_tokens], n_layers, layer,
-                                                kv_heads, kvh, page_tokens, key2 % page_tokens,
-                                                head_dim);
+                                                kv_heads, kvh, page_tokens, 0, head_dim) +
+                          key2 % page_tokens;
             const float pk = ps[kk];
 #pragma unroll
             for (int j = 0; j < ATT_MAX_DIM_CHUNKS; ++j) {
                 const int d = lane + j * CELEG_WAVE;
-                if (d < head_dim) acc[j] = fmaf(pk, to_float(vp[d]), acc[j]);
+                if (d < head_dim)
+                    acc[j] = fmaf(pk, to_float(vp[static_cast<size_t>(d) * page_tokens]), acc[j]);
             }
         }
         __syncthreads();

@@ -1,0 +1,390 @@
+// bfloat16 attention over the paged cache for gfx950: an MFMA kernel for the rows of
+// prompt portions (and mixed batches), and a split-key kernel for batches in which
+// every request brings one row (decode).
+//
+// Cache layout of a group (one page id covers all layers of the group):
+//   K [pages, layers, kv_heads, page_tokens, head_dim]   one key after the other
+//   V [pages, layers, kv_heads, head_dim, page_tokens]   transposed inside the page
+// K rows feed the MFMA of q.k directly (head_dim runs along the instruction's k), and
+// the transposed V feeds the MFMA of p.v directly (keys run along its k), so neither
+// operand is shuffled through LDS.
+//
+// Scores are (q.k)*scale, causal (key position <= row position) and, with a window w,
+// key position > row position - w.  Softmax statistics and accumulators are 32-bit; the
+// probabilities enter the second product rounded to bfloat16.
+// Reference semantics: src/backend/cpu/attention/paged_attention.cpp:229-283; tiled CUDA
+// form src/backend/cuda/kernels/attention_gemm.cuh:15-200; split-key CUDA form
+// src/backend/cuda/kernels/attention_paged.cuh:287-487.
+#include "common.h"
+
+typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ size_t kv_block(int page, int n_layers, int layer, int kv_heads,
+                                           int head, int page_tokens, int head_dim) {
+    return ((static_cast<size_t>(page) * n_layers + layer) * kv_heads + head) *
+           static_cast<size_t>(page_tokens) * head_dim;
+}
+
+__device__ __forceinline__ short bf16_bits(float x) { return static_cast<short>(from_float<bf16>(x).bits); }
+
+// ================================================================ rows of portions
+// One workgroup of 4 wavefronts per (tile of 64 rows of one request, query head); a
+// wavefront owns 16 rows.  Per 64 keys: S^T = K Q^T (16x16x16 MFMA: A = 16 keys x 16
+// dims, B = 16 dims x 16 rows), online softmax per row (a row is a lane column), then
+// O^T += V^T P^T (A = 16 dims x 16 keys from the transposed V, B = P^T straight from the
+// accumulator registers of S^T).
+template <int HD>
+__global__ __launch_bounds__(256) void attention_rows_kernel(
+    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
+    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
+    const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_start, int n_seqs, bf16* __restrict__ out, int ldo, int q_heads,
+    int kv_heads, int page_tokens, int n_layers, int layer, float scale_log2e, int window) {
+    constexpr int DQ = HD / 4;   // dims a lane quad covers in q.k
+    constexpr int KS = DQ / 4;   // MFMA steps along head_dim
+    constexpr int DT = HD / 16;  // 16-dim tiles of the output
+    int tile = blockIdx.x;
+    const int h = blockIdx.y;
+    int s = 0, len = 0;
+    bool found = false;
+    for (; s < n_seqs; ++s) {
+        len = cu_seqlens[s + 1] - cu_seqlens[s];
+        const int tiles = (len + 63) >> 6;
+        if (tile < tiles) { found = true; break; }
+        tile -= tiles;
+    }
+    if (!found) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c = lane & 15, qd = lane >> 4;
+    const int wrow0 = tile * 64 + wave * 16;
+    if (wrow0 >= len) return;  // no row of this wavefront exists (no barrier is used below)
+    const int row = wrow0 + c;
+    const bool row_valid = row < len;
+    const int row_c = row_valid ? row : len - 1;
+    const int start = seq_start[s];
+    const int pq = start + row_c;                       // this lane's row position
+    const int lo_q = window > 0 ? max(0, pq - window + 1) : 0;
+    const int kmax = start + min(wrow0 + 15, len - 1);  // last key any row of the wavefront sees
+    const int kmin = window > 0 ? max(0, start + wrow0 - window + 1) : 0;
+    const int kvh = h / (q_heads / kv_heads);
+    const int* __restrict__ pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
+    const size_t row_base = static_cast<size_t>(cu_seqlens[s]);
+
+    bf16x4_t qreg[KS];
+    {
+        const bf16* qrow = q + (row_base + row_c) * ldq + static_cast<size_t>(h) * HD + qd * DQ;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) qreg[st] = *reinterpret_cast<const bf16x4_t*>(qrow + st * 4);
+    }
+    floatx4_t oacc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+
+    for (int kb = (kmin >> 6) << 6; kb <= kmax; kb += 64) {
+        floatx4_t sacc[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            sacc[kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+            const int key0 = kb + kt * 16;
+            if (key0 > kmax) continue;
+            const int key = min(key0 + c, kmax);  // a valid address; masked below if beyond
+            const bf16* kp = k_pool +
+                             kv_block(pages[key / page_tokens], n_layers, layer, kv_heads, kvh,
+                                      page_tokens, HD) +
+                             static_cast<size_t>(key % page_tokens) * HD + qd * DQ;
+#pragma unroll
+            for (int st = 0; st < KS; ++st) {
+                const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(kp + st * 4);
+                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qreg[st], sacc[kt], 0, 0, 0);
+            }
+        }
+        // sacc[kt][r] = (key kb + 16 kt + 4 qd + r) . (row c)
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = kb + kt * 16 + 4 * qd + r;
+                const float sv = (key <= pq && key >= lo_q) ? sacc[kt][r] * scale_log2e : -INFINITY;
+                sacc[kt][r] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
+        const float alpha = exp2f(m - m_use);
+        float psum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float p = exp2f(sacc[kt][r] - m_use);
+                sacc[kt][r] = p;
+                psum += p;
+            }
+        l = l * alpha + psum;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            const int key0 = kb + kt * 16;
+            if (key0 > kmax) continue;
+            const bf16x4_t pb = {bf16_bits(sacc[kt][0]), bf16_bits(sacc[kt][1]),
+                                 bf16_bits(sacc[kt][2]), bf16_bits(sacc[kt][3])};
+            const bf16* vp = v_pool +
+                             kv_block(pages[key0 / page_tokens], n_layers, layer, kv_heads, kvh,
+                                      page_tokens, HD) +
+                             static_cast<size_t>(c) * page_tokens + (key0 % page_tokens) + 4 * qd;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(
+                    vp + static_cast<size_t>(dt) * 16 * page_tokens);
+                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, oacc[dt], 0, 0, 0);
+            }
+        }
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!row_valid) return;
+    const float inv_l = 1.0f / l;
+    bf16* orow = out + (row_base + row) * ldo + static_cast<size_t>(h) * HD + 4 * qd;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const bf16x4_t o = {bf16_bits(oacc[dt][0] * inv_l), bf16_bits(oacc[dt][1] * inv_l),
+                            bf16_bits(oacc[dt][2] * inv_l), bf16_bits(oacc[dt][3] * inv_l)};
+        *reinterpret_cast<bf16x4_t*>(orow + dt * 16) = o;
+    }
+}
+
+extern "C" int celeg_attention_rows_bf16(
+    const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+    int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
+    int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int head_dim,
+    int page_tokens, int n_layers, int layer, float scale, int window, hipStream_t stream) {
+    if (n_tokens <= 0 || n_seqs <= 0) return 0;
+    if (page_tokens % 16 || q_heads % kv_heads || (ldq % 4) || (ldo % 4))
+        return static_cast<int>(hipErrorInvalidValue);
+    const int max_tiles = n_tokens / 64 + n_seqs;  // >= sum over requests of ceil(rows / 64)
+    dim3 grid(max_tiles, q_heads), block(256);
+    const float scale_log2e = scale * 1.4426950408889634f;
+#define CELEG_ROWS(HD_)                                                                          \
+    hipLaunchKernelGGL(attention_rows_kernel<HD_>, grid, block, 0, stream,                       \
+                       static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
+                       static_cast<const bf16*>(v_pool), table, table_stride, cu_seqlens,        \
+                       seq_slot, seq_start, n_seqs, static_cast<bf16*>(out), ldo, q_heads,       \
+                       kv_heads, page_tokens, n_layers, layer, scale_log2e, window)
+    switch (head_dim) {
+        case 32: CELEG_ROWS(32); break;
+        case 64: CELEG_ROWS(64); break;
+        case 96: CELEG_ROWS(96); break;
+        case 128: CELEG_ROWS(128); break;
+        default: return static_cast<int>(hipErrorInvalidValue);
+    }
+#undef CELEG_ROWS
+    return CELEG_LAUNCH_RESULT();
+}
+
+// ================================================================ one row per request
+// One wavefront per (range of `split_keys` keys, GH query heads that share a key/value
+// head, request).  Keys are taken 64 at a time: for q.k a lane owns (key j, an eighth of
+// head_dim) and eight lanes add up a score; for p.v a lane owns a dimension and reads
+// its row of the transposed V.  Partial (max, sum, accumulator) go to a workspace and a
+// second kernel joins the ranges.
+template <int HD, int GH>
+__global__ __launch_bounds__(64) void attention_decode_kernel(
+    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
+    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
+    const int* __restrict__ token_slot, const int* __restrict__ positions,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits, int split_keys,
+    int q_heads, int kv_heads, int page_tokens, int n_layers, int layer, float scale, int window) {
+    constexpr int DL = HD / 8;    // dims of a key a lane multiplies
+    constexpr int DD = HD / 64;   // output dims a lane accumulates
+    __shared__ float ps[GH][64];
+    const int split = blockIdx.x, hb = blockIdx.y, t = blockIdx.z;
+    const int lane = threadIdx.x;
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int k_lo = max(lo, split * split_keys);
+    const int k_hi = min(pos, (split + 1) * split_keys - 1);
+    if (k_lo > k_hi) return;
+    const int h0 = hb * GH;
+    const int kvh = h0 / (q_heads / kv_heads);
+    const int j8 = lane >> 3, seg = lane & 7;
+    const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
+
+    float qf[GH][DL];
+#pragma unroll
+    for (int g = 0; g < GH; ++g) {
+        const bf16* qrow = q + static_cast<size_t>(t) * ldq + static_cast<size_t>(h0 + g) * HD + seg * DL;
+#pragma unroll
+        for (int d = 0; d < DL; ++d) qf[g][d] = to_float(qrow[d]) * scale;
+    }
+    float m[GH], l[GH], acc[GH][DD];
+#pragma unroll
+    for (int g = 0; g < GH; ++g) {
+        m[g] = -INFINITY; l[g] = 0.f;
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) acc[g][dd] = 0.f;
+    }
+
+    for (int kb = (k_lo >> 6) << 6; kb <= k_hi; kb += 64) {
+        float sc[8][GH];
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int key = kb + it * 8 + j8;
+            const bool valid = key >= k_lo && key <= k_hi;
+            const int keyc = min(max(key, k_lo), k_hi);
+            const bf16* kp = k_pool +
+                             kv_block(pages[keyc / page_tokens], n_layers, layer, kv_heads, kvh,
+                                      page_tokens, HD) +
+                             static_cast<size_t>(keyc % page_tokens) * HD + seg * DL;
+            float kf[DL];
+#pragma unroll
+            for (int v8 = 0; v8 < DL / 8; ++v8) {
+                const uint4 raw = *reinterpret_cast<const uint4*>(kp + v8 * 8);
+                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    kf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
+                    kf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < GH; ++g) {
+                float dot = 0.f;
+#pragma unroll
+                for (int d = 0; d < DL; ++d) dot = fmaf(qf[g][d], kf[d], dot);
+                dot += __shfl_xor(dot, 1, 64);
+                dot += __shfl_xor(dot, 2, 64);
+                dot += __shfl_xor(dot, 4, 64);
+                sc[it][g] = valid ? dot : -INFINITY;
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < GH; ++g) {
+            float mx = sc[0][g];
+#pragma unroll
+            for (int it = 1; it < 8; ++it) mx = fmaxf(mx, sc[it][g]);
+            mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m[g], mx);   // finite: the chunk holds a key of the range
+            const float corr = expf(m[g] - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int it = 0; it < 8; ++it) {
+                const float p = expf(sc[it][g] - m_new);
+                psum += p;
+                if (seg == 0) ps[g][it * 8 + j8] = p;
+            }
+            l[g] = l[g] * corr + psum;
+            m[g] = m_new;
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) acc[g][dd] *= corr;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int pg = 0; pg < 4; ++pg) {
+            const int key0 = kb + pg * 16;
+            if (key0 > k_hi || key0 + 15 < k_lo) continue;
+            const bf16* vbase = v_pool +
+                                kv_block(pages[key0 / page_tokens], n_layers, layer, kv_heads, kvh,
+                                         page_tokens, HD) + (key0 % page_tokens);
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) {
+                const bf16* vp = vbase + static_cast<size_t>(lane + 64 * dd) * page_tokens;
+                float vf[16];
+#pragma unroll
+                for (int v8 = 0; v8 < 2; ++v8) {
+                    const uint4 raw = *reinterpret_cast<const uint4*>(vp + v8 * 8);
+                    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        vf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
+                        vf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                    }
+                }
+#pragma unroll
+                for (int g = 0; g < GH; ++g)
+#pragma unroll
+                    for (int j = 0; j < 16; ++j)
+                        acc[g][dd] = fmaf(ps[g][pg * 16 + j], vf[j], acc[g][dd]);
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int g = 0; g < GH; ++g) {
+        float lt = l[g];   // the eight lanes of a key hold the same p: add over keys only
+        lt += __shfl_xor(lt, 8, 64);
+        lt += __shfl_xor(lt, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        const size_t idx = (static_cast<size_t>(t) * q_heads + h0 + g) * n_splits + split;
+        if (lane == 0) { ws_ml[2 * idx] = m[g]; ws_ml[2 * idx + 1] = lt; }
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) ws_o[idx * HD + lane + 64 * dd] = acc[g][dd];
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
+    const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
+    const int* __restrict__ positions, bf16* __restrict__ out, int ldo, int q_heads, int n_splits,
+    int split_keys, int window) {
+    const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int first = lo / split_keys, last = pos / split_keys;
+    const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits;
+    float m = -INFINITY;
+    for (int i = first; i <= last; ++i) m = fmaxf(m, ws_ml[2 * (base + i)]);
+    float denom = 0.f, acc[HD / 64];
+#pragma unroll
+    for (int dd = 0; dd < HD / 64; ++dd) acc[dd] = 0.f;
+    for (int i = first; i <= last; ++i) {
+        const float w = expf(ws_ml[2 * (base + i)] - m);
+        denom += w * ws_ml[2 * (base + i) + 1];
+#pragma unroll
+        for (int dd = 0; dd < HD / 64; ++dd) acc[dd] += w * ws_o[(base + i) * HD + lane + 64 * dd];
+    }
+    bf16* orow = out + static_cast<size_t>(t) * ldo + static_cast<size_t>(h) * HD;
+#pragma unroll
+    for (int dd = 0; dd < HD / 64; ++dd) orow[lane + 64 * dd] = from_float<bf16>(acc[dd] / denom);
+}
+
+// workspace: ws_o [rows, q_heads, n_splits, head_dim] and ws_ml [rows, q_heads, n_splits, 2]
+// floats, n_splits = ceil(max_context / split_keys).
+extern "C" int celeg_attention_decode_bf16(
+    const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+    int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
+    int n_splits, int split_keys, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
+    int head_dim, int page_tokens, int n_layers, int layer, float scale, int window,
+    hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    const int group = q_heads / kv_heads;
+    if (q_heads % kv_heads || page_tokens % 16 || split_keys % 64 || n_splits <= 0 || (ldq % 8))
+        return static_cast<int>(hipErrorInvalidValue);
+    const int gh = (group % 4 == 0) ? 4 : ((group % 2 == 0) ? 2 : 1);
+    dim3 grid(n_splits, q_heads / gh, n_rows), block(64);
+#define CELEG_DEC(HD_, GH_)                                                                      \
+    hipLaunchKernelGGL((attention_decode_kernel<HD_, GH_>), grid, block, 0, stream,              \
+                       static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
+                       static_cast<const bf16*>(v_pool), table, table_stride, token_slot,        \
+                       positions, ws_o, ws_ml, n_splits, split_keys, q_heads, kv_heads,          \
+                       page_tokens, n_layers, layer, scale, window)
+#define CELEG_DEC_HD(HD_)                                                                        \
+    if (gh == 4) CELEG_DEC(HD_, 4); else if (gh == 2) CELEG_DEC(HD_, 2); else CELEG_DEC(HD_, 1);  \
+    hipLaunchKernelGGL(attention_decode_reduce_kernel<HD_>, dim3(q_heads, n_rows), dim3(64), 0,  \
+                       stream, ws_o, ws_ml, positions, static_cast<bf16*>(out), ldo, q_heads,    \
+                       n_splits, split_keys, window)
+    if (head_dim == 64) { CELEG_DEC_HD(64); }
+    else if (head_dim == 128) { CELEG_DEC_HD(128); }
+    else return static_cast<int>(hipErrorInvalidValue);
+#undef CELEG_DEC_HD
+#undef CELEG_DEC
+    return CELEG_LAUNCH_RESULT();
+}

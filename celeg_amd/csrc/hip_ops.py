@@ -40,6 +40,11 @@ class HipOps:
             raise KernelError(f"celeg_amd runs on a GPU only, not on '{device}'")
         self._libs: Dict[str, ctypes.CDLL] = {}
         self.loaded_libraries: Dict[str, str] = {}
+        # "auto": the matrix-core and split-key kernels where they apply; "general": always
+        # the general kernel (tests compare the two)
+        self.attention_impl = "auto"
+        self.decode_split_keys = None      # None: chosen from the number of rows
+        self._decode_ws = None
 
     # ------------------------------------------------------------------ plumbing
     def _lib(self, module: str) -> ctypes.CDLL:
@@ -230,10 +235,10 @@ class HipOps:
     def _check_kv(self, kv, kv_heads, head_dim, dtype):
         if kv.kv_heads != kv_heads or kv.head_dim != head_dim:
             raise KernelError("attention: the cache has other head sizes than the mixer")
-        for name, pool in (("k", kv.k), ("v", kv.v)):
-            self._dev(pool, f"{name} cache", dtype)
-            if pool.shape[1:] != (kv.n_layers, kv_heads, kv.page_tokens, head_dim):
-                raise KernelError("attention: unexpected cache shape")
+        self._dev(kv.k, "k cache", dtype); self._dev(kv.v, "v cache", dtype)
+        if kv.k.shape[1:] != (kv.n_layers, kv_heads, kv.page_tokens, head_dim) or \
+                kv.v.shape[1:] != (kv.n_layers, kv_heads, head_dim, kv.page_tokens):
+            raise KernelError("attention: unexpected cache shape")
         self._dev(kv.table, "block table", torch.int32)
         if not 0 <= kv.layer < kv.n_layers:
             raise KernelError("attention: layer index outside the cache")
@@ -282,6 +287,21 @@ class HipOps:
         if heads % kv_heads:
             raise KernelError("paged_attention: heads must be a multiple of kv_heads")
         self._check_kv(kv, kv_heads, head_dim, q.dtype)
+        if q.dtype == torch.bfloat16 and self.attention_impl != "general" \
+                and kv.page_tokens % 16 == 0 and self._rows(q, "q") % 8 == 0:
+            if batch.decode_only and head_dim in (64, 128) and batch.n_seqs == T:
+                return self._attention_decode(q, out, heads, kv_heads, head_dim, scale, window,
+                                              batch, kv)
+            if head_dim in (32, 64, 96, 128):
+                code = self._lib("attention_fast").celeg_attention_rows_bf16(
+                    _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v), _ptr(kv.table),
+                    _c_int(kv.table.shape[1]), _ptr(batch.cu_seqlens), _ptr(batch.seq_slot),
+                    _ptr(batch.seq_start), _c_int(batch.n_seqs), _c_int(T), _ptr(out),
+                    _c_int(heads * head_dim), _c_int(heads), _c_int(kv_heads), _c_int(head_dim),
+                    _c_int(kv.page_tokens), _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
+                    _c_int(window if window else 0), self._stream())
+                self._check(code, "attention over rows (bfloat16)")
+                return
         code = self._lib("attention").celeg_paged_attention(
             _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v),
             _c_int(self._dtype(q, "q")), _ptr(kv.table), _c_int(kv.table.shape[1]),
@@ -290,6 +310,32 @@ class HipOps:
             _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
             _c_int(window if window else 0), self._stream())
         self._check(code, "paged_attention")
+
+    def _attention_decode(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv):
+        T = q.shape[0]
+        group = heads // kv_heads
+        gh = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
+        split_keys = self.decode_split_keys
+        if split_keys is None:
+            blocks = T * (heads // gh)
+            split_keys = 64 if blocks <= 16 else (128 if blocks <= 128 else 256)
+        if split_keys % 64:
+            raise KernelError("attention: decode_split_keys must be a multiple of 64")
+        max_context = kv.table.shape[1] * kv.page_tokens
+        n_splits = (max_context + split_keys - 1) // split_keys
+        need = T * heads * n_splits * (head_dim + 2)
+        if self._decode_ws is None or self._decode_ws.numel() < need:
+            self._decode_ws = torch.empty(need, dtype=torch.float32, device=q.device)
+        ws_o = self._decode_ws[:T * heads * n_splits * head_dim]
+        ws_ml = self._decode_ws[T * heads * n_splits * head_dim:need]
+        code = self._lib("attention_fast").celeg_attention_decode_bf16(
+            _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v), _ptr(kv.table),
+            _c_int(kv.table.shape[1]), _ptr(batch.token_slot), _ptr(batch.positions), _ptr(ws_o),
+            _ptr(ws_ml), _c_int(n_splits), _c_int(split_keys), _ptr(out), _c_int(heads * head_dim),
+            _c_int(T), _c_int(heads), _c_int(kv_heads), _c_int(head_dim), _c_int(kv.page_tokens),
+            _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
+            _c_int(window if window else 0), self._stream())
+        self._check(code, "attention for decode rows (bfloat16)")
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, fparams, iparams, seen, out_tokens):

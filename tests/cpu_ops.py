@@ -113,7 +113,7 @@ class CpuOps:
             p = int(pos[t])
             page = int(kv.table[int(batch.token_slot[t]), p // P])
             kv.k[page, kv.layer, :, p % P, :] = kk[t]
-            kv.v[page, kv.layer, :, p % P, :] = vv[t]
+            kv.v[page, kv.layer, :, :, p % P] = vv[t]
 
     def paged_attention(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv):
         T = q.shape[0]
@@ -126,7 +126,7 @@ class CpuOps:
             first = max(0, p - window + 1) if window else 0
             keys = torch.stack([kv.k[int(kv.table[slot, u // P]), kv.layer, :, u % P, :]
                                 for u in range(first, p + 1)]).float()   # [n, Hkv, hd]
-            vals = torch.stack([kv.v[int(kv.table[slot, u // P]), kv.layer, :, u % P, :]
+            vals = torch.stack([kv.v[int(kv.table[slot, u // P]), kv.layer, :, :, u % P]
                                 for u in range(first, p + 1)]).float()
             for h in range(heads):
                 g = h // group

@@ -91,6 +91,10 @@ def test_state_slots_are_separate_zeroed_and_typed():
     assert float(bx0[b].min()) == 3.0
     assert m.layer_cache(1).states == {} and m.layer_cache(1).kv.layer == 0
     assert m.layer_cache(3).kv.layer == 1 and m.layer_cache(3).kv.k.shape == (13, 2, 2, 16, 16)
+    wide = CacheManager(CacheLayout([KVNeed(2, 32)], [1], {0: (0, 0, True)}, []), page_tokens=16,
+                        n_pages=3, max_requests=1, max_context=64, device="cpu", dtype=torch.float32)
+    kv = wide.layer_cache(0).kv         # keys row by row, values transposed inside the page
+    assert kv.k.shape == (4, 1, 2, 16, 32) and kv.v.shape == (4, 1, 2, 32, 16)
 
 
 def test_window_group_gives_pages_back_as_the_window_passes():

@@ -264,10 +264,34 @@ def attention_case(ops, dtype, heads, kv_heads, head_dim, lengths, cuts, window=
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,kv_heads,head_dim", [(6, 3, 48), (5, 5, 16), (8, 1, 128), (4, 2, 80)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [
+    (6, 3, 48), (5, 5, 16), (8, 1, 128), (4, 2, 80), (16, 8, 64), (3, 3, 64), (6, 2, 96),
+    (8, 2, 32), (12, 4, 128)])
 def test_attention_mixed_steps(ops, dtype, heads, kv_heads, head_dim):
     attention_case(ops, dtype, heads, kv_heads, head_dim, lengths=[70, 33, 150],
                    cuts=[7, 1, 2, 30, 1, 16, 5])
+
+
+@pytest.mark.parametrize("split_keys", [64, 128, None])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(4, 2, 64), (8, 1, 128), (3, 1, 64)])
+def test_attention_long_prompt_then_decode_rows(ops, heads, kv_heads, head_dim, split_keys):
+    """A long portion through the matrix-core kernel, then rows one by one through the
+    split-key kernel, several requests per step, ranges of keys of 64, 128 or chosen."""
+    ops.decode_split_keys = split_keys
+    try:
+        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[333, 150, 420],
+                       cuts=[300] + [1] * 40, boost=(2, 331))
+    finally:
+        ops.decode_split_keys = None
+
+
+def test_fast_and_general_attention_agree(ops):
+    """The same bfloat16 case through the general kernel."""
+    ops.attention_impl = "general"
+    try:
+        attention_case(ops, torch.bfloat16, 4, 2, 64, lengths=[333, 150], cuts=[300] + [1] * 40)
+    finally:
+        ops.attention_impl = "auto"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -286,6 +310,15 @@ def test_attention_window_edge(ops, dtype):
                    boost=(3, 23), qk_norm=False, rotary_dim=0)
 
 
-def test_attention_partial_rotary_and_other_page_size(ops):
-    attention_case(ops, torch.float32, 4, 4, 64, lengths=[45, 80], cuts=[9, 1, 3],
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_partial_rotary_and_other_page_size(ops, dtype):
+    attention_case(ops, dtype, 4, 4, 64, lengths=[45, 80], cuts=[9, 1, 3],
                    rotary_dim=32, theta=1e6, page_tokens=32)
+
+
+def test_attention_window_fast_kernels(ops):
+    # head size 64: the matrix-core and split-key kernels, window 70, pages of 32
+    attention_case(ops, torch.bfloat16, 4, 2, 64, lengths=[260], cuts=[100, 1, 1, 60, 1],
+                   window=70, boost=(31, 100), qk_norm=False, rotary_dim=0, page_tokens=32)
+    attention_case(ops, torch.bfloat16, 4, 2, 64, lengths=[260], cuts=[100, 1, 1, 60, 1],
+                   window=70, boost=(31, 101), qk_norm=False, rotary_dim=0, page_tokens=32)
