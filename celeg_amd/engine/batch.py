@@ -40,6 +40,7 @@ class StepBatch:
         self.n_tokens = 0
         self.n_seqs = 0
         self.n_logit_rows = 0
+        self.n_real_seqs = 0
         self.max_seg_len = 0
         self.max_context_len = 0
         self.decode_only = False
@@ -79,27 +80,37 @@ class BatchBuilder:
         self._stage = [torch.empty(capacity_ints, dtype=torch.int32, pin_memory=pin)
                        for _ in range(2)]
         self._events = [None, None]
+        self._event_objects = [torch.cuda.Event(), torch.cuda.Event()] \
+            if self.device.type == "cuda" else [None, None]
+        self._iota = np.arange(max(capacity_ints, 1 << 16), dtype=np.int32)
         self._turn = 0
         self.device_buffer = torch.zeros(capacity_ints, dtype=torch.int32, device=self.device)
 
     def build(self, entries: Sequence[StepEntry], updates: Sequence[Sequence[Tuple[int, int, int]]],
               pad_to: Optional[int] = None, null_slot: int = 0,
               update_caps: Optional[Sequence[int]] = None) -> StepBatch:
-        """``pad_to``: for decode-only batches, the fixed number of rows of a captured
-        graph; missing rows are filled with the null slot at position 0."""
+        """``pad_to``: for batches of single rows, the fixed number of rows of a captured
+        graph; missing rows are filled with the null slot at position 0, and logits are
+        produced for every row (wanted or not), so that the layout is the same every time."""
         seg_lens = [len(e.tokens) for e in entries]
         S_real = len(entries)
-        T_real = int(sum(seg_lens))
+        decode_only = all(n == 1 for n in seg_lens)
+        if pad_to is not None and (not decode_only or pad_to < S_real):
+            raise ValueError("only batches of single rows can be padded, and only upwards")
+        T_real = S_real if decode_only else int(sum(seg_lens))
         S = S_real if pad_to is None else pad_to
         T = T_real if pad_to is None else pad_to
-        want_rows: List[int] = []
-        row = 0
-        for e, n in zip(entries, seg_lens):
-            for w in e.want:
-                if not 0 <= int(w) < n:
-                    raise ValueError(f"wanted place {w} is outside the entry's {n} tokens")
-                want_rows.append(row + int(w))
-            row += n
+        if pad_to is not None:
+            want_rows = list(range(T))
+        else:
+            want_rows = []
+            row = 0
+            for e, n in zip(entries, seg_lens):
+                for w in e.want:
+                    if not 0 <= int(w) < n:
+                        raise ValueError(f"wanted place {w} is outside the entry's {n} tokens")
+                    want_rows.append(row + int(w))
+                row += n
         R = len(want_rows)
         if update_caps is None:
             update_caps = [len(u) for u in updates]
@@ -123,27 +134,31 @@ class BatchBuilder:
         token_ids, positions = arr("token_ids"), arr("positions")
         token_seq, token_slot = arr("token_seq"), arr("token_slot")
         cu, seq_slot, seq_start = arr("cu_seqlens"), arr("seq_slot"), arr("seq_start")
-        row = 0
-        cu[0] = 0
-        for i, (e, n) in enumerate(zip(entries, seg_lens)):
-            token_ids[row:row + n] = np.asarray(e.tokens, dtype=np.int32)
-            positions[row:row + n] = np.arange(e.start_pos, e.start_pos + n, dtype=np.int32)
-            token_seq[row:row + n] = i
-            token_slot[row:row + n] = e.slot
-            seq_slot[i] = e.slot
-            seq_start[i] = e.start_pos
-            row += n
-            cu[i + 1] = row
-        for i in range(S_real, S):          # padding rows of a fixed-size decode batch
-            token_ids[row] = 0
-            positions[row] = 0
-            token_seq[row] = i
-            token_slot[row] = null_slot
-            seq_slot[i] = null_slot
-            seq_start[i] = 0
-            row += 1
-            cu[i + 1] = row
-        arr("logit_rows")[:] = np.asarray(want_rows, dtype=np.int32)
+        if decode_only:
+            token_ids[:S_real] = [e.tokens[0] for e in entries]
+            positions[:S_real] = [e.start_pos for e in entries]
+            token_slot[:S_real] = [e.slot for e in entries]
+            token_ids[S_real:] = 0
+            positions[S_real:] = 0
+            token_slot[S_real:] = null_slot
+            token_seq[:] = self._iota[:T]
+            cu[:] = self._iota[:S + 1]
+            seq_slot[:] = token_slot
+            seq_start[:] = positions
+        else:
+            row = 0
+            cu[0] = 0
+            for i, (e, n) in enumerate(zip(entries, seg_lens)):
+                token_ids[row:row + n] = e.tokens
+                positions[row:row + n] = self._iota[e.start_pos:e.start_pos + n] \
+                    if e.start_pos + n <= self._iota.size else np.arange(e.start_pos, e.start_pos + n)
+                token_seq[row:row + n] = i
+                token_slot[row:row + n] = e.slot
+                seq_slot[i] = e.slot
+                seq_start[i] = e.start_pos
+                row += n
+                cu[i + 1] = row
+        arr("logit_rows")[:] = want_rows
         for g, u in enumerate(updates):
             a = arr(f"updates{g}")
             a[0] = len(u)
@@ -151,15 +166,16 @@ class BatchBuilder:
                 a[1:1 + 3 * len(u)] = np.asarray(u, dtype=np.int32).reshape(-1)
         self.device_buffer[:total].copy_(self._stage[turn][:total], non_blocking=True)
         if self.device.type == "cuda":
-            ev = torch.cuda.Event()
+            ev = self._event_objects[turn]
             ev.record()
             self._events[turn] = ev
 
         b = StepBatch()
         b.n_tokens, b.n_seqs, b.n_logit_rows = T, S, R
+        b.n_real_seqs = S_real
         b.max_seg_len = max(seg_lens) if seg_lens else 0
         b.max_context_len = max((e.start_pos + n for e, n in zip(entries, seg_lens)), default=0)
-        b.decode_only = all(n == 1 for n in seg_lens)
+        b.decode_only = decode_only
 
         def dev(name):
             off, count = layout[name]

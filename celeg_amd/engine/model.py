@@ -60,6 +60,11 @@ class Model:
             if used and layer not in writes_somewhere and self._mixer(layer).kv_need() is not None:
                 self._mixer(layer).set_reads_foreign_kv()
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a recorded step of this model may be replayed from a HIP graph."""
+        return all(part.graph_safe for _, part in self.named_parts())
+
     def named_parts(self) -> List[Tuple[str, Part]]:
         out = [("embedding", self.embedding)]
         for i, block in enumerate(self.blocks):

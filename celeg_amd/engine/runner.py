@@ -66,6 +66,8 @@ class ModelRunner:
                                     pin=torch.device(rt.device).type == "cuda")
         self.steps_run = 0
         self.use_graphs = True
+        self._graphs: Dict[int, tuple] = {}
+        self._buckets = sorted({min(1 << i, S) for i in range(0, 12)})
         self.last_batch: Optional[StepBatch] = None
 
     # ------------------------------------------------------------------ checks
@@ -88,8 +90,12 @@ class ModelRunner:
             if e.start_pos < 0 or e.start_pos + n > self.cache.max_context:
                 raise ValueError(f"context limit reached: position {e.start_pos + n} exceeds "
                                  f"{self.cache.max_context}")
-            toks = np.asarray(e.tokens)
-            if toks.min() < 0 or toks.max() >= vocab:
+            if n == 1:
+                in_range = 0 <= e.tokens[0] < vocab
+            else:
+                toks = np.asarray(e.tokens)
+                in_range = toks.min() >= 0 and toks.max() < vocab
+            if not in_range:
                 raise ValueError(f"step: token id out of range [0, {vocab})")
             if not self.cache.covers(e.slot, e.start_pos, n):
                 raise ValueError(f"step: the pages of slot {e.slot} do not cover positions "
@@ -105,6 +111,8 @@ class ModelRunner:
         and of each entry's ``want``.  The tensor is a view of a reused buffer: it holds
         until the next step."""
         self._validate(entries)
+        if self._graph_applies(entries):
+            return self._step_from_graph(entries)
         updates = self.cache.drain_table_updates()
         batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
         self._apply_table_updates(batch)
@@ -112,6 +120,64 @@ class ModelRunner:
         logits = self.model.forward(batch, self.rt)
         self.steps_run += 1
         return logits
+
+    # ------------------------------------------------------------------ captured decode steps
+    # A step in which every request brings one token and wants its logits is launch-bound:
+    # it is captured once per batch-size bucket as a HIP graph and replayed (the reference
+    # captures its decode step likewise, src/backend/cuda/model/execution.cu:168-246).
+    # Rows that pad the batch to the bucket use the null slot and the spare page, so they
+    # touch no request's cache.  Capture and its warm-up run on such padding rows only:
+    # a request's state is never advanced twice.
+    def _graph_applies(self, entries: Sequence[StepEntry]) -> bool:
+        if not self.use_graphs or torch.device(self.rt.device).type != "cuda" \
+                or not self.model.graph_safe:
+            return False
+        if len(entries) > self._buckets[-1]:
+            return False
+        return all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+
+    def _step_from_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        S = len(entries)
+        bucket = next(b for b in self._buckets if b >= S)
+        caps = [bucket + 8] * len(self.cache.groups)
+        captured = self._graphs.get(bucket)
+        if captured is None or captured[2] != self.rt.ws.generation:
+            captured = self._capture(bucket, caps)
+        updates = self.cache.drain_table_updates()
+        for g, u in enumerate(updates):
+            if len(u) > caps[g]:           # a burst (a large reservation): ship it on its own
+                self._ship_table_updates(g, u)
+                updates[g] = []
+        batch = self.builder.build(entries, updates, pad_to=bucket,
+                                   null_slot=self.cache.null_slot, update_caps=caps)
+        self.last_batch = batch
+        captured[0].replay()
+        self.steps_run += 1
+        return captured[1][:S]
+
+    def _capture(self, bucket: int, caps):
+        empty = [[] for _ in self.cache.groups]
+        batch = self.builder.build([], empty, pad_to=bucket, null_slot=self.cache.null_slot,
+                                   update_caps=caps)
+        self._apply_table_updates(batch)
+        self.model.forward(batch, self.rt)          # warm-up: buffers, libraries, heuristics
+        torch.cuda.synchronize(self.rt.device)
+        graph = torch.cuda.CUDAGraph()
+        self.rt.ws.frozen = True
+        try:
+            with torch.cuda.graph(graph):
+                self._apply_table_updates(batch)
+                logits = self.model.forward(batch, self.rt)
+        finally:
+            self.rt.ws.frozen = False
+        captured = (graph, logits, self.rt.ws.generation)
+        self._graphs[bucket] = captured
+        return captured
+
+    def _ship_table_updates(self, group: int, updates) -> None:
+        flat = torch.tensor([len(updates)] + [v for u in updates for v in u], dtype=torch.int32)
+        self.rt.ops.apply_table_updates(self.cache.groups[group].table, flat.to(self.rt.device),
+                                        len(updates))
 
     def _apply_table_updates(self, batch: StepBatch) -> None:
         for g, (upd, cap) in enumerate(zip(batch.table_updates, batch.table_update_caps)):

@@ -22,6 +22,8 @@ from .base import KVNeed, Mixer, WeightSpec, build_part, register_part
 
 
 class GqaAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         p = self.params

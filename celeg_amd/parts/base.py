@@ -68,6 +68,13 @@ class Runtime:
 
 
 class Part:
+    # True if ``forward`` only enqueues device work whose arguments do not depend on the
+    # step's contents (every per-step number is read from the batch's device arrays), so
+    # that a recorded step can be replayed from a HIP graph.  A part that plans on the
+    # host (reads ``batch.host``, loops over requests in Python) must leave this False;
+    # a model with such a part is never replayed from a graph.
+    graph_safe = False
+
     def __init__(self, spec: PartSpec):
         self.spec = spec
         self.params = dict(spec.params)

@@ -11,6 +11,8 @@ from .base import Embedding, Head, WeightSpec, register_part
 
 
 class TokenEmbedding(Embedding):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.vocab = int(self.params["vocab"])
@@ -30,6 +32,7 @@ class TokenEmbedding(Embedding):
 
 class TiedHead(Head):
     """Uses the embedding table; wants no tensor of its own."""
+    graph_safe = True
 
     def __init__(self, spec):
         super().__init__(spec)
@@ -41,6 +44,8 @@ class TiedHead(Head):
 
 
 class LinearHead(Head):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.vocab = int(self.params["vocab"])

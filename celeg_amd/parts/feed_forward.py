@@ -11,6 +11,8 @@ from .base import FeedForward, WeightSpec, register_part
 
 
 class SwiGlu(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.width = int(self.params["width"])

@@ -7,6 +7,8 @@ from .base import Norm, WeightSpec, register_part
 
 
 class RmsNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.width = int(self.params["width"])

@@ -22,6 +22,8 @@ from .base import PositionEncoding, register_part
 
 
 class Rope(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.theta = float(self.params["theta"])
@@ -45,6 +47,8 @@ class Rope(PositionEncoding):
 
 
 class NoPosition(PositionEncoding):
+    graph_safe = True
+
     def tables(self, rt):
         return {"inv_freq": None, "rotary_dim": 0}
 

@@ -24,6 +24,8 @@ from .base import Mixer, StateNeed, WeightSpec, register_part
 
 
 class ShortConv(Mixer):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.width = int(self.params["width"])

@@ -70,3 +70,29 @@ def test_host_logic_with_kernel_double(model_folders, name, mode):
     from cpu_ops import CpuOps
     run_mode(model_folders, name, "float32", mode, "cpu", ops=CpuOps(),
              subset=["r0", "r1", "r5"] if mode != "mixed" else None)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_steps_equal_eager_steps(model_folders, dtype):
+    """Decode steps replayed from a captured graph against the same steps run eagerly:
+    several replays with other work (portions, other batch sizes) between them, every
+    replay checked."""
+    from celeg_amd.engine import load_model
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders("B", storage, WEIGHT_STD)
+    reqs = requests_of("B")
+    steps = mixed_schedule(reqs, max_live=3, seed=4, decode_tail=20)
+    out = {}
+    for use_graphs in (False, True):
+        lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16,
+                        max_requests=4, max_batched_tokens=256)
+        lm.runner.use_graphs = use_graphs
+        out[use_graphs] = EngineDriver(lm).run(steps)
+        if use_graphs:
+            assert lm.runner._graphs, "no decode step was replayed from a graph"
+    for rid in reqs:
+        if dtype == "float32":
+            assert torch.equal(out[True][rid], out[False][rid])
+        else:
+            assert_close(out[True][rid], out[False][rid].double(), dtype, f"graph/{rid}")

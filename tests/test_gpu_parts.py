@@ -236,6 +236,7 @@ def test_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path):
     lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2,
                     max_batched_tokens=64)
     assert [n.name for _, n in lm.cache.layout.states] == ["sum", "count", "sum", "count"]
+    assert not lm.model.graph_safe      # the toy plans on the host: its steps are never replayed
     got = EngineDriver(lm).run(portions_schedule(reqs))
     got2 = EngineDriver(lm).run(portions_schedule(dict(reversed(list(reqs.items())))))   # slots reused
     for rid, toks in reqs.items():
