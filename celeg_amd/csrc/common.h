@@ -24,17 +24,11 @@ __device__ __forceinline__ T from_float(float x);
 template <>
 __device__ __forceinline__ float from_float<float>(float x) { return x; }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even (gfx950 converts in hardware: v_cvt_pk_bf16_f32)
 template <>
 __device__ __forceinline__ bf16 from_float<bf16>(float x) {
-    uint32_t u = __float_as_uint(x);
     bf16 r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        r.bits = static_cast<uint16_t>((u >> 16) | 0x0040u);
-    } else {
-        u += 0x7fffu + ((u >> 16) & 1u);
-        r.bits = static_cast<uint16_t>(u >> 16);
-    }
+    r.bits = __builtin_bit_cast(uint16_t, static_cast<__bf16>(x));
     return r;
 }
 

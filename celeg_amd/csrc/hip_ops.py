@@ -45,6 +45,7 @@ class HipOps:
         self.attention_impl = "auto"
         self.decode_split_keys = None      # None: chosen from the number of rows
         self._decode_ws = None
+        self._retired = []
 
     # ------------------------------------------------------------------ plumbing
     def _lib(self, module: str) -> ctypes.CDLL:
@@ -325,6 +326,8 @@ class HipOps:
         n_splits = (max_context + split_keys - 1) // split_keys
         need = T * heads * n_splits * (head_dim + 2)
         if self._decode_ws is None or self._decode_ws.numel() < need:
+            if self._decode_ws is not None:
+                self._retired.append(self._decode_ws)   # recorded graphs may still point at it
             self._decode_ws = torch.empty(need, dtype=torch.float32, device=q.device)
         ws_o = self._decode_ws[:T * heads * n_splits * head_dim]
         ws_ml = self._decode_ws[T * heads * n_splits * head_dim:need]
@@ -364,3 +367,130 @@ class HipOps:
             _ptr(seen), _c_size_t(seen.stride(0)), _c_int(seen.shape[0]), _c_int(seen.shape[1]),
             _ptr(token_ids), _ptr(token_slot), _c_int(n), self._stream())
         self._check(code, "mark_seen")
+
+    # ------------------------------------------------------------------ fused skinny products
+    has_fused_linear = True
+    _EPILOGUES = {"store": 0, "store_f32": 1, "residual": 2, "swiglu": 3, "conv": 4}
+
+    def fused_linear_ok(self, rows: int, *inner_sizes: int) -> bool:
+        """Whether the fused skinny product takes ``rows`` rows and these inner sizes."""
+        return 0 < rows <= 64 and all(k > 0 and k % 8 == 0 for k in inner_sizes)
+
+    def embed_stats(self, table, token_ids, out, stats):
+        """Embedding gather that also leaves every row's sum of squares in ``stats[0, :rows]``."""
+        self._dev(table, "table", torch.bfloat16); self._dev(token_ids, "token_ids", torch.int32)
+        self._dev(out, "out", torch.float32); self._dev(stats, "stats", torch.float32)
+        rows, width = out.shape
+        if table.shape[1] != width or token_ids.numel() != rows or stats.shape[1] < rows:
+            raise KernelError("embed_stats: shapes do not fit")
+        code = self._lib("gemv_fused").celeg_embed_stats(
+            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(stats), _c_int(rows), _c_int(width),
+            _c_int(table.shape[0]), self._stream())
+        self._check(code, "embed_stats")
+
+    def fused_linear(self, a, w, out, *, epilogue="store", norm_weight=None, eps=0.0, stats=None,
+                     stat_blocks=0, rows=None, bias=None, stats_out=None, conv=None, n_rows=None):
+        """out = epilogue(prologue(a) w^T) for up to 64 rows, bfloat16 weights.
+
+        ``a``: bfloat16 rows [M, K], or, with ``norm_weight``, the 32-bit residual stream,
+        normalised on the fly (``stats[:stat_blocks]`` holding partial sums of squares of its
+        rows if ``stat_blocks`` > 0).  ``rows`` picks rows of ``a``.  Epilogues: "store"
+        (bfloat16 [M, N]), "store_f32", "residual" (``out`` is the stream, [M, N] 32-bit,
+        added to in place; ``stats_out`` [ceil(N/16), >= M] receives partial sums of squares
+        of the new rows), "swiglu" (``w`` is [2N, K]: gate rows then up rows), "conv"
+        (``w`` is [3N, K]: B, C, x rows; ``conv`` = (taps [N, L], bias or None, state
+        [slots, L, N], seq_slot [M]); one new token per request)."""
+        if epilogue not in self._EPILOGUES:
+            raise KernelError(f"fused_linear: unknown epilogue '{epilogue}'")
+        self._dev(w, "w", torch.bfloat16)
+        streams = {"swiglu": 2, "conv": 3}.get(epilogue, 1)
+        K = w.shape[1]
+        if w.shape[0] % streams:
+            raise KernelError("fused_linear: weight rows do not split into the epilogue's streams")
+        N = w.shape[0] // streams
+        M = n_rows if n_rows is not None else (rows.numel() if rows is not None else a.shape[0])
+        if not self.fused_linear_ok(M, K):
+            raise KernelError(f"fused_linear: {M} rows with inner size {K} are not supported "
+                              "(1..64 rows, inner size a multiple of 8)")
+        self._dev(a, "a", contiguous=False)
+        lda = self._rows(a, "a")
+        if a.shape[1] != K or (rows is None and a.shape[0] < M):
+            raise KernelError("fused_linear: a does not fit the weights")
+        if norm_weight is not None:
+            if a.dtype != torch.float32:
+                raise KernelError("fused_linear: the normalising prologue reads a 32-bit stream")
+            self._dev(norm_weight, "norm_weight", torch.float32)
+            if norm_weight.numel() != K:
+                raise KernelError("fused_linear: norm weight must have the inner size")
+            if epilogue == "residual":
+                raise KernelError("fused_linear: this combination is not built")
+        else:
+            if a.dtype != torch.bfloat16:
+                raise KernelError("fused_linear: rows must be bfloat16 (or 32-bit with a norm weight)")
+            if epilogue in ("swiglu", "conv"):
+                raise KernelError("fused_linear: this combination is not built")
+        if lda % 8:
+            raise KernelError("fused_linear: the row stride of a must be a multiple of 8")
+        if rows is not None:
+            self._dev(rows, "rows", torch.int32)
+        out_dtype = torch.float32 if epilogue in ("store_f32", "residual") else torch.bfloat16
+        self._dev(out, "out", out_dtype, contiguous=False)
+        if out.shape[0] < M or out.shape[1] != N:
+            raise KernelError(f"fused_linear: out must be [{M}, {N}], got {tuple(out.shape)}")
+        if bias is not None:
+            self._dev(bias, "bias", torch.float32)
+            if bias.numel() != streams * N:
+                raise KernelError("fused_linear: bias does not fit")
+        prm = _GemvParams()
+        prm.a, prm.lda = a.data_ptr(), lda
+        prm.rows = rows.data_ptr() if rows is not None else None
+        prm.norm_w = norm_weight.data_ptr() if norm_weight is not None else None
+        prm.eps = eps
+        if norm_weight is not None and stat_blocks > 0:
+            self._dev(stats, "stats", torch.float32)
+            if stats.shape[0] < stat_blocks:
+                raise KernelError("fused_linear: fewer partial sums than stat_blocks")
+            prm.stats, prm.n_stat_blocks, prm.stats_ld = stats.data_ptr(), stat_blocks, stats.stride(0)
+        prm.w, prm.stream_rows = w.data_ptr(), N
+        prm.bias = bias.data_ptr() if bias is not None else None
+        prm.M, prm.N, prm.K = M, N, K
+        prm.out, prm.ldo = out.data_ptr(), self._rows(out, "out")
+        if epilogue == "residual" and stats_out is not None:
+            self._dev(stats_out, "stats_out", torch.float32)
+            if stats_out.shape[0] < (N + 15) // 16 or stats_out.shape[1] < M:
+                raise KernelError("fused_linear: stats_out must be [ceil(N/16), >= rows]")
+            prm.stats_out, prm.stats_ld_out = stats_out.data_ptr(), stats_out.stride(0)
+        if epilogue == "conv":
+            taps_w, conv_bias, state, seq_slot = conv
+            self._dev(taps_w, "conv taps", torch.float32); self._dev(seq_slot, "seq_slot", torch.int32)
+            self._dev(state, "state", torch.float32, contiguous=False)
+            L = taps_w.shape[1]
+            if taps_w.shape[0] != N or state.shape[1:] != (L, N) or state.stride(1) != N \
+                    or state.stride(2) != 1 or seq_slot.numel() < M:
+                raise KernelError("fused_linear: convolution operands do not fit")
+            prm.conv_w = taps_w.data_ptr()
+            prm.conv_b = conv_bias.data_ptr() if conv_bias is not None else None
+            prm.state, prm.state_slot_stride = state.data_ptr(), state.stride(0)
+            prm.seq_slot, prm.taps = seq_slot.data_ptr(), L
+        tiles, chunks = (N + 15) // 16, (K + 63) // 64
+        waves = 8 if (tiles < 512 and M <= 32 and chunks >= 16) else 4
+        code = self._lib("gemv_fused").celeg_gemv_fused(
+            ctypes.byref(prm), _c_int(1 if norm_weight is not None else 0),
+            _c_int(self._EPILOGUES[epilogue]), _c_int(waves), self._stream())
+        self._check(code, f"fused_linear ({epilogue})")
+        return out
+
+
+class _GemvParams(ctypes.Structure):
+    """Mirror of ``GemvParams`` in gemv_fused.hip."""
+    _fields_ = [
+        ("a", ctypes.c_void_p), ("lda", ctypes.c_int), ("rows", ctypes.c_void_p),
+        ("norm_w", ctypes.c_void_p), ("eps", ctypes.c_float), ("stats", ctypes.c_void_p),
+        ("n_stat_blocks", ctypes.c_int), ("stats_ld", ctypes.c_int),
+        ("w", ctypes.c_void_p), ("stream_rows", ctypes.c_int), ("bias", ctypes.c_void_p),
+        ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
+        ("out", ctypes.c_void_p), ("ldo", ctypes.c_int), ("stats_out", ctypes.c_void_p),
+        ("stats_ld_out", ctypes.c_int),
+        ("conv_w", ctypes.c_void_p), ("conv_b", ctypes.c_void_p), ("state", ctypes.c_void_p),
+        ("state_slot_stride", ctypes.c_size_t), ("seq_slot", ctypes.c_void_p), ("taps", ctypes.c_int),
+    ]

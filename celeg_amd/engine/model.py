@@ -129,12 +129,16 @@ class Model:
         T, R = batch.n_tokens, batch.n_logit_rows
         width, vocab = self.spec.hidden_size, self.spec.vocab_size
         h = rt.ws.buf("hidden", (T, width), torch.float32)
-        self.embedding.forward(batch.token_ids, h, rt)
+        rt.stream_stat_blocks = 0
+        self.embedding.forward(batch.token_ids, h, rt, batch=batch)
         delta = None
         for i, step in enumerate(self.spec.order):
             delta = self.blocks[step.layer].forward(h, delta, batch, self._caches[i], rt)
         logits = rt.ws.buf("logits", (R, vocab), torch.float32)
         if R == 0:
+            return logits
+        if delta is None and hasattr(self.head, "forward_fused") and \
+                self.head.forward_fused(h, self.final_norm, batch, logits, rt, self.embedding):
             return logits
         normed = rt.ws.buf("final_normed", (R, width), rt.dtype)
         self.final_norm.forward(h, normed, rt, delta=delta, rows=batch.logit_rows)

@@ -19,6 +19,7 @@ import torch
 
 from ..config.spec import PartSpec
 from .base import KVNeed, Mixer, WeightSpec, build_part, register_part
+from .fused import fused_rows_ok, linear_into_stream, norm_linear
 
 
 class GqaAttention(Mixer):
@@ -84,21 +85,47 @@ class GqaAttention(Mixer):
 
     # -- work
     def forward(self, x, batch, cache, rt):
+        attended = self._project_and_attend(x, None, batch, cache, rt)
+        out = rt.ws.buf("mixer_out", (x.shape[0], self.width), rt.dtype)
+        rt.ops.linear(attended, self.w_o, out)
+        return out
+
+    def forward_fused(self, h, norm, batch, cache, rt) -> bool:
+        """h += mixer(norm(h)) with the norm folded into the q/k/v product and the residual
+        addition into the output product.  False if the step cannot take the fused path."""
+        q_width = self.heads * self.head_dim
+        w_in = self.w_qkv if cache.writes_kv else self.w_q
+        if not fused_rows_ok(rt, batch, self.width, q_width) \
+                or (w_in.dtype, self.w_o.dtype) != (rt.dtype,) * 2:
+            return False
+        attended = self._project_and_attend(h, norm, batch, cache, rt)
+        linear_into_stream(rt, attended, self.w_o, h)
+        return True
+
+    def _project_and_attend(self, x, norm, batch, cache, rt):
+        """``norm`` None: ``x`` are normalised rows; else ``x`` is the residual stream and the
+        norm is applied inside the product."""
         T = x.shape[0]
         q_width, kv_width = self.heads * self.head_dim, self.kv_heads * self.head_dim
         writes = cache.writes_kv
         if writes and not self.own_kv:
             raise RuntimeError("gqa_attention: built without key/value projections but asked "
                                "to write a cache")
+
+        def project(w, out):
+            if norm is None:
+                rt.ops.linear(x, w, out)
+            else:
+                norm_linear(rt, x, norm, w, out)
         if writes:
             qkv = rt.ws.buf("attn_qkv", (T, q_width + 2 * kv_width), rt.dtype)
-            rt.ops.linear(x, self.w_qkv, qkv)
+            project(self.w_qkv, qkv)
             q = qkv[:, :q_width]
             k = qkv[:, q_width:q_width + kv_width]
             v = qkv[:, q_width + kv_width:]
         else:
             q = rt.ws.buf("attn_q", (T, q_width), rt.dtype)
-            rt.ops.linear(x, self.w_q, q)
+            project(self.w_q, q)
             k = v = None
         tables = self.position.tables(rt)
         rt.ops.qk_norm_rope_store(
@@ -108,9 +135,7 @@ class GqaAttention(Mixer):
         attended = rt.ws.buf("attn_out", (T, q_width), rt.dtype)
         rt.ops.paged_attention(q, attended, self.heads, self.kv_heads, self.head_dim,
                                self.scale, self.window, batch, cache.kv)
-        out = rt.ws.buf("mixer_out", (T, self.width), rt.dtype)
-        rt.ops.linear(attended, self.w_o, out)
-        return out
+        return attended
 
 
 register_part("mixer", "gqa_attention", GqaAttention)

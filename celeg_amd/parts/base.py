@@ -117,7 +117,7 @@ class PositionEncoding(Part):
 
 
 class Embedding(Part):
-    def forward(self, token_ids, out, rt):
+    def forward(self, token_ids, out, rt, batch=None):
         raise NotImplementedError
 
 

@@ -12,6 +12,7 @@ A block arrangement is a class with ``__init__(layer_spec)`` that builds its par
 from __future__ import annotations
 
 from .base import build_part, register_part
+from .norm import RmsNorm
 
 
 class PreNormBlock:
@@ -31,8 +32,21 @@ class PreNormBlock:
         Returns the feed-forward's output, which the caller's next norm adds."""
         T, width = h.shape
         normed = rt.ws.buf("normed", (T, width), rt.dtype)
-        self.mixer_norm.forward(h, normed, rt, delta=delta)
-        mixed = self.mixer.forward(normed, batch, cache, rt)
+        # Few rows: parts that can, take the norm in front of them and the addition behind
+        # them into their own products and write the stream themselves.
+        fusable = isinstance(self.mixer_norm, RmsNorm) and isinstance(self.ffn_norm, RmsNorm)
+        mixed = delta
+        if not (fusable and delta is None and hasattr(self.mixer, "forward_fused")
+                and self.mixer.forward_fused(h, self.mixer_norm, batch, cache, rt)):
+            rt.stream_stat_blocks = 0
+            self.mixer_norm.forward(h, normed, rt, delta=delta)
+            mixed = self.mixer.forward(normed, batch, cache, rt)
+        else:
+            mixed = None
+        if fusable and mixed is None and hasattr(self.ffn, "forward_fused") \
+                and self.ffn.forward_fused(h, self.ffn_norm, batch, rt):
+            return None
+        rt.stream_stat_blocks = 0
         self.ffn_norm.forward(h, normed, rt, delta=mixed)
         return self.ffn.forward(normed, batch, rt)
 

@@ -7,7 +7,11 @@ E_out = E when the head is tied, else lm_head
 src/model/inference/layer_bindings.cpp:24-95).  Logits leave in 32-bit."""
 from __future__ import annotations
 
+import torch
+
 from .base import Embedding, Head, WeightSpec, register_part
+from .fused import fused_rows_ok, norm_linear, stream_stats
+from .norm import RmsNorm
 
 
 class TokenEmbedding(Embedding):
@@ -25,8 +29,14 @@ class TokenEmbedding(Embedding):
     def load(self, tensors, rt):
         self.table = tensors["table"].contiguous()
 
-    def forward(self, token_ids, out, rt):
-        rt.ops.embed(self.table, token_ids, out)
+    def forward(self, token_ids, out, rt, batch=None):
+        if batch is not None and self.table.dtype == torch.bfloat16 \
+                and fused_rows_ok(rt, batch, self.width):
+            # few rows: leave every row's sum of squares for the first norm
+            rt.ops.embed_stats(self.table, token_ids, out, stream_stats(rt, self.width))
+            rt.stream_stat_blocks = 1
+        else:
+            rt.ops.embed(self.table, token_ids, out)
         return out
 
 
@@ -41,6 +51,9 @@ class TiedHead(Head):
     def forward(self, x, out, rt, embedding=None):
         rt.ops.linear(x, embedding.table, out)
         return out
+
+    def forward_fused(self, h, norm, batch, out, rt, embedding=None) -> bool:
+        return _head_fused(h, norm, batch, out, rt, embedding.table)
 
 
 class LinearHead(Head):
@@ -61,6 +74,19 @@ class LinearHead(Head):
     def forward(self, x, out, rt, embedding=None):
         rt.ops.linear(x, self.weight, out)
         return out
+
+    def forward_fused(self, h, norm, batch, out, rt, embedding=None) -> bool:
+        return _head_fused(h, norm, batch, out, rt, self.weight)
+
+
+def _head_fused(h, norm, batch, out, rt, weight) -> bool:
+    """Final norm and output product in one kernel for few wanted rows, 32-bit logits."""
+    R = batch.n_logit_rows
+    if not (isinstance(norm, RmsNorm) and weight.dtype == torch.bfloat16
+            and fused_rows_ok(rt, batch, h.shape[1]) and 0 < R <= 64):
+        return False
+    norm_linear(rt, h, norm, weight, out, epilogue="store_f32", rows=batch.logit_rows, n_rows=R)
+    return True
 
 
 register_part("embedding", "embedding", TokenEmbedding)

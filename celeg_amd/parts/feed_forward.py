@@ -8,6 +8,7 @@ from __future__ import annotations
 import torch
 
 from .base import FeedForward, WeightSpec, register_part
+from .fused import fused_rows_ok, linear_into_stream, norm_linear
 
 
 class SwiGlu(FeedForward):
@@ -42,6 +43,18 @@ class SwiGlu(FeedForward):
         out = rt.ws.buf("ffn_out", (T, self.width), rt.dtype)
         rt.ops.linear(act, self.w_down, out)
         return out
+
+
+    def forward_fused(self, h, norm, batch, rt) -> bool:
+        """h += ffn(norm(h)): the norm and the SwiGLU folded into the first product, the
+        residual addition into the second.  False if the step cannot take the fused path."""
+        if not fused_rows_ok(rt, batch, self.width, self.ff) \
+                or (self.w_gate_up.dtype, self.w_down.dtype) != (rt.dtype,) * 2:
+            return False
+        act = rt.ws.buf("ffn_act", (batch.n_tokens, self.ff), rt.dtype)
+        norm_linear(rt, h, norm, self.w_gate_up, act, epilogue="swiglu")
+        linear_into_stream(rt, act, self.w_down, h)
+        return True
 
 
 register_part("ffn", "swiglu", SwiGlu)

@@ -1,0 +1,46 @@
+"""Helpers of the fused path for steps of few rows (decode and small portions).
+
+A step of up to 64 rows is bound by the number of dependent kernels, so the parts
+fold their neighbours into their matrix products (``HipOps.fused_linear``): the norm in
+front of a product is applied to the rows of the 32-bit residual stream as they are
+read, and a product that ends a sub-block adds its result into the stream itself.
+Whoever writes the stream this way also leaves partial sums of squares of its rows
+("stream statistics"), which the next norm reads instead of walking the rows again.
+
+``rt.stream_stat_blocks`` says how many partial sums are valid (0: none; the prologue
+then recomputes the sums).  Anything else that writes the stream resets it to 0.
+"""
+from __future__ import annotations
+
+import torch
+
+STAT_COLUMNS = 64   # most rows of a fused step
+
+
+def fused_rows_ok(rt, batch, *inner_sizes) -> bool:
+    """Whether this step's rows can take the fused path through products with these
+    inner sizes."""
+    ops = rt.ops
+    return (rt.dtype == torch.bfloat16 and getattr(ops, "has_fused_linear", False)
+            and getattr(rt, "use_fused", True)
+            and ops.fused_linear_ok(batch.n_tokens, *inner_sizes))
+
+
+def stream_stats(rt, width: int) -> torch.Tensor:
+    return rt.ws.buf("stream_stats", ((width + 15) // 16, STAT_COLUMNS), torch.float32)
+
+
+def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None, **kw):
+    """out = epilogue(norm(h) w^T), the norm applied while the rows of ``h`` are read."""
+    blocks = getattr(rt, "stream_stat_blocks", 0)
+    return rt.ops.fused_linear(h, w, out, epilogue=epilogue, norm_weight=norm.weight,
+                               eps=norm.eps, stats=stream_stats(rt, h.shape[1]) if blocks else None,
+                               stat_blocks=blocks, rows=rows, n_rows=n_rows, **kw)
+
+
+def linear_into_stream(rt, a, w, h, bias=None):
+    """h += a w^T, leaving the partial sums of squares of the new rows."""
+    stats = stream_stats(rt, h.shape[1])
+    rt.ops.fused_linear(a, w, h, epilogue="residual", bias=bias, stats_out=stats)
+    rt.stream_stat_blocks = (h.shape[1] + 15) // 16
+    return h

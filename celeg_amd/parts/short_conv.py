@@ -21,6 +21,7 @@ from __future__ import annotations
 import torch
 
 from .base import Mixer, StateNeed, WeightSpec, register_part
+from .fused import fused_rows_ok, linear_into_stream, norm_linear
 
 
 class ShortConv(Mixer):
@@ -68,6 +69,26 @@ class ShortConv(Mixer):
         out = rt.ws.buf("mixer_out", (T, H), rt.dtype)
         rt.ops.linear(y, self.w_out, out, bias=self.b_out)
         return out
+
+
+    def forward_fused(self, h, norm, batch, cache, rt) -> bool:
+        """h += mixer(norm(h)) with the norm, the convolution (for one new token per
+        request) and the residual addition folded into the two products.  False if this
+        step cannot take the fused path (nothing is done then)."""
+        H = self.width
+        if not fused_rows_ok(rt, batch, H) or (self.w_in.dtype, self.w_out.dtype) != (rt.dtype,) * 2:
+            return False
+        T = batch.n_tokens
+        y = rt.ws.buf("conv_y", (T, H), rt.dtype)
+        if batch.decode_only and batch.n_seqs == T:
+            norm_linear(rt, h, norm, self.w_in, y, epilogue="conv", bias=self.b_in,
+                        conv=(self.w_conv, self.b_conv, cache.states["bx"], batch.seq_slot))
+        else:
+            bcx = rt.ws.buf("conv_bcx", (T, 3 * H), rt.dtype)
+            norm_linear(rt, h, norm, self.w_in, bcx, bias=self.b_in)
+            rt.ops.short_conv(bcx, self.w_conv, self.b_conv, cache.states["bx"], y, batch)
+        linear_into_stream(rt, y, self.w_out, h, bias=self.b_out)
+        return True
 
 
 register_part("mixer", "short_conv", ShortConv)

@@ -1,0 +1,154 @@
+"""The fused skinny matrix products alone, against torch: every prologue and epilogue, at
+row counts from 1 to 64 and sizes that are no multiple of the tiles."""
+import pytest
+import torch
+
+import plain_lfm2 as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF = torch.bfloat16
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from celeg_amd.csrc.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+def randn(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, ref, rel=1.5e-2):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    bound = rel * max(1.0, float(ref.abs().max()))
+    assert float((got - ref).abs().max()) <= bound, float((got - ref).abs().max())
+
+
+SHAPES = [(1, 331, 96), (7, 64, 64), (8, 1024, 1024), (16, 130, 200), (17, 48, 4608),
+          (33, 1000, 352), (64, 272, 1024)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_plain_rows_store_and_32bit_store_with_bias(ops, M, N, K):
+    a = randn(M, K, seed=1, dtype=BF)
+    w = randn(N, K, seed=2, scale=0.1, dtype=BF)
+    b = randn(N, seed=3)
+    ref = a.double() @ w.double().T + b.double()
+    out = torch.empty(M, N, dtype=BF, device=DEV)
+    ops.fused_linear(a, w, out, bias=b)
+    close(out, ref)
+    out32 = torch.empty(M, N, device=DEV)
+    ops.fused_linear(a, w, out32, epilogue="store_f32", bias=b)
+    close(out32, ref, rel=2e-3)
+    # a row alone gives the same 32-bit result as inside the batch, up to the order in
+    # which the wavefronts' partial sums are added (their number depends on the rows)
+    one = torch.empty(1, N, device=DEV)
+    ops.fused_linear(a[M // 2:M // 2 + 1], w, one, epilogue="store_f32", bias=b)
+    if M <= 32:
+        assert torch.equal(one[0], out32[M // 2])
+    close(one[0], out32[M // 2], rel=1e-5)
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+@pytest.mark.parametrize("with_stats", [False, True])
+def test_norm_prologue_with_and_without_partial_sums(ops, M, N, K, with_stats):
+    h = randn(M + 3, K, seed=4)
+    nw = 1 + randn(K, seed=5, scale=0.1)
+    w = randn(N, K, seed=6, scale=0.1, dtype=BF)
+    rows = torch.tensor([(3 * i + 1) % (M + 3) for i in range(M)], dtype=torch.int32, device=DEV)
+    eps = 1e-5
+    x = plain.rmsnorm(h.cpu(), nw.cpu(), eps)[rows.long().cpu()].to(BF)
+    ref = x.double() @ w.double().cpu().T
+    stats, blocks = None, 0
+    if with_stats:   # partial sums over 5 uneven column blocks
+        blocks = 5
+        cuts = [0, K // 7, K // 3, K // 2, K - 8, K]
+        stats = torch.zeros(blocks, 80, device=DEV)
+        for j in range(blocks):
+            stats[j, :M + 3] = (h[:, cuts[j]:cuts[j + 1]] ** 2).sum(dim=1)
+    out = torch.empty(M, N, dtype=BF, device=DEV)
+    ops.fused_linear(h, w, out, norm_weight=nw, eps=eps, rows=rows, stats=stats, stat_blocks=blocks)
+    close(out, ref)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (8, 1024, 1024), (20, 200, 352), (64, 96, 4608)])
+def test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, M, N, K):
+    a = randn(M, K, seed=7, dtype=BF)
+    w = randn(N, K, seed=8, scale=0.1, dtype=BF)
+    b = randn(N, seed=9)
+    h = randn(M, N, seed=10)
+    h0 = h.clone()
+    stats = torch.full(((N + 15) // 16, 64), -1.0, device=DEV)
+    ops.fused_linear(a, w, h, epilogue="residual", bias=b, stats_out=stats)
+    delta = (a.double() @ w.double().T + b.double())
+    close(h, h0.double() + delta)
+    # the product enters the sum rounded to bfloat16
+    close(h - h0, delta.to(BF), rel=2e-3)
+    torch.testing.assert_close(stats[:, :M].sum(dim=0), (h ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
+    assert float(stats[:, M:].max()) == -1.0 if M < 64 else True
+
+
+@pytest.mark.parametrize("M,ff,K", [(1, 192, 64), (8, 4608, 1024), (19, 352, 128), (64, 200, 96)])
+def test_swiglu_epilogue(ops, M, ff, K):
+    h = randn(M, K, seed=11)
+    nw = 1 + randn(K, seed=12, scale=0.1)
+    w = randn(2 * ff, K, seed=13, scale=0.2, dtype=BF)
+    x = plain.rmsnorm(h.cpu(), nw.cpu(), 1e-6).to(BF).double()
+    g = (x @ w[:ff].double().cpu().T).to(BF).double()
+    u = (x @ w[ff:].double().cpu().T).to(BF).double()
+    out = torch.empty(M, ff, dtype=BF, device=DEV)
+    ops.fused_linear(h, w, out, epilogue="swiglu", norm_weight=nw, eps=1e-6)
+    close(out, plain.silu(g) * u, rel=2e-2)
+
+
+@pytest.mark.parametrize("M,H,taps,bias", [(1, 64, 3, False), (8, 1024, 3, False), (5, 128, 4, True),
+                                           (33, 96, 1, True), (64, 48, 5, False)])
+def test_conv_epilogue_token_by_token_equals_the_whole_convolution(ops, M, H, taps, bias):
+    """M requests advance one token per call, each in its own slot (in another order than
+    the rows); their outputs over 6 calls equal the plain whole-sequence convolution."""
+    steps = 6
+    nw = 1 + randn(H, seed=14, scale=0.1)
+    w_in = randn(3 * H, H, seed=15, scale=0.2, dtype=BF)
+    b_in = randn(3 * H, seed=16, scale=0.1) if bias else None
+    cw = randn(H, taps, seed=17)
+    cb = randn(H, seed=18) if bias else None
+    hs = randn(steps, M, H, seed=19)
+    state = torch.zeros(M + 2, taps, H, device=DEV)
+    slots = torch.tensor([(M + 1 - i) for i in range(M)], dtype=torch.int32, device=DEV)
+    outs = []
+    for t in range(steps):
+        y = torch.empty(M, H, dtype=BF, device=DEV)
+        ops.fused_linear(hs[t], w_in, y, epilogue="conv", norm_weight=nw, eps=1e-5, bias=b_in,
+                         conv=(cw, cb, state, slots))
+        outs.append(y.double().cpu())
+    got = torch.stack(outs)              # [steps, M, H]
+    for m in range(0, M, max(1, M // 4)):
+        x = plain.rmsnorm(hs[:, m].cpu(), nw.cpu(), 1e-5).to(BF).double()
+        bcx = x @ w_in.double().cpu().T + (b_in.double().cpu() if bias else 0)
+        ref = plain.short_conv(bcx.to(BF), cw.cpu(), cb.cpu() if bias else None)
+        close(got[:, m], ref, rel=2e-2)
+    assert float(state[0].abs().max()) == 0.0          # a slot nobody uses stays zero
+
+
+def test_embed_stats(ops):
+    table = randn(331, 96, seed=20, dtype=BF)
+    ids = torch.tensor([5, 330, 0, 17], dtype=torch.int32, device=DEV)
+    out = torch.empty(4, 96, device=DEV)
+    stats = torch.zeros(6, 64, device=DEV)
+    ops.embed_stats(table, ids, out, stats)
+    assert torch.equal(out, table[ids.long()].float())
+    torch.testing.assert_close(stats[0, :4], (out ** 2).sum(dim=1), rtol=1e-6, atol=1e-6)
+
+
+def test_unsupported_sizes_are_refused(ops):
+    from celeg_amd.csrc.hip_ops import KernelError
+    w = randn(32, 100, dtype=BF)
+    with pytest.raises(KernelError, match="not supported"):
+        ops.fused_linear(randn(4, 100, dtype=BF), w, torch.empty(4, 32, dtype=BF, device=DEV))
+    w = randn(32, 64, dtype=BF)
+    with pytest.raises(KernelError, match="not supported"):
+        ops.fused_linear(randn(65, 64, dtype=BF), w, torch.empty(65, 32, dtype=BF, device=DEV))
+    assert not ops.fused_linear_ok(8, 100) and ops.fused_linear_ok(64, 96)
