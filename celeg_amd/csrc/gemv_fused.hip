@@ -70,151 +70,14 @@ template <int EPI> struct Streams { static constexpr int n = 1; };
 template <> struct Streams<E_SWIGLU> { static constexpr int n = 2; };
 template <> struct Streams<E_CONV> { static constexpr int n = 3; };
 
-template <int MT, int NW, int AMODE, int EPI>
-__global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(const GemvParams p) {
-    constexpr int NS = Streams<EPI>::n;
-    __shared__ floatx4_t red[NW][MT * NS][64];
-    __shared__ float inv_rms[MT * 16];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+// ---- epilogue of one 16-column tile: this lane holds column n0 + lane%16 of rows
+// 4*(lane/16)..+3 of every row tile
+template <int MT, int NS, int EPI>
+__device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&acc)[MT][NS],
+                                              int tile, int lane) {
     const int c16 = lane & 15, q = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    const int K = p.K, M = p.M;
-
-    // ---- A_NORM: 1/rms of every row
-    if (AMODE == A_NORM) {
-        const float* h = static_cast<const float*>(p.a);
-        if (p.stats) {
-            // one wavefront per row; its lanes read the partial sums side by side
-            for (int m = wave; m < MT * 16; m += NW) {
-                float s = 0.f;
-                if (m < M) {
-                    const int src = p.rows ? p.rows[m] : m;
-                    for (int j = lane; j < p.n_stat_blocks; j += 64)
-                        s += p.stats[static_cast<size_t>(j) * p.stats_ld + src];
-                }
-                s = wave_sum(s);
-                if (lane == 0) inv_rms[m] = 1.0f / sqrtf(s / static_cast<float>(K) + p.eps);
-            }
-        } else {
-            // one wavefront per row, rows dealt round robin
-            for (int m = wave; m < MT * 16; m += NW) {
-                float s = 0.f;
-                if (m < M) {
-                    const float* row = h + static_cast<size_t>(p.rows ? p.rows[m] : m) * p.lda;
-                    for (int k = lane; k < K; k += 64) s += row[k] * row[k];
-                }
-                s = wave_sum(s);
-                if (lane == 0) inv_rms[m] = 1.0f / sqrtf(s / static_cast<float>(K) + p.eps);
-            }
-        }
-        __syncthreads();
-    }
-
-    floatx4_t acc[MT][NS];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int s = 0; s < NS; ++s) acc[mt][s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-
-    // rows of A this lane feeds (one per row tile) and their 1/rms
-    size_t a_off[MT];
-    float a_inv[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = min(mt * 16 + c16, M - 1);
-        a_off[mt] = static_cast<size_t>(p.rows ? p.rows[m] : m) * p.lda;
-        a_inv[mt] = AMODE == A_NORM ? inv_rms[mt * 16 + c16 < M ? mt * 16 + c16 : M - 1] : 1.f;
-    }
-    const bf16* wrow[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s)
-        wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + c16, p.N - 1)) * K;
-
-    // K is cut in chunks of 64 which are dealt to the wavefronts.  Inside a chunk, lane
-    // group q holds the k values {q*8..q*8+7} and {32+q*8..32+q*8+7}: each of the two
-    // 16-byte loads of a lane is then side by side with its neighbours' in the row.  U chunks
-    // are loaded before any is multiplied, so that several loads are in flight.
-    constexpr int U = MT == 1 ? 4 : (MT == 2 ? 2 : 1);
-    const int chunks = (K + 63) >> 6;
-    const int c_begin = wave * chunks / NW, c_end = (wave + 1) * chunks / NW;
-    for (int c0 = c_begin; c0 < c_end; c0 += U) {
-        Frag2 wv[U][NS][2];
-        Frag2 av[U][MT][2];          // A_BF16
-        floatx4_t hv[U][MT][4];      // A_NORM
-        floatx4_t nv[U][4];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const bool live = c0 + u < c_end;
-#pragma unroll
-            for (int v = 0; v < 2; ++v) {
-                const int k = (c0 + u) * 64 + v * 32 + q * 8;   // 8 values from here
-                const bool in = live && k + 8 <= K;              // K % 8 == 0
-#pragma unroll
-                for (int s = 0; s < NS; ++s)
-                    wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
-                    if (AMODE == A_BF16) {
-                        av[u][mt][v] = in ? *reinterpret_cast<const Frag2*>(
-                                                static_cast<const bf16*>(p.a) + a_off[mt] + k)
-                                          : Frag2{};
-                    } else {
-                        const float* hr = static_cast<const float*>(p.a) + a_off[mt] + k;
-                        hv[u][mt][2 * v] = in ? *reinterpret_cast<const floatx4_t*>(hr) : floatx4_t{};
-                        hv[u][mt][2 * v + 1] = in ? *reinterpret_cast<const floatx4_t*>(hr + 4) : floatx4_t{};
-                    }
-                }
-                if (AMODE == A_NORM) {
-                    nv[u][2 * v] = in ? *reinterpret_cast<const floatx4_t*>(p.norm_w + k) : floatx4_t{};
-                    nv[u][2 * v + 1] = in ? *reinterpret_cast<const floatx4_t*>(p.norm_w + k + 4) : floatx4_t{};
-                }
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            bf16x4_t af[MT][4];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                if (AMODE == A_BF16) {
-                    af[mt][0] = av[u][mt][0].lo; af[mt][1] = av[u][mt][0].hi;
-                    af[mt][2] = av[u][mt][1].lo; af[mt][3] = av[u][mt][1].hi;
-                } else {
-#pragma unroll
-                    for (int s4 = 0; s4 < 4; ++s4)
-                        af[mt][s4] = __builtin_bit_cast(
-                            bf16x4_t, __builtin_convertvector(hv[u][mt][s4] * a_inv[mt] * nv[u][s4], nbf16x4_t));
-                }
-            }
-#pragma unroll
-            for (int s = 0; s < NS; ++s) {
-                const bf16x4_t bfr[4] = {wv[u][s][0].lo, wv[u][s][0].hi, wv[u][s][1].lo, wv[u][s][1].hi};
-#pragma unroll
-                for (int s4 = 0; s4 < 4; ++s4)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[mt][s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(af[mt][s4], bfr[s4], acc[mt][s], 0, 0, 0);
-            }
-        }
-    }
-
-    // ---- add the wavefronts' partial tiles, in wavefront order
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int s = 0; s < NS; ++s) red[wave][mt * NS + s][lane] = acc[mt][s];
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            floatx4_t t = red[0][mt * NS + s][lane];
-            for (int w = 1; w < NW; ++w) t += red[w][mt * NS + s][lane];
-            acc[mt][s] = t;
-        }
-
-    // ---- epilogue: this lane holds column n of rows 4q..4q+3 of every row tile
-    const int n = n0 + c16;
+    const int M = p.M;
+    const int n = tile * 16 + c16;
     const bool col_ok = n < p.N;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -274,17 +137,243 @@ __global__ __launch_bounds__(NW * 64) void gemv_fused_kernel(const GemvParams p)
                 s += __shfl_xor(s, 8, 64);
                 const int m = mt * 16 + 4 * q + r;
                 if (c16 == 0 && m < M)
-                    p.stats_out[static_cast<size_t>(blockIdx.x) * p.stats_ld_out + m] = s;
+                    p.stats_out[static_cast<size_t>(tile) * p.stats_ld_out + m] = s;
             }
         }
     }
 }
 
-template <int MT, int NW>
-static int launch_mt_nw(const GemvParams& p, int amode, int epi, hipStream_t stream) {
-    dim3 grid((p.N + 15) / 16), block(NW * 64);
-#define CELEG_GEMV(AM, EP)                                                                      \
-    hipLaunchKernelGGL((gemv_fused_kernel<MT, NW, AM, EP>), grid, block, 0, stream, p)
+// A workgroup of TW*KW wavefronts: wavefront (tw, kw) works on column tile
+// blockIdx.x*TW + tw and on the kw-th share of K.  ALDS: the rows of A (normalised, if
+// asked) are put into LDS once per workgroup as bfloat16 and every wavefront reads its
+// operands from there; otherwise every wavefront reads (and normalises) them itself.
+// Dynamic LDS: [partial tiles (KW > 1)] [1/rms of the rows] [rows of A (ALDS)].
+template <int MT, int TW, int KW, int AMODE, int EPI, int ALDS>
+__global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvParams p) {
+    constexpr int NS = Streams<EPI>::n;
+    constexpr int NW = TW * KW;
+    constexpr int RED = KW > 1 ? NW * MT * NS * 64 : 0;   // floatx4 entries
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    floatx4_t* red = reinterpret_cast<floatx4_t*>(lds_raw);
+    float* inv_rms = reinterpret_cast<float*>(lds_raw + static_cast<size_t>(RED) * 16);
+    bf16* xs = reinterpret_cast<bf16*>(lds_raw + static_cast<size_t>(RED) * 16 + 64 * sizeof(float));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c16 = lane & 15, q = lane >> 4;
+    const int tw = wave / KW, kw = wave % KW;
+    const int K = p.K, M = p.M;
+    const int ldx = K + 8;          // row stride in LDS: 16 bytes more than a row
+    const int tile = blockIdx.x * TW + tw;
+    const bool tile_ok = tile * 16 < p.N;
+
+    floatx4_t acc[MT][NS];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int s = 0; s < NS; ++s) acc[mt][s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    const bf16* wrow[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(tile * 16 + c16, p.N - 1)) * K;
+
+    // K is cut in chunks of 64 which are dealt to the KW wavefronts of a tile.  Inside a
+    // chunk, lane group q holds the k values {q*8..q*8+7} and {32+q*8..32+q*8+7}: each of
+    // the two 16-byte loads of a lane is side by side with its neighbours' in the row.
+    // U chunks of weights are loaded before any is multiplied, and the first U are asked
+    // for before the rows of A are prepared, so that memory latency and that work overlap.
+    constexpr int U = ALDS ? (MT * NS <= 2 ? 8 : (MT * NS <= 4 ? 4 : 2))
+                           : (MT == 1 ? 4 : (MT == 2 ? 2 : 1));
+    const int chunks = (K + 63) >> 6;
+    const int c_begin = tile_ok ? kw * chunks / KW : 0, c_end = tile_ok ? (kw + 1) * chunks / KW : 0;
+    Frag2 wv[U][NS][2];
+    auto load_weights = [&](int c0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int v = 0; v < 2; ++v) {
+                const int k = (c0 + u) * 64 + v * 32 + q * 8;   // 8 values from here
+                const bool in = c0 + u < c_end && k + 8 <= K;    // K % 8 == 0
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                    wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
+            }
+    };
+    load_weights(c_begin);
+
+    // ---- rows of A: 1/rms (A_NORM), and the rows themselves into LDS (ALDS); one wavefront
+    // per row.  The loads of a row are issued before the sum of squares is reduced.
+    if (AMODE == A_NORM || ALDS) {
+        for (int m = wave; m < M; m += NW) {
+            const size_t src = static_cast<size_t>(p.rows ? p.rows[m] : m);
+            if (AMODE == A_NORM) {
+                const float* row = static_cast<const float*>(p.a) + src * p.lda;
+                float s = 0.f;
+                if (p.stats) {
+                    for (int j = lane; j < p.n_stat_blocks; j += 64)
+                        s += p.stats[static_cast<size_t>(j) * p.stats_ld + src];
+                }
+                float inv = 0.f;
+                for (int k0 = 0; k0 < K; k0 += 1024) {
+                    floatx4_t hv4[4], nw4[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int k = k0 + i * 256 + lane * 4;
+                        hv4[i] = k < K ? *reinterpret_cast<const floatx4_t*>(row + k) : floatx4_t{};
+                        if (ALDS) nw4[i] = k < K ? *reinterpret_cast<const floatx4_t*>(p.norm_w + k) : floatx4_t{};
+                    }
+                    if (k0 == 0) {
+                        if (!p.stats) {   // no partial sums were left: walk the row
+                            for (int k = lane * 4; k < K; k += 256) {
+                                const floatx4_t v = *reinterpret_cast<const floatx4_t*>(row + k);
+                                s += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+                            }
+                        }
+                        s = wave_sum(s);
+                        inv = 1.0f / sqrtf(s / static_cast<float>(K) + p.eps);
+                        if (lane == 0) inv_rms[m] = inv;
+                        if (!ALDS) break;
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int k = k0 + i * 256 + lane * 4;
+                        if (k < K)
+                            *reinterpret_cast<bf16x4_t*>(xs + static_cast<size_t>(m) * ldx + k) =
+                                __builtin_bit_cast(bf16x4_t, __builtin_convertvector(hv4[i] * inv * nw4[i], nbf16x4_t));
+                    }
+                }
+            } else {
+                const bf16* row = static_cast<const bf16*>(p.a) + src * p.lda;
+                for (int k = lane * 8; k < K; k += 512)
+                    *reinterpret_cast<Frag2*>(xs + static_cast<size_t>(m) * ldx + k) =
+                        *reinterpret_cast<const Frag2*>(row + k);
+            }
+        }
+        __syncthreads();
+    }
+
+    // the row of A this lane feeds in every row tile (rows beyond M repeat the last one;
+    // their results are dropped)
+    size_t a_off[MT];
+    float a_inv[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = min(mt * 16 + c16, M - 1);
+        a_off[mt] = ALDS ? static_cast<size_t>(m) * ldx
+                         : static_cast<size_t>(p.rows ? p.rows[m] : m) * p.lda;
+        a_inv[mt] = (AMODE == A_NORM && !ALDS) ? inv_rms[m] : 1.f;
+    }
+
+    for (int c0 = c_begin; c0 < c_end;) {
+        Frag2 av[ALDS ? 1 : U][MT][2];            // rows read from memory: bfloat16
+        floatx4_t hv[ALDS ? 1 : U][MT][4];        //   or 32-bit, to be normalised
+        floatx4_t nv[ALDS ? 1 : U][4];
+        if (!ALDS) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int v = 0; v < 2; ++v) {
+                    const int k = (c0 + u) * 64 + v * 32 + q * 8;
+                    const bool in = c0 + u < c_end && k + 8 <= K;
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) {
+                        if (AMODE == A_BF16) {
+                            av[u][mt][v] = in ? *reinterpret_cast<const Frag2*>(
+                                                    static_cast<const bf16*>(p.a) + a_off[mt] + k)
+                                              : Frag2{};
+                        } else {
+                            const float* hr = static_cast<const float*>(p.a) + a_off[mt] + k;
+                            hv[u][mt][2 * v] = in ? *reinterpret_cast<const floatx4_t*>(hr) : floatx4_t{};
+                            hv[u][mt][2 * v + 1] = in ? *reinterpret_cast<const floatx4_t*>(hr + 4) : floatx4_t{};
+                        }
+                    }
+                    if (AMODE == A_NORM) {
+                        nv[u][2 * v] = in ? *reinterpret_cast<const floatx4_t*>(p.norm_w + k) : floatx4_t{};
+                        nv[u][2 * v + 1] = in ? *reinterpret_cast<const floatx4_t*>(p.norm_w + k + 4) : floatx4_t{};
+                    }
+                }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            bf16x4_t af[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                if (ALDS) {
+#pragma unroll
+                    for (int v = 0; v < 2; ++v) {
+                        const int k = min((c0 + u) * 64 + v * 32 + q * 8, K - 8);   // stay inside the row
+                        const Frag2 f = *reinterpret_cast<const Frag2*>(xs + a_off[mt] + k);
+                        af[mt][2 * v] = f.lo;
+                        af[mt][2 * v + 1] = f.hi;
+                    }
+                } else if (AMODE == A_BF16) {
+                    af[mt][0] = av[u][mt][0].lo; af[mt][1] = av[u][mt][0].hi;
+                    af[mt][2] = av[u][mt][1].lo; af[mt][3] = av[u][mt][1].hi;
+                } else {
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4)
+                        af[mt][s4] = __builtin_bit_cast(
+                            bf16x4_t, __builtin_convertvector(hv[u][mt][s4] * a_inv[mt] * nv[u][s4], nbf16x4_t));
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const bf16x4_t bfr[4] = {wv[u][s][0].lo, wv[u][s][0].hi, wv[u][s][1].lo, wv[u][s][1].hi};
+#pragma unroll
+                for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt][s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(af[mt][s4], bfr[s4], acc[mt][s], 0, 0, 0);
+            }
+        }
+        c0 += U;
+        if (c0 < c_end) load_weights(c0);
+    }
+
+    // ---- add the partial tiles of the KW wavefronts of a tile, in their order
+    if (KW > 1) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int s = 0; s < NS; ++s) red[(wave * MT * NS + mt * NS + s) * 64 + lane] = acc[mt][s];
+        __syncthreads();
+        if (kw != 0) return;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                floatx4_t t = red[(wave * MT * NS + mt * NS + s) * 64 + lane];
+                for (int w = 1; w < KW; ++w) t += red[((wave + w) * MT * NS + mt * NS + s) * 64 + lane];
+                acc[mt][s] = t;
+            }
+    }
+    if (!tile_ok) return;
+    gemv_epilogue<MT, NS, EPI>(p, acc, tile, lane);
+}
+
+static size_t gemv_lds_bytes(int mt, int tw, int kw, int streams, int alds, int m, int k) {
+    size_t bytes = 64 * sizeof(float);
+    if (kw > 1) bytes += static_cast<size_t>(tw) * kw * mt * streams * 64 * 16;
+    if (alds) bytes += static_cast<size_t>(m) * (k + 8) * 2;
+    return bytes;
+}
+
+template <int MT, int TW, int KW, int ALDS>
+static int launch_shape(const GemvParams& p, int amode, int epi, hipStream_t stream) {
+    const int tiles = (p.N + 15) / 16;
+    dim3 grid((tiles + TW - 1) / TW), block(TW * KW * 64);
+    const int streams = epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3 : 1);
+    const size_t lds = gemv_lds_bytes(MT, TW, KW, streams, ALDS, p.M, p.K);
+#define CELEG_GEMV(AM, EP)                                                                       \
+    do {                                                                                         \
+        auto kernel = gemv_fused_kernel<MT, TW, KW, AM, EP, ALDS>;                               \
+        if (lds > 48 * 1024) {                                                                   \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),            \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,       \
+                                               static_cast<int>(lds));                           \
+            if (e != hipSuccess) return static_cast<int>(e);                                     \
+        }                                                                                        \
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);                                 \
+    } while (0)
     if (amode == A_BF16) {
         switch (epi) {
             case E_STORE: CELEG_GEMV(A_BF16, E_STORE); break;
@@ -305,27 +394,36 @@ static int launch_mt_nw(const GemvParams& p, int amode, int epi, hipStream_t str
     return CELEG_LAUNCH_RESULT();
 }
 
-template <int MT>
-static int launch_mt(const GemvParams& p, int amode, int epi, int waves, hipStream_t stream) {
-    if (waves == 8 && MT <= 2) return launch_mt_nw<(MT <= 2 ? MT : 1), 8>(p, amode, epi, stream);
-    if (waves == 4 || waves == 8) return launch_mt_nw<MT, 4>(p, amode, epi, stream);
-    return static_cast<int>(hipErrorInvalidValue);
-}
-
-// waves: wavefronts per workgroup that split K: 4, or 8 (which is honoured up to 32 rows).
-extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, int waves,
-                                hipStream_t stream) {
+// The shape of the workgroup follows the number of column tiles: many tiles, one
+// wavefront a tile over all of K (8 tiles a workgroup); few tiles, 8 (or 4) wavefronts
+// share a tile's K.  The rows of A go through LDS when they fit (up to 144 KiB).
+extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, hipStream_t stream) {
     const GemvParams& p = *params;
     if (p.M <= 0 || p.N <= 0) return 0;
     if (p.M > 64 || p.K <= 0 || (p.K % 8) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.stream_rows != p.N)) return static_cast<int>(hipErrorInvalidValue);
-    const int mt = (p.M + 15) / 16;
-    switch (mt) {
-        case 1: return launch_mt<1>(p, amode, epi, waves, stream);
-        case 2: return launch_mt<2>(p, amode, epi, waves, stream);
-        case 3: return launch_mt<3>(p, amode, epi, waves, stream);
-        default: return launch_mt<4>(p, amode, epi, waves, stream);
+    const int tiles = (p.N + 15) / 16, chunks = (p.K + 63) / 64;
+    const int streams = epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3 : 1);
+    const int mt = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
+    const size_t limit = 144 * 1024;
+#define CELEG_SHAPE(MT_, TW_, KW_)                                                               \
+    (gemv_lds_bytes(MT_, TW_, KW_, streams, 1, p.M, p.K) <= limit                                \
+         ? launch_shape<MT_, TW_, KW_, 1>(p, amode, epi, stream)                                 \
+         : launch_shape<MT_, 1, 4, 0>(p, amode, epi, stream))
+    if (mt == 1) {
+        if (tiles >= 2048) return CELEG_SHAPE(1, 8, 1);
+        if (tiles >= 512) return CELEG_SHAPE(1, 2, 4);
+        if (chunks >= 8) return CELEG_SHAPE(1, 1, 8);
+        return CELEG_SHAPE(1, 1, 4);
     }
+    if (mt == 2) {
+        if (tiles >= 2048) return CELEG_SHAPE(2, 8, 1);
+        if (tiles >= 512) return CELEG_SHAPE(2, 2, 4);
+        return CELEG_SHAPE(2, 1, 4);
+    }
+    if (tiles >= 2048) return CELEG_SHAPE(4, 8, 1);
+    return CELEG_SHAPE(4, 1, 4);
+#undef CELEG_SHAPE
 }
 
 // Embedding gather that also leaves the sum of squares of every row, for the first norm:

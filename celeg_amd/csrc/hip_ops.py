@@ -472,11 +472,9 @@ class HipOps:
             prm.conv_b = conv_bias.data_ptr() if conv_bias is not None else None
             prm.state, prm.state_slot_stride = state.data_ptr(), state.stride(0)
             prm.seq_slot, prm.taps = seq_slot.data_ptr(), L
-        tiles, chunks = (N + 15) // 16, (K + 63) // 64
-        waves = 8 if (tiles < 512 and M <= 32 and chunks >= 16) else 4
         code = self._lib("gemv_fused").celeg_gemv_fused(
             ctypes.byref(prm), _c_int(1 if norm_weight is not None else 0),
-            _c_int(self._EPILOGUES[epilogue]), _c_int(waves), self._stream())
+            _c_int(self._EPILOGUES[epilogue]), self._stream())
         self._check(code, f"fused_linear ({epilogue})")
         return out
 
