@@ -189,33 +189,68 @@ extern "C" int celeg_attention_rows_bf16(
 }
 
 // ================================================================ one row per request
-// One wavefront per (range of `split_keys` keys, GH query heads that share a key/value
-// head, request).  Keys are taken 64 at a time: for q.k a lane owns (key j, an eighth of
-// head_dim) and eight lanes add up a score; for p.v a lane owns a dimension and reads
-// its row of the transposed V.  Partial (max, sum, accumulator) go to a workspace and a
-// second kernel joins the ranges.
+// One wavefront per (64 keys, GH query heads that share a key/value head, request): all
+// its loads (the page ids, then the 64 keys and the 64 values) are in flight before
+// anything is computed.  For q.k a lane owns (key j, an eighth of head_dim) and eight
+// lanes add up a score; for p.v a lane owns a dimension and reads its row of the
+// transposed V.  Partial (max, sum, accumulator) go to a workspace and a second kernel
+// joins the ranges of 64 keys.
+#define DEC_KEYS 64
+
 template <int HD, int GH>
 __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ token_slot, const int* __restrict__ positions,
-    float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits, int split_keys,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
     int q_heads, int kv_heads, int page_tokens, int n_layers, int layer, float scale, int window) {
     constexpr int DL = HD / 8;    // dims of a key a lane multiplies
     constexpr int DD = HD / 64;   // output dims a lane accumulates
-    __shared__ float ps[GH][64];
+    __shared__ float ps[GH][DEC_KEYS];
     const int split = blockIdx.x, hb = blockIdx.y, t = blockIdx.z;
     const int lane = threadIdx.x;
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int k_lo = max(lo, split * split_keys);
-    const int k_hi = min(pos, (split + 1) * split_keys - 1);
+    const int kb = split * DEC_KEYS;
+    const int k_lo = max(lo, kb);
+    const int k_hi = min(pos, kb + DEC_KEYS - 1);
     if (k_lo > k_hi) return;
     const int h0 = hb * GH;
     const int kvh = h0 / (q_heads / kv_heads);
     const int j8 = lane >> 3, seg = lane & 7;
     const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
 
+    // page ids of the chunk: lane i holds the i-th page that the 64 keys touch
+    const int first_page = kb / page_tokens;
+    const int last_page = k_hi / page_tokens;
+    const int my_page = pages[min(first_page + lane, last_page)];
+
+    // keys: 8 rounds of 8 keys, a lane reads DL values of its key
+    uint4 kraw[8][DL / 8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int keyc = min(max(kb + it * 8 + j8, k_lo), k_hi);
+        const int page = __shfl(my_page, keyc / page_tokens - first_page, 64);
+        const bf16* kp = k_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
+                         static_cast<size_t>(keyc % page_tokens) * HD + seg * DL;
+#pragma unroll
+        for (int v8 = 0; v8 < DL / 8; ++v8) kraw[it][v8] = *reinterpret_cast<const uint4*>(kp + v8 * 8);
+    }
+    // values: 4 groups of 16 keys, a lane reads the 16 values of its dimension(s)
+    uint4 vraw[4][DD][2];
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg) {
+        const int key0 = min(max(kb + pg * 16, k_lo & ~15), k_hi & ~15);   // a group inside the range
+        const int page = __shfl(my_page, key0 / page_tokens - first_page, 64);
+        const bf16* vbase = v_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
+                            (key0 % page_tokens);
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd)
+#pragma unroll
+            for (int v8 = 0; v8 < 2; ++v8)
+                vraw[pg][dd][v8] = *reinterpret_cast<const uint4*>(
+                    vbase + static_cast<size_t>(lane + 64 * dd) * page_tokens + v8 * 8);
+    }
     float qf[GH][DL];
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
@@ -223,133 +258,137 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 #pragma unroll
         for (int d = 0; d < DL; ++d) qf[g][d] = to_float(qrow[d]) * scale;
     }
-    float m[GH], l[GH], acc[GH][DD];
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-        m[g] = -INFINITY; l[g] = 0.f;
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) acc[g][dd] = 0.f;
-    }
 
-    for (int kb = (k_lo >> 6) << 6; kb <= k_hi; kb += 64) {
-        float sc[8][GH];
+    float sc[8][GH];
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
-            const int key = kb + it * 8 + j8;
-            const bool valid = key >= k_lo && key <= k_hi;
-            const int keyc = min(max(key, k_lo), k_hi);
-            const bf16* kp = k_pool +
-                             kv_block(pages[keyc / page_tokens], n_layers, layer, kv_heads, kvh,
-                                      page_tokens, HD) +
-                             static_cast<size_t>(keyc % page_tokens) * HD + seg * DL;
-            float kf[DL];
+    for (int it = 0; it < 8; ++it) {
+        const int key = kb + it * 8 + j8;
+        const bool valid = key >= k_lo && key <= k_hi;
+        float kf[DL];
 #pragma unroll
-            for (int v8 = 0; v8 < DL / 8; ++v8) {
-                const uint4 raw = *reinterpret_cast<const uint4*>(kp + v8 * 8);
-                const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        for (int v8 = 0; v8 < DL / 8; ++v8) {
+            const uint32_t w[4] = {kraw[it][v8].x, kraw[it][v8].y, kraw[it][v8].z, kraw[it][v8].w};
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    kf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
-                    kf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-                }
-            }
-#pragma unroll
-            for (int g = 0; g < GH; ++g) {
-                float dot = 0.f;
-#pragma unroll
-                for (int d = 0; d < DL; ++d) dot = fmaf(qf[g][d], kf[d], dot);
-                dot += __shfl_xor(dot, 1, 64);
-                dot += __shfl_xor(dot, 2, 64);
-                dot += __shfl_xor(dot, 4, 64);
-                sc[it][g] = valid ? dot : -INFINITY;
+            for (int i = 0; i < 4; ++i) {
+                kf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
+                kf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
             }
         }
 #pragma unroll
         for (int g = 0; g < GH; ++g) {
-            float mx = sc[0][g];
+            float dot = 0.f;
 #pragma unroll
-            for (int it = 1; it < 8; ++it) mx = fmaxf(mx, sc[it][g]);
-            mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m[g], mx);   // finite: the chunk holds a key of the range
-            const float corr = expf(m[g] - m_new);
-            float psum = 0.f;
-#pragma unroll
-            for (int it = 0; it < 8; ++it) {
-                const float p = expf(sc[it][g] - m_new);
-                psum += p;
-                if (seg == 0) ps[g][it * 8 + j8] = p;
-            }
-            l[g] = l[g] * corr + psum;
-            m[g] = m_new;
-#pragma unroll
-            for (int dd = 0; dd < DD; ++dd) acc[g][dd] *= corr;
+            for (int d = 0; d < DL; ++d) dot = fmaf(qf[g][d], kf[d], dot);
+            dot += __shfl_xor(dot, 1, 64);
+            dot += __shfl_xor(dot, 2, 64);
+            dot += __shfl_xor(dot, 4, 64);
+            sc[it][g] = valid ? dot : -INFINITY;
         }
-        __syncthreads();
+    }
+    float m[GH], l[GH];
 #pragma unroll
-        for (int pg = 0; pg < 4; ++pg) {
-            const int key0 = kb + pg * 16;
-            if (key0 > k_hi || key0 + 15 < k_lo) continue;
-            const bf16* vbase = v_pool +
-                                kv_block(pages[key0 / page_tokens], n_layers, layer, kv_heads, kvh,
-                                         page_tokens, HD) + (key0 % page_tokens);
+    for (int g = 0; g < GH; ++g) {
+        float mx = sc[0][g];
 #pragma unroll
-            for (int dd = 0; dd < DD; ++dd) {
-                const bf16* vp = vbase + static_cast<size_t>(lane + 64 * dd) * page_tokens;
-                float vf[16];
+        for (int it = 1; it < 8; ++it) mx = fmaxf(mx, sc[it][g]);
+        mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));   // finite: the chunk holds a key of the range
+        float psum = 0.f;
 #pragma unroll
-                for (int v8 = 0; v8 < 2; ++v8) {
-                    const uint4 raw = *reinterpret_cast<const uint4*>(vp + v8 * 8);
-                    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        for (int it = 0; it < 8; ++it) {
+            const float p = expf(sc[it][g] - mx);
+            psum += p;
+            if (seg == 0) ps[g][it * 8 + j8] = p;
+        }
+        psum += __shfl_xor(psum, 8, 64);    // the eight lanes of a key hold the same p:
+        psum += __shfl_xor(psum, 16, 64);   // add over keys only
+        psum += __shfl_xor(psum, 32, 64);
+        m[g] = mx;
+        l[g] = psum;
+    }
+    __syncthreads();
+    float acc[GH][DD];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        vf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
-                        vf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-                    }
+    for (int g = 0; g < GH; ++g)
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) acc[g][dd] = 0.f;
+#pragma unroll
+    for (int pg = 0; pg < 4; ++pg) {
+        // groups outside the range were redirected to one inside: their p are all zero
+        const int key0 = kb + pg * 16;
+        if (key0 > k_hi || key0 + 15 < k_lo) continue;
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) {
+            float vf[16];
+#pragma unroll
+            for (int v8 = 0; v8 < 2; ++v8) {
+                const uint32_t w[4] = {vraw[pg][dd][v8].x, vraw[pg][dd][v8].y, vraw[pg][dd][v8].z,
+                                       vraw[pg][dd][v8].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    vf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
+                    vf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
                 }
-#pragma unroll
-                for (int g = 0; g < GH; ++g)
-#pragma unroll
-                    for (int j = 0; j < 16; ++j)
-                        acc[g][dd] = fmaf(ps[g][pg * 16 + j], vf[j], acc[g][dd]);
             }
+#pragma unroll
+            for (int g = 0; g < GH; ++g)
+#pragma unroll
+                for (int j = 0; j < 16; ++j) acc[g][dd] = fmaf(ps[g][pg * 16 + j], vf[j], acc[g][dd]);
         }
-        __syncthreads();
     }
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
-        float lt = l[g];   // the eight lanes of a key hold the same p: add over keys only
-        lt += __shfl_xor(lt, 8, 64);
-        lt += __shfl_xor(lt, 16, 64);
-        lt += __shfl_xor(lt, 32, 64);
         const size_t idx = (static_cast<size_t>(t) * q_heads + h0 + g) * n_splits + split;
-        if (lane == 0) { ws_ml[2 * idx] = m[g]; ws_ml[2 * idx + 1] = lt; }
+        if (lane == 0) { ws_ml[2 * idx] = m[g]; ws_ml[2 * idx + 1] = l[g]; }
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd) ws_o[idx * HD + lane + 64 * dd] = acc[g][dd];
     }
 }
 
+// Joins the ranges of one (request, query head): out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
 template <int HD>
 __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int* __restrict__ positions, bf16* __restrict__ out, int ldo, int q_heads, int n_splits,
-    int split_keys, int window) {
+    int window) {
     const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int first = lo / split_keys, last = pos / split_keys;
+    const int first = lo / DEC_KEYS, last = pos / DEC_KEYS;
     const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits;
     float m = -INFINITY;
-    for (int i = first; i <= last; ++i) m = fmaxf(m, ws_ml[2 * (base + i)]);
+    for (int i0 = first; i0 <= last; i0 += 64) {
+        const int i = i0 + lane;
+        m = fmaxf(m, i <= last ? ws_ml[2 * (base + i)] : -INFINITY);
+    }
+    m = wave_max(m);
     float denom = 0.f, acc[HD / 64];
 #pragma unroll
     for (int dd = 0; dd < HD / 64; ++dd) acc[dd] = 0.f;
-    for (int i = first; i <= last; ++i) {
-        const float w = expf(ws_ml[2 * (base + i)] - m);
-        denom += w * ws_ml[2 * (base + i) + 1];
+    for (int i0 = first; i0 <= last; i0 += 64) {
+        const int i = i0 + lane;
+        float w = 0.f, wl = 0.f;
+        if (i <= last) {
+            w = expf(ws_ml[2 * (base + i)] - m);
+            wl = w * ws_ml[2 * (base + i) + 1];
+        }
+        denom += wave_sum(wl);
+        const int n = min(64, last - i0 + 1);
+        for (int j0 = 0; j0 < n; j0 += 8) {     // eight ranges' accumulators are read side by side
+            float o[8][HD / 64];
 #pragma unroll
-        for (int dd = 0; dd < HD / 64; ++dd) acc[dd] += w * ws_o[(base + i) * HD + lane + 64 * dd];
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int dd = 0; dd < HD / 64; ++dd)
+                    o[j][dd] = j0 + j < n ? ws_o[(base + i0 + j0 + j) * HD + lane + 64 * dd] : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float wj = __shfl(w, min(j0 + j, 63), 64);
+#pragma unroll
+                for (int dd = 0; dd < HD / 64; ++dd) acc[dd] = fmaf(j0 + j < n ? wj : 0.f, o[j][dd], acc[dd]);
+            }
+        }
     }
     bf16* orow = out + static_cast<size_t>(t) * ldo + static_cast<size_t>(h) * HD;
 #pragma unroll
@@ -357,16 +396,16 @@ __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
 }
 
 // workspace: ws_o [rows, q_heads, n_splits, head_dim] and ws_ml [rows, q_heads, n_splits, 2]
-// floats, n_splits = ceil(max_context / split_keys).
+// floats, n_splits = ceil(max_context / 64).
 extern "C" int celeg_attention_decode_bf16(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
-    int n_splits, int split_keys, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
+    int n_splits, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
     int head_dim, int page_tokens, int n_layers, int layer, float scale, int window,
     hipStream_t stream) {
     if (n_rows <= 0) return 0;
     const int group = q_heads / kv_heads;
-    if (q_heads % kv_heads || page_tokens % 16 || split_keys % 64 || n_splits <= 0 || (ldq % 8))
+    if (q_heads % kv_heads || page_tokens % 16 || n_splits <= 0 || (ldq % 8))
         return static_cast<int>(hipErrorInvalidValue);
     const int gh = (group % 4 == 0) ? 4 : ((group % 2 == 0) ? 2 : 1);
     dim3 grid(n_splits, q_heads / gh, n_rows), block(64);
@@ -374,13 +413,13 @@ extern "C" int celeg_attention_decode_bf16(
     hipLaunchKernelGGL((attention_decode_kernel<HD_, GH_>), grid, block, 0, stream,              \
                        static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
                        static_cast<const bf16*>(v_pool), table, table_stride, token_slot,        \
-                       positions, ws_o, ws_ml, n_splits, split_keys, q_heads, kv_heads,          \
+                       positions, ws_o, ws_ml, n_splits, q_heads, kv_heads,                      \
                        page_tokens, n_layers, layer, scale, window)
 #define CELEG_DEC_HD(HD_)                                                                        \
     if (gh == 4) CELEG_DEC(HD_, 4); else if (gh == 2) CELEG_DEC(HD_, 2); else CELEG_DEC(HD_, 1);  \
     hipLaunchKernelGGL(attention_decode_reduce_kernel<HD_>, dim3(q_heads, n_rows), dim3(64), 0,  \
                        stream, ws_o, ws_ml, positions, static_cast<bf16*>(out), ldo, q_heads,    \
-                       n_splits, split_keys, window)
+                       n_splits, window)
     if (head_dim == 64) { CELEG_DEC_HD(64); }
     else if (head_dim == 128) { CELEG_DEC_HD(128); }
     else return static_cast<int>(hipErrorInvalidValue);

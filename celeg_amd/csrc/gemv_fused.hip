@@ -70,10 +70,53 @@ template <int EPI> struct Streams { static constexpr int n = 1; };
 template <> struct Streams<E_SWIGLU> { static constexpr int n = 2; };
 template <> struct Streams<E_CONV> { static constexpr int n = 3; };
 
+// What the epilogue reads besides the product, asked for before the product is computed:
+// the old value of the residual stream, or the convolution's state, taps and bias.
+#define CONV_PREFETCH_TAPS 8
+template <int MT, int EPI>
+struct EpiloguePrefetch {
+    float old[EPI == E_RESIDUAL ? MT : 1][4];
+    float state[EPI == E_CONV ? MT : 1][4][EPI == E_CONV ? CONV_PREFETCH_TAPS - 1 : 1];
+    float taps[EPI == E_CONV ? CONV_PREFETCH_TAPS : 1];
+    int slot_row[EPI == E_CONV ? MT : 1][4];
+};
+
+template <int MT, int EPI>
+__device__ __forceinline__ void gemv_prefetch(const GemvParams& p, EpiloguePrefetch<MT, EPI>& pre,
+                                              int tile, int lane) {
+    const int c16 = lane & 15, q = lane >> 4;
+    const int n = min(tile * 16 + c16, p.N - 1);
+    if (EPI == E_RESIDUAL) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = min(mt * 16 + 4 * q + r, p.M - 1);
+                pre.old[mt][r] = static_cast<const float*>(p.out)[static_cast<size_t>(m) * p.ldo + n];
+            }
+    }
+    if (EPI == E_CONV) {
+#pragma unroll
+        for (int t = 0; t < CONV_PREFETCH_TAPS; ++t)
+            pre.taps[t] = t < p.taps ? p.conv_w[static_cast<size_t>(n) * p.taps + t] : 0.f;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = min(mt * 16 + 4 * q + r, p.M - 1);
+                const float* st = p.state + static_cast<size_t>(p.seq_slot[m]) * p.state_slot_stride + n;
+#pragma unroll
+                for (int t = 0; t < CONV_PREFETCH_TAPS - 1; ++t)
+                    pre.state[mt][r][t] = t + 1 < p.taps ? st[static_cast<size_t>(t + 1) * p.N] : 0.f;
+            }
+    }
+}
+
 // ---- epilogue of one 16-column tile: this lane holds column n0 + lane%16 of rows
 // 4*(lane/16)..+3 of every row tile
 template <int MT, int NS, int EPI>
 __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&acc)[MT][NS],
+                                              const EpiloguePrefetch<MT, EPI>& pre,
                                               int tile, int lane) {
     const int c16 = lane & 15, q = lane >> 4;
     const int M = p.M;
@@ -96,7 +139,7 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&a
                 if (ok) {
                     float* hp = static_cast<float*>(p.out) + static_cast<size_t>(m) * p.ldo + n;
                     // the product enters the sum rounded to bfloat16, as when it is stored first
-                    const float v = *hp + round_bf16(acc[mt][0][r] + (p.bias ? p.bias[n] : 0.f));
+                    const float v = pre.old[mt][r] + round_bf16(acc[mt][0][r] + (p.bias ? p.bias[n] : 0.f));
                     *hp = v;
                     sq[r] = v * v;
                 }
@@ -113,14 +156,20 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&a
                     const float xx = round_bf16(acc[mt][2][r] + (p.bias ? p.bias[2 * p.stream_rows + n] : 0.f));
                     const float bx = bb * xx;
                     float* st = p.state + static_cast<size_t>(p.seq_slot[m]) * p.state_slot_stride + n;
-                    const float* cw = p.conv_w + static_cast<size_t>(n) * p.taps;
                     float conv = 0.f;
-                    for (int tap = 0; tap + 1 < p.taps; ++tap) {
-                        const float old = st[static_cast<size_t>(tap + 1) * p.N];
-                        conv = fmaf(cw[tap], old, conv);
-                        st[static_cast<size_t>(tap) * p.N] = old;     // shift by one position
+#pragma unroll
+                    for (int tap = 0; tap < CONV_PREFETCH_TAPS - 1; ++tap) {
+                        if (tap + 1 < p.taps) {
+                            const float old = pre.state[mt][r][tap];
+                            conv = fmaf(pre.taps[tap], old, conv);
+                            st[static_cast<size_t>(tap) * p.N] = old;     // shift by one position
+                        }
                     }
-                    conv = fmaf(cw[p.taps - 1], bx, conv);
+                    float last_tap = 0.f;
+#pragma unroll
+                    for (int tap = 0; tap < CONV_PREFETCH_TAPS; ++tap)
+                        if (tap == p.taps - 1) last_tap = pre.taps[tap];
+                    conv = fmaf(last_tap, bx, conv);
                     st[static_cast<size_t>(p.taps - 1) * p.N] = bx;
                     if (p.conv_b) conv += p.conv_b[n];
                     static_cast<bf16*>(p.out)[static_cast<size_t>(m) * p.ldo + n] = from_float<bf16>(cc * conv);
@@ -185,6 +234,8 @@ __global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvPara
                            : (MT == 1 ? 4 : (MT == 2 ? 2 : 1));
     const int chunks = (K + 63) >> 6;
     const int c_begin = tile_ok ? kw * chunks / KW : 0, c_end = tile_ok ? (kw + 1) * chunks / KW : 0;
+    EpiloguePrefetch<MT, EPI> pre;
+    if (kw == 0 && tile_ok) gemv_prefetch<MT, EPI>(p, pre, tile, lane);
     Frag2 wv[U][NS][2];
     auto load_weights = [&](int c0) {
 #pragma unroll
@@ -347,7 +398,7 @@ __global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvPara
             }
     }
     if (!tile_ok) return;
-    gemv_epilogue<MT, NS, EPI>(p, acc, tile, lane);
+    gemv_epilogue<MT, NS, EPI>(p, acc, pre, tile, lane);
 }
 
 static size_t gemv_lds_bytes(int mt, int tw, int kw, int streams, int alds, int m, int k) {
@@ -397,11 +448,15 @@ static int launch_shape(const GemvParams& p, int amode, int epi, hipStream_t str
 // The shape of the workgroup follows the number of column tiles: many tiles, one
 // wavefront a tile over all of K (8 tiles a workgroup); few tiles, 8 (or 4) wavefronts
 // share a tile's K.  The rows of A go through LDS when they fit (up to 144 KiB).
-extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, hipStream_t stream) {
+// shape: 0 lets the tile count decide; 1..4 force (TW, KW) = (8,1), (2,4), (1,8), (1,4) (for
+// up to 16 rows; a tuning aid).
+extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, int shape,
+                                hipStream_t stream) {
     const GemvParams& p = *params;
     if (p.M <= 0 || p.N <= 0) return 0;
     if (p.M > 64 || p.K <= 0 || (p.K % 8) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
-    if (epi == E_CONV && (p.taps < 1 || p.stream_rows != p.N)) return static_cast<int>(hipErrorInvalidValue);
+    if (epi == E_CONV && (p.taps < 1 || p.taps > CONV_PREFETCH_TAPS || p.stream_rows != p.N))
+        return static_cast<int>(hipErrorInvalidValue);
     const int tiles = (p.N + 15) / 16, chunks = (p.K + 63) / 64;
     const int streams = epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3 : 1);
     const int mt = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
@@ -411,14 +466,20 @@ extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, hi
          ? launch_shape<MT_, TW_, KW_, 1>(p, amode, epi, stream)                                 \
          : launch_shape<MT_, 1, 4, 0>(p, amode, epi, stream))
     if (mt == 1) {
+        if (shape == 1) return CELEG_SHAPE(1, 8, 1);
+        if (shape == 2) return CELEG_SHAPE(1, 2, 4);
+        if (shape == 3) return CELEG_SHAPE(1, 1, 8);
+        if (shape == 4) return CELEG_SHAPE(1, 1, 4);
         if (tiles >= 2048) return CELEG_SHAPE(1, 8, 1);
-        if (tiles >= 512) return CELEG_SHAPE(1, 2, 4);
+        // two tiles a workgroup (they share the prepared rows) once there are enough tiles
+        // and K is short enough that four wavefronts a tile keep their loads in one batch
+        if (tiles >= 512 || (tiles >= 128 && chunks <= 32)) return CELEG_SHAPE(1, 2, 4);
         if (chunks >= 8) return CELEG_SHAPE(1, 1, 8);
         return CELEG_SHAPE(1, 1, 4);
     }
     if (mt == 2) {
         if (tiles >= 2048) return CELEG_SHAPE(2, 8, 1);
-        if (tiles >= 512) return CELEG_SHAPE(2, 2, 4);
+        if (tiles >= 512 || (tiles >= 128 && chunks <= 32)) return CELEG_SHAPE(2, 2, 4);
         return CELEG_SHAPE(2, 1, 4);
     }
     if (tiles >= 2048) return CELEG_SHAPE(4, 8, 1);

@@ -43,9 +43,9 @@ class HipOps:
         # "auto": the matrix-core and split-key kernels where they apply; "general": always
         # the general kernel (tests compare the two)
         self.attention_impl = "auto"
-        self.decode_split_keys = None      # None: chosen from the number of rows
         self._decode_ws = None
         self._retired = []
+        self.fused_linear_shape = 0        # 0: chosen from the sizes; 1..4 force a workgroup shape
 
     # ------------------------------------------------------------------ plumbing
     def _lib(self, module: str) -> ctypes.CDLL:
@@ -314,16 +314,8 @@ class HipOps:
 
     def _attention_decode(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv):
         T = q.shape[0]
-        group = heads // kv_heads
-        gh = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
-        split_keys = self.decode_split_keys
-        if split_keys is None:
-            blocks = T * (heads // gh)
-            split_keys = 64 if blocks <= 16 else (128 if blocks <= 128 else 256)
-        if split_keys % 64:
-            raise KernelError("attention: decode_split_keys must be a multiple of 64")
         max_context = kv.table.shape[1] * kv.page_tokens
-        n_splits = (max_context + split_keys - 1) // split_keys
+        n_splits = (max_context + 63) // 64          # the kernel takes 64 keys a wavefront
         need = T * heads * n_splits * (head_dim + 2)
         if self._decode_ws is None or self._decode_ws.numel() < need:
             if self._decode_ws is not None:
@@ -334,7 +326,7 @@ class HipOps:
         code = self._lib("attention_fast").celeg_attention_decode_bf16(
             _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v), _ptr(kv.table),
             _c_int(kv.table.shape[1]), _ptr(batch.token_slot), _ptr(batch.positions), _ptr(ws_o),
-            _ptr(ws_ml), _c_int(n_splits), _c_int(split_keys), _ptr(out), _c_int(heads * head_dim),
+            _ptr(ws_ml), _c_int(n_splits), _ptr(out), _c_int(heads * head_dim),
             _c_int(T), _c_int(heads), _c_int(kv_heads), _c_int(head_dim), _c_int(kv.page_tokens),
             _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
             _c_int(window if window else 0), self._stream())
@@ -465,6 +457,8 @@ class HipOps:
             self._dev(taps_w, "conv taps", torch.float32); self._dev(seq_slot, "seq_slot", torch.int32)
             self._dev(state, "state", torch.float32, contiguous=False)
             L = taps_w.shape[1]
+            if L > 8:
+                raise KernelError(f"fused_linear: the convolution epilogue holds up to 8 taps, not {L}")
             if taps_w.shape[0] != N or state.shape[1:] != (L, N) or state.stride(1) != N \
                     or state.stride(2) != 1 or seq_slot.numel() < M:
                 raise KernelError("fused_linear: convolution operands do not fit")
@@ -474,7 +468,7 @@ class HipOps:
             prm.seq_slot, prm.taps = seq_slot.data_ptr(), L
         code = self._lib("gemv_fused").celeg_gemv_fused(
             ctypes.byref(prm), _c_int(1 if norm_weight is not None else 0),
-            _c_int(self._EPILOGUES[epilogue]), self._stream())
+            _c_int(self._EPILOGUES[epilogue]), _c_int(self.fused_linear_shape), self._stream())
         self._check(code, f"fused_linear ({epilogue})")
         return out
 

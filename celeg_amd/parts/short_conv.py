@@ -80,7 +80,7 @@ class ShortConv(Mixer):
             return False
         T = batch.n_tokens
         y = rt.ws.buf("conv_y", (T, H), rt.dtype)
-        if batch.decode_only and batch.n_seqs == T:
+        if batch.decode_only and batch.n_seqs == T and self.taps <= 8:   # the fused form holds 8 taps
             norm_linear(rt, h, norm, self.w_in, y, epilogue="conv", bias=self.b_in,
                         conv=(self.w_conv, self.b_conv, cache.states["bx"], batch.seq_slot))
         else:

@@ -272,17 +272,13 @@ def test_attention_mixed_steps(ops, dtype, heads, kv_heads, head_dim):
                    cuts=[7, 1, 2, 30, 1, 16, 5])
 
 
-@pytest.mark.parametrize("split_keys", [64, 128, None])
+@pytest.mark.parametrize("page_tokens", [16, 32, 64, 128])
 @pytest.mark.parametrize("heads,kv_heads,head_dim", [(4, 2, 64), (8, 1, 128), (3, 1, 64)])
-def test_attention_long_prompt_then_decode_rows(ops, heads, kv_heads, head_dim, split_keys):
+def test_attention_long_prompt_then_decode_rows(ops, heads, kv_heads, head_dim, page_tokens):
     """A long portion through the matrix-core kernel, then rows one by one through the
-    split-key kernel, several requests per step, ranges of keys of 64, 128 or chosen."""
-    ops.decode_split_keys = split_keys
-    try:
-        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[333, 150, 420],
-                       cuts=[300] + [1] * 40, boost=(2, 331))
-    finally:
-        ops.decode_split_keys = None
+    split-key kernel (64 keys a wavefront), several requests per step, at several page sizes."""
+    attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[333, 150, 420],
+                   cuts=[300] + [1] * 40, boost=(2, 331), page_tokens=page_tokens)
 
 
 def test_fast_and_general_attention_agree(ops):
