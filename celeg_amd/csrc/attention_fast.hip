@@ -33,7 +33,9 @@ __device__ __forceinline__ short bf16_bits(float x) { return static_cast<short>(
 // wavefront owns 16 rows.  Per 64 keys: S^T = K Q^T (16x16x16 MFMA: A = 16 keys x 16
 // dims, B = 16 dims x 16 rows), online softmax per row (a row is a lane column), then
 // O^T += V^T P^T (A = 16 dims x 16 keys from the transposed V, B = P^T straight from the
-// accumulator registers of S^T).
+// accumulator registers of S^T).  The request's page ids are put into LDS once; the keys
+// of the next 64 are asked for while the current 64 are worked on, and the values of the
+// current 64 before its scores are computed.
 template <int HD>
 __global__ __launch_bounds__(256) void attention_rows_kernel(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
@@ -44,6 +46,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
     constexpr int DQ = HD / 4;   // dims a lane quad covers in q.k
     constexpr int KS = DQ / 4;   // MFMA steps along head_dim
     constexpr int DT = HD / 16;  // 16-dim tiles of the output
+    extern __shared__ int spages[];   // table_stride page ids
     int tile = blockIdx.x;
     const int h = blockIdx.y;
     int s = 0, len = 0;
@@ -54,7 +57,15 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
         if (tile < tiles) { found = true; break; }
         tile -= tiles;
     }
-    if (!found) return;
+    if (!found) return;   // the whole workgroup
+    const int start = seq_start[s];
+    {
+        // pages up to the last key this tile of rows can see
+        const int last_key = start + min(tile * 64 + 63, len - 1);
+        const int* __restrict__ pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
+        for (int i = threadIdx.x; i <= last_key / page_tokens; i += 256) spages[i] = pages[i];
+    }
+    __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int c = lane & 15, qd = lane >> 4;
     const int wrow0 = tile * 64 + wave * 16;
@@ -62,14 +73,15 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
     const int row = wrow0 + c;
     const bool row_valid = row < len;
     const int row_c = row_valid ? row : len - 1;
-    const int start = seq_start[s];
     const int pq = start + row_c;                       // this lane's row position
     const int lo_q = window > 0 ? max(0, pq - window + 1) : 0;
     const int kmax = start + min(wrow0 + 15, len - 1);  // last key any row of the wavefront sees
     const int kmin = window > 0 ? max(0, start + wrow0 - window + 1) : 0;
     const int kvh = h / (q_heads / kv_heads);
-    const int* __restrict__ pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
     const size_t row_base = static_cast<size_t>(cu_seqlens[s]);
+    const size_t head_block = static_cast<size_t>(page_tokens) * HD;
+    const size_t page_stride = static_cast<size_t>(n_layers) * kv_heads * head_block;
+    const size_t layer_head = (static_cast<size_t>(layer) * kv_heads + kvh) * head_block;
 
     bf16x4_t qreg[KS];
     {
@@ -82,23 +94,42 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    for (int kb = (kmin >> 6) << 6; kb <= kmax; kb += 64) {
+    // keys of 64 positions from kb: lane (key c of tile kt, quad qd) reads DQ values
+    bf16x4_t kreg[4][KS], knext[4][KS];
+    auto load_keys = [&](int kb, bf16x4_t (&dst)[4][KS]) {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            const int key = min(kb + kt * 16 + c, kmax);  // a valid address; masked if beyond
+            const bf16* kp = k_pool + static_cast<size_t>(spages[key / page_tokens]) * page_stride +
+                             layer_head + static_cast<size_t>(key % page_tokens) * HD + qd * DQ;
+#pragma unroll
+            for (int st = 0; st < KS; ++st) dst[kt][st] = *reinterpret_cast<const bf16x4_t*>(kp + st * 4);
+        }
+    };
+    const int kb0 = (kmin >> 6) << 6;
+    load_keys(kb0, kreg);
+    for (int kb = kb0; kb <= kmax; kb += 64) {
+        // values of this round: lane (dim c of tile dt, quad qd) reads 4 keys' values
+        bf16x4_t vreg[4][DT];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            const int key0 = min(kb + kt * 16, kmax & ~15);
+            const bf16* vp = v_pool + static_cast<size_t>(spages[key0 / page_tokens]) * page_stride +
+                             layer_head + static_cast<size_t>(c) * page_tokens +
+                             (key0 % page_tokens) + 4 * qd;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                vreg[kt][dt] = *reinterpret_cast<const bf16x4_t*>(vp + static_cast<size_t>(dt) * 16 * page_tokens);
+        }
+        if (kb + 64 <= kmax) load_keys(kb + 64, knext);
+
         floatx4_t sacc[4];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             sacc[kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-            const int key0 = kb + kt * 16;
-            if (key0 > kmax) continue;
-            const int key = min(key0 + c, kmax);  // a valid address; masked below if beyond
-            const bf16* kp = k_pool +
-                             kv_block(pages[key / page_tokens], n_layers, layer, kv_heads, kvh,
-                                      page_tokens, HD) +
-                             static_cast<size_t>(key % page_tokens) * HD + qd * DQ;
 #pragma unroll
-            for (int st = 0; st < KS; ++st) {
-                const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(kp + st * 4);
-                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, qreg[st], sacc[kt], 0, 0, 0);
-            }
+            for (int st = 0; st < KS; ++st)
+                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[kt][st], qreg[st], sacc[kt], 0, 0, 0);
         }
         // sacc[kt][r] = (key kb + 16 kt + 4 qd + r) . (row c)
         float mx = -INFINITY;
@@ -131,21 +162,17 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
         for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
-            const int key0 = kb + kt * 16;
-            if (key0 > kmax) continue;
+            // a tile beyond the last key was read from the last tile's place: its p are zero
             const bf16x4_t pb = {bf16_bits(sacc[kt][0]), bf16_bits(sacc[kt][1]),
                                  bf16_bits(sacc[kt][2]), bf16_bits(sacc[kt][3])};
-            const bf16* vp = v_pool +
-                             kv_block(pages[key0 / page_tokens], n_layers, layer, kv_heads, kvh,
-                                      page_tokens, HD) +
-                             static_cast<size_t>(c) * page_tokens + (key0 % page_tokens) + 4 * qd;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const bf16x4_t a = *reinterpret_cast<const bf16x4_t*>(
-                    vp + static_cast<size_t>(dt) * 16 * page_tokens);
-                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, oacc[dt], 0, 0, 0);
-            }
+            for (int dt = 0; dt < DT; ++dt)
+                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[kt][dt], pb, oacc[dt], 0, 0, 0);
         }
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int st = 0; st < KS; ++st) kreg[kt][st] = knext[kt][st];
     }
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -166,13 +193,14 @@ extern "C" int celeg_attention_rows_bf16(
     int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int head_dim,
     int page_tokens, int n_layers, int layer, float scale, int window, hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
-    if (page_tokens % 16 || q_heads % kv_heads || (ldq % 4) || (ldo % 4))
+    if (page_tokens % 16 || q_heads % kv_heads || (ldq % 4) || (ldo % 4) || table_stride > 15360)
         return static_cast<int>(hipErrorInvalidValue);
     const int max_tiles = n_tokens / 64 + n_seqs;  // >= sum over requests of ceil(rows / 64)
     dim3 grid(max_tiles, q_heads), block(256);
+    const size_t lds = static_cast<size_t>(table_stride) * sizeof(int);
     const float scale_log2e = scale * 1.4426950408889634f;
 #define CELEG_ROWS(HD_)                                                                          \
-    hipLaunchKernelGGL(attention_rows_kernel<HD_>, grid, block, 0, stream,                       \
+    hipLaunchKernelGGL(attention_rows_kernel<HD_>, grid, block, lds, stream,                     \
                        static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
                        static_cast<const bf16*>(v_pool), table, table_stride, cu_seqlens,        \
                        seq_slot, seq_start, n_seqs, static_cast<bf16*>(out), ldo, q_heads,       \
