@@ -42,7 +42,8 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_start, int n_seqs, bf16* __restrict__ out, int ldo, int q_heads,
-    int kv_heads, int page_tokens, int n_layers, int layer, float scale_log2e, int window) {
+    int kv_heads, int page_tokens, int page_shift, int n_layers, int layer, float scale_log2e,
+    int window) {
     constexpr int DQ = HD / 4;   // dims a lane quad covers in q.k
     constexpr int KS = DQ / 4;   // MFMA steps along head_dim
     constexpr int DT = HD / 16;  // 16-dim tiles of the output
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
         // pages up to the last key this tile of rows can see
         const int last_key = start + min(tile * 64 + 63, len - 1);
         const int* __restrict__ pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
-        for (int i = threadIdx.x; i <= last_key / page_tokens; i += 256) spages[i] = pages[i];
+        for (int i = threadIdx.x; i <= last_key >> page_shift; i += 256) spages[i] = pages[i];
     }
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -94,34 +95,39 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
 
-    // keys of 64 positions from kb: lane (key c of tile kt, quad qd) reads DQ values
-    bf16x4_t kreg[4][KS], knext[4][KS];
+    // A tile of 16 keys lies in one page (page_tokens is a multiple of 16), so its page id
+    // is the same for every lane: it is read once into a scalar, and a lane's own offset
+    // inside the tile never changes.  Tiles beyond the last key are read from the last
+    // key's page (any place there is allocated memory) and masked.
+    const int last_page = kmax >> page_shift;
+    const size_t k_lane = static_cast<size_t>(c) * HD + qd * DQ;
+    const size_t v_lane = static_cast<size_t>(c) * page_tokens + 4 * qd;
     auto load_keys = [&](int kb, bf16x4_t (&dst)[4][KS]) {
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
-            const int key = min(kb + kt * 16 + c, kmax);  // a valid address; masked if beyond
-            const bf16* kp = k_pool + static_cast<size_t>(spages[key / page_tokens]) * page_stride +
-                             layer_head + static_cast<size_t>(key % page_tokens) * HD + qd * DQ;
+            const int key0 = kb + kt * 16;
+            const int page = __builtin_amdgcn_readfirstlane(spages[min(key0 >> page_shift, last_page)]);
+            const bf16* kp = k_pool + static_cast<size_t>(page) * page_stride + layer_head +
+                             static_cast<size_t>(key0 & (page_tokens - 1)) * HD + k_lane;
 #pragma unroll
             for (int st = 0; st < KS; ++st) dst[kt][st] = *reinterpret_cast<const bf16x4_t*>(kp + st * 4);
         }
     };
-    const int kb0 = (kmin >> 6) << 6;
-    load_keys(kb0, kreg);
-    for (int kb = kb0; kb <= kmax; kb += 64) {
+    const float neg_inf = -INFINITY;
+    auto round64 = [&](int kb, bf16x4_t (&kcur)[4][KS], bf16x4_t (&knxt)[4][KS]) {
         // values of this round: lane (dim c of tile dt, quad qd) reads 4 keys' values
         bf16x4_t vreg[4][DT];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
-            const int key0 = min(kb + kt * 16, kmax & ~15);
-            const bf16* vp = v_pool + static_cast<size_t>(spages[key0 / page_tokens]) * page_stride +
-                             layer_head + static_cast<size_t>(c) * page_tokens +
-                             (key0 % page_tokens) + 4 * qd;
+            const int key0 = kb + kt * 16;
+            const int page = __builtin_amdgcn_readfirstlane(spages[min(key0 >> page_shift, last_page)]);
+            const bf16* vp = v_pool + static_cast<size_t>(page) * page_stride + layer_head +
+                             (key0 & (page_tokens - 1)) + v_lane;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
                 vreg[kt][dt] = *reinterpret_cast<const bf16x4_t*>(vp + static_cast<size_t>(dt) * 16 * page_tokens);
         }
-        if (kb + 64 <= kmax) load_keys(kb + 64, knext);
+        if (kb + 64 <= kmax) load_keys(kb + 64, knxt);
 
         floatx4_t sacc[4];
 #pragma unroll
@@ -129,30 +135,39 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
             sacc[kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int st = 0; st < KS; ++st)
-                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[kt][st], qreg[st], sacc[kt], 0, 0, 0);
+                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kcur[kt][st], qreg[st], sacc[kt], 0, 0, 0);
         }
-        // sacc[kt][r] = (key kb + 16 kt + 4 qd + r) . (row c)
-        float mx = -INFINITY;
+        // sacc[kt][r] = (key kb + 16 kt + 4 qd + r) . (row c); rounds that lie wholly inside
+        // every row's range need no mask
+        const bool full = kb + 63 <= start + wrow0 && (window <= 0 || kb >= start + min(wrow0 + 15, len - 1) - window + 1);
+        float mx = neg_inf;
+        if (full) {
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+            for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = kb + kt * 16 + 4 * qd + r;
-                const float sv = (key <= pq && key >= lo_q) ? sacc[kt][r] * scale_log2e : -INFINITY;
-                sacc[kt][r] = sv;
-                mx = fmaxf(mx, sv);
-            }
+                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sacc[kt][r]);
+        } else {
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = kb + kt * 16 + 4 * qd + r;
+                    const float sv = (key <= pq && key >= lo_q) ? sacc[kt][r] : neg_inf;
+                    sacc[kt][r] = sv;
+                    mx = fmaxf(mx, sv);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row that has seen no key yet
-        const float alpha = exp2f(m - m_use);
+        const float m_new = fmaxf(m, mx * scale_log2e);          // the scale is positive
+        const float m_use = m_new == neg_inf ? 0.f : m_new;      // a row that has seen no key yet
+        const float alpha = __builtin_amdgcn_exp2f(m - m_use);
         float psum = 0.f;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float p = exp2f(sacc[kt][r] - m_use);
+                const float p = __builtin_amdgcn_exp2f(fmaf(sacc[kt][r], scale_log2e, -m_use));
                 sacc[kt][r] = p;
                 psum += p;
             }
@@ -162,17 +177,23 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
         for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
-            // a tile beyond the last key was read from the last tile's place: its p are zero
             const bf16x4_t pb = {bf16_bits(sacc[kt][0]), bf16_bits(sacc[kt][1]),
                                  bf16_bits(sacc[kt][2]), bf16_bits(sacc[kt][3])};
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
                 oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[kt][dt], pb, oacc[dt], 0, 0, 0);
         }
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-            for (int st = 0; st < KS; ++st) kreg[kt][st] = knext[kt][st];
+    };
+    // two sets of key registers take turns: one is multiplied while the other is filled
+    bf16x4_t kreg_a[4][KS], kreg_b[4][KS];
+    int kb = (kmin >> 6) << 6;
+    load_keys(kb, kreg_a);
+    while (kb <= kmax) {
+        round64(kb, kreg_a, kreg_b);
+        kb += 64;
+        if (kb > kmax) break;
+        round64(kb, kreg_b, kreg_a);
+        kb += 64;
     }
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -193,8 +214,10 @@ extern "C" int celeg_attention_rows_bf16(
     int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int head_dim,
     int page_tokens, int n_layers, int layer, float scale, int window, hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
-    if (page_tokens % 16 || q_heads % kv_heads || (ldq % 4) || (ldo % 4) || table_stride > 15360)
+    if (page_tokens < 16 || (page_tokens & (page_tokens - 1)) || q_heads % kv_heads || (ldq % 4) ||
+        (ldo % 4) || table_stride > 15360)
         return static_cast<int>(hipErrorInvalidValue);
+    const int page_shift = __builtin_ctz(page_tokens);
     const int max_tiles = n_tokens / 64 + n_seqs;  // >= sum over requests of ceil(rows / 64)
     dim3 grid(max_tiles, q_heads), block(256);
     const size_t lds = static_cast<size_t>(table_stride) * sizeof(int);
@@ -204,7 +227,7 @@ extern "C" int celeg_attention_rows_bf16(
                        static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
                        static_cast<const bf16*>(v_pool), table, table_stride, cu_seqlens,        \
                        seq_slot, seq_start, n_seqs, static_cast<bf16*>(out), ldo, q_heads,       \
-                       kv_heads, page_tokens, n_layers, layer, scale_log2e, window)
+                       kv_heads, page_tokens, page_shift, n_layers, layer, scale_log2e, window)
     switch (head_dim) {
         case 32: CELEG_ROWS(32); break;
         case 64: CELEG_ROWS(64); break;
@@ -231,7 +254,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ token_slot, const int* __restrict__ positions,
     float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
-    int q_heads, int kv_heads, int page_tokens, int n_layers, int layer, float scale, int window) {
+    int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer, float scale,
+    int window) {
     constexpr int DL = HD / 8;    // dims of a key a lane multiplies
     constexpr int DD = HD / 64;   // output dims a lane accumulates
     __shared__ float ps[GH][DEC_KEYS];
@@ -249,8 +273,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
 
     // page ids of the chunk: lane i holds the i-th page that the 64 keys touch
-    const int first_page = kb / page_tokens;
-    const int last_page = k_hi / page_tokens;
+    const int first_page = kb >> page_shift;
+    const int last_page = k_hi >> page_shift;
     const int my_page = pages[min(first_page + lane, last_page)];
 
     // keys: 8 rounds of 8 keys, a lane reads DL values of its key
@@ -258,9 +282,9 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 #pragma unroll
     for (int it = 0; it < 8; ++it) {
         const int keyc = min(max(kb + it * 8 + j8, k_lo), k_hi);
-        const int page = __shfl(my_page, keyc / page_tokens - first_page, 64);
+        const int page = __shfl(my_page, (keyc >> page_shift) - first_page, 64);
         const bf16* kp = k_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
-                         static_cast<size_t>(keyc % page_tokens) * HD + seg * DL;
+                         static_cast<size_t>(keyc & (page_tokens - 1)) * HD + seg * DL;
 #pragma unroll
         for (int v8 = 0; v8 < DL / 8; ++v8) kraw[it][v8] = *reinterpret_cast<const uint4*>(kp + v8 * 8);
     }
@@ -269,9 +293,9 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 #pragma unroll
     for (int pg = 0; pg < 4; ++pg) {
         const int key0 = min(max(kb + pg * 16, k_lo & ~15), k_hi & ~15);   // a group inside the range
-        const int page = __shfl(my_page, key0 / page_tokens - first_page, 64);
+        const int page = __shfl(my_page, (key0 >> page_shift) - first_page, 64);
         const bf16* vbase = v_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
-                            (key0 % page_tokens);
+                            (key0 & (page_tokens - 1));
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd)
 #pragma unroll
@@ -433,8 +457,10 @@ extern "C" int celeg_attention_decode_bf16(
     hipStream_t stream) {
     if (n_rows <= 0) return 0;
     const int group = q_heads / kv_heads;
-    if (q_heads % kv_heads || page_tokens % 16 || n_splits <= 0 || (ldq % 8))
+    if (q_heads % kv_heads || page_tokens < 16 || (page_tokens & (page_tokens - 1)) || n_splits <= 0 ||
+        (ldq % 8))
         return static_cast<int>(hipErrorInvalidValue);
+    const int page_shift = __builtin_ctz(page_tokens);
     const int gh = (group % 4 == 0) ? 4 : ((group % 2 == 0) ? 2 : 1);
     dim3 grid(n_splits, q_heads / gh, n_rows), block(64);
 #define CELEG_DEC(HD_, GH_)                                                                      \
@@ -442,7 +468,7 @@ extern "C" int celeg_attention_decode_bf16(
                        static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
                        static_cast<const bf16*>(v_pool), table, table_stride, token_slot,        \
                        positions, ws_o, ws_ml, n_splits, q_heads, kv_heads,                      \
-                       page_tokens, n_layers, layer, scale, window)
+                       page_tokens, page_shift, n_layers, layer, scale, window)
 #define CELEG_DEC_HD(HD_)                                                                        \
     if (gh == 4) CELEG_DEC(HD_, 4); else if (gh == 2) CELEG_DEC(HD_, 2); else CELEG_DEC(HD_, 1);  \
     hipLaunchKernelGGL(attention_decode_reduce_kernel<HD_>, dim3(q_heads, n_rows), dim3(64), 0,  \

@@ -289,7 +289,8 @@ class HipOps:
             raise KernelError("paged_attention: heads must be a multiple of kv_heads")
         self._check_kv(kv, kv_heads, head_dim, q.dtype)
         if q.dtype == torch.bfloat16 and self.attention_impl != "general" \
-                and kv.page_tokens % 16 == 0 and self._rows(q, "q") % 8 == 0:
+                and kv.page_tokens >= 16 and kv.page_tokens & (kv.page_tokens - 1) == 0 \
+                and self._rows(q, "q") % 8 == 0:
             if batch.decode_only and head_dim in (64, 128) and batch.n_seqs == T:
                 return self._attention_decode(q, out, heads, kv_heads, head_dim, scale, window,
                                               batch, kv)
