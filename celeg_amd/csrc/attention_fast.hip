@@ -17,8 +17,11 @@
 // src/backend/cuda/kernels/attention_paged.cuh:287-487.
 #include "common.h"
 
-typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
+// (arrays of HIP's own uint4 class are not always kept in registers; this type is)
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ size_t kv_block(int page, int n_layers, int layer, int kv_heads,
                                            int head, int page_tokens, int head_dim) {
@@ -26,217 +29,347 @@ __device__ __forceinline__ size_t kv_block(int page, int n_layers, int layer, in
            static_cast<size_t>(page_tokens) * head_dim;
 }
 
-__device__ __forceinline__ short bf16_bits(float x) { return static_cast<short>(from_float<bf16>(x).bits); }
+// Rows a workgroup of the portion kernel takes when the caller leaves the choice open.
+#define CELEG_ROWS_DEFAULT(n_tokens, n_seqs) 64
+
+
+// Combining a value with the one that lane ^ 16 (lane ^ 32) holds, by the lane-swap
+// instructions of gfx950: both operands start as x; the swap leaves (row 0, row 0, row 2,
+// row 2) in one and (row 1, row 1, row 3, row 3) in the other (rows of 16 lanes; halves of
+// 32 lanes likewise), so the two results are the lane's own value and its partner's.
+__device__ __forceinline__ float max_row16(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_half32(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_row16(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_half32(float x) {
+    const unsigned u = __float_as_uint(x);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 // ================================================================ rows of portions
-// One workgroup of 4 wavefronts per (tile of 64 rows of one request, query head); a
-// wavefront owns 16 rows.  Per 64 keys: S^T = K Q^T (16x16x16 MFMA: A = 16 keys x 16
-// dims, B = 16 dims x 16 rows), online softmax per row (a row is a lane column), then
-// O^T += V^T P^T (A = 16 dims x 16 keys from the transposed V, B = P^T straight from the
-// accumulator registers of S^T).  The request's page ids are put into LDS once; the keys
-// of the next 64 are asked for while the current 64 are worked on, and the values of the
-// current 64 before its scores are computed.
-template <int HD>
-__global__ __launch_bounds__(256) void attention_rows_kernel(
+// A tile is 64*RT rows of one request for one query head; 4 wavefronts work on it, each
+// on RT tiles of 16 rows.  A workgroup of 8 wavefronts takes two tiles of a request, the
+// i-th from the front and the i-th from the back: under the causal mask their key counts
+// add up to the same for every pair, and the wavefronts are spread over the SIMDs so that
+// each SIMD gets one of either tile.  The keys and values of 64 positions are staged in
+// LDS once for the 4 wavefronts of a tile (two buffers: the next 64 are fetched into registers
+// while the current 64 are worked on, and written to the other buffer before the one
+// barrier of the round).  Per 64 keys: S^T = K Q^T (16x16x32 MFMA: A = 16 keys x 32 dims,
+// B = 32 dims x 16 rows), online softmax per row (a row is a lane column), then
+// O^T += V^T P^T (A = 16 dims x 32 keys from the transposed V, B = P^T straight from the
+// accumulator registers of S^T).  The 16 keys of a score tile are chosen so that a lane
+// ends up with the probabilities of 8 neighbouring keys, which is what one 16-byte read
+// of the transposed V delivers.
+template <int HD, int RT>
+__global__ __launch_bounds__(512) void attention_rows_kernel(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
-    const int* __restrict__ seq_start, int n_seqs, bf16* __restrict__ out, int ldo, int q_heads,
-    int kv_heads, int page_tokens, int page_shift, int n_layers, int layer, float scale_log2e,
-    int window) {
-    constexpr int DQ = HD / 4;   // dims a lane quad covers in q.k
-    constexpr int KS = DQ / 4;   // MFMA steps along head_dim
-    constexpr int DT = HD / 16;  // 16-dim tiles of the output
-    extern __shared__ int spages[];   // table_stride page ids
-    int tile = blockIdx.x;
+    const int* __restrict__ seq_start, int n_seqs, bf16* __restrict__ out, int ldo,
+    int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer,
+    float scale_log2e, int window) {
+    constexpr int ROWS = 64 * RT;   // rows of a workgroup
+    constexpr int WROWS = 16 * RT;  // rows of a wavefront
+    constexpr int DQ = HD / 4;      // dims a lane quad covers in q.k
+    constexpr int KS = DQ / 8;      // MFMA steps of 32 along head_dim
+    constexpr int DT = HD / 16;     // 16-dim tiles of the output
+    constexpr int KROW = HD + 8;    // LDS row of a key, padded against bank conflicts
+    constexpr int VROW = 64 + 8;    // LDS row of a dimension: 64 keys, padded
+    constexpr int CH = HD / 32;     // 16-byte pieces of K, and of V, a thread moves per round
+    extern __shared__ int smem[];
+    const int half = threadIdx.x >> 8, tid = threadIdx.x & 255;
+    __bf16* const sK = reinterpret_cast<__bf16*>(smem) + half * (2 * 64 * KROW);       // [2][2][64][KROW]
+    __bf16* const sV = reinterpret_cast<__bf16*>(smem) + 4 * 64 * KROW + half * (2 * HD * VROW);  // [2][2][HD][VROW]
+    int* const spages = reinterpret_cast<int*>(reinterpret_cast<__bf16*>(smem) + 4 * 64 * KROW + 4 * HD * VROW);
+    int pair = blockIdx.x;
     const int h = blockIdx.y;
-    int s = 0, len = 0;
+    int s = 0, len = 0, tiles = 0;
     bool found = false;
     for (; s < n_seqs; ++s) {
         len = cu_seqlens[s + 1] - cu_seqlens[s];
-        const int tiles = (len + 63) >> 6;
-        if (tile < tiles) { found = true; break; }
-        tile -= tiles;
+        tiles = (len + ROWS - 1) / ROWS;
+        if (pair < (tiles + 1) / 2) { found = true; break; }
+        pair -= (tiles + 1) / 2;
     }
     if (!found) return;   // the whole workgroup
     const int start = seq_start[s];
+    // first round and number of rounds of a tile of rows
+    auto first_key = [&](int t) { return ((window > 0 ? max(0, start + t * ROWS - window + 1) : 0) >> 6) << 6; };
+    auto last_key = [&](int t) { return start + min(t * ROWS + ROWS - 1, len - 1); };
+    const int heavy = tiles - 1 - pair;
+    const bool has_tile = half == 1 || pair != heavy;   // the middle tile of an odd count has no partner
+    const int tile = half == 1 ? heavy : pair;
+    const int rounds_heavy = ((last_key(heavy) - first_key(heavy)) >> 6) + 1;
+    const int rounds_light = pair != heavy ? ((last_key(pair) - first_key(pair)) >> 6) + 1 : 0;
+    const int n_rounds = max(rounds_heavy, rounds_light);
+    const int my_rounds = half == 1 ? rounds_heavy : rounds_light;
+    const int brow0 = tile * ROWS;
+    const int bkmax = last_key(tile);             // last key this half sees
+    const int last_page = bkmax >> page_shift;
     {
-        // pages up to the last key this tile of rows can see
-        const int last_key = start + min(tile * 64 + 63, len - 1);
         const int* __restrict__ pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
-        for (int i = threadIdx.x; i <= last_key >> page_shift; i += 256) spages[i] = pages[i];
+        for (int i = threadIdx.x; i <= last_key(heavy) >> page_shift; i += 512) spages[i] = pages[i];
     }
     __syncthreads();
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = tid >> 6, lane = tid & 63;
     const int c = lane & 15, qd = lane >> 4;
-    const int wrow0 = tile * 64 + wave * 16;
-    if (wrow0 >= len) return;  // no row of this wavefront exists (no barrier is used below)
-    const int row = wrow0 + c;
-    const bool row_valid = row < len;
-    const int row_c = row_valid ? row : len - 1;
-    const int pq = start + row_c;                       // this lane's row position
-    const int lo_q = window > 0 ? max(0, pq - window + 1) : 0;
-    const int kmax = start + min(wrow0 + 15, len - 1);  // last key any row of the wavefront sees
-    const int kmin = window > 0 ? max(0, start + wrow0 - window + 1) : 0;
+    const int wrow0 = brow0 + wave * WROWS;
+    const bool wave_active = has_tile && wrow0 < len;
+    const int wkmax = start + min(wrow0 + WROWS - 1, len - 1);  // last key any row of the wavefront sees
+    const int wkmin = window > 0 ? max(0, start + wrow0 - window + 1) : 0;
     const int kvh = h / (q_heads / kv_heads);
     const size_t row_base = static_cast<size_t>(cu_seqlens[s]);
     const size_t head_block = static_cast<size_t>(page_tokens) * HD;
     const size_t page_stride = static_cast<size_t>(n_layers) * kv_heads * head_block;
     const size_t layer_head = (static_cast<size_t>(layer) * kv_heads + kvh) * head_block;
 
-    bf16x4_t qreg[KS];
-    {
+    int pq[RT], lo_q[RT];
+    bool row_valid[RT];
+    bf16x8_t qreg[RT][KS];
+    floatx4_t oacc[RT][DT];
+    float m[RT], l[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = wrow0 + rt * 16 + c;
+        row_valid[rt] = row < len;
+        const int row_c = row_valid[rt] ? row : len - 1;
+        pq[rt] = start + row_c;
+        lo_q[rt] = window > 0 ? max(0, pq[rt] - window + 1) : 0;
         const bf16* qrow = q + (row_base + row_c) * ldq + static_cast<size_t>(h) * HD + qd * DQ;
 #pragma unroll
-        for (int st = 0; st < KS; ++st) qreg[st] = *reinterpret_cast<const bf16x4_t*>(qrow + st * 4);
+        for (int st = 0; st < KS; ++st) qreg[rt][st] = *reinterpret_cast<const bf16x8_t*>(qrow + st * 8);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        m[rt] = -INFINITY;
+        l[rt] = 0.f;
     }
-    floatx4_t oacc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) oacc[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, l = 0.f;
 
-    // A tile of 16 keys lies in one page (page_tokens is a multiple of 16), so its page id
-    // is the same for every lane: it is read once into a scalar, and a lane's own offset
-    // inside the tile never changes.  Tiles beyond the last key are read from the last
-    // key's page (any place there is allocated memory) and masked.
-    const int last_page = kmax >> page_shift;
-    const size_t k_lane = static_cast<size_t>(c) * HD + qd * DQ;
-    const size_t v_lane = static_cast<size_t>(c) * page_tokens + 4 * qd;
-    auto load_keys = [&](int kb, bf16x4_t (&dst)[4][KS]) {
+    // What a thread moves per round: piece i of K is 8 dims of one key; piece i of V is 8
+    // keys of one dimension, walked page by page so that neighbouring threads read
+    // neighbouring memory.  Positions beyond the last key are read from the last key's
+    // page (allocated memory) and masked.
+    const int pt_shift = min(page_shift, 6);          // keys of a page inside a round: 1 << pt_shift
+    u32x4_t kstage[CH], vstage[CH];
+    auto fetch = [&](int kb) __attribute__((always_inline)) {
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-            const int key0 = kb + kt * 16;
-            const int page = __builtin_amdgcn_readfirstlane(spages[min(key0 >> page_shift, last_page)]);
-            const bf16* kp = k_pool + static_cast<size_t>(page) * page_stride + layer_head +
-                             static_cast<size_t>(key0 & (page_tokens - 1)) * HD + k_lane;
+        for (int j = 0; j < CH; ++j) {
+            const int i = tid + 256 * j;
+            {
+                const int key = kb + i / (HD / 8), part = i % (HD / 8);
+                const int page = spages[min(key >> page_shift, last_page)];
+                kstage[j] = *reinterpret_cast<const u32x4_t*>(
+                    k_pool + static_cast<size_t>(page) * page_stride + layer_head +
+                    static_cast<size_t>(key & (page_tokens - 1)) * HD + part * 8);
+            }
+            {
+                const int per_dim = 1 << (pt_shift - 3);           // pieces of a dimension inside a page
+                const int piece = (i >> (pt_shift - 3)) / HD;      // which page of the round
+                const int rem = i - piece * (HD << (pt_shift - 3));
+                const int d = rem >> (pt_shift - 3), g = rem & (per_dim - 1);
+                const int key0 = kb + (piece << pt_shift) + g * 8;
+                const int page = spages[min(key0 >> page_shift, last_page)];
+                vstage[j] = *reinterpret_cast<const u32x4_t*>(
+                    v_pool + static_cast<size_t>(page) * page_stride + layer_head +
+                    static_cast<size_t>(d) * page_tokens + (key0 & (page_tokens - 1)));
+            }
+        }
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
-            for (int st = 0; st < KS; ++st) dst[kt][st] = *reinterpret_cast<const bf16x4_t*>(kp + st * 4);
+        for (int j = 0; j < CH; ++j) {
+            const int i = tid + 256 * j;
+            *reinterpret_cast<u32x4_t*>(sK + (buf * 64 + i / (HD / 8)) * KROW + (i % (HD / 8)) * 8) = kstage[j];
+            const int per_dim = 1 << (pt_shift - 3);
+            const int piece = (i >> (pt_shift - 3)) / HD;
+            const int rem = i - piece * (HD << (pt_shift - 3));
+            const int d = rem >> (pt_shift - 3), g = rem & (per_dim - 1);
+            *reinterpret_cast<u32x4_t*>(sV + (buf * HD + d) * VROW + (piece << pt_shift) + g * 8) = vstage[j];
         }
     };
     const float neg_inf = -INFINITY;
-    auto round64 = [&](int kb, bf16x4_t (&kcur)[4][KS], bf16x4_t (&knxt)[4][KS]) {
-        // values of this round: lane (dim c of tile dt, quad qd) reads 4 keys' values
-        bf16x4_t vreg[4][DT];
+    // score tile kt, A row i  <->  key 32 (kt/2) + 8 (i/4) + 4 (kt%2) + i%4 of the round, so
+    // that accumulator register r of lane quad qd is key 32 (kt/2) + 8 qd + 4 (kt%2) + r
+    auto compute = [&](int kb, int buf) __attribute__((always_inline)) {
+        floatx4_t sacc[RT][4];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) sacc[rt][kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
-            const int key0 = kb + kt * 16;
-            const int page = __builtin_amdgcn_readfirstlane(spages[min(key0 >> page_shift, last_page)]);
-            const bf16* vp = v_pool + static_cast<size_t>(page) * page_stride + layer_head +
-                             (key0 & (page_tokens - 1)) + v_lane;
+            const int key_row = 32 * (kt >> 1) + 8 * (c >> 2) + 4 * (kt & 1) + (c & 3);
+            const __bf16* kp = sK + (buf * 64 + key_row) * KROW + qd * DQ;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                vreg[kt][dt] = *reinterpret_cast<const bf16x4_t*>(vp + static_cast<size_t>(dt) * 16 * page_tokens);
+            for (int st = 0; st < KS; ++st) {
+                const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kp + st * 8);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    sacc[rt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qreg[rt][st], sacc[rt][kt], 0, 0, 0);
+            }
         }
-        if (kb + 64 <= kmax) load_keys(kb + 64, knxt);
-
-        floatx4_t sacc[4];
+        bf16x8_t pb[RT][2];
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-            sacc[kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        for (int rt = 0; rt < RT; ++rt) {
+            // rounds that lie wholly inside every row's range need no mask
+            const int first_row = start + wrow0 + rt * 16;
+            const bool full = kb + 63 <= first_row &&
+                              (window <= 0 || kb >= min(first_row + 15, start + len - 1) - window + 1);
+            float mx = neg_inf;
+            if (full) {
 #pragma unroll
-            for (int st = 0; st < KS; ++st)
-                sacc[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kcur[kt][st], qreg[st], sacc[kt], 0, 0, 0);
-        }
-        // sacc[kt][r] = (key kb + 16 kt + 4 qd + r) . (row c); rounds that lie wholly inside
-        // every row's range need no mask
-        const bool full = kb + 63 <= start + wrow0 && (window <= 0 || kb >= start + min(wrow0 + 15, len - 1) - window + 1);
-        float mx = neg_inf;
-        if (full) {
+                for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-            for (int kt = 0; kt < 4; ++kt)
+                    for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sacc[rt][kt][r]);
+            } else {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sacc[kt][r]);
-        } else {
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = kb + 32 * (kt >> 1) + 8 * qd + 4 * (kt & 1) + r;
+                        const float sv = (key <= pq[rt] && key >= lo_q[rt]) ? sacc[rt][kt][r] : neg_inf;
+                        sacc[rt][kt][r] = sv;
+                        mx = fmaxf(mx, sv);
+                    }
+            }
+            mx = max_half32(max_row16(mx));
+            const float m_new = fmaxf(m[rt], mx * scale_log2e);      // the scale is positive
+            const float m_use = m_new == neg_inf ? 0.f : m_new;      // a row that has seen no key yet
+            const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);
+            float psum = 0.f;
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int key = kb + kt * 16 + 4 * qd + r;
-                    const float sv = (key <= pq && key >= lo_q) ? sacc[kt][r] : neg_inf;
-                    sacc[kt][r] = sv;
-                    mx = fmaxf(mx, sv);
+                    const float p = __builtin_amdgcn_exp2f(fmaf(sacc[rt][kt][r], scale_log2e, -m_use));
+                    sacc[rt][kt][r] = p;
+                    psum += p;
                 }
+            l[rt] = l[rt] * alpha + psum;
+            m[rt] = m_new;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] *= alpha;
+#pragma unroll
+            for (int kp = 0; kp < 2; ++kp)
+                pb[rt][kp] = bf16x8_t{
+                    static_cast<__bf16>(sacc[rt][2 * kp][0]), static_cast<__bf16>(sacc[rt][2 * kp][1]),
+                    static_cast<__bf16>(sacc[rt][2 * kp][2]), static_cast<__bf16>(sacc[rt][2 * kp][3]),
+                    static_cast<__bf16>(sacc[rt][2 * kp + 1][0]), static_cast<__bf16>(sacc[rt][2 * kp + 1][1]),
+                    static_cast<__bf16>(sacc[rt][2 * kp + 1][2]), static_cast<__bf16>(sacc[rt][2 * kp + 1][3])};
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx * scale_log2e);          // the scale is positive
-        const float m_use = m_new == neg_inf ? 0.f : m_new;      // a row that has seen no key yet
-        const float alpha = __builtin_amdgcn_exp2f(m - m_use);
-        float psum = 0.f;
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int kp = 0; kp < 2; ++kp)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float p = __builtin_amdgcn_exp2f(fmaf(sacc[kt][r], scale_log2e, -m_use));
-                sacc[kt][r] = p;
-                psum += p;
+            for (int dt = 0; dt < DT; ++dt) {
+                const bf16x8_t vf = *reinterpret_cast<const bf16x8_t*>(
+                    sV + (buf * HD + dt * 16 + c) * VROW + 32 * kp + 8 * qd);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    oacc[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[rt][kp], oacc[rt][dt], 0, 0, 0);
             }
-        l = l * alpha + psum;
-        m = m_new;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) oacc[dt] *= alpha;
-#pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
-            const bf16x4_t pb = {bf16_bits(sacc[kt][0]), bf16_bits(sacc[kt][1]),
-                                 bf16_bits(sacc[kt][2]), bf16_bits(sacc[kt][3])};
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                oacc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[kt][dt], pb, oacc[dt], 0, 0, 0);
-        }
     };
-    // two sets of key registers take turns: one is multiplied while the other is filled
-    bf16x4_t kreg_a[4][KS], kreg_b[4][KS];
-    int kb = (kmin >> 6) << 6;
-    load_keys(kb, kreg_a);
-    while (kb <= kmax) {
-        round64(kb, kreg_a, kreg_b);
-        kb += 64;
-        if (kb > kmax) break;
-        round64(kb, kreg_b, kreg_a);
-        kb += 64;
+
+    // Round r works on LDS buffer r % 2 while the registers hold round r + 1 (asked for a
+    // whole round earlier); at its end they go to the other buffer and round r + 2 is asked
+    // for.  Both halves pass the same barriers; the one with fewer rounds idles at the end.
+    int kb = first_key(tile);
+    int buf = 0;
+    if (my_rounds > 0) { fetch(kb); stage(0); }
+    if (my_rounds > 1) fetch(kb + 64);
+    __syncthreads();
+    for (int it = 0; it < n_rounds; ++it, kb += 64) {
+        if (it < my_rounds && wave_active && kb <= wkmax && kb + 63 >= wkmin) compute(kb, buf);
+        if (it + 1 < my_rounds) {
+            stage(buf ^ 1);
+            if (it + 2 < my_rounds) fetch(kb + 128);
+        }
+        __syncthreads();
+        buf ^= 1;
     }
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    if (!row_valid) return;
-    const float inv_l = 1.0f / l;
-    bf16* orow = out + (row_base + row) * ldo + static_cast<size_t>(h) * HD + 4 * qd;
+    if (!wave_active) return;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        const bf16x4_t o = {bf16_bits(oacc[dt][0] * inv_l), bf16_bits(oacc[dt][1] * inv_l),
-                            bf16_bits(oacc[dt][2] * inv_l), bf16_bits(oacc[dt][3] * inv_l)};
-        *reinterpret_cast<bf16x4_t*>(orow + dt * 16) = o;
+    for (int rt = 0; rt < RT; ++rt) {
+        float lt = l[rt];
+        lt = sum_half32(sum_row16(lt));
+        if (!row_valid[rt]) continue;
+        const float inv_l = 1.0f / lt;
+        bf16* orow = out + (row_base + wrow0 + rt * 16 + c) * ldo + static_cast<size_t>(h) * HD + 4 * qd;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x4_t o = {static_cast<__bf16>(oacc[rt][dt][0] * inv_l), static_cast<__bf16>(oacc[rt][dt][1] * inv_l),
+                                static_cast<__bf16>(oacc[rt][dt][2] * inv_l), static_cast<__bf16>(oacc[rt][dt][3] * inv_l)};
+            *reinterpret_cast<bf16x4_t*>(orow + dt * 16) = o;
+        }
     }
 }
 
+template <int HD, int RT>
+static int launch_attention_rows(
+    const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+    int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
+    int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int page_tokens,
+    int n_layers, int layer, float scale, int window, hipStream_t stream) {
+    const size_t lds = (4 * 64 * (HD + 8) + 4 * HD * (64 + 8)) * sizeof(bf16) +
+                       static_cast<size_t>(table_stride) * sizeof(int);
+    if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
+    auto kernel = attention_rows_kernel<HD, RT>;
+    if (lds > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 static_cast<int>(lds));
+        if (e != hipSuccess) return static_cast<int>(e);
+    }
+    // >= sum over requests of ceil(tiles / 2), tiles = ceil(rows / (64 RT))
+    const int max_pairs = (n_tokens / (64 * RT) + 2 * n_seqs + 1) / 2;
+    dim3 grid(max_pairs, q_heads), block(512);
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,
+                       static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
+                       table_stride, cu_seqlens, seq_slot, seq_start, n_seqs,
+                       static_cast<bf16*>(out), ldo, q_heads, kv_heads, page_tokens,
+                       __builtin_ctz(page_tokens), n_layers, layer, scale * 1.4426950408889634f, window);
+    return CELEG_LAUNCH_RESULT();
+}
+
+// rows_per_tile: 64 or 128 rows a workgroup (0: chosen from the number of rows).
 extern "C" int celeg_attention_rows_bf16(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
     int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int head_dim,
-    int page_tokens, int n_layers, int layer, float scale, int window, hipStream_t stream) {
+    int page_tokens, int n_layers, int layer, float scale, int window, int rows_per_tile,
+    hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
-    if (page_tokens < 16 || (page_tokens & (page_tokens - 1)) || q_heads % kv_heads || (ldq % 4) ||
-        (ldo % 4) || table_stride > 15360)
+    if (page_tokens < 16 || (page_tokens & (page_tokens - 1)) || q_heads % kv_heads || (ldq % 8) ||
+        (ldo % 4))
         return static_cast<int>(hipErrorInvalidValue);
-    const int page_shift = __builtin_ctz(page_tokens);
-    const int max_tiles = n_tokens / 64 + n_seqs;  // >= sum over requests of ceil(rows / 64)
-    dim3 grid(max_tiles, q_heads), block(256);
-    const size_t lds = static_cast<size_t>(table_stride) * sizeof(int);
-    const float scale_log2e = scale * 1.4426950408889634f;
+    if (rows_per_tile == 0) rows_per_tile = CELEG_ROWS_DEFAULT(n_tokens, n_seqs);
+    if (rows_per_tile != 64 && rows_per_tile != 128) return static_cast<int>(hipErrorInvalidValue);
 #define CELEG_ROWS(HD_)                                                                          \
-    hipLaunchKernelGGL(attention_rows_kernel<HD_>, grid, block, lds, stream,                     \
-                       static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
-                       static_cast<const bf16*>(v_pool), table, table_stride, cu_seqlens,        \
-                       seq_slot, seq_start, n_seqs, static_cast<bf16*>(out), ldo, q_heads,       \
-                       kv_heads, page_tokens, page_shift, n_layers, layer, scale_log2e, window)
+    return rows_per_tile == 64                                                                   \
+        ? launch_attention_rows<HD_, 1>(q, ldq, k_pool, v_pool, table, table_stride, cu_seqlens, \
+              seq_slot, seq_start, n_seqs, n_tokens, out, ldo, q_heads, kv_heads, page_tokens,   \
+              n_layers, layer, scale, window, stream)                                            \
+        : launch_attention_rows<HD_, 2>(q, ldq, k_pool, v_pool, table, table_stride, cu_seqlens, \
+              seq_slot, seq_start, n_seqs, n_tokens, out, ldo, q_heads, kv_heads, page_tokens,   \
+              n_layers, layer, scale, window, stream)
     switch (head_dim) {
-        case 32: CELEG_ROWS(32); break;
-        case 64: CELEG_ROWS(64); break;
-        case 96: CELEG_ROWS(96); break;
-        case 128: CELEG_ROWS(128); break;
+        case 32: CELEG_ROWS(32);
+        case 64: CELEG_ROWS(64);
+        case 96: CELEG_ROWS(96);
+        case 128: CELEG_ROWS(128);
         default: return static_cast<int>(hipErrorInvalidValue);
     }
 #undef CELEG_ROWS
-    return CELEG_LAUNCH_RESULT();
 }
 
 // ================================================================ one row per request

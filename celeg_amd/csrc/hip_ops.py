@@ -42,6 +42,7 @@ class HipOps:
         self.loaded_libraries: Dict[str, str] = {}
         # "auto": the matrix-core and split-key kernels where they apply; "general": always
         # the general kernel (tests compare the two)
+        self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
         self.attention_impl = "auto"
         self._decode_ws = None
         self._retired = []
@@ -301,7 +302,8 @@ class HipOps:
                     _ptr(batch.seq_start), _c_int(batch.n_seqs), _c_int(T), _ptr(out),
                     _c_int(heads * head_dim), _c_int(heads), _c_int(kv_heads), _c_int(head_dim),
                     _c_int(kv.page_tokens), _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
-                    _c_int(window if window else 0), self._stream())
+                    _c_int(window if window else 0), _c_int(self.attention_rows_per_tile),
+                    self._stream())
                 self._check(code, "attention over rows (bfloat16)")
                 return
         code = self._lib("attention").celeg_paged_attention(

@@ -318,3 +318,24 @@ def test_attention_window_fast_kernels(ops):
                    window=70, boost=(31, 100), qk_norm=False, rotary_dim=0, page_tokens=32)
     attention_case(ops, torch.bfloat16, 4, 2, 64, lengths=[260], cuts=[100, 1, 1, 60, 1],
                    window=70, boost=(31, 101), qk_norm=False, rotary_dim=0, page_tokens=32)
+
+
+@pytest.mark.parametrize("rows_per_tile", [64, 128])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [
+    (4, 2, 64, 16), (2, 1, 128, 32), (3, 3, 96, 16), (4, 1, 32, 64)])
+def test_attention_rows_tile_pairs(ops, rows_per_tile, heads, kv_heads, head_dim, page_tokens):
+    """Portions of many row tiles (an odd and an even number of them, so that a tile with
+    and without a partner occurs), continued at a position inside a tile, at either tile
+    size; then the same with a window that ends inside a round of keys."""
+    ops.attention_rows_per_tile = rows_per_tile
+    try:
+        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[717, 150, 390],
+                       cuts=[330, 61, 200], boost=(2, 700), page_tokens=page_tokens)
+        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[500],
+                       cuts=[270, 230], window=150, boost=(301, 450), qk_norm=False, rotary_dim=0,
+                       page_tokens=page_tokens)
+        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[500],
+                       cuts=[270, 230], window=150, boost=(300, 450), qk_norm=False, rotary_dim=0,
+                       page_tokens=page_tokens)
+    finally:
+        ops.attention_rows_per_tile = 0
