@@ -72,6 +72,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
+                    help="for profiling: run only the prefill measurement, or only the batch-8 "
+                         "decode measurement (the line printed then holds only that part)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported "
@@ -90,7 +93,7 @@ def main() -> int:
         cfg["num_hidden_layers"] = args.layers
         cfg["layer_types"] = cfg["layer_types"][:args.layers]
     context = cfg["max_position_embeddings"]
-    max_batch = BATCH if args.no_points else 64
+    max_batch = BATCH if args.no_points or args.phase != "all" else 64
     need = PROMPT_TOKENS + args.steps + args.warmup + 1
     if need > context:
         raise SystemExit(f"--steps + --warmup exceed the context of {context}")
@@ -104,8 +107,17 @@ def main() -> int:
     w_bytes = weight_bytes(lm.model)
     kv_per_token = lm.cache.layout.kv_bytes_per_token(2)
 
-    prefill = measure_prefill(lm, PROMPT_TOKENS, repeats=7, warmup=3)
     flops = prefill_flops(cfg, PROMPT_TOKENS, ff)
+    if args.phase == "decode":
+        prefill = None
+    else:
+        prefill = measure_prefill(lm, PROMPT_TOKENS, repeats=7, warmup=3)
+    if args.phase == "prefill":
+        print(json.dumps({"metric": "prefill tok/s @ 2048 tokens (LFM2-350M shape, bf16)",
+                          "value": round(prefill["tokens_per_second"], 1), "unit": "tokens/s",
+                          "ms": round(prefill["ms"], 4), "phase": "prefill",
+                          "frac": round(flops / (prefill["ms"] * 1e-3) / PEAK_FLOPS["bf16"], 5)}))
+        return 0
 
     def decode(batch: int):
         bench = DecodeBench(lm, batch, PROMPT_TOKENS, seed=batch, prefill_chunk=PROMPT_TOKENS)
@@ -115,7 +127,7 @@ def main() -> int:
 
     main_run = decode(BATCH)
     points = {}
-    if not args.no_points:
+    if not args.no_points and args.phase == "all":
         points = {"decode_b1": round(decode(1)["tokens_per_second"], 1),
                   "decode_b64": round(decode(64)["tokens_per_second"], 1)}
     mean_context = PROMPT_TOKENS + args.warmup + (args.steps + 1) / 2.0
@@ -135,9 +147,10 @@ def main() -> int:
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "ff": ff, "vocab_size": cfg["vocab_size"], "conv_L_cache": cfg["conv_L_cache"],
                    "rope_theta": cfg["rope_theta"], "tied_embeddings": True, "page_tokens": 16},
-        "prefill": {"value": round(prefill["tokens_per_second"], 1), "tokens": PROMPT_TOKENS,
-                    "ms": round(prefill["ms"], 4),
-                    "frac": round(flops / (prefill["ms"] * 1e-3) / PEAK_FLOPS["bf16"], 5)},
+        "prefill": None if prefill is None else {
+            "value": round(prefill["tokens_per_second"], 1), "tokens": PROMPT_TOKENS,
+            "ms": round(prefill["ms"], 4),
+            "frac": round(flops / (prefill["ms"] * 1e-3) / PEAK_FLOPS["bf16"], 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5)},
         "points": points,

@@ -1,7 +1,7 @@
 """Compiling the HIP sources for gfx950 and finding the built libraries.
 
 Every ``<name>.hip`` in this folder becomes one shared library
-``lib/<name>-<hash>.so`` beside it, the hash covering the source, the shared header
+``lib/<name>-<hash>.so`` beside it, the hash covering the source, the shared headers
 and the compiler flags, so a library is never used with a source it was not built
 from.  If the package folder cannot be written, the libraries go to a per-user
 folder under the system's temporary directory.  ``ensure_built(name)`` compiles on
@@ -23,7 +23,8 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]
-MODULES = ["elementwise", "gemm_f32", "short_conv", "attention", "attention_fast", "gemv_fused", "sampling"]
+MODULES = ["elementwise", "gemm_f32", "short_conv", "attention", "attention_fast", "gemv_fused", "gemv_slices",
+           "sampling"]
 
 
 class BuildError(RuntimeError):
@@ -44,7 +45,8 @@ def source_path(name: str) -> str:
 
 def _digest(name: str) -> str:
     h = hashlib.sha256()
-    for path in (source_path(name), os.path.join(HERE, "common.h")):
+    headers = sorted(f for f in os.listdir(HERE) if f.endswith(".h"))
+    for path in [source_path(name)] + [os.path.join(HERE, f) for f in headers]:
         with open(path, "rb") as fh:
             h.update(fh.read())
     h.update(" ".join(FLAGS).encode())

@@ -24,6 +24,7 @@
 // projections y = x W^T src/model/weight_plan.cpp:82-130; the reference fuses the residual
 // addition into its products with beta = 1 (src/backend/cuda/model/prefill_batched/non_attention.cpp:175-201).
 #include "common.h"
+#include "gemv_params.h"
 
 typedef short bf16x4_t __attribute__((ext_vector_type(4)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
@@ -35,33 +36,6 @@ struct __attribute__((aligned(16))) Frag2 {   // 16 bytes = 8 bfloat16 = two MFM
 enum { A_BF16 = 0, A_NORM = 1 };
 enum { E_STORE = 0, E_STORE_F32 = 1, E_RESIDUAL = 2, E_SWIGLU = 3, E_CONV = 4 };
 
-struct GemvParams {
-    // A side
-    const void* a;          // bf16 [M, lda] or float [*, lda]
-    int lda;
-    const int* rows;        // optional: A row of output row m is rows[m]
-    const float* norm_w;    // A_NORM: [K]
-    float eps;
-    const float* stats;     // A_NORM: [n_stat_blocks, stats_ld] partial sums of squares, or null
-    int n_stat_blocks, stats_ld;
-    // weights: stream s starts at row s * stream_rows
-    const bf16* w;
-    int stream_rows;
-    const float* bias;      // optional [streams * stream_rows]
-    int M, N, K;
-    // outputs
-    void* out;              // bf16 or float [M, ldo]; E_RESIDUAL: the residual stream itself
-    int ldo;
-    float* stats_out;       // E_RESIDUAL: [gridDim.x, stats_ld_out] or null
-    int stats_ld_out;
-    // E_CONV
-    const float* conv_w;    // [N, taps]
-    const float* conv_b;    // optional [N]
-    float* state;           // [slots, taps, N]
-    size_t state_slot_stride;
-    const int* seq_slot;    // [M]
-    int taps;
-};
 
 __device__ __forceinline__ short to_bits(float x) { return static_cast<short>(from_float<bf16>(x).bits); }
 __device__ __forceinline__ float round_bf16(float x) { return to_float(from_float<bf16>(x)); }
@@ -249,34 +223,49 @@ __global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvPara
                     wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
             }
     };
-    load_weights(c_begin);
-
     // ---- rows of A: 1/rms (A_NORM), and the rows themselves into LDS (ALDS); one wavefront
-    // per row.  The loads of a row are issued before the sum of squares is reduced.
+    // per row.  Loads come back in the order they were asked for, so the (cached) rows of A
+    // are asked for first and the weights right after: preparing the rows then overlaps
+    // with the weights' way from memory instead of waiting behind it.
     if (AMODE == A_NORM || ALDS) {
-        for (int m = wave; m < M; m += NW) {
-            const size_t src = static_cast<size_t>(p.rows ? p.rows[m] : m);
+        constexpr int RV = AMODE == A_NORM ? 4 : 8;   // 16-byte loads of a row kept in flight
+        floatx4_t hv4[AMODE == A_NORM ? 4 : 1], nw4[AMODE == A_NORM ? 4 : 1];
+        Frag2 rv[AMODE == A_NORM ? 1 : RV];
+        float s = 0.f;
+        bool weights_asked = false;
+        for (int m = wave; m < M || !weights_asked; m += NW) {
+            const bool row_ok = m < M;
+            const size_t src = row_ok ? static_cast<size_t>(p.rows ? p.rows[m] : m) : 0;
             if (AMODE == A_NORM) {
                 const float* row = static_cast<const float*>(p.a) + src * p.lda;
-                float s = 0.f;
-                if (p.stats) {
+                s = 0.f;
+                if (p.stats && row_ok) {
                     for (int j = lane; j < p.n_stat_blocks; j += 64)
                         s += p.stats[static_cast<size_t>(j) * p.stats_ld + src];
                 }
                 float inv = 0.f;
                 for (int k0 = 0; k0 < K; k0 += 1024) {
-                    floatx4_t hv4[4], nw4[4];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int k = k0 + i * 256 + lane * 4;
-                        hv4[i] = k < K ? *reinterpret_cast<const floatx4_t*>(row + k) : floatx4_t{};
-                        if (ALDS) nw4[i] = k < K ? *reinterpret_cast<const floatx4_t*>(p.norm_w + k) : floatx4_t{};
+                        const bool in = row_ok && k < K;
+                        hv4[i] = in ? *reinterpret_cast<const floatx4_t*>(row + k) : floatx4_t{};
+                        if (ALDS) nw4[i] = in ? *reinterpret_cast<const floatx4_t*>(p.norm_w + k) : floatx4_t{};
                     }
+                    if (!weights_asked) { load_weights(c_begin); weights_asked = true; }
+                    if (!row_ok) break;
                     if (k0 == 0) {
                         if (!p.stats) {   // no partial sums were left: walk the row
-                            for (int k = lane * 4; k < K; k += 256) {
-                                const floatx4_t v = *reinterpret_cast<const floatx4_t*>(row + k);
-                                s += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+                            if (K <= 1024) {
+#pragma unroll
+                                for (int i = 0; i < 4; ++i)
+                                    s += hv4[i][0] * hv4[i][0] + hv4[i][1] * hv4[i][1] +
+                                         hv4[i][2] * hv4[i][2] + hv4[i][3] * hv4[i][3];
+                            } else {
+                                for (int k = lane * 4; k < K; k += 256) {
+                                    const floatx4_t v = *reinterpret_cast<const floatx4_t*>(row + k);
+                                    s += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+                                }
                             }
                         }
                         s = wave_sum(s);
@@ -294,12 +283,25 @@ __global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvPara
                 }
             } else {
                 const bf16* row = static_cast<const bf16*>(p.a) + src * p.lda;
-                for (int k = lane * 8; k < K; k += 512)
-                    *reinterpret_cast<Frag2*>(xs + static_cast<size_t>(m) * ldx + k) =
-                        *reinterpret_cast<const Frag2*>(row + k);
+                for (int k0 = 0; k0 < K; k0 += 512 * RV) {
+#pragma unroll
+                    for (int i = 0; i < RV; ++i) {
+                        const int k = k0 + i * 512 + lane * 8;
+                        rv[i] = (row_ok && k < K) ? *reinterpret_cast<const Frag2*>(row + k) : Frag2{};
+                    }
+                    if (!weights_asked) { load_weights(c_begin); weights_asked = true; }
+                    if (!row_ok) break;
+#pragma unroll
+                    for (int i = 0; i < RV; ++i) {
+                        const int k = k0 + i * 512 + lane * 8;
+                        if (k < K) *reinterpret_cast<Frag2*>(xs + static_cast<size_t>(m) * ldx + k) = rv[i];
+                    }
+                }
             }
         }
         __syncthreads();
+    } else {
+        load_weights(c_begin);
     }
 
     // the row of A this lane feeds in every row tile (rows beyond M repeat the last one;
@@ -470,6 +472,10 @@ extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, in
         if (shape == 2) return CELEG_SHAPE(1, 2, 4);
         if (shape == 3) return CELEG_SHAPE(1, 1, 8);
         if (shape == 4) return CELEG_SHAPE(1, 1, 4);
+        if (shape == 5) return launch_shape<1, 8, 1, 0>(p, amode, epi, stream);
+        if (shape == 6) return launch_shape<1, 2, 4, 0>(p, amode, epi, stream);
+        if (shape == 7) return launch_shape<1, 1, 8, 0>(p, amode, epi, stream);
+        if (shape == 8) return launch_shape<1, 1, 4, 0>(p, amode, epi, stream);
         if (tiles >= 2048) return CELEG_SHAPE(1, 8, 1);
         // two tiles a workgroup (they share the prepared rows) once there are enough tiles
         // and K is short enough that four wavefronts a tile keep their loads in one batch

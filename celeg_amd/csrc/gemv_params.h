@@ -1,0 +1,32 @@
+// Arguments of the fused skinny products (one struct for every prologue and epilogue, so
+// that the caller fills one block of memory whatever the combination).
+#pragma once
+#include "common.h"
+
+struct GemvParams {
+    // A side
+    const void* a;          // bf16 [M, lda] or float [*, lda]
+    int lda;
+    const int* rows;        // optional: A row of output row m is rows[m]
+    const float* norm_w;    // A_NORM: [K]
+    float eps;
+    const float* stats;     // A_NORM: [n_stat_blocks, stats_ld] partial sums of squares, or null
+    int n_stat_blocks, stats_ld;
+    // weights: stream s starts at row s * stream_rows
+    const bf16* w;
+    int stream_rows;
+    const float* bias;      // optional [streams * stream_rows]
+    int M, N, K;
+    // outputs
+    void* out;              // bf16 or float [M, ldo]; E_RESIDUAL: the residual stream itself
+    int ldo;
+    float* stats_out;       // E_RESIDUAL: [gridDim.x, stats_ld_out] or null
+    int stats_ld_out;
+    // E_CONV
+    const float* conv_w;    // [N, taps]
+    const float* conv_b;    // optional [N]
+    float* state;           // [slots, taps, N]
+    size_t state_slot_stride;
+    const int* seq_slot;    // [M]
+    int taps;
+};

@@ -46,6 +46,8 @@ class HipOps:
         self.attention_impl = "auto"
         self._decode_ws = None
         self._retired = []
+        self.use_sliced_residual = True    # up to 16 rows: the k-sliced kernel for "residual"
+        self.last_stat_blocks = 0
         self.fused_linear_shape = 0        # 0: chosen from the sizes; 1..4 force a workgroup shape
 
     # ------------------------------------------------------------------ plumbing
@@ -371,6 +373,14 @@ class HipOps:
         """Whether the fused skinny product takes ``rows`` rows and these inner sizes."""
         return 0 < rows <= 64 and all(k > 0 and k % 8 == 0 for k in inner_sizes)
 
+    def residual_stat_blocks(self, rows: int, n: int, k: int) -> int:
+        """How many partial sums of squares per row the "residual" epilogue of
+        ``fused_linear`` leaves for these sizes (the rows ``stats_out`` needs)."""
+        if rows <= 16 and self.use_sliced_residual:
+            return int(self._lib("gemv_slices").celeg_gemv_slices_blocks(
+                _c_int(rows), _c_int(n), _c_int(k)))
+        return (n + 15) // 16
+
     def embed_stats(self, table, token_ids, out, stats):
         """Embedding gather that also leaves every row's sum of squares in ``stats[0, :rows]``."""
         self._dev(table, "table", torch.bfloat16); self._dev(token_ids, "token_ids", torch.int32)
@@ -391,8 +401,8 @@ class HipOps:
         normalised on the fly (``stats[:stat_blocks]`` holding partial sums of squares of its
         rows if ``stat_blocks`` > 0).  ``rows`` picks rows of ``a``.  Epilogues: "store"
         (bfloat16 [M, N]), "store_f32", "residual" (``out`` is the stream, [M, N] 32-bit,
-        added to in place; ``stats_out`` [ceil(N/16), >= M] receives partial sums of squares
-        of the new rows), "swiglu" (``w`` is [2N, K]: gate rows then up rows), "conv"
+        added to in place; ``stats_out`` [``residual_stat_blocks``, >= M] receives partial
+        sums of squares of the new rows, ``last_stat_blocks`` says how many), "swiglu" (``w`` is [2N, K]: gate rows then up rows), "conv"
         (``w`` is [3N, K]: B, C, x rows; ``conv`` = (taps [N, L], bias or None, state
         [slots, L, N], seq_slot [M]); one new token per request)."""
         if epilogue not in self._EPILOGUES:
@@ -450,10 +460,14 @@ class HipOps:
         prm.bias = bias.data_ptr() if bias is not None else None
         prm.M, prm.N, prm.K = M, N, K
         prm.out, prm.ldo = out.data_ptr(), self._rows(out, "out")
+        sliced = epilogue == "residual" and M <= 16 and rows is None and self.use_sliced_residual
+        if epilogue == "residual":
+            # partial sums of squares: one per workgroup and row
+            self.last_stat_blocks = self.residual_stat_blocks(M, N, K) if sliced else (N + 15) // 16
         if epilogue == "residual" and stats_out is not None:
             self._dev(stats_out, "stats_out", torch.float32)
-            if stats_out.shape[0] < (N + 15) // 16 or stats_out.shape[1] < M:
-                raise KernelError("fused_linear: stats_out must be [ceil(N/16), >= rows]")
+            if stats_out.shape[0] < self.last_stat_blocks or stats_out.shape[1] < M:
+                raise KernelError(f"fused_linear: stats_out must be [{self.last_stat_blocks}, >= rows]")
             prm.stats_out, prm.stats_ld_out = stats_out.data_ptr(), stats_out.stride(0)
         if epilogue == "conv":
             taps_w, conv_bias, state, seq_slot = conv
@@ -469,6 +483,10 @@ class HipOps:
             prm.conv_b = conv_bias.data_ptr() if conv_bias is not None else None
             prm.state, prm.state_slot_stride = state.data_ptr(), state.stride(0)
             prm.seq_slot, prm.taps = seq_slot.data_ptr(), L
+        if sliced:
+            code = self._lib("gemv_slices").celeg_gemv_slices_residual(ctypes.byref(prm), self._stream())
+            self._check(code, "fused_linear (residual, sliced)")
+            return out
         code = self._lib("gemv_fused").celeg_gemv_fused(
             ctypes.byref(prm), _c_int(1 if norm_weight is not None else 0),
             _c_int(self._EPILOGUES[epilogue]), _c_int(self.fused_linear_shape), self._stream())

@@ -32,7 +32,8 @@ def fused_rows_ok(rt, batch, *inner_sizes) -> bool:
 
 
 def stream_stats(rt, width: int) -> torch.Tensor:
-    return rt.ws.buf("stream_stats", ((width + 15) // 16, STAT_COLUMNS), torch.float32)
+    # up to one partial sum per 4 columns (the products for few rows use narrow workgroups)
+    return rt.ws.buf("stream_stats", ((width + 3) // 4, STAT_COLUMNS), torch.float32)
 
 
 def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None, **kw):
@@ -47,5 +48,5 @@ def linear_into_stream(rt, a, w, h, bias=None):
     """h += a w^T, leaving the partial sums of squares of the new rows."""
     stats = stream_stats(rt, h.shape[1])
     rt.ops.fused_linear(a, w, h, epilogue="residual", bias=bias, stats_out=stats)
-    rt.stream_stat_blocks = (h.shape[1] + 15) // 16
+    rt.stream_stat_blocks = rt.ops.last_stat_blocks
     return h

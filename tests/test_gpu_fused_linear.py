@@ -74,15 +74,19 @@ def test_norm_prologue_with_and_without_partial_sums(ops, M, N, K, with_stats):
     close(out, ref)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (8, 1024, 1024), (20, 200, 352), (64, 96, 4608)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (8, 1024, 1024), (20, 200, 352), (64, 96, 4608),
+                                   (3, 130, 72), (4, 1024, 4608), (7, 77, 352), (8, 1024, 4608),
+                                   (13, 50, 1160), (16, 1024, 1024), (2, 36, 8), (5, 24, 40)])
 def test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, M, N, K):
     a = randn(M, K, seed=7, dtype=BF)
     w = randn(N, K, seed=8, scale=0.1, dtype=BF)
     b = randn(N, seed=9)
     h = randn(M, N, seed=10)
     h0 = h.clone()
-    stats = torch.full(((N + 15) // 16, 64), -1.0, device=DEV)
+    blocks = ops.residual_stat_blocks(M, N, K)
+    stats = torch.full((blocks, 64), -1.0, device=DEV)
     ops.fused_linear(a, w, h, epilogue="residual", bias=b, stats_out=stats)
+    assert ops.last_stat_blocks == blocks
     delta = (a.double() @ w.double().T + b.double())
     close(h, h0.double() + delta)
     # the product enters the sum rounded to bfloat16
