@@ -29,4 +29,7 @@ struct GemvParams {
     size_t state_slot_stride;
     const int* seq_slot;    // [M]
     int taps;
+    // E_RESIDUAL of the k-sliced kernels: the bfloat16 copy of the stream, or null
+    void* out_bf16;
+    int ld_bf16;
 };

@@ -1,22 +1,31 @@
-// Skinny bfloat16 products that end a sub-block, for up to 16 rows on gfx950:
-//   h[M,N] += A[M,K] W[N,K]^T (+ bias),  h the 32-bit residual stream,
-// leaving partial sums of squares of the new rows for the norm that follows.
+// Skinny bfloat16 products for up to 16 rows on gfx950 (decode steps), with what
+// surrounds them fused in:
+//   out[M,N] = epilogue(scale[m] * (A[M,K] W[N,K]^T) + bias)
+// A is bfloat16.  For a product behind an RMSNorm, A is the bfloat16 copy of the residual
+// stream, W has the norm's weight folded into its columns by the caller, and scale[m] =
+// rsqrt(mean(x_m^2) + eps) is taken from the partial sums of squares that the producer of
+// the stream left; the scaling is applied to the 32-bit sums at the end.
+// Epilogues: store | 32-bit store | add into the 32-bit residual stream, refresh its
+// bfloat16 copy and leave partial sums of squares | SwiGLU of a gate and an up stream |
+// the double-gated short convolution of a B, a C and an x stream for one new token per
+// request, with its state update.
 //
-// Such a product has few output columns (the model's width) and a long K, so a layout
-// with 16 columns a workgroup leaves most of the chip idle.  Here the 16x16 tile of the
-// MFMA is cut in G x G blocks of MP x MP (MP = 16 / G >= M): the instruction's row index
-// is (k-slice g, row m) and its column index (k-slice g', column j); A rows of slice g
-// hold A[m, g*K/G + k] and B columns of slice g' hold W[n0 + j, g'*K/G + k], so the
-// diagonal blocks g == g' are G partial products over G parts of K for the same MP x MP
-// outputs, and the others are dropped.  A workgroup then owns only MP columns (G times as
-// many workgroups), every lane's loads are useful for M == MP, and the rows of A are read
-// straight from cache into the instruction's operand layout (no staging).  KW wavefronts
-// split each slice's K; their tiles meet in LDS and MP x MP threads finish one output each,
-// always adding in the same order.
+// Layout.  These products have few rows and are bound by memory latency and by how much
+// of the chip takes part, so the 16x16 tile of the MFMA is cut in G x G blocks of MP x MP
+// (MP = 16 / G >= M): the instruction's row index is (k-slice g, row m) and its column
+// index (k-slice g', column j); A rows of slice g hold A[m, g*K/G + k] and B columns of
+// slice g' hold W[n0 + j, g'*K/G + k], so the diagonal blocks g == g' are G partial
+// products over G parts of K for the same MP x MP outputs, and the others are dropped.  A
+// workgroup then owns only MP columns (of every weight stream) - G times as many
+// workgroups -, every lane's loads are useful when M == MP, and the rows of A are read
+// from cache straight into the instruction's operand layout (no staging, no barrier
+// before the products).  KW wavefronts split each slice's K; their tiles meet in LDS and
+// MP x MP threads finish one output each, always adding in the same order.
 //
-// Reference semantics: projections y = x W^T src/model/weight_plan.cpp:82-130; the residual
-// addition fused into the product as with beta = 1 in
-// src/backend/cuda/model/prefill_batched/non_attention.cpp:175-201.
+// Reference semantics of the fused parts: RMSNorm src/backend/cpu/kernels/elementwise.cpp:56-76,
+// SwiGLU elementwise.cpp:101-119, short convolution src/backend/cpu/kernels/convolution.cpp:7-28,
+// projections y = x W^T src/model/weight_plan.cpp:82-130; the reference fuses the residual
+// addition into its products with beta = 1 (src/backend/cuda/model/prefill_batched/non_attention.cpp:175-201).
 #include "common.h"
 #include "gemv_params.h"
 
@@ -26,79 +35,173 @@ struct __attribute__((aligned(16))) Frag2 {   // 16 bytes = 8 bfloat16 = two MFM
     bf16x4_t lo, hi;
 };
 
+enum { E_STORE = 0, E_STORE_F32 = 1, E_RESIDUAL = 2, E_SWIGLU = 3, E_CONV = 4 };
+#define SLICES_MAX_TAPS 8
+
+__device__ __forceinline__ float round_bf16(float x) { return to_float(from_float<bf16>(x)); }
+
+template <int EPI> struct Streams { static constexpr int n = 1; };
+template <> struct Streams<E_SWIGLU> { static constexpr int n = 2; };
+template <> struct Streams<E_CONV> { static constexpr int n = 3; };
+
 // U: chunks of 64 along K that a wavefront keeps in flight at a time.
-template <int G, int KW, int U>
-__global__ __launch_bounds__(KW * 64) void gemv_slices_residual_kernel(const GemvParams p) {
+template <int G, int KW, int U, int EPI>
+__global__ __launch_bounds__(KW * 64) void gemv_slices_kernel(const GemvParams p) {
     constexpr int MP = 16 / G;
-    __shared__ floatx4_t red[KW][64];
+    constexpr int NS = Streams<EPI>::n;
+    __shared__ floatx4_t red[NS][KW][64];
+    __shared__ float scale_s[16];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int c16 = lane & 15, q = lane >> 4;
     const int idx = c16 & (MP - 1), slice = c16 / MP;
     const int M = p.M, N = p.N, K = p.K;
     const int Ks = K / G;                       // K % (8 G) == 0 (checked by the host)
     const int n0 = blockIdx.x * MP;
-    const int t = threadIdx.x;                  // threads 0 .. MP*MP-1 finish one output each
-    const int em = t / MP, ej = t % MP;
+    // threads 0 .. MP*MP-1 finish one output each: row em, column n0 + ej
+    const int t = threadIdx.x;
+    const int em = (t / MP) & (MP - 1), ej = t % MP;
     const bool e_ok = t < MP * MP && em < M && n0 + ej < N;
-    float* hp = static_cast<float*>(p.out) + static_cast<size_t>(min(em, M - 1)) * p.ldo + min(n0 + ej, N - 1);
-    // what the end needs is asked for first
-    const float old = e_ok ? *hp : 0.f;
-    const float bias = (e_ok && p.bias) ? p.bias[n0 + ej] : 0.f;
+    const int en = min(n0 + ej, N - 1), emc = min(em, M - 1);
 
-    const bf16* wrow = p.w + static_cast<size_t>(min(n0 + idx, N - 1)) * K + slice * Ks;
-    const bf16* arow = static_cast<const bf16*>(p.a) + static_cast<size_t>(min(idx, M - 1)) * p.lda + slice * Ks;
+    // ---- what the end needs is asked for first (loads come back in the order they were
+    // asked for, and these are short)
+    float old = 0.f, taps[EPI == E_CONV ? SLICES_MAX_TAPS : 1], state[EPI == E_CONV ? SLICES_MAX_TAPS - 1 : 1];
+    float* state_ptr = nullptr;
+    if (EPI == E_RESIDUAL && e_ok)
+        old = static_cast<const float*>(p.out)[static_cast<size_t>(emc) * p.ldo + en];
+    if (EPI == E_CONV && t < MP * MP) {
+        state_ptr = p.state + static_cast<size_t>(p.seq_slot[emc]) * p.state_slot_stride + en;
+#pragma unroll
+        for (int i = 0; i < SLICES_MAX_TAPS; ++i) taps[i] = i < p.taps ? p.conv_w[static_cast<size_t>(en) * p.taps + i] : 0.f;
+#pragma unroll
+        for (int i = 0; i < SLICES_MAX_TAPS - 1; ++i) state[i] = i + 1 < p.taps ? state_ptr[static_cast<size_t>(i + 1) * N] : 0.f;
+    }
+
+    // ---- the products
+    const size_t a_row = static_cast<size_t>(p.rows ? p.rows[min(idx, M - 1)] : min(idx, M - 1));
+    const bf16* arow = static_cast<const bf16*>(p.a) + a_row * p.lda + slice * Ks;
+    const bf16* wrow[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+        wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + idx, N - 1)) * K + slice * Ks;
     const int chunks = (Ks + 63) >> 6;
     const int c_begin = wave * chunks / KW, c_end = (wave + 1) * chunks / KW;
-    floatx4_t acc = {0.f, 0.f, 0.f, 0.f};
-    for (int c0 = c_begin; c0 < c_end; c0 += U) {
-        Frag2 wv[U][2], av[U][2];
+    floatx4_t acc[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) acc[s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    float ssq = 0.f;                 // this lane's share of a row's partial sums of squares
+    bool scale_pending = p.stats != nullptr;
+    for (int c0 = c_begin; c0 < c_end || scale_pending; c0 += U) {
+        Frag2 wv[U][NS][2], av[U][2];
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
             for (int v = 0; v < 2; ++v) {
                 const int k = (c0 + u) * 64 + v * 32 + q * 8;
                 const bool in = c0 + u < c_end && k + 8 <= Ks;
-                wv[u][v] = in ? *reinterpret_cast<const Frag2*>(wrow + k) : Frag2{};
                 av[u][v] = in ? *reinterpret_cast<const Frag2*>(arow + k) : Frag2{};
+#pragma unroll
+                for (int s = 0; s < NS; ++s)
+                    wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
             }
+        if (scale_pending) {
+            // 1/rms of the rows: wavefront w adds up the partial sums of rows w, w + KW, ...;
+            // asked for behind the first weights, so that it does not hold them up
+            scale_pending = false;
+            for (int m = wave; m < M; m += KW) {
+                const size_t src = static_cast<size_t>(p.rows ? p.rows[m] : m);
+                float s = 0.f;
+                for (int j = lane; j < p.n_stat_blocks; j += 64)
+                    s += p.stats[static_cast<size_t>(j) * p.stats_ld + src];
+                s = wave_sum(s);
+                if (lane == 0) scale_s[m] = 1.0f / sqrtf(s / static_cast<float>(K) + p.eps);
+            }
+        }
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int v = 0; v < 2; ++v) {
-                acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].lo, wv[u][v].lo, acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].hi, wv[u][v].hi, acc, 0, 0, 0);
-            }
+            for (int v = 0; v < 2; ++v)
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].lo, wv[u][s][v].lo, acc[s], 0, 0, 0);
+                    acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].hi, wv[u][s][v].hi, acc[s], 0, 0, 0);
+                }
     }
     // acc: lane l holds column l%16 of rows 4*(l/16)..+3 of the 16x16 tile
-    red[wave][lane] = acc;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) red[s][wave][lane] = acc[s];
     __syncthreads();
     if (wave * 64 >= MP * MP) return;           // whole wavefronts leave; the rest finish
-    float sum = 0.f;
+    float sum[NS];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const int r = g * MP + (em & (MP - 1)), c = g * MP + ej;
-        const int src = c + 16 * (r >> 2), reg = r & 3;
+    for (int s = 0; s < NS; ++s) {
+        sum[s] = 0.f;
 #pragma unroll
-        for (int w = 0; w < KW; ++w) sum += red[w][src][reg];
+        for (int g = 0; g < G; ++g) {
+            const int r = g * MP + em, c = g * MP + ej;
+            const int src = c + 16 * (r >> 2), reg = r & 3;
+#pragma unroll
+            for (int w = 0; w < KW; ++w) sum[s] += red[s][w][src][reg];
+        }
+        if (p.stats) sum[s] *= scale_s[emc];
+        if (p.bias) sum[s] += p.bias[static_cast<size_t>(s) * p.stream_rows + en];
     }
-    // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
-    const float v = e_ok ? old + to_float(from_float<bf16>(sum + bias)) : 0.f;
-    if (e_ok) *hp = v;
-    if (p.stats_out) {
-        float sq = v * v;                       // the MP columns of a row sit in MP neighbouring lanes
+    const size_t o = static_cast<size_t>(emc) * p.ldo + en;
+    if (EPI == E_STORE) {
+        if (e_ok) static_cast<bf16*>(p.out)[o] = from_float<bf16>(sum[0]);
+    } else if (EPI == E_STORE_F32) {
+        if (e_ok) static_cast<float*>(p.out)[o] = sum[0];
+    } else if (EPI == E_RESIDUAL) {
+        // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
+        const float v = e_ok ? old + round_bf16(sum[0]) : 0.f;
+        if (e_ok) {
+            static_cast<float*>(p.out)[o] = v;
+            if (p.out_bf16) static_cast<bf16*>(p.out_bf16)[static_cast<size_t>(em) * p.ld_bf16 + en] = from_float<bf16>(v);
+        }
+        if (p.stats_out) {
+            float sq = v * v;                   // the MP columns of a row sit in MP neighbouring lanes
 #pragma unroll
-        for (int off = MP / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
-        if (ej == 0 && em < M && t < MP * MP)
-            p.stats_out[static_cast<size_t>(blockIdx.x) * p.stats_ld_out + em] = sq;
+            for (int off = MP / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+            if (ej == 0 && em < M && t < MP * MP)
+                p.stats_out[static_cast<size_t>(blockIdx.x) * p.stats_ld_out + em] = sq;
+        }
+    } else if (EPI == E_SWIGLU) {
+        if (e_ok) {
+            const float g = round_bf16(sum[0]), u = round_bf16(sum[1]);
+            static_cast<bf16*>(p.out)[o] = from_float<bf16>((g / (1.0f + expf(-g))) * u);
+        }
+    } else if (EPI == E_CONV) {
+        if (e_ok) {
+            const float bb = round_bf16(sum[0]), cc = round_bf16(sum[1]), xx = round_bf16(sum[2]);
+            const float bx = bb * xx;
+            float conv = 0.f, last_tap = 0.f;
+#pragma unroll
+            for (int tap = 0; tap < SLICES_MAX_TAPS - 1; ++tap)
+                if (tap + 1 < p.taps) {
+                    conv = fmaf(taps[tap], state[tap], conv);
+                    state_ptr[static_cast<size_t>(tap) * N] = state[tap];     // shift by one position
+                }
+#pragma unroll
+            for (int tap = 0; tap < SLICES_MAX_TAPS; ++tap)
+                if (tap == p.taps - 1) last_tap = taps[tap];
+            conv = fmaf(last_tap, bx, conv);
+            state_ptr[static_cast<size_t>(p.taps - 1) * N] = bx;
+            if (p.conv_b) conv += p.conv_b[en];
+            static_cast<bf16*>(p.out)[o] = from_float<bf16>(cc * conv);
+        }
     }
 }
 
-template <int G, int KW>
+template <int G, int KW, int EPI>
 static int launch_slices(const GemvParams& p, int chunks_per_wave, hipStream_t stream) {
     dim3 grid((p.N + 16 / G - 1) / (16 / G)), block(KW * 64);
-    if (chunks_per_wave <= 2) hipLaunchKernelGGL((gemv_slices_residual_kernel<G, KW, 2>), grid, block, 0, stream, p);
-    else if (chunks_per_wave <= 4) hipLaunchKernelGGL((gemv_slices_residual_kernel<G, KW, 4>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((gemv_slices_residual_kernel<G, KW, 6>), grid, block, 0, stream, p);
+    constexpr int NS = Streams<EPI>::n;
+    if (chunks_per_wave <= 2)
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, EPI>), grid, block, 0, stream, p);
+    else if (chunks_per_wave <= 4 || NS > 1)
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, EPI>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), EPI>), grid, block, 0, stream, p);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -109,24 +212,99 @@ static int slices_for(int M, int K) {
     return g;
 }
 
-// Number of partial sums of squares a row gets (= workgroups): the caller sizes stats_out
-// [blocks, >= M] with it.
+template <int EPI>
+static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
+    const int g = slices_for(p.M, p.K);
+    const int chunks = (p.K / g + 63) / 64;
+    const int kw = chunks >= 24 ? 8 : 4;
+    const int cpw = (chunks + kw - 1) / kw;
+    if (g == 4) return kw == 8 ? launch_slices<4, 8, EPI>(p, cpw, stream) : launch_slices<4, 4, EPI>(p, cpw, stream);
+    if (g == 2) return kw == 8 ? launch_slices<2, 8, EPI>(p, cpw, stream) : launch_slices<2, 4, EPI>(p, cpw, stream);
+    return kw == 8 ? launch_slices<1, 8, EPI>(p, cpw, stream) : launch_slices<1, 4, EPI>(p, cpw, stream);
+}
+
+extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvParams)); }
+
+// Number of workgroups for these sizes, which is also the number of partial sums of
+// squares a row gets from the "residual" epilogue: the caller sizes stats_out [blocks, >= M].
 extern "C" int celeg_gemv_slices_blocks(int M, int N, int K) {
     const int mp = 16 / slices_for(M, K);
     return (N + mp - 1) / mp;
 }
 
-// h[M,N] += a[M,K] w[N,K]^T + bias with partial sums of squares; M <= 16, K % 8 == 0.
-// Uses of GemvParams: a, lda, w, bias, M, N, K, out, ldo, stats_out, stats_ld_out.
-extern "C" int celeg_gemv_slices_residual(const GemvParams* params, hipStream_t stream) {
+// M <= 16, K % 8 == 0, bfloat16 a and w.  Fields of GemvParams that are read: a, lda, rows,
+// stats/n_stat_blocks/stats_ld/eps (scale by 1/rms if stats is set), w, stream_rows, bias,
+// M, N, K, out, ldo, and per epilogue out_bf16/ld_bf16/stats_out/stats_ld_out (residual) or
+// conv_w/conv_b/state/state_slot_stride/seq_slot/taps (conv).
+extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t stream) {
     const GemvParams& p = *params;
     if (p.M <= 0 || p.N <= 0) return 0;
-    if (p.M > 16 || p.K <= 0 || (p.K % 8) || (p.lda % 8) || p.rows) return static_cast<int>(hipErrorInvalidValue);
-    const int g = slices_for(p.M, p.K);
-    const int chunks = (p.K / g + 63) / 64;
-    const int kw = chunks >= 24 ? 8 : 4;
-    const int cpw = (chunks + kw - 1) / kw;
-    if (g == 4) return kw == 8 ? launch_slices<4, 8>(p, cpw, stream) : launch_slices<4, 4>(p, cpw, stream);
-    if (g == 2) return kw == 8 ? launch_slices<2, 8>(p, cpw, stream) : launch_slices<2, 4>(p, cpw, stream);
-    return kw == 8 ? launch_slices<1, 8>(p, cpw, stream) : launch_slices<1, 4>(p, cpw, stream);
+    if (p.M > 16 || p.K <= 0 || (p.K % 8) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
+    if (epi == E_CONV && (p.taps < 1 || p.taps > SLICES_MAX_TAPS || p.stream_rows != p.N))
+        return static_cast<int>(hipErrorInvalidValue);
+    switch (epi) {
+        case E_STORE: return launch_epilogue<E_STORE>(p, stream);
+        case E_STORE_F32: return launch_epilogue<E_STORE_F32>(p, stream);
+        case E_RESIDUAL: return launch_epilogue<E_RESIDUAL>(p, stream);
+        case E_SWIGLU: return launch_epilogue<E_SWIGLU>(p, stream);
+        case E_CONV: return launch_epilogue<E_CONV>(p, stream);
+        default: return static_cast<int>(hipErrorInvalidValue);
+    }
+}
+
+// Prepares a 32-bit stream for products behind a norm: its bfloat16 copy and every row's
+// sum of squares (one partial sum a row: stats[row]).  Used where the stream was written by
+// something that leaves neither.
+__global__ void stream_prepare_kernel(const float* __restrict__ h, int ldh, bf16* __restrict__ xb,
+                                      int ldx, float* __restrict__ stats, int width) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const float* src = h + static_cast<size_t>(row) * ldh;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = src[i];
+        xb[static_cast<size_t>(row) * ldx + i] = from_float<bf16>(v);
+        s += v * v;
+    }
+    s = block_sum(s, scratch);
+    if (threadIdx.x == 0) stats[row] = s;
+}
+
+extern "C" int celeg_stream_prepare(const float* h, int ldh, void* xb, int ldx, float* stats,
+                                    int rows, int width, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    hipLaunchKernelGGL(stream_prepare_kernel, dim3(rows), dim3(256), 0, stream, h, ldh,
+                       static_cast<bf16*>(xb), ldx, stats, width);
+    return CELEG_LAUNCH_RESULT();
+}
+
+// Embedding gather into the 32-bit stream, its bfloat16 copy and the rows' sums of squares:
+// out[row, :] = table[ids[row], :], stats[row] = sum(out[row, :]^2).
+__global__ void embed_stream_kernel(const bf16* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ out, bf16* __restrict__ xb,
+                                    float* __restrict__ stats, int width, int vocab) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const int id = ids[row];
+    const bool ok = id >= 0 && id < vocab;
+    const bf16* src = table + static_cast<size_t>(ok ? id : 0) * width;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const bf16 raw = ok ? src[i] : bf16{0};
+        const float v = to_float(raw);
+        out[static_cast<size_t>(row) * width + i] = v;
+        xb[static_cast<size_t>(row) * width + i] = raw;
+        s += v * v;
+    }
+    s = block_sum(s, scratch);
+    if (threadIdx.x == 0) stats[row] = s;
+}
+
+extern "C" int celeg_embed_stream(const void* table, const int* ids, float* out, void* xb,
+                                  float* stats, int rows, int width, int vocab, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    hipLaunchKernelGGL(embed_stream_kernel, dim3(rows), dim3(256), 0, stream,
+                       static_cast<const bf16*>(table), ids, out, static_cast<bf16*>(xb), stats,
+                       width, vocab);
+    return CELEG_LAUNCH_RESULT();
 }

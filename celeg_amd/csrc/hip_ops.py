@@ -46,7 +46,7 @@ class HipOps:
         self.attention_impl = "auto"
         self._decode_ws = None
         self._retired = []
-        self.use_sliced_residual = True    # up to 16 rows: the k-sliced kernel for "residual"
+        self.use_sliced = True             # up to 16 bfloat16 rows: the k-sliced kernels
         self.last_stat_blocks = 0
         self.fused_linear_shape = 0        # 0: chosen from the sizes; 1..4 force a workgroup shape
 
@@ -59,6 +59,8 @@ class HipOps:
                 lib = ctypes.CDLL(path)
             except OSError as err:
                 raise KernelError(f"cannot load the built kernels {path}: {err}") from err
+            if module == "gemv_slices" and lib.celeg_gemv_params_size() != ctypes.sizeof(_GemvParams):
+                raise KernelError("the argument block of the skinny products does not match the built kernels")
             self._libs[module] = lib
             self.loaded_libraries[module] = path
         return lib
@@ -376,10 +378,38 @@ class HipOps:
     def residual_stat_blocks(self, rows: int, n: int, k: int) -> int:
         """How many partial sums of squares per row the "residual" epilogue of
         ``fused_linear`` leaves for these sizes (the rows ``stats_out`` needs)."""
-        if rows <= 16 and self.use_sliced_residual:
+        if rows <= 16 and self.use_sliced:
             return int(self._lib("gemv_slices").celeg_gemv_slices_blocks(
                 _c_int(rows), _c_int(n), _c_int(k)))
         return (n + 15) // 16
+
+    def stream_prepare(self, h, xb, stats):
+        """The bfloat16 copy ``xb`` of the 32-bit stream ``h`` and its rows' sums of squares
+        (``stats[0, :rows]``)."""
+        self._dev(h, "h", torch.float32, contiguous=False); self._dev(xb, "xb", torch.bfloat16, contiguous=False)
+        self._dev(stats, "stats", torch.float32)
+        rows, width = h.shape
+        if xb.shape[0] < rows or xb.shape[1] != width or stats.shape[1] < rows:
+            raise KernelError("stream_prepare: shapes do not fit")
+        code = self._lib("gemv_slices").celeg_stream_prepare(
+            _ptr(h), _c_int(self._rows(h, "h")), _ptr(xb), _c_int(self._rows(xb, "xb")), _ptr(stats),
+            _c_int(rows), _c_int(width), self._stream())
+        self._check(code, "stream_prepare")
+
+    def embed_stream(self, table, token_ids, out, xb, stats):
+        """Embedding gather into the 32-bit stream ``out``, its bfloat16 copy ``xb`` and the
+        rows' sums of squares (``stats[0, :rows]``)."""
+        self._dev(table, "table", torch.bfloat16); self._dev(token_ids, "token_ids", torch.int32)
+        self._dev(out, "out", torch.float32); self._dev(xb, "xb", torch.bfloat16)
+        self._dev(stats, "stats", torch.float32)
+        rows, width = out.shape
+        if table.shape[1] != width or token_ids.numel() != rows or stats.shape[1] < rows \
+                or xb.shape != out.shape:
+            raise KernelError("embed_stream: shapes do not fit")
+        code = self._lib("gemv_slices").celeg_embed_stream(
+            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(xb), _ptr(stats), _c_int(rows),
+            _c_int(width), _c_int(table.shape[0]), self._stream())
+        self._check(code, "embed_stream")
 
     def embed_stats(self, table, token_ids, out, stats):
         """Embedding gather that also leaves every row's sum of squares in ``stats[0, :rows]``."""
@@ -394,7 +424,8 @@ class HipOps:
         self._check(code, "embed_stats")
 
     def fused_linear(self, a, w, out, *, epilogue="store", norm_weight=None, eps=0.0, stats=None,
-                     stat_blocks=0, rows=None, bias=None, stats_out=None, conv=None, n_rows=None):
+                     stat_blocks=0, rows=None, bias=None, stats_out=None, conv=None, n_rows=None,
+                     out_bf16=None):
         """out = epilogue(prologue(a) w^T) for up to 64 rows, bfloat16 weights.
 
         ``a``: bfloat16 rows [M, K], or, with ``norm_weight``, the 32-bit residual stream,
@@ -404,7 +435,13 @@ class HipOps:
         added to in place; ``stats_out`` [``residual_stat_blocks``, >= M] receives partial
         sums of squares of the new rows, ``last_stat_blocks`` says how many), "swiglu" (``w`` is [2N, K]: gate rows then up rows), "conv"
         (``w`` is [3N, K]: B, C, x rows; ``conv`` = (taps [N, L], bias or None, state
-        [slots, L, N], seq_slot [M]); one new token per request)."""
+        [slots, L, N], seq_slot [M]); one new token per request).
+
+        Up to 16 bfloat16 rows go to the k-sliced kernels, which also take the form behind a
+        norm whose weight the caller has folded into ``w``: ``a`` is then the bfloat16 copy
+        of the stream and ``stats[:stat_blocks]`` its partial sums of squares, from which
+        the rows' 1/rms (with ``eps``) scales the sums; their "residual" epilogue refreshes
+        ``out_bf16``, the bfloat16 copy of the stream, if given."""
         if epilogue not in self._EPILOGUES:
             raise KernelError(f"fused_linear: unknown epilogue '{epilogue}'")
         self._dev(w, "w", torch.bfloat16)
@@ -432,7 +469,7 @@ class HipOps:
         else:
             if a.dtype != torch.bfloat16:
                 raise KernelError("fused_linear: rows must be bfloat16 (or 32-bit with a norm weight)")
-            if epilogue in ("swiglu", "conv"):
+            if (epilogue in ("swiglu", "conv") or stat_blocks > 0) and not (M <= 16 and self.use_sliced):
                 raise KernelError("fused_linear: this combination is not built")
         if lda % 8:
             raise KernelError("fused_linear: the row stride of a must be a multiple of 8")
@@ -451,7 +488,7 @@ class HipOps:
         prm.rows = rows.data_ptr() if rows is not None else None
         prm.norm_w = norm_weight.data_ptr() if norm_weight is not None else None
         prm.eps = eps
-        if norm_weight is not None and stat_blocks > 0:
+        if stat_blocks > 0:
             self._dev(stats, "stats", torch.float32)
             if stats.shape[0] < stat_blocks:
                 raise KernelError("fused_linear: fewer partial sums than stat_blocks")
@@ -460,7 +497,14 @@ class HipOps:
         prm.bias = bias.data_ptr() if bias is not None else None
         prm.M, prm.N, prm.K = M, N, K
         prm.out, prm.ldo = out.data_ptr(), self._rows(out, "out")
-        sliced = epilogue == "residual" and M <= 16 and rows is None and self.use_sliced_residual
+        sliced = norm_weight is None and M <= 16 and self.use_sliced
+        if out_bf16 is not None:
+            if not (sliced and epilogue == "residual"):
+                raise KernelError("fused_linear: out_bf16 goes with the residual epilogue for up to 16 rows")
+            self._dev(out_bf16, "out_bf16", torch.bfloat16, contiguous=False)
+            if out_bf16.shape[0] < M or out_bf16.shape[1] != N:
+                raise KernelError("fused_linear: out_bf16 does not fit")
+            prm.out_bf16, prm.ld_bf16 = out_bf16.data_ptr(), self._rows(out_bf16, "out_bf16")
         if epilogue == "residual":
             # partial sums of squares: one per workgroup and row
             self.last_stat_blocks = self.residual_stat_blocks(M, N, K) if sliced else (N + 15) // 16
@@ -484,8 +528,9 @@ class HipOps:
             prm.state, prm.state_slot_stride = state.data_ptr(), state.stride(0)
             prm.seq_slot, prm.taps = seq_slot.data_ptr(), L
         if sliced:
-            code = self._lib("gemv_slices").celeg_gemv_slices_residual(ctypes.byref(prm), self._stream())
-            self._check(code, "fused_linear (residual, sliced)")
+            code = self._lib("gemv_slices").celeg_gemv_slices(
+                ctypes.byref(prm), _c_int(self._EPILOGUES[epilogue]), self._stream())
+            self._check(code, f"fused_linear ({epilogue}, k-sliced)")
             return out
         code = self._lib("gemv_fused").celeg_gemv_fused(
             ctypes.byref(prm), _c_int(1 if norm_weight is not None else 0),
@@ -495,7 +540,7 @@ class HipOps:
 
 
 class _GemvParams(ctypes.Structure):
-    """Mirror of ``GemvParams`` in gemv_fused.hip."""
+    """Mirror of ``GemvParams`` in gemv_params.h (its size is checked when the library loads)."""
     _fields_ = [
         ("a", ctypes.c_void_p), ("lda", ctypes.c_int), ("rows", ctypes.c_void_p),
         ("norm_w", ctypes.c_void_p), ("eps", ctypes.c_float), ("stats", ctypes.c_void_p),
@@ -506,4 +551,5 @@ class _GemvParams(ctypes.Structure):
         ("stats_ld_out", ctypes.c_int),
         ("conv_w", ctypes.c_void_p), ("conv_b", ctypes.c_void_p), ("state", ctypes.c_void_p),
         ("state_slot_stride", ctypes.c_size_t), ("seq_slot", ctypes.c_void_p), ("taps", ctypes.c_int),
+        ("out_bf16", ctypes.c_void_p), ("ld_bf16", ctypes.c_int),
     ]

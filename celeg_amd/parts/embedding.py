@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from .base import Embedding, Head, WeightSpec, register_part
-from .fused import fused_rows_ok, norm_linear, stream_stats
+from .fused import _sliced, fused_rows_ok, norm_linear, stream_bf16, stream_stats
 from .norm import RmsNorm
 
 
@@ -32,8 +32,16 @@ class TokenEmbedding(Embedding):
     def forward(self, token_ids, out, rt, batch=None):
         if batch is not None and self.table.dtype == torch.bfloat16 \
                 and fused_rows_ok(rt, batch, self.width):
-            # few rows: leave every row's sum of squares for the first norm
-            rt.ops.embed_stats(self.table, token_ids, out, stream_stats(rt, self.width))
+            # few rows: leave every row's sum of squares (and the bfloat16 copy of the
+            # stream) for the first norm
+            if _sliced(rt, out.shape[0]):
+                rt.ops.embed_stream(self.table, token_ids, out,
+                                    stream_bf16(rt, out.shape[0], self.width),
+                                    stream_stats(rt, self.width))
+                rt.stream_has_bf16 = True
+            else:
+                rt.ops.embed_stats(self.table, token_ids, out, stream_stats(rt, self.width))
+                rt.stream_has_bf16 = False
             rt.stream_stat_blocks = 1
         else:
             rt.ops.embed(self.table, token_ids, out)

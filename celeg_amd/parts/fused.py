@@ -31,22 +31,65 @@ def fused_rows_ok(rt, batch, *inner_sizes) -> bool:
             and ops.fused_linear_ok(batch.n_tokens, *inner_sizes))
 
 
+SLICED_MAX_ROWS = 16      # rows of the k-sliced kernels
+SLICED_MAX_COLUMNS = 16384   # wider products (the output head) keep their rows in LDS instead
+
+
 def stream_stats(rt, width: int) -> torch.Tensor:
     # up to one partial sum per 4 columns (the products for few rows use narrow workgroups)
     return rt.ws.buf("stream_stats", ((width + 3) // 4, STAT_COLUMNS), torch.float32)
 
 
+def stream_bf16(rt, rows: int, width: int) -> torch.Tensor:
+    """The bfloat16 copy of the residual stream that products behind a norm read."""
+    return rt.ws.buf("stream_bf16", (STAT_COLUMNS, width), torch.bfloat16)[:rows]
+
+
+def _sliced(rt, rows: int) -> bool:
+    return rows <= SLICED_MAX_ROWS and getattr(rt.ops, "use_sliced", False)
+
+
+def folded_weight(rt, w: torch.Tensor, norm_weight: torch.Tensor) -> torch.Tensor:
+    """``w`` with the norm's weight multiplied into its columns: (x * nw) w^T = x (w * nw)^T.
+    Made once per (weight, norm) pair and kept."""
+    cache = rt.__dict__.setdefault("folded_weights", {})
+    key = (w.data_ptr(), norm_weight.data_ptr())
+    hit = cache.get(key)
+    if hit is None:
+        hit = (w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype).contiguous()
+        cache[key] = hit
+    return hit
+
+
 def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None, **kw):
     """out = epilogue(norm(h) w^T), the norm applied while the rows of ``h`` are read."""
     blocks = getattr(rt, "stream_stat_blocks", 0)
+    M = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
+    streams = {"swiglu": 2, "conv": 3}.get(epilogue, 1)
+    if _sliced(rt, M) and w.shape[0] // streams <= SLICED_MAX_COLUMNS:
+        # the stream's bfloat16 copy times the weight with the norm's weight folded in,
+        # scaled by the rows' 1/rms at the end
+        stats = stream_stats(rt, h.shape[1])
+        xb = stream_bf16(rt, h.shape[0], h.shape[1])
+        if not (blocks and getattr(rt, "stream_has_bf16", False)):
+            rt.ops.stream_prepare(h, xb, stats)
+            rt.stream_stat_blocks = blocks = 1
+            rt.stream_has_bf16 = True
+        return rt.ops.fused_linear(xb, folded_weight(rt, w, norm.weight), out, epilogue=epilogue,
+                                   eps=norm.eps, stats=stats, stat_blocks=blocks, rows=rows,
+                                   n_rows=n_rows, **kw)
     return rt.ops.fused_linear(h, w, out, epilogue=epilogue, norm_weight=norm.weight,
                                eps=norm.eps, stats=stream_stats(rt, h.shape[1]) if blocks else None,
                                stat_blocks=blocks, rows=rows, n_rows=n_rows, **kw)
 
 
 def linear_into_stream(rt, a, w, h, bias=None):
-    """h += a w^T, leaving the partial sums of squares of the new rows."""
+    """h += a w^T, leaving the partial sums of squares of the new rows (and, for few rows,
+    the stream's bfloat16 copy)."""
     stats = stream_stats(rt, h.shape[1])
-    rt.ops.fused_linear(a, w, h, epilogue="residual", bias=bias, stats_out=stats)
+    sliced = _sliced(rt, h.shape[0])
+    rt.ops.fused_linear(a, w, h, epilogue="residual", bias=bias, stats_out=stats,
+                        out_bf16=stream_bf16(rt, h.shape[0], h.shape[1]) if sliced else None)
     rt.stream_stat_blocks = rt.ops.last_stat_blocks
+    rt.stream_has_bf16 = sliced
     return h

@@ -47,7 +47,7 @@ def test_plain_rows_store_and_32bit_store_with_bias(ops, M, N, K):
     # which the wavefronts' partial sums are added (their number depends on the rows)
     one = torch.empty(1, N, device=DEV)
     ops.fused_linear(a[M // 2:M // 2 + 1], w, one, epilogue="store_f32", bias=b)
-    if M <= 16:
+    if ops.residual_stat_blocks(M, N, K) == ops.residual_stat_blocks(1, N, K):   # the same layout
         assert torch.equal(one[0], out32[M // 2])
     close(one[0], out32[M // 2], rel=1e-5)
 
@@ -135,6 +135,115 @@ def test_conv_epilogue_token_by_token_equals_the_whole_convolution(ops, M, H, ta
         ref = plain.short_conv(bcx.to(BF), cw.cpu(), cb.cpu() if bias else None)
         close(got[:, m], ref, rel=2e-2)
     assert float(state[0].abs().max()) == 0.0          # a slot nobody uses stays zero
+
+
+SLICED = [(1, 64, 64), (3, 130, 200), (4, 1024, 1024), (5, 77, 352), (8, 3072, 1024), (8, 96, 4608),
+          (13, 50, 1160), (16, 272, 1024)]
+
+
+def scaled_case(M, N, K, streams, seed):
+    """A stream h, its bfloat16 copy, uneven partial sums of squares, a norm weight, weights
+    and the same weights with the norm weight folded in; rows picked in another order."""
+    h = randn(M + 3, K, seed=seed)
+    nw = 1 + randn(K, seed=seed + 1, scale=0.1)
+    w = randn(streams * N, K, seed=seed + 2, scale=0.2, dtype=BF)
+    folded = (w.float() * nw.reshape(1, -1)).to(BF)
+    rows = torch.tensor([(3 * i + 1) % (M + 3) for i in range(M)], dtype=torch.int32, device=DEV)
+    cuts = [0, K // 7, K // 3, K // 2, K - 8, K]
+    stats = torch.zeros(5, 80, device=DEV)
+    for j in range(5):
+        stats[j, :M + 3] = (h[:, cuts[j]:cuts[j + 1]] ** 2).sum(dim=1)
+    x = plain.rmsnorm(h.cpu(), nw.cpu(), 1e-5)[rows.long().cpu()].to(BF).double()
+    return h, h.to(BF), stats, nw, w, folded, rows, x
+
+
+@pytest.mark.parametrize("M,N,K", SLICED)
+def test_sliced_products_behind_a_norm(ops, M, N, K):
+    """The form for up to 16 rows: bfloat16 copy of the stream, norm weight folded into the
+    weights, 1/rms from the partial sums applied at the end; against the plain norm and
+    product."""
+    h, xb, stats, nw, w, folded, rows, x = scaled_case(M, N, K, 1, 40)
+    b = randn(N, seed=44)
+    ref = x @ w.double().cpu().T + b.double().cpu()
+    out = torch.empty(M, N, dtype=BF, device=DEV)
+    ops.fused_linear(xb, folded, out, eps=1e-5, stats=stats, stat_blocks=5, rows=rows, bias=b)
+    close(out, ref)
+    out32 = torch.empty(M, N, device=DEV)
+    ops.fused_linear(xb, folded, out32, epilogue="store_f32", eps=1e-5, stats=stats, stat_blocks=5,
+                     rows=rows, bias=b)
+    close(out32, ref, rel=8e-3)
+    # the older form (32-bit rows normalised on the fly) agrees
+    old = torch.empty(M, N, device=DEV)
+    ops.fused_linear(h, w, old, epilogue="store_f32", norm_weight=nw, eps=1e-5, rows=rows, bias=b,
+                     stats=stats, stat_blocks=5)
+    close(out32, old, rel=8e-3)
+
+
+@pytest.mark.parametrize("M,ff,K", [(1, 192, 64), (8, 4608, 1024), (7, 352, 128), (16, 200, 96), (4, 100, 1160)])
+def test_sliced_swiglu(ops, M, ff, K):
+    h, xb, stats, nw, w, folded, rows, x = scaled_case(M, ff, K, 2, 50)
+    g = (x @ w[:ff].double().cpu().T).to(BF).double()
+    u = (x @ w[ff:].double().cpu().T).to(BF).double()
+    out = torch.empty(M, ff, dtype=BF, device=DEV)
+    ops.fused_linear(xb, folded, out, epilogue="swiglu", eps=1e-5, stats=stats, stat_blocks=5, rows=rows)
+    close(out, plain.silu(g) * u, rel=2.5e-2)
+
+
+@pytest.mark.parametrize("M,H,taps,bias", [(1, 64, 3, False), (8, 1024, 3, False), (5, 128, 4, True),
+                                           (16, 96, 1, True), (3, 48, 5, False), (12, 200, 8, True)])
+def test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, M, H, taps, bias):
+    """M requests advance one token per call, each in its own slot (in another order than
+    the rows); their outputs over 6 calls equal the plain whole-sequence convolution."""
+    steps = 6
+    nw = 1 + randn(H, seed=14, scale=0.1)
+    w_in = randn(3 * H, H, seed=15, scale=0.2, dtype=BF)
+    folded = (w_in.float() * nw.reshape(1, -1)).to(BF)
+    b_in = randn(3 * H, seed=16, scale=0.1) if bias else None
+    cw = randn(H, taps, seed=17)
+    cb = randn(H, seed=18) if bias else None
+    hs = randn(steps, M, H, seed=19)
+    state = torch.zeros(M + 2, taps, H, device=DEV)
+    slots = torch.tensor([(M + 1 - i) for i in range(M)], dtype=torch.int32, device=DEV)
+    stats = torch.zeros(1, 64, device=DEV)
+    outs = []
+    for t in range(steps):
+        y = torch.empty(M, H, dtype=BF, device=DEV)
+        xb = torch.empty(M, H, dtype=BF, device=DEV)
+        ops.stream_prepare(hs[t], xb, stats)
+        assert torch.equal(xb, hs[t].to(BF))
+        torch.testing.assert_close(stats[0, :M], (hs[t] ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
+        ops.fused_linear(xb, folded, y, epilogue="conv", eps=1e-5, stats=stats, stat_blocks=1,
+                         bias=b_in, conv=(cw, cb, state, slots))
+        outs.append(y.double().cpu())
+    got = torch.stack(outs)              # [steps, M, H]
+    for m in range(0, M, max(1, M // 4)):
+        x = plain.rmsnorm(hs[:, m].cpu(), nw.cpu(), 1e-5).to(BF).double()
+        bcx = x @ w_in.double().cpu().T + (b_in.double().cpu() if bias else 0)
+        ref = plain.short_conv(bcx.to(BF), cw.cpu(), cb.cpu() if bias else None)
+        close(got[:, m], ref, rel=2.5e-2)
+    assert float(state[0].abs().max()) == 0.0          # a slot nobody uses stays zero
+
+
+def test_residual_refreshes_the_bfloat16_copy(ops):
+    M, N, K = 6, 200, 352
+    a = randn(M, K, seed=60, dtype=BF)
+    w = randn(N, K, seed=61, scale=0.1, dtype=BF)
+    h = randn(M, N, seed=62)
+    xb = torch.zeros(M + 2, N, dtype=BF, device=DEV)
+    stats = torch.zeros(ops.residual_stat_blocks(M, N, K), 64, device=DEV)
+    ops.fused_linear(a, w, h, epilogue="residual", stats_out=stats, out_bf16=xb)
+    assert torch.equal(xb[:M], h.to(BF)) and float(xb[M:].abs().max()) == 0.0
+
+
+def test_embed_stream(ops):
+    table = randn(331, 96, seed=20, dtype=BF)
+    ids = torch.tensor([5, 330, 0, 17], dtype=torch.int32, device=DEV)
+    out = torch.empty(4, 96, device=DEV)
+    xb = torch.empty(4, 96, dtype=BF, device=DEV)
+    stats = torch.zeros(6, 64, device=DEV)
+    ops.embed_stream(table, ids, out, xb, stats)
+    assert torch.equal(out, table[ids.long()].float()) and torch.equal(xb, table[ids.long()])
+    torch.testing.assert_close(stats[0, :4], (out ** 2).sum(dim=1), rtol=1e-6, atol=1e-6)
 
 
 def test_embed_stats(ops):
