@@ -160,7 +160,7 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&a
                 s += __shfl_xor(s, 8, 64);
                 const int m = mt * 16 + 4 * q + r;
                 if (c16 == 0 && m < M)
-                    p.stats_out[static_cast<size_t>(tile) * p.stats_ld_out + m] = s;
+                    p.stats_out[static_cast<size_t>(m) * p.stats_ld_out + tile] = s;
             }
         }
     }
@@ -241,7 +241,7 @@ __global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvPara
                 s = 0.f;
                 if (p.stats && row_ok) {
                     for (int j = lane; j < p.n_stat_blocks; j += 64)
-                        s += p.stats[static_cast<size_t>(j) * p.stats_ld + src];
+                        s += p.stats[src * p.stats_ld + j];
                 }
                 float inv = 0.f;
                 for (int k0 = 0; k0 < K; k0 += 1024) {
@@ -494,10 +494,10 @@ extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, in
 }
 
 // Embedding gather that also leaves the sum of squares of every row, for the first norm:
-// out[row, :] = table[ids[row], :] (32-bit), stats[row] = sum(out[row, :]^2).
+// out[row, :] = table[ids[row], :] (32-bit), stats[row * stats_ld] = sum(out[row, :]^2).
 __global__ void embed_stats_kernel(const bf16* __restrict__ table, const int* __restrict__ ids,
-                                   float* __restrict__ out, float* __restrict__ stats, int width,
-                                   int vocab) {
+                                   float* __restrict__ out, float* __restrict__ stats, int stats_ld,
+                                   int width, int vocab) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const int id = ids[row];
@@ -514,13 +514,13 @@ __global__ void embed_stats_kernel(const bf16* __restrict__ table, const int* __
         for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = 0.f;
     }
     s = block_sum(s, scratch);
-    if (threadIdx.x == 0) stats[row] = s;
+    if (threadIdx.x == 0) stats[static_cast<size_t>(row) * stats_ld] = s;
 }
 
-extern "C" int celeg_embed_stats(const void* table, const int* ids, float* out, float* stats,
+extern "C" int celeg_embed_stats(const void* table, const int* ids, float* out, float* stats, int stats_ld,
                                  int rows, int width, int vocab, hipStream_t stream) {
     if (rows <= 0) return 0;
     hipLaunchKernelGGL(embed_stats_kernel, dim3(rows), dim3(256), 0, stream,
-                       static_cast<const bf16*>(table), ids, out, stats, width, vocab);
+                       static_cast<const bf16*>(table), ids, out, stats, stats_ld, width, vocab);
     return CELEG_LAUNCH_RESULT();
 }

@@ -10,7 +10,7 @@ struct GemvParams {
     const int* rows;        // optional: A row of output row m is rows[m]
     const float* norm_w;    // A_NORM: [K]
     float eps;
-    const float* stats;     // A_NORM: [n_stat_blocks, stats_ld] partial sums of squares, or null
+    const float* stats;     // partial sums of squares of the rows of the stream: [rows, stats_ld], n_stat_blocks valid per row; or null
     int n_stat_blocks, stats_ld;
     // weights: stream s starts at row s * stream_rows
     const bf16* w;
@@ -20,7 +20,7 @@ struct GemvParams {
     // outputs
     void* out;              // bf16 or float [M, ldo]; E_RESIDUAL: the residual stream itself
     int ldo;
-    float* stats_out;       // E_RESIDUAL: [gridDim.x, stats_ld_out] or null
+    float* stats_out;       // E_RESIDUAL: [rows, stats_ld_out], one partial sum per workgroup and row; or null
     int stats_ld_out;
     // E_CONV
     const float* conv_w;    // [N, taps]

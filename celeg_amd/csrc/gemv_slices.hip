@@ -37,6 +37,7 @@ struct __attribute__((aligned(16))) Frag2 {   // 16 bytes = 8 bfloat16 = two MFM
 
 enum { E_STORE = 0, E_STORE_F32 = 1, E_RESIDUAL = 2, E_SWIGLU = 3, E_CONV = 4 };
 #define SLICES_MAX_TAPS 8
+#define SLICES_MAX_STAT_BLOCKS 512   // partial sums of squares a row may come with
 
 __device__ __forceinline__ float round_bf16(float x) { return to_float(from_float<bf16>(x)); }
 
@@ -45,93 +46,123 @@ template <> struct Streams<E_SWIGLU> { static constexpr int n = 2; };
 template <> struct Streams<E_CONV> { static constexpr int n = 3; };
 
 // U: chunks of 64 along K that a wavefront keeps in flight at a time.
+// Wavefronts 0 .. KW-1 multiply: nothing stands in front of their weight loads.  The
+// wavefronts behind them (FW of them: MP*MP threads, one output each) first fetch what
+// the end needs - the old value of the stream, or the convolution's state through the
+// request's slot, and the partial sums of squares for the rows' 1/rms - while the
+// products are under way, wait at the barrier, and finish.
 template <int G, int KW, int U, int EPI>
-__global__ __launch_bounds__(KW * 64) void gemv_slices_kernel(const GemvParams p) {
+__global__ __launch_bounds__((KW + (16 / G) * (16 / G) / 64 + ((16 / G) * (16 / G) % 64 ? 1 : 0)) * 64)
+void gemv_slices_kernel(const GemvParams p) {
     constexpr int MP = 16 / G;
     constexpr int NS = Streams<EPI>::n;
+    constexpr int ROWS_FW = MP * MP >= 64 ? 64 / MP : MP;   // rows a finishing wavefront holds
     __shared__ floatx4_t red[NS][KW][64];
-    __shared__ float scale_s[16];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int c16 = lane & 15, q = lane >> 4;
-    const int idx = c16 & (MP - 1), slice = c16 / MP;
     const int M = p.M, N = p.N, K = p.K;
-    const int Ks = K / G;                       // K % (8 G) == 0 (checked by the host)
     const int n0 = blockIdx.x * MP;
-    // threads 0 .. MP*MP-1 finish one output each: row em, column n0 + ej
-    const int t = threadIdx.x;
+
+    if (wave < KW) {
+        // ---- the products
+        const int c16 = lane & 15, q = lane >> 4;
+        const int idx = c16 & (MP - 1), slice = c16 / MP;
+        const int Ks = K / G;                   // K % (8 G) == 0 (checked by the host)
+        const size_t a_row = static_cast<size_t>(p.rows ? p.rows[min(idx, M - 1)] : min(idx, M - 1));
+        const bf16* arow = static_cast<const bf16*>(p.a) + a_row * p.lda + slice * Ks;
+        const bf16* wrow[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + idx, N - 1)) * K + slice * Ks;
+        const int chunks = (Ks + 63) >> 6;
+        const int c_begin = wave * chunks / KW, c_end = (wave + 1) * chunks / KW;
+        floatx4_t acc[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) acc[s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        for (int c0 = c_begin; c0 < c_end; c0 += U) {
+            Frag2 wv[U][NS][2], av[U][2];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int v = 0; v < 2; ++v) {
+                    const int k = (c0 + u) * 64 + v * 32 + q * 8;
+                    const bool in = c0 + u < c_end && k + 8 <= Ks;
+                    av[u][v] = in ? *reinterpret_cast<const Frag2*>(arow + k) : Frag2{};
+#pragma unroll
+                    for (int s = 0; s < NS; ++s)
+                        wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
+                }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int v = 0; v < 2; ++v)
+#pragma unroll
+                    for (int s = 0; s < NS; ++s) {
+                        acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].lo, wv[u][s][v].lo, acc[s], 0, 0, 0);
+                        acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].hi, wv[u][s][v].hi, acc[s], 0, 0, 0);
+                    }
+        }
+        // acc: lane l holds column l%16 of rows 4*(l/16)..+3 of the 16x16 tile
+#pragma unroll
+        for (int s = 0; s < NS; ++s) red[s][wave][lane] = acc[s];
+        __syncthreads();
+        return;
+    }
+
+    // ---- the finishing wavefronts: thread t finishes row em, column n0 + ej
+    const int fw = wave - KW;
+    const int t = fw * 64 + lane;
     const int em = (t / MP) & (MP - 1), ej = t % MP;
     const bool e_ok = t < MP * MP && em < M && n0 + ej < N;
     const int en = min(n0 + ej, N - 1), emc = min(em, M - 1);
-
-    // ---- what the end needs is asked for first (loads come back in the order they were
-    // asked for, and these are short)
     float old = 0.f, taps[EPI == E_CONV ? SLICES_MAX_TAPS : 1], state[EPI == E_CONV ? SLICES_MAX_TAPS - 1 : 1];
+    float bias[NS];
     float* state_ptr = nullptr;
-    if (EPI == E_RESIDUAL && e_ok)
-        old = static_cast<const float*>(p.out)[static_cast<size_t>(emc) * p.ldo + en];
-    if (EPI == E_CONV && t < MP * MP) {
-        state_ptr = p.state + static_cast<size_t>(p.seq_slot[emc]) * p.state_slot_stride + en;
+    int slot = 0;
+    if (EPI == E_CONV) slot = p.seq_slot[emc];
+    // partial sums of squares of the ROWS_FW rows this wavefront holds: LPR lanes share a
+    // row, every lane takes each LPR-th partial sum; all are asked for at once.  (Loads are
+    // made without conditions, from clamped places, and masked afterwards: a load under a
+    // condition of its own is waited for before the next one is asked for.)
+    constexpr int LPR = 64 / ROWS_FW;
+    constexpr int NFIRST = 16, NREST = SLICES_MAX_STAT_BLOCKS / LPR > NFIRST ? SLICES_MAX_STAT_BLOCKS / LPR - NFIRST : 0;
+    float ssq = 0.f;
+    if (p.stats) {
+        const int nb = p.n_stat_blocks;
+        const int sm = min(fw * ROWS_FW + lane / LPR, M - 1), sj = lane % LPR;
+        const float* srow = p.stats + static_cast<size_t>(p.rows ? p.rows[sm] : sm) * p.stats_ld;
+        float part[NFIRST];
 #pragma unroll
-        for (int i = 0; i < SLICES_MAX_TAPS; ++i) taps[i] = i < p.taps ? p.conv_w[static_cast<size_t>(en) * p.taps + i] : 0.f;
+        for (int i = 0; i < NFIRST; ++i) part[i] = srow[min(sj + LPR * i, nb - 1)];
+        if (nb > NFIRST * LPR) {                // the same for every lane
+            float rest[NREST > 0 ? NREST : 1];
 #pragma unroll
-        for (int i = 0; i < SLICES_MAX_TAPS - 1; ++i) state[i] = i + 1 < p.taps ? state_ptr[static_cast<size_t>(i + 1) * N] : 0.f;
-    }
-
-    // ---- the products
-    const size_t a_row = static_cast<size_t>(p.rows ? p.rows[min(idx, M - 1)] : min(idx, M - 1));
-    const bf16* arow = static_cast<const bf16*>(p.a) + a_row * p.lda + slice * Ks;
-    const bf16* wrow[NS];
+            for (int i = 0; i < NREST; ++i) rest[i] = srow[min(sj + LPR * (NFIRST + i), nb - 1)];
 #pragma unroll
-    for (int s = 0; s < NS; ++s)
-        wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + idx, N - 1)) * K + slice * Ks;
-    const int chunks = (Ks + 63) >> 6;
-    const int c_begin = wave * chunks / KW, c_end = (wave + 1) * chunks / KW;
-    floatx4_t acc[NS];
-#pragma unroll
-    for (int s = 0; s < NS; ++s) acc[s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-    float ssq = 0.f;                 // this lane's share of a row's partial sums of squares
-    bool scale_pending = p.stats != nullptr;
-    for (int c0 = c_begin; c0 < c_end || scale_pending; c0 += U) {
-        Frag2 wv[U][NS][2], av[U][2];
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int v = 0; v < 2; ++v) {
-                const int k = (c0 + u) * 64 + v * 32 + q * 8;
-                const bool in = c0 + u < c_end && k + 8 <= Ks;
-                av[u][v] = in ? *reinterpret_cast<const Frag2*>(arow + k) : Frag2{};
-#pragma unroll
-                for (int s = 0; s < NS; ++s)
-                    wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
-            }
-        if (scale_pending) {
-            // 1/rms of the rows: wavefront w adds up the partial sums of rows w, w + KW, ...;
-            // asked for behind the first weights, so that it does not hold them up
-            scale_pending = false;
-            for (int m = wave; m < M; m += KW) {
-                const size_t src = static_cast<size_t>(p.rows ? p.rows[m] : m);
-                float s = 0.f;
-                for (int j = lane; j < p.n_stat_blocks; j += 64)
-                    s += p.stats[static_cast<size_t>(j) * p.stats_ld + src];
-                s = wave_sum(s);
-                if (lane == 0) scale_s[m] = 1.0f / sqrtf(s / static_cast<float>(K) + p.eps);
-            }
+            for (int i = 0; i < NREST; ++i) ssq += sj + LPR * (NFIRST + i) < nb ? rest[i] : 0.f;
         }
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int v = 0; v < 2; ++v)
-#pragma unroll
-                for (int s = 0; s < NS; ++s) {
-                    acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].lo, wv[u][s][v].lo, acc[s], 0, 0, 0);
-                    acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].hi, wv[u][s][v].hi, acc[s], 0, 0, 0);
-                }
+        for (int i = 0; i < NFIRST; ++i) ssq += sj + LPR * i < nb ? part[i] : 0.f;
     }
-    // acc: lane l holds column l%16 of rows 4*(l/16)..+3 of the 16x16 tile
+    if (EPI == E_RESIDUAL)
+        old = static_cast<const float*>(p.out)[static_cast<size_t>(emc) * p.ldo + en];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) red[s][wave][lane] = acc[s];
+    for (int s = 0; s < NS; ++s) bias[s] = p.bias ? p.bias[static_cast<size_t>(s) * p.stream_rows + en] : 0.f;
+    if (EPI == E_CONV) {
+#pragma unroll
+        for (int i = 0; i < SLICES_MAX_TAPS; ++i) taps[i] = p.conv_w[static_cast<size_t>(en) * p.taps + min(i, p.taps - 1)];
+        state_ptr = p.state + static_cast<size_t>(slot) * p.state_slot_stride + en;
+#pragma unroll
+        for (int i = 0; i < SLICES_MAX_TAPS - 1; ++i) state[i] = state_ptr[static_cast<size_t>(min(i + 1, p.taps - 1)) * N];
+    }
+    float scale = 1.f;
+    if (p.stats) {
+#pragma unroll
+        for (int off = LPR / 2; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+        // the lanes of row em - fw * ROWS_FW hold its sum
+        const float total = __shfl(ssq, ((em - fw * ROWS_FW) & (ROWS_FW - 1)) * LPR, 64);
+        scale = 1.0f / sqrtf(total / static_cast<float>(K) + p.eps);
+    }
     __syncthreads();
-    if (wave * 64 >= MP * MP) return;           // whole wavefronts leave; the rest finish
     float sum[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -143,8 +174,7 @@ __global__ __launch_bounds__(KW * 64) void gemv_slices_kernel(const GemvParams p
 #pragma unroll
             for (int w = 0; w < KW; ++w) sum[s] += red[s][w][src][reg];
         }
-        if (p.stats) sum[s] *= scale_s[emc];
-        if (p.bias) sum[s] += p.bias[static_cast<size_t>(s) * p.stream_rows + en];
+        sum[s] = sum[s] * scale + bias[s];
     }
     const size_t o = static_cast<size_t>(emc) * p.ldo + en;
     if (EPI == E_STORE) {
@@ -163,7 +193,7 @@ __global__ __launch_bounds__(KW * 64) void gemv_slices_kernel(const GemvParams p
 #pragma unroll
             for (int off = MP / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
             if (ej == 0 && em < M && t < MP * MP)
-                p.stats_out[static_cast<size_t>(blockIdx.x) * p.stats_ld_out + em] = sq;
+                p.stats_out[static_cast<size_t>(em) * p.stats_ld_out + blockIdx.x] = sq;
         }
     } else if (EPI == E_SWIGLU) {
         if (e_ok) {
@@ -194,7 +224,8 @@ __global__ __launch_bounds__(KW * 64) void gemv_slices_kernel(const GemvParams p
 
 template <int G, int KW, int EPI>
 static int launch_slices(const GemvParams& p, int chunks_per_wave, hipStream_t stream) {
-    dim3 grid((p.N + 16 / G - 1) / (16 / G)), block(KW * 64);
+    constexpr int MP = 16 / G;
+    dim3 grid((p.N + MP - 1) / MP), block((KW + (MP * MP + 63) / 64) * 64);
     constexpr int NS = Streams<EPI>::n;
     if (chunks_per_wave <= 2)
         hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, EPI>), grid, block, 0, stream, p);
@@ -226,7 +257,7 @@ static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
 extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvParams)); }
 
 // Number of workgroups for these sizes, which is also the number of partial sums of
-// squares a row gets from the "residual" epilogue: the caller sizes stats_out [blocks, >= M].
+// squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
 extern "C" int celeg_gemv_slices_blocks(int M, int N, int K) {
     const int mp = 16 / slices_for(M, K);
     return (N + mp - 1) / mp;
@@ -240,6 +271,8 @@ extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t 
     const GemvParams& p = *params;
     if (p.M <= 0 || p.N <= 0) return 0;
     if (p.M > 16 || p.K <= 0 || (p.K % 8) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
+    if (p.stats && (p.n_stat_blocks < 1 || p.n_stat_blocks > SLICES_MAX_STAT_BLOCKS))
+        return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.taps > SLICES_MAX_TAPS || p.stream_rows != p.N))
         return static_cast<int>(hipErrorInvalidValue);
     switch (epi) {
@@ -253,10 +286,10 @@ extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t 
 }
 
 // Prepares a 32-bit stream for products behind a norm: its bfloat16 copy and every row's
-// sum of squares (one partial sum a row: stats[row]).  Used where the stream was written by
+// sum of squares (one partial sum a row: stats[row * stats_ld]).  Used where the stream was written by
 // something that leaves neither.
 __global__ void stream_prepare_kernel(const float* __restrict__ h, int ldh, bf16* __restrict__ xb,
-                                      int ldx, float* __restrict__ stats, int width) {
+                                      int ldx, float* __restrict__ stats, int stats_ld, int width) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const float* src = h + static_cast<size_t>(row) * ldh;
@@ -267,22 +300,22 @@ __global__ void stream_prepare_kernel(const float* __restrict__ h, int ldh, bf16
         s += v * v;
     }
     s = block_sum(s, scratch);
-    if (threadIdx.x == 0) stats[row] = s;
+    if (threadIdx.x == 0) stats[static_cast<size_t>(row) * stats_ld] = s;
 }
 
 extern "C" int celeg_stream_prepare(const float* h, int ldh, void* xb, int ldx, float* stats,
-                                    int rows, int width, hipStream_t stream) {
+                                    int stats_ld, int rows, int width, hipStream_t stream) {
     if (rows <= 0) return 0;
     hipLaunchKernelGGL(stream_prepare_kernel, dim3(rows), dim3(256), 0, stream, h, ldh,
-                       static_cast<bf16*>(xb), ldx, stats, width);
+                       static_cast<bf16*>(xb), ldx, stats, stats_ld, width);
     return CELEG_LAUNCH_RESULT();
 }
 
 // Embedding gather into the 32-bit stream, its bfloat16 copy and the rows' sums of squares:
-// out[row, :] = table[ids[row], :], stats[row] = sum(out[row, :]^2).
+// out[row, :] = table[ids[row], :], stats[row * stats_ld] = sum(out[row, :]^2).
 __global__ void embed_stream_kernel(const bf16* __restrict__ table, const int* __restrict__ ids,
                                     float* __restrict__ out, bf16* __restrict__ xb,
-                                    float* __restrict__ stats, int width, int vocab) {
+                                    float* __restrict__ stats, int stats_ld, int width, int vocab) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const int id = ids[row];
@@ -297,14 +330,15 @@ __global__ void embed_stream_kernel(const bf16* __restrict__ table, const int* _
         s += v * v;
     }
     s = block_sum(s, scratch);
-    if (threadIdx.x == 0) stats[row] = s;
+    if (threadIdx.x == 0) stats[static_cast<size_t>(row) * stats_ld] = s;
 }
 
 extern "C" int celeg_embed_stream(const void* table, const int* ids, float* out, void* xb,
-                                  float* stats, int rows, int width, int vocab, hipStream_t stream) {
+                                  float* stats, int stats_ld, int rows, int width, int vocab,
+                                  hipStream_t stream) {
     if (rows <= 0) return 0;
     hipLaunchKernelGGL(embed_stream_kernel, dim3(rows), dim3(256), 0, stream,
                        static_cast<const bf16*>(table), ids, out, static_cast<bf16*>(xb), stats,
-                       width, vocab);
+                       stats_ld, width, vocab);
     return CELEG_LAUNCH_RESULT();
 }

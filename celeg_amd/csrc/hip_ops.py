@@ -385,41 +385,42 @@ class HipOps:
 
     def stream_prepare(self, h, xb, stats):
         """The bfloat16 copy ``xb`` of the 32-bit stream ``h`` and its rows' sums of squares
-        (``stats[0, :rows]``)."""
+        (``stats[:rows, 0]``)."""
         self._dev(h, "h", torch.float32, contiguous=False); self._dev(xb, "xb", torch.bfloat16, contiguous=False)
         self._dev(stats, "stats", torch.float32)
         rows, width = h.shape
-        if xb.shape[0] < rows or xb.shape[1] != width or stats.shape[1] < rows:
+        if xb.shape[0] < rows or xb.shape[1] != width or stats.shape[0] < rows:
             raise KernelError("stream_prepare: shapes do not fit")
         code = self._lib("gemv_slices").celeg_stream_prepare(
             _ptr(h), _c_int(self._rows(h, "h")), _ptr(xb), _c_int(self._rows(xb, "xb")), _ptr(stats),
-            _c_int(rows), _c_int(width), self._stream())
+            _c_int(stats.stride(0)), _c_int(rows), _c_int(width), self._stream())
         self._check(code, "stream_prepare")
 
     def embed_stream(self, table, token_ids, out, xb, stats):
         """Embedding gather into the 32-bit stream ``out``, its bfloat16 copy ``xb`` and the
-        rows' sums of squares (``stats[0, :rows]``)."""
+        rows' sums of squares (``stats[:rows, 0]``)."""
         self._dev(table, "table", torch.bfloat16); self._dev(token_ids, "token_ids", torch.int32)
         self._dev(out, "out", torch.float32); self._dev(xb, "xb", torch.bfloat16)
         self._dev(stats, "stats", torch.float32)
         rows, width = out.shape
-        if table.shape[1] != width or token_ids.numel() != rows or stats.shape[1] < rows \
+        if table.shape[1] != width or token_ids.numel() != rows or stats.shape[0] < rows \
                 or xb.shape != out.shape:
             raise KernelError("embed_stream: shapes do not fit")
         code = self._lib("gemv_slices").celeg_embed_stream(
-            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(xb), _ptr(stats), _c_int(rows),
-            _c_int(width), _c_int(table.shape[0]), self._stream())
+            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(xb), _ptr(stats), _c_int(stats.stride(0)),
+            _c_int(rows), _c_int(width), _c_int(table.shape[0]), self._stream())
         self._check(code, "embed_stream")
 
     def embed_stats(self, table, token_ids, out, stats):
-        """Embedding gather that also leaves every row's sum of squares in ``stats[0, :rows]``."""
+        """Embedding gather that also leaves every row's sum of squares in ``stats[:rows, 0]``."""
         self._dev(table, "table", torch.bfloat16); self._dev(token_ids, "token_ids", torch.int32)
         self._dev(out, "out", torch.float32); self._dev(stats, "stats", torch.float32)
         rows, width = out.shape
-        if table.shape[1] != width or token_ids.numel() != rows or stats.shape[1] < rows:
+        if table.shape[1] != width or token_ids.numel() != rows or stats.shape[0] < rows:
             raise KernelError("embed_stats: shapes do not fit")
         code = self._lib("gemv_fused").celeg_embed_stats(
-            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(stats), _c_int(rows), _c_int(width),
+            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(stats), _c_int(stats.stride(0)),
+            _c_int(rows), _c_int(width),
             _c_int(table.shape[0]), self._stream())
         self._check(code, "embed_stats")
 
@@ -429,17 +430,17 @@ class HipOps:
         """out = epilogue(prologue(a) w^T) for up to 64 rows, bfloat16 weights.
 
         ``a``: bfloat16 rows [M, K], or, with ``norm_weight``, the 32-bit residual stream,
-        normalised on the fly (``stats[:stat_blocks]`` holding partial sums of squares of its
-        rows if ``stat_blocks`` > 0).  ``rows`` picks rows of ``a``.  Epilogues: "store"
+        normalised on the fly (``stats[row, :stat_blocks]`` holding partial sums of squares
+        of its rows if ``stat_blocks`` > 0).  ``rows`` picks rows of ``a``.  Epilogues: "store"
         (bfloat16 [M, N]), "store_f32", "residual" (``out`` is the stream, [M, N] 32-bit,
-        added to in place; ``stats_out`` [``residual_stat_blocks``, >= M] receives partial
-        sums of squares of the new rows, ``last_stat_blocks`` says how many), "swiglu" (``w`` is [2N, K]: gate rows then up rows), "conv"
+        added to in place; ``stats_out`` [>= M, ``residual_stat_blocks``] receives partial
+        sums of squares of the new rows, ``last_stat_blocks`` says how many a row), "swiglu" (``w`` is [2N, K]: gate rows then up rows), "conv"
         (``w`` is [3N, K]: B, C, x rows; ``conv`` = (taps [N, L], bias or None, state
         [slots, L, N], seq_slot [M]); one new token per request).
 
         Up to 16 bfloat16 rows go to the k-sliced kernels, which also take the form behind a
         norm whose weight the caller has folded into ``w``: ``a`` is then the bfloat16 copy
-        of the stream and ``stats[:stat_blocks]`` its partial sums of squares, from which
+        of the stream and ``stats[row, :stat_blocks]`` its partial sums of squares, from which
         the rows' 1/rms (with ``eps``) scales the sums; their "residual" epilogue refreshes
         ``out_bf16``, the bfloat16 copy of the stream, if given."""
         if epilogue not in self._EPILOGUES:
@@ -490,7 +491,7 @@ class HipOps:
         prm.eps = eps
         if stat_blocks > 0:
             self._dev(stats, "stats", torch.float32)
-            if stats.shape[0] < stat_blocks:
+            if stats.shape[1] < stat_blocks:
                 raise KernelError("fused_linear: fewer partial sums than stat_blocks")
             prm.stats, prm.n_stat_blocks, prm.stats_ld = stats.data_ptr(), stat_blocks, stats.stride(0)
         prm.w, prm.stream_rows = w.data_ptr(), N
@@ -510,8 +511,8 @@ class HipOps:
             self.last_stat_blocks = self.residual_stat_blocks(M, N, K) if sliced else (N + 15) // 16
         if epilogue == "residual" and stats_out is not None:
             self._dev(stats_out, "stats_out", torch.float32)
-            if stats_out.shape[0] < self.last_stat_blocks or stats_out.shape[1] < M:
-                raise KernelError(f"fused_linear: stats_out must be [{self.last_stat_blocks}, >= rows]")
+            if stats_out.shape[1] < self.last_stat_blocks or stats_out.shape[0] < M:
+                raise KernelError(f"fused_linear: stats_out must be [>= rows, >= {self.last_stat_blocks}]")
             prm.stats_out, prm.stats_ld_out = stats_out.data_ptr(), stats_out.stride(0)
         if epilogue == "conv":
             taps_w, conv_bias, state, seq_slot = conv

@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import torch
 
-STAT_COLUMNS = 64   # most rows of a fused step
+STAT_COLUMNS = 64   # most rows of a fused step (rows of the partial-sum table)
 # Above this many rows the library's product (with separate norm and activation kernels)
 # is the faster one on MI355X (measured on the 1024-wide shape: 32 rows fused 1.28 ms a
 # step against 1.37 ms, 64 rows 2.28 ms against 1.67 ms).
@@ -32,12 +32,13 @@ def fused_rows_ok(rt, batch, *inner_sizes) -> bool:
 
 
 SLICED_MAX_ROWS = 16      # rows of the k-sliced kernels
+SLICED_MAX_STAT_BLOCKS = 512   # partial sums of squares a row may come with
 SLICED_MAX_COLUMNS = 16384   # wider products (the output head) keep their rows in LDS instead
 
 
 def stream_stats(rt, width: int) -> torch.Tensor:
     # up to one partial sum per 4 columns (the products for few rows use narrow workgroups)
-    return rt.ws.buf("stream_stats", ((width + 3) // 4, STAT_COLUMNS), torch.float32)
+    return rt.ws.buf("stream_stats", (STAT_COLUMNS, (width + 3) // 4), torch.float32)
 
 
 def stream_bf16(rt, rows: int, width: int) -> torch.Tensor:
@@ -71,7 +72,7 @@ def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None
         # scaled by the rows' 1/rms at the end
         stats = stream_stats(rt, h.shape[1])
         xb = stream_bf16(rt, h.shape[0], h.shape[1])
-        if not (blocks and getattr(rt, "stream_has_bf16", False)):
+        if not (0 < blocks <= SLICED_MAX_STAT_BLOCKS and getattr(rt, "stream_has_bf16", False)):
             rt.ops.stream_prepare(h, xb, stats)
             rt.stream_stat_blocks = blocks = 1
             rt.stream_has_bf16 = True

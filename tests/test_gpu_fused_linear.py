@@ -66,9 +66,9 @@ def test_norm_prologue_with_and_without_partial_sums(ops, M, N, K, with_stats):
     if with_stats:   # partial sums over 5 uneven column blocks
         blocks = 5
         cuts = [0, K // 7, K // 3, K // 2, K - 8, K]
-        stats = torch.zeros(blocks, 80, device=DEV)
+        stats = torch.zeros(80, blocks, device=DEV)
         for j in range(blocks):
-            stats[j, :M + 3] = (h[:, cuts[j]:cuts[j + 1]] ** 2).sum(dim=1)
+            stats[:M + 3, j] = (h[:, cuts[j]:cuts[j + 1]] ** 2).sum(dim=1)
     out = torch.empty(M, N, dtype=BF, device=DEV)
     ops.fused_linear(h, w, out, norm_weight=nw, eps=eps, rows=rows, stats=stats, stat_blocks=blocks)
     close(out, ref)
@@ -84,15 +84,15 @@ def test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, M, N, K):
     h = randn(M, N, seed=10)
     h0 = h.clone()
     blocks = ops.residual_stat_blocks(M, N, K)
-    stats = torch.full((blocks, 64), -1.0, device=DEV)
+    stats = torch.full((64, blocks), -1.0, device=DEV)
     ops.fused_linear(a, w, h, epilogue="residual", bias=b, stats_out=stats)
     assert ops.last_stat_blocks == blocks
     delta = (a.double() @ w.double().T + b.double())
     close(h, h0.double() + delta)
     # the product enters the sum rounded to bfloat16
     close(h - h0, delta.to(BF), rel=2e-3)
-    torch.testing.assert_close(stats[:, :M].sum(dim=0), (h ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
-    assert float(stats[:, M:].max()) == -1.0 if M < 64 else True
+    torch.testing.assert_close(stats[:M].sum(dim=1), (h ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
+    assert float(stats[M:].max()) == -1.0 if M < 64 else True
 
 
 @pytest.mark.parametrize("M,ff,K", [(1, 192, 64), (8, 4608, 1024), (19, 352, 128), (64, 200, 96)])
@@ -150,9 +150,9 @@ def scaled_case(M, N, K, streams, seed):
     folded = (w.float() * nw.reshape(1, -1)).to(BF)
     rows = torch.tensor([(3 * i + 1) % (M + 3) for i in range(M)], dtype=torch.int32, device=DEV)
     cuts = [0, K // 7, K // 3, K // 2, K - 8, K]
-    stats = torch.zeros(5, 80, device=DEV)
+    stats = torch.zeros(80, 5, device=DEV)
     for j in range(5):
-        stats[j, :M + 3] = (h[:, cuts[j]:cuts[j + 1]] ** 2).sum(dim=1)
+        stats[:M + 3, j] = (h[:, cuts[j]:cuts[j + 1]] ** 2).sum(dim=1)
     x = plain.rmsnorm(h.cpu(), nw.cpu(), 1e-5)[rows.long().cpu()].to(BF).double()
     return h, h.to(BF), stats, nw, w, folded, rows, x
 
@@ -204,14 +204,14 @@ def test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, M, H, taps
     hs = randn(steps, M, H, seed=19)
     state = torch.zeros(M + 2, taps, H, device=DEV)
     slots = torch.tensor([(M + 1 - i) for i in range(M)], dtype=torch.int32, device=DEV)
-    stats = torch.zeros(1, 64, device=DEV)
+    stats = torch.zeros(64, 1, device=DEV)
     outs = []
     for t in range(steps):
         y = torch.empty(M, H, dtype=BF, device=DEV)
         xb = torch.empty(M, H, dtype=BF, device=DEV)
         ops.stream_prepare(hs[t], xb, stats)
         assert torch.equal(xb, hs[t].to(BF))
-        torch.testing.assert_close(stats[0, :M], (hs[t] ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(stats[:M, 0], (hs[t] ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
         ops.fused_linear(xb, folded, y, epilogue="conv", eps=1e-5, stats=stats, stat_blocks=1,
                          bias=b_in, conv=(cw, cb, state, slots))
         outs.append(y.double().cpu())
@@ -230,7 +230,7 @@ def test_residual_refreshes_the_bfloat16_copy(ops):
     w = randn(N, K, seed=61, scale=0.1, dtype=BF)
     h = randn(M, N, seed=62)
     xb = torch.zeros(M + 2, N, dtype=BF, device=DEV)
-    stats = torch.zeros(ops.residual_stat_blocks(M, N, K), 64, device=DEV)
+    stats = torch.zeros(64, ops.residual_stat_blocks(M, N, K), device=DEV)
     ops.fused_linear(a, w, h, epilogue="residual", stats_out=stats, out_bf16=xb)
     assert torch.equal(xb[:M], h.to(BF)) and float(xb[M:].abs().max()) == 0.0
 
@@ -240,20 +240,20 @@ def test_embed_stream(ops):
     ids = torch.tensor([5, 330, 0, 17], dtype=torch.int32, device=DEV)
     out = torch.empty(4, 96, device=DEV)
     xb = torch.empty(4, 96, dtype=BF, device=DEV)
-    stats = torch.zeros(6, 64, device=DEV)
+    stats = torch.zeros(64, 6, device=DEV)
     ops.embed_stream(table, ids, out, xb, stats)
     assert torch.equal(out, table[ids.long()].float()) and torch.equal(xb, table[ids.long()])
-    torch.testing.assert_close(stats[0, :4], (out ** 2).sum(dim=1), rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(stats[:4, 0], (out ** 2).sum(dim=1), rtol=1e-6, atol=1e-6)
 
 
 def test_embed_stats(ops):
     table = randn(331, 96, seed=20, dtype=BF)
     ids = torch.tensor([5, 330, 0, 17], dtype=torch.int32, device=DEV)
     out = torch.empty(4, 96, device=DEV)
-    stats = torch.zeros(6, 64, device=DEV)
+    stats = torch.zeros(64, 6, device=DEV)
     ops.embed_stats(table, ids, out, stats)
     assert torch.equal(out, table[ids.long()].float())
-    torch.testing.assert_close(stats[0, :4], (out ** 2).sum(dim=1), rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(stats[:4, 0], (out ** 2).sum(dim=1), rtol=1e-6, atol=1e-6)
 
 
 def test_unsupported_sizes_are_refused(ops):
