@@ -32,4 +32,9 @@ struct GemvParams {
     // E_RESIDUAL of the k-sliced kernels: the bfloat16 copy of the stream, or null
     void* out_bf16;
     int ld_bf16;
+    // weight layout of the k-sliced kernels: element (n, k) of w lies at
+    //   n * w_row_stride + (k / 32) * w_kb_stride + k % 32
+    // (rows one after the other: K and 32; blocks of 32 k-values with the rows side by side
+    // inside a block: 32 and rows * 32)
+    long long w_row_stride, w_kb_stride;
 };

@@ -72,7 +72,8 @@ void gemv_slices_kernel(const GemvParams p) {
         const bf16* wrow[NS];
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + idx, N - 1)) * K + slice * Ks;
+            wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + idx, N - 1)) * p.w_row_stride;
+        const int k_slice = slice * Ks;
         const int chunks = (Ks + 63) >> 6;
         const int c_begin = wave * chunks / KW, c_end = (wave + 1) * chunks / KW;
         floatx4_t acc[NS];
@@ -86,10 +87,12 @@ void gemv_slices_kernel(const GemvParams p) {
                 for (int v = 0; v < 2; ++v) {
                     const int k = (c0 + u) * 64 + v * 32 + q * 8;
                     const bool in = c0 + u < c_end && k + 8 <= Ks;
+                    const int kw_ = k_slice + k;      // 8 values from here never leave a block of 32
+                    const size_t w_off = static_cast<size_t>(kw_ >> 5) * p.w_kb_stride + (kw_ & 31);
                     av[u][v] = in ? *reinterpret_cast<const Frag2*>(arow + k) : Frag2{};
 #pragma unroll
                     for (int s = 0; s < NS; ++s)
-                        wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
+                        wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + w_off) : Frag2{};
                 }
 #pragma unroll
             for (int u = 0; u < U; ++u)
@@ -124,7 +127,7 @@ void gemv_slices_kernel(const GemvParams p) {
     // made without conditions, from clamped places, and masked afterwards: a load under a
     // condition of its own is waited for before the next one is asked for.)
     constexpr int LPR = 64 / ROWS_FW;
-    constexpr int NFIRST = 16, NREST = SLICES_MAX_STAT_BLOCKS / LPR > NFIRST ? SLICES_MAX_STAT_BLOCKS / LPR - NFIRST : 0;
+    constexpr int NFIRST = 16;
     float ssq = 0.f;
     if (p.stats) {
         const int nb = p.n_stat_blocks;
@@ -133,12 +136,12 @@ void gemv_slices_kernel(const GemvParams p) {
         float part[NFIRST];
 #pragma unroll
         for (int i = 0; i < NFIRST; ++i) part[i] = srow[min(sj + LPR * i, nb - 1)];
-        if (nb > NFIRST * LPR) {                // the same for every lane
-            float rest[NREST > 0 ? NREST : 1];
+        for (int i0 = NFIRST; i0 * LPR < nb; i0 += 8) {   // the same for every lane; rare
+            float rest[8];
 #pragma unroll
-            for (int i = 0; i < NREST; ++i) rest[i] = srow[min(sj + LPR * (NFIRST + i), nb - 1)];
+            for (int i = 0; i < 8; ++i) rest[i] = srow[min(sj + LPR * (i0 + i), nb - 1)];
 #pragma unroll
-            for (int i = 0; i < NREST; ++i) ssq += sj + LPR * (NFIRST + i) < nb ? rest[i] : 0.f;
+            for (int i = 0; i < 8; ++i) ssq += sj + LPR * (i0 + i) < nb ? rest[i] : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < NFIRST; ++i) ssq += sj + LPR * i < nb ? part[i] : 0.f;
@@ -263,7 +266,8 @@ extern "C" int celeg_gemv_slices_blocks(int M, int N, int K) {
     return (N + mp - 1) / mp;
 }
 
-// M <= 16, K % 8 == 0, bfloat16 a and w.  Fields of GemvParams that are read: a, lda, rows,
+// M <= 16, K % 8 == 0, bfloat16 a and w (w in either layout that w_row_stride and
+// w_kb_stride describe).  Fields of GemvParams that are read: a, lda, rows,
 // stats/n_stat_blocks/stats_ld/eps (scale by 1/rms if stats is set), w, stream_rows, bias,
 // M, N, K, out, ldo, and per epilogue out_bf16/ld_bf16/stats_out/stats_ld_out (residual) or
 // conv_w/conv_b/state/state_slot_stride/seq_slot/taps (conv).
@@ -271,6 +275,8 @@ extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t 
     const GemvParams& p = *params;
     if (p.M <= 0 || p.N <= 0) return 0;
     if (p.M > 16 || p.K <= 0 || (p.K % 8) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
+    if ((p.w_row_stride % 8) || (p.w_kb_stride % 8) || p.w_row_stride <= 0 || p.w_kb_stride <= 0)
+        return static_cast<int>(hipErrorInvalidValue);
     if (p.stats && (p.n_stat_blocks < 1 || p.n_stat_blocks > SLICES_MAX_STAT_BLOCKS))
         return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.taps > SLICES_MAX_TAPS || p.stream_rows != p.N))

@@ -383,6 +383,16 @@ class HipOps:
                 _c_int(rows), _c_int(n), _c_int(k)))
         return (n + 15) // 16
 
+    @staticmethod
+    def pack_weight(w: torch.Tensor) -> torch.Tensor:
+        """``w`` [rows, K] as [K/32, rows, 32]: blocks of 32 k-values with the rows side by
+        side inside a block, the layout in which the k-sliced products read whole runs of
+        memory per load.  K must be a multiple of 32."""
+        rows, K = w.shape
+        if K % 32:
+            raise KernelError("pack_weight: the inner size must be a multiple of 32")
+        return w.reshape(rows, K // 32, 32).permute(1, 0, 2).contiguous()
+
     def stream_prepare(self, h, xb, stats):
         """The bfloat16 copy ``xb`` of the 32-bit stream ``h`` and its rows' sums of squares
         (``stats[:rows, 0]``)."""
@@ -442,15 +452,19 @@ class HipOps:
         norm whose weight the caller has folded into ``w``: ``a`` is then the bfloat16 copy
         of the stream and ``stats[row, :stat_blocks]`` its partial sums of squares, from which
         the rows' 1/rms (with ``eps``) scales the sums; their "residual" epilogue refreshes
-        ``out_bf16``, the bfloat16 copy of the stream, if given."""
+        ``out_bf16``, the bfloat16 copy of the stream, if given.  They also take ``w`` in the
+        layout of ``pack_weight``."""
         if epilogue not in self._EPILOGUES:
             raise KernelError(f"fused_linear: unknown epilogue '{epilogue}'")
         self._dev(w, "w", torch.bfloat16)
         streams = {"swiglu": 2, "conv": 3}.get(epilogue, 1)
-        K = w.shape[1]
-        if w.shape[0] % streams:
+        packed = w.dim() == 3                  # [K/32, rows, 32], see pack_weight
+        if packed and w.shape[2] != 32:
+            raise KernelError("fused_linear: a packed weight is [K/32, rows, 32]")
+        w_rows, K = (w.shape[1], w.shape[0] * 32) if packed else (w.shape[0], w.shape[1])
+        if w_rows % streams:
             raise KernelError("fused_linear: weight rows do not split into the epilogue's streams")
-        N = w.shape[0] // streams
+        N = w_rows // streams
         M = n_rows if n_rows is not None else (rows.numel() if rows is not None else a.shape[0])
         if not self.fused_linear_ok(M, K):
             raise KernelError(f"fused_linear: {M} rows with inner size {K} are not supported "
@@ -499,6 +513,9 @@ class HipOps:
         prm.M, prm.N, prm.K = M, N, K
         prm.out, prm.ldo = out.data_ptr(), self._rows(out, "out")
         sliced = norm_weight is None and M <= 16 and self.use_sliced
+        if packed and not sliced:
+            raise KernelError("fused_linear: packed weights go with bfloat16 rows, up to 16 of them")
+        prm.w_row_stride, prm.w_kb_stride = (32, w_rows * 32) if packed else (K, 32)
         if out_bf16 is not None:
             if not (sliced and epilogue == "residual"):
                 raise KernelError("fused_linear: out_bf16 goes with the residual epilogue for up to 16 rows")
@@ -553,4 +570,5 @@ class _GemvParams(ctypes.Structure):
         ("conv_w", ctypes.c_void_p), ("conv_b", ctypes.c_void_p), ("state", ctypes.c_void_p),
         ("state_slot_stride", ctypes.c_size_t), ("seq_slot", ctypes.c_void_p), ("taps", ctypes.c_int),
         ("out_bf16", ctypes.c_void_p), ("ld_bf16", ctypes.c_int),
+        ("w_row_stride", ctypes.c_longlong), ("w_kb_stride", ctypes.c_longlong),
     ]

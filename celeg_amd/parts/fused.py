@@ -50,15 +50,29 @@ def _sliced(rt, rows: int) -> bool:
     return rows <= SLICED_MAX_ROWS and getattr(rt.ops, "use_sliced", False)
 
 
+def _pack(rt, w: torch.Tensor) -> torch.Tensor:
+    return rt.ops.pack_weight(w) if w.shape[1] % 32 == 0 and hasattr(rt.ops, "pack_weight") else w
+
+
 def folded_weight(rt, w: torch.Tensor, norm_weight: torch.Tensor) -> torch.Tensor:
-    """``w`` with the norm's weight multiplied into its columns: (x * nw) w^T = x (w * nw)^T.
-    Made once per (weight, norm) pair and kept."""
+    """``w`` with the norm's weight multiplied into its columns: (x * nw) w^T = x (w * nw)^T,
+    in the layout the products for few rows read best.  Made once per (weight, norm) pair
+    and kept."""
     cache = rt.__dict__.setdefault("folded_weights", {})
     key = (w.data_ptr(), norm_weight.data_ptr())
     hit = cache.get(key)
     if hit is None:
-        hit = (w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype).contiguous()
+        hit = _pack(rt, (w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype))
         cache[key] = hit
+    return hit
+
+
+def packed_weight(rt, w: torch.Tensor) -> torch.Tensor:
+    """A copy of ``w`` in the layout the products for few rows read best; made once."""
+    cache = rt.__dict__.setdefault("packed_weights", {})
+    hit = cache.get(w.data_ptr())
+    if hit is None:
+        hit = cache[w.data_ptr()] = _pack(rt, w)
     return hit
 
 
@@ -67,7 +81,7 @@ def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None
     blocks = getattr(rt, "stream_stat_blocks", 0)
     M = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
     streams = {"swiglu": 2, "conv": 3}.get(epilogue, 1)
-    if _sliced(rt, M) and w.shape[0] // streams <= SLICED_MAX_COLUMNS:
+    if _sliced(rt, M) and w.shape[0] // streams <= SLICED_MAX_COLUMNS and w.dtype == torch.bfloat16:
         # the stream's bfloat16 copy times the weight with the norm's weight folded in,
         # scaled by the rows' 1/rms at the end
         stats = stream_stats(rt, h.shape[1])
@@ -89,7 +103,8 @@ def linear_into_stream(rt, a, w, h, bias=None):
     the stream's bfloat16 copy)."""
     stats = stream_stats(rt, h.shape[1])
     sliced = _sliced(rt, h.shape[0])
-    rt.ops.fused_linear(a, w, h, epilogue="residual", bias=bias, stats_out=stats,
+    rt.ops.fused_linear(a, packed_weight(rt, w) if sliced else w, h, epilogue="residual", bias=bias,
+                        stats_out=stats,
                         out_bf16=stream_bf16(rt, h.shape[0], h.shape[1]) if sliced else None)
     rt.stream_stat_blocks = rt.ops.last_stat_blocks
     rt.stream_has_bf16 = sliced

@@ -224,6 +224,32 @@ def test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, M, H, taps
     assert float(state[0].abs().max()) == 0.0          # a slot nobody uses stays zero
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (4, 1024, 1024), (5, 77, 352), (8, 96, 4608), (16, 272, 1024)])
+def test_packed_weights_give_the_same_bits(ops, M, N, K):
+    """The layout of blocks of 32 k-values changes where the weights lie, not what is added
+    in which order: every epilogue gives identical results from either layout."""
+    h, xb, stats, nw, w, folded, rows, x = scaled_case(M, N, K, 1, 70)
+    b = randn(N, seed=74)
+    packed = ops.pack_weight(folded)
+    assert packed.shape == (K // 32, N, 32)
+    outs = []
+    for wt in (folded, packed):
+        out32 = torch.empty(M, N, device=DEV)
+        ops.fused_linear(xb, wt, out32, epilogue="store_f32", eps=1e-5, stats=stats, stat_blocks=5,
+                         rows=rows, bias=b)
+        hh = randn(M, N, seed=75)
+        so = torch.zeros(64, ops.residual_stat_blocks(M, N, K), device=DEV)
+        ops.fused_linear(xb[:M], wt, hh, epilogue="residual", stats_out=so)
+        outs.append((out32, hh, so))
+    for got, ref in zip(outs[1], outs[0]):
+        assert torch.equal(got, ref)
+    if N % 2 == 0:   # two streams from one packed tensor
+        act = [torch.empty(M, N // 2, dtype=BF, device=DEV) for _ in range(2)]
+        for o, wt in zip(act, (folded, packed)):
+            ops.fused_linear(xb, wt, o, epilogue="swiglu", eps=1e-5, stats=stats, stat_blocks=5, rows=rows)
+        assert torch.equal(act[0], act[1])
+
+
 def test_residual_refreshes_the_bfloat16_copy(ops):
     M, N, K = 6, 200, 352
     a = randn(M, K, seed=60, dtype=BF)
