@@ -11,6 +11,7 @@
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_MAX_K 128
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float penalised_logit(const float* __restrict__ row,
                                                  const uint8_t* __restrict__ seen, float penalty,
@@ -58,12 +59,39 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
     if (temperature <= 0.0f || top_k == 1) {
         // ---- penalised argmax, lowest index wins ties
+        // Groups of 4 logits, 8 groups of a thread asked for before any is looked at (a
+        // row of 65,536 logits is then two round trips to memory instead of 64).
         float best = -INFINITY;
         int best_i = 0x7fffffff;
-        for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-            const float v = penalised_logit(row, seen, penalty, i);
+        const bool pen = seen && penalty > 1.0f;
+        const bool vec = (reinterpret_cast<uintptr_t>(row) & 15) == 0 &&
+                         (!pen || (reinterpret_cast<uintptr_t>(seen) & 3) == 0);
+        const int n4 = vec ? vocab >> 2 : 0;
+        auto take = [&](float v, unsigned seen_byte, int i) {
+            if (seen_byte) v = v >= 0.0f ? v / penalty : v * penalty;
             if (best_i == 0x7fffffff || v > best) { best = v; best_i = i; }
+        };
+        constexpr int UN = 8;
+        for (int g0 = tid; g0 < n4; g0 += SAMPLE_THREADS * UN) {
+            floatx4_t v[UN];
+            unsigned sn[UN];
+#pragma unroll
+            for (int j = 0; j < UN; ++j) {
+                const int g = min(g0 + j * SAMPLE_THREADS, n4 - 1);      // clamped, masked below
+                v[j] = reinterpret_cast<const floatx4_t*>(row)[g];
+                sn[j] = pen ? reinterpret_cast<const unsigned*>(seen)[g] : 0u;
+            }
+#pragma unroll
+            for (int j = 0; j < UN; ++j) {
+                const int g = g0 + j * SAMPLE_THREADS;
+                if (g < n4) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) take(v[j][e], (sn[j] >> (8 * e)) & 0xffu, 4 * g + e);
+                }
+            }
         }
+        for (int i = 4 * n4 + tid; i < vocab; i += SAMPLE_THREADS)      // what the groups left
+            take(row[i], pen ? seen[i] : 0u, i);
         for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) {
             const float ov = __shfl_xor(best, off, CELEG_WAVE);
             const int oi = __shfl_xor(best_i, off, CELEG_WAVE);
