@@ -176,6 +176,29 @@ def test_sampling_kernel_equals_plain_sampler(ops, vocab):
         assert got[r] == want, f"row {r}"
 
 
+@pytest.mark.parametrize("vocab", [5, 331, 4100, 65536, 70001])
+def test_arg_max_lowest_index_wins_with_and_without_penalty(ops, vocab):
+    g = torch.Generator().manual_seed(vocab + 1)
+    R = 7
+    logits = torch.randn(R, vocab, generator=g)
+    top = float(logits.max()) + 1.0
+    for r in range(R):     # the maximum several times, first at a place that differs per row
+        first = (r * 977 + vocab // 3) % vocab
+        logits[r, first] = top
+        logits[r, (first + vocab // 2) % vocab] = top
+        logits[r, vocab - 1] = top
+    rows, want = [], []
+    for r in range(R):
+        ties = sorted({(r * 977 + vocab // 3) % vocab, ((r * 977 + vocab // 3) % vocab + vocab // 2) % vocab, vocab - 1})
+        if r % 2:    # the first maximum was seen and is pushed down by the penalty
+            rows.append((0.0, 1, 1.0, 1.5, 0.0, [ties[0]]))
+            want.append(ties[1] if len(ties) > 1 else ties[0])
+        else:
+            rows.append((0.0, 1, 1.0, 1.0, 0.0, None))
+            want.append(ties[0])
+    assert run_sample(ops, logits, rows) == want
+
+
 def test_mark_seen(ops):
     seen = torch.zeros(3, 100, dtype=torch.uint8, device=DEV)
     toks = torch.tensor([5, 99, 5, 17], dtype=torch.int32, device=DEV)
