@@ -4,3 +4,11 @@ from .config import (Lfm2Config, ModelSpec, PartSpec, LayerSpec, RunStep, regist
                      registered_architectures, spec_from_config)
 
 __version__ = "0.1.0"
+
+
+def __getattr__(name):
+    # the engine pulls in the GPU side; it is loaded when first asked for
+    if name in ("Engine", "load_model"):
+        from . import engine
+        return getattr(engine, name)
+    raise AttributeError(f"module 'celeg_amd' has no attribute '{name}'")
