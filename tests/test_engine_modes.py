@@ -96,3 +96,70 @@ def test_captured_decode_steps_equal_eager_steps(model_folders, dtype):
             assert torch.equal(out[True][rid], out[False][rid])
         else:
             assert_close(out[True][rid], out[False][rid].double(), dtype, f"graph/{rid}")
+
+
+def merged_schedule(per_request_steps):
+    """Steps of several requests laid side by side: step k holds the k-th step of each."""
+    merged = []
+    for k in range(max(len(v) for v in per_request_steps.values())):
+        entries, end = [], []
+        for v in per_request_steps.values():
+            if k < len(v):
+                entries += v[k]["entries"]
+                end += v[k]["end"]
+        merged.append({"step": k, "entries": entries, "end": end})
+    return merged
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_long_decoding(model_folders, name, dtype):
+    """Three requests decoded one token a step for most of the context (hundreds of steps
+    through the replayed graphs, across many page edges), every position compared with the
+    plain implementation."""
+    from celeg_amd.engine import load_model
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders(name, storage, WEIGHT_STD)
+    cfg = TINY[name][0]
+    n = min(cfg["max_position_embeddings"], 250)
+    reqs = {f"long{i}": random_tokens(cfg["vocab_size"], n - 7 * i, seed=900 + i) for i in range(3)}
+    steps = merged_schedule({rid: tail_decode_schedule({rid: toks}, tail=len(toks) - 20)
+                             for rid, toks in reqs.items()})
+    max_tokens = peak_tokens(steps)
+    lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=max_tokens // 16, max_requests=4,
+                    max_batched_tokens=256)
+    got = EngineDriver(lm).run(steps)
+    cfgp, W = plain.load_model_folder(folder)
+    for rid, toks in reqs.items():
+        assert_close(got[rid], plain.model_logits(cfgp, W, toks), dtype, f"{name}/{dtype}/long/{rid}")
+    assert lm.runner._graphs, "no decode step was replayed from a graph"
+    lm.cache.check()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(model_folders, name, dtype):
+    """Position 0 and its neighbours: requests that start with one, two and three tokens
+    side by side, then go on token by token."""
+    from celeg_amd.engine import load_model
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders(name, storage, WEIGHT_STD)
+    vocab = TINY[name][0]["vocab_size"]
+    reqs = {f"first{i}": random_tokens(vocab, 7, seed=950 + i) for i in range(3)}
+    per = {}
+    for i, (rid, toks) in enumerate(reqs.items()):
+        first = i + 1
+        mine = [{"step": 0, "entries": [{"id": rid, "tokens": toks[:first], "want": list(range(first))}], "end": []}]
+        for p in range(first, len(toks)):
+            mine.append({"step": len(mine), "entries": [{"id": rid, "tokens": [toks[p]], "want": [0]}],
+                         "end": [rid] if p == len(toks) - 1 else []})
+        per[rid] = mine
+    lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=8, max_requests=4, max_batched_tokens=64)
+    got = EngineDriver(lm).run(merged_schedule(per))
+    cfgp, W = plain.load_model_folder(folder)
+    for rid, toks in reqs.items():
+        assert len(got[rid]) == 7
+        assert_close(got[rid], plain.model_logits(cfgp, W, toks), dtype, f"{name}/{dtype}/first/{rid}")
+    lm.cache.check()
