@@ -82,10 +82,14 @@ class Sampler:
         self._seen: Optional[torch.Tensor] = None   # [max_requests, vocab] uint8, made on need
         cap = max_requests
         pin = torch.device(device).type == "cuda"
-        self._fparams = torch.empty(cap * 4, dtype=torch.float32, pin_memory=pin)
-        self._iparams = torch.empty(cap * 2, dtype=torch.int32, pin_memory=pin)
-        self._fparams_dev = torch.empty(cap * 4, dtype=torch.float32, device=device)
-        self._iparams_dev = torch.empty(cap * 2, dtype=torch.int32, device=device)
+        # one staging buffer and one device buffer for a step's parameters: 4 floats a row,
+        # then 2 ints a row (the same bytes seen as 32-bit floats and as 32-bit ints)
+        self._params = torch.zeros(cap * 6, dtype=torch.float32, pin_memory=pin)
+        self._params_dev = torch.zeros(cap * 6, dtype=torch.float32, device=device)
+        self._fparams, self._iparams = self._params[:cap * 4], self._params[cap * 4:].view(torch.int32)
+        self._fparams_dev = self._params_dev[:cap * 4]
+        self._iparams_dev = self._params_dev[cap * 4:].view(torch.int32)
+        self._uploaded = None      # what the device buffer holds: a copy of the staged values
         self._tokens_dev = torch.empty(cap, dtype=torch.int32, device=device)
 
     def begin(self, slot: int, config: GenerationConfig, rng: Optional[XorShift64Star] = None) -> None:
@@ -130,8 +134,12 @@ class Sampler:
                                    0.0 if c.greedy else self._rng[slot].next_unit())
             i[2 * r] = c.top_k
             i[2 * r + 1] = slot if (c.repetition_penalty > 1.0 and self._seen is not None) else -1
-        self._fparams_dev[:4 * R].copy_(self._fparams[:4 * R], non_blocking=True)
-        self._iparams_dev[:2 * R].copy_(self._iparams[:2 * R], non_blocking=True)
+        # greedy rows have nothing that changes from step to step: ship only what differs
+        # from what the device holds
+        staged = self._params.numpy()
+        if self._uploaded is None or not np.array_equal(staged.view(np.int32), self._uploaded):
+            self._params_dev.copy_(self._params, non_blocking=True)
+            self._uploaded = staged.view(np.int32).copy()
         self.ops.sample(logits, self._fparams_dev, self._iparams_dev, self._seen,
                         self._tokens_dev[:R])
         return self._tokens_dev[:R].tolist()   # the step's one synchronisation
