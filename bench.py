@@ -72,6 +72,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--batch", type=int, default=BATCH,
+                    help="for profiling with --phase decode: another batch size than the headline's 8")
     ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
                          "decode measurement (the line printed then holds only that part)")
@@ -93,7 +95,7 @@ def main() -> int:
         cfg["num_hidden_layers"] = args.layers
         cfg["layer_types"] = cfg["layer_types"][:args.layers]
     context = cfg["max_position_embeddings"]
-    max_batch = BATCH if args.no_points or args.phase != "all" else 64
+    max_batch = max(BATCH, args.batch) if args.no_points or args.phase != "all" else 64
     need = PROMPT_TOKENS + args.steps + args.warmup + 1
     if need > context:
         raise SystemExit(f"--steps + --warmup exceed the context of {context}")
@@ -125,6 +127,12 @@ def main() -> int:
         bench.close()
         return result
 
+    if args.phase == "decode" and args.batch != BATCH:
+        result = decode(args.batch)
+        print(json.dumps({"metric": f"decode tok/s @ batch {args.batch} (LFM2-350M shape, bf16)",
+                          "value": round(result["tokens_per_second"], 1), "unit": "tokens/s",
+                          "ms_per_step": round(result["ms_per_step"], 4), "phase": "decode"}))
+        return 0
     main_run = decode(BATCH)
     points = {}
     if not args.no_points and args.phase == "all":

@@ -65,11 +65,90 @@ __global__ void rmsnorm_kernel(TX* __restrict__ x, const TD* __restrict__ delta,
     }
 }
 
+// The same with the row kept in registers: groups of 4 values, up to RMS_NV groups a
+// thread (width <= 4 * RMS_NV * 256), every load of a row asked for before the first is used.
+#define RMS_NV 4
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    typedef float raw __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        const raw r = *reinterpret_cast<const raw*>(p);
+        v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+        *reinterpret_cast<raw*>(p) = raw{v[0], v[1], v[2], v[3]};
+    }
+};
+template <> struct Vec4<bf16> {
+    typedef __bf16 raw __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ void load(const bf16* p, float (&v)[4]) {
+        const raw r = *reinterpret_cast<const raw*>(p);
+        v[0] = static_cast<float>(r[0]); v[1] = static_cast<float>(r[1]);
+        v[2] = static_cast<float>(r[2]); v[3] = static_cast<float>(r[3]);
+    }
+    static __device__ __forceinline__ void store(bf16* p, const float (&v)[4]) {
+        *reinterpret_cast<raw*>(p) = raw{static_cast<__bf16>(v[0]), static_cast<__bf16>(v[1]),
+                                         static_cast<__bf16>(v[2]), static_cast<__bf16>(v[3])};
+    }
+};
+
+template <typename TX, typename TD, typename TO>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(
+    TX* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+    TO* __restrict__ out, const int* __restrict__ rows, int width, float eps, int write_back) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const size_t src = static_cast<size_t>(rows ? rows[r] : r) * width;
+    const int groups = width >> 2;
+    float v[RMS_NV][4], d[RMS_NV][4], wv[RMS_NV][4];
+#pragma unroll
+    for (int j = 0; j < RMS_NV; ++j) {
+        const int g = min(static_cast<int>(threadIdx.x) + j * 256, groups - 1);   // clamped, masked below
+        Vec4<TX>::load(x + src + 4 * g, v[j]);
+        if (delta) Vec4<TD>::load(delta + src + 4 * g, d[j]);
+        Vec4<float>::load(w + 4 * g, wv[j]);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < RMS_NV; ++j) {
+        const bool in = static_cast<int>(threadIdx.x) + j * 256 < groups;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (delta) v[j][e] += d[j][e];
+            if (in) sum += v[j][e] * v[j][e];
+        }
+        if (in && delta && write_back) Vec4<TX>::store(x + src + 4 * (threadIdx.x + j * 256), v[j]);
+    }
+    sum = block_sum(sum, scratch);
+    const float inv = 1.0f / sqrtf(sum / static_cast<float>(width) + eps);
+    TO* dst = out + static_cast<size_t>(r) * width;
+#pragma unroll
+    for (int j = 0; j < RMS_NV; ++j) {
+        if (static_cast<int>(threadIdx.x) + j * 256 < groups) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = v[j][e] * inv * wv[j][e];
+            Vec4<TO>::store(dst + 4 * (threadIdx.x + j * 256), o);
+        }
+    }
+}
+
 template <typename TX, typename TD>
 static int rmsnorm_dispatch_out(TX* x, const TD* delta, const float* w, void* out, int out_dtype,
                                 const int* rows, int n_rows, int width, float eps,
                                 int write_back, hipStream_t stream) {
     dim3 grid(n_rows), block(width >= 1024 ? 256 : (width >= 256 ? 128 : 64));
+    const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (width % 4 == 0 && width >= 512 && width <= 4 * RMS_NV * 256 && aligned(x) && aligned(w) &&
+        aligned(out) && (!delta || aligned(delta))) {
+        if (out_dtype == CELEG_F32)
+            hipLaunchKernelGGL((rmsnorm_vec_kernel<TX, TD, float>), grid, dim3(256), 0, stream, x, delta,
+                               w, static_cast<float*>(out), rows, width, eps, write_back);
+        else
+            hipLaunchKernelGGL((rmsnorm_vec_kernel<TX, TD, bf16>), grid, dim3(256), 0, stream, x, delta,
+                               w, static_cast<bf16*>(out), rows, width, eps, write_back);
+        return CELEG_LAUNCH_RESULT();
+    }
     if (out_dtype == CELEG_F32)
         hipLaunchKernelGGL((rmsnorm_kernel<TX, TD, float>), grid, block, 0, stream, x, delta, w,
                            static_cast<float*>(out), rows, width, eps, write_back);
@@ -120,10 +199,44 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     out[i] = from_float<T>((g / (1.0f + expf(-g))) * u);
 }
 
+// groups of 8 values a thread (ff % 8 == 0)
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out,
+                                                         int ff, size_t groups) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= groups) return;
+    const int per_row = ff >> 3;
+    const size_t t = i / per_row;
+    const int c = static_cast<int>(i - t * per_row) * 8;
+    float g[2][4], u[2][4], o[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        Vec4<T>::load(gu + t * 2 * ff + c + 4 * h, g[h]);
+        Vec4<T>::load(gu + t * 2 * ff + ff + c + 4 * h, u[h]);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[h][e] = (g[h][e] / (1.0f + expf(-g[h][e]))) * u[h][e];
+        Vec4<T>::store(out + t * ff + c + 4 * h, o[h]);
+    }
+}
+
 extern "C" int celeg_swiglu(const void* gu, void* out, int dtype, int rows, int ff,
                             hipStream_t stream) {
     const size_t total = static_cast<size_t>(rows) * ff;
     if (total == 0) return 0;
+    if (ff % 8 == 0 && (reinterpret_cast<uintptr_t>(gu) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        const size_t groups = total / 8;
+        dim3 vblock(256), vgrid(static_cast<unsigned>((groups + 255) / 256));
+        if (dtype == CELEG_F32)
+            hipLaunchKernelGGL(swiglu_vec_kernel<float>, vgrid, vblock, 0, stream,
+                               static_cast<const float*>(gu), static_cast<float*>(out), ff, groups);
+        else
+            hipLaunchKernelGGL(swiglu_vec_kernel<bf16>, vgrid, vblock, 0, stream,
+                               static_cast<const bf16*>(gu), static_cast<bf16*>(out), ff, groups);
+        return CELEG_LAUNCH_RESULT();
+    }
     dim3 block(256), grid(static_cast<unsigned>((total + 255) / 256));
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream,

@@ -41,7 +41,7 @@ def test_embed(ops, dtype, vocab, width, rows):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,width", [(5, 96), (3, 1000), (9, 4100)])
+@pytest.mark.parametrize("rows,width", [(5, 96), (3, 1000), (9, 4100), (7, 1024), (4, 4096), (3, 516), (5, 2052)])
 def test_rmsnorm_with_delta_and_rows(ops, dtype, rows, width):
     x = randn(rows, width, seed=3)
     delta = randn(rows, width, seed=4, dtype=dtype)
@@ -77,8 +77,8 @@ def test_rmsnorm_reference_vector(ops):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_swiglu(ops, dtype):
-    rows, ff = 11, 352
+@pytest.mark.parametrize("rows,ff", [(11, 352), (3, 4608), (5, 100), (2, 8)])
+def test_swiglu(ops, dtype, rows, ff):
     gu = randn(rows, 2 * ff, seed=6, scale=2.0, dtype=dtype)
     out = torch.empty(rows, ff, dtype=dtype, device=DEV)
     ops.swiglu(gu, out)
