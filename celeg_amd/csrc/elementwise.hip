@@ -133,14 +133,68 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(
     }
 }
 
+// One wavefront per row (width <= 4 * RMS_NV * 64): no barrier, 4 rows a workgroup.
+template <typename TX, typename TD, typename TO>
+__global__ __launch_bounds__(256) void rmsnorm_wave_kernel(
+    TX* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+    TO* __restrict__ out, const int* __restrict__ rows, int n_rows, int width, float eps,
+    int write_back) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= n_rows) return;
+    const size_t src = static_cast<size_t>(rows ? rows[r] : r) * width;
+    const int groups = width >> 2;
+    float v[RMS_NV][4], d[RMS_NV][4], wv[RMS_NV][4];
+#pragma unroll
+    for (int j = 0; j < RMS_NV; ++j) {
+        const int g = min(lane + j * 64, groups - 1);   // clamped, masked below
+        Vec4<TX>::load(x + src + 4 * g, v[j]);
+        if (delta) Vec4<TD>::load(delta + src + 4 * g, d[j]);
+        Vec4<float>::load(w + 4 * g, wv[j]);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < RMS_NV; ++j) {
+        const bool in = lane + j * 64 < groups;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (delta) v[j][e] += d[j][e];
+            if (in) sum += v[j][e] * v[j][e];
+        }
+        if (in && delta && write_back) Vec4<TX>::store(x + src + 4 * (lane + j * 64), v[j]);
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sqrtf(sum / static_cast<float>(width) + eps);
+    TO* dst = out + static_cast<size_t>(r) * width;
+#pragma unroll
+    for (int j = 0; j < RMS_NV; ++j) {
+        if (lane + j * 64 < groups) {
+            float o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = v[j][e] * inv * wv[j][e];
+            Vec4<TO>::store(dst + 4 * (lane + j * 64), o);
+        }
+    }
+}
+
 template <typename TX, typename TD>
 static int rmsnorm_dispatch_out(TX* x, const TD* delta, const float* w, void* out, int out_dtype,
                                 const int* rows, int n_rows, int width, float eps,
                                 int write_back, hipStream_t stream) {
     dim3 grid(n_rows), block(width >= 1024 ? 256 : (width >= 256 ? 128 : 64));
     const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    if (width % 4 == 0 && width >= 512 && width <= 4 * RMS_NV * 256 && aligned(x) && aligned(w) &&
+    if (width % 4 == 0 && width >= 256 && width <= 4 * RMS_NV * 256 && aligned(x) && aligned(w) &&
         aligned(out) && (!delta || aligned(delta))) {
+        if (width <= 4 * RMS_NV * 64 && n_rows >= 64) {   // many short rows: a wavefront each
+            dim3 wgrid((n_rows + 3) / 4);
+            if (out_dtype == CELEG_F32)
+                hipLaunchKernelGGL((rmsnorm_wave_kernel<TX, TD, float>), wgrid, dim3(256), 0, stream, x,
+                                   delta, w, static_cast<float*>(out), rows, n_rows, width, eps, write_back);
+            else
+                hipLaunchKernelGGL((rmsnorm_wave_kernel<TX, TD, bf16>), wgrid, dim3(256), 0, stream, x,
+                                   delta, w, static_cast<bf16*>(out), rows, n_rows, width, eps, write_back);
+            return CELEG_LAUNCH_RESULT();
+        }
         if (out_dtype == CELEG_F32)
             hipLaunchKernelGGL((rmsnorm_vec_kernel<TX, TD, float>), grid, dim3(256), 0, stream, x, delta,
                                w, static_cast<float*>(out), rows, width, eps, write_back);

@@ -41,7 +41,7 @@ def test_embed(ops, dtype, vocab, width, rows):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,width", [(5, 96), (3, 1000), (9, 4100), (7, 1024), (4, 4096), (3, 516), (5, 2052)])
+@pytest.mark.parametrize("rows,width", [(5, 96), (3, 1000), (9, 4100), (7, 1024), (4, 4096), (3, 516), (5, 2052), (70, 1024), (131, 260), (65, 1000)])
 def test_rmsnorm_with_delta_and_rows(ops, dtype, rows, width):
     x = randn(rows, width, seed=3)
     delta = randn(rows, width, seed=4, dtype=dtype)
@@ -57,8 +57,9 @@ def test_rmsnorm_with_delta_and_rows(ops, dtype, rows, width):
     torch.testing.assert_close(out.double().cpu(), ref, **tol(dtype))
     # listed rows only, x untouched
     x2 = x.clone()
-    idx = torch.tensor([rows - 1, 0, rows // 2], dtype=torch.int32, device=DEV)
-    out2 = torch.empty(3, width, dtype=dtype, device=DEV)
+    picked = list(range(rows - 1, -1, -1)) if rows >= 64 else [rows - 1, 0, rows // 2]
+    idx = torch.tensor(picked, dtype=torch.int32, device=DEV)
+    out2 = torch.empty(len(picked), width, dtype=dtype, device=DEV)
     ops.rmsnorm(x2, w, eps, out2, delta=delta, rows=idx)
     assert torch.equal(x2, x)
     torch.testing.assert_close(out2.double().cpu(), ref[idx.long().cpu()], **tol(dtype))
