@@ -46,6 +46,87 @@ __global__ void short_conv_fwd_kernel(
     out[static_cast<size_t>(t) * width + ch] = from_float<T>(c * conv);
 }
 
+// The same for groups of channels (16 bytes of a row per load): a thread takes VEC
+// neighbouring channels of one token.  Tokens whose taps all lie in rows of this step (all
+// but the first taps-1 of a portion) ask for every row at once; the others go the slower way
+// through the state.
+template <typename T> struct ConvVec;
+template <> struct ConvVec<float> {
+    static constexpr int n = 4;
+    typedef float raw __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ float at(const raw& r, int i) { return r[i]; }
+    static __device__ __forceinline__ void set(raw& r, int i, float v) { r[i] = v; }
+};
+template <> struct ConvVec<bf16> {
+    static constexpr int n = 8;
+    typedef __bf16 raw __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ float at(const raw& r, int i) { return static_cast<float>(r[i]); }
+    static __device__ __forceinline__ void set(raw& r, int i, float v) { r[i] = static_cast<__bf16>(v); }
+};
+#define CONV_VEC_MAX_TAPS 8
+
+template <typename T>
+__global__ void short_conv_fwd_vec_kernel(
+    const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
+    const float* __restrict__ bias, const float* __restrict__ state, size_t state_slot_stride,
+    T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_seq,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_seqlens, int width, int taps) {
+    constexpr int VEC = ConvVec<T>::n;
+    typedef typename ConvVec<T>::raw raw;
+    const int ch = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
+    if (ch >= width) return;
+    const int t = blockIdx.x;
+    const int s = token_seq[t];
+    const int start = seq_start[s];
+    const int row0 = cu_seqlens[s];
+    const int pos = positions[t];
+    float conv[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) conv[i] = bias ? bias[ch + i] : 0.f;
+    const raw cv = *reinterpret_cast<const raw*>(bcx + static_cast<size_t>(t) * ld_bcx + width + ch);
+    if (pos - (taps - 1) >= start) {        // the same for the whole workgroup
+        raw bv[CONV_VEC_MAX_TAPS], xv[CONV_VEC_MAX_TAPS];
+#pragma unroll
+        for (int tap = 0; tap < CONV_VEC_MAX_TAPS; ++tap) {
+            // rows t - (taps-1-tap); taps beyond the kernel's length repeat the token's own row
+            const int back = max(taps - 1 - tap, 0);
+            const T* row = bcx + static_cast<size_t>(t - back) * ld_bcx;
+            bv[tap] = *reinterpret_cast<const raw*>(row + ch);
+            xv[tap] = *reinterpret_cast<const raw*>(row + 2 * width + ch);
+        }
+#pragma unroll
+        for (int tap = 0; tap < CONV_VEC_MAX_TAPS; ++tap)
+            if (tap < taps) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i)
+                    conv[i] = fmaf(w[static_cast<size_t>(ch + i) * taps + tap],
+                                   ConvVec<T>::at(bv[tap], i) * ConvVec<T>::at(xv[tap], i), conv[i]);
+            }
+    } else {
+        const float* st = state + static_cast<size_t>(seq_slot[s]) * state_slot_stride;
+        for (int tap = 0; tap < taps; ++tap) {
+            const int q = pos - (taps - 1 - tap);
+            if (q < 0) continue;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) {
+                float bx;
+                if (q >= start) {
+                    const T* row = bcx + static_cast<size_t>(row0 + (q - start)) * ld_bcx;
+                    bx = to_float(row[ch + i]) * to_float(row[2 * width + ch + i]);
+                } else {
+                    bx = st[static_cast<size_t>(q - start + taps) * width + ch + i];
+                }
+                conv[i] = fmaf(w[static_cast<size_t>(ch + i) * taps + tap], bx, conv[i]);
+            }
+        }
+    }
+    raw o;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) ConvVec<T>::set(o, i, ConvVec<T>::at(cv, i) * conv[i]);
+    *reinterpret_cast<raw*>(out + static_cast<size_t>(t) * width + ch) = o;
+}
+
 template <typename T>
 __global__ void short_conv_state_kernel(
     const T* __restrict__ bcx, int ld_bcx, float* __restrict__ state, size_t state_slot_stride,
@@ -82,6 +163,31 @@ extern "C" int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const fl
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
     dim3 block(256);
     dim3 grid_fwd(n_tokens, (width + 255) / 256), grid_state(n_seqs, (width + 255) / 256);
+    const int vec = dtype == CELEG_F32 ? 4 : 8;
+    const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    if (n_tokens >= 16 && taps <= CONV_VEC_MAX_TAPS && width % vec == 0 && ld_bcx % vec == 0 &&
+        aligned(bcx) && aligned(out)) {
+        const int threads = min(256, (width / vec + 63) / 64 * 64);
+        dim3 vblock(threads), vgrid(n_tokens, (width / vec + threads - 1) / threads);
+        if (dtype == CELEG_F32) {
+            hipLaunchKernelGGL(short_conv_fwd_vec_kernel<float>, vgrid, vblock, 0, stream,
+                               static_cast<const float*>(bcx), ld_bcx, w, bias, state,
+                               state_slot_stride, static_cast<float*>(out), positions, token_seq,
+                               seq_start, seq_slot, cu_seqlens, width, taps);
+            hipLaunchKernelGGL(short_conv_state_kernel<float>, grid_state, block, 0, stream,
+                               static_cast<const float*>(bcx), ld_bcx, state, state_slot_stride,
+                               seq_start, seq_slot, cu_seqlens, width, taps);
+        } else {
+            hipLaunchKernelGGL(short_conv_fwd_vec_kernel<bf16>, vgrid, vblock, 0, stream,
+                               static_cast<const bf16*>(bcx), ld_bcx, w, bias, state,
+                               state_slot_stride, static_cast<bf16*>(out), positions, token_seq,
+                               seq_start, seq_slot, cu_seqlens, width, taps);
+            hipLaunchKernelGGL(short_conv_state_kernel<bf16>, grid_state, block, 0, stream,
+                               static_cast<const bf16*>(bcx), ld_bcx, state, state_slot_stride,
+                               seq_start, seq_slot, cu_seqlens, width, taps);
+        }
+        return CELEG_LAUNCH_RESULT();
+    }
     if (dtype == CELEG_F32) {
         hipLaunchKernelGGL(short_conv_fwd_kernel<float>, grid_fwd, block, 0, stream,
                            static_cast<const float*>(bcx), ld_bcx, w, bias, state,

@@ -153,7 +153,7 @@ def test_short_conv_whole_chunked_and_token_by_token(ops, dtype, width, taps, bi
     w = randn(width, taps, seed=13)
     b = randn(width, seed=14) if bias else None
     ref = plain.short_conv(bcx.cpu(), w.cpu(), b.cpu() if bias else None)
-    for cuts in ([T], [1] * T, [7, 2, 1, 9, 4]):
+    for cuts in ([T], [1] * T, [7, 2, 1, 9, 4], [3, 20], [20, 3], [1, 1, 21]):
         cache = make_cache(0, 0, 0, dtype, states=[(0, StateNeed("bx", (taps, width)))])
         slot_other = cache.open()     # a neighbour slot whose state must stay zero
         slot = cache.open()
