@@ -23,18 +23,22 @@ __device__ __forceinline__ size_t cache_offset(int page, int n_layers, int layer
 // split-half rotation of pairs (i, i+rot/2) by angle = float(pos)*inv_freq[i] (if a
 // frequency table is given); q goes back in place, k and v go to the cache.
 // Reference: src/backend/cpu/kernels/rope.cpp:61-111; CUDA kernels/rope.cuh:333-393.
+#define ROPE_WAVES 4
 template <typename T>
-__global__ void qk_norm_rope_store_kernel(
+__global__ __launch_bounds__(ROPE_WAVES * CELEG_WAVE) void qk_norm_rope_store_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
-    const float* __restrict__ inv_freq, int rotary_dim, const int* __restrict__ positions,
+    const float* __restrict__ inv_freq, const float* __restrict__ cos_sin, int rotary_dim,
+    const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ table, int table_stride,
     T* __restrict__ k_pool, T* __restrict__ v_pool, int n_layers, int layer, int page_tokens,
-    int q_heads, int kv_heads, int head_dim) {
-    extern __shared__ float vals[];  // head_dim floats
+    int q_heads, int kv_heads, int head_dim, int n_heads) {
+    extern __shared__ float lds[];   // head_dim floats for each wavefront
+    const int wave = threadIdx.x / CELEG_WAVE, lane = threadIdx.x % CELEG_WAVE;
+    float* vals = lds + wave * head_dim;
     const int t = blockIdx.x;
-    const int head = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int head = blockIdx.y * ROPE_WAVES + wave;     // a wavefront per head, no barrier between them
+    if (head >= n_heads) return;
     const int pos = positions[t];
     const bool is_q = head < q_heads;
     const bool is_k = !is_q && head < q_heads + kv_heads;
@@ -70,14 +74,25 @@ __global__ void qk_norm_rope_store_kernel(
         const float inv = 1.0f / sqrtf(sum / static_cast<float>(head_dim) + eps);
         for (int d = lane; d < head_dim; d += CELEG_WAVE) vals[d] = vals[d] * inv * weight[d];
     }
-    __syncthreads();
+    // the wavefront's own part of LDS: its lanes only have to see each other's writes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int half = rotary_dim / 2;
     for (int d = lane; d < head_dim; d += CELEG_WAVE) {
         float y = vals[d];
         if (inv_freq && d < rotary_dim) {
             const int i = d < half ? d : d - half;
-            const float angle = static_cast<float>(pos) * inv_freq[i];
-            const float c = cosf(angle), s = sinf(angle);
+            float c, s;
+            if (cos_sin) {       // the table of celeg_rope_table: the same values, computed once
+                const float* cs = cos_sin + (static_cast<size_t>(pos) * half + i) * 2;
+                c = cs[0];
+                s = cs[1];
+            } else {
+                const float angle = static_cast<float>(pos) * inv_freq[i];
+                c = cosf(angle);
+                s = sinf(angle);
+            }
             const float a = vals[i], b = vals[i + half];
             y = d < half ? a * c - b * s : b * c + a * s;
         }
@@ -85,29 +100,202 @@ __global__ void qk_norm_rope_store_kernel(
     }
 }
 
+// The same for head sizes 32, 64 and 128 with rotation over the whole head (or none) and
+// the table of cosines and sines: LPH = head_dim / 4 lanes share a head, a lane holds 4
+// neighbouring values, a wavefront 64 / LPH heads of one row.  The sum of squares is
+// reduced inside the LPH lanes, and the rotation's partner (the value half a head away) sits
+// in lane ^ (LPH / 2), so nothing goes through LDS.
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+    typedef float raw __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        const raw r = *reinterpret_cast<const raw*>(p);
+        v[0] = r[0]; v[1] = r[1]; v[2] = r[2]; v[3] = r[3];
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+        *reinterpret_cast<raw*>(p) = raw{v[0], v[1], v[2], v[3]};
+    }
+};
+template <> struct Quad<bf16> {
+    typedef __bf16 raw __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ void load(const bf16* p, float (&v)[4]) {
+        const raw r = *reinterpret_cast<const raw*>(p);
+        v[0] = static_cast<float>(r[0]); v[1] = static_cast<float>(r[1]);
+        v[2] = static_cast<float>(r[2]); v[3] = static_cast<float>(r[3]);
+    }
+    static __device__ __forceinline__ void store(bf16* p, const float (&v)[4]) {
+        *reinterpret_cast<raw*>(p) = raw{static_cast<__bf16>(v[0]), static_cast<__bf16>(v[1]),
+                                         static_cast<__bf16>(v[2]), static_cast<__bf16>(v[3])};
+    }
+};
+
+template <typename T, int LPH>
+__global__ __launch_bounds__(ROPE_WAVES * CELEG_WAVE) void qk_norm_rope_store_quad_kernel(
+    T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
+    const float* __restrict__ cos_sin, const int* __restrict__ positions,
+    const int* __restrict__ token_slot, const int* __restrict__ table, int table_stride,
+    T* __restrict__ k_pool, T* __restrict__ v_pool, int n_layers, int layer, int page_tokens,
+    int q_heads, int kv_heads, int n_heads) {
+    constexpr int HD = 4 * LPH, HPW = CELEG_WAVE / LPH, HALF = HD / 2;
+    const int wave = threadIdx.x / CELEG_WAVE, lane = threadIdx.x % CELEG_WAVE;
+    const int t = blockIdx.x;
+    const int head_raw = (blockIdx.y * ROPE_WAVES + wave) * HPW + lane / LPH;
+    const bool live = head_raw < n_heads;
+    const int head = live ? head_raw : n_heads - 1;          // idle lanes repeat the last head
+    const int l = lane % LPH, d0 = 4 * l;
+    const int pos = positions[t];
+    const bool is_q = head < q_heads;
+    const bool is_k = !is_q && head < q_heads + kv_heads;
+    const int kv_head = is_q ? 0 : (is_k ? head - q_heads : head - q_heads - kv_heads);
+    const T* src = is_q ? q + static_cast<size_t>(t) * ldq + static_cast<size_t>(head) * HD
+                        : (is_k ? k + static_cast<size_t>(t) * ldk + static_cast<size_t>(kv_head) * HD
+                                : v + static_cast<size_t>(t) * ldv + static_cast<size_t>(kv_head) * HD);
+    float x[4], w[4] = {1.f, 1.f, 1.f, 1.f}, cs[8];
+    Quad<T>::load(src + d0, x);
+    const float* weight = is_q ? q_weight : (is_k ? k_weight : nullptr);
+    if (weight) Quad<float>::load(weight + d0, w);
+    if (cos_sin) {
+        const float* c = cos_sin + (static_cast<size_t>(pos) * HALF + (d0 % HALF)) * 2;
+        float c0[4], c1[4];
+        Quad<float>::load(c, c0);
+        Quad<float>::load(c + 4, c1);
+        cs[0] = c0[0]; cs[1] = c0[1]; cs[2] = c0[2]; cs[3] = c0[3];
+        cs[4] = c1[0]; cs[5] = c1[1]; cs[6] = c1[2]; cs[7] = c1[3];
+    }
+    int page = 0;
+    if (!is_q) page = table[static_cast<size_t>(token_slot[t]) * table_stride + pos / page_tokens];
+    float sum = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+#pragma unroll
+    for (int off = LPH / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, CELEG_WAVE);
+    if (weight) {
+        const float inv = 1.0f / sqrtf(sum / static_cast<float>(HD) + eps);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = x[e] * inv * w[e];
+    }
+    float y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float other = __shfl_xor(x[e], LPH / 2, CELEG_WAVE);
+        // first half: a c - b s with b the partner; second half: b c + a s with a the partner
+        y[e] = (cos_sin && (is_q || is_k))
+                   ? (l < LPH / 2 ? x[e] * cs[2 * e] - other * cs[2 * e + 1]
+                                  : x[e] * cs[2 * e] + other * cs[2 * e + 1])
+                   : x[e];
+    }
+    if (!live) return;
+    if (is_q) {
+        Quad<T>::store(q + static_cast<size_t>(t) * ldq + static_cast<size_t>(head) * HD + d0, y);
+    } else if (is_k) {
+        Quad<T>::store(k_pool + cache_offset(page, n_layers, layer, kv_heads, kv_head, page_tokens,
+                                             pos % page_tokens, HD) + d0, y);
+    } else {                               // v: copy, transposed inside the page
+        T* vdst = v_pool + cache_offset(page, n_layers, layer, kv_heads, kv_head, page_tokens, 0, HD) +
+                  pos % page_tokens;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vdst[static_cast<size_t>(d0 + e) * page_tokens] = from_float<T>(x[e]);
+    }
+}
+
+template <typename T, int LPH>
+static int launch_rope_quad(T* q, int ldq, const T* k, int ldk, const T* v, int ldv,
+                            const float* q_weight, const float* k_weight, float eps,
+                            const float* cos_sin, const int* positions, const int* token_slot,
+                            const int* table, int table_stride, T* k_pool, T* v_pool, int n_layers,
+                            int layer, int page_tokens, int n_tokens, int q_heads, int kv_heads,
+                            int n_heads, hipStream_t stream) {
+    const int per_block = ROPE_WAVES * (CELEG_WAVE / LPH);
+    dim3 grid(n_tokens, (n_heads + per_block - 1) / per_block), block(ROPE_WAVES * CELEG_WAVE);
+    hipLaunchKernelGGL((qk_norm_rope_store_quad_kernel<T, LPH>), grid, block, 0, stream, q, ldq, k, ldk,
+                       v, ldv, q_weight, k_weight, eps, cos_sin, positions, token_slot, table,
+                       table_stride, k_pool, v_pool, n_layers, layer, page_tokens, q_heads, kv_heads,
+                       n_heads);
+    return CELEG_LAUNCH_RESULT();
+}
+
+template <typename T>
+static int rope_quad_dispatch(void* q, int ldq, const void* k, int ldk, const void* v, int ldv,
+                              const float* q_weight, const float* k_weight, float eps,
+                              const float* cos_sin, const int* positions, const int* token_slot,
+                              const int* table, int table_stride, void* k_pool, void* v_pool,
+                              int n_layers, int layer, int page_tokens, int n_tokens, int q_heads,
+                              int kv_heads, int head_dim, int n_heads, hipStream_t stream) {
+#define CELEG_ROPE_QUAD(LPH_)                                                                     \
+    return launch_rope_quad<T, LPH_>(static_cast<T*>(q), ldq, static_cast<const T*>(k), ldk,      \
+                                     static_cast<const T*>(v), ldv, q_weight, k_weight, eps,      \
+                                     cos_sin, positions, token_slot, table, table_stride,         \
+                                     static_cast<T*>(k_pool), static_cast<T*>(v_pool), n_layers,  \
+                                     layer, page_tokens, n_tokens, q_heads, kv_heads, n_heads, stream)
+    if (head_dim == 32) { CELEG_ROPE_QUAD(8); }
+    if (head_dim == 64) { CELEG_ROPE_QUAD(16); }
+    CELEG_ROPE_QUAD(32);
+#undef CELEG_ROPE_QUAD
+}
+
+// cos and sin of position * inv_freq[i] for positions 0 .. n_positions-1, interleaved:
+// out[(pos * half + i) * 2 + {0, 1}].  The angle is the 32-bit product of the position and
+// the frequency, as in the kernel above when it has no table.
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, int half, int n_positions,
+                                  float* __restrict__ out) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= static_cast<size_t>(n_positions) * half) return;
+    const int pos = static_cast<int>(idx / half), i = static_cast<int>(idx % half);
+    const float angle = static_cast<float>(pos) * inv_freq[i];
+    out[2 * idx] = cosf(angle);
+    out[2 * idx + 1] = sinf(angle);
+}
+
+extern "C" int celeg_rope_table(const float* inv_freq, int half, int n_positions, float* out,
+                                hipStream_t stream) {
+    if (half <= 0 || n_positions <= 0) return 0;
+    const size_t total = static_cast<size_t>(n_positions) * half;
+    hipLaunchKernelGGL(rope_table_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       stream, inv_freq, half, n_positions, out);
+    return CELEG_LAUNCH_RESULT();
+}
+
+// cos_sin: the table of celeg_rope_table covering every position of the step, or null.
 extern "C" int celeg_qk_norm_rope_store(
     void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype,
     const float* q_weight, const float* k_weight, float eps, const float* inv_freq,
-    int rotary_dim, const int* positions, const int* token_slot, const int* table,
+    const float* cos_sin, int rotary_dim, const int* positions, const int* token_slot, const int* table,
     int table_stride, void* k_pool, void* v_pool, int n_layers, int layer, int page_tokens,
     int n_tokens, int q_heads, int kv_heads, int head_dim, int store_kv, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    dim3 grid(n_tokens, q_heads + (store_kv ? 2 * kv_heads : 0)), block(CELEG_WAVE);
-    const size_t lds = static_cast<size_t>(head_dim) * sizeof(float);
+    const int n_heads = q_heads + (store_kv ? 2 * kv_heads : 0);
+    const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool whole_rotation = !inv_freq || (cos_sin && rotary_dim == head_dim);
+    if ((head_dim == 32 || head_dim == 64 || head_dim == 128) && whole_rotation && ldq % 4 == 0 &&
+        (!store_kv || (ldk % 4 == 0 && ldv % 4 == 0 && aligned(k) && aligned(v))) && aligned(q) &&
+        aligned(k_pool) && (!q_weight || aligned(q_weight)) && (!k_weight || aligned(k_weight)) &&
+        (!cos_sin || aligned(cos_sin))) {
+        const float* cs = inv_freq ? cos_sin : nullptr;
+        if (dtype == CELEG_F32)
+            return rope_quad_dispatch<float>(q, ldq, k, ldk, v, ldv, q_weight, k_weight, eps, cs,
+                                             positions, token_slot, table, table_stride, k_pool, v_pool,
+                                             n_layers, layer, page_tokens, n_tokens, q_heads, kv_heads,
+                                             head_dim, n_heads, stream);
+        return rope_quad_dispatch<bf16>(q, ldq, k, ldk, v, ldv, q_weight, k_weight, eps, cs, positions,
+                                        token_slot, table, table_stride, k_pool, v_pool, n_layers,
+                                        layer, page_tokens, n_tokens, q_heads, kv_heads, head_dim,
+                                        n_heads, stream);
+    }
+    dim3 grid(n_tokens, (n_heads + ROPE_WAVES - 1) / ROPE_WAVES), block(ROPE_WAVES * CELEG_WAVE);
+    const size_t lds = static_cast<size_t>(ROPE_WAVES) * head_dim * sizeof(float);
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(qk_norm_rope_store_kernel<float>, grid, block, lds, stream,
                            static_cast<float*>(q), ldq, static_cast<const float*>(k), ldk,
                            static_cast<const float*>(v), ldv, q_weight, k_weight, eps, inv_freq,
-                           rotary_dim, positions, token_slot, table, table_stride,
+                           cos_sin, rotary_dim, positions, token_slot, table, table_stride,
                            static_cast<float*>(k_pool), static_cast<float*>(v_pool), n_layers,
-                           layer, page_tokens, q_heads, kv_heads, head_dim);
+                           layer, page_tokens, q_heads, kv_heads, head_dim, n_heads);
     else
         hipLaunchKernelGGL(qk_norm_rope_store_kernel<bf16>, grid, block, lds, stream,
                            static_cast<bf16*>(q), ldq, static_cast<const bf16*>(k), ldk,
                            static_cast<const bf16*>(v), ldv, q_weight, k_weight, eps, inv_freq,
-                           rotary_dim, positions, token_slot, table, table_stride,
+                           cos_sin, rotary_dim, positions, token_slot, table, table_stride,
                            static_cast<bf16*>(k_pool), static_cast<bf16*>(v_pool), n_layers,
-                           layer, page_tokens, q_heads, kv_heads, head_dim);
+                           layer, page_tokens, q_heads, kv_heads, head_dim, n_heads);
     return CELEG_LAUNCH_RESULT();
 }
 

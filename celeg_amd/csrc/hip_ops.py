@@ -46,6 +46,8 @@ class HipOps:
         self.attention_impl = "auto"
         self._decode_ws = None
         self._retired = []
+        self._rope_tables = {}
+        self.use_rope_table = True         # cos/sin of every position from a table made once
         self.use_sliced = True             # up to 16 bfloat16 rows: the k-sliced kernels
         self.last_stat_blocks = 0
         self.fused_linear_shape = 0        # 0: chosen from the sizes; 1..4 force a workgroup shape
@@ -249,6 +251,22 @@ class HipOps:
         if not 0 <= kv.layer < kv.n_layers:
             raise KernelError("attention: layer index outside the cache")
 
+    def _rope_table(self, inv_freq, n_positions: int) -> torch.Tensor:
+        """cos and sin of position * frequency for every position a request can reach
+        ([n_positions, rotary_dim/2, 2], 32-bit), made once per frequency table."""
+        key = (inv_freq.data_ptr(), n_positions)
+        table = self._rope_tables.get(key)
+        if table is None:
+            table = torch.empty((n_positions, inv_freq.numel(), 2), dtype=torch.float32,
+                                device=inv_freq.device)
+            code = self._lib("attention").celeg_rope_table(
+                _ptr(inv_freq), _c_int(inv_freq.numel()), _c_int(n_positions), _ptr(table),
+                self._stream())
+            self._check(code, "rope_table")
+            self._rope_tables[key] = (table, inv_freq)   # the key's tensor is kept alive with it
+            return table
+        return table[0]
+
     def qk_norm_rope_store(self, q, k, v, q_weight, k_weight, eps, inv_freq, rotary_dim,
                            heads, kv_heads, head_dim, batch, kv):
         self._dev(q, "q", contiguous=False)
@@ -273,11 +291,14 @@ class HipOps:
             self._dev(inv_freq, "inv_freq", torch.float32)
             if rotary_dim % 2 or rotary_dim > head_dim or inv_freq.numel() != rotary_dim // 2:
                 raise KernelError("qk_norm_rope_store: rotary_dim and the frequency table disagree")
+        cos_sin = None
+        if inv_freq is not None and rotary_dim > 0 and self.use_rope_table:
+            cos_sin = self._rope_table(inv_freq, kv.table.shape[1] * kv.page_tokens)
         code = self._lib("attention").celeg_qk_norm_rope_store(
             _ptr(q), _c_int(self._rows(q, "q")), _ptr(k), _c_int(self._rows(k, "k") if store else 0),
             _ptr(v), _c_int(self._rows(v, "v") if store else 0), _c_int(self._dtype(q, "q")),
             _ptr(q_weight), _ptr(k_weight if store else None), _c_float(eps), _ptr(inv_freq),
-            _c_int(rotary_dim), _ptr(batch.positions), _ptr(batch.token_slot), _ptr(kv.table),
+            _ptr(cos_sin), _c_int(rotary_dim), _ptr(batch.positions), _ptr(batch.token_slot), _ptr(kv.table),
             _c_int(kv.table.shape[1]), _ptr(kv.k), _ptr(kv.v), _c_int(kv.n_layers),
             _c_int(kv.layer), _c_int(kv.page_tokens), _c_int(T), _c_int(heads), _c_int(kv_heads),
             _c_int(head_dim), _c_int(1 if store else 0), self._stream())
