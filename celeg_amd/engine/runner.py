@@ -67,6 +67,8 @@ class ModelRunner:
         self.steps_run = 0
         self.use_graphs = True
         self._graphs: Dict[int, tuple] = {}
+        self._portion_graphs: Dict[tuple, tuple] = {}
+        self._portion_seen: Dict[tuple, int] = {}
         self._buckets = sorted({min(1 << i, S) for i in range(0, 12)})
         self.last_batch: Optional[StepBatch] = None
 
@@ -113,6 +115,9 @@ class ModelRunner:
         self._validate(entries)
         if self._graph_applies(entries):
             return self._step_from_graph(entries)
+        portion = self._portion_shape(entries)
+        if portion is not None:
+            return self._portion_from_graph(entries, portion)
         updates = self.cache.drain_table_updates()
         batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
         self._apply_table_updates(batch)
@@ -157,8 +162,62 @@ class ModelRunner:
 
     def _capture(self, bucket: int, caps):
         empty = [[] for _ in self.cache.groups]
-        batch = self.builder.build([], empty, pad_to=bucket, null_slot=self.cache.null_slot,
-                                   update_caps=caps)
+        captured = self._capture_batch(lambda: self.builder.build(
+            [], empty, pad_to=bucket, null_slot=self.cache.null_slot, update_caps=caps))
+        self._graphs[bucket] = captured
+        return captured
+
+    # ------------------------------------------------------------------ captured portions
+    # A step that is one portion of one prompt launches some 150 kernels and is bound by
+    # the host's launches at this model size.  Portions of a size that has come before (the
+    # token budget makes long prompts arrive in equal portions) are replayed from a graph
+    # captured for that size, on the null slot like the decode graphs.
+    PORTION_GRAPHS = 8          # sizes kept
+    PORTION_MIN_TOKENS = 32
+
+    def _portion_shape(self, entries: Sequence[StepEntry]):
+        if not self.use_graphs or torch.device(self.rt.device).type != "cuda" \
+                or not self.model.graph_safe or len(entries) != 1:
+            return None
+        e = entries[0]
+        n = len(e.tokens)
+        if n < self.PORTION_MIN_TOKENS:
+            return None
+        want = list(e.want)
+        if want not in ([], [n - 1]):
+            return None
+        shape = (n, len(want))
+        if shape not in self._portion_graphs:
+            seen = self._portion_seen.get(shape, 0) + 1
+            self._portion_seen[shape] = seen
+            if seen < 2 or len(self._portion_graphs) >= self.PORTION_GRAPHS:
+                return None
+        return shape
+
+    def _portion_from_graph(self, entries: Sequence[StepEntry], shape) -> torch.Tensor:
+        n, n_want = shape
+        caps = [n // self.cache.page_tokens + 10] * len(self.cache.groups)
+        captured = self._portion_graphs.get(shape)
+        if captured is None or captured[2] != self.rt.ws.generation:
+            null = [StepEntry(self.cache.null_slot, 0, [0] * n, [n - 1] if n_want else [])]
+            captured = self._capture_batch(lambda: self.builder.build(
+                null, [[] for _ in self.cache.groups], null_slot=self.cache.null_slot, update_caps=caps))
+            self._portion_graphs[shape] = captured
+        updates = self.cache.drain_table_updates()
+        for g, u in enumerate(updates):
+            if len(u) > caps[g]:
+                self._ship_table_updates(g, u)
+                updates[g] = []
+        batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot, update_caps=caps)
+        self.last_batch = batch
+        captured[0].replay()
+        self.steps_run += 1
+        return captured[1]
+
+    def _capture_batch(self, make_batch):
+        """Warm-up run and capture of the model's forward over the batch ``make_batch()``
+        builds (of null-slot rows only): (graph, logits, workspace generation)."""
+        batch = make_batch()
         self._apply_table_updates(batch)
         self.model.forward(batch, self.rt)          # warm-up: buffers, libraries, heuristics
         torch.cuda.synchronize(self.rt.device)
@@ -170,9 +229,7 @@ class ModelRunner:
                 logits = self.model.forward(batch, self.rt)
         finally:
             self.rt.ws.frozen = False
-        captured = (graph, logits, self.rt.ws.generation)
-        self._graphs[bucket] = captured
-        return captured
+        return (graph, logits, self.rt.ws.generation)
 
     def _ship_table_updates(self, group: int, updates) -> None:
         flat = torch.tensor([len(updates)] + [v for u in updates for v in u], dtype=torch.int32)

@@ -163,3 +163,35 @@ def test_first_tokens_of_a_sequence(model_folders, name, dtype):
         assert len(got[rid]) == 7
         assert_close(got[rid], plain.model_logits(cfgp, W, toks), dtype, f"{name}/{dtype}/first/{rid}")
     lm.cache.check()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_portions_of_a_repeated_size_are_replayed(model_folders, name, dtype):
+    """Prompts that arrive in equal portions: from the second portion of a size on, the
+    step is replayed from a graph captured for that size (on the null slot).  Every replay
+    is checked against the plain implementation, with other steps (decode tokens, another
+    size) between them."""
+    from celeg_amd.engine import load_model
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders(name, storage, WEIGHT_STD)
+    vocab = TINY[name][0]["vocab_size"]
+    reqs = {f"eq{i}": random_tokens(vocab, 48 * 3 + 2, seed=970 + i) for i in range(4)}
+    steps = []
+    for rid, toks in reqs.items():
+        for p in range(3):      # 48, 48 (no logits), then 48 with the last row's logits
+            steps.append({"step": len(steps), "entries": [
+                {"id": rid, "tokens": toks[48 * p:48 * p + 48], "want": [47] if p == 2 else []}], "end": []})
+        for p in (144, 145):    # two decode tokens
+            steps.append({"step": len(steps), "entries": [
+                {"id": rid, "tokens": [toks[p]], "want": [0]}], "end": [rid] if p == 145 else []})
+    lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16 + 1,
+                    max_requests=4, max_batched_tokens=64)
+    got = EngineDriver(lm).run(steps)
+    assert set(lm.runner._portion_graphs) == {(48, 0), (48, 1)}
+    cfgp, W = plain.load_model_folder(folder)
+    for rid, toks in reqs.items():
+        ref = plain.model_logits(cfgp, W, toks)
+        assert_close(got[rid], ref[[143, 144, 145]], dtype, f"{name}/{dtype}/replayed/{rid}")
+    lm.cache.check()
