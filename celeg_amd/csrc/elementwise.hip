@@ -372,3 +372,22 @@ extern "C" int celeg_table_update(int* table, int stride, int n_slots, const int
                        updates, capacity);
     return CELEG_LAUNCH_RESULT();
 }
+
+// ---------------------------------------------------------------- tokens from the device
+// A row whose token id is negative takes the token its request sampled last:
+// token_ids[i] = last_tokens[token_slot[i]].  Lets the host launch a decode step before it
+// has read the previous step's tokens.
+__global__ void resolve_tokens_kernel(int* __restrict__ token_ids, const int* __restrict__ token_slot,
+                                      const int* __restrict__ last_tokens, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    if (token_ids[i] < 0) token_ids[i] = last_tokens[token_slot[i]];
+}
+
+extern "C" int celeg_resolve_tokens(int* token_ids, const int* token_slot, const int* last_tokens,
+                                    int n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    hipLaunchKernelGGL(resolve_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, token_ids,
+                       token_slot, last_tokens, n);
+    return CELEG_LAUNCH_RESULT();
+}

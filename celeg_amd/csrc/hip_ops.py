@@ -361,13 +361,25 @@ class HipOps:
         self._check(code, "attention for decode rows (bfloat16)")
 
     # ------------------------------------------------------------------ sampling
-    def sample(self, logits, fparams, iparams, seen, out_tokens):
+    def resolve_tokens(self, token_ids, token_slot, last_tokens, n):
+        """token_ids[i] = last_tokens[token_slot[i]] where token_ids[i] < 0 (i < n)."""
+        for t, name in ((token_ids, "token_ids"), (token_slot, "token_slot"), (last_tokens, "last_tokens")):
+            self._dev(t, name, torch.int32)
+        if token_ids.numel() < n or token_slot.numel() < n:
+            raise KernelError("resolve_tokens: fewer rows than n")
+        code = self._lib("elementwise").celeg_resolve_tokens(
+            _ptr(token_ids), _ptr(token_slot), _ptr(last_tokens), _c_int(n), self._stream())
+        self._check(code, "resolve_tokens")
+
+    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None):
         self._dev(logits, "logits", torch.float32, contiguous=False)
         self._dev(fparams, "fparams", torch.float32); self._dev(iparams, "iparams", torch.int32)
         self._dev(out_tokens, "out_tokens", torch.int32)
         R, V = logits.shape
-        if out_tokens.numel() != R or fparams.numel() < 4 * R or iparams.numel() < 2 * R:
+        if out_tokens.numel() != R or fparams.numel() < 4 * R or iparams.numel() < 3 * R:
             raise KernelError("sample: parameter arrays do not fit the rows")
+        if last_tokens is not None:
+            self._dev(last_tokens, "last_tokens", torch.int32)
         if seen is not None:
             self._dev(seen, "seen", torch.uint8)
             if seen.shape[1] != V:
@@ -375,7 +387,8 @@ class HipOps:
         code = self._lib("sampling").celeg_sample(
             _ptr(logits), _c_int(self._rows(logits, "logits")), _c_int(R), _c_int(V),
             _ptr(fparams), _ptr(iparams), _ptr(seen),
-            _c_size_t(seen.stride(0) if seen is not None else 0), _ptr(out_tokens), self._stream())
+            _c_size_t(seen.stride(0) if seen is not None else 0), _ptr(out_tokens),
+            _ptr(last_tokens), self._stream())
         self._check(code, "sample")
 
     def mark_seen(self, seen, token_ids, token_slot, n):

@@ -31,11 +31,13 @@ __device__ __forceinline__ bool better(float sa, int ia, float sb, int ib) {
     return sa == sb ? ia < ib : sa > sb;
 }
 
-// fparams[row] = {temperature, top_p, penalty, u}; iparams[row] = {top_k, seen_row or -1}
+// fparams[row] = {temperature, top_p, penalty, u}; iparams[row] = {top_k, seen_row or -1,
+// slot or -1}; the token also goes to last_tokens[slot] (if given and slot >= 0), where the
+// next step can take it from without the host in between.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ fparams,
     const int* __restrict__ iparams, const uint8_t* __restrict__ seen_all, size_t seen_stride,
-    int* __restrict__ out_tokens) {
+    int* __restrict__ out_tokens, int* __restrict__ last_tokens) {
     __shared__ float s_val[SAMPLE_THREADS / CELEG_WAVE];
     __shared__ int s_idx[SAMPLE_THREADS / CELEG_WAVE];
     __shared__ unsigned int hist[256];
@@ -52,8 +54,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* row = logits + static_cast<size_t>(r) * ld;
     const float temperature = fparams[4 * r + 0], top_p = fparams[4 * r + 1];
     const float penalty = fparams[4 * r + 2], u = fparams[4 * r + 3];
-    int top_k = iparams[2 * r + 0];
-    const int seen_row = iparams[2 * r + 1];
+    int top_k = iparams[3 * r + 0];
+    const int seen_row = iparams[3 * r + 1];
+    const int slot = iparams[3 * r + 2];
     const uint8_t* seen = (seen_all && seen_row >= 0)
                               ? seen_all + static_cast<size_t>(seen_row) * seen_stride : nullptr;
 
@@ -108,6 +111,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                     best = s_val[w]; best_i = s_idx[w];
                 }
             out_tokens[r] = best_i;
+            if (last_tokens && slot >= 0) last_tokens[slot] = best_i;
         }
         return;
     }
@@ -228,16 +232,18 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
             if (target <= 0.0f) { chosen = cand_id[i]; break; }
         }
         out_tokens[r] = chosen;
+        if (last_tokens && slot >= 0) last_tokens[slot] = chosen;
     }
 }
 
 extern "C" int celeg_sample(const float* logits, int ld, int rows, int vocab,
                             const float* fparams, const int* iparams, const uint8_t* seen,
-                            size_t seen_stride, int* out_tokens, hipStream_t stream) {
+                            size_t seen_stride, int* out_tokens, int* last_tokens,
+                            hipStream_t stream) {
     if (rows <= 0) return 0;
     if (vocab <= 0) return static_cast<int>(hipErrorInvalidValue);
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld,
-                       vocab, fparams, iparams, seen, seen_stride, out_tokens);
+                       vocab, fparams, iparams, seen, seen_stride, out_tokens, last_tokens);
     return CELEG_LAUNCH_RESULT();
 }
 

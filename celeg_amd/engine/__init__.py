@@ -1,4 +1,4 @@
-from .batch import StepEntry, StepBatch
+from .batch import TOKEN_FROM_DEVICE, StepEntry, StepBatch
 from .model import Model
 from .runner import ModelRunner, Workspace
 from .loading import load_model, LoadedModel, make_runtime, parse_dtype
@@ -6,6 +6,6 @@ from .scheduler import (Scheduler, SchedulerOptions, RequestOptions, RequestStat
                         PlannedEntry)
 from .engine import Engine
 
-__all__ = ["StepEntry", "StepBatch", "Model", "ModelRunner", "Workspace", "load_model",
+__all__ = ["TOKEN_FROM_DEVICE", "StepEntry", "StepBatch", "Model", "ModelRunner", "Workspace", "load_model",
            "LoadedModel", "make_runtime", "parse_dtype", "Scheduler", "SchedulerOptions",
            "RequestOptions", "RequestStatus", "Request", "PlannedEntry", "Engine"]

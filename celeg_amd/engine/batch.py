@@ -18,11 +18,14 @@ import numpy as np
 import torch
 
 
+TOKEN_FROM_DEVICE = -1        # a single-token entry whose token the device supplies
+
+
 @dataclass
 class StepEntry:
     slot: int                 # the request's slot in the cache manager
     start_pos: int            # position of tokens[0] in the request's sequence
-    tokens: Sequence[int]
+    tokens: Sequence[int]     # [TOKEN_FROM_DEVICE]: the token the request sampled last, taken on the device
     want: Sequence[int] = ()  # indices into ``tokens`` whose logits are wanted
 
 
@@ -84,6 +87,7 @@ class BatchBuilder:
             if self.device.type == "cuda" else [None, None]
         self._iota = np.arange(max(capacity_ints, 1 << 16), dtype=np.int32)
         self._turn = 0
+        self._layouts = {}      # (rows, requests, logit rows, update room) -> layout, size, device views
         self.device_buffer = torch.zeros(capacity_ints, dtype=torch.int32, device=self.device)
 
     def build(self, entries: Sequence[StepEntry], updates: Sequence[Sequence[Tuple[int, int, int]]],
@@ -117,7 +121,13 @@ class BatchBuilder:
         for u, cap in zip(updates, update_caps):
             if len(u) > cap:
                 raise ValueError("more block-table updates than the step has room for")
-        layout, total = packed_layout(T, S, R, update_caps)
+        key = (T, S, R, tuple(update_caps))
+        cached = self._layouts.get(key)
+        if cached is None:
+            if len(self._layouts) > 256:
+                self._layouts.clear()
+            cached = self._layouts[key] = packed_layout(T, S, R, update_caps) + ({},)
+        layout, total, views = cached
         if total > self.capacity:
             raise ValueError(f"step metadata ({total} ints) exceeds the staging buffer "
                              f"({self.capacity} ints)")
@@ -177,9 +187,12 @@ class BatchBuilder:
         b.max_context_len = max((e.start_pos + n for e, n in zip(entries, seg_lens)), default=0)
         b.decode_only = decode_only
 
-        def dev(name):
-            off, count = layout[name]
-            return self.device_buffer[off:off + count]
+        def dev(name):       # the same views of the device buffer for the same layout
+            view = views.get(name)
+            if view is None:
+                off, count = layout[name]
+                view = views[name] = self.device_buffer[off:off + count]
+            return view
 
         b.token_ids, b.positions = dev("token_ids"), dev("positions")
         b.token_seq, b.token_slot = dev("token_seq"), dev("token_slot")

@@ -14,7 +14,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..sampling.sampler import GREEDY, Sampler
-from .batch import StepEntry
+from .batch import TOKEN_FROM_DEVICE, StepEntry
 from .loading import LoadedModel
 
 
@@ -62,6 +62,7 @@ class DecodeBench:
         self.slots: List[int] = []
         self.pos: List[int] = []
         self.next_tokens: List[int] = []
+        self.generated: List[List[int]] = []      # the tokens of every step, per request
         vocab = lm.spec.vocab_size
         for b in range(batch):
             slot = lm.cache.open()
@@ -84,6 +85,7 @@ class DecodeBench:
             self.next_tokens.append(self.sampler.sample(logits, [slot])[0])
 
     def step(self) -> None:
+        """One decode step, the host waiting for its tokens before it goes on."""
         lm = self.lm
         entries = []
         for b, slot in enumerate(self.slots):
@@ -92,16 +94,51 @@ class DecodeBench:
             entries.append(StepEntry(slot, self.pos[b], [self.next_tokens[b]], [0]))
         logits = lm.runner.step(entries)
         self.next_tokens = self.sampler.sample(logits, self.slots)
+        self.generated.append(self.next_tokens)
         for b in range(self.batch):
             self.pos[b] += 1
 
-    def run(self, steps: int, warmup: int) -> Dict[str, float]:
-        for _ in range(warmup):
-            self.step()
+    def steps_pipelined(self, steps: int) -> None:
+        """``steps`` decode steps with the host one step ahead of the device: a step takes
+        its input tokens on the device from what the previous step sampled
+        (``TOKEN_FROM_DEVICE``), so it is launched before those tokens have reached the host;
+        the host reads a step's tokens while the next step runs."""
+        lm = self.lm
+        lm.runner.token_source = self.sampler.last_tokens
+        open_fetches = 0
+        for k in range(steps):
+            entries = []
+            for b, slot in enumerate(self.slots):
+                if not lm.cache.prepare(slot, self.pos[b], 1):
+                    raise RuntimeError("decode benchmark: out of cache pages")
+                token = self.next_tokens[b] if k == 0 else TOKEN_FROM_DEVICE
+                entries.append(StepEntry(slot, self.pos[b], [token], [0]))
+            logits = lm.runner.step(entries)
+            self.sampler.launch(logits, self.slots)
+            open_fetches += 1
+            for b in range(self.batch):
+                self.pos[b] += 1
+            if open_fetches == 2:           # the tokens of the step before this one
+                self.generated.append(self.sampler.fetch())
+                open_fetches -= 1
+        while open_fetches:
+            self.generated.append(self.sampler.fetch())
+            open_fetches -= 1
+        self.next_tokens = self.generated[-1]
+
+    def run(self, steps: int, warmup: int, pipelined: bool = True) -> Dict[str, float]:
+        if pipelined:
+            self.steps_pipelined(warmup)
+        else:
+            for _ in range(warmup):
+                self.step()
         _sync(self.lm.rt.device)
         start = time.perf_counter()
-        for _ in range(steps):
-            self.step()
+        if pipelined:
+            self.steps_pipelined(steps)
+        else:
+            for _ in range(steps):
+                self.step()
         _sync(self.lm.rt.device)
         elapsed = time.perf_counter() - start
         return {"steps": steps, "batch": self.batch, "ms_per_step": elapsed / steps * 1e3,

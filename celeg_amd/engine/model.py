@@ -63,7 +63,10 @@ class Model:
     @property
     def graph_safe(self) -> bool:
         """Whether a recorded step of this model may be replayed from a HIP graph."""
-        return all(part.graph_safe for _, part in self.named_parts())
+        safe = self.__dict__.get("_graph_safe")
+        if safe is None:      # the parts are fixed once the model is built
+            safe = self.__dict__["_graph_safe"] = all(part.graph_safe for _, part in self.named_parts())
+        return safe
 
     def named_parts(self) -> List[Tuple[str, Part]]:
         out = [("embedding", self.embedding)]

@@ -16,7 +16,7 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..parts.base import Runtime
-from .batch import BatchBuilder, StepBatch, StepEntry, packed_layout
+from .batch import TOKEN_FROM_DEVICE, BatchBuilder, StepBatch, StepEntry, packed_layout
 from .model import Model
 
 
@@ -69,6 +69,7 @@ class ModelRunner:
         self._graphs: Dict[int, tuple] = {}
         self._portion_graphs: Dict[tuple, tuple] = {}
         self._portion_seen: Dict[tuple, int] = {}
+        self._token_source: Optional[torch.Tensor] = None
         self._buckets = sorted({min(1 << i, S) for i in range(0, 12)})
         self.last_batch: Optional[StepBatch] = None
 
@@ -93,7 +94,8 @@ class ModelRunner:
                 raise ValueError(f"context limit reached: position {e.start_pos + n} exceeds "
                                  f"{self.cache.max_context}")
             if n == 1:
-                in_range = 0 <= e.tokens[0] < vocab
+                in_range = 0 <= e.tokens[0] < vocab or \
+                    (e.tokens[0] == TOKEN_FROM_DEVICE and self._token_source is not None)
             else:
                 toks = np.asarray(e.tokens)
                 in_range = toks.min() >= 0 and toks.max() < vocab
@@ -121,6 +123,7 @@ class ModelRunner:
         updates = self.cache.drain_table_updates()
         batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
         self._apply_table_updates(batch)
+        self._resolve_tokens(batch)
         self.last_batch = batch
         logits = self.model.forward(batch, self.rt)
         self.steps_run += 1
@@ -219,6 +222,7 @@ class ModelRunner:
         builds (of null-slot rows only): (graph, logits, workspace generation)."""
         batch = make_batch()
         self._apply_table_updates(batch)
+        self._resolve_tokens(batch)
         self.model.forward(batch, self.rt)          # warm-up: buffers, libraries, heuristics
         torch.cuda.synchronize(self.rt.device)
         graph = torch.cuda.CUDAGraph()
@@ -226,10 +230,33 @@ class ModelRunner:
         try:
             with torch.cuda.graph(graph):
                 self._apply_table_updates(batch)
+                self._resolve_tokens(batch)
                 logits = self.model.forward(batch, self.rt)
         finally:
             self.rt.ws.frozen = False
         return (graph, logits, self.rt.ws.generation)
+
+    # ------------------------------------------------------------------ tokens from the device
+    @property
+    def token_source(self) -> Optional[torch.Tensor]:
+        """int32 [slots]: the token every slot sampled last, on the device.  With it set, an
+        entry may bring ``[TOKEN_FROM_DEVICE]`` instead of a token, and the step can be
+        launched before the host has read the previous step's tokens."""
+        return self._token_source
+
+    @token_source.setter
+    def token_source(self, tensor: Optional[torch.Tensor]) -> None:
+        if tensor is not None and (tensor.dtype != torch.int32 or tensor.numel() <= self.cache.null_slot):
+            raise ValueError("token_source must be int32 with an entry for every slot and the null slot")
+        if tensor is not self._token_source:
+            self._graphs.clear()            # recorded steps do or do not hold the lookup
+            self._portion_graphs.clear()
+        self._token_source = tensor
+
+    def _resolve_tokens(self, batch: StepBatch) -> None:
+        if self._token_source is not None:
+            self.rt.ops.resolve_tokens(batch.token_ids, batch.token_slot, self._token_source,
+                                       batch.n_tokens)
 
     def _ship_table_updates(self, group: int, updates) -> None:
         flat = torch.tensor([len(updates)] + [v for u in updates for v in u], dtype=torch.int32)

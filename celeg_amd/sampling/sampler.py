@@ -83,14 +83,23 @@ class Sampler:
         cap = max_requests
         pin = torch.device(device).type == "cuda"
         # one staging buffer and one device buffer for a step's parameters: 4 floats a row,
-        # then 2 ints a row (the same bytes seen as 32-bit floats and as 32-bit ints)
-        self._params = torch.zeros(cap * 6, dtype=torch.float32, pin_memory=pin)
-        self._params_dev = torch.zeros(cap * 6, dtype=torch.float32, device=device)
-        self._fparams, self._iparams = self._params[:cap * 4], self._params[cap * 4:].view(torch.int32)
+        # then 3 ints a row (the same bytes seen as 32-bit floats and as 32-bit ints)
+        # (two staging buffers take turns, like the buffers the tokens come back through)
+        self._params = [torch.zeros(cap * 7, dtype=torch.float32, pin_memory=pin) for _ in range(2)]
+        self._params_dev = torch.zeros(cap * 7, dtype=torch.float32, device=device)
         self._fparams_dev = self._params_dev[:cap * 4]
         self._iparams_dev = self._params_dev[cap * 4:].view(torch.int32)
         self._uploaded = None      # what the device buffer holds: a copy of the staged values
         self._tokens_dev = torch.empty(cap, dtype=torch.int32, device=device)
+        # the token every slot sampled last, on the device: a following step can take its
+        # input from here (``ModelRunner.token_source``) before the host has read it
+        self.last_tokens = torch.zeros(cap + 1, dtype=torch.int32, device=device)
+        # sampled tokens come back through two pinned buffers that take turns, so that one
+        # step's tokens can still be on their way while the next step is launched
+        self._tokens_host = [torch.zeros(cap, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self._events = [torch.cuda.Event() if pin else None for _ in range(2)]
+        self._pending = []         # launched and not fetched yet: (turn, rows)
+        self._turn = 0
 
     def begin(self, slot: int, config: GenerationConfig, rng: Optional[XorShift64Star] = None) -> None:
         """Bind a request to ``slot``.  ``rng`` continues an existing generator (a request
@@ -120,26 +129,54 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, slots: Sequence[int]) -> List[int]:
         """One token per row of ``logits``; row i belongs to the request in ``slots[i]``."""
-        R = len(slots)
-        if R == 0:
+        if len(slots) == 0:
             return []
+        self.launch(logits, slots)
+        return self.fetch()
+
+    def launch(self, logits: torch.Tensor, slots: Sequence[int]) -> None:
+        """Starts the sampling of one token per row without waiting for it; ``fetch``
+        returns the tokens of the oldest launch not fetched yet (at most two may be open)."""
+        R = len(slots)
         if logits.shape[0] != R or logits.shape[1] != self.vocab:
             raise ValueError("sample: one row of logits per slot is needed")
         if R > self.max_requests:
             raise ValueError("sample: more rows than requests")
-        f, i = self._fparams.numpy(), self._iparams.numpy()
+        if len(self._pending) >= 2:
+            raise RuntimeError("sample: two launches are open; fetch one first")
+        turn = self._turn          # its previous launch has been fetched: its buffers are free
+        self._turn ^= 1
+        cap = self.max_requests
+        staged = self._params[turn].numpy()
+        f, i = staged[:cap * 4], staged[cap * 4:].view(np.int32)
         for r, slot in enumerate(slots):
             c = self._configs[slot]
             f[4 * r: 4 * r + 4] = (c.temperature, c.top_p, c.repetition_penalty,
                                    0.0 if c.greedy else self._rng[slot].next_unit())
-            i[2 * r] = c.top_k
-            i[2 * r + 1] = slot if (c.repetition_penalty > 1.0 and self._seen is not None) else -1
+            i[3 * r] = c.top_k
+            i[3 * r + 1] = slot if (c.repetition_penalty > 1.0 and self._seen is not None) else -1
+            i[3 * r + 2] = slot
         # greedy rows have nothing that changes from step to step: ship only what differs
         # from what the device holds
-        staged = self._params.numpy()
-        if self._uploaded is None or not np.array_equal(staged.view(np.int32), self._uploaded):
-            self._params_dev.copy_(self._params, non_blocking=True)
-            self._uploaded = staged.view(np.int32).copy()
+        used = np.concatenate([f[:4 * R].view(np.int32), i[:3 * R]])
+        if self._uploaded is None or not np.array_equal(used, self._uploaded):
+            self._params_dev.copy_(self._params[turn], non_blocking=True)
+            self._uploaded = used
         self.ops.sample(logits, self._fparams_dev, self._iparams_dev, self._seen,
-                        self._tokens_dev[:R])
-        return self._tokens_dev[:R].tolist()   # the step's one synchronisation
+                        self._tokens_dev[:R], last_tokens=self.last_tokens)
+        self._tokens_host[turn][:R].copy_(self._tokens_dev[:R], non_blocking=True)
+        if self._events[turn] is not None:
+            self._events[turn].record()
+        self._pending.append((turn, R))
+
+    def _sync(self, turn: int) -> None:
+        if self._events[turn] is not None:
+            self._events[turn].synchronize()
+
+    def fetch(self) -> List[int]:
+        """The tokens of the oldest open launch (waits for them)."""
+        if not self._pending:
+            return []
+        turn, R = self._pending.pop(0)
+        self._sync(turn)
+        return self._tokens_host[turn][:R].tolist()

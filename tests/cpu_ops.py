@@ -134,15 +134,17 @@ class CpuOps:
                 pr = torch.softmax(s, dim=0)
                 out[t, h * head_dim:(h + 1) * head_dim] = (pr @ vals[:, g]).to(out.dtype)
 
-    def sample(self, logits, fparams, iparams, seen, out_tokens):
+    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None):
         import plain_lfm2 as plain   # the double may lean on the plain sampler
         R, V = logits.shape
         for r in range(R):
             t, top_p, pen, u = (float(x) for x in fparams[4 * r: 4 * r + 4])
-            k, row = int(iparams[2 * r]), int(iparams[2 * r + 1])
+            k, row, slot = (int(x) for x in iparams[3 * r: 3 * r + 3])
             s = seen[row].bool().tolist() if (seen is not None and row >= 0) else [False] * V
             # the draw comes from the host: walk with it instead of a generator state
             out_tokens[r] = _sample_with_draw(plain, logits[r].tolist(), t, k, top_p, pen, s, u)
+            if last_tokens is not None and slot >= 0:
+                last_tokens[slot] = out_tokens[r]
 
     def mark_seen(self, seen, token_ids, token_slot, n):
         for t, s in zip(token_ids[:n].tolist(), token_slot[:n].tolist()):

@@ -137,7 +137,7 @@ def run_sample(ops, logits, rows):
     for r, (t, k, p, pen, u, s) in enumerate(rows):
         if s is not None:
             seen[r, torch.tensor(s, dtype=torch.long)] = 1
-        i.append([k, r if s is not None else -1])
+        i.append([k, r if s is not None else -1, -1])
     out = torch.empty(R, dtype=torch.int32, device=DEV)
     ops.sample(logits.to(DEV), f.reshape(-1).to(DEV), torch.tensor(i, dtype=torch.int32).reshape(-1).to(DEV),
                seen.to(DEV), out)
@@ -205,3 +205,25 @@ def test_mark_seen(ops):
     slots = torch.tensor([0, 2, 2, 3], dtype=torch.int32, device=DEV)   # slot 3 is outside: ignored
     ops.mark_seen(seen, toks, slots, 4)
     assert seen.sum().item() == 3 and seen[0, 5] == 1 and seen[2, 99] == 1 and seen[2, 5] == 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_launched_ahead_of_their_tokens_give_the_same_tokens(model_folders, dtype):
+    """Decode steps that take their input token on the device from what the previous step
+    sampled, launched before the host has read it, against steps the host feeds one by one."""
+    import torch
+    from celeg_amd.engine import load_model
+    from celeg_amd.engine.benchmark import DecodeBench
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders("B", storage, 0.05)
+    runs = {}
+    for pipelined in (False, True):
+        lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=64, max_requests=4,
+                        max_batched_tokens=64)
+        bench = DecodeBench(lm, 3, 20, seed=5, prefill_chunk=16)
+        bench.run(steps=40, warmup=7, pipelined=pipelined)
+        runs[pipelined] = bench.generated
+        assert len(bench.generated) == 47 and all(len(t) == 3 for t in bench.generated)
+        bench.close()
+        lm.cache.check()
+    assert runs[True] == runs[False]
