@@ -14,7 +14,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 from ..sampling.sampler import GenerationConfig, Sampler, XorShift64Star
-from .batch import StepEntry
+from .batch import TOKEN_FROM_DEVICE, StepEntry
 from .loading import LoadedModel, load_model
 from .scheduler import (PlannedEntry, Request, RequestOptions, RequestStatus, Scheduler,
                         SchedulerOptions)
@@ -37,8 +37,12 @@ class Engine:
         self.sampler = sampler or Sampler(loaded.rt.ops, loaded.rt.device,
                                           loaded.spec.vocab_size, loaded.cache.max_requests)
         self._rng: Dict[int, XorShift64Star] = {}
+        # ``generate`` launches decode steps one ahead of their tokens (see _plan_ahead)
+        self.run_ahead = torch.device(loaded.rt.device).type == "cuda"
+        if self.run_ahead:
+            loaded.runner.token_source = self.sampler.last_tokens
         self.last_logits: Optional[torch.Tensor] = None
-        self.metrics = {"steps": 0, "step_seconds": 0.0}
+        self.metrics = {"steps": 0, "steps_ahead": 0, "step_seconds": 0.0}
 
     @classmethod
     def from_folder(cls, model_dir: str, *, dtype="bfloat16", device="cuda:0",
@@ -83,28 +87,83 @@ class Engine:
 
     def step(self) -> int:
         """Runs one batch; returns the number of tokens it fed (0 if there was nothing)."""
-        start = time.perf_counter()
         plan = self.scheduler.plan()
         self._sync_slots()
         if not plan:
             return 0
-        entries = [StepEntry(e.request.slot, e.start, e.request.tokens(e.start, e.count),
+        return self._complete(self._launch(plan))
+
+    # A step in two halves, so that ``generate`` can launch the next step before it reads
+    # this one's tokens.
+    def _launch(self, plan: List[PlannedEntry], device_tokens: bool = False):
+        start = time.perf_counter()
+        entries = [StepEntry(e.request.slot, e.start,
+                             [TOKEN_FROM_DEVICE] if device_tokens else e.request.tokens(e.start, e.count),
                              [e.count - 1] if e.samples else []) for e in plan]
         logits = self.loaded.runner.step(entries)
         self.last_logits = logits
-        sampled: List[int] = []
+        self.metrics["steps_ahead"] += int(device_tokens)
         slots = [e.request.slot for e in plan if e.samples]
         if self.sampler.uses_seen():
             self.sampler.mark_seen(self.loaded.runner.last_batch)
         if slots:
-            sampled = self.sampler.sample(logits, slots)
-        self.scheduler.accept(plan, sampled)
+            self.sampler.launch(logits, slots)
+        return plan, bool(slots), start
+
+    def _complete(self, launched) -> int:
+        plan, sampled_rows, start = launched
+        sampled = self.sampler.fetch() if sampled_rows else []
+        # a request that ended while this step was already under way: its row is dropped
+        it = iter(sampled)
+        entries, tokens = [], []
+        for e in plan:
+            token = next(it) if e.samples else None
+            if e.request.status.done:
+                continue
+            entries.append(e)
+            if e.samples:
+                tokens.append(token)
+        self.scheduler.accept(entries, tokens)
         self._sync_slots()
         for req in [e.request for e in plan if e.request.status.done]:
             self._rng.pop(req.id, None)
         self.metrics["steps"] += 1
         self.metrics["step_seconds"] += time.perf_counter() - start
-        return sum(e.count for e in plan)
+        return sum(e.count for e in entries)
+
+    def _plan_ahead(self, plan: List[PlannedEntry]) -> Optional[List[PlannedEntry]]:
+        """The step after ``plan``, decided before ``plan``'s tokens are known: possible when
+        every active request is decoding (nothing waits, nothing is being prefilled), for the
+        requests that this step's token cannot end by count or context.  A request that the
+        token does end (an end token) rides along for one row that is dropped afterwards;
+        what it writes lies in its own pages and state, which are only handed on by later
+        steps on the same stream."""
+        sched = self.scheduler
+        if not self.run_ahead or self.loaded.runner.token_source is None or sched.queue \
+                or len(plan) != len(sched.active):
+            return None
+        ahead = []
+        for e in plan:
+            req = e.request
+            if e.count != 1 or not e.samples or req.status != RequestStatus.DECODING or req.cancel_requested:
+                return None
+            if len(req.generated) + 1 >= req.options.max_new_tokens \
+                    or e.start + 2 >= sched.max_context:
+                continue
+            ahead.append(PlannedEntry(req, e.start + 1, 1, True))
+        if not ahead:
+            return None
+        cache = self.loaded.cache
+        need = [0] * len(cache.groups)
+        for e in ahead:
+            for g, n in enumerate(cache.pages_needed(e.request.slot, e.start, 1)):
+                need[g] += n
+        if any(n > free for n, free in zip(need, cache.free_pages())):
+            return None              # let the ordinary step decide what to do without pages
+        for e in ahead:
+            if not cache.prepare(e.request.slot, e.start, 1):
+                return None
+        return ahead
 
     # ------------------------------------------------------------------ convenience
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 128,
@@ -119,8 +178,18 @@ class Engine:
             ids.append(self.submit(prompt, RequestOptions(max_new_tokens=max_new_tokens,
                                                           eos_token_ids=eos_token_ids,
                                                           generation=g)))
-        while self.has_work():
-            self.step()
+        launched = None
+        while launched is not None or self.has_work():
+            if launched is None:
+                plan = self.scheduler.plan()
+                self._sync_slots()
+                if not plan:
+                    continue
+                launched = self._launch(plan)
+            ahead = self._plan_ahead(launched[0])
+            following = self._launch(ahead, device_tokens=True) if ahead else None
+            self._complete(launched)
+            launched = following
         out = []
         for rid in ids:
             req = self.scheduler.requests[rid]

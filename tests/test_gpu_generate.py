@@ -227,3 +227,40 @@ def test_steps_launched_ahead_of_their_tokens_give_the_same_tokens(model_folders
         bench.close()
         lm.cache.check()
     assert runs[True] == runs[False]
+
+
+def test_generation_ahead_of_the_tokens_with_requests_that_end_early(model_folders):
+    """``generate`` launches decode steps before it has read the previous step's tokens.
+    With end tokens chosen so that requests end at different steps (a request that ends
+    rides along for one dropped row), and with sampling, the tokens equal the plain
+    implementation's and those of an engine that never runs ahead."""
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY, GenerationConfig
+    folder = model_folders("B", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=300 + n) for n in (6, 11, 19, 4)]
+    free_run = [plain_generate(cfg, W, p, 24) for p in prompts]
+    # end tokens: what request 0 says at step 5, request 2 at step 11
+    eos = [free_run[0][5], free_run[2][11]]
+    outs = {}
+    for ahead in (True, False):
+        engine = Engine.from_folder(folder, dtype="float32", max_active_requests=4, n_pages=24,
+                                    max_batched_tokens=64, prefill_chunk_tokens=32)
+        engine.run_ahead = ahead
+        outs[ahead] = engine.generate(prompts, max_new_tokens=24, generation=GREEDY, eos_token_ids=eos)
+        assert (engine.metrics["steps_ahead"] > 10) == ahead
+        assert engine.loaded.cache.free_pages() == [24] and engine.loaded.cache.n_free_slots == 4
+        engine.loaded.cache.check()
+    assert outs[True] == outs[False]
+    for run, out in zip(free_run, outs[True]):
+        cut = next((i + 1 for i, t in enumerate(run) if t in eos), len(run))
+        assert out == run[:cut]
+    assert len(outs[True][0]) <= 6 and len(outs[True][2]) <= 12
+    # with a generator per request
+    gen = GenerationConfig(temperature=0.9, top_k=30, top_p=0.95, repetition_penalty=1.2, seed=11)
+    engine = Engine.from_folder(folder, dtype="float32", max_active_requests=4, n_pages=24,
+                                max_batched_tokens=64, prefill_chunk_tokens=32)
+    sampled = engine.generate(prompts, max_new_tokens=12, generation=gen, eos_token_ids=[])
+    assert engine.metrics["steps_ahead"] > 5
+    for prompt, out in zip(prompts, sampled):
+        assert out == plain_generate(cfg, W, prompt, 12, generation=gen)
