@@ -381,31 +381,20 @@ extern "C" int celeg_attention_rows_bf16(
 // joins the ranges of 64 keys.
 #define DEC_KEYS 64
 
+// The work on one range of 64 keys [kb, kb + 63] cut to [k_lo, k_hi] (not empty), by one
+// wavefront: scores, probabilities relative to the range's own maximum (left in ps for the
+// second product), and the accumulators.  ps: this wavefront's own GH x 64 floats of LDS.
 template <int HD, int GH>
-__global__ __launch_bounds__(64) void attention_decode_kernel(
+__device__ __forceinline__ void decode_range(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
-    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
-    const int* __restrict__ token_slot, const int* __restrict__ positions,
-    float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
-    int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer, float scale,
-    int window) {
+    const bf16* __restrict__ v_pool, const int* __restrict__ pages, int t, int h0, int kvh, int kb,
+    int k_lo, int k_hi, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer,
+    float scale, float (*ps)[DEC_KEYS], float (&m)[GH], float (&l)[GH], float (&acc)[GH][HD / 64]) {
     constexpr int DL = HD / 8;    // dims of a key a lane multiplies
     constexpr int DD = HD / 64;   // output dims a lane accumulates
-    __shared__ float ps[GH][DEC_KEYS];
-    const int split = blockIdx.x, hb = blockIdx.y, t = blockIdx.z;
-    const int lane = threadIdx.x;
-    const int pos = positions[t];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int kb = split * DEC_KEYS;
-    const int k_lo = max(lo, kb);
-    const int k_hi = min(pos, kb + DEC_KEYS - 1);
-    if (k_lo > k_hi) return;
-    const int h0 = hb * GH;
-    const int kvh = h0 / (q_heads / kv_heads);
+    const int lane = threadIdx.x & 63;
     const int j8 = lane >> 3, seg = lane & 7;
-    const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
-
-    // page ids of the chunk: lane i holds the i-th page that the 64 keys touch
+    // page ids of the range: lane i holds the i-th page that the 64 keys touch
     const int first_page = kb >> page_shift;
     const int last_page = k_hi >> page_shift;
     const int my_page = pages[min(first_page + lane, last_page)];
@@ -470,7 +459,6 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
             sc[it][g] = valid ? dot : -INFINITY;
         }
     }
-    float m[GH], l[GH];
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
         float mx = sc[0][g];
@@ -478,7 +466,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
         for (int it = 1; it < 8; ++it) mx = fmaxf(mx, sc[it][g]);
         mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));   // finite: the chunk holds a key of the range
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));   // finite: the range holds a key
         float psum = 0.f;
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
@@ -492,8 +480,10 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
         m[g] = mx;
         l[g] = psum;
     }
-    __syncthreads();
-    float acc[GH][DD];
+    // ps is this wavefront's own: its lanes only have to see each other's writes
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
     for (int g = 0; g < GH; ++g)
 #pragma unroll
@@ -522,6 +512,34 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
                 for (int j = 0; j < 16; ++j) acc[g][dd] = fmaf(ps[g][pg * 16 + j], vf[j], acc[g][dd]);
         }
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // ps may be written again by the caller's next range
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <int HD, int GH>
+__global__ __launch_bounds__(64) void attention_decode_kernel(
+    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
+    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
+    const int* __restrict__ token_slot, const int* __restrict__ positions,
+    float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
+    int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer, float scale,
+    int window) {
+    constexpr int DD = HD / 64;
+    __shared__ float ps[GH][DEC_KEYS];
+    const int split = blockIdx.x, hb = blockIdx.y, t = blockIdx.z;
+    const int lane = threadIdx.x;
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int kb = split * DEC_KEYS;
+    const int k_lo = max(lo, kb);
+    const int k_hi = min(pos, kb + DEC_KEYS - 1);
+    if (k_lo > k_hi) return;
+    const int h0 = hb * GH;
+    const int kvh = h0 / (q_heads / kv_heads);
+    const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
+    float m[GH], l[GH], acc[GH][DD];
+    decode_range<HD, GH>(q, ldq, k_pool, v_pool, pages, t, h0, kvh, kb, k_lo, k_hi, kv_heads,
+                         page_tokens, page_shift, n_layers, layer, scale, ps, m, l, acc);
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
         const size_t idx = (static_cast<size_t>(t) * q_heads + h0 + g) * n_splits + split;
@@ -529,6 +547,79 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 #pragma unroll
         for (int dd = 0; dd < DD; ++dd) ws_o[idx * HD + lane + 64 * dd] = acc[g][dd];
     }
+}
+
+// The same without a second kernel: one workgroup of DEC_WAVES wavefronts per (GH query
+// heads, request); wavefront w takes the ranges w, w + DEC_WAVES, ... and keeps a running
+// (max, sum, accumulator); the wavefronts' results meet in LDS and are joined in wavefront
+// order.  Fewer workgroups than the kernel above (it suits batches, not one long context).
+#define DEC_WAVES 16
+template <int HD, int GH>
+__global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_whole_kernel(
+    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
+    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
+    const int* __restrict__ token_slot, const int* __restrict__ positions, bf16* __restrict__ out,
+    int ldo, int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer,
+    float scale, int window) {
+    constexpr int DD = HD / 64;
+    __shared__ float ps_all[DEC_WAVES][GH][DEC_KEYS];
+    __shared__ float part_o[DEC_WAVES][GH][HD];
+    __shared__ float part_ml[DEC_WAVES][GH][2];
+    const int hb = blockIdx.x, t = blockIdx.y;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int h0 = hb * GH;
+    const int kvh = h0 / (q_heads / kv_heads);
+    const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
+    float M[GH], L[GH], O[GH][DD];
+#pragma unroll
+    for (int g = 0; g < GH; ++g) {
+        M[g] = -INFINITY;
+        L[g] = 0.f;
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) O[g][dd] = 0.f;
+    }
+    for (int r = lo / DEC_KEYS + wave; r <= pos / DEC_KEYS; r += DEC_WAVES) {
+        const int kb = r * DEC_KEYS;
+        float m[GH], l[GH], acc[GH][DD];
+        decode_range<HD, GH>(q, ldq, k_pool, v_pool, pages, t, h0, kvh, kb, max(lo, kb),
+                             min(pos, kb + DEC_KEYS - 1), kv_heads, page_tokens, page_shift, n_layers,
+                             layer, scale, ps_all[wave], m, l, acc);
+#pragma unroll
+        for (int g = 0; g < GH; ++g) {
+            const float mn = fmaxf(M[g], m[g]);
+            const float a = expf(M[g] - mn), b = expf(m[g] - mn);   // e^(-inf) = 0 the first time
+            L[g] = L[g] * a + l[g] * b;
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) O[g][dd] = O[g][dd] * a + acc[g][dd] * b;
+            M[g] = mn;
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < GH; ++g) {
+        if (lane == 0) { part_ml[wave][g][0] = M[g]; part_ml[wave][g][1] = L[g]; }
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) part_o[wave][g][lane + 64 * dd] = O[g][dd];
+    }
+    __syncthreads();
+    // wavefront g of the first GH joins head h0 + g
+    if (wave >= GH) return;
+    const int g = wave;
+    float mx = -INFINITY;
+    for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, part_ml[w][g][0]);
+    float denom = 0.f, o[DD];
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd) o[dd] = 0.f;
+    for (int w = 0; w < DEC_WAVES; ++w) {
+        const float wgt = expf(part_ml[w][g][0] - mx);      // a wavefront without a range: e^(-inf) = 0
+        denom += wgt * part_ml[w][g][1];
+#pragma unroll
+        for (int dd = 0; dd < DD; ++dd) o[dd] = fmaf(wgt, part_o[w][g][lane + 64 * dd], o[dd]);
+    }
+    bf16* orow = out + static_cast<size_t>(t) * ldo + static_cast<size_t>(h0 + g) * HD;
+#pragma unroll
+    for (int dd = 0; dd < DD; ++dd) orow[lane + 64 * dd] = from_float<bf16>(o[dd] / denom);
 }
 
 // Joins the ranges of one (request, query head): out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
@@ -586,7 +677,7 @@ extern "C" int celeg_attention_decode_bf16(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
     int n_splits, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
-    int head_dim, int page_tokens, int n_layers, int layer, float scale, int window,
+    int head_dim, int page_tokens, int n_layers, int layer, float scale, int window, int whole,
     hipStream_t stream) {
     if (n_rows <= 0) return 0;
     const int group = q_heads / kv_heads;
@@ -595,6 +686,28 @@ extern "C" int celeg_attention_decode_bf16(
         return static_cast<int>(hipErrorInvalidValue);
     const int page_shift = __builtin_ctz(page_tokens);
     const int gh = (group % 4 == 0) ? 4 : ((group % 2 == 0) ? 2 : 1);
+    // enough (heads, request) pairs to occupy every compute unit: one workgroup each and no
+    // second kernel (measured at context 2,176, 8 key/value heads: batch 64 54 us against 68 us;
+    // batch 8 20 us against 15.5 us, a workgroup then being bound by what one compute unit
+    // can pull).  whole: 0 the split-key kernels, 1 the whole-context kernel, -1 decide here.
+    if (whole < 0) whole = (q_heads / gh) * n_rows >= 192 ? 1 : 0;
+    if (whole) {
+        dim3 wgrid(q_heads / gh, n_rows), wblock(DEC_WAVES * 64);
+#define CELEG_WHOLE(HD_, GH_)                                                                    \
+    hipLaunchKernelGGL((attention_decode_whole_kernel<HD_, GH_>), wgrid, wblock, 0, stream,      \
+                       static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
+                       static_cast<const bf16*>(v_pool), table, table_stride, token_slot,        \
+                       positions, static_cast<bf16*>(out), ldo, q_heads, kv_heads, page_tokens,  \
+                       page_shift, n_layers, layer, scale, window)
+#define CELEG_WHOLE_HD(HD_)                                                                      \
+    if (gh == 4) CELEG_WHOLE(HD_, 4); else if (gh == 2) CELEG_WHOLE(HD_, 2); else CELEG_WHOLE(HD_, 1)
+        if (head_dim == 64) { CELEG_WHOLE_HD(64); }
+        else if (head_dim == 128) { CELEG_WHOLE_HD(128); }
+        else return static_cast<int>(hipErrorInvalidValue);
+#undef CELEG_WHOLE_HD
+#undef CELEG_WHOLE
+        return CELEG_LAUNCH_RESULT();
+    }
     dim3 grid(n_splits, q_heads / gh, n_rows), block(64);
 #define CELEG_DEC(HD_, GH_)                                                                      \
     hipLaunchKernelGGL((attention_decode_kernel<HD_, GH_>), grid, block, 0, stream,              \

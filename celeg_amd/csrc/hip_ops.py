@@ -42,6 +42,7 @@ class HipOps:
         self.loaded_libraries: Dict[str, str] = {}
         # "auto": the matrix-core and split-key kernels where they apply; "general": always
         # the general kernel (tests compare the two)
+        self.attention_decode_whole = -1     # -1: chosen from the batch; 0 split-key kernels; 1 one workgroup a request
         self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
         self.attention_impl = "auto"
         self._decode_ws = None
@@ -357,7 +358,7 @@ class HipOps:
             _ptr(ws_ml), _c_int(n_splits), _ptr(out), _c_int(heads * head_dim),
             _c_int(T), _c_int(heads), _c_int(kv_heads), _c_int(head_dim), _c_int(kv.page_tokens),
             _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
-            _c_int(window if window else 0), self._stream())
+            _c_int(window if window else 0), _c_int(self.attention_decode_whole), self._stream())
         self._check(code, "attention for decode rows (bfloat16)")
 
     # ------------------------------------------------------------------ sampling

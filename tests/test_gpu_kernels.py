@@ -340,3 +340,22 @@ def test_attention_rows_tile_pairs(ops, rows_per_tile, heads, kv_heads, head_dim
                        page_tokens=page_tokens)
     finally:
         ops.attention_rows_per_tile = 0
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [(4, 2, 64, 16), (8, 1, 128, 32), (3, 1, 64, 64)])
+def test_attention_decode_one_workgroup_per_request(ops, heads, kv_heads, head_dim, page_tokens):
+    """The decode kernel that walks a request's whole context in one workgroup (16
+    wavefronts, joined in LDS): long contexts (more ranges of 64 keys than wavefronts), a
+    boosted far key, and a window that cuts the first range."""
+    ops.attention_decode_whole = 1
+    try:
+        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[1300, 150, 70],
+                       cuts=[1260] + [1] * 40, boost=(2, 1290), page_tokens=page_tokens)
+        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[400],
+                       cuts=[300, 1, 1, 60, 1] + [1] * 40, window=150, boost=(231, 380),
+                       qk_norm=False, rotary_dim=0, page_tokens=page_tokens)
+        attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[400],
+                       cuts=[300, 1, 1, 60, 1] + [1] * 40, window=150, boost=(230, 380),
+                       qk_norm=False, rotary_dim=0, page_tokens=page_tokens)
+    finally:
+        ops.attention_decode_whole = -1
