@@ -240,15 +240,21 @@ static int launch_slices(const GemvParams& p, int chunks_per_wave, hipStream_t s
 }
 
 // How many k-slices share the matrix instruction's tile for this many rows and this K.
-static int slices_for(int M, int K) {
+static int g_force_slices = 0;     // a tuning aid: 1, 2 or 4 overrides the choice below where it fits
+extern "C" void celeg_gemv_slices_force(int g) { g_force_slices = g; }
+
+static int slices_for(int M, int N, int K) {
     int g = M <= 4 ? 4 : (M <= 8 ? 2 : 1);
+    if (g_force_slices > 0 && g_force_slices <= g) g = g_force_slices;
     while (g > 1 && K % (8 * g)) g >>= 1;
+    // more than about a thousand workgroups gain nothing (measured on 4,608 columns)
+    while (g > 1 && g_force_slices == 0 && (N + 16 / g - 1) / (16 / g) > 1024) g >>= 1;
     return g;
 }
 
 template <int EPI>
 static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
-    const int g = slices_for(p.M, p.K);
+    const int g = slices_for(p.M, p.N, p.K);
     const int chunks = (p.K / g + 63) / 64;
     const int kw = chunks >= 24 ? 8 : 4;
     const int cpw = (chunks + kw - 1) / kw;
@@ -262,7 +268,7 @@ extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvPar
 // Number of workgroups for these sizes, which is also the number of partial sums of
 // squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
 extern "C" int celeg_gemv_slices_blocks(int M, int N, int K) {
-    const int mp = 16 / slices_for(M, K);
+    const int mp = 16 / slices_for(M, N, K);
     return (N + mp - 1) / mp;
 }
 

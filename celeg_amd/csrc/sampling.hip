@@ -11,15 +11,8 @@
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_MAX_K 128
+#define SAMPLE_HIST_COPIES 16
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ float penalised_logit(const float* __restrict__ row,
-                                                 const uint8_t* __restrict__ seen, float penalty,
-                                                 int i) {
-    float v = row[i];
-    if (seen && penalty > 1.0f && seen[i]) v = v >= 0.0f ? v / penalty : v * penalty;
-    return v;
-}
 
 // larger float <-> larger key
 __device__ __forceinline__ uint32_t order_key(float f) {
@@ -31,6 +24,225 @@ __device__ __forceinline__ bool better(float sa, int ia, float sb, int ib) {
     return sa == sb ? ia < ib : sa > sb;
 }
 
+// Walks a row of logits: f(penalised value, index) for this thread's share, groups of 4
+// logits, 8 groups of a thread asked for before any is looked at (a row of 65,536 logits is
+// then two round trips to memory instead of 64).  A thread's indices come in rising order.
+template <typename F>
+__device__ __forceinline__ void for_each_logit(const float* __restrict__ row,
+                                               const uint8_t* __restrict__ seen, float penalty,
+                                               int vocab, int tid, F f) {
+    const bool pen = seen && penalty > 1.0f;
+    const bool vec = (reinterpret_cast<uintptr_t>(row) & 15) == 0 &&
+                     (!pen || (reinterpret_cast<uintptr_t>(seen) & 3) == 0);
+    const int n4 = vec ? vocab >> 2 : 0;
+    auto take = [&](float v, unsigned seen_byte, int i) {
+        if (seen_byte) v = v >= 0.0f ? v / penalty : v * penalty;
+        f(v, i);
+    };
+    constexpr int UN = 8;
+    for (int g0 = tid; g0 < n4; g0 += SAMPLE_THREADS * UN) {
+        floatx4_t v[UN];
+        unsigned sn[UN];
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const int g = min(g0 + j * SAMPLE_THREADS, n4 - 1);      // clamped, masked below
+            v[j] = reinterpret_cast<const floatx4_t*>(row)[g];
+            sn[j] = pen ? reinterpret_cast<const unsigned*>(seen)[g] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const int g = g0 + j * SAMPLE_THREADS;
+            if (g < n4) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) take(v[j][e], (sn[j] >> (8 * e)) & 0xffu, 4 * g + e);
+            }
+        }
+    }
+    for (int i = 4 * n4 + tid; i < vocab; i += SAMPLE_THREADS)      // what the groups left
+        take(row[i], pen ? seen[i] : 0u, i);
+}
+
+__device__ __forceinline__ float key_score(uint32_t key) {      // the inverse of order_key
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+// The top_k scores of a row (score = penalised logit / temperature) by (score desc, id
+// asc), left unordered in cand_score / cand_id [0, top_k).  All threads of the workgroup
+// call it.  KPT > 0: the row's keys are held in registers, KPT a thread, element
+// tid + SAMPLE_THREADS * j in place j (vocab <= SAMPLE_THREADS * KPT); KPT == 0: every pass
+// walks the row in memory.
+template <int KPT>
+__device__ __forceinline__ void top_k_candidates(
+    const float* __restrict__ row, const uint8_t* __restrict__ seen, float penalty, float temperature,
+    int vocab, int top_k, unsigned int* hist, unsigned int* sel, int* running, float* cand_score,
+    int* cand_id) {
+    const int tid = threadIdx.x;
+    const int lane = tid & (CELEG_WAVE - 1);
+    constexpr int NK = KPT > 0 ? KPT : 1;
+    uint32_t keys[NK];
+    if (KPT > 0) {
+        const bool pen = seen && penalty > 1.0f;
+        float v[NK];
+        unsigned char sn[NK];
+#pragma unroll
+        for (int j = 0; j < NK; ++j) {
+            const int i = min(tid + SAMPLE_THREADS * j, vocab - 1);      // clamped, masked below
+            v[j] = row[i];
+            sn[j] = pen ? seen[i] : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < NK; ++j) {
+            float x = v[j];
+            if (sn[j]) x = x >= 0.0f ? x / penalty : x * penalty;
+            keys[j] = tid + SAMPLE_THREADS * j < vocab ? order_key(x / temperature) : 0u;
+        }
+    }
+    // f(key, index) for this thread's share of the row
+    auto walk = [&](auto f) {
+        if (KPT > 0) {
+#pragma unroll
+            for (int j = 0; j < NK; ++j)
+                if (tid + SAMPLE_THREADS * j < vocab) f(keys[j], tid + SAMPLE_THREADS * j);
+        } else {
+            for_each_logit(row, seen, penalty, vocab, tid,
+                           [&](float x, int i) { f(order_key(x / temperature), i); });
+        }
+    };
+    // One counting pass: bins of bin_of(key, index) >= 0.  The counts go to
+    // SAMPLE_HIST_COPIES copies of the 256 bins, a lane using copy lane % copies: scores
+    // crowd into a few bins of the top byte, and lanes that hit one address take turns.
+    auto count_pass = [&](auto bin_of) {
+        for (int i = tid; i < 256 * SAMPLE_HIST_COPIES; i += SAMPLE_THREADS) hist[i] = 0u;
+        __syncthreads();
+        unsigned int* mine = hist + (lane % SAMPLE_HIST_COPIES) * 256;
+        walk([&](uint32_t key, int i) {
+            const int bin = bin_of(key, i);
+            if (bin >= 0) atomicAdd(&mine[bin], 1u);
+        });
+        __syncthreads();
+        if (tid < 256) {
+            unsigned int total = 0u;
+#pragma unroll
+            for (int c = 0; c < SAMPLE_HIST_COPIES; ++c) total += hist[c * 256 + tid];
+            hist[tid] = total;
+        }
+        __syncthreads();
+    };
+    // after a pass: the bin in which the sought place lies, counted from the top (largest
+    // first) or from the bottom; sel = {prefix so far, places still to go, size of that bin}
+    auto choose_bin = [&](int shift, bool from_top) {
+        if (tid < CELEG_WAVE) {       // one wavefront: lane l takes the l-th four bins of the walk
+            const unsigned int remaining = sel[1];
+            unsigned int c[4], mine = 0u;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int pos = 4 * lane + e;
+                c[e] = hist[from_top ? 255 - pos : pos];
+                mine += c[e];
+            }
+            unsigned int before = mine;      // inclusive sum over the lanes in front, then exclusive
+#pragma unroll
+            for (int off = 1; off < CELEG_WAVE; off <<= 1) {
+                const unsigned int o = __shfl_up(before, off, CELEG_WAVE);
+                if (lane >= off) before += o;
+            }
+            before -= mine;
+            // the first place of the walk at which the running count reaches what is sought;
+            // if none does (it cannot, the counts add up to at least that), the last bin
+            const bool here = before < remaining && before + mine >= remaining;
+            const unsigned long long found = __ballot(here);
+            const int owner = found ? __ffsll(static_cast<long long>(found)) - 1 : CELEG_WAVE - 1;
+            if (lane == owner) {
+                unsigned int passed = before;
+                int e = 0;
+                for (; e < 3; ++e) {
+                    if (passed + c[e] >= remaining) break;
+                    passed += c[e];
+                }
+                const int pos = 4 * lane + e;
+                const int bin = from_top ? 255 - pos : pos;
+                sel[0] |= static_cast<unsigned>(bin) << shift;
+                sel[1] = remaining - passed;
+                sel[2] = c[e];
+            }
+        }
+        __syncthreads();
+    };
+
+    // ---- a bound from below first, so that few scores take part in the counting: every
+    // thread's largest score is a score of its own, so the top_k-th largest of these maxima is
+    // not above the top_k-th largest score overall.  Found by the same selection (8 bits a
+    // pass, from the top), one count a thread a pass.
+    uint32_t my_max = 0u;
+    walk([&](uint32_t key, int) { my_max = max(my_max, key); });
+    if (tid == 0) { sel[0] = 0u; sel[1] = static_cast<unsigned>(top_k); }
+    __syncthreads();
+    unsigned int mask = 0u;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        const unsigned int prefix = sel[0];
+        for (int i = tid; i < 256; i += SAMPLE_THREADS) hist[i] = 0u;
+        __syncthreads();
+        if ((my_max & mask) == prefix) atomicAdd(&hist[(my_max >> shift) & 255u], 1u);
+        __syncthreads();
+        choose_bin(shift, true);
+        mask |= 255u << shift;
+    }
+    const uint32_t lower = sel[0];
+    __syncthreads();
+
+    // ---- the top_k-th largest score itself
+    if (tid == 0) { sel[0] = 0u; sel[1] = static_cast<unsigned>(top_k); }
+    __syncthreads();
+    mask = 0u;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        const unsigned int prefix = sel[0];
+        count_pass([&](uint32_t key, int) {
+            return (key >= lower && (key & mask) == prefix) ? static_cast<int>((key >> shift) & 255u) : -1;
+        });
+        choose_bin(shift, true);
+        mask |= 255u << shift;
+    }
+    const uint32_t kth = sel[0];
+    const int need_eq = static_cast<int>(sel[1]);  // how many of the ties at the threshold to take
+    const int n_eq = static_cast<int>(sel[2]);     // how many scores equal the threshold
+    const int n_gt = top_k - need_eq;
+    __syncthreads();
+
+    // ---- of the ties at the threshold the lowest ids are taken: if not all of them, the
+    // need_eq-th lowest id is found the same way (ids rising, 8 bits a pass)
+    int last_tie = 0x7fffffff;
+    if (need_eq < n_eq) {
+        if (tid == 0) { sel[0] = 0u; sel[1] = static_cast<unsigned>(need_eq); }
+        __syncthreads();
+        unsigned int imask = 0u;
+        for (int shift = 24; shift >= 0; shift -= 8) {
+            const unsigned int prefix = sel[0];
+            count_pass([&](uint32_t key, int i) {
+                return (key == kth && (static_cast<unsigned>(i) & imask) == prefix)
+                           ? static_cast<int>((static_cast<unsigned>(i) >> shift) & 255u) : -1;
+            });
+            choose_bin(shift, false);
+            imask |= 255u << shift;
+        }
+        last_tie = static_cast<int>(sel[0]);
+        __syncthreads();
+    }
+
+    // ---- the candidates, in any order (the caller sorts them)
+    if (tid == 0) { running[0] = 0; running[1] = 0; }
+    __syncthreads();
+    walk([&](uint32_t key, int i) {
+        if (key > kth) {
+            const int p = atomicAdd(&running[0], 1);
+            if (p < n_gt) { cand_score[p] = key_score(key); cand_id[p] = i; }
+        } else if (key == kth && i <= last_tie) {
+            const int e = atomicAdd(&running[1], 1);
+            if (e < need_eq) { cand_score[n_gt + e] = key_score(key); cand_id[n_gt + e] = i; }
+        }
+    });
+    __syncthreads();
+}
+
 // fparams[row] = {temperature, top_p, penalty, u}; iparams[row] = {top_k, seen_row or -1,
 // slot or -1}; the token also goes to last_tokens[slot] (if given and slot >= 0), where the
 // next step can take it from without the host in between.
@@ -40,9 +252,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int* __restrict__ out_tokens, int* __restrict__ last_tokens) {
     __shared__ float s_val[SAMPLE_THREADS / CELEG_WAVE];
     __shared__ int s_idx[SAMPLE_THREADS / CELEG_WAVE];
-    __shared__ unsigned int hist[256];
-    __shared__ unsigned int sel[3];       // prefix, remaining, (unused)
-    __shared__ int wave_gt[SAMPLE_THREADS / CELEG_WAVE], wave_eq[SAMPLE_THREADS / CELEG_WAVE];
+    __shared__ unsigned int hist[256 * SAMPLE_HIST_COPIES];
+    __shared__ unsigned int sel[3];       // prefix, remaining, size of the last bin
     __shared__ int running[2];
     __shared__ float cand_score[SAMPLE_MAX_K];
     __shared__ int cand_id[SAMPLE_MAX_K];
@@ -62,39 +273,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 
     if (temperature <= 0.0f || top_k == 1) {
         // ---- penalised argmax, lowest index wins ties
-        // Groups of 4 logits, 8 groups of a thread asked for before any is looked at (a
-        // row of 65,536 logits is then two round trips to memory instead of 64).
         float best = -INFINITY;
         int best_i = 0x7fffffff;
-        const bool pen = seen && penalty > 1.0f;
-        const bool vec = (reinterpret_cast<uintptr_t>(row) & 15) == 0 &&
-                         (!pen || (reinterpret_cast<uintptr_t>(seen) & 3) == 0);
-        const int n4 = vec ? vocab >> 2 : 0;
-        auto take = [&](float v, unsigned seen_byte, int i) {
-            if (seen_byte) v = v >= 0.0f ? v / penalty : v * penalty;
+        for_each_logit(row, seen, penalty, vocab, tid, [&](float v, int i) {
             if (best_i == 0x7fffffff || v > best) { best = v; best_i = i; }
-        };
-        constexpr int UN = 8;
-        for (int g0 = tid; g0 < n4; g0 += SAMPLE_THREADS * UN) {
-            floatx4_t v[UN];
-            unsigned sn[UN];
-#pragma unroll
-            for (int j = 0; j < UN; ++j) {
-                const int g = min(g0 + j * SAMPLE_THREADS, n4 - 1);      // clamped, masked below
-                v[j] = reinterpret_cast<const floatx4_t*>(row)[g];
-                sn[j] = pen ? reinterpret_cast<const unsigned*>(seen)[g] : 0u;
-            }
-#pragma unroll
-            for (int j = 0; j < UN; ++j) {
-                const int g = g0 + j * SAMPLE_THREADS;
-                if (g < n4) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) take(v[j][e], (sn[j] >> (8 * e)) & 0xffu, 4 * g + e);
-                }
-            }
-        }
-        for (int i = 4 * n4 + tid; i < vocab; i += SAMPLE_THREADS)      // what the groups left
-            take(row[i], pen ? seen[i] : 0u, i);
+        });
         for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) {
             const float ov = __shfl_xor(best, off, CELEG_WAVE);
             const int oi = __shfl_xor(best_i, off, CELEG_WAVE);
@@ -117,120 +300,71 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
 
     top_k = min(min(top_k, vocab), SAMPLE_MAX_K);
-    // ---- radix select of the top_k-th largest score
-    if (tid == 0) { sel[0] = 0u; sel[1] = static_cast<unsigned>(top_k); }
-    unsigned int mask = 0u;
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        if (tid < 256) hist[tid] = 0u;
-        __syncthreads();
-        const unsigned int prefix = sel[0];
-        for (int i = tid; i < vocab; i += SAMPLE_THREADS) {
-            const uint32_t key = order_key(penalised_logit(row, seen, penalty, i) / temperature);
-            if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
-        }
-        __syncthreads();
-        if (tid == 0) {
-            unsigned int remaining = sel[1], above = 0u;
-            int bin = 255;
-            for (; bin > 0; --bin) {
-                if (above + hist[bin] >= remaining) break;
-                above += hist[bin];
-            }
-            sel[0] = prefix | (static_cast<unsigned>(bin) << shift);
-            sel[1] = remaining - above;
-        }
-        mask |= 255u << shift;
-        __syncthreads();
-    }
-    const uint32_t kth = sel[0];
-    const int need_eq = static_cast<int>(sel[1]);  // how many of the ties at the threshold to take
-    const int n_gt = top_k - need_eq;
-
-    // ---- ordered compaction: all above the threshold, and the lowest-id ties
-    if (tid == 0) { running[0] = 0; running[1] = 0; }
-    __syncthreads();
-    for (int base = 0; base < vocab; base += SAMPLE_THREADS) {
-        const int i = base + tid;
-        float score = 0.f;
-        bool gt = false, eq = false;
-        if (i < vocab) {
-            score = penalised_logit(row, seen, penalty, i) / temperature;
-            const uint32_t key = order_key(score);
-            gt = key > kth;
-            eq = key == kth;
-        }
-        const unsigned long long m_gt = __ballot(gt), m_eq = __ballot(eq);
-        const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (CELEG_WAVE - lane));
-        const int p_gt = __popcll(m_gt & below), p_eq = __popcll(m_eq & below);
-        if (lane == 0) { wave_gt[wave] = __popcll(m_gt); wave_eq[wave] = __popcll(m_eq); }
-        __syncthreads();
-        int off_gt = running[0], off_eq = running[1];
-        for (int w = 0; w < wave; ++w) { off_gt += wave_gt[w]; off_eq += wave_eq[w]; }
-        if (gt) {
-            const int p = off_gt + p_gt;
-            if (p < n_gt) { cand_score[p] = score; cand_id[p] = i; }
-        } else if (eq) {
-            const int e = off_eq + p_eq;
-            if (e < need_eq) { cand_score[n_gt + e] = score; cand_id[n_gt + e] = i; }
-        }
-        __syncthreads();
-        if (tid == 0) {
-            int a = 0, b = 0;
-            for (int w = 0; w < n_waves; ++w) { a += wave_gt[w]; b += wave_eq[w]; }
-            running[0] += a; running[1] += b;
-        }
-        __syncthreads();
-    }
+    // the scores of the row are turned into keys once and kept in registers (up to 128 a
+    // thread); larger vocabularies walk the row again for every pass
+    if (vocab <= SAMPLE_THREADS * 64)
+        top_k_candidates<64>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
+    else if (vocab <= SAMPLE_THREADS * 128)
+        top_k_candidates<128>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
+    else
+        top_k_candidates<0>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
     if (tid >= top_k && tid < SAMPLE_MAX_K) { cand_score[tid] = -INFINITY; cand_id[tid] = 0x7fffffff; }
     __syncthreads();
+    if (wave != 0) return;         // one wavefront does the rest: no workgroup barriers from here
 
-    // ---- bitonic sort of 128 candidates by (score desc, id asc)
+    // ---- bitonic sort of 128 candidates by (score desc, id asc): lane l owns the pair whose
+    // lower member is the l-th position with the stride's bit clear
     for (int size = 2; size <= SAMPLE_MAX_K; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            if (tid < SAMPLE_MAX_K) {
-                const int partner = tid ^ stride;
-                if (partner > tid) {
-                    const bool ascending_block = (tid & size) == 0;  // "best first" blocks
-                    const float sa = cand_score[tid], sb = cand_score[partner];
-                    const int ia = cand_id[tid], ib = cand_id[partner];
-                    const bool a_first = better(sa, ia, sb, ib);
-                    if (ascending_block ? !a_first : a_first) {
-                        cand_score[tid] = sb; cand_id[tid] = ib;
-                        cand_score[partner] = sa; cand_id[partner] = ia;
-                    }
-                }
+            const int a = ((lane & ~(stride - 1)) << 1) | (lane & (stride - 1));
+            const int partner = a | stride;
+            const bool ascending_block = (a & size) == 0;  // "best first" blocks
+            const float sa = cand_score[a], sb = cand_score[partner];
+            const int ia = cand_id[a], ib = cand_id[partner];
+            const bool a_first = better(sa, ia, sb, ib);
+            if (ascending_block ? !a_first : a_first) {
+                cand_score[a] = sb; cand_id[a] = ib;
+                cand_score[partner] = sa; cand_id[partner] = ia;
             }
-            __syncthreads();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
     }
 
-    // ---- softmax, top-p prefix and the walk, sequentially as the reference does
-    if (tid == 0) {
-        const float maximum = cand_score[0];
-        float total = 0.f;
-        for (int i = 0; i < top_k; ++i) {
-            cand_score[i] = expf(cand_score[i] - maximum);
-            total += cand_score[i];
-        }
-        for (int i = 0; i < top_k; ++i) cand_score[i] /= total;
-        int active = top_k;
-        if (top_p < 1.0f) {
-            float cumulative = 0.f;
-            active = 0;
-            do {
-                cumulative += cand_score[active++];
-            } while (active < top_k && cumulative < top_p);
-            total = 0.f;
-            for (int i = 0; i < active; ++i) total += cand_score[i];
-        } else {
-            total = 1.0f;
-        }
-        float target = u * total;
-        int chosen = cand_id[active - 1];
-        for (int i = 0; i < active; ++i) {
-            target -= cand_score[i];
-            if (target <= 0.0f) { chosen = cand_id[i]; break; }
-        }
+    // ---- softmax, top-p prefix and the walk.  The sums run over the candidates one after
+    // the other, in the reference's order; a candidate's value comes from the lane that
+    // holds it (lane i % 64, first or second register), so that the loops touch no memory.
+    const float maximum = cand_score[0];
+    float e0 = expf(cand_score[lane] - maximum), e1 = expf(cand_score[lane + 64] - maximum);
+    const int id0 = cand_id[lane], id1 = cand_id[lane + 64];
+    auto value_at = [&](float first, float second, int i) {
+        return __shfl(i < 64 ? first : second, i & 63, CELEG_WAVE);
+    };
+    float total = 0.f;
+    for (int i = 0; i < top_k; ++i) total += value_at(e0, e1, i);
+    e0 /= total;
+    e1 /= total;
+    int active = top_k;
+    if (top_p < 1.0f) {
+        float cumulative = 0.f;
+        active = 0;
+        do {
+            cumulative += value_at(e0, e1, active++);
+        } while (active < top_k && cumulative < top_p);
+        total = 0.f;
+        for (int i = 0; i < active; ++i) total += value_at(e0, e1, i);
+    } else {
+        total = 1.0f;
+    }
+    float target = u * total;
+    int chosen_at = active - 1;
+    for (int i = 0; i < active; ++i) {
+        target -= value_at(e0, e1, i);
+        if (target <= 0.0f) { chosen_at = i; break; }
+    }
+    const int chosen = __shfl(chosen_at < 64 ? id0 : id1, chosen_at & 63, CELEG_WAVE);
+    if (lane == 0) {
         out_tokens[r] = chosen;
         if (last_tokens && slot >= 0) last_tokens[slot] = chosen;
     }
