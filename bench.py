@@ -38,6 +38,26 @@ PROMPT_TOKENS = 2048
 BATCH = 8
 
 
+def lfm2_shape(hidden, heads, kv_heads, intermediate, attention_layers, layers, context):
+    cfg = dict(LFM2_350M)
+    cfg.update(hidden_size=hidden, num_attention_heads=heads, num_key_value_heads=kv_heads,
+               intermediate_size=intermediate, num_hidden_layers=layers,
+               layer_types=["full_attention" if i in attention_layers else "conv" for i in range(layers)],
+               max_position_embeddings=context)
+    return cfg
+
+
+# The other LFM2 shapes, each with the serving workload it is measured on (--phase serve):
+# requests, prompt lengths (lowest, highest), new tokens, prefill portion, most tokens a step.
+SHAPES = {
+    "350m": (LFM2_350M, dict(requests=64, prompt=(2048, 2048), new_tokens=256, chunk=2048, budget=2048)),
+    "1.2b": (lfm2_shape(2048, 32, 8, 12288, {2, 5, 8, 10, 12, 14}, 16, 4096),
+             dict(requests=64, prompt=(128, 2048), new_tokens=256, chunk=2048, budget=2048)),
+    "2.6b": (lfm2_shape(2048, 32, 8, 10752, {2, 6, 10, 14, 18, 21, 24, 27}, 30, 8192),
+             dict(requests=32, prompt=(4096, 4096), new_tokens=512, chunk=512, budget=1024)),
+}
+
+
 def weight_bytes(model) -> int:
     seen = {}
     for _, part in model.named_parts():
@@ -65,6 +85,51 @@ def prefill_flops(cfg, tokens: int, ff: int) -> float:
     return per_token * tokens + attention + 2.0 * H * cfg["vocab_size"]   # head for one row
 
 
+def serve(shape: str) -> int:
+    """The whole engine on a serving workload: every request submitted at once, the scheduler
+    cuts the prompts into portions beside the decoding requests, sampling is greedy on the
+    device.  Prints one JSON line: generated tokens a second over the whole run."""
+    import random
+    import torch
+    from celeg_amd.engine import Engine
+    from celeg_amd.weights import write_random_model
+
+    cfg, load = SHAPES[shape]
+    rng = random.Random(0)
+    lengths = [rng.randint(*load["prompt"]) for _ in range(load["requests"])]
+    prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(n)] for n in lengths]
+    pages = sum((n + load["new_tokens"] + 15) // 16 + 1 for n in lengths)
+    with tempfile.TemporaryDirectory(prefix="celeg_bench_") as folder:
+        write_random_model(cfg, folder, seed=0, dtype=torch.bfloat16, std=0.02)
+        engine = Engine.from_folder(folder, dtype="bfloat16", device="cuda:0", page_tokens=16,
+                                    n_pages=pages, max_active_requests=load["requests"],
+                                    max_batched_tokens=load["budget"],
+                                    prefill_chunk_tokens=load["chunk"],
+                                    context=cfg["max_position_embeddings"])
+    # a short run first: kernels loaded, graphs captured for the decode batch sizes
+    engine.generate(prompts[:2], max_new_tokens=4, eos_token_ids=[])
+    for key in engine.metrics:
+        engine.metrics[key] = type(engine.metrics[key])()
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    out = engine.generate(prompts, max_new_tokens=load["new_tokens"], eos_token_ids=[])
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - start
+    generated = sum(len(o) for o in out)
+    print(json.dumps({
+        "metric": f"serve: generated tok/s (LFM2-{shape.upper()} shape, bf16, whole engine)",
+        "value": round(generated / seconds, 1), "unit": "tokens/s", "phase": "serve",
+        "seconds": round(seconds, 3), "generated_tokens": generated,
+        "prompt_tokens": sum(lengths),
+        "all_tokens_per_second": round((generated + sum(lengths)) / seconds, 1),
+        "requests": load["requests"], "prompt_lengths": list(load["prompt"]),
+        "new_tokens": load["new_tokens"], "prefill_chunk": load["chunk"],
+        "step_token_budget": load["budget"], "context": cfg["max_position_embeddings"],
+        "engine_steps": engine.metrics["steps"], "steps_launched_ahead": engine.metrics["steps_ahead"],
+        "dtype": "bf16", "data": "synthetic"}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -74,14 +139,20 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     ap.add_argument("--batch", type=int, default=BATCH,
                     help="for profiling with --phase decode: another batch size than the headline's 8")
-    ap.add_argument("--phase", choices=["all", "prefill", "decode"], default="all",
+    ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
-                         "decode measurement (the line printed then holds only that part)")
+                         "decode measurement (the line printed then holds only that part); "
+                         "serve: the whole engine on the serving workload of --shape")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="350m",
+                    help="the LFM2 shape (the headline line is the 350m one)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported "
               "(this engine runs on a single MI355X)")
         return 2
+
+    if args.phase == "serve":
+        return serve(args.shape)
 
     import torch
     import celeg_amd  # noqa: F401
@@ -89,7 +160,7 @@ def main() -> int:
     from celeg_amd.engine.benchmark import DecodeBench, measure_prefill
     from celeg_amd.weights import write_random_model
 
-    cfg = dict(LFM2_350M)
+    cfg = dict(SHAPES[args.shape][0])
     full_layers = cfg["num_hidden_layers"]
     if args.layers and args.layers < full_layers:
         cfg["num_hidden_layers"] = args.layers
@@ -115,7 +186,7 @@ def main() -> int:
     else:
         prefill = measure_prefill(lm, PROMPT_TOKENS, repeats=7, warmup=3)
     if args.phase == "prefill":
-        print(json.dumps({"metric": "prefill tok/s @ 2048 tokens (LFM2-350M shape, bf16)",
+        print(json.dumps({"metric": f"prefill tok/s @ 2048 tokens (LFM2-{args.shape.upper()} shape, bf16)",
                           "value": round(prefill["tokens_per_second"], 1), "unit": "tokens/s",
                           "ms": round(prefill["ms"], 4), "phase": "prefill",
                           "frac": round(flops / (prefill["ms"] * 1e-3) / PEAK_FLOPS["bf16"], 5)}))
@@ -129,7 +200,7 @@ def main() -> int:
 
     if args.phase == "decode" and args.batch != BATCH:
         result = decode(args.batch)
-        print(json.dumps({"metric": f"decode tok/s @ batch {args.batch} (LFM2-350M shape, bf16)",
+        print(json.dumps({"metric": f"decode tok/s @ batch {args.batch} (LFM2-{args.shape.upper()} shape, bf16)",
                           "value": round(result["tokens_per_second"], 1), "unit": "tokens/s",
                           "ms_per_step": round(result["ms_per_step"], 4), "phase": "decode"}))
         return 0
@@ -142,12 +213,12 @@ def main() -> int:
     step_bytes = w_bytes + kv_per_token * mean_context * BATCH
     achieved = step_bytes / (main_run["ms_per_step"] * 1e-3) / 1e9
     line = {
-        "metric": "decode tok/s @ batch 8 (LFM2-350M shape, bf16, context 2048+)",
+        "metric": f"decode tok/s @ batch 8 (LFM2-{args.shape.upper()} shape, bf16, context 2048+)",
         "value": round(main_run["tokens_per_second"], 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(main_run["ms_per_step"], 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"model": "LFM2-350M shape, random weights", "global_batch": BATCH,
+        "config": {"model": f"LFM2-{args.shape.upper()} shape, random weights", "global_batch": BATCH,
                    "seq_len": context, "prompt_tokens": PROMPT_TOKENS, "parallelism": "single GPU",
                    "layers": cfg["num_hidden_layers"], "layers_of_shape": full_layers,
                    "attention_layers": cfg["layer_types"].count("full_attention"),

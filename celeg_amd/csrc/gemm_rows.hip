@@ -1,0 +1,311 @@
+// bfloat16 products for 17 to 64 rows on gfx950 (decode steps of many requests, short
+// portions of prompts), with what surrounds them fused in, as for the products of up to
+// 16 rows:
+//   out[M,N] = epilogue(scale[m] * (A[M,K] W[N,K]^T) + bias)
+// A is bfloat16; behind an RMSNorm it is the bfloat16 copy of the residual stream, W has
+// the norm's weight folded in and scale[m] = rsqrt(mean(x_m^2) + eps) comes from the
+// partial sums of squares that the producer of the stream left.
+// Epilogues: store | 32-bit store | add into the 32-bit residual stream, refresh its
+// bfloat16 copy and leave partial sums of squares | SwiGLU of a gate and an up stream |
+// the double-gated short convolution of a B, a C and an x stream for one new token per
+// request, with its state update.
+//
+// Layout.  At these sizes the weights are read once from memory and the rows of A come
+// from cache.  A workgroup owns CT tiles of 16 columns (of every weight stream) over the
+// WHOLE of K, which its wavefronts split between them; a wavefront keeps
+// MT x (streams x CT) tiles of 16x16 sums, reads 16 bytes of weights per lane and tile for
+// 32 values of k and the rows of A straight into the instruction's operand layout (whole
+// runs of memory where A lies with its rows side by side inside every group of 8 values:
+// rows that lie one after the other cost a cache line per lane), and holds the loads of
+// the next 32 values in flight while it multiplies.  The wavefronts' tiles meet in LDS;
+// every thread then finishes outputs of one row, always adding in the same order, so a
+// result does not depend on what else is in the batch.  No workgroup needs another one's
+// sums.  (Cutting K across workgroups, with a second kernel that adds the slices, was
+// measured and gained nothing: narrow tiles and many wavefronts a workgroup were as fast
+// or faster at every size tried, 1024 to 14336 columns and 1024 to 7168 values of k.)
+//
+// Reference semantics of the fused parts: RMSNorm src/backend/cpu/kernels/elementwise.cpp:56-76,
+// SwiGLU elementwise.cpp:101-119, short convolution src/backend/cpu/kernels/convolution.cpp:7-28,
+// projections y = x W^T src/model/weight_plan.cpp:82-130; the reference fuses the residual
+// addition into its products with beta = 1 (src/backend/cuda/model/prefill_batched/non_attention.cpp:175-201).
+#include "common.h"
+#include "gemv_params.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+
+enum { E_STORE = 0, E_STORE_F32 = 1, E_RESIDUAL = 2, E_SWIGLU = 3, E_CONV = 4 };
+#define ROWS_MAX_TAPS 8
+#define ROWS_MAX_STAT_BLOCKS 512
+#define ROWS_MAX_LDS (128 * 1024)
+
+__device__ __forceinline__ float round_bf16(float x) { return to_float(from_float<bf16>(x)); }
+
+template <int EPI> struct Streams { static constexpr int n = 1; };
+template <> struct Streams<E_SWIGLU> { static constexpr int n = 2; };
+template <> struct Streams<E_CONV> { static constexpr int n = 3; };
+
+// Most wavefronts of a workgroup: what LDS holds of their tiles (a power of two, up to 16).
+constexpr int rows_max_waves(int mt, int sc) {
+    int w = 16;
+    while (w > 1 && w * mt * sc * 1024 + 256 > ROWS_MAX_LDS) w >>= 1;
+    return w;
+}
+
+// Finishes one output: row r, column n (both inside the sizes), from the sums of its weight
+// streams (scale and bias applied).  Returns the new value of the residual stream (E_RESIDUAL).
+template <int EPI>
+__device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n, const float* sum) {
+    const size_t o = static_cast<size_t>(r) * p.ldo + n;      // 32-bit outputs: rows one after the other
+    const size_t ob = static_cast<size_t>(r) * p.ldo + static_cast<size_t>(n >> 3) * p.out_k8_stride + (n & 7);
+    if (EPI == E_STORE) {
+        static_cast<bf16*>(p.out)[ob] = from_float<bf16>(sum[0]);
+    } else if (EPI == E_STORE_F32) {
+        static_cast<float*>(p.out)[o] = sum[0];
+    } else if (EPI == E_RESIDUAL) {
+        // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
+        const float v = static_cast<const float*>(p.out)[o] + round_bf16(sum[0]);
+        static_cast<float*>(p.out)[o] = v;
+        if (p.out_bf16)
+            static_cast<bf16*>(p.out_bf16)[static_cast<size_t>(r) * p.ld_bf16 + static_cast<size_t>(n >> 3) * p.bf16_k8_stride + (n & 7)] = from_float<bf16>(v);
+        return v;
+    } else if (EPI == E_SWIGLU) {
+        const float g = round_bf16(sum[0]), u = round_bf16(sum[1]);
+        static_cast<bf16*>(p.out)[ob] = from_float<bf16>((g / (1.0f + expf(-g))) * u);
+    } else if (EPI == E_CONV) {
+        const float bb = round_bf16(sum[0]), cc = round_bf16(sum[1]), xx = round_bf16(sum[2]);
+        const float bx = bb * xx;
+        float* state = p.state + static_cast<size_t>(p.seq_slot[r]) * p.state_slot_stride + n;
+        const float* taps = p.conv_w + static_cast<size_t>(n) * p.taps;
+        float conv = 0.f;
+        for (int tap = 0; tap + 1 < p.taps; ++tap) {
+            const float sv = state[static_cast<size_t>(tap + 1) * p.N];
+            conv = fmaf(taps[tap], sv, conv);
+            state[static_cast<size_t>(tap) * p.N] = sv;          // shift by one position
+        }
+        conv = fmaf(taps[p.taps - 1], bx, conv);
+        state[static_cast<size_t>(p.taps - 1) * p.N] = bx;
+        if (p.conv_b) conv += p.conv_b[n];
+        static_cast<bf16*>(p.out)[ob] = from_float<bf16>(cc * conv);
+    }
+    return 0.f;
+}
+
+// MT: tiles of 16 rows; CT: tiles of 16 columns per weight stream; blockDim.x / 64
+// wavefronts split K.  LDS: [waves][MT][streams * CT][4][64] floats, then MT*16 scales.
+template <int MT, int CT, int EPI>
+__global__ __launch_bounds__(64 * rows_max_waves(MT, Streams<EPI>::n * CT))
+void gemm_rows_kernel(const GemvParams p) {
+    constexpr int NS = Streams<EPI>::n;
+    constexpr int SC = NS * CT;
+    constexpr int COLS = CT * 16;
+    constexpr int ROWS = MT * 16;
+    extern __shared__ float smem[];
+    const int n_waves = blockDim.x >> 6;
+    float* const red = smem;
+    float* const s_scale = smem + static_cast<size_t>(n_waves) * MT * SC * 256;
+    // the wavefront's number as a scalar: the branches on its range of k are then uniform
+    // ones (the matrix instructions do not honour a lane mask)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int M = p.M, N = p.N, K = p.K;
+    const int n0 = blockIdx.x * COLS;
+    const int c16 = lane & 15, q = lane >> 4;
+
+    // ---- operands: A rows t*16 + c16, W columns n0 + ct*16 + c16 of every stream
+    const bf16* arow[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = min(t * 16 + c16, M - 1);
+        arow[t] = static_cast<const bf16*>(p.a) + static_cast<size_t>(p.rows ? p.rows[m] : m) * p.lda + q * p.a_k8_stride;
+    }
+    const bf16* wcol[SC];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+            wcol[s * CT + ct] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + ct * 16 + c16, N - 1)) * p.w_row_stride + q * p.w_q_stride;
+    const int nkb = K >> 5;                    // K % 32 == 0 (checked by the host)
+    const int kb_begin = wave * nkb / n_waves, kb_end = (wave + 1) * nkb / n_waves;
+
+    floatx4_t acc[MT][SC];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int s = 0; s < SC; ++s) acc[t][s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    bf16x8_t a0[MT], w0[SC], a1[MT], w1[SC];
+    auto fetch = [&](int kb, bf16x8_t (&av)[MT], bf16x8_t (&wv)[SC]) {
+#pragma unroll
+        for (int s = 0; s < SC; ++s)
+            wv[s] = *reinterpret_cast<const bf16x8_t*>(wcol[s] + static_cast<size_t>(kb) * p.w_kb_stride);
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+            av[t] = *reinterpret_cast<const bf16x8_t*>(arow[t] + static_cast<size_t>(kb) * 4 * p.a_k8_stride);
+    };
+    auto multiply = [&](const bf16x8_t (&av)[MT], const bf16x8_t (&wv)[SC]) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int s = 0; s < SC; ++s)
+                acc[t][s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[t], wv[s], acc[t][s], 0, 0, 0);
+    };
+    if (kb_begin < kb_end) fetch(kb_begin, a0, w0);
+    if (kb_begin + 1 < kb_end) fetch(kb_begin + 1, a1, w1);
+
+    // ---- the rows' 1/rms from the partial sums of squares (asked for behind the first
+    // weights, used at the end): LPR neighbouring threads share a row
+    if (p.stats) {
+        const int lpr = blockDim.x / ROWS;           // a power of two, 1 .. 32
+        const int r = threadIdx.x / lpr, sub = threadIdx.x % lpr;
+        const int nb = p.n_stat_blocks;
+        const int m = min(r, M - 1);
+        const float* srow = p.stats + static_cast<size_t>(p.rows ? p.rows[m] : m) * p.stats_ld;
+        float ssq = 0.f;
+        for (int b0 = 0; b0 < nb; b0 += 8 * lpr) {   // the same trips for every thread
+            float part[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) part[i] = srow[min(b0 + sub + lpr * i, nb - 1)];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ssq += b0 + sub + lpr * i < nb ? part[i] : 0.f;
+        }
+        for (int off = lpr >> 1; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
+        if (sub == 0) s_scale[r] = 1.0f / sqrtf(ssq / static_cast<float>(K) + p.eps);
+    }
+
+    for (int kb = kb_begin; kb < kb_end; kb += 2) {
+        multiply(a0, w0);
+        if (kb + 2 < kb_end) fetch(kb + 2, a0, w0);
+        if (kb + 1 < kb_end) multiply(a1, w1);
+        if (kb + 3 < kb_end) fetch(kb + 3, a1, w1);
+    }
+
+    // acc[t][s]: lane l holds column l%16 of rows 4*(l/16)..+3 of the tile
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int s = 0; s < SC; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                red[(((static_cast<size_t>(wave) * MT + t) * SC + s) * 4 + i) * 64 + lane] = acc[t][s][i];
+    __syncthreads();
+
+    // ---- thread e takes row e / COLS, column e % COLS of the workgroup's tile
+    const int n_threads = blockDim.x;
+    for (int e = threadIdx.x; e < ROWS * COLS; e += n_threads) {
+        const int r = e / COLS, j = e % COLS;
+        const int t = r >> 4, rr = r & 15, ct = j >> 4, jj = j & 15;
+        const int src = jj + 16 * (rr >> 2), reg = rr & 3;
+        const int n = n0 + j;
+        const bool ok = r < M && n < N;
+        const int rc = min(r, M - 1), nc = min(n, N - 1);
+        float sum[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            float v = 0.f;
+            for (int w = 0; w < n_waves; ++w)
+                v += red[(((static_cast<size_t>(w) * MT + t) * SC + s * CT + ct) * 4 + reg) * 64 + src];
+            sum[s] = v;
+        }
+        const float scale = p.stats ? s_scale[r] : 1.f;
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            sum[s] = sum[s] * scale + (p.bias ? p.bias[static_cast<size_t>(s) * p.stream_rows + nc] : 0.f);
+        float v = 0.f;
+        if (ok) v = finish_output<EPI>(p, rc, nc, sum);
+        if (EPI == E_RESIDUAL && p.stats_out) {
+            float sq = v * v;               // the COLS columns of a row sit in COLS neighbouring lanes
+#pragma unroll
+            for (int off = COLS / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
+            if (j == 0 && r < M) p.stats_out[static_cast<size_t>(r) * p.stats_ld_out + blockIdx.x] = sq;
+        }
+    }
+}
+
+// The shape of the work for these sizes: narrow tiles, so that there are many workgroups
+// (wide ones only where even they give thousands, as for an output head), and as many
+// wavefronts as LDS holds tiles of and as still have two blocks of 32 each.
+struct RowsShape {
+    int mt, ct, waves;
+};
+
+static int g_force_ct = 0, g_force_waves = 0;   // tuning aids: override the choice below where they fit
+extern "C" void celeg_gemm_rows_force(int ct, int waves) { g_force_ct = ct; g_force_waves = waves; }
+
+static RowsShape rows_shape(int M, int N, int K, int streams) {
+    RowsShape s;
+    s.mt = M <= 32 ? 2 : 4;
+    const int max_ct = streams == 1 ? 4 : (streams == 2 ? 2 : 1);
+    s.ct = 1;
+    while (s.ct < max_ct && (N + 32 * s.ct - 1) / (32 * s.ct) >= 1024) s.ct *= 2;
+    if (g_force_ct > 0 && g_force_ct <= max_ct) s.ct = g_force_ct;
+    const int nkb = K / 32;
+    s.waves = rows_max_waves(s.mt, streams * s.ct);
+    while (s.waves > 1 && s.waves * 2 > nkb) s.waves >>= 1;
+    if (g_force_waves > 0 && g_force_waves <= rows_max_waves(s.mt, streams * s.ct)) s.waves = g_force_waves;
+    return s;
+}
+
+template <int MT, int CT, int EPI>
+static int launch_rows(const GemvParams& p, int waves, hipStream_t stream) {
+    constexpr int NS = Streams<EPI>::n;
+    const size_t lds = static_cast<size_t>(waves) * MT * NS * CT * 1024 + MT * 16 * sizeof(float);
+    static bool raised = false;              // once per instantiation: more LDS than the default limit
+    if (lds > 48 * 1024 && !raised) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_kernel<MT, CT, EPI>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, ROWS_MAX_LDS);
+        if (err != hipSuccess) return static_cast<int>(err);
+        raised = true;
+    }
+    dim3 grid((p.N + CT * 16 - 1) / (CT * 16)), block(waves * 64);
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p);
+    return CELEG_LAUNCH_RESULT();
+}
+
+template <int EPI>
+static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
+    constexpr int NS = Streams<EPI>::n;
+    const RowsShape s = rows_shape(p.M, p.N, p.K, NS);
+#define ROWS_CASE(MT_, CT_) \
+    if (s.mt == MT_ && s.ct == CT_) return launch_rows<MT_, CT_, EPI>(p, s.waves, stream);
+    ROWS_CASE(2, 1) ROWS_CASE(4, 1)
+    if constexpr (NS <= 2) { ROWS_CASE(2, 2) ROWS_CASE(4, 2) }
+    if constexpr (NS == 1) { ROWS_CASE(2, 4) ROWS_CASE(4, 4) }
+#undef ROWS_CASE
+    return static_cast<int>(hipErrorInvalidValue);
+}
+
+static int streams_of(int epi) { return epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3 : 1); }
+
+// Number of workgroups for these sizes, which is also the number of partial sums of
+// squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
+extern "C" int celeg_gemm_rows_blocks(int M, int N, int K, int epi) {
+    const RowsShape s = rows_shape(M, N, K, streams_of(epi));
+    return (N + s.ct * 16 - 1) / (s.ct * 16);
+}
+
+// 16 < M <= 64 (fewer rows work too, at the cost of idle lanes), K % 32 == 0, bfloat16 a and
+// w (in the layouts that the strides describe).  The fields of GemvParams that are read are
+// those of the products for up to 16 rows and the strides of the operands' groups of 8.
+extern "C" int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t stream) {
+    const GemvParams& p = *params;
+    if (p.M <= 0 || p.N <= 0) return 0;
+    if (p.M > 64 || p.K <= 0 || (p.K % 32) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
+    if ((p.w_row_stride % 8) || (p.w_kb_stride % 8) || (p.w_q_stride % 8) || p.w_row_stride <= 0 ||
+        p.w_kb_stride <= 0 || p.w_q_stride <= 0)
+        return static_cast<int>(hipErrorInvalidValue);
+    if ((p.a_k8_stride % 8) || p.a_k8_stride <= 0 || (p.out_k8_stride % 8) || p.out_k8_stride <= 0 ||
+        (p.out_bf16 && ((p.bf16_k8_stride % 8) || p.bf16_k8_stride <= 0)))
+        return static_cast<int>(hipErrorInvalidValue);
+    if (p.stats && (p.n_stat_blocks < 1 || p.n_stat_blocks > ROWS_MAX_STAT_BLOCKS))
+        return static_cast<int>(hipErrorInvalidValue);
+    if (epi == E_CONV && (p.taps < 1 || p.taps > ROWS_MAX_TAPS || p.stream_rows != p.N))
+        return static_cast<int>(hipErrorInvalidValue);
+    switch (epi) {
+        case E_STORE: return launch_epilogue<E_STORE>(p, stream);
+        case E_STORE_F32: return launch_epilogue<E_STORE_F32>(p, stream);
+        case E_RESIDUAL: return launch_epilogue<E_RESIDUAL>(p, stream);
+        case E_SWIGLU: return launch_epilogue<E_SWIGLU>(p, stream);
+        case E_CONV: return launch_epilogue<E_CONV>(p, stream);
+        default: return static_cast<int>(hipErrorInvalidValue);
+    }
+}

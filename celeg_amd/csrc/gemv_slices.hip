@@ -300,34 +300,37 @@ extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t 
 // Prepares a 32-bit stream for products behind a norm: its bfloat16 copy and every row's
 // sum of squares (one partial sum a row: stats[row * stats_ld]).  Used where the stream was written by
 // something that leaves neither.
+// (xb: element (row, i) at row * ldx + (i / 8) * xb_k8 + i % 8; rows one after the other: xb_k8 = 8)
 __global__ void stream_prepare_kernel(const float* __restrict__ h, int ldh, bf16* __restrict__ xb,
-                                      int ldx, float* __restrict__ stats, int stats_ld, int width) {
+                                      int ldx, long long xb_k8, float* __restrict__ stats, int stats_ld,
+                                      int width) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const float* src = h + static_cast<size_t>(row) * ldh;
     float s = 0.f;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         const float v = src[i];
-        xb[static_cast<size_t>(row) * ldx + i] = from_float<bf16>(v);
+        xb[static_cast<size_t>(row) * ldx + static_cast<size_t>(i >> 3) * xb_k8 + (i & 7)] = from_float<bf16>(v);
         s += v * v;
     }
     s = block_sum(s, scratch);
     if (threadIdx.x == 0) stats[static_cast<size_t>(row) * stats_ld] = s;
 }
 
-extern "C" int celeg_stream_prepare(const float* h, int ldh, void* xb, int ldx, float* stats,
-                                    int stats_ld, int rows, int width, hipStream_t stream) {
+extern "C" int celeg_stream_prepare(const float* h, int ldh, void* xb, int ldx, long long xb_k8,
+                                    float* stats, int stats_ld, int rows, int width, hipStream_t stream) {
     if (rows <= 0) return 0;
     hipLaunchKernelGGL(stream_prepare_kernel, dim3(rows), dim3(256), 0, stream, h, ldh,
-                       static_cast<bf16*>(xb), ldx, stats, stats_ld, width);
+                       static_cast<bf16*>(xb), ldx, xb_k8, stats, stats_ld, width);
     return CELEG_LAUNCH_RESULT();
 }
 
 // Embedding gather into the 32-bit stream, its bfloat16 copy and the rows' sums of squares:
 // out[row, :] = table[ids[row], :], stats[row * stats_ld] = sum(out[row, :]^2).
 __global__ void embed_stream_kernel(const bf16* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ out, bf16* __restrict__ xb,
-                                    float* __restrict__ stats, int stats_ld, int width, int vocab) {
+                                    float* __restrict__ out, bf16* __restrict__ xb, int ldx,
+                                    long long xb_k8, float* __restrict__ stats, int stats_ld,
+                                    int width, int vocab) {
     __shared__ float scratch[16];
     const int row = blockIdx.x;
     const int id = ids[row];
@@ -338,19 +341,19 @@ __global__ void embed_stream_kernel(const bf16* __restrict__ table, const int* _
         const bf16 raw = ok ? src[i] : bf16{0};
         const float v = to_float(raw);
         out[static_cast<size_t>(row) * width + i] = v;
-        xb[static_cast<size_t>(row) * width + i] = raw;
+        xb[static_cast<size_t>(row) * ldx + static_cast<size_t>(i >> 3) * xb_k8 + (i & 7)] = raw;
         s += v * v;
     }
     s = block_sum(s, scratch);
     if (threadIdx.x == 0) stats[static_cast<size_t>(row) * stats_ld] = s;
 }
 
-extern "C" int celeg_embed_stream(const void* table, const int* ids, float* out, void* xb,
-                                  float* stats, int stats_ld, int rows, int width, int vocab,
-                                  hipStream_t stream) {
+extern "C" int celeg_embed_stream(const void* table, const int* ids, float* out, void* xb, int ldx,
+                                  long long xb_k8, float* stats, int stats_ld, int rows, int width,
+                                  int vocab, hipStream_t stream) {
     if (rows <= 0) return 0;
     hipLaunchKernelGGL(embed_stream_kernel, dim3(rows), dim3(256), 0, stream,
-                       static_cast<const bf16*>(table), ids, out, static_cast<bf16*>(xb), stats,
-                       stats_ld, width, vocab);
+                       static_cast<const bf16*>(table), ids, out, static_cast<bf16*>(xb), ldx, xb_k8,
+                       stats, stats_ld, width, vocab);
     return CELEG_LAUNCH_RESULT();
 }

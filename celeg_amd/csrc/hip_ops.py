@@ -50,6 +50,7 @@ class HipOps:
         self._rope_tables = {}
         self.use_rope_table = True         # cos/sin of every position from a table made once
         self.use_sliced = True             # up to 16 bfloat16 rows: the k-sliced kernels
+        self.use_rows_kernel = True        # 17 to 64 bfloat16 rows: the kernel that streams the weights
         self.last_stat_blocks = 0
         self.fused_linear_shape = 0        # 0: chosen from the sizes; 1..4 force a workgroup shape
 
@@ -90,6 +91,25 @@ class HipOps:
         if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
             raise KernelError(f"{name} must be 2-D with dense rows")
         return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+    def _operand(self, t: torch.Tensor, name: str):
+        """(rows, width, row stride, stride of a group of 8 values) of a bfloat16 operand:
+        [rows, width] with dense rows, or [rows, width/8, 8], a view of a buffer in which the
+        rows lie side by side inside every group of 8 values (``chunked_rows``)."""
+        if t.dim() == 2:
+            return t.shape[0], t.shape[1], self._rows(t, name), 8
+        if t.dim() != 3 or t.shape[2] != 8 or t.stride(2) != 1:
+            raise KernelError(f"{name} must be [rows, width] or [rows, width/8, 8]")
+        return t.shape[0], t.shape[1] * 8, t.stride(0), t.stride(1)
+
+    @staticmethod
+    def chunked_rows(rows: int, width: int, device, max_rows: int = 64) -> torch.Tensor:
+        """Room for ``rows`` bfloat16 rows of ``width`` values in the layout that the products
+        for 17 to 64 rows read best: [width/8, max_rows, 8], returned as its view
+        [rows, width/8, 8] (element (m, k) at [m, k // 8, k % 8])."""
+        if width % 8 or rows > max_rows:
+            raise KernelError("chunked_rows: the width must be a multiple of 8 and rows <= max_rows")
+        return torch.empty(width // 8, max_rows, 8, dtype=torch.bfloat16, device=device).permute(1, 0, 2)[:rows]
 
     def _dtype(self, t: torch.Tensor, name: str) -> int:
         if t.dtype not in _DT:
@@ -320,17 +340,25 @@ class HipOps:
                 and self._rows(q, "q") % 8 == 0:
             if batch.decode_only and head_dim in (64, 128) and batch.n_seqs == T:
                 return self._attention_decode(q, out, heads, kv_heads, head_dim, scale, window,
-                                              batch, kv)
+                                              batch, kv, T)
             if head_dim in (32, 64, 96, 128):
-                code = self._lib("attention_fast").celeg_attention_rows_bf16(
-                    _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v), _ptr(kv.table),
-                    _c_int(kv.table.shape[1]), _ptr(batch.cu_seqlens), _ptr(batch.seq_slot),
-                    _ptr(batch.seq_start), _c_int(batch.n_seqs), _c_int(T), _ptr(out),
-                    _c_int(heads * head_dim), _c_int(heads), _c_int(kv_heads), _c_int(head_dim),
-                    _c_int(kv.page_tokens), _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
-                    _c_int(window if window else 0), _c_int(self.attention_rows_per_tile),
-                    self._stream())
-                self._check(code, "attention over rows (bfloat16)")
+                # entries of one token lie first: they go to the kernel for single rows (a
+                # tile of the rows kernel would hold one row), the portions to the rows kernel
+                single = batch.single_rows if head_dim in (64, 128) else 0
+                if single:
+                    self._attention_decode(q, out, heads, kv_heads, head_dim, scale, window,
+                                           batch, kv, single)
+                if single < batch.n_seqs:
+                    code = self._lib("attention_fast").celeg_attention_rows_bf16(
+                        _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v), _ptr(kv.table),
+                        _c_int(kv.table.shape[1]), _ptr(batch.cu_seqlens[single:]),
+                        _ptr(batch.seq_slot[single:]), _ptr(batch.seq_start[single:]),
+                        _c_int(batch.n_seqs - single), _c_int(T - single), _ptr(out),
+                        _c_int(heads * head_dim), _c_int(heads), _c_int(kv_heads), _c_int(head_dim),
+                        _c_int(kv.page_tokens), _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
+                        _c_int(window if window else 0), _c_int(self.attention_rows_per_tile),
+                        self._stream())
+                    self._check(code, "attention over rows (bfloat16)")
                 return
         code = self._lib("attention").celeg_paged_attention(
             _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v),
@@ -341,8 +369,8 @@ class HipOps:
             _c_int(window if window else 0), self._stream())
         self._check(code, "paged_attention")
 
-    def _attention_decode(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv):
-        T = q.shape[0]
+    def _attention_decode(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv, T):
+        """The first ``T`` rows of the step, each the one new token of its request."""
         max_context = kv.table.shape[1] * kv.page_tokens
         n_splits = (max_context + 63) // 64          # the kernel takes 64 keys a wavefront
         need = T * heads * n_splits * (head_dim + 2)
@@ -416,7 +444,15 @@ class HipOps:
         if rows <= 16 and self.use_sliced:
             return int(self._lib("gemv_slices").celeg_gemv_slices_blocks(
                 _c_int(rows), _c_int(n), _c_int(k)))
+        if self.rows_kernel_ok(rows, k):
+            return int(self._lib("gemm_rows").celeg_gemm_rows_blocks(
+                _c_int(rows), _c_int(n), _c_int(k), _c_int(self._EPILOGUES["residual"])))
         return (n + 15) // 16
+
+    def rows_kernel_ok(self, rows: int, *inner_sizes: int) -> bool:
+        """Whether bfloat16 products of ``rows`` rows with these inner sizes go to the kernel
+        for 17 to 64 rows."""
+        return self.use_rows_kernel and 16 < rows <= 64 and all(k % 32 == 0 for k in inner_sizes)
 
     @staticmethod
     def pack_weight(w: torch.Tensor) -> torch.Tensor:
@@ -434,25 +470,28 @@ class HipOps:
         self._dev(h, "h", torch.float32, contiguous=False); self._dev(xb, "xb", torch.bfloat16, contiguous=False)
         self._dev(stats, "stats", torch.float32)
         rows, width = h.shape
-        if xb.shape[0] < rows or xb.shape[1] != width or stats.shape[0] < rows:
+        xb_rows, xb_width, ldx, xb_k8 = self._operand(xb, "xb")
+        if xb_rows < rows or xb_width != width or stats.shape[0] < rows:
             raise KernelError("stream_prepare: shapes do not fit")
         code = self._lib("gemv_slices").celeg_stream_prepare(
-            _ptr(h), _c_int(self._rows(h, "h")), _ptr(xb), _c_int(self._rows(xb, "xb")), _ptr(stats),
-            _c_int(stats.stride(0)), _c_int(rows), _c_int(width), self._stream())
+            _ptr(h), _c_int(self._rows(h, "h")), _ptr(xb), _c_int(ldx), ctypes.c_longlong(xb_k8),
+            _ptr(stats), _c_int(stats.stride(0)), _c_int(rows), _c_int(width), self._stream())
         self._check(code, "stream_prepare")
 
     def embed_stream(self, table, token_ids, out, xb, stats):
         """Embedding gather into the 32-bit stream ``out``, its bfloat16 copy ``xb`` and the
         rows' sums of squares (``stats[:rows, 0]``)."""
         self._dev(table, "table", torch.bfloat16); self._dev(token_ids, "token_ids", torch.int32)
-        self._dev(out, "out", torch.float32); self._dev(xb, "xb", torch.bfloat16)
+        self._dev(out, "out", torch.float32); self._dev(xb, "xb", torch.bfloat16, contiguous=False)
         self._dev(stats, "stats", torch.float32)
         rows, width = out.shape
+        xb_rows, xb_width, ldx, xb_k8 = self._operand(xb, "xb")
         if table.shape[1] != width or token_ids.numel() != rows or stats.shape[0] < rows \
-                or xb.shape != out.shape:
+                or (xb_rows, xb_width) != (rows, width):
             raise KernelError("embed_stream: shapes do not fit")
         code = self._lib("gemv_slices").celeg_embed_stream(
-            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(xb), _ptr(stats), _c_int(stats.stride(0)),
+            _ptr(table), _ptr(token_ids), _ptr(out), _ptr(xb), _c_int(ldx), ctypes.c_longlong(xb_k8),
+            _ptr(stats), _c_int(stats.stride(0)),
             _c_int(rows), _c_int(width), _c_int(table.shape[0]), self._stream())
         self._check(code, "embed_stream")
 
@@ -483,7 +522,8 @@ class HipOps:
         (``w`` is [3N, K]: B, C, x rows; ``conv`` = (taps [N, L], bias or None, state
         [slots, L, N], seq_slot [M]); one new token per request).
 
-        Up to 16 bfloat16 rows go to the k-sliced kernels, which also take the form behind a
+        Up to 16 bfloat16 rows go to the k-sliced kernels, and 17 to 64 rows with an inner size
+        that is a multiple of 32 to the kernel that streams the weights.  Both also take the form behind a
         norm whose weight the caller has folded into ``w``: ``a`` is then the bfloat16 copy
         of the stream and ``stats[row, :stat_blocks]`` its partial sums of squares, from which
         the rows' 1/rms (with ``eps``) scales the sums; their "residual" epilogue refreshes
@@ -505,8 +545,8 @@ class HipOps:
             raise KernelError(f"fused_linear: {M} rows with inner size {K} are not supported "
                               "(1..64 rows, inner size a multiple of 8)")
         self._dev(a, "a", contiguous=False)
-        lda = self._rows(a, "a")
-        if a.shape[1] != K or (rows is None and a.shape[0] < M):
+        a_rows, a_width, lda, a_k8 = self._operand(a, "a")
+        if a_width != K or (rows is None and a_rows < M):
             raise KernelError("fused_linear: a does not fit the weights")
         if norm_weight is not None:
             if a.dtype != torch.float32:
@@ -519,7 +559,8 @@ class HipOps:
         else:
             if a.dtype != torch.bfloat16:
                 raise KernelError("fused_linear: rows must be bfloat16 (or 32-bit with a norm weight)")
-            if (epilogue in ("swiglu", "conv") or stat_blocks > 0) and not (M <= 16 and self.use_sliced):
+            if (epilogue in ("swiglu", "conv") or stat_blocks > 0) \
+                    and not (M <= 16 and self.use_sliced) and not self.rows_kernel_ok(M, K):
                 raise KernelError("fused_linear: this combination is not built")
         if lda % 8:
             raise KernelError("fused_linear: the row stride of a must be a multiple of 8")
@@ -527,7 +568,8 @@ class HipOps:
             self._dev(rows, "rows", torch.int32)
         out_dtype = torch.float32 if epilogue in ("store_f32", "residual") else torch.bfloat16
         self._dev(out, "out", out_dtype, contiguous=False)
-        if out.shape[0] < M or out.shape[1] != N:
+        out_rows, out_width, ldo, out_k8 = self._operand(out, "out")
+        if out_rows < M or out_width != N:
             raise KernelError(f"fused_linear: out must be [{M}, {N}], got {tuple(out.shape)}")
         if bias is not None:
             self._dev(bias, "bias", torch.float32)
@@ -546,21 +588,30 @@ class HipOps:
         prm.w, prm.stream_rows = w.data_ptr(), N
         prm.bias = bias.data_ptr() if bias is not None else None
         prm.M, prm.N, prm.K = M, N, K
-        prm.out, prm.ldo = out.data_ptr(), self._rows(out, "out")
+        prm.out, prm.ldo = out.data_ptr(), ldo
         sliced = norm_weight is None and M <= 16 and self.use_sliced
-        if packed and not sliced:
-            raise KernelError("fused_linear: packed weights go with bfloat16 rows, up to 16 of them")
+        streamed = norm_weight is None and not sliced and self.rows_kernel_ok(M, K)
+        prm.a_k8_stride, prm.out_k8_stride, prm.w_q_stride = a_k8, out_k8, 8
+        if (a.dim() == 3 or out.dim() == 3 or (out_bf16 is not None and out_bf16.dim() == 3)) \
+                and not streamed:
+            raise KernelError("fused_linear: operands with the rows side by side go with 17 to 64 rows")
+        if out.dim() == 3 and out_dtype != torch.bfloat16:
+            raise KernelError("fused_linear: a 32-bit output has its rows one after the other")
+        if packed and not (sliced or streamed):
+            raise KernelError("fused_linear: packed weights go with bfloat16 rows")
         prm.w_row_stride, prm.w_kb_stride = (32, w_rows * 32) if packed else (K, 32)
         if out_bf16 is not None:
-            if not (sliced and epilogue == "residual"):
-                raise KernelError("fused_linear: out_bf16 goes with the residual epilogue for up to 16 rows")
+            if not ((sliced or streamed) and epilogue == "residual"):
+                raise KernelError("fused_linear: out_bf16 goes with the residual epilogue of bfloat16 rows")
             self._dev(out_bf16, "out_bf16", torch.bfloat16, contiguous=False)
-            if out_bf16.shape[0] < M or out_bf16.shape[1] != N:
+            b_rows, b_width, ld_bf16, bf16_k8 = self._operand(out_bf16, "out_bf16")
+            if b_rows < M or b_width != N:
                 raise KernelError("fused_linear: out_bf16 does not fit")
-            prm.out_bf16, prm.ld_bf16 = out_bf16.data_ptr(), self._rows(out_bf16, "out_bf16")
+            prm.out_bf16, prm.ld_bf16, prm.bf16_k8_stride = out_bf16.data_ptr(), ld_bf16, bf16_k8
         if epilogue == "residual":
             # partial sums of squares: one per workgroup and row
-            self.last_stat_blocks = self.residual_stat_blocks(M, N, K) if sliced else (N + 15) // 16
+            self.last_stat_blocks = self.residual_stat_blocks(M, N, K) if sliced or streamed \
+                else (N + 15) // 16
         if epilogue == "residual" and stats_out is not None:
             self._dev(stats_out, "stats_out", torch.float32)
             if stats_out.shape[1] < self.last_stat_blocks or stats_out.shape[0] < M:
@@ -585,6 +636,11 @@ class HipOps:
                 ctypes.byref(prm), _c_int(self._EPILOGUES[epilogue]), self._stream())
             self._check(code, f"fused_linear ({epilogue}, k-sliced)")
             return out
+        if streamed:
+            code = self._lib("gemm_rows").celeg_gemm_rows(
+                ctypes.byref(prm), _c_int(self._EPILOGUES[epilogue]), self._stream())
+            self._check(code, f"fused_linear ({epilogue}, 17 to 64 rows)")
+            return out
         code = self._lib("gemv_fused").celeg_gemv_fused(
             ctypes.byref(prm), _c_int(1 if norm_weight is not None else 0),
             _c_int(self._EPILOGUES[epilogue]), _c_int(self.fused_linear_shape), self._stream())
@@ -606,4 +662,6 @@ class _GemvParams(ctypes.Structure):
         ("state_slot_stride", ctypes.c_size_t), ("seq_slot", ctypes.c_void_p), ("taps", ctypes.c_int),
         ("out_bf16", ctypes.c_void_p), ("ld_bf16", ctypes.c_int),
         ("w_row_stride", ctypes.c_longlong), ("w_kb_stride", ctypes.c_longlong),
+        ("a_k8_stride", ctypes.c_longlong), ("out_k8_stride", ctypes.c_longlong),
+        ("bf16_k8_stride", ctypes.c_longlong), ("w_q_stride", ctypes.c_longlong),
     ]

@@ -32,9 +32,10 @@ class StepEntry:
 class StepBatch:
     """Device views (int32) into the packed buffer, plus host-side facts.
 
-    token_ids[T], positions[T], token_seq[T] (which entry a row belongs to),
+    token_ids[T], positions[T], token_seq[T] (which sequence a row belongs to),
     token_slot[T] (that entry's cache slot), cu_seqlens[S+1] (row offsets of the
-    entries), seq_slot[S], seq_start[S] (position of the entry's first row),
+    sequences), seq_slot[S], seq_start[S] (position of the sequence's first row),
+    the sequences being the entries with those of a single token moved to the front,
     logit_rows[R] (rows whose logits are wanted), table_updates[g] ([1 + 3*cap]:
     a count, then (slot, logical page, physical page) triples) per cache group.
     """
@@ -47,6 +48,8 @@ class StepBatch:
         self.max_seg_len = 0
         self.max_context_len = 0
         self.decode_only = False
+        self.single_rows = 0      # rows [0, single_rows) are entries of one token each
+        self.entry_order: List[int] = []   # which entry each sequence of the layout is
         self.token_ids = self.positions = self.token_seq = self.token_slot = None
         self.cu_seqlens = self.seq_slot = self.seq_start = self.logit_rows = None
         self.table_updates: List[Optional[torch.Tensor]] = []
@@ -104,17 +107,26 @@ class BatchBuilder:
         T_real = S_real if decode_only else int(sum(seg_lens))
         S = S_real if pad_to is None else pad_to
         T = T_real if pad_to is None else pad_to
+        # Rows are laid out with the entries of a single token first (their order kept), so
+        # that kernels made for single rows can take them as one range also beside portions
+        # of prompts; logits still come back in the order of the entries.
+        order = list(range(S_real)) if decode_only else \
+            sorted(range(S_real), key=lambda i: seg_lens[i] != 1)
+        single_rows = S_real if decode_only else sum(1 for n in seg_lens if n == 1)
         if pad_to is not None:
             want_rows = list(range(T))
         else:
-            want_rows = []
+            first_row = [0] * S_real
             row = 0
-            for e, n in zip(entries, seg_lens):
+            for i in order:
+                first_row[i] = row
+                row += seg_lens[i]
+            want_rows = []
+            for i, (e, n) in enumerate(zip(entries, seg_lens)):
                 for w in e.want:
                     if not 0 <= int(w) < n:
                         raise ValueError(f"wanted place {w} is outside the entry's {n} tokens")
-                    want_rows.append(row + int(w))
-                row += n
+                    want_rows.append(first_row[i] + int(w))
         R = len(want_rows)
         if update_caps is None:
             update_caps = [len(u) for u in updates]
@@ -158,7 +170,7 @@ class BatchBuilder:
         else:
             row = 0
             cu[0] = 0
-            for i, (e, n) in enumerate(zip(entries, seg_lens)):
+            for i, (e, n) in enumerate((entries[j], seg_lens[j]) for j in order):
                 token_ids[row:row + n] = e.tokens
                 positions[row:row + n] = self._iota[e.start_pos:e.start_pos + n] \
                     if e.start_pos + n <= self._iota.size else np.arange(e.start_pos, e.start_pos + n)
@@ -186,6 +198,8 @@ class BatchBuilder:
         b.max_seg_len = max(seg_lens) if seg_lens else 0
         b.max_context_len = max((e.start_pos + n for e, n in zip(entries, seg_lens)), default=0)
         b.decode_only = decode_only
+        b.single_rows = S if decode_only else single_rows
+        b.entry_order = order
 
         def dev(name):       # the same views of the device buffer for the same layout
             view = views.get(name)
@@ -200,7 +214,7 @@ class BatchBuilder:
         b.logit_rows = dev("logit_rows")
         b.table_updates = [dev(f"updates{g}") for g in range(len(updates))]
         b.table_update_caps = list(update_caps)
-        b.host = {"seg_lens": np.asarray(seg_lens + [1] * (S - S_real), dtype=np.int32),
+        b.host = {"seg_lens": np.asarray([seg_lens[j] for j in order] + [1] * (S - S_real), dtype=np.int32),
                   "seq_slot": seq_slot.copy(), "seq_start": seq_start.copy(),
                   "cu_seqlens": cu.copy(), "want_rows": np.asarray(want_rows, dtype=np.int32)}
         return b

@@ -34,7 +34,7 @@ class TokenEmbedding(Embedding):
                 and fused_rows_ok(rt, batch, self.width):
             # few rows: leave every row's sum of squares (and the bfloat16 copy of the
             # stream) for the first norm
-            if _sliced(rt, out.shape[0]):
+            if _sliced(rt, out.shape[0], self.width):
                 rt.ops.embed_stream(self.table, token_ids, out,
                                     stream_bf16(rt, out.shape[0], self.width),
                                     stream_stats(rt, self.width))

@@ -8,7 +8,7 @@ from __future__ import annotations
 import torch
 
 from .base import FeedForward, WeightSpec, register_part
-from .fused import fused_rows_ok, linear_into_stream, norm_linear
+from .fused import fused_rows_ok, linear_into_stream, norm_linear, operand_rows
 
 
 class SwiGlu(FeedForward):
@@ -51,7 +51,7 @@ class SwiGlu(FeedForward):
         if not fused_rows_ok(rt, batch, self.width, self.ff) \
                 or (self.w_gate_up.dtype, self.w_down.dtype) != (rt.dtype,) * 2:
             return False
-        act = rt.ws.buf("ffn_act", (batch.n_tokens, self.ff), rt.dtype)
+        act = operand_rows(rt, "ffn_act_fused", batch.n_tokens, self.ff, self.width)
         norm_linear(rt, h, norm, self.w_gate_up, act, epilogue="swiglu")
         linear_into_stream(rt, act, self.w_down, h)
         return True

@@ -15,20 +15,26 @@ from __future__ import annotations
 import torch
 
 STAT_COLUMNS = 64   # most rows of a fused step (rows of the partial-sum table)
-# Above this many rows the library's product (with separate norm and activation kernels)
-# is the faster one on MI355X (measured on the 1024-wide shape: 32 rows fused 1.28 ms a
-# step against 1.37 ms, 64 rows 2.28 ms against 1.67 ms).
-FUSED_MAX_ROWS = 32
+# Most rows of the fused path: 64 where every inner size is a multiple of 32 (the kernel
+# for 17 to 64 rows); else 32, above which the library's product (with separate norm and
+# activation kernels) is the faster one on MI355X.
+FUSED_MAX_ROWS = 64
+FUSED_MAX_ROWS_OLD_KERNEL = 32
 
 
 def fused_rows_ok(rt, batch, *inner_sizes) -> bool:
     """Whether this step's rows can take the fused path through products with these
     inner sizes."""
     ops = rt.ops
-    return (rt.dtype == torch.bfloat16 and getattr(ops, "has_fused_linear", False)
-            and getattr(rt, "use_fused", True)
-            and batch.n_tokens <= getattr(rt, "fused_max_rows", FUSED_MAX_ROWS)
-            and ops.fused_linear_ok(batch.n_tokens, *inner_sizes))
+    rows = batch.n_tokens
+    if not (rt.dtype == torch.bfloat16 and getattr(ops, "has_fused_linear", False)
+            and getattr(rt, "use_fused", True) and ops.fused_linear_ok(rows, *inner_sizes)):
+        return False
+    limit = getattr(rt, "fused_max_rows", None)
+    if limit is None:
+        streamed = hasattr(ops, "rows_kernel_ok") and ops.rows_kernel_ok(rows, *inner_sizes)
+        limit = FUSED_MAX_ROWS if streamed else FUSED_MAX_ROWS_OLD_KERNEL
+    return rows <= limit
 
 
 SLICED_MAX_ROWS = 16      # rows of the k-sliced kernels
@@ -41,13 +47,36 @@ def stream_stats(rt, width: int) -> torch.Tensor:
     return rt.ws.buf("stream_stats", (STAT_COLUMNS, (width + 3) // 4), torch.float32)
 
 
+def _side_by_side(rt, rows: int, width: int, *producer_inner: int) -> bool:
+    """Whether a bfloat16 operand of ``width`` values a row, of a step of ``rows`` rows, lies
+    with the rows side by side inside every group of 8 values (the layout that the kernel for
+    17 to 64 rows reads whole runs of memory from) rather than one row after the other: where
+    that kernel both reads it and, if a product writes it (inner size ``producer_inner``),
+    writes it."""
+    return rows > SLICED_MAX_ROWS and hasattr(rt.ops, "rows_kernel_ok") \
+        and rt.ops.rows_kernel_ok(rows, width, *producer_inner)
+
+
+def operand_rows(rt, name: str, rows: int, width: int, *producer_inner: int) -> torch.Tensor:
+    """Room for a bfloat16 operand of the fused products, [rows, width] (up to 16 rows, or
+    sizes the kernel for 17 to 64 rows does not take) or the view [rows, width/8, 8] of
+    [width/8, 64, 8]."""
+    if _side_by_side(rt, rows, width, *producer_inner):
+        return rt.ws.buf(name + "_side_by_side", (width // 8, STAT_COLUMNS, 8), torch.bfloat16).permute(1, 0, 2)[:rows]
+    return rt.ws.buf(name, (STAT_COLUMNS, width), torch.bfloat16)[:rows]
+
+
 def stream_bf16(rt, rows: int, width: int) -> torch.Tensor:
     """The bfloat16 copy of the residual stream that products behind a norm read."""
-    return rt.ws.buf("stream_bf16", (STAT_COLUMNS, width), torch.bfloat16)[:rows]
+    return operand_rows(rt, "stream_bf16", rows, width)
 
 
-def _sliced(rt, rows: int) -> bool:
-    return rows <= SLICED_MAX_ROWS and getattr(rt.ops, "use_sliced", False)
+def _sliced(rt, rows: int, inner: int) -> bool:
+    """Whether a product of ``rows`` bfloat16 rows with this inner size takes the form with
+    the norm folded into the weights (the kernels for up to 16 and for 17 to 64 rows)."""
+    if rows <= SLICED_MAX_ROWS:
+        return getattr(rt.ops, "use_sliced", False)
+    return hasattr(rt.ops, "rows_kernel_ok") and rt.ops.rows_kernel_ok(rows, inner)
 
 
 def _pack(rt, w: torch.Tensor) -> torch.Tensor:
@@ -81,12 +110,19 @@ def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None
     blocks = getattr(rt, "stream_stat_blocks", 0)
     M = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
     streams = {"swiglu": 2, "conv": 3}.get(epilogue, 1)
-    if _sliced(rt, M) and w.shape[0] // streams <= SLICED_MAX_COLUMNS and w.dtype == torch.bfloat16:
+    if _sliced(rt, M, h.shape[1]) and w.dtype == torch.bfloat16 \
+            and (M > SLICED_MAX_ROWS or w.shape[0] // streams <= SLICED_MAX_COLUMNS):
         # the stream's bfloat16 copy times the weight with the norm's weight folded in,
         # scaled by the rows' 1/rms at the end
         stats = stream_stats(rt, h.shape[1])
         xb = stream_bf16(rt, h.shape[0], h.shape[1])
-        if not (0 < blocks <= SLICED_MAX_STAT_BLOCKS and getattr(rt, "stream_has_bf16", False)):
+        if xb.dim() == 3 and M <= SLICED_MAX_ROWS:
+            # few wanted rows of a step of many: the kernel for few rows reads rows that lie one
+            # after the other, so the stream gets such a copy too
+            xb = rt.ws.buf("stream_bf16", (STAT_COLUMNS, h.shape[1]), torch.bfloat16)[:h.shape[0]]
+            rt.ops.stream_prepare(h, xb, stats)
+            rt.stream_stat_blocks = blocks = 1
+        elif not (0 < blocks <= SLICED_MAX_STAT_BLOCKS and getattr(rt, "stream_has_bf16", False)):
             rt.ops.stream_prepare(h, xb, stats)
             rt.stream_stat_blocks = blocks = 1
             rt.stream_has_bf16 = True
@@ -102,7 +138,7 @@ def linear_into_stream(rt, a, w, h, bias=None):
     """h += a w^T, leaving the partial sums of squares of the new rows (and, for few rows,
     the stream's bfloat16 copy)."""
     stats = stream_stats(rt, h.shape[1])
-    sliced = _sliced(rt, h.shape[0])
+    sliced = _sliced(rt, h.shape[0], a.shape[1] * (8 if a.dim() == 3 else 1))
     rt.ops.fused_linear(a, packed_weight(rt, w) if sliced else w, h, epilogue="residual", bias=bias,
                         stats_out=stats,
                         out_bf16=stream_bf16(rt, h.shape[0], h.shape[1]) if sliced else None)

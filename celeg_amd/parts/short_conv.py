@@ -21,7 +21,7 @@ from __future__ import annotations
 import torch
 
 from .base import Mixer, StateNeed, WeightSpec, register_part
-from .fused import fused_rows_ok, linear_into_stream, norm_linear
+from .fused import fused_rows_ok, linear_into_stream, norm_linear, operand_rows
 
 
 class ShortConv(Mixer):
@@ -79,11 +79,12 @@ class ShortConv(Mixer):
         if not fused_rows_ok(rt, batch, H) or (self.w_in.dtype, self.w_out.dtype) != (rt.dtype,) * 2:
             return False
         T = batch.n_tokens
-        y = rt.ws.buf("conv_y", (T, H), rt.dtype)
         if batch.decode_only and batch.n_seqs == T and self.taps <= 8:   # the fused form holds 8 taps
+            y = operand_rows(rt, "conv_y_fused", T, H, H)
             norm_linear(rt, h, norm, self.w_in, y, epilogue="conv", bias=self.b_in,
                         conv=(self.w_conv, self.b_conv, cache.states["bx"], batch.seq_slot))
         else:
+            y = rt.ws.buf("conv_y", (T, H), rt.dtype)
             bcx = rt.ws.buf("conv_bcx", (T, 3 * H), rt.dtype)
             norm_linear(rt, h, norm, self.w_in, bcx, bias=self.b_in)
             rt.ops.short_conv(bcx, self.w_conv, self.b_conv, cache.states["bx"], y, batch)

@@ -48,7 +48,19 @@ TINY_C = {
     "tie_word_embeddings": True, "norm_eps": 3e-5, "max_position_embeddings": 512,
     "bos_token_id": 0, "eos_token_id": 5, "pad_token_id": 1,
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+# A fourth one with the head size of the matrix-core and split-key attention kernels (64),
+# two taps and two attention layers in a row.
+TINY_D = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "vocab_size": 500, "hidden_size": 160, "num_hidden_layers": 5,
+    "layer_types": ["conv", "full_attention", "full_attention", "conv", "full_attention"],
+    "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64,
+    "intermediate_size": 320, "block_auto_adjust_ff_dim": False,
+    "rope_theta": 100000.0, "conv_L_cache": 2, "conv_bias": True,
+    "tie_word_embeddings": False, "norm_eps": 2e-5, "max_position_embeddings": 512,
+    "bos_token_id": 0, "eos_token_id": 4, "pad_token_id": 1,
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
 
 
 @pytest.fixture(scope="session")

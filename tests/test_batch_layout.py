@@ -1,0 +1,43 @@
+"""The packed step metadata: rows, sequences and wanted rows of a mixed batch."""
+import numpy as np
+import torch
+
+from celeg_amd.engine import StepEntry
+from celeg_amd.engine.batch import BatchBuilder
+
+
+def build(entries, pad_to=None):
+    builder = BatchBuilder("cpu", 4096, 1, pin=False)
+    batch = builder.build(entries, [[]], pad_to=pad_to, null_slot=9)
+    return batch
+
+
+def test_single_tokens_lie_first_and_logits_keep_the_entries_order():
+    entries = [StepEntry(3, 10, [5, 6, 7], [2]), StepEntry(1, 40, [8], [0]),
+               StepEntry(2, 0, [1, 2], [0, 1]), StepEntry(0, 7, [9], [0])]
+    b = build(entries)
+    assert (b.n_tokens, b.n_seqs, b.single_rows, b.decode_only) == (7, 4, 2, False)
+    assert b.entry_order == [1, 3, 0, 2]
+    assert b.token_ids.tolist() == [8, 9, 5, 6, 7, 1, 2]
+    assert b.positions.tolist() == [40, 7, 10, 11, 12, 0, 1]
+    assert b.token_slot.tolist() == [1, 0, 3, 3, 3, 2, 2]
+    assert b.token_seq.tolist() == [0, 1, 2, 2, 2, 3, 3]
+    assert b.cu_seqlens.tolist() == [0, 1, 2, 5, 7]
+    assert b.seq_slot.tolist() == [1, 0, 3, 2] and b.seq_start.tolist() == [40, 7, 10, 0]
+    # wanted rows in the order of the entries and of their ``want``
+    assert b.logit_rows.tolist() == [4, 0, 5, 6, 1]
+    assert b.host["seg_lens"].tolist() == [1, 1, 3, 2]
+
+
+def test_single_rows_only_and_padding():
+    entries = [StepEntry(2, 5, [11], [0]), StepEntry(0, 9, [12], [0])]
+    b = build(entries)
+    assert b.decode_only and b.single_rows == 2 and b.entry_order == [0, 1]
+    b = build(entries, pad_to=4)
+    assert (b.n_tokens, b.n_seqs, b.single_rows) == (4, 4, 4)
+    assert b.token_slot.tolist() == [2, 0, 9, 9] and b.logit_rows.tolist() == [0, 1, 2, 3]
+
+
+def test_a_portion_alone_has_no_single_rows():
+    b = build([StepEntry(0, 0, [1, 2, 3, 4], [3])])
+    assert b.single_rows == 0 and b.logit_rows.tolist() == [3]

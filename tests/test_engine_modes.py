@@ -14,7 +14,7 @@ from helpers import (WEIGHT_STD, EngineDriver, assert_close, mixed_schedule, pea
                      portions_schedule, random_tokens, tail_decode_schedule, whole_schedule)
 
 LENGTHS = {"A": [40, 57, 90, 128, 65, 33], "B": [45, 200, 64, 100, 256, 33],
-           "C": [70, 33, 150, 97, 48, 260]}
+           "C": [70, 33, 150, 97, 48, 260], "D": [300, 66, 129, 40, 210, 77]}
 SCHEDULES = {"whole": whole_schedule, "tail32": tail_decode_schedule,
              "portions": portions_schedule, "mixed": mixed_schedule}
 
@@ -59,7 +59,7 @@ def run_mode(model_folders, name, dtype, mode, device, ops=None, subset=None):
 @pytest.mark.gpu
 @pytest.mark.parametrize("mode", list(SCHEDULES))
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_gpu_engine_matches_plain(model_folders, name, dtype, mode):
     run_mode(model_folders, name, dtype, mode, "cuda:0")
 

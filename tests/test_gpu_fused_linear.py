@@ -76,7 +76,8 @@ def test_norm_prologue_with_and_without_partial_sums(ops, M, N, K, with_stats):
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (8, 1024, 1024), (20, 200, 352), (64, 96, 4608),
                                    (3, 130, 72), (4, 1024, 4608), (7, 77, 352), (8, 1024, 4608),
-                                   (13, 50, 1160), (16, 1024, 1024), (2, 36, 8), (5, 24, 40)])
+                                   (13, 50, 1160), (16, 1024, 1024), (2, 36, 8), (5, 24, 40),
+                                   (33, 1000, 96), (64, 8192, 64), (17, 14400, 32), (48, 1024, 2048)])
 def test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, M, N, K):
     a = randn(M, K, seed=7, dtype=BF)
     w = randn(N, K, seed=8, scale=0.1, dtype=BF)
@@ -89,8 +90,15 @@ def test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, M, N, K):
     assert ops.last_stat_blocks == blocks
     delta = (a.double() @ w.double().T + b.double())
     close(h, h0.double() + delta)
-    # the product enters the sum rounded to bfloat16
-    close(h - h0, delta.to(BF), rel=2e-3)
+    # the product enters the sum rounded to bfloat16: what was added is the product rounded
+    # (an element whose 32-bit sum lies at a rounding boundary may land one step away, never
+    # more, and few do)
+    added, rounded = (h - h0).double().cpu(), delta.to(BF).double().cpu()
+    step = rounded.abs() * 2.0 ** -7 + 1e-30         # at least one step of bfloat16 at this size
+    err = (added - rounded).abs()
+    slack = 4e-6 * h0.abs().double().cpu().clamp_min(1.0) + 1e-6 * rounded.abs()   # 32-bit rounding of the sum
+    assert bool((err <= step + slack).all()), float((err - step).max())
+    assert float((err > slack).double().mean()) < 0.01
     torch.testing.assert_close(stats[:M].sum(dim=1), (h ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
     assert float(stats[M:].max()) == -1.0 if M < 64 else True
 
@@ -139,6 +147,10 @@ def test_conv_epilogue_token_by_token_equals_the_whole_convolution(ops, M, H, ta
 
 SLICED = [(1, 64, 64), (3, 130, 200), (4, 1024, 1024), (5, 77, 352), (8, 3072, 1024), (8, 96, 4608),
           (13, 50, 1160), (16, 272, 1024)]
+# 17 to 64 rows: the kernel that streams the weights (inner sizes in steps of 32), at widths
+# that give it one, two and four column tiles a workgroup, and few and many blocks of k
+STREAMED = [(17, 64, 64), (20, 130, 352), (32, 1024, 1024), (33, 77, 96), (48, 3072, 1024),
+            (64, 272, 4608), (64, 8192, 128), (33, 14400, 64), (50, 1000, 32)]
 
 
 def scaled_case(M, N, K, streams, seed):
@@ -157,9 +169,9 @@ def scaled_case(M, N, K, streams, seed):
     return h, h.to(BF), stats, nw, w, folded, rows, x
 
 
-@pytest.mark.parametrize("M,N,K", SLICED)
+@pytest.mark.parametrize("M,N,K", SLICED + STREAMED)
 def test_sliced_products_behind_a_norm(ops, M, N, K):
-    """The form for up to 16 rows: bfloat16 copy of the stream, norm weight folded into the
+    """The form for up to 16 rows, and for 17 to 64: bfloat16 copy of the stream, norm weight folded into the
     weights, 1/rms from the partial sums applied at the end; against the plain norm and
     product."""
     h, xb, stats, nw, w, folded, rows, x = scaled_case(M, N, K, 1, 40)
@@ -179,7 +191,8 @@ def test_sliced_products_behind_a_norm(ops, M, N, K):
     close(out32, old, rel=8e-3)
 
 
-@pytest.mark.parametrize("M,ff,K", [(1, 192, 64), (8, 4608, 1024), (7, 352, 128), (16, 200, 96), (4, 100, 1160)])
+@pytest.mark.parametrize("M,ff,K", [(1, 192, 64), (8, 4608, 1024), (7, 352, 128), (16, 200, 96), (4, 100, 1160),
+                                    (19, 352, 128), (40, 4608, 1024), (64, 200, 96), (33, 7200, 64)])
 def test_sliced_swiglu(ops, M, ff, K):
     h, xb, stats, nw, w, folded, rows, x = scaled_case(M, ff, K, 2, 50)
     g = (x @ w[:ff].double().cpu().T).to(BF).double()
@@ -190,7 +203,9 @@ def test_sliced_swiglu(ops, M, ff, K):
 
 
 @pytest.mark.parametrize("M,H,taps,bias", [(1, 64, 3, False), (8, 1024, 3, False), (5, 128, 4, True),
-                                           (16, 96, 1, True), (3, 48, 5, False), (12, 200, 8, True)])
+                                           (16, 96, 1, True), (3, 48, 5, False), (12, 200, 8, True),
+                                           (17, 64, 3, False), (40, 1024, 3, True), (62, 96, 4, True),
+                                           (33, 160, 8, False)])
 def test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, M, H, taps, bias):
     """M requests advance one token per call, each in its own slot (in another order than
     the rows); their outputs over 6 calls equal the plain whole-sequence convolution."""
@@ -224,7 +239,8 @@ def test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, M, H, taps
     assert float(state[0].abs().max()) == 0.0          # a slot nobody uses stays zero
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (4, 1024, 1024), (5, 77, 352), (8, 96, 4608), (16, 272, 1024)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 64), (4, 1024, 1024), (5, 77, 352), (8, 96, 4608), (16, 272, 1024),
+                                   (20, 77, 352), (33, 1024, 1024), (64, 272, 1024)])
 def test_packed_weights_give_the_same_bits(ops, M, N, K):
     """The layout of blocks of 32 k-values changes where the weights lie, not what is added
     in which order: every epilogue gives identical results from either layout."""
@@ -250,8 +266,54 @@ def test_packed_weights_give_the_same_bits(ops, M, N, K):
         assert torch.equal(act[0], act[1])
 
 
-def test_residual_refreshes_the_bfloat16_copy(ops):
-    M, N, K = 6, 200, 352
+@pytest.mark.parametrize("M,N,K", [(17, 64, 64), (33, 80, 96), (40, 1024, 1024), (64, 272, 4608)])
+def test_operands_with_rows_side_by_side_give_the_same_bits(ops, M, N, K):
+    """For 17 to 64 rows the bfloat16 operands may lie as [width/8, 64, 8] (the rows side by
+    side inside every group of 8 values): inputs and outputs in that layout give the same bits
+    as rows that lie one after the other."""
+    h, xb, stats, nw, w, folded, rows, x = scaled_case(M, N, K, 1, 90)
+    xc = ops.chunked_rows(M + 3, K, DEV, max_rows=80)
+    assert xc.shape == (M + 3, K // 8, 8) and xc.stride() == (8, 80 * 8, 1)
+    st = torch.zeros(80, 1, device=DEV)
+    ops.stream_prepare(h, xc, st)
+    assert torch.equal(xc.reshape(M + 3, K), xb)
+    torch.testing.assert_close(st[:M + 3, 0], (h ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
+    b = randn(N, seed=94)
+    flat, side = torch.empty(M, N, dtype=BF, device=DEV), ops.chunked_rows(M, N, DEV)
+    for a_, out in ((xb, flat), (xc, side)):
+        ops.fused_linear(a_, folded, out, eps=1e-5, stats=stats, stat_blocks=5, rows=rows, bias=b)
+    assert torch.equal(side.reshape(M, N), flat)
+    act = [torch.empty(M, N // 2, dtype=BF, device=DEV), ops.chunked_rows(M, N // 2, DEV)]
+    for a_, out in zip((xb, xc), act):
+        ops.fused_linear(a_, folded, out, epilogue="swiglu", eps=1e-5, stats=stats, stat_blocks=5, rows=rows)
+    assert torch.equal(act[1].reshape(M, N // 2), act[0])
+    hh = [randn(M, N, seed=95) for _ in range(2)]
+    copies = [torch.zeros(M, N, dtype=BF, device=DEV), ops.chunked_rows(M, N, DEV)]
+    so = [torch.zeros(64, ops.residual_stat_blocks(M, N, K), device=DEV) for _ in range(2)]
+    for a_, h_, c_, s_ in zip((xb[:M], xc[:M]), hh, copies, so):
+        ops.fused_linear(a_, folded, h_, epilogue="residual", stats_out=s_, out_bf16=c_)
+    assert torch.equal(hh[0], hh[1]) and torch.equal(so[0], so[1])
+    assert torch.equal(copies[1].reshape(M, N), copies[0]) and torch.equal(copies[0], hh[0].to(BF))
+    # the kernels for up to 16 rows read rows that lie one after the other only
+    from celeg_amd.csrc.hip_ops import KernelError
+    with pytest.raises(KernelError, match="side by side"):
+        ops.fused_linear(xc[:8], folded, torch.empty(8, N, dtype=BF, device=DEV))
+
+
+def test_embed_stream_with_rows_side_by_side(ops):
+    table = randn(300, 96, seed=96, dtype=BF)
+    ids = torch.tensor([(7 * i) % 300 for i in range(40)], dtype=torch.int32, device=DEV)
+    out = torch.empty(40, 96, device=DEV)
+    xc = ops.chunked_rows(40, 96, DEV)
+    st = torch.zeros(64, 2, device=DEV)
+    ops.embed_stream(table, ids, out, xc, st)
+    assert torch.equal(out, table[ids.long()].float()) and torch.equal(xc.reshape(40, 96), table[ids.long()])
+    torch.testing.assert_close(st[:40, 0], (out ** 2).sum(dim=1), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("M", [6, 40])
+def test_residual_refreshes_the_bfloat16_copy(ops, M):
+    N, K = 200, 352
     a = randn(M, K, seed=60, dtype=BF)
     w = randn(N, K, seed=61, scale=0.1, dtype=BF)
     h = randn(M, N, seed=62)

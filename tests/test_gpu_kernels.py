@@ -233,6 +233,7 @@ def attention_case(ops, dtype, heads, kv_heads, head_dim, lengths, cuts, window=
             parts.append((i, pos[i], c))
             pos[i] += c
         batch, keep = build_batch(ops, cache, entries)
+        parts = [parts[j] for j in batch.entry_order]     # single tokens lie first in the rows
         q = torch.cat([reqs[i][0][p:p + c] for i, p, c in parts]).contiguous()
         k = torch.cat([reqs[i][1][p:p + c] for i, p, c in parts]).contiguous()
         v = torch.cat([reqs[i][2][p:p + c] for i, p, c in parts]).contiguous()
