@@ -549,79 +549,6 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     }
 }
 
-// The same without a second kernel: one workgroup of DEC_WAVES wavefronts per (GH query
-// heads, request); wavefront w takes the ranges w, w + DEC_WAVES, ... and keeps a running
-// (max, sum, accumulator); the wavefronts' results meet in LDS and are joined in wavefront
-// order.  Fewer workgroups than the kernel above (it suits batches, not one long context).
-#define DEC_WAVES 16
-template <int HD, int GH>
-__global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_whole_kernel(
-    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
-    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
-    const int* __restrict__ token_slot, const int* __restrict__ positions, bf16* __restrict__ out,
-    int ldo, int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer,
-    float scale, int window) {
-    constexpr int DD = HD / 64;
-    __shared__ float ps_all[DEC_WAVES][GH][DEC_KEYS];
-    __shared__ float part_o[DEC_WAVES][GH][HD];
-    __shared__ float part_ml[DEC_WAVES][GH][2];
-    const int hb = blockIdx.x, t = blockIdx.y;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int pos = positions[t];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int h0 = hb * GH;
-    const int kvh = h0 / (q_heads / kv_heads);
-    const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
-    float M[GH], L[GH], O[GH][DD];
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-        M[g] = -INFINITY;
-        L[g] = 0.f;
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) O[g][dd] = 0.f;
-    }
-    for (int r = lo / DEC_KEYS + wave; r <= pos / DEC_KEYS; r += DEC_WAVES) {
-        const int kb = r * DEC_KEYS;
-        float m[GH], l[GH], acc[GH][DD];
-        decode_range<HD, GH>(q, ldq, k_pool, v_pool, pages, t, h0, kvh, kb, max(lo, kb),
-                             min(pos, kb + DEC_KEYS - 1), kv_heads, page_tokens, page_shift, n_layers,
-                             layer, scale, ps_all[wave], m, l, acc);
-#pragma unroll
-        for (int g = 0; g < GH; ++g) {
-            const float mn = fmaxf(M[g], m[g]);
-            const float a = expf(M[g] - mn), b = expf(m[g] - mn);   // e^(-inf) = 0 the first time
-            L[g] = L[g] * a + l[g] * b;
-#pragma unroll
-            for (int dd = 0; dd < DD; ++dd) O[g][dd] = O[g][dd] * a + acc[g][dd] * b;
-            M[g] = mn;
-        }
-    }
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-        if (lane == 0) { part_ml[wave][g][0] = M[g]; part_ml[wave][g][1] = L[g]; }
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) part_o[wave][g][lane + 64 * dd] = O[g][dd];
-    }
-    __syncthreads();
-    // wavefront g of the first GH joins head h0 + g
-    if (wave >= GH) return;
-    const int g = wave;
-    float mx = -INFINITY;
-    for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, part_ml[w][g][0]);
-    float denom = 0.f, o[DD];
-#pragma unroll
-    for (int dd = 0; dd < DD; ++dd) o[dd] = 0.f;
-    for (int w = 0; w < DEC_WAVES; ++w) {
-        const float wgt = expf(part_ml[w][g][0] - mx);      // a wavefront without a range: e^(-inf) = 0
-        denom += wgt * part_ml[w][g][1];
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) o[dd] = fmaf(wgt, part_o[w][g][lane + 64 * dd], o[dd]);
-    }
-    bf16* orow = out + static_cast<size_t>(t) * ldo + static_cast<size_t>(h0 + g) * HD;
-#pragma unroll
-    for (int dd = 0; dd < DD; ++dd) orow[lane + 64 * dd] = from_float<bf16>(o[dd] / denom);
-}
-
 // Joins the ranges of one (request, query head): out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
 template <int HD>
 __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
@@ -671,8 +598,173 @@ __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
     for (int dd = 0; dd < HD / 64; ++dd) orow[lane + 64 * dd] = from_float<bf16>(acc[dd] / denom);
 }
 
-// workspace: ws_o [rows, q_heads, n_splits, head_dim] and ws_ml [rows, q_heads, n_splits, 2]
-// floats, n_splits = ceil(max_context / 64).
+// Decode attention without a second kernel, for batches that fill the chip: one workgroup
+// per (request, key/value head, chunk of 16 query heads of its group).  The heads of the
+// group are the rows of matrix instructions, so the work per key does not grow with the
+// group; the wavefronts take rounds of 64 keys in turn, each keeps a running maximum, sum
+// and output of its own, and they meet in LDS.
+//   S^T[key, head] = K Q^T : a lane holds head lane%16, keys 4*(lane/16)..+3 of a 16-key tile;
+//   O^T[dim, head] = V^T P : P's operand wants 8 keys a lane, which are rows 4q..4q+3 of two
+//   tiles: tile 2j holds keys 32j + 8*(row/4) + row%4, tile 2j+1 those + 4, so that a lane's
+//   eight p are eight keys in a row and V (stored [dim][key] in a page) is read 16 bytes a lane.
+template <int HD, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
+    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
+    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
+    const int* __restrict__ token_slot, const int* __restrict__ positions, bf16* __restrict__ out,
+    int ldo, int kv_heads, int group, int page_tokens, int page_shift, int n_layers, int layer,
+    float scale, int window) {
+    constexpr int KS = HD / 32;   // steps of 32 dims in q.k
+    constexpr int DT = HD / 16;   // 16-dim tiles of the output
+    extern __shared__ float smem_heads[];
+    const int chunks = (group + 15) >> 4;
+    const int kvh = blockIdx.x / chunks, chunk = blockIdx.x % chunks;
+    const int gp = min(group - chunk * 16, 16);          // heads of this workgroup
+    const int h0 = kvh * group + chunk * 16;
+    const int t = blockIdx.y;
+    float* const part_o = smem_heads;                                      // [waves][gp][HD]
+    float* const part_ml = smem_heads + static_cast<size_t>(WAVES) * gp * HD;   // [waves][gp][2]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int c = lane & 15, qd = lane >> 4;
+    const int pos = positions[t];
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
+    const int page_mask = page_tokens - 1;
+
+    bf16x8_t qf[KS];
+    {
+        const bf16* qrow = q + static_cast<size_t>(t) * ldq + static_cast<size_t>(h0 + min(c, gp - 1)) * HD + qd * 8;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8_t*>(qrow + s * 32);
+    }
+    float m_run = -INFINITY, l_run = 0.f;
+    floatx4_t o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int r = lo / DEC_KEYS + wave; r <= pos / DEC_KEYS; r += WAVES) {
+        const int kb = r * DEC_KEYS;
+        const int k_lo = max(lo, kb), k_hi = min(pos, kb + DEC_KEYS - 1);
+        const int first_page = kb >> page_shift, last_page = k_hi >> page_shift;
+        const int my_page = pages[min(first_page + lane, last_page)];
+        bf16x8_t kf[4][KS], vf[DT][2];
+#pragma unroll
+        for (int T = 0; T < 4; ++T) {
+            const int keyc = min(max(kb + 32 * (T >> 1) + 8 * (c >> 2) + 4 * (T & 1) + (c & 3), k_lo), k_hi);
+            const int page = __shfl(my_page, (keyc >> page_shift) - first_page, 64);
+            const bf16* kp = k_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
+                             static_cast<size_t>(keyc & page_mask) * HD + qd * 8;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) kf[T][s] = *reinterpret_cast<const bf16x8_t*>(kp + s * 32);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            // eight keys in a row; a group outside the range reads one inside (its p are zero)
+            const int key0 = min(max(kb + 32 * j + 8 * qd, k_lo & ~7), k_hi & ~7);
+            const int page = __shfl(my_page, (key0 >> page_shift) - first_page, 64);
+            const bf16* vbase = v_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
+                                (key0 & page_mask);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                vf[dt][j] = *reinterpret_cast<const bf16x8_t*>(vbase + static_cast<size_t>(16 * dt + c) * page_tokens);
+        }
+        float sc[4][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int T = 0; T < 4; ++T) {
+            floatx4_t acc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[T][s], qf[s], acc, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = kb + 32 * (T >> 1) + 8 * qd + 4 * (T & 1) + i;
+                sc[T][i] = (key >= k_lo && key <= k_hi) ? acc[i] * scale : -INFINITY;
+                mx = fmaxf(mx, sc[T][i]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));        // finite: the round holds a key
+        const float m_new = fmaxf(m_run, mx);
+        const float keep = expf(m_run - m_new);         // e^(-inf) = 0 the first time
+        float psum = 0.f;
+#pragma unroll
+        for (int T = 0; T < 4; ++T)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sc[T][i] = expf(sc[T][i] - m_new);
+                psum += sc[T][i];
+            }
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * keep + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[dt][i] *= keep;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            bf16x8_t pb;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pb[i] = static_cast<__bf16>(sc[2 * j][i]);
+                pb[4 + i] = static_cast<__bf16>(sc[2 * j + 1][i]);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt][j], pb, o[dt], 0, 0, 0);
+        }
+    }
+    if (c < gp) {
+        if (qd == 0) {
+            part_ml[(wave * gp + c) * 2] = m_run;
+            part_ml[(wave * gp + c) * 2 + 1] = l_run;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                part_o[(static_cast<size_t>(wave) * gp + c) * HD + 16 * dt + 4 * qd + i] = o[dt][i];
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < gp * HD; e += WAVES * 64) {
+        const int g = e / HD, d = e % HD;
+        float mxw = -INFINITY;
+        for (int w = 0; w < WAVES; ++w) mxw = fmaxf(mxw, part_ml[(w * gp + g) * 2]);
+        float denom = 0.f, val = 0.f;
+        for (int w = 0; w < WAVES; ++w) {
+            const float wgt = expf(part_ml[(w * gp + g) * 2] - mxw);   // a wavefront without a round: e^(-inf) = 0
+            denom += wgt * part_ml[(w * gp + g) * 2 + 1];
+            val = fmaf(wgt, part_o[(static_cast<size_t>(w) * gp + g) * HD + d], val);
+        }
+        out[static_cast<size_t>(t) * ldo + static_cast<size_t>(h0 + g) * HD + d] = from_float<bf16>(val / denom);
+    }
+}
+
+template <int HD>
+static int launch_decode_heads(const void* q, int ldq, const void* k_pool, const void* v_pool,
+                               const int* table, int table_stride, const int* token_slot,
+                               const int* positions, void* out, int ldo, int n_rows, int kv_heads,
+                               int group, int page_tokens, int page_shift, int n_layers, int layer,
+                               float scale, int window, hipStream_t stream) {
+    constexpr int WAVES = HD <= 64 ? 16 : 8;   // what the registers of a CU hold of this head size
+    const int chunks = (group + 15) / 16;
+    const size_t lds = static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
+    static bool raised = false;
+    if (lds > 48 * 1024 && !raised) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (err != hipSuccess) return static_cast<int>(err);
+        raised = true;
+    }
+    hipLaunchKernelGGL((attention_decode_heads_kernel<HD, WAVES>), dim3(kv_heads * chunks, n_rows),
+                       dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
+                       static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
+                       table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
+                       group, page_tokens, page_shift, n_layers, layer, scale, window);
+    return CELEG_LAUNCH_RESULT();
+}
+
 extern "C" int celeg_attention_decode_bf16(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
@@ -686,27 +778,22 @@ extern "C" int celeg_attention_decode_bf16(
         return static_cast<int>(hipErrorInvalidValue);
     const int page_shift = __builtin_ctz(page_tokens);
     const int gh = (group % 4 == 0) ? 4 : ((group % 2 == 0) ? 2 : 1);
-    // enough (heads, request) pairs to occupy every compute unit: one workgroup each and no
-    // second kernel (measured at context 2,176, 8 key/value heads: batch 64 54 us against 68 us;
-    // batch 8 20 us against 15.5 us, a workgroup then being bound by what one compute unit
-    // can pull).  whole: 0 the split-key kernels, 1 the whole-context kernel, -1 decide here.
-    if (whole < 0) whole = (q_heads / gh) * n_rows >= 192 ? 1 : 0;
+    // whole: 0 the split-key kernels, 1 one workgroup per (request, key/value head), -1 decide
+    // here: one workgroup each, and no second kernel, once there are enough of them (measured
+    // at context 2,100 with 8 key/value heads: groups of 4 heads gain from 8 requests on, 1.48
+    // against 1.53 ms a step of the 2.6B shape, groups of 2 from 16 on, 0.70 against 0.72 ms of
+    // the 350M shape; below that a workgroup is bound by what one compute unit can pull).
+    if (whole < 0) whole = kv_heads * n_rows >= (group >= 3 ? 64 : 128) ? 1 : 0;
     if (whole) {
-        dim3 wgrid(q_heads / gh, n_rows), wblock(DEC_WAVES * 64);
-#define CELEG_WHOLE(HD_, GH_)                                                                    \
-    hipLaunchKernelGGL((attention_decode_whole_kernel<HD_, GH_>), wgrid, wblock, 0, stream,      \
-                       static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
-                       static_cast<const bf16*>(v_pool), table, table_stride, token_slot,        \
-                       positions, static_cast<bf16*>(out), ldo, q_heads, kv_heads, page_tokens,  \
-                       page_shift, n_layers, layer, scale, window)
-#define CELEG_WHOLE_HD(HD_)                                                                      \
-    if (gh == 4) CELEG_WHOLE(HD_, 4); else if (gh == 2) CELEG_WHOLE(HD_, 2); else CELEG_WHOLE(HD_, 1)
-        if (head_dim == 64) { CELEG_WHOLE_HD(64); }
-        else if (head_dim == 128) { CELEG_WHOLE_HD(128); }
-        else return static_cast<int>(hipErrorInvalidValue);
-#undef CELEG_WHOLE_HD
-#undef CELEG_WHOLE
-        return CELEG_LAUNCH_RESULT();
+        if (head_dim == 64)
+            return launch_decode_heads<64>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
+                                           out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
+                                           n_layers, layer, scale, window, stream);
+        if (head_dim == 128)
+            return launch_decode_heads<128>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
+                                            out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
+                                            n_layers, layer, scale, window, stream);
+        return static_cast<int>(hipErrorInvalidValue);
     }
     dim3 grid(n_splits, q_heads / gh, n_rows), block(64);
 #define CELEG_DEC(HD_, GH_)                                                                      \

@@ -52,10 +52,45 @@ constexpr int rows_max_waves(int mt, int sc) {
     return w;
 }
 
-// Finishes one output: row r, column n (both inside the sizes), from the sums of its weight
-// streams (scale and bias applied).  Returns the new value of the residual stream (E_RESIDUAL).
+// What the end of an output (row r, column n, both inside the sizes) needs from memory:
+// asked for before the products, so that it has long arrived when they are done.
 template <int EPI>
-__device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n, const float* sum) {
+struct Early {
+    float bias[Streams<EPI>::n];
+    float old;                                           // E_RESIDUAL: the stream's value
+    float taps[EPI == E_CONV ? ROWS_MAX_TAPS : 1];       // E_CONV
+    float state[EPI == E_CONV ? ROWS_MAX_TAPS - 1 : 1];
+    float conv_b;
+    float* state_ptr;
+};
+
+template <int EPI>
+__device__ __forceinline__ Early<EPI> early_fetch(const GemvParams& p, int r, int n) {
+    Early<EPI> e;
+#pragma unroll
+    for (int s = 0; s < Streams<EPI>::n; ++s)
+        e.bias[s] = p.bias ? p.bias[static_cast<size_t>(s) * p.stream_rows + n] : 0.f;
+    e.old = 0.f; e.conv_b = 0.f; e.state_ptr = nullptr;
+    if (EPI == E_RESIDUAL) e.old = static_cast<const float*>(p.out)[static_cast<size_t>(r) * p.ldo + n];
+    if (EPI == E_CONV) {
+        e.state_ptr = p.state + static_cast<size_t>(p.seq_slot[r]) * p.state_slot_stride + n;
+#pragma unroll
+        for (int i = 0; i < ROWS_MAX_TAPS; ++i) e.taps[i] = p.conv_w[static_cast<size_t>(n) * p.taps + min(i, p.taps - 1)];
+#pragma unroll
+        for (int i = 0; i < ROWS_MAX_TAPS - 1; ++i) e.state[i] = e.state_ptr[static_cast<size_t>(min(i + 1, p.taps - 1)) * p.N];
+        if (p.conv_b) e.conv_b = p.conv_b[n];
+    }
+    return e;
+}
+
+// Finishes one output from the scaled sums of its weight streams.  Returns the new value of
+// the residual stream (E_RESIDUAL).
+template <int EPI>
+__device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n, const float* scaled,
+                                               const Early<EPI>& early) {
+    float sum[Streams<EPI>::n];
+#pragma unroll
+    for (int s = 0; s < Streams<EPI>::n; ++s) sum[s] = scaled[s] + early.bias[s];
     const size_t o = static_cast<size_t>(r) * p.ldo + n;      // 32-bit outputs: rows one after the other
     const size_t ob = static_cast<size_t>(r) * p.ldo + static_cast<size_t>(n >> 3) * p.out_k8_stride + (n & 7);
     if (EPI == E_STORE) {
@@ -64,7 +99,7 @@ __device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n
         static_cast<float*>(p.out)[o] = sum[0];
     } else if (EPI == E_RESIDUAL) {
         // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
-        const float v = static_cast<const float*>(p.out)[o] + round_bf16(sum[0]);
+        const float v = early.old + round_bf16(sum[0]);
         static_cast<float*>(p.out)[o] = v;
         if (p.out_bf16)
             static_cast<bf16*>(p.out_bf16)[static_cast<size_t>(r) * p.ld_bf16 + static_cast<size_t>(n >> 3) * p.bf16_k8_stride + (n & 7)] = from_float<bf16>(v);
@@ -75,18 +110,19 @@ __device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n
     } else if (EPI == E_CONV) {
         const float bb = round_bf16(sum[0]), cc = round_bf16(sum[1]), xx = round_bf16(sum[2]);
         const float bx = bb * xx;
-        float* state = p.state + static_cast<size_t>(p.seq_slot[r]) * p.state_slot_stride + n;
-        const float* taps = p.conv_w + static_cast<size_t>(n) * p.taps;
-        float conv = 0.f;
-        for (int tap = 0; tap + 1 < p.taps; ++tap) {
-            const float sv = state[static_cast<size_t>(tap + 1) * p.N];
-            conv = fmaf(taps[tap], sv, conv);
-            state[static_cast<size_t>(tap) * p.N] = sv;          // shift by one position
-        }
-        conv = fmaf(taps[p.taps - 1], bx, conv);
-        state[static_cast<size_t>(p.taps - 1) * p.N] = bx;
-        if (p.conv_b) conv += p.conv_b[n];
-        static_cast<bf16*>(p.out)[ob] = from_float<bf16>(cc * conv);
+        float conv = 0.f, last_tap = 0.f;
+#pragma unroll
+        for (int tap = 0; tap < ROWS_MAX_TAPS - 1; ++tap)
+            if (tap + 1 < p.taps) {
+                conv = fmaf(early.taps[tap], early.state[tap], conv);
+                early.state_ptr[static_cast<size_t>(tap) * p.N] = early.state[tap];     // shift by one position
+            }
+#pragma unroll
+        for (int tap = 0; tap < ROWS_MAX_TAPS; ++tap)
+            if (tap == p.taps - 1) last_tap = early.taps[tap];
+        conv = fmaf(last_tap, bx, conv);
+        early.state_ptr[static_cast<size_t>(p.taps - 1) * p.N] = bx;
+        static_cast<bf16*>(p.out)[ob] = from_float<bf16>(cc * (conv + early.conv_b));
     }
     return 0.f;
 }
@@ -152,8 +188,12 @@ void gemm_rows_kernel(const GemvParams p) {
     if (kb_begin < kb_end) fetch(kb_begin, a0, w0);
     if (kb_begin + 1 < kb_end) fetch(kb_begin + 1, a1, w1);
 
-    // ---- the rows' 1/rms from the partial sums of squares (asked for behind the first
-    // weights, used at the end): LPR neighbouring threads share a row
+    // ---- what the end of this thread's first output needs (asked for behind the first weights)
+    const int e0 = min(static_cast<int>(threadIdx.x), ROWS * COLS - 1);
+    const Early<EPI> early0 = early_fetch<EPI>(p, min(e0 / COLS, M - 1), min(n0 + e0 % COLS, N - 1));
+
+    // ---- the rows' 1/rms from the partial sums of squares (likewise): LPR neighbouring
+    // threads share a row
     if (p.stats) {
         const int lpr = blockDim.x / ROWS;           // a power of two, 1 .. 32
         const int r = threadIdx.x / lpr, sub = threadIdx.x % lpr;
@@ -208,10 +248,13 @@ void gemm_rows_kernel(const GemvParams p) {
         }
         const float scale = p.stats ? s_scale[r] : 1.f;
 #pragma unroll
-        for (int s = 0; s < NS; ++s)
-            sum[s] = sum[s] * scale + (p.bias ? p.bias[static_cast<size_t>(s) * p.stream_rows + nc] : 0.f);
+        for (int s = 0; s < NS; ++s) sum[s] *= scale;
         float v = 0.f;
-        if (ok) v = finish_output<EPI>(p, rc, nc, sum);
+        if (e == static_cast<int>(threadIdx.x)) {
+            if (ok) v = finish_output<EPI>(p, rc, nc, sum, early0);
+        } else if (ok) {
+            v = finish_output<EPI>(p, rc, nc, sum, early_fetch<EPI>(p, rc, nc));
+        }
         if (EPI == E_RESIDUAL && p.stats_out) {
             float sq = v * v;               // the COLS columns of a row sit in COLS neighbouring lanes
 #pragma unroll

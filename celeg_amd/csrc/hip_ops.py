@@ -42,7 +42,7 @@ class HipOps:
         self.loaded_libraries: Dict[str, str] = {}
         # "auto": the matrix-core and split-key kernels where they apply; "general": always
         # the general kernel (tests compare the two)
-        self.attention_decode_whole = -1     # -1: chosen from the batch; 0 split-key kernels; 1 one workgroup a request
+        self.attention_decode_whole = -1     # -1: chosen from the batch; 0 split-key kernels; 1 one workgroup per request and key/value head
         self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
         self.attention_impl = "auto"
         self._decode_ws = None

@@ -343,11 +343,15 @@ def test_attention_rows_tile_pairs(ops, rows_per_tile, heads, kv_heads, head_dim
         ops.attention_rows_per_tile = 0
 
 
-@pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [(4, 2, 64, 16), (8, 1, 128, 32), (3, 1, 64, 64)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [
+    (8, 2, 64, 16), (3, 1, 64, 64), (6, 1, 128, 32), (16, 1, 64, 16), (40, 2, 64, 32), (4, 4, 64, 16),
+    (32, 8, 64, 16), (12, 2, 128, 16), (4, 2, 64, 16), (8, 1, 128, 32)])
 def test_attention_decode_one_workgroup_per_request(ops, heads, kv_heads, head_dim, page_tokens):
-    """The decode kernel that walks a request's whole context in one workgroup (16
-    wavefronts, joined in LDS): long contexts (more ranges of 64 keys than wavefronts), a
-    boosted far key, and a window that cuts the first range."""
+    """The decode kernel that walks a request's whole context in one workgroup, the query
+    heads of a key/value head being the rows of its matrix instructions (groups of 1 to 20
+    heads; more than 16 take two workgroups): long contexts (more rounds of 64 keys than
+    wavefronts), a boosted far key, a window that cuts the first round of keys, the last round
+    ending inside a page."""
     ops.attention_decode_whole = 1
     try:
         attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[1300, 150, 70],
