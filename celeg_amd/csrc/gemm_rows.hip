@@ -1,6 +1,6 @@
-// bfloat16 products for 17 to 64 rows on gfx950 (decode steps of many requests, short
-// portions of prompts), with what surrounds them fused in, as for the products of up to
-// 16 rows:
+// bfloat16 products for 9 to 64 rows on gfx950 (decode steps of many requests, short
+// portions of prompts), with what surrounds them fused in, as for the products of fewer
+// rows:
 //   out[M,N] = epilogue(scale[m] * (A[M,K] W[N,K]^T) + bias)
 // A is bfloat16; behind an RMSNorm it is the bfloat16 copy of the residual stream, W has
 // the norm's weight folded in and scale[m] = rsqrt(mean(x_m^2) + eps) comes from the
@@ -276,7 +276,7 @@ extern "C" void celeg_gemm_rows_force(int ct, int waves) { g_force_ct = ct; g_fo
 
 static RowsShape rows_shape(int M, int N, int K, int streams) {
     RowsShape s;
-    s.mt = M <= 32 ? 2 : 4;
+    s.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
     const int max_ct = streams == 1 ? 4 : (streams == 2 ? 2 : 1);
     s.ct = 1;
     while (s.ct < max_ct && (N + 32 * s.ct - 1) / (32 * s.ct) >= 1024) s.ct *= 2;
@@ -310,9 +310,9 @@ static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
     const RowsShape s = rows_shape(p.M, p.N, p.K, NS);
 #define ROWS_CASE(MT_, CT_) \
     if (s.mt == MT_ && s.ct == CT_) return launch_rows<MT_, CT_, EPI>(p, s.waves, stream);
-    ROWS_CASE(2, 1) ROWS_CASE(4, 1)
-    if constexpr (NS <= 2) { ROWS_CASE(2, 2) ROWS_CASE(4, 2) }
-    if constexpr (NS == 1) { ROWS_CASE(2, 4) ROWS_CASE(4, 4) }
+    ROWS_CASE(1, 1) ROWS_CASE(2, 1) ROWS_CASE(4, 1)
+    if constexpr (NS <= 2) { ROWS_CASE(1, 2) ROWS_CASE(2, 2) ROWS_CASE(4, 2) }
+    if constexpr (NS == 1) { ROWS_CASE(1, 4) ROWS_CASE(2, 4) ROWS_CASE(4, 4) }
 #undef ROWS_CASE
     return static_cast<int>(hipErrorInvalidValue);
 }
@@ -326,7 +326,7 @@ extern "C" int celeg_gemm_rows_blocks(int M, int N, int K, int epi) {
     return (N + s.ct * 16 - 1) / (s.ct * 16);
 }
 
-// 16 < M <= 64 (fewer rows work too, at the cost of idle lanes), K % 32 == 0, bfloat16 a and
+// M <= 64 (made for 17 and more; fewer rows work too), K % 32 == 0, bfloat16 a and
 // w (in the layouts that the strides describe).  The fields of GemvParams that are read are
 // those of the products for up to 16 rows and the strides of the operands' groups of 8.
 extern "C" int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t stream) {

@@ -37,7 +37,7 @@ struct GemvParams {
     // (rows one after the other: K and 32; blocks of 32 k-values with the rows side by side
     // inside a block: 32 and rows * 32)
     long long w_row_stride, w_kb_stride;
-    // layouts that only the kernel for 17 to 64 rows reads: element (m, k) of a lies at
+    // layouts that only the kernel for 9 to 64 rows reads: element (m, k) of a lies at
     //   m * lda + (k / 8) * a_k8_stride + k % 8
     // (rows one after the other: 8; groups of 8 k-values with the rows side by side: rows * 8),
     // bfloat16 outputs out and out_bf16 likewise with ldo / out_k8_stride and ld_bf16 /

@@ -50,7 +50,11 @@ class HipOps:
         self._rope_tables = {}
         self.use_rope_table = True         # cos/sin of every position from a table made once
         self.use_sliced = True             # up to 16 bfloat16 rows: the k-sliced kernels
-        self.use_rows_kernel = True        # 17 to 64 bfloat16 rows: the kernel that streams the weights
+        self.use_rows_kernel = True        # 9 to 64 bfloat16 rows: the kernel that streams the weights
+        # fewest rows it is used for (it takes any number up to 64).  Measured per decode step: at 16
+        # rows it equals the k-sliced kernels on 1,024-wide layers and is 20 % faster on 2,048-wide
+        # ones (1.55 against 1.94 ms at the 2.6B shape); at 8 rows it loses 19 % on the former
+        self.rows_kernel_min_rows = 9
         self.last_stat_blocks = 0
         self.fused_linear_shape = 0        # 0: chosen from the sizes; 1..4 force a workgroup shape
 
@@ -105,7 +109,7 @@ class HipOps:
     @staticmethod
     def chunked_rows(rows: int, width: int, device, max_rows: int = 64) -> torch.Tensor:
         """Room for ``rows`` bfloat16 rows of ``width`` values in the layout that the products
-        for 17 to 64 rows read best: [width/8, max_rows, 8], returned as its view
+        for 9 to 64 rows read best: [width/8, max_rows, 8], returned as its view
         [rows, width/8, 8] (element (m, k) at [m, k // 8, k % 8])."""
         if width % 8 or rows > max_rows:
             raise KernelError("chunked_rows: the width must be a multiple of 8 and rows <= max_rows")
@@ -441,18 +445,19 @@ class HipOps:
     def residual_stat_blocks(self, rows: int, n: int, k: int) -> int:
         """How many partial sums of squares per row the "residual" epilogue of
         ``fused_linear`` leaves for these sizes (the rows ``stats_out`` needs)."""
-        if rows <= 16 and self.use_sliced:
-            return int(self._lib("gemv_slices").celeg_gemv_slices_blocks(
-                _c_int(rows), _c_int(n), _c_int(k)))
         if self.rows_kernel_ok(rows, k):
             return int(self._lib("gemm_rows").celeg_gemm_rows_blocks(
                 _c_int(rows), _c_int(n), _c_int(k), _c_int(self._EPILOGUES["residual"])))
+        if rows <= 16 and self.use_sliced:
+            return int(self._lib("gemv_slices").celeg_gemv_slices_blocks(
+                _c_int(rows), _c_int(n), _c_int(k)))
         return (n + 15) // 16
 
     def rows_kernel_ok(self, rows: int, *inner_sizes: int) -> bool:
         """Whether bfloat16 products of ``rows`` rows with these inner sizes go to the kernel
-        for 17 to 64 rows."""
-        return self.use_rows_kernel and 16 < rows <= 64 and all(k % 32 == 0 for k in inner_sizes)
+        for 9 to 64 rows."""
+        return self.use_rows_kernel and self.rows_kernel_min_rows <= rows <= 64 \
+            and all(k % 32 == 0 for k in inner_sizes)
 
     @staticmethod
     def pack_weight(w: torch.Tensor) -> torch.Tensor:
@@ -522,7 +527,7 @@ class HipOps:
         (``w`` is [3N, K]: B, C, x rows; ``conv`` = (taps [N, L], bias or None, state
         [slots, L, N], seq_slot [M]); one new token per request).
 
-        Up to 16 bfloat16 rows go to the k-sliced kernels, and 17 to 64 rows with an inner size
+        Up to 16 bfloat16 rows go to the k-sliced kernels, and 9 to 64 rows with an inner size
         that is a multiple of 32 to the kernel that streams the weights.  Both also take the form behind a
         norm whose weight the caller has folded into ``w``: ``a`` is then the bfloat16 copy
         of the stream and ``stats[row, :stat_blocks]`` its partial sums of squares, from which
@@ -589,12 +594,12 @@ class HipOps:
         prm.bias = bias.data_ptr() if bias is not None else None
         prm.M, prm.N, prm.K = M, N, K
         prm.out, prm.ldo = out.data_ptr(), ldo
-        sliced = norm_weight is None and M <= 16 and self.use_sliced
-        streamed = norm_weight is None and not sliced and self.rows_kernel_ok(M, K)
+        streamed = norm_weight is None and self.rows_kernel_ok(M, K)
+        sliced = norm_weight is None and not streamed and M <= 16 and self.use_sliced
         prm.a_k8_stride, prm.out_k8_stride, prm.w_q_stride = a_k8, out_k8, 8
         if (a.dim() == 3 or out.dim() == 3 or (out_bf16 is not None and out_bf16.dim() == 3)) \
                 and not streamed:
-            raise KernelError("fused_linear: operands with the rows side by side go with 17 to 64 rows")
+            raise KernelError("fused_linear: operands with the rows side by side go with the kernel for 9 to 64 rows")
         if out.dim() == 3 and out_dtype != torch.bfloat16:
             raise KernelError("fused_linear: a 32-bit output has its rows one after the other")
         if packed and not (sliced or streamed):
@@ -639,7 +644,7 @@ class HipOps:
         if streamed:
             code = self._lib("gemm_rows").celeg_gemm_rows(
                 ctypes.byref(prm), _c_int(self._EPILOGUES[epilogue]), self._stream())
-            self._check(code, f"fused_linear ({epilogue}, 17 to 64 rows)")
+            self._check(code, f"fused_linear ({epilogue}, 9 to 64 rows)")
             return out
         code = self._lib("gemv_fused").celeg_gemv_fused(
             ctypes.byref(prm), _c_int(1 if norm_weight is not None else 0),

@@ -16,7 +16,7 @@ import torch
 
 STAT_COLUMNS = 64   # most rows of a fused step (rows of the partial-sum table)
 # Most rows of the fused path: 64 where every inner size is a multiple of 32 (the kernel
-# for 17 to 64 rows); else 32, above which the library's product (with separate norm and
+# for 9 to 64 rows); else 32, above which the library's product (with separate norm and
 # activation kernels) is the faster one on MI355X.
 FUSED_MAX_ROWS = 64
 FUSED_MAX_ROWS_OLD_KERNEL = 32
@@ -50,16 +50,15 @@ def stream_stats(rt, width: int) -> torch.Tensor:
 def _side_by_side(rt, rows: int, width: int, *producer_inner: int) -> bool:
     """Whether a bfloat16 operand of ``width`` values a row, of a step of ``rows`` rows, lies
     with the rows side by side inside every group of 8 values (the layout that the kernel for
-    17 to 64 rows reads whole runs of memory from) rather than one row after the other: where
+    9 to 64 rows reads whole runs of memory from) rather than one row after the other: where
     that kernel both reads it and, if a product writes it (inner size ``producer_inner``),
     writes it."""
-    return rows > SLICED_MAX_ROWS and hasattr(rt.ops, "rows_kernel_ok") \
-        and rt.ops.rows_kernel_ok(rows, width, *producer_inner)
+    return hasattr(rt.ops, "rows_kernel_ok") and rt.ops.rows_kernel_ok(rows, width, *producer_inner)
 
 
 def operand_rows(rt, name: str, rows: int, width: int, *producer_inner: int) -> torch.Tensor:
     """Room for a bfloat16 operand of the fused products, [rows, width] (up to 16 rows, or
-    sizes the kernel for 17 to 64 rows does not take) or the view [rows, width/8, 8] of
+    sizes the kernel for 9 to 64 rows does not take) or the view [rows, width/8, 8] of
     [width/8, 64, 8]."""
     if _side_by_side(rt, rows, width, *producer_inner):
         return rt.ws.buf(name + "_side_by_side", (width // 8, STAT_COLUMNS, 8), torch.bfloat16).permute(1, 0, 2)[:rows]
@@ -73,10 +72,10 @@ def stream_bf16(rt, rows: int, width: int) -> torch.Tensor:
 
 def _sliced(rt, rows: int, inner: int) -> bool:
     """Whether a product of ``rows`` bfloat16 rows with this inner size takes the form with
-    the norm folded into the weights (the kernels for up to 16 and for 17 to 64 rows)."""
-    if rows <= SLICED_MAX_ROWS:
-        return getattr(rt.ops, "use_sliced", False)
-    return hasattr(rt.ops, "rows_kernel_ok") and rt.ops.rows_kernel_ok(rows, inner)
+    the norm folded into the weights (the kernels for up to 16 and for 9 to 64 rows)."""
+    if hasattr(rt.ops, "rows_kernel_ok") and rt.ops.rows_kernel_ok(rows, inner):
+        return True
+    return rows <= SLICED_MAX_ROWS and getattr(rt.ops, "use_sliced", False)
 
 
 def _pack(rt, w: torch.Tensor) -> torch.Tensor:
@@ -110,13 +109,14 @@ def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None
     blocks = getattr(rt, "stream_stat_blocks", 0)
     M = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
     streams = {"swiglu": 2, "conv": 3}.get(epilogue, 1)
+    streamed = hasattr(rt.ops, "rows_kernel_ok") and rt.ops.rows_kernel_ok(M, h.shape[1])
     if _sliced(rt, M, h.shape[1]) and w.dtype == torch.bfloat16 \
-            and (M > SLICED_MAX_ROWS or w.shape[0] // streams <= SLICED_MAX_COLUMNS):
+            and (streamed or w.shape[0] // streams <= SLICED_MAX_COLUMNS):
         # the stream's bfloat16 copy times the weight with the norm's weight folded in,
         # scaled by the rows' 1/rms at the end
         stats = stream_stats(rt, h.shape[1])
         xb = stream_bf16(rt, h.shape[0], h.shape[1])
-        if xb.dim() == 3 and M <= SLICED_MAX_ROWS:
+        if xb.dim() == 3 and not streamed:
             # few wanted rows of a step of many: the kernel for few rows reads rows that lie one
             # after the other, so the stream gets such a copy too
             xb = rt.ws.buf("stream_bf16", (STAT_COLUMNS, h.shape[1]), torch.bfloat16)[:h.shape[0]]
@@ -138,10 +138,13 @@ def linear_into_stream(rt, a, w, h, bias=None):
     """h += a w^T, leaving the partial sums of squares of the new rows (and, for few rows,
     the stream's bfloat16 copy)."""
     stats = stream_stats(rt, h.shape[1])
-    sliced = _sliced(rt, h.shape[0], a.shape[1] * (8 if a.dim() == 3 else 1))
+    inner = a.shape[1] * (8 if a.dim() == 3 else 1)
+    sliced = _sliced(rt, h.shape[0], inner)
+    xb = stream_bf16(rt, h.shape[0], h.shape[1]) if sliced else None
+    if xb is not None and xb.dim() == 3 and not rt.ops.rows_kernel_ok(h.shape[0], inner):
+        xb = None      # this product's kernel writes rows one after the other only: the next norm prepares the copy
     rt.ops.fused_linear(a, packed_weight(rt, w) if sliced else w, h, epilogue="residual", bias=bias,
-                        stats_out=stats,
-                        out_bf16=stream_bf16(rt, h.shape[0], h.shape[1]) if sliced else None)
+                        stats_out=stats, out_bf16=xb)
     rt.stream_stat_blocks = rt.ops.last_stat_blocks
-    rt.stream_has_bf16 = sliced
+    rt.stream_has_bf16 = xb is not None
     return h

@@ -147,7 +147,7 @@ def test_conv_epilogue_token_by_token_equals_the_whole_convolution(ops, M, H, ta
 
 SLICED = [(1, 64, 64), (3, 130, 200), (4, 1024, 1024), (5, 77, 352), (8, 3072, 1024), (8, 96, 4608),
           (13, 50, 1160), (16, 272, 1024)]
-# 17 to 64 rows: the kernel that streams the weights (inner sizes in steps of 32), at widths
+# 9 to 64 rows: the kernel that streams the weights (inner sizes in steps of 32), at widths
 # that give it one, two and four column tiles a workgroup, and few and many blocks of k
 STREAMED = [(17, 64, 64), (20, 130, 352), (32, 1024, 1024), (33, 77, 96), (48, 3072, 1024),
             (64, 272, 4608), (64, 8192, 128), (33, 14400, 64), (50, 1000, 32)]
@@ -171,7 +171,7 @@ def scaled_case(M, N, K, streams, seed):
 
 @pytest.mark.parametrize("M,N,K", SLICED + STREAMED)
 def test_sliced_products_behind_a_norm(ops, M, N, K):
-    """The form for up to 16 rows, and for 17 to 64: bfloat16 copy of the stream, norm weight folded into the
+    """The form for up to 16 rows, and for 9 to 64: bfloat16 copy of the stream, norm weight folded into the
     weights, 1/rms from the partial sums applied at the end; against the plain norm and
     product."""
     h, xb, stats, nw, w, folded, rows, x = scaled_case(M, N, K, 1, 40)
@@ -268,7 +268,7 @@ def test_packed_weights_give_the_same_bits(ops, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(17, 64, 64), (33, 80, 96), (40, 1024, 1024), (64, 272, 4608)])
 def test_operands_with_rows_side_by_side_give_the_same_bits(ops, M, N, K):
-    """For 17 to 64 rows the bfloat16 operands may lie as [width/8, 64, 8] (the rows side by
+    """For 9 to 64 rows the bfloat16 operands may lie as [width/8, 64, 8] (the rows side by
     side inside every group of 8 values): inputs and outputs in that layout give the same bits
     as rows that lie one after the other."""
     h, xb, stats, nw, w, folded, rows, x = scaled_case(M, N, K, 1, 90)

@@ -37,7 +37,8 @@ def plain_generate(cfg, W, prompt, n, generation=None, eos=()):
     return out
 
 
-@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("A", "bfloat16")])
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "float32"), ("A", "bfloat16"),
+                                        ("D", "float32"), ("D", "bfloat16")])
 def test_greedy_generation_through_the_entry_point(model_folders, name, dtype):
     from celeg_amd.engine import Engine
     from celeg_amd.sampling import GREEDY
