@@ -92,6 +92,7 @@ def serve(shape: str) -> int:
     import random
     import torch
     from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY
     from celeg_amd.weights import write_random_model
 
     cfg, load = SHAPES[shape]
@@ -107,12 +108,12 @@ def serve(shape: str) -> int:
                                     prefill_chunk_tokens=load["chunk"],
                                     context=cfg["max_position_embeddings"])
     # a short run first: kernels loaded, graphs captured for the decode batch sizes
-    engine.generate(prompts[:2], max_new_tokens=4, eos_token_ids=[])
+    engine.generate(prompts[:2], max_new_tokens=4, generation=GREEDY, eos_token_ids=[])
     for key in engine.metrics:
         engine.metrics[key] = type(engine.metrics[key])()
     torch.cuda.synchronize()
     start = time.perf_counter()
-    out = engine.generate(prompts, max_new_tokens=load["new_tokens"], eos_token_ids=[])
+    out = engine.generate(prompts, max_new_tokens=load["new_tokens"], generation=GREEDY, eos_token_ids=[])
     torch.cuda.synchronize()
     seconds = time.perf_counter() - start
     generated = sum(len(o) for o in out)

@@ -195,3 +195,72 @@ def test_portions_of_a_repeated_size_are_replayed(model_folders, name, dtype):
         ref = plain.model_logits(cfgp, W, toks)
         assert_close(got[rid], ref[[143, 144, 145]], dtype, f"{name}/{dtype}/replayed/{rid}")
     lm.cache.check()
+
+
+def many_requests_schedule(requests, tail, join_every=0):
+    """Every request's head in a step of its own, then decode steps that hold ALL requests
+    (one token each); with ``join_every`` the heads are spread between the decode steps instead,
+    a portion beside the tokens of the requests that already decode."""
+    ids = list(requests)
+    steps = []
+    heads = {rid: len(requests[rid]) - tail for rid in ids}
+    started = []
+    def head_entry(rid):
+        return {"id": rid, "tokens": requests[rid][:heads[rid]], "want": list(range(heads[rid]))}
+    if not join_every:
+        for rid in ids:
+            steps.append({"step": len(steps), "entries": [head_entry(rid)], "end": []})
+        started = list(ids)
+    done = {rid: 0 for rid in ids}
+    waiting = [rid for rid in ids if rid not in started]
+    while waiting or any(done[r] < tail for r in started):
+        entries = []
+        for rid in started:
+            if done[rid] < tail:
+                i = heads[rid] + done[rid]
+                entries.append({"id": rid, "tokens": requests[rid][i:i + 1], "want": [0]})
+                done[rid] += 1
+        joined = []
+        if waiting and (len(steps) % join_every == 0 if join_every else False):
+            rid = waiting.pop(0)
+            entries.insert(len(entries) // 2, head_entry(rid))     # a portion between single tokens
+            joined.append(rid)
+        if entries:
+            steps.append({"step": len(steps), "entries": entries,
+                          "end": [r for r in started if done[r] == tail and r not in
+                                  [x for st in steps for x in st["end"]]]})
+        else:
+            steps.append({"step": len(steps), "entries": [head_entry(waiting.pop(0))], "end": []})
+            joined.append(steps[-1]["entries"][0]["id"])
+        started += joined
+    return steps
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n_requests,join_every", [("D", 12, 0), ("D", 40, 0), ("B", 23, 0), ("D", 20, 2),
+                                                       ("A", 64, 0)])
+def test_many_requests_decoding_together(model_folders, name, n_requests, join_every, dtype):
+    """Decode steps of 9 to 64 rows (the products for many rows, their convolution and residual
+    epilogues, the decode attention for batches), and portions joining between the single
+    tokens of requests that already decode: every request's logits equal the plain ones."""
+    from celeg_amd.engine import load_model
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders(name, storage, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    vocab = cfg["vocab_size"]
+    tail = 30 if join_every else 6
+    lengths = [tail + 3 + (7 * i) % 50 for i in range(n_requests)]
+    reqs = {f"m{i}": random_tokens(vocab, n, seed=900 + i) for i, n in enumerate(lengths)}
+    steps = many_requests_schedule(reqs, tail, join_every)
+    most = max(len(s["entries"]) for s in steps)
+    assert most == n_requests if not join_every else most >= 12
+    pages = sum((n + 15) // 16 for n in lengths)
+    lm = load_model(folder, dtype=dtype, device="cuda:0", page_tokens=16, n_pages=pages,
+                    max_requests=n_requests, max_batched_tokens=128)
+    got = EngineDriver(lm).run(steps)
+    for rid in list(reqs)[::max(1, n_requests // 8)]:
+        ref = plain.model_logits(cfg, W, reqs[rid])
+        assert_close(got[rid], ref, dtype, f"{name}/{dtype}/{n_requests} together/{rid}")
+    lm.cache.check()
+    assert lm.cache.n_free_slots == n_requests and lm.cache.free_pages() == [pages]
