@@ -169,7 +169,9 @@ void gemm_rows_kernel(const GemvParams p) {
 #pragma unroll
         for (int s = 0; s < SC; ++s) acc[t][s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    bf16x8_t a0[MT], w0[SC], a1[MT], w1[SC];
+    // D blocks of 32 values of k in flight (four where the registers hold them were no faster)
+    constexpr int D = 2;
+    bf16x8_t av_[D][MT], wv_[D][SC];
     auto fetch = [&](int kb, bf16x8_t (&av)[MT], bf16x8_t (&wv)[SC]) {
 #pragma unroll
         for (int s = 0; s < SC; ++s)
@@ -185,8 +187,9 @@ void gemm_rows_kernel(const GemvParams p) {
             for (int s = 0; s < SC; ++s)
                 acc[t][s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[t], wv[s], acc[t][s], 0, 0, 0);
     };
-    if (kb_begin < kb_end) fetch(kb_begin, a0, w0);
-    if (kb_begin + 1 < kb_end) fetch(kb_begin + 1, a1, w1);
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if (kb_begin + d < kb_end) fetch(kb_begin + d, av_[d], wv_[d]);
 
     // ---- what the end of this thread's first output needs (asked for behind the first weights)
     const int e0 = min(static_cast<int>(threadIdx.x), ROWS * COLS - 1);
@@ -212,11 +215,12 @@ void gemm_rows_kernel(const GemvParams p) {
         if (sub == 0) s_scale[r] = 1.0f / sqrtf(ssq / static_cast<float>(K) + p.eps);
     }
 
-    for (int kb = kb_begin; kb < kb_end; kb += 2) {
-        multiply(a0, w0);
-        if (kb + 2 < kb_end) fetch(kb + 2, a0, w0);
-        if (kb + 1 < kb_end) multiply(a1, w1);
-        if (kb + 3 < kb_end) fetch(kb + 3, a1, w1);
+    for (int kb = kb_begin; kb < kb_end; kb += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            if (kb + d < kb_end) multiply(av_[d], wv_[d]);
+            if (kb + d + D < kb_end) fetch(kb + d + D, av_[d], wv_[d]);
+        }
     }
 
     // acc[t][s]: lane l holds column l%16 of rows 4*(l/16)..+3 of the tile
