@@ -66,17 +66,14 @@ template <> struct ConvVec<bf16> {
 #define CONV_VEC_MAX_TAPS 8
 
 template <typename T>
-__global__ void short_conv_fwd_vec_kernel(
-    const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
+__device__ __forceinline__ void short_conv_token_vec(
+    int t, int ch, const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ state, size_t state_slot_stride,
     T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_seqlens, int width, int taps) {
     constexpr int VEC = ConvVec<T>::n;
     typedef typename ConvVec<T>::raw raw;
-    const int ch = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
-    if (ch >= width) return;
-    const int t = blockIdx.x;
     const int s = token_seq[t];
     const int start = seq_start[s];
     const int row0 = cu_seqlens[s];
@@ -128,6 +125,78 @@ __global__ void short_conv_fwd_vec_kernel(
 }
 
 template <typename T>
+__global__ void short_conv_fwd_vec_kernel(
+    const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
+    const float* __restrict__ bias, const float* __restrict__ state, size_t state_slot_stride,
+    T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_seq,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_seqlens, int width, int taps) {
+    const int ch = (blockIdx.y * blockDim.x + threadIdx.x) * ConvVec<T>::n;
+    if (ch >= width) return;
+    short_conv_token_vec<T>(blockIdx.x, ch, bcx, ld_bcx, w, bias, state, state_slot_stride, out, positions,
+                            token_seq, seq_start, seq_slot, cu_seqlens, width, taps);
+}
+
+// The same for TT tokens in a row per thread: where they all belong to one request and every
+// tap lies in rows of this step, a row's B and x are read once for all the tokens that use it
+// (a window that slides down the rows) instead of once per tap.  The sums are formed in the
+// same order as above, so the results are the same bits.
+#define CONV_BLOCK_TOKENS 8
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
+    const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
+    const float* __restrict__ bias, const float* __restrict__ state, size_t state_slot_stride,
+    T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_seq,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_seqlens, int width, int n_tokens) {
+    constexpr int VEC = ConvVec<T>::n;
+    constexpr int TT = CONV_BLOCK_TOKENS;
+    typedef typename ConvVec<T>::raw raw;
+    const int ch = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
+    if (ch >= width) return;
+    const int t0 = blockIdx.x * TT;
+    const int n = min(TT, n_tokens - t0);
+    const int s = token_seq[t0];
+    // the same for the whole workgroup
+    if (n < TT || token_seq[t0 + TT - 1] != s || t0 - (TAPS - 1) < cu_seqlens[s]) {
+        for (int j = 0; j < n; ++j)
+            short_conv_token_vec<T>(t0 + j, ch, bcx, ld_bcx, w, bias, state, state_slot_stride, out,
+                                    positions, token_seq, seq_start, seq_slot, cu_seqlens, width, TAPS);
+        return;
+    }
+    raw bv[TT + TAPS - 1], xv[TT + TAPS - 1], cv[TT];
+#pragma unroll
+    for (int j = 0; j < TT + TAPS - 1; ++j) {
+        const T* row = bcx + static_cast<size_t>(t0 - (TAPS - 1) + j) * ld_bcx;
+        bv[j] = *reinterpret_cast<const raw*>(row + ch);
+        xv[j] = *reinterpret_cast<const raw*>(row + 2 * width + ch);
+    }
+#pragma unroll
+    for (int j = 0; j < TT; ++j)
+        cv[j] = *reinterpret_cast<const raw*>(bcx + static_cast<size_t>(t0 + j) * ld_bcx + width + ch);
+    float wt[VEC][TAPS], b0[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        b0[i] = bias ? bias[ch + i] : 0.f;
+#pragma unroll
+        for (int tap = 0; tap < TAPS; ++tap) wt[i][tap] = w[static_cast<size_t>(ch + i) * TAPS + tap];
+    }
+#pragma unroll
+    for (int j = 0; j < TT; ++j) {
+        raw o;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            float conv = b0[i];
+#pragma unroll
+            for (int tap = 0; tap < TAPS; ++tap)
+                conv = fmaf(wt[i][tap], ConvVec<T>::at(bv[j + tap], i) * ConvVec<T>::at(xv[j + tap], i), conv);
+            ConvVec<T>::set(o, i, ConvVec<T>::at(cv[j], i) * conv);
+        }
+        *reinterpret_cast<raw*>(out + static_cast<size_t>(t0 + j) * width + ch) = o;
+    }
+}
+
+template <typename T>
 __global__ void short_conv_state_kernel(
     const T* __restrict__ bcx, int ld_bcx, float* __restrict__ state, size_t state_slot_stride,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
@@ -169,6 +238,24 @@ extern "C" int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const fl
         aligned(bcx) && aligned(out)) {
         const int threads = min(256, (width / vec + 63) / 64 * 64);
         dim3 vblock(threads), vgrid(n_tokens, (width / vec + threads - 1) / threads);
+        if (n_tokens >= 64 && taps >= 2 && taps <= 4) {
+            dim3 bgrid((n_tokens + CONV_BLOCK_TOKENS - 1) / CONV_BLOCK_TOKENS, vgrid.y);
+#define CELEG_CONV_BLOCK(T_, TAPS_)                                                                \
+    hipLaunchKernelGGL((short_conv_fwd_block_kernel<T_, TAPS_>), bgrid, vblock, 0, stream,          \
+                       static_cast<const T_*>(bcx), ld_bcx, w, bias, state, state_slot_stride,      \
+                       static_cast<T_*>(out), positions, token_seq, seq_start, seq_slot, cu_seqlens, \
+                       width, n_tokens);                                                           \
+    hipLaunchKernelGGL(short_conv_state_kernel<T_>, grid_state, block, 0, stream,                   \
+                       static_cast<const T_*>(bcx), ld_bcx, state, state_slot_stride, seq_start,    \
+                       seq_slot, cu_seqlens, width, taps)
+#define CELEG_CONV_BLOCK_T(T_)                                                                     \
+    if (taps == 2) { CELEG_CONV_BLOCK(T_, 2); } else if (taps == 3) { CELEG_CONV_BLOCK(T_, 3); }     \
+    else { CELEG_CONV_BLOCK(T_, 4); }
+            if (dtype == CELEG_F32) { CELEG_CONV_BLOCK_T(float) } else { CELEG_CONV_BLOCK_T(bf16) }
+#undef CELEG_CONV_BLOCK_T
+#undef CELEG_CONV_BLOCK
+            return CELEG_LAUNCH_RESULT();
+        }
         if (dtype == CELEG_F32) {
             hipLaunchKernelGGL(short_conv_fwd_vec_kernel<float>, vgrid, vblock, 0, stream,
                                static_cast<const float*>(bcx), ld_bcx, w, bias, state,

@@ -175,6 +175,48 @@ def test_short_conv_whole_chunked_and_token_by_token(ops, dtype, width, taps, bi
         torch.testing.assert_close(state[slot], want_state, rtol=0, atol=0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,taps,bias", [(128, 3, True), (1032, 4, False), (96, 2, True), (64, 5, False)])
+def test_short_conv_long_portions_of_several_requests(ops, dtype, width, taps, bias):
+    """Steps of 64 and more tokens (the kernel that takes eight tokens in a row per thread):
+    two requests per step, so that blocks of eight tokens straddle the border between them, begin
+    at a request's first token, and continue from its state at positions inside a block."""
+    from celeg_amd.engine import StepEntry
+    from celeg_amd.parts.base import StateNeed
+    lengths = [131, 77]
+    data = [randn(n, 3 * width, seed=60 + i, dtype=dtype) for i, n in enumerate(lengths)]
+    w = randn(width, taps, seed=63)
+    b = randn(width, seed=64) if bias else None
+    cache = make_cache(0, 0, 0, dtype, states=[(0, StateNeed("bx", (taps, width)))], slots=4)
+    slots = [cache.open() for _ in lengths]
+    state = cache.layer_cache(0).states["bx"]
+    got = [[] for _ in lengths]
+    pos = [0, 0]
+    for cuts in ((70, 37), (33, 40), (28, 0)):
+        entries, parts = [], []
+        for i, n in enumerate(cuts):
+            if n:
+                entries.append(StepEntry(slots[i], pos[i], [0] * n))
+                parts.append((i, pos[i], n))
+        batch, keep = build_batch(ops, cache, entries)
+        parts = [parts[j] for j in batch.entry_order]
+        bcx = torch.cat([data[i][p:p + n] for i, p, n in parts]).contiguous()
+        out = torch.empty(bcx.shape[0], width, dtype=dtype, device=DEV)
+        ops.short_conv(bcx, w, b, state, out, batch)
+        torch.cuda.synchronize()
+        row = 0
+        for i, p, n in parts:
+            got[i].append(out[row:row + n].double().cpu())
+            row += n
+            pos[i] += n
+    assert pos == lengths
+    for i in range(len(lengths)):
+        ref = plain.short_conv(data[i].cpu(), w.cpu(), b.cpu() if bias else None)
+        torch.testing.assert_close(torch.cat(got[i]), ref, **tol(dtype))
+        bx = data[i][:, :width].float() * data[i][:, 2 * width:].float()
+        torch.testing.assert_close(state[slots[i]], bx[-taps:], rtol=0, atol=0)
+
+
 def test_short_conv_reference_vector(ops):
     # tests/reference_test.cpp:68-73: hidden 2, L 3, bcx {1,1 | 1,1 | 2,4}, weights
     # {1,2,3 ; 1,2,3} channel-major, position 0, zero state -> {6, 12}
