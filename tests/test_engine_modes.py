@@ -239,11 +239,12 @@ def many_requests_schedule(requests, tail, join_every=0):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,n_requests,join_every", [("D", 12, 0), ("D", 40, 0), ("B", 23, 0), ("D", 20, 2),
-                                                       ("A", 64, 0)])
+                                                       ("A", 64, 0), ("D", 100, 0)])
 def test_many_requests_decoding_together(model_folders, name, n_requests, join_every, dtype):
     """Decode steps of 9 to 64 rows (the products for many rows, their convolution and residual
-    epilogues, the decode attention for batches), and portions joining between the single
-    tokens of requests that already decode: every request's logits equal the plain ones."""
+    epilogues, the decode attention for batches), of 100 rows (the library's products), and
+    portions joining between the single tokens of requests that already decode: every
+    request's logits equal the plain ones."""
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders(name, storage, WEIGHT_STD)
