@@ -398,6 +398,14 @@ __device__ __forceinline__ void decode_range(
     const int first_page = kb >> page_shift;
     const int last_page = k_hi >> page_shift;
     const int my_page = pages[min(first_page + lane, last_page)];
+    // q is asked for before the keys (whose addresses wait for the page ids)
+    uint4 qraw[GH][DL / 8];
+#pragma unroll
+    for (int g = 0; g < GH; ++g) {
+        const bf16* qrow = q + static_cast<size_t>(t) * ldq + static_cast<size_t>(h0 + g) * HD + seg * DL;
+#pragma unroll
+        for (int v8 = 0; v8 < DL / 8; ++v8) qraw[g][v8] = *reinterpret_cast<const uint4*>(qrow + v8 * 8);
+    }
 
     // keys: 8 rounds of 8 keys, a lane reads DL values of its key
     uint4 kraw[8][DL / 8];
@@ -427,11 +435,16 @@ __device__ __forceinline__ void decode_range(
     }
     float qf[GH][DL];
 #pragma unroll
-    for (int g = 0; g < GH; ++g) {
-        const bf16* qrow = q + static_cast<size_t>(t) * ldq + static_cast<size_t>(h0 + g) * HD + seg * DL;
+    for (int g = 0; g < GH; ++g)
 #pragma unroll
-        for (int d = 0; d < DL; ++d) qf[g][d] = to_float(qrow[d]) * scale;
-    }
+        for (int v8 = 0; v8 < DL / 8; ++v8) {
+            const uint32_t w[4] = {qraw[g][v8].x, qraw[g][v8].y, qraw[g][v8].z, qraw[g][v8].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                qf[g][v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16) * scale;
+                qf[g][v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u) * scale;
+            }
+        }
 
     float sc[8][GH];
 #pragma unroll
@@ -774,7 +787,7 @@ extern "C" int celeg_attention_decode_bf16(
     if (n_rows <= 0) return 0;
     const int group = q_heads / kv_heads;
     if (q_heads % kv_heads || page_tokens < 16 || (page_tokens & (page_tokens - 1)) || n_splits <= 0 ||
-        (ldq % 8))
+        (ldq % 8) || (reinterpret_cast<uintptr_t>(q) & 15))     // q is read 16 bytes at a time
         return static_cast<int>(hipErrorInvalidValue);
     const int page_shift = __builtin_ctz(page_tokens);
     const int gh = (group % 4 == 0) ? 4 : ((group % 2 == 0) ? 2 : 1);
