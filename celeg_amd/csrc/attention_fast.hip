@@ -1,6 +1,6 @@
 // bfloat16 attention over the paged cache for gfx950: an MFMA kernel for the rows of
-// prompt portions (and mixed batches), and a split-key kernel for batches in which
-// every request brings one row (decode).
+// prompt portions (and mixed batches), and MFMA kernels for batches in which every request
+// brings one row (decode): the query heads that share a key/value head are the rows.
 //
 // Cache layout of a group (one page id covers all layers of the group):
 //   K [pages, layers, kv_heads, page_tokens, head_dim]   one key after the other
@@ -373,194 +373,8 @@ extern "C" int celeg_attention_rows_bf16(
 }
 
 // ================================================================ one row per request
-// One wavefront per (64 keys, GH query heads that share a key/value head, request): all
-// its loads (the page ids, then the 64 keys and the 64 values) are in flight before
-// anything is computed.  For q.k a lane owns (key j, an eighth of head_dim) and eight
-// lanes add up a score; for p.v a lane owns a dimension and reads its row of the
-// transposed V.  Partial (max, sum, accumulator) go to a workspace and a second kernel
-// joins the ranges of 64 keys.
+// Decode attention works on rounds of 64 keys.
 #define DEC_KEYS 64
-
-// The work on one range of 64 keys [kb, kb + 63] cut to [k_lo, k_hi] (not empty), by one
-// wavefront: scores, probabilities relative to the range's own maximum (left in ps for the
-// second product), and the accumulators.  ps: this wavefront's own GH x 64 floats of LDS.
-template <int HD, int GH>
-__device__ __forceinline__ void decode_range(
-    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
-    const bf16* __restrict__ v_pool, const int* __restrict__ pages, int t, int h0, int kvh, int kb,
-    int k_lo, int k_hi, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer,
-    float scale, float (*ps)[DEC_KEYS], float (&m)[GH], float (&l)[GH], float (&acc)[GH][HD / 64]) {
-    constexpr int DL = HD / 8;    // dims of a key a lane multiplies
-    constexpr int DD = HD / 64;   // output dims a lane accumulates
-    const int lane = threadIdx.x & 63;
-    const int j8 = lane >> 3, seg = lane & 7;
-    // page ids of the range: lane i holds the i-th page that the 64 keys touch
-    const int first_page = kb >> page_shift;
-    const int last_page = k_hi >> page_shift;
-    const int my_page = pages[min(first_page + lane, last_page)];
-    // q is asked for before the keys (whose addresses wait for the page ids)
-    uint4 qraw[GH][DL / 8];
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-        const bf16* qrow = q + static_cast<size_t>(t) * ldq + static_cast<size_t>(h0 + g) * HD + seg * DL;
-#pragma unroll
-        for (int v8 = 0; v8 < DL / 8; ++v8) qraw[g][v8] = *reinterpret_cast<const uint4*>(qrow + v8 * 8);
-    }
-
-    // keys: 8 rounds of 8 keys, a lane reads DL values of its key
-    uint4 kraw[8][DL / 8];
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int keyc = min(max(kb + it * 8 + j8, k_lo), k_hi);
-        const int page = __shfl(my_page, (keyc >> page_shift) - first_page, 64);
-        const bf16* kp = k_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
-                         static_cast<size_t>(keyc & (page_tokens - 1)) * HD + seg * DL;
-#pragma unroll
-        for (int v8 = 0; v8 < DL / 8; ++v8) kraw[it][v8] = *reinterpret_cast<const uint4*>(kp + v8 * 8);
-    }
-    // values: 4 groups of 16 keys, a lane reads the 16 values of its dimension(s)
-    uint4 vraw[4][DD][2];
-#pragma unroll
-    for (int pg = 0; pg < 4; ++pg) {
-        const int key0 = min(max(kb + pg * 16, k_lo & ~15), k_hi & ~15);   // a group inside the range
-        const int page = __shfl(my_page, (key0 >> page_shift) - first_page, 64);
-        const bf16* vbase = v_pool + kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD) +
-                            (key0 & (page_tokens - 1));
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd)
-#pragma unroll
-            for (int v8 = 0; v8 < 2; ++v8)
-                vraw[pg][dd][v8] = *reinterpret_cast<const uint4*>(
-                    vbase + static_cast<size_t>(lane + 64 * dd) * page_tokens + v8 * 8);
-    }
-    float qf[GH][DL];
-#pragma unroll
-    for (int g = 0; g < GH; ++g)
-#pragma unroll
-        for (int v8 = 0; v8 < DL / 8; ++v8) {
-            const uint32_t w[4] = {qraw[g][v8].x, qraw[g][v8].y, qraw[g][v8].z, qraw[g][v8].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                qf[g][v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16) * scale;
-                qf[g][v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u) * scale;
-            }
-        }
-
-    float sc[8][GH];
-#pragma unroll
-    for (int it = 0; it < 8; ++it) {
-        const int key = kb + it * 8 + j8;
-        const bool valid = key >= k_lo && key <= k_hi;
-        float kf[DL];
-#pragma unroll
-        for (int v8 = 0; v8 < DL / 8; ++v8) {
-            const uint32_t w[4] = {kraw[it][v8].x, kraw[it][v8].y, kraw[it][v8].z, kraw[it][v8].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                kf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
-                kf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < GH; ++g) {
-            float dot = 0.f;
-#pragma unroll
-            for (int d = 0; d < DL; ++d) dot = fmaf(qf[g][d], kf[d], dot);
-            dot += __shfl_xor(dot, 1, 64);
-            dot += __shfl_xor(dot, 2, 64);
-            dot += __shfl_xor(dot, 4, 64);
-            sc[it][g] = valid ? dot : -INFINITY;
-        }
-    }
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-        float mx = sc[0][g];
-#pragma unroll
-        for (int it = 1; it < 8; ++it) mx = fmaxf(mx, sc[it][g]);
-        mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));   // finite: the range holds a key
-        float psum = 0.f;
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-            const float p = expf(sc[it][g] - mx);
-            psum += p;
-            if (seg == 0) ps[g][it * 8 + j8] = p;
-        }
-        psum += __shfl_xor(psum, 8, 64);    // the eight lanes of a key hold the same p:
-        psum += __shfl_xor(psum, 16, 64);   // add over keys only
-        psum += __shfl_xor(psum, 32, 64);
-        m[g] = mx;
-        l[g] = psum;
-    }
-    // ps is this wavefront's own: its lanes only have to see each other's writes
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int g = 0; g < GH; ++g)
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) acc[g][dd] = 0.f;
-#pragma unroll
-    for (int pg = 0; pg < 4; ++pg) {
-        // groups outside the range were redirected to one inside: their p are all zero
-        const int key0 = kb + pg * 16;
-        if (key0 > k_hi || key0 + 15 < k_lo) continue;
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) {
-            float vf[16];
-#pragma unroll
-            for (int v8 = 0; v8 < 2; ++v8) {
-                const uint32_t w[4] = {vraw[pg][dd][v8].x, vraw[pg][dd][v8].y, vraw[pg][dd][v8].z,
-                                       vraw[pg][dd][v8].w};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    vf[v8 * 8 + 2 * i] = __uint_as_float(w[i] << 16);
-                    vf[v8 * 8 + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-                }
-            }
-#pragma unroll
-            for (int g = 0; g < GH; ++g)
-#pragma unroll
-                for (int j = 0; j < 16; ++j) acc[g][dd] = fmaf(ps[g][pg * 16 + j], vf[j], acc[g][dd]);
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // ps may be written again by the caller's next range
-    __builtin_amdgcn_wave_barrier();
-}
-
-template <int HD, int GH>
-__global__ __launch_bounds__(64) void attention_decode_kernel(
-    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
-    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
-    const int* __restrict__ token_slot, const int* __restrict__ positions,
-    float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
-    int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer, float scale,
-    int window) {
-    constexpr int DD = HD / 64;
-    __shared__ float ps[GH][DEC_KEYS];
-    const int split = blockIdx.x, hb = blockIdx.y, t = blockIdx.z;
-    const int lane = threadIdx.x;
-    const int pos = positions[t];
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int kb = split * DEC_KEYS;
-    const int k_lo = max(lo, kb);
-    const int k_hi = min(pos, kb + DEC_KEYS - 1);
-    if (k_lo > k_hi) return;
-    const int h0 = hb * GH;
-    const int kvh = h0 / (q_heads / kv_heads);
-    const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
-    float m[GH], l[GH], acc[GH][DD];
-    decode_range<HD, GH>(q, ldq, k_pool, v_pool, pages, t, h0, kvh, kb, k_lo, k_hi, kv_heads,
-                         page_tokens, page_shift, n_layers, layer, scale, ps, m, l, acc);
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-        const size_t idx = (static_cast<size_t>(t) * q_heads + h0 + g) * n_splits + split;
-        if (lane == 0) { ws_ml[2 * idx] = m[g]; ws_ml[2 * idx + 1] = l[g]; }
-#pragma unroll
-        for (int dd = 0; dd < DD; ++dd) ws_o[idx * HD + lane + 64 * dd] = acc[g][dd];
-    }
-}
 
 // Joins the ranges of one (request, query head): out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
 template <int HD>
@@ -611,22 +425,25 @@ __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
     for (int dd = 0; dd < HD / 64; ++dd) orow[lane + 64 * dd] = from_float<bf16>(acc[dd] / denom);
 }
 
-// Decode attention without a second kernel, for batches that fill the chip: one workgroup
-// per (request, key/value head, chunk of 16 query heads of its group).  The heads of the
-// group are the rows of matrix instructions, so the work per key does not grow with the
-// group; the wavefronts take rounds of 64 keys in turn, each keeps a running maximum, sum
-// and output of its own, and they meet in LDS.
+// Decode attention: the query heads of a key/value head (up to 16 of them a workgroup) are
+// the rows of matrix instructions, so the work per key does not grow with the group.  Two
+// forms.  For batches that fill the chip, one workgroup per (request, key/value head, chunk of
+// 16 heads) and no second kernel: its wavefronts take rounds of 64 keys in turn, each keeps
+// a running maximum, sum and output of its own, and they meet in LDS.  For few requests
+// (SPLIT), a workgroup of one wavefront per round of 64 keys, so that a long context spreads
+// over the chip; the rounds' (max, sum, output) go to a workspace and
+// attention_decode_reduce_kernel joins them.
 //   S^T[key, head] = K Q^T : a lane holds head lane%16, keys 4*(lane/16)..+3 of a 16-key tile;
 //   O^T[dim, head] = V^T P : P's operand wants 8 keys a lane, which are rows 4q..4q+3 of two
 //   tiles: tile 2j holds keys 32j + 8*(row/4) + row%4, tile 2j+1 those + 4, so that a lane's
 //   eight p are eight keys in a row and V (stored [dim][key] in a page) is read 16 bytes a lane.
-template <int HD, int WAVES>
+template <int HD, int WAVES, bool SPLIT>
 __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ token_slot, const int* __restrict__ positions, bf16* __restrict__ out,
     int ldo, int kv_heads, int group, int page_tokens, int page_shift, int n_layers, int layer,
-    float scale, int window) {
+    float scale, int window, float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits) {
     constexpr int KS = HD / 32;   // steps of 32 dims in q.k
     constexpr int DT = HD / 16;   // 16-dim tiles of the output
     extern __shared__ float smem_heads[];
@@ -655,7 +472,9 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    for (int r = lo / DEC_KEYS + wave; r <= pos / DEC_KEYS; r += WAVES) {
+    const int r_first = SPLIT ? static_cast<int>(blockIdx.z) : lo / DEC_KEYS + wave;
+    if (SPLIT && (r_first < lo / DEC_KEYS || r_first > pos / DEC_KEYS)) return;     // the whole workgroup
+    for (int r = r_first; r <= pos / DEC_KEYS; r += SPLIT ? (1 << 30) : WAVES) {
         const int kb = r * DEC_KEYS;
         const int k_lo = max(lo, kb), k_hi = min(pos, kb + DEC_KEYS - 1);
         const int first_page = kb >> page_shift, last_page = k_hi >> page_shift;
@@ -728,6 +547,16 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt][j], pb, o[dt], 0, 0, 0);
         }
     }
+    if (SPLIT) {
+        if (c < gp) {
+            const size_t idx = (static_cast<size_t>(t) * (kv_heads * group) + h0 + c) * n_splits + blockIdx.z;
+            if (qd == 0) { ws_ml[2 * idx] = m_run; ws_ml[2 * idx + 1] = l_run; }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                *reinterpret_cast<floatx4_t*>(ws_o + idx * HD + 16 * dt + 4 * qd) = o[dt];
+        }
+        return;
+    }
     if (c < gp) {
         if (qd == 0) {
             part_ml[(wave * gp + c) * 2] = m_run;
@@ -765,16 +594,16 @@ static int launch_decode_heads(const void* q, int ldq, const void* k_pool, const
     const size_t lds = static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES>),
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, false>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (err != hipSuccess) return static_cast<int>(err);
         raised = true;
     }
-    hipLaunchKernelGGL((attention_decode_heads_kernel<HD, WAVES>), dim3(kv_heads * chunks, n_rows),
+    hipLaunchKernelGGL((attention_decode_heads_kernel<HD, WAVES, false>), dim3(kv_heads * chunks, n_rows),
                        dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
                        table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
-                       group, page_tokens, page_shift, n_layers, layer, scale, window);
+                       group, page_tokens, page_shift, n_layers, layer, scale, window, nullptr, nullptr, 0);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -790,13 +619,13 @@ extern "C" int celeg_attention_decode_bf16(
         (ldq % 8) || (reinterpret_cast<uintptr_t>(q) & 15))     // q is read 16 bytes at a time
         return static_cast<int>(hipErrorInvalidValue);
     const int page_shift = __builtin_ctz(page_tokens);
-    const int gh = (group % 4 == 0) ? 4 : ((group % 2 == 0) ? 2 : 1);
-    // whole: 0 the split-key kernels, 1 one workgroup per (request, key/value head), -1 decide
-    // here: one workgroup each, and no second kernel, once there are enough of them (measured
-    // at context 2,100 with 8 key/value heads: groups of 4 heads gain from 8 requests on, 1.48
-    // against 1.53 ms a step of the 2.6B shape, groups of 2 from 16 on, 0.70 against 0.72 ms of
-    // the 350M shape; below that a workgroup is bound by what one compute unit can pull).
-    if (whole < 0) whole = kv_heads * n_rows >= (group >= 3 ? 64 : 128) ? 1 : 0;
+    const int chunks = (group + 15) / 16;
+    // whole: 0 a workgroup per round of 64 keys and a second kernel, 1 one workgroup per
+    // (request, key/value head), -1 decide here: the latter once there are enough of them to
+    // fill the chip (measured at context 2,100 with 8 key/value heads, groups of 2 and of 4
+    // heads: equal at 16 requests, one workgroup each 5 to 8 % of a decode step faster at 32
+    // and 64 requests, a workgroup per round 2 to 5 % faster at 1 to 8).
+    if (whole < 0) whole = kv_heads * chunks * n_rows >= 192 ? 1 : 0;
     if (whole) {
         if (head_dim == 64)
             return launch_decode_heads<64>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
@@ -808,22 +637,19 @@ extern "C" int celeg_attention_decode_bf16(
                                             n_layers, layer, scale, window, stream);
         return static_cast<int>(hipErrorInvalidValue);
     }
-    dim3 grid(n_splits, q_heads / gh, n_rows), block(64);
-#define CELEG_DEC(HD_, GH_)                                                                      \
-    hipLaunchKernelGGL((attention_decode_kernel<HD_, GH_>), grid, block, 0, stream,              \
+    dim3 sgrid(kv_heads * chunks, n_rows, n_splits);
+#define CELEG_SPLIT_HEADS(HD_)                                                                   \
+    hipLaunchKernelGGL((attention_decode_heads_kernel<HD_, 1, true>), sgrid, dim3(64), 0, stream, \
                        static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
                        static_cast<const bf16*>(v_pool), table, table_stride, token_slot,        \
-                       positions, ws_o, ws_ml, n_splits, q_heads, kv_heads,                      \
-                       page_tokens, page_shift, n_layers, layer, scale, window)
-#define CELEG_DEC_HD(HD_)                                                                        \
-    if (gh == 4) CELEG_DEC(HD_, 4); else if (gh == 2) CELEG_DEC(HD_, 2); else CELEG_DEC(HD_, 1);  \
+                       positions, static_cast<bf16*>(out), ldo, kv_heads, group, page_tokens,    \
+                       page_shift, n_layers, layer, scale, window, ws_o, ws_ml, n_splits);       \
     hipLaunchKernelGGL(attention_decode_reduce_kernel<HD_>, dim3(q_heads, n_rows), dim3(64), 0,  \
                        stream, ws_o, ws_ml, positions, static_cast<bf16*>(out), ldo, q_heads,    \
                        n_splits, window)
-    if (head_dim == 64) { CELEG_DEC_HD(64); }
-    else if (head_dim == 128) { CELEG_DEC_HD(128); }
+    if (head_dim == 64) { CELEG_SPLIT_HEADS(64); }
+    else if (head_dim == 128) { CELEG_SPLIT_HEADS(128); }
     else return static_cast<int>(hipErrorInvalidValue);
-#undef CELEG_DEC_HD
-#undef CELEG_DEC
+#undef CELEG_SPLIT_HEADS
     return CELEG_LAUNCH_RESULT();
 }
