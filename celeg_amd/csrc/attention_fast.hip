@@ -376,53 +376,56 @@ extern "C" int celeg_attention_rows_bf16(
 // Decode attention works on rounds of 64 keys.
 #define DEC_KEYS 64
 
-// Joins the ranges of one (request, query head): out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
+// Joins the rounds of one (request, query head): out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
+// A lane owns an output dimension (and the (m, l) of rounds lane, lane + 64, ..).  The rounds'
+// outputs are asked for 32 at a time without conditions, the first 32 before anything is
+// waited for, so that a context of 2,048 keys costs two trips to memory.
 template <int HD>
 __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int* __restrict__ positions, bf16* __restrict__ out, int ldo, int q_heads, int n_splits,
     int window) {
+    constexpr int DD = HD / 64, CH = 32;
     const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int first = lo / DEC_KEYS, last = pos / DEC_KEYS;
-    const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits;
-    float m = -INFINITY;
-    for (int i0 = first; i0 <= last; i0 += 64) {
-        const int i = i0 + lane;
-        m = fmaxf(m, i <= last ? ws_ml[2 * (base + i)] : -INFINITY);
-    }
-    m = wave_max(m);
-    float denom = 0.f, acc[HD / 64];
+    const int first = lo / DEC_KEYS, n_all = pos / DEC_KEYS - first + 1;
+    const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits + first;
+    const float* __restrict__ op = ws_o + base * HD + lane;
+    float o[CH][DD];
+    auto fetch = [&](int j0) {
 #pragma unroll
-    for (int dd = 0; dd < HD / 64; ++dd) acc[dd] = 0.f;
-    for (int i0 = first; i0 <= last; i0 += 64) {
-        const int i = i0 + lane;
-        float w = 0.f, wl = 0.f;
-        if (i <= last) {
-            w = expf(ws_ml[2 * (base + i)] - m);
-            wl = w * ws_ml[2 * (base + i) + 1];
+        for (int j = 0; j < CH; ++j) {
+            const size_t jj = static_cast<size_t>(min(j0 + j, n_all - 1));     // past the end: the last one, weighted 0
+#pragma unroll
+            for (int dd = 0; dd < DD; ++dd) o[j][dd] = op[jj * HD + 64 * dd];
         }
-        denom += wave_sum(wl);
-        const int n = min(64, last - i0 + 1);
-        for (int j0 = 0; j0 < n; j0 += 8) {     // eight ranges' accumulators are read side by side
-            float o[8][HD / 64];
+    };
+    fetch(0);
+    float m = -INFINITY;
+    for (int i = lane; i < n_all; i += 64) m = fmaxf(m, ws_ml[2 * (base + i)]);
+    m = wave_max(m);
+    float denom = 0.f, acc[DD];
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+    for (int dd = 0; dd < DD; ++dd) acc[dd] = 0.f;
+    for (int i0 = 0; i0 < n_all; i0 += 64) {
+        const int i = min(i0 + lane, n_all - 1);
+        const float w = i0 + lane < n_all ? expf(ws_ml[2 * (base + i)] - m) : 0.f;
+        denom += wave_sum(w * ws_ml[2 * (base + i) + 1]);
+        const int n = min(64, n_all - i0);
+        for (int j0 = 0; j0 < n; j0 += CH) {
+            if (i0 + j0 > 0) fetch(i0 + j0);          // the first 32 are here already
 #pragma unroll
-                for (int dd = 0; dd < HD / 64; ++dd)
-                    o[j][dd] = j0 + j < n ? ws_o[(base + i0 + j0 + j) * HD + lane + 64 * dd] : 0.f;
+            for (int j = 0; j < CH; ++j) {
+                const float wj = j0 + j < n ? __shfl(w, min(j0 + j, 63), 64) : 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float wj = __shfl(w, min(j0 + j, 63), 64);
-#pragma unroll
-                for (int dd = 0; dd < HD / 64; ++dd) acc[dd] = fmaf(j0 + j < n ? wj : 0.f, o[j][dd], acc[dd]);
+                for (int dd = 0; dd < DD; ++dd) acc[dd] = fmaf(wj, o[j][dd], acc[dd]);
             }
         }
     }
     bf16* orow = out + static_cast<size_t>(t) * ldo + static_cast<size_t>(h) * HD;
 #pragma unroll
-    for (int dd = 0; dd < HD / 64; ++dd) orow[lane + 64 * dd] = from_float<bf16>(acc[dd] / denom);
+    for (int dd = 0; dd < DD; ++dd) orow[lane + 64 * dd] = from_float<bf16>(acc[dd] / denom);
 }
 
 // Decode attention: the query heads of a key/value head (up to 16 of them a workgroup) are
