@@ -384,6 +384,33 @@ __global__ void resolve_tokens_kernel(int* __restrict__ token_ids, const int* __
     if (token_ids[i] < 0) token_ids[i] = last_tokens[token_slot[i]];
 }
 
+// Both of the above in one launch (a step begins with them; one kernel fewer in a step that is
+// bound by its number of kernels).  Threads [0, capacity) take the triples, threads
+// [0, n) the rows; last_tokens null: no rows to resolve.
+__global__ void step_prologue_kernel(int* __restrict__ table, int stride, int n_slots,
+                                     const int* __restrict__ updates, int capacity,
+                                     int* __restrict__ token_ids, const int* __restrict__ token_slot,
+                                     const int* __restrict__ last_tokens, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < min(updates[0], capacity)) {
+        const int slot = updates[1 + 3 * i], logical = updates[2 + 3 * i], page = updates[3 + 3 * i];
+        if (slot >= 0 && slot < n_slots && logical >= 0 && logical < stride)
+            table[static_cast<size_t>(slot) * stride + logical] = page;
+    }
+    if (last_tokens && i < n && token_ids[i] < 0) token_ids[i] = last_tokens[token_slot[i]];
+}
+
+extern "C" int celeg_step_prologue(int* table, int stride, int n_slots, const int* updates, int capacity,
+                                   int* token_ids, const int* token_slot, const int* last_tokens, int n,
+                                   hipStream_t stream) {
+    const int threads = max(capacity, last_tokens ? n : 0);
+    if (threads <= 0) return 0;
+    if (capacity <= 0) return static_cast<int>(hipErrorInvalidValue);   // the update list is read
+    hipLaunchKernelGGL(step_prologue_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, table,
+                       stride, n_slots, updates, capacity, token_ids, token_slot, last_tokens, n);
+    return CELEG_LAUNCH_RESULT();
+}
+
 extern "C" int celeg_resolve_tokens(int* token_ids, const int* token_slot, const int* last_tokens,
                                     int n, hipStream_t stream) {
     if (n <= 0) return 0;

@@ -196,6 +196,23 @@ class HipOps:
             _c_int(capacity), self._stream())
         self._check(code, "apply_table_updates")
 
+    def step_prologue(self, table, updates, capacity, token_ids, token_slot, last_tokens, n):
+        """``apply_table_updates`` (capacity > 0) and ``resolve_tokens`` (``last_tokens`` given)
+        in one launch."""
+        self._dev(table, "table", torch.int32); self._dev(updates, "updates", torch.int32)
+        if capacity <= 0 or updates.numel() < 1 + 3 * capacity:
+            raise KernelError("step_prologue: the update list is shorter than its capacity")
+        for t, name in ((token_ids, "token_ids"), (token_slot, "token_slot")):
+            self._dev(t, name, torch.int32)
+        if last_tokens is not None:
+            self._dev(last_tokens, "last_tokens", torch.int32)
+            if token_ids.numel() < n or token_slot.numel() < n:
+                raise KernelError("step_prologue: fewer rows than n")
+        code = self._lib("elementwise").celeg_step_prologue(
+            _ptr(table), _c_int(table.shape[1]), _c_int(table.shape[0]), _ptr(updates), _c_int(capacity),
+            _ptr(token_ids), _ptr(token_slot), _ptr(last_tokens), _c_int(n), self._stream())
+        self._check(code, "step_prologue")
+
     # ------------------------------------------------------------------ matrix products
     def linear(self, x, w, out, bias=None):
         """out = x w^T (+ bias).  x [M,K] (rows may be strided), w [N,K], out [M,N] in the

@@ -122,8 +122,7 @@ class ModelRunner:
             return self._portion_from_graph(entries, portion)
         updates = self.cache.drain_table_updates()
         batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
-        self._apply_table_updates(batch)
-        self._resolve_tokens(batch)
+        self._begin_step(batch)
         self.last_batch = batch
         logits = self.model.forward(batch, self.rt)
         self.steps_run += 1
@@ -221,16 +220,14 @@ class ModelRunner:
         """Warm-up run and capture of the model's forward over the batch ``make_batch()``
         builds (of null-slot rows only): (graph, logits, workspace generation)."""
         batch = make_batch()
-        self._apply_table_updates(batch)
-        self._resolve_tokens(batch)
+        self._begin_step(batch)
         self.model.forward(batch, self.rt)          # warm-up: buffers, libraries, heuristics
         torch.cuda.synchronize(self.rt.device)
         graph = torch.cuda.CUDAGraph()
         self.rt.ws.frozen = True
         try:
             with torch.cuda.graph(graph):
-                self._apply_table_updates(batch)
-                self._resolve_tokens(batch)
+                self._begin_step(batch)
                 logits = self.model.forward(batch, self.rt)
         finally:
             self.rt.ws.frozen = False
@@ -262,6 +259,18 @@ class ModelRunner:
         flat = torch.tensor([len(updates)] + [v for u in updates for v in u], dtype=torch.int32)
         self.rt.ops.apply_table_updates(self.cache.groups[group].table, flat.to(self.rt.device),
                                         len(updates))
+
+    def _begin_step(self, batch: StepBatch) -> None:
+        """The block-table updates the step brings and the tokens it takes from the device: one
+        launch where there is one cache group and the kernels have that form."""
+        caps = batch.table_update_caps
+        if len(caps) == 1 and caps[0] > 0 and hasattr(self.rt.ops, "step_prologue"):
+            self.rt.ops.step_prologue(self.cache.groups[0].table, batch.table_updates[0], caps[0],
+                                      batch.token_ids, batch.token_slot, self._token_source,
+                                      batch.n_tokens)
+            return
+        self._apply_table_updates(batch)
+        self._resolve_tokens(batch)
 
     def _apply_table_updates(self, batch: StepBatch) -> None:
         for g, (upd, cap) in enumerate(zip(batch.table_updates, batch.table_update_caps)):
