@@ -243,6 +243,106 @@ __device__ __forceinline__ void top_k_candidates(
     __syncthreads();
 }
 
+// The same candidates by ranking, for rows whose logits fit in registers, already in the
+// order (score desc, id asc); false (nothing written) if more logits than SAMPLE_RANK_CAP
+// reach the bound from below, as when very many are equal: the caller then selects by
+// counting passes as above.
+//   1. Every thread keeps its logits as ordered keys of a cheap stand-in for the score
+//      (the penalty applied by multiplication, no division by the temperature: the same
+//      order up to a unit or two in the last place) and finds its largest.
+//   2. A bound from below: with c = ceil(top_k / 16), the c-th largest thread maximum of
+//      each of the 16 wavefronts; at least 16 c >= top_k logits reach the smallest of these
+//      16 values, so the top_k-th largest stand-in does too.  Eight units in the last place
+//      are taken off, which covers what the stand-in can differ from the score by.
+//   3. The logits at or above the bound (two or three times top_k of them as a rule) are
+//      gathered; their exact scores are computed as the reference does (true divisions), and
+//      a thread per such logit counts the ones that come before it: that is its place.
+// Five workgroup barriers instead of about forty, and two divisions per gathered logit
+// instead of per logit.
+#define SAMPLE_RANK_CAP 2048
+template <int KPT>
+__device__ __forceinline__ bool top_k_ranked(
+    const float* __restrict__ row, const uint8_t* __restrict__ seen, float penalty, float temperature,
+    int vocab, int top_k, uint32_t* wave_bound, uint2* gathered, unsigned int* sel, float* cand_score,
+    int* cand_id) {
+    const int tid = threadIdx.x;
+    const int lane = tid & (CELEG_WAVE - 1), wave = tid / CELEG_WAVE;
+    const bool pen = seen && penalty > 1.0f;
+    const float inv_penalty = 1.0f / penalty;
+    uint32_t keys[KPT];
+    {
+        float v[KPT];
+        unsigned char sn[KPT];
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            const int i = min(tid + SAMPLE_THREADS * j, vocab - 1);      // clamped, masked below
+            v[j] = row[i];
+            sn[j] = pen ? seen[i] : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < KPT; ++j) {
+            const float x = sn[j] ? (v[j] >= 0.0f ? v[j] * inv_penalty : v[j] * penalty) : v[j];
+            keys[j] = tid + SAMPLE_THREADS * j < vocab ? order_key(x) : 0u;
+        }
+    }
+    uint32_t my_max = 0u;
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) my_max = max(my_max, keys[j]);
+    // the c-th largest maximum of this wavefront: c times the largest, one lane struck out each time
+    const int c = (top_k + SAMPLE_THREADS / CELEG_WAVE - 1) / (SAMPLE_THREADS / CELEG_WAVE);
+    uint32_t left = my_max, cth = 0u;
+    for (int round = 0; round < c; ++round) {
+        uint32_t m = left;
+#pragma unroll
+        for (int off = CELEG_WAVE / 2; off > 0; off >>= 1)
+            m = max(m, static_cast<uint32_t>(__shfl_xor(static_cast<int>(m), off, CELEG_WAVE)));
+        cth = m;
+        const unsigned long long holders = __ballot(left == m);
+        if (lane == __ffsll(static_cast<long long>(holders)) - 1) left = 0u;
+    }
+    if (lane == 0) wave_bound[wave] = cth;
+    if (tid == 0) { sel[0] = 0u; sel[1] = 0u; }
+    __syncthreads();
+    uint32_t lower = wave_bound[0];
+#pragma unroll
+    for (int w = 1; w < SAMPLE_THREADS / CELEG_WAVE; ++w) lower = min(lower, wave_bound[w]);
+    lower = lower > 8u ? lower - 8u : 0u;
+#pragma unroll
+    for (int j = 0; j < KPT; ++j)
+        if (tid + SAMPLE_THREADS * j < vocab && keys[j] >= lower) {
+            const unsigned int p = atomicAdd(&sel[1], 1u);
+            if (p < SAMPLE_RANK_CAP) gathered[p].y = static_cast<unsigned>(tid + SAMPLE_THREADS * j);
+        }
+    __syncthreads();
+    const int n = static_cast<int>(sel[1]);
+    if (n > SAMPLE_RANK_CAP) return false;       // the same for every thread
+    // the exact scores of the gathered logits, as the reference computes them
+    for (int e = tid; e < n; e += SAMPLE_THREADS) {
+        const int id = static_cast<int>(gathered[e].y);
+        float x = row[id];
+        if (pen && seen[id]) x = x >= 0.0f ? x / penalty : x * penalty;
+        gathered[e].x = __float_as_uint(x / temperature);
+    }
+    __syncthreads();
+    for (int e = tid; e < n; e += SAMPLE_THREADS) {
+        const uint2 mine = gathered[e];
+        const float score = __uint_as_float(mine.x);
+        const int id = static_cast<int>(mine.y);
+        int place = 0;
+        for (int u0 = 0; u0 < n; u0 += 16) {            // sixteen reads from LDS under way at a time
+            uint2 other[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) other[j] = gathered[min(u0 + j, n - 1)];
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                place += (u0 + j < n && better(__uint_as_float(other[j].x), static_cast<int>(other[j].y), score, id)) ? 1 : 0;
+        }
+        if (place < top_k) { cand_score[place] = score; cand_id[place] = id; }
+    }
+    __syncthreads();
+    return true;
+}
+
 // fparams[row] = {temperature, top_p, penalty, u}; iparams[row] = {top_k, seen_row or -1,
 // slot or -1}; the token also goes to last_tokens[slot] (if given and slot >= 0), where the
 // next step can take it from without the host in between.
@@ -252,7 +352,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     int* __restrict__ out_tokens, int* __restrict__ last_tokens) {
     __shared__ float s_val[SAMPLE_THREADS / CELEG_WAVE];
     __shared__ int s_idx[SAMPLE_THREADS / CELEG_WAVE];
-    __shared__ unsigned int hist[256 * SAMPLE_HIST_COPIES];
+    __shared__ __attribute__((aligned(16))) unsigned int hist[256 * SAMPLE_HIST_COPIES];   // or SAMPLE_RANK_CAP gathered (key, id)
+    __shared__ uint32_t maxes[SAMPLE_THREADS / CELEG_WAVE];       // per wavefront: the bound it offers
     __shared__ unsigned int sel[3];       // prefix, remaining, size of the last bin
     __shared__ int running[2];
     __shared__ float cand_score[SAMPLE_MAX_K];
@@ -302,19 +403,28 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     top_k = min(min(top_k, vocab), SAMPLE_MAX_K);
     // the scores of the row are turned into keys once and kept in registers (up to 128 a
     // thread); larger vocabularies walk the row again for every pass
+    static_assert(sizeof(hist) >= SAMPLE_RANK_CAP * sizeof(uint2), "the gathered scores share the histograms' room");
+    uint2* gathered = reinterpret_cast<uint2*>(hist);
+    bool sorted = false;
     if (vocab <= SAMPLE_THREADS * 64)
-        top_k_candidates<64>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
+        sorted = top_k_ranked<64>(row, seen, penalty, temperature, vocab, top_k, maxes, gathered, sel, cand_score, cand_id);
     else if (vocab <= SAMPLE_THREADS * 128)
-        top_k_candidates<128>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
-    else
-        top_k_candidates<0>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
+        sorted = top_k_ranked<128>(row, seen, penalty, temperature, vocab, top_k, maxes, gathered, sel, cand_score, cand_id);
+    if (!sorted) {
+        if (vocab <= SAMPLE_THREADS * 64)
+            top_k_candidates<64>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
+        else if (vocab <= SAMPLE_THREADS * 128)
+            top_k_candidates<128>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
+        else
+            top_k_candidates<0>(row, seen, penalty, temperature, vocab, top_k, hist, sel, running, cand_score, cand_id);
+    }
     if (tid >= top_k && tid < SAMPLE_MAX_K) { cand_score[tid] = -INFINITY; cand_id[tid] = 0x7fffffff; }
     __syncthreads();
     if (wave != 0) return;         // one wavefront does the rest: no workgroup barriers from here
 
-    // ---- bitonic sort of 128 candidates by (score desc, id asc): lane l owns the pair whose
-    // lower member is the l-th position with the stride's bit clear
-    for (int size = 2; size <= SAMPLE_MAX_K; size <<= 1) {
+    // ---- bitonic sort of 128 candidates by (score desc, id asc), unless they came in that
+    // order: lane l owns the pair whose lower member is the l-th position with the stride's bit clear
+    for (int size = sorted ? 2 * SAMPLE_MAX_K : 2; size <= SAMPLE_MAX_K; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             const int a = ((lane & ~(stride - 1)) << 1) | (lane & (stride - 1));
             const int partner = a | stride;
