@@ -49,6 +49,8 @@ class HipOps:
         self._retired = []
         self._rope_tables = {}
         self.use_rope_table = True         # cos/sin of every position from a table made once
+        self.use_argmax_parts = True       # up to 16 greedy rows: many workgroups a row (1 row 6.9 against 11.8 us, 8 rows 8.2 against 11.4)
+        self._argmax_state = None
         self.use_sliced = True             # up to 16 bfloat16 rows: the k-sliced kernels
         self.use_rows_kernel = True        # 9 to 64 bfloat16 rows: the kernel that streams the weights
         # fewest rows it is used for (it takes any number up to 64).  Measured per decode step: at 16
@@ -421,7 +423,9 @@ class HipOps:
             _ptr(token_ids), _ptr(token_slot), _ptr(last_tokens), _c_int(n), self._stream())
         self._check(code, "resolve_tokens")
 
-    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None):
+    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None, all_greedy=False):
+        """One token per row.  ``all_greedy``: the caller knows that every row takes its
+        (penalised) largest logit; the rows are then cut into parts over many workgroups."""
         self._dev(logits, "logits", torch.float32, contiguous=False)
         self._dev(fparams, "fparams", torch.float32); self._dev(iparams, "iparams", torch.int32)
         self._dev(out_tokens, "out_tokens", torch.int32)
@@ -434,6 +438,20 @@ class HipOps:
             self._dev(seen, "seen", torch.uint8)
             if seen.shape[1] != V:
                 raise KernelError("sample: the seen table must be [slots, vocab]")
+        if all_greedy and self.use_argmax_parts and R <= 16:    # (64 rows: 23 us against 12 us, one workgroup a row)
+            if self._argmax_state is None or self._argmax_state[0].numel() < R:
+                if self._argmax_state is not None:
+                    self._retired.append(self._argmax_state)      # recorded graphs may still point at it
+                self._argmax_state = (torch.zeros(max(R, 64), dtype=torch.int64, device=logits.device),
+                                      torch.zeros(max(R, 64), dtype=torch.int32, device=logits.device))
+            best, arrived = self._argmax_state
+            code = self._lib("sampling").celeg_argmax_rows(
+                _ptr(logits), _c_int(self._rows(logits, "logits")), _c_int(R), _c_int(V),
+                _ptr(fparams), _ptr(iparams), _ptr(seen),
+                _c_size_t(seen.stride(0) if seen is not None else 0), _ptr(out_tokens),
+                _ptr(last_tokens), _ptr(best), _ptr(arrived), self._stream())
+            self._check(code, "argmax of rows")
+            return
         code = self._lib("sampling").celeg_sample(
             _ptr(logits), _c_int(self._rows(logits, "logits")), _c_int(R), _c_int(V),
             _ptr(fparams), _ptr(iparams), _ptr(seen),

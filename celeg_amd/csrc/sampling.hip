@@ -480,6 +480,85 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     }
 }
 
+// Penalised argmax of rows that are all greedy, a row cut into parts of ARGMAX_PART logits,
+// a workgroup each (one workgroup a row is bound by what one compute unit can pull: 11 us at
+// 65,536 logits).  A part's best goes into best[row] by a 64-bit atomic maximum of
+// (ordered key of the value, ~index): the largest value wins and, among equal values, the
+// lowest index.  The part that arrives last (a counter) reads the winner, writes the token
+// and leaves best and arrived at zero for the next launch.  Everything the workgroups tell
+// each other goes through these atomics.
+#define ARGMAX_PART 4096
+#define ARGMAX_THREADS 256
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(
+    const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ fparams,
+    const int* __restrict__ iparams, const uint8_t* __restrict__ seen_all, size_t seen_stride,
+    int* __restrict__ out_tokens, int* __restrict__ last_tokens, unsigned long long* __restrict__ best,
+    unsigned int* __restrict__ arrived) {
+    constexpr int PER = ARGMAX_PART / ARGMAX_THREADS;
+    __shared__ unsigned long long s_best[ARGMAX_THREADS / CELEG_WAVE];
+    const int r = blockIdx.y, tid = threadIdx.x;
+    const int lane = tid & (CELEG_WAVE - 1), wave = tid / CELEG_WAVE;
+    const float* row = logits + static_cast<size_t>(r) * ld;
+    const float penalty = fparams[4 * r + 2];
+    const int seen_row = iparams[3 * r + 1], slot = iparams[3 * r + 2];
+    const uint8_t* seen = (seen_all && seen_row >= 0 && penalty > 1.0f)
+                              ? seen_all + static_cast<size_t>(seen_row) * seen_stride : nullptr;
+    const int lo = blockIdx.x * ARGMAX_PART;
+    float v[PER];
+    unsigned char sn[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = min(lo + tid + ARGMAX_THREADS * j, vocab - 1);     // clamped, masked below
+        v[j] = row[i];
+        sn[j] = seen ? seen[i] : 0;
+    }
+    unsigned long long mine = 0ull;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = lo + tid + ARGMAX_THREADS * j;
+        float x = v[j];
+        if (sn[j]) x = x >= 0.0f ? x / penalty : x * penalty;
+        x += 0.0f;                                                       // -0 and +0 are one value
+        const unsigned long long packed = (static_cast<unsigned long long>(order_key(x)) << 32) |
+                                          (0xffffffffu - static_cast<unsigned>(i));
+        if (i < vocab) mine = max(mine, packed);
+    }
+#pragma unroll
+    for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) {
+        const unsigned long long other = __shfl_xor(mine, off, CELEG_WAVE);
+        mine = max(mine, other);
+    }
+    if (lane == 0) s_best[wave] = mine;
+    __syncthreads();
+    if (tid != 0) return;
+#pragma unroll
+    for (int w = 1; w < ARGMAX_THREADS / CELEG_WAVE; ++w) mine = max(mine, s_best[w]);
+    atomicMax(&best[r], mine);
+    __threadfence();
+    if (atomicAdd(&arrived[r], 1u) != gridDim.x - 1) return;
+    __threadfence();
+    const unsigned long long winner = atomicExch(&best[r], 0ull);
+    atomicExch(&arrived[r], 0u);
+    const int token = static_cast<int>(0xffffffffu - static_cast<unsigned>(winner & 0xffffffffull));
+    out_tokens[r] = token;
+    if (last_tokens && slot >= 0) last_tokens[slot] = token;
+}
+
+// rows that are all greedy (temperature <= 0 or top_k == 1): best [rows] and arrived [rows]
+// must hold zeros when the first launch comes (the kernel leaves them so).  Launches that
+// share them must run one after the other.
+extern "C" int celeg_argmax_rows(const float* logits, int ld, int rows, int vocab, const float* fparams,
+                                 const int* iparams, const uint8_t* seen, size_t seen_stride,
+                                 int* out_tokens, int* last_tokens, unsigned long long* best,
+                                 unsigned int* arrived, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (vocab <= 0) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(argmax_parts_kernel, dim3((vocab + ARGMAX_PART - 1) / ARGMAX_PART, rows),
+                       dim3(ARGMAX_THREADS), 0, stream, logits, ld, vocab, fparams, iparams, seen,
+                       seen_stride, out_tokens, last_tokens, best, arrived);
+    return CELEG_LAUNCH_RESULT();
+}
+
 extern "C" int celeg_sample(const float* logits, int ld, int rows, int vocab,
                             const float* fparams, const int* iparams, const uint8_t* seen,
                             size_t seen_stride, int* out_tokens, int* last_tokens,

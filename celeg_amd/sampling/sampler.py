@@ -162,8 +162,9 @@ class Sampler:
         if self._uploaded is None or not np.array_equal(used, self._uploaded):
             self._params_dev.copy_(self._params[turn], non_blocking=True)
             self._uploaded = used
+        all_greedy = all(self._configs[slot].greedy for slot in slots)
         self.ops.sample(logits, self._fparams_dev, self._iparams_dev, self._seen,
-                        self._tokens_dev[:R], last_tokens=self.last_tokens)
+                        self._tokens_dev[:R], last_tokens=self.last_tokens, **({"all_greedy": True} if all_greedy else {}))
         self._tokens_host[turn][:R].copy_(self._tokens_dev[:R], non_blocking=True)
         if self._events[turn] is not None:
             self._events[turn].record()

@@ -134,7 +134,7 @@ class CpuOps:
                 pr = torch.softmax(s, dim=0)
                 out[t, h * head_dim:(h + 1) * head_dim] = (pr @ vals[:, g]).to(out.dtype)
 
-    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None):
+    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None, all_greedy=False):
         import plain_lfm2 as plain   # the double may lean on the plain sampler
         R, V = logits.shape
         for r in range(R):

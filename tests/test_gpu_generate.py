@@ -129,7 +129,7 @@ def ops():
     return HipOps(DEV)
 
 
-def run_sample(ops, logits, rows):
+def run_sample(ops, logits, rows, all_greedy=False):
     """rows: list of (temperature, top_k, top_p, penalty, u, seen list or None)"""
     R, V = logits.shape
     f = torch.tensor([[t, p, pen, u] for t, k, p, pen, u, s in rows], dtype=torch.float32)
@@ -141,7 +141,7 @@ def run_sample(ops, logits, rows):
         i.append([k, r if s is not None else -1, -1])
     out = torch.empty(R, dtype=torch.int32, device=DEV)
     ops.sample(logits.to(DEV), f.reshape(-1).to(DEV), torch.tensor(i, dtype=torch.int32).reshape(-1).to(DEV),
-               seen.to(DEV), out)
+               seen.to(DEV), out, all_greedy=all_greedy)
     return out.tolist()
 
 
@@ -198,6 +198,18 @@ def test_arg_max_lowest_index_wins_with_and_without_penalty(ops, vocab):
             rows.append((0.0, 1, 1.0, 1.0, 0.0, None))
             want.append(ties[0])
     assert run_sample(ops, logits, rows) == want
+    # the same by the kernel that cuts every row into parts over many workgroups, twice (it
+    # leaves its counters ready for the next launch), and with a zero of either sign as maximum
+    assert run_sample(ops, logits, rows, all_greedy=True) == want
+    assert run_sample(ops, logits, rows, all_greedy=True) == want
+    zeros = -torch.rand(2, vocab) - 0.5
+    zeros[0, vocab - 1] = 0.0
+    zeros[0, vocab // 2] = -0.0
+    zeros[1, vocab // 2] = 0.0
+    zeros[1, 0] = -0.0
+    plain_rows = [(0.0, 1, 1.0, 1.0, 0.0, None)] * 2
+    assert run_sample(ops, zeros, plain_rows, all_greedy=True) == run_sample(ops, zeros, plain_rows) \
+        == [min(vocab // 2, vocab - 1), 0]
 
 
 def test_mark_seen(ops):
