@@ -472,10 +472,6 @@ extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, in
         if (shape == 2) return CELEG_SHAPE(1, 2, 4);
         if (shape == 3) return CELEG_SHAPE(1, 1, 8);
         if (shape == 4) return CELEG_SHAPE(1, 1, 4);
-        if (shape == 5) return launch_shape<1, 8, 1, 0>(p, amode, epi, stream);
-        if (shape == 6) return launch_shape<1, 2, 4, 0>(p, amode, epi, stream);
-        if (shape == 7) return launch_shape<1, 1, 8, 0>(p, amode, epi, stream);
-        if (shape == 8) return launch_shape<1, 1, 4, 0>(p, amode, epi, stream);
         if (tiles >= 2048) return CELEG_SHAPE(1, 8, 1);
         // two tiles a workgroup (they share the prepared rows) once there are enough tiles
         // and K is short enough that four wavefronts a tile keep their loads in one batch
