@@ -29,8 +29,6 @@ __device__ __forceinline__ size_t kv_block(int page, int n_layers, int layer, in
            static_cast<size_t>(page_tokens) * head_dim;
 }
 
-// Rows a workgroup of the portion kernel takes when the caller leaves the choice open.
-#define CELEG_ROWS_DEFAULT(n_tokens, n_seqs) 64
 
 
 // Combining a value with the one that lane ^ 16 (lane ^ 32) holds, by the lane-swap
@@ -59,21 +57,28 @@ __device__ __forceinline__ float sum_half32(float x) {
 }
 
 // ================================================================ rows of portions
-// A tile is 64*RT rows of one request for one query head; 4 wavefronts work on it, each
-// on RT tiles of 16 rows.  A workgroup of 8 wavefronts takes two tiles of a request, the
-// i-th from the front and the i-th from the back: under the causal mask their key counts
-// add up to the same for every pair, and the wavefronts are spread over the SIMDs so that
-// each SIMD gets one of either tile.  The keys and values of 64 positions are staged in
-// LDS once for the 4 wavefronts of a tile (two buffers: the next 64 are fetched into registers
-// while the current 64 are worked on, and written to the other buffer before the one
-// barrier of the round).  Per 64 keys: S^T = K Q^T (16x16x32 MFMA: A = 16 keys x 32 dims,
+// A workgroup takes a tile of 64*RT rows of one request for one query head.  Its 8
+// wavefronts are two halves of 4; the wavefronts of a half each own RT tiles of 16 rows of
+// the same 64*RT rows, and the halves take the rounds of 64 keys in turn (half 0 the even
+// rounds of the tile's key range, half 1 the odd ones), each with a running maximum, sum
+// and output of its own.  At the end half 1 hands its (maximum, sum, output) over through
+// LDS, and half 0 joins the two and writes.  Under the causal mask the last tile of a
+// request sees the most keys, so a request's tiles are handed out last first.
+// The keys and values of a round are staged in LDS once for the 4 wavefronts of a half
+// (two buffers a half: the half's next round is fetched into registers while the current
+// one is worked on, and written to the other buffer before the one barrier of the
+// round).  Per 64 keys: S^T = K Q^T (16x16x32 MFMA: A = 16 keys x 32 dims,
 // B = 32 dims x 16 rows), online softmax per row (a row is a lane column), then
 // O^T += V^T P^T (A = 16 dims x 32 keys from the transposed V, B = P^T straight from the
 // accumulator registers of S^T).  The 16 keys of a score tile are chosen so that a lane
 // ends up with the probabilities of 8 neighbouring keys, which is what one 16-byte read
-// of the transposed V delivers.
-template <int HD, int RT>
-__global__ __launch_bounds__(512) void attention_rows_kernel(
+// of the transposed V delivers; in LDS the keys lie in the order of the score tiles, so
+// that the 16 lanes of a read touch 16 rows in a row (no bank is asked twice).
+// The running maximum of a row follows the scores only when some row's grows by more than
+// 8 (a factor 2^8): until then probabilities are taken against the older value, stay below
+// 2^8, and numerator and denominator carry the same factor.
+template <int HD, int RT, int NH, bool SHARE>
+__global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
@@ -87,53 +92,74 @@ __global__ __launch_bounds__(512) void attention_rows_kernel(
     constexpr int DT = HD / 16;     // 16-dim tiles of the output
     constexpr int KROW = HD + 8;    // LDS row of a key, padded against bank conflicts
     constexpr int VROW = 64 + 8;    // LDS row of a dimension: 64 keys, padded
-    constexpr int CH = HD / 32;     // 16-byte pieces of K, and of V, a thread moves per round
+    constexpr int NSET = SHARE ? 1 : NH;          // sets of staging buffers
+    constexpr int NT = SHARE ? 256 * NH : 256;    // threads that fill a set
+    constexpr int CH = (8 * HD + NT - 1) / NT;    // 16-byte pieces of K, and of V, a thread moves per round
+    constexpr float LAZY = 8.f;     // growth of a row's maximum that is let pass
     extern __shared__ int smem[];
-    const int half = threadIdx.x >> 8, tid = threadIdx.x & 255;
-    __bf16* const sK = reinterpret_cast<__bf16*>(smem) + half * (2 * 64 * KROW);       // [2][2][64][KROW]
-    __bf16* const sV = reinterpret_cast<__bf16*>(smem) + 4 * 64 * KROW + half * (2 * HD * VROW);  // [2][2][HD][VROW]
-    int* const spages = reinterpret_cast<int*>(reinterpret_cast<__bf16*>(smem) + 4 * 64 * KROW + 4 * HD * VROW);
-    int pair = blockIdx.x;
-    const int h = blockIdx.y;
+    // wavefront-uniform values are kept in scalar registers
+    const int half = NH == 1 ? 0 : __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 8);
+    const int tid = threadIdx.x & 255;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int set = SHARE ? 0 : half;
+    __bf16* const sK = reinterpret_cast<__bf16*>(smem) + set * (2 * 64 * KROW);       // [NSET][2][64][KROW]
+    __bf16* const sV = reinterpret_cast<__bf16*>(smem) + NSET * 2 * 64 * KROW + set * (2 * HD * VROW);  // [NSET][2][HD][VROW]
+    int* const spages = reinterpret_cast<int*>(reinterpret_cast<__bf16*>(smem) + NSET * 2 * (64 * KROW + HD * VROW));
+    // Which tile and head.  Workgroups go to the chip's 8 dies in turn (number % 8), and each
+    // die has an L2 of its own; so the list of all (key/value head, tile, query head of the
+    // group, or NH of them where the halves share the staged keys), in this order, is cut into 8
+    // runs, one per die: a die then reads the keys and values of few heads, and workgroups that
+    // start together read the same ones.
+    int all_tiles = 0;
+    for (int i = 0; i < n_seqs; ++i) all_tiles += (cu_seqlens[i + 1] - cu_seqlens[i] + ROWS - 1) / ROWS;
+    const int group = q_heads / kv_heads;
+    const int per_group = SHARE ? (group + NH - 1) / NH : group;   // workgroups a tile of a key/value head takes
+    const long long all_items = static_cast<long long>(all_tiles) * kv_heads * per_group;
+    const int die = blockIdx.x & 7;
+    const long long item = (all_items * die + 7) / 8 + (blockIdx.x >> 3);
+    if (item >= (all_items * (die + 1) + 7) / 8) return;   // the whole workgroup
+    const int in_group = static_cast<int>(item % per_group) * (SHARE ? NH : 1) + (SHARE ? half : 0);
+    const bool head_valid = in_group < group;      // a group that the halves do not divide
+    const int h = static_cast<int>(item / per_group / all_tiles) * group + min(in_group, group - 1);
+    int idx = static_cast<int>(item / per_group % all_tiles);
     int s = 0, len = 0, tiles = 0;
-    bool found = false;
-    for (; s < n_seqs; ++s) {
+    for (;; ++s) {
         len = cu_seqlens[s + 1] - cu_seqlens[s];
         tiles = (len + ROWS - 1) / ROWS;
-        if (pair < (tiles + 1) / 2) { found = true; break; }
-        pair -= (tiles + 1) / 2;
+        if (idx < tiles) break;
+        idx -= tiles;
     }
-    if (!found) return;   // the whole workgroup
+    const int tile = tiles - 1 - idx;
     const int start = seq_start[s];
-    // first round and number of rounds of a tile of rows
-    auto first_key = [&](int t) { return ((window > 0 ? max(0, start + t * ROWS - window + 1) : 0) >> 6) << 6; };
-    auto last_key = [&](int t) { return start + min(t * ROWS + ROWS - 1, len - 1); };
-    const int heavy = tiles - 1 - pair;
-    const bool has_tile = half == 1 || pair != heavy;   // the middle tile of an odd count has no partner
-    const int tile = half == 1 ? heavy : pair;
-    const int rounds_heavy = ((last_key(heavy) - first_key(heavy)) >> 6) + 1;
-    const int rounds_light = pair != heavy ? ((last_key(pair) - first_key(pair)) >> 6) + 1 : 0;
-    const int n_rounds = max(rounds_heavy, rounds_light);
-    const int my_rounds = half == 1 ? rounds_heavy : rounds_light;
     const int brow0 = tile * ROWS;
-    const int bkmax = last_key(tile);             // last key this half sees
-    const int last_page = bkmax >> page_shift;
+    const int first = ((window > 0 ? max(0, start + brow0 - window + 1) : 0) >> 6) << 6;   // first key of round 0
+    const int bkmax = start + min(brow0 + ROWS - 1, len - 1);                              // last key the tile sees
+    const int total_rounds = ((bkmax - first) >> 6) + 1;
+    constexpr int TURNS = SHARE ? 1 : NH;          // halves that take the rounds in turn
+    const int my_rounds = SHARE ? total_rounds : (total_rounds - half + NH - 1) / NH;   // rounds half, half + NH, ..
+    const int n_it = (total_rounds + TURNS - 1) / TURNS;
+    // the pages of the tile's rounds; behind the last key's page, that page again (allocated
+    // memory for the positions of the last round that are masked anyway)
+    const int page0 = first >> page_shift;
     {
         const int* __restrict__ pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
-        for (int i = threadIdx.x; i <= last_key(heavy) >> page_shift; i += 512) spages[i] = pages[i];
+        const int last_page = bkmax >> page_shift;
+        const int n_fill = ((first + 64 * total_rounds - 1) >> page_shift) - page0 + 1;
+        for (int i = threadIdx.x; i < n_fill; i += 256 * NH) spages[i] = pages[min(page0 + i, last_page)];
     }
     __syncthreads();
-    const int wave = tid >> 6, lane = tid & 63;
     const int c = lane & 15, qd = lane >> 4;
     const int wrow0 = brow0 + wave * WROWS;
-    const bool wave_active = has_tile && wrow0 < len;
+    const bool wave_active = wrow0 < len && head_valid;
     const int wkmax = start + min(wrow0 + WROWS - 1, len - 1);  // last key any row of the wavefront sees
     const int wkmin = window > 0 ? max(0, start + wrow0 - window + 1) : 0;
     const int kvh = h / (q_heads / kv_heads);
     const size_t row_base = static_cast<size_t>(cu_seqlens[s]);
     const size_t head_block = static_cast<size_t>(page_tokens) * HD;
-    const size_t page_stride = static_cast<size_t>(n_layers) * kv_heads * head_block;
+    const unsigned page_stride = static_cast<unsigned>(n_layers * kv_heads) * static_cast<unsigned>(head_block);   // the host has checked that it fits
     const size_t layer_head = (static_cast<size_t>(layer) * kv_heads + kvh) * head_block;
+    const bf16* __restrict__ const kbase = k_pool + layer_head;
+    const bf16* __restrict__ const vbase = v_pool + layer_head;
 
     int pq[RT], lo_q[RT];
     bool row_valid[RT];
@@ -158,49 +184,55 @@ __global__ __launch_bounds__(512) void attention_rows_kernel(
 
     // What a thread moves per round: piece i of K is 8 dims of one key; piece i of V is 8
     // keys of one dimension, walked page by page so that neighbouring threads read
-    // neighbouring memory.  Positions beyond the last key are read from the last key's
-    // page (allocated memory) and masked.
+    // neighbouring memory.  What does not change from round to round is worked out here:
+    // the page of the round a piece lies in, its place inside the page, its place in LDS.
     const int pt_shift = min(page_shift, 6);          // keys of a page inside a round: 1 << pt_shift
+    const int in_page = page_tokens - 1;
+    int k_pg[CH], k_off[CH], k_lds[CH], v_pg[CH], v_off[CH], v_lds[CH];
+    bool has_piece[CH];      // the last one may be past the end
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+        const int i_all = (SHARE ? static_cast<int>(threadIdx.x) : tid) + NT * j;
+        has_piece[j] = (8 * HD) % NT == 0 || i_all < 8 * HD;
+        const int i = min(i_all, 8 * HD - 1);
+        const int key = i / (HD / 8), part = i % (HD / 8);
+        k_pg[j] = key >> page_shift;
+        k_off[j] = (key & in_page) * HD + part * 8;
+        // key 32 a + 8 b + 4 t + r of the round is row b*4 + r of score tile 2 a + t
+        const int krow = 16 * (2 * (key >> 5) + ((key >> 2) & 1)) + 4 * ((key >> 3) & 3) + (key & 3);
+        k_lds[j] = krow * KROW + part * 8;
+        const int piece = (i >> (pt_shift - 3)) / HD;      // which page of the round
+        const int rem = i - piece * (HD << (pt_shift - 3));
+        const int d = rem >> (pt_shift - 3), g = rem & ((1 << (pt_shift - 3)) - 1);
+        v_pg[j] = piece;
+        v_off[j] = d * page_tokens + g * 8;
+        v_lds[j] = d * VROW + (piece << pt_shift) + g * 8;
+    }
     u32x4_t kstage[CH], vstage[CH];
     auto fetch = [&](int kb) __attribute__((always_inline)) {
+        const int pg = (kb >> page_shift) - page0;
+        const int inp = kb & in_page;     // a round inside a longer page starts here
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
-            const int i = tid + 256 * j;
-            {
-                const int key = kb + i / (HD / 8), part = i % (HD / 8);
-                const int page = spages[min(key >> page_shift, last_page)];
-                kstage[j] = *reinterpret_cast<const u32x4_t*>(
-                    k_pool + static_cast<size_t>(page) * page_stride + layer_head +
-                    static_cast<size_t>(key & (page_tokens - 1)) * HD + part * 8);
-            }
-            {
-                const int per_dim = 1 << (pt_shift - 3);           // pieces of a dimension inside a page
-                const int piece = (i >> (pt_shift - 3)) / HD;      // which page of the round
-                const int rem = i - piece * (HD << (pt_shift - 3));
-                const int d = rem >> (pt_shift - 3), g = rem & (per_dim - 1);
-                const int key0 = kb + (piece << pt_shift) + g * 8;
-                const int page = spages[min(key0 >> page_shift, last_page)];
-                vstage[j] = *reinterpret_cast<const u32x4_t*>(
-                    v_pool + static_cast<size_t>(page) * page_stride + layer_head +
-                    static_cast<size_t>(d) * page_tokens + (key0 & (page_tokens - 1)));
-            }
+            if (!has_piece[j]) continue;
+            const unsigned kpage = spages[pg + k_pg[j]];
+            kstage[j] = *reinterpret_cast<const u32x4_t*>(
+                kbase + (static_cast<unsigned long long>(kpage) * page_stride + static_cast<unsigned>(inp * HD + k_off[j])));
+            const unsigned vpage = spages[pg + v_pg[j]];
+            vstage[j] = *reinterpret_cast<const u32x4_t*>(
+                vbase + (static_cast<unsigned long long>(vpage) * page_stride + static_cast<unsigned>(inp + v_off[j])));
         }
     };
     auto stage = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
-            const int i = tid + 256 * j;
-            *reinterpret_cast<u32x4_t*>(sK + (buf * 64 + i / (HD / 8)) * KROW + (i % (HD / 8)) * 8) = kstage[j];
-            const int per_dim = 1 << (pt_shift - 3);
-            const int piece = (i >> (pt_shift - 3)) / HD;
-            const int rem = i - piece * (HD << (pt_shift - 3));
-            const int d = rem >> (pt_shift - 3), g = rem & (per_dim - 1);
-            *reinterpret_cast<u32x4_t*>(sV + (buf * HD + d) * VROW + (piece << pt_shift) + g * 8) = vstage[j];
+            if (!has_piece[j]) continue;
+            *reinterpret_cast<u32x4_t*>(sK + buf * 64 * KROW + k_lds[j]) = kstage[j];
+            *reinterpret_cast<u32x4_t*>(sV + buf * HD * VROW + v_lds[j]) = vstage[j];
         }
     };
     const float neg_inf = -INFINITY;
-    // score tile kt, A row i  <->  key 32 (kt/2) + 8 (i/4) + 4 (kt%2) + i%4 of the round, so
-    // that accumulator register r of lane quad qd is key 32 (kt/2) + 8 qd + 4 (kt%2) + r
+    // accumulator register r of lane quad qd, score tile kt, is key 32 (kt/2) + 8 qd + 4 (kt%2) + r
     auto compute = [&](int kb, int buf) __attribute__((always_inline)) {
         floatx4_t sacc[RT][4];
 #pragma unroll
@@ -209,8 +241,7 @@ __global__ __launch_bounds__(512) void attention_rows_kernel(
             for (int kt = 0; kt < 4; ++kt) sacc[rt][kt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
-            const int key_row = 32 * (kt >> 1) + 8 * (c >> 2) + 4 * (kt & 1) + (c & 3);
-            const __bf16* kp = sK + (buf * 64 + key_row) * KROW + qd * DQ;
+            const __bf16* kp = sK + (buf * 64 + 16 * kt + c) * KROW + qd * DQ;
 #pragma unroll
             for (int st = 0; st < KS; ++st) {
                 const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kp + st * 8);
@@ -226,27 +257,30 @@ __global__ __launch_bounds__(512) void attention_rows_kernel(
             const int first_row = start + wrow0 + rt * 16;
             const bool full = kb + 63 <= first_row &&
                               (window <= 0 || kb >= min(first_row + 15, start + len - 1) - window + 1);
-            float mx = neg_inf;
-            if (full) {
-#pragma unroll
-                for (int kt = 0; kt < 4; ++kt)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sacc[rt][kt][r]);
-            } else {
+            if (!full) {
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int key = kb + 32 * (kt >> 1) + 8 * qd + 4 * (kt & 1) + r;
-                        const float sv = (key <= pq[rt] && key >= lo_q[rt]) ? sacc[rt][kt][r] : neg_inf;
-                        sacc[rt][kt][r] = sv;
-                        mx = fmaxf(mx, sv);
+                        if (key > pq[rt] || key < lo_q[rt]) sacc[rt][kt][r] = neg_inf;
                     }
             }
-            mx = max_half32(max_row16(mx));
-            const float m_new = fmaxf(m[rt], mx * scale_log2e);      // the scale is positive
-            const float m_use = m_new == neg_inf ? 0.f : m_new;      // a row that has seen no key yet
-            const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);
+            float mx = neg_inf;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) mx = fmaxf(mx, sacc[rt][kt][r]);
+            mx = max_half32(max_row16(mx)) * scale_log2e;      // the scale is positive
+            if (__builtin_amdgcn_ballot_w64(mx > m[rt] + LAZY) != 0) {
+                const float m_new = fmaxf(m[rt], mx);
+                const float alpha = __builtin_amdgcn_exp2f(m[rt] - (m_new == neg_inf ? 0.f : m_new));
+                l[rt] *= alpha;
+                m[rt] = m_new;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] *= alpha;
+            }
+            const float m_use = m[rt] == neg_inf ? 0.f : m[rt];      // a row that has seen no key yet
             float psum = 0.f;
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt)
@@ -256,10 +290,7 @@ __global__ __launch_bounds__(512) void attention_rows_kernel(
                     sacc[rt][kt][r] = p;
                     psum += p;
                 }
-            l[rt] = l[rt] * alpha + psum;
-            m[rt] = m_new;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) oacc[rt][dt] *= alpha;
+            l[rt] += psum;
 #pragma unroll
             for (int kp = 0; kp < 2; ++kp)
                 pb[rt][kp] = bf16x8_t{
@@ -280,26 +311,58 @@ __global__ __launch_bounds__(512) void attention_rows_kernel(
             }
     };
 
-    // Round r works on LDS buffer r % 2 while the registers hold round r + 1 (asked for a
-    // whole round earlier); at its end they go to the other buffer and round r + 2 is asked
-    // for.  Both halves pass the same barriers; the one with fewer rounds idles at the end.
-    int kb = first_key(tile);
+    // Round r of a set of staging buffers works on LDS buffer r % 2 while the registers hold
+    // round r + 1 (asked for a whole round earlier); at its end they go to the other buffer and
+    // round r + 2 is asked for.  Halves that take the rounds in turn have a set each (round r
+    // of half i is key block first + 64 (i + NH r)), and all pass the same barriers.
+    int kb = first + (SHARE ? 0 : 64 * half);
     int buf = 0;
     if (my_rounds > 0) { fetch(kb); stage(0); }
-    if (my_rounds > 1) fetch(kb + 64);
+    if (my_rounds > 1) fetch(kb + 64 * TURNS);
     __syncthreads();
-    for (int it = 0; it < n_rounds; ++it, kb += 64) {
+    for (int it = 0; it < n_it; ++it, kb += 64 * TURNS) {
         if (it < my_rounds && wave_active && kb <= wkmax && kb + 63 >= wkmin) compute(kb, buf);
         if (it + 1 < my_rounds) {
             stage(buf ^ 1);
-            if (it + 2 < my_rounds) fetch(kb + 128);
+            if (it + 2 < my_rounds) fetch(kb + 128 * TURNS);
         }
         __syncthreads();
         buf ^= 1;
     }
-    if (!wave_active) return;
+    // half 1 hands over: register by register, a lane to the same lane (the halves' wavefronts
+    // of one number own the same rows).  The staging buffers are free after the last barrier.
+    float* const xch = reinterpret_cast<float*>(smem) + wave * (RT * (4 * DT + 2) * 64) + lane;
+    if (TURNS > 1 && total_rounds > 1) {
+        if (half == 1 && wave_active) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                float* x = xch + rt * (4 * DT + 2) * 64;
+                x[0] = m[rt];
+                x[64] = l[rt];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) x[(2 + 4 * dt + r) * 64] = oacc[rt][dt][r];
+            }
+        }
+        __syncthreads();
+    }
+    if ((TURNS > 1 && half == 1) || !wave_active) return;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
+        if (TURNS > 1 && total_rounds > 1) {
+            const float* x = xch + rt * (4 * DT + 2) * 64;
+            const float m1 = x[0];
+            const float m_new = fmaxf(m[rt], m1);
+            const float m_use = m_new == neg_inf ? 0.f : m_new;
+            const float a0 = __builtin_amdgcn_exp2f(m[rt] - m_use), a1 = __builtin_amdgcn_exp2f(m1 - m_use);
+            l[rt] = l[rt] * a0 + x[64] * a1;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    oacc[rt][dt][r] = oacc[rt][dt][r] * a0 + x[(2 + 4 * dt + r) * 64] * a1;
+        }
         float lt = l[rt];
         lt = sum_half32(sum_row16(lt));
         if (!row_valid[rt]) continue;
@@ -314,25 +377,31 @@ __global__ __launch_bounds__(512) void attention_rows_kernel(
     }
 }
 
-template <int HD, int RT>
+template <int HD, int RT, int NH, bool SHARE>
 static int launch_attention_rows(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
     int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int page_tokens,
     int n_layers, int layer, float scale, int window, hipStream_t stream) {
-    const size_t lds = (4 * 64 * (HD + 8) + 4 * HD * (64 + 8)) * sizeof(bf16) +
-                       static_cast<size_t>(table_stride) * sizeof(int);
+    // staging buffers, and a request's pages with room for a round's worth behind the last
+    const size_t lds = (SHARE ? 1 : NH) * 2 * (64 * (HD + 8) + HD * (64 + 8)) * sizeof(bf16) +
+                       (static_cast<size_t>(table_stride) + 8) * sizeof(int);
     if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
-    auto kernel = attention_rows_kernel<HD, RT>;
+    // the kernel multiplies page numbers by the elements of a page in 32 x 32 -> 64 bits
+    if (static_cast<size_t>(n_layers) * kv_heads * page_tokens * HD >= (size_t{1} << 31))
+        return static_cast<int>(hipErrorInvalidValue);
+    auto kernel = attention_rows_kernel<HD, RT, NH, SHARE>;
     if (lds > 48 * 1024) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize,
                                                  static_cast<int>(lds));
         if (e != hipSuccess) return static_cast<int>(e);
     }
-    // >= sum over requests of ceil(tiles / 2), tiles = ceil(rows / (64 RT))
-    const int max_pairs = (n_tokens / (64 * RT) + 2 * n_seqs + 1) / 2;
-    dim3 grid(max_pairs, q_heads), block(512);
+    // >= sum over requests of ceil(rows / (64 RT))
+    const int max_tiles = n_tokens / (64 * RT) + n_seqs;
+    const int group = q_heads / kv_heads;
+    const long long max_items = static_cast<long long>(max_tiles) * kv_heads * (SHARE ? (group + NH - 1) / NH : group);
+    dim3 grid(static_cast<unsigned>(8 * ((max_items + 7) / 8 + 1))), block(256 * NH);
     hipLaunchKernelGGL(kernel, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
                        table_stride, cu_seqlens, seq_slot, seq_start, n_seqs,
@@ -341,27 +410,47 @@ static int launch_attention_rows(
     return CELEG_LAUNCH_RESULT();
 }
 
-// rows_per_tile: 64 or 128 rows a workgroup (0: chosen from the number of rows).
+// rows_per_tile: 64 or 128 rows a workgroup.  form: 1, a workgroup of 4 wavefronts takes all
+// rounds of keys of its tile for one query head; 2, two such sets take the rounds in turn and
+// join at the end (more workgroups in flight and half as long a way for a tile with many
+// keys: for few rows); 3, two sets take a query head each of those that share a key/value
+// head, and the staged keys and values with it (half the traffic: for many rows).  0 leaves
+// a choice to this function, which then goes by the number of rows and by context_hint, the
+// longest context among the step's requests (0: not known).
 extern "C" int celeg_attention_rows_bf16(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
     int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int head_dim,
     int page_tokens, int n_layers, int layer, float scale, int window, int rows_per_tile,
-    hipStream_t stream) {
+    int form, int context_hint, hipStream_t stream) {
     if (n_tokens <= 0 || n_seqs <= 0) return 0;
     if (page_tokens < 16 || (page_tokens & (page_tokens - 1)) || q_heads % kv_heads || (ldq % 8) ||
         (ldo % 4))
         return static_cast<int>(hipErrorInvalidValue);
-    if (rows_per_tile == 0) rows_per_tile = CELEG_ROWS_DEFAULT(n_tokens, n_seqs);
+    if (rows_per_tile == 0) {
+        // tiles of 128 rows read the staged keys for twice the rows, tiles of 64 rows put twice
+        // the workgroups on the chip: the larger ones once there are enough, sooner if each
+        // has many keys to go through
+        const long long small_tiles = static_cast<long long>(n_tokens / 64 + n_seqs) * q_heads;
+        int keys = context_hint > 0 ? context_hint : n_tokens;
+        if (window > 0 && window < keys) keys = window;
+        rows_per_tile = small_tiles >= 1024 || (small_tiles >= 512 && keys >= 4096) ? 128 : 64;
+    }
     if (rows_per_tile != 64 && rows_per_tile != 128) return static_cast<int>(hipErrorInvalidValue);
-#define CELEG_ROWS(HD_)                                                                          \
-    return rows_per_tile == 64                                                                   \
-        ? launch_attention_rows<HD_, 1>(q, ldq, k_pool, v_pool, table, table_stride, cu_seqlens, \
-              seq_slot, seq_start, n_seqs, n_tokens, out, ldo, q_heads, kv_heads, page_tokens,   \
-              n_layers, layer, scale, window, stream)                                            \
-        : launch_attention_rows<HD_, 2>(q, ldq, k_pool, v_pool, table, table_stride, cu_seqlens, \
-              seq_slot, seq_start, n_seqs, n_tokens, out, ldo, q_heads, kv_heads, page_tokens,   \
-              n_layers, layer, scale, window, stream)
+    if (form == 0) {
+        const int group = q_heads / kv_heads;
+        const long long shared = static_cast<long long>(n_tokens / rows_per_tile + n_seqs) * kv_heads * ((group + 1) / 2);
+        form = group >= 2 && shared >= 1024 ? 3 : 2;
+    }
+    if (form < 1 || form > 3) return static_cast<int>(hipErrorInvalidValue);
+#define CELEG_ROWS_ARGS                                                                            \
+    q, ldq, k_pool, v_pool, table, table_stride, cu_seqlens, seq_slot, seq_start, n_seqs, n_tokens, \
+        out, ldo, q_heads, kv_heads, page_tokens, n_layers, layer, scale, window, stream
+#define CELEG_ROWS_RT(HD_, RT_)                                                              \
+    (form == 1 ? launch_attention_rows<HD_, RT_, 1, false>(CELEG_ROWS_ARGS)                   \
+     : form == 2 ? launch_attention_rows<HD_, RT_, 2, false>(CELEG_ROWS_ARGS)                 \
+                 : launch_attention_rows<HD_, RT_, 2, true>(CELEG_ROWS_ARGS))
+#define CELEG_ROWS(HD_) return rows_per_tile == 64 ? CELEG_ROWS_RT(HD_, 1) : CELEG_ROWS_RT(HD_, 2)
     switch (head_dim) {
         case 32: CELEG_ROWS(32);
         case 64: CELEG_ROWS(64);
@@ -370,6 +459,8 @@ extern "C" int celeg_attention_rows_bf16(
         default: return static_cast<int>(hipErrorInvalidValue);
     }
 #undef CELEG_ROWS
+#undef CELEG_ROWS_RT
+#undef CELEG_ROWS_ARGS
 }
 
 // ================================================================ one row per request

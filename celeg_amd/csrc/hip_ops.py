@@ -44,6 +44,7 @@ class HipOps:
         # the general kernel (tests compare the two)
         self.attention_decode_whole = -1     # -1: chosen from the batch; 0 split-key kernels; 1 one workgroup per request and key/value head
         self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
+        self.attention_rows_form = 0         # 0: the kernel chooses; 1, 2 or 3 to force (see attention_fast.hip)
         self.attention_impl = "auto"
         self._decode_ws = None
         self._retired = []
@@ -380,6 +381,7 @@ class HipOps:
                         _c_int(heads * head_dim), _c_int(heads), _c_int(kv_heads), _c_int(head_dim),
                         _c_int(kv.page_tokens), _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
                         _c_int(window if window else 0), _c_int(self.attention_rows_per_tile),
+                        _c_int(self.attention_rows_form), _c_int(getattr(batch, "max_context_len", 0) or 0),
                         self._stream())
                     self._check(code, "attention over rows (bfloat16)")
                 return

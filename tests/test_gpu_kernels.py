@@ -365,13 +365,19 @@ def test_attention_window_fast_kernels(ops):
 
 
 @pytest.mark.parametrize("rows_per_tile", [64, 128])
+@pytest.mark.parametrize("form", [1, 2, 3])
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [
-    (4, 2, 64, 16), (2, 1, 128, 32), (3, 3, 96, 16), (4, 1, 32, 64)])
-def test_attention_rows_tile_pairs(ops, rows_per_tile, heads, kv_heads, head_dim, page_tokens):
-    """Portions of many row tiles (an odd and an even number of them, so that a tile with
-    and without a partner occurs), continued at a position inside a tile, at either tile
-    size; then the same with a window that ends inside a round of keys."""
+    (4, 2, 64, 16), (2, 1, 128, 32), (3, 3, 96, 16), (4, 1, 32, 64), (2, 2, 64, 128), (6, 2, 64, 16),
+    (3, 1, 96, 32)])
+def test_attention_rows_tiles_and_forms(ops, rows_per_tile, form, heads, kv_heads, head_dim, page_tokens):
+    """Portions of many row tiles (tiles with an odd and an even number of rounds of keys,
+    so that the wavefronts that take the rounds in turn get equal and unequal shares),
+    continued at a position inside a tile, at either tile size, with the rounds of keys taken
+    by one set of wavefronts, shared between two, or by two sets that each take a query head
+    of a group (groups of 1, 2, 3 and 4 heads); then the same with a window that ends inside a
+    round of keys.  Pages shorter and longer than a round."""
     ops.attention_rows_per_tile = rows_per_tile
+    ops.attention_rows_form = form
     try:
         attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[717, 150, 390],
                        cuts=[330, 61, 200], boost=(2, 700), page_tokens=page_tokens)
@@ -383,6 +389,7 @@ def test_attention_rows_tile_pairs(ops, rows_per_tile, heads, kv_heads, head_dim
                        page_tokens=page_tokens)
     finally:
         ops.attention_rows_per_tile = 0
+        ops.attention_rows_form = 0
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [
