@@ -245,6 +245,162 @@ def test_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path):
         assert_close_f32(got2[rid], ref, f"toy again/{rid}")
 
 
+# ---------------------------------------------------------------- a toy routed feed-forward and position encoding
+def register_toy_routed():
+    """A feed-forward that routes every token to the one expert its router scores highest
+    (SwiGLU experts, the router's score in 32-bit, written with torch), and a rotary
+    encoding whose frequencies are the usual ones divided by a factor (positions stretched).
+    Both are registered here, from outside the framework, with an architecture that mixes
+    routed and dense layers."""
+    from celeg_amd.config import (Architecture, LayerSpec, ModelSpec, PartSpec, RunStep,
+                                  register_architecture, registered_architectures)
+    from celeg_amd.parts import (FeedForward, PositionEncoding, WeightSpec, register_part,
+                                 registered_parts)
+
+    class TopOneExperts(FeedForward):
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.width, self.ff = int(self.params["width"]), int(self.params["ff"])
+            self.experts = int(self.params["experts"])
+
+        def weight_specs(self):
+            specs = {"router": WeightSpec((self.experts, self.width))}
+            for e in range(self.experts):
+                specs[f"gate{e}"] = WeightSpec((self.ff, self.width))
+                specs[f"up{e}"] = WeightSpec((self.ff, self.width))
+                specs[f"down{e}"] = WeightSpec((self.width, self.ff))
+            return specs
+
+        def load(self, tensors, rt):
+            self.w = tensors
+
+        def forward(self, x, batch, rt):
+            xf = x.float()
+            choice = (xf @ self.w["router"].float().t()).argmax(dim=1)
+            out = rt.ws.buf("toy_routed_out", (x.shape[0], self.width), rt.dtype)
+            for e in range(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                xe = xf[rows]
+                act = torch.nn.functional.silu(xe @ self.w[f"gate{e}"].float().t()) * (xe @ self.w[f"up{e}"].float().t())
+                out[rows] = (act @ self.w[f"down{e}"].float().t()).to(rt.dtype)
+            return out
+
+    class StretchedRope(PositionEncoding):
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.theta, self.factor = float(self.params["theta"]), float(self.params["factor"])
+            self.rotary_dim = int(self.params["rotary_dim"])
+
+        def tables(self, rt):
+            freq = [self.theta ** (-2.0 * i / self.rotary_dim) / self.factor for i in range(self.rotary_dim // 2)]
+            return {"inv_freq": torch.tensor(freq, dtype=torch.float64).to(torch.float32).to(rt.device),
+                    "rotary_dim": self.rotary_dim}
+
+    if "toy_top_one" not in registered_parts("ffn"):
+        register_part("ffn", "toy_top_one", TopOneExperts)
+    if "toy_stretched_rope" not in registered_parts("position"):
+        register_part("position", "toy_stretched_rope", StretchedRope)
+
+    def build_spec(cfg):
+        H, ff, E = cfg["width"], cfg["ff"], cfg["experts"]
+        norm = lambda name: PartSpec("rmsnorm", {"width": H, "eps": 1e-5}, {"weight": name})
+        layers = []
+        for i, kind in enumerate(cfg["layers"]):
+            p = f"blocks.{i}."
+            mixer = PartSpec("gqa_attention",
+                             {"width": H, "heads": 3, "kv_heads": 1, "head_dim": 16, "qk_norm": False,
+                              "position": PartSpec("toy_stretched_rope",
+                                                   {"theta": 50.0, "factor": cfg["stretch"], "rotary_dim": 8})},
+                             {"q_proj": p + "att.q", "k_proj": p + "att.k", "v_proj": p + "att.v",
+                              "out_proj": p + "att.o"})
+            if kind == "routed":
+                names = {"router": p + "router"}
+                for e in range(E):
+                    names.update({f"gate{e}": p + f"e{e}.g", f"up{e}": p + f"e{e}.u", f"down{e}": p + f"e{e}.d"})
+                ffn = PartSpec("toy_top_one", {"width": H, "ff": ff, "experts": E}, names)
+            else:
+                ffn = PartSpec("swiglu", {"width": H, "ff": ff},
+                               {"gate": p + "ff.g", "up": p + "ff.u", "down": p + "ff.d"})
+            layers.append(LayerSpec(mixer, norm(p + "n1"), ffn, norm(p + "n2")))
+        return ModelSpec("ToyRoutedForCausalLM", cfg["vocab"], H, 128,
+                         PartSpec("embedding", {"vocab": cfg["vocab"], "width": H}, {"table": "emb"}),
+                         tuple(layers), tuple(RunStep(i) for i in range(len(layers))),
+                         norm("final"), PartSpec("tied_head", {"vocab": cfg["vocab"], "width": H}))
+
+    if "ToyRoutedForCausalLM" not in registered_architectures():
+        register_architecture(Architecture("ToyRoutedForCausalLM", lambda d: d, build_spec))
+
+
+def toy_routed_plain_logits(cfg, W, tokens):
+    """Whole-sequence reference of the routed toy model, from the plain parts; also the
+    expert every token took in every routed layer."""
+    h = plain.embedding(W["emb"], tokens)
+    T = len(tokens)
+    taken = []
+    for i, kind in enumerate(cfg["layers"]):
+        p = f"blocks.{i}."
+        n = plain.rmsnorm(h, W[p + "n1"], 1e-5)
+        q = plain.linear(n, W[p + "att.q"]).reshape(T, 3, 16)
+        k = plain.linear(n, W[p + "att.k"]).reshape(T, 1, 16)
+        v = plain.linear(n, W[p + "att.v"]).reshape(T, 1, 16)
+        # stretched positions: the angle is position / factor times the usual frequency
+        cos, sin = plain.rope_cos_sin([t / cfg["stretch"] for t in range(T)], 50.0, 8)
+        o = plain.causal_attention(plain.rope_apply(q, cos, sin), plain.rope_apply(k, cos, sin), v)
+        h = h + plain.linear(o.reshape(T, -1), W[p + "att.o"])
+        n = plain.rmsnorm(h, W[p + "n2"], 1e-5)
+        if kind == "routed":
+            scores = plain.linear(n, W[p + "router"])
+            choice = scores.argmax(dim=1)
+            taken.append((choice, scores))
+            out = torch.zeros_like(h)
+            for t in range(T):
+                e = int(choice[t])
+                out[t] = plain.swiglu_ffn(n[t:t + 1], W[p + f"e{e}.g"], W[p + f"e{e}.u"], W[p + f"e{e}.d"])[0]
+            h = h + out
+        else:
+            h = h + plain.swiglu_ffn(n, W[p + "ff.g"], W[p + "ff.u"], W[p + "ff.d"])
+    return plain.linear(plain.rmsnorm(h, W["final"], 1e-5), W["emb"]), taken
+
+
+def test_toy_routed_feed_forward_and_position_encoding_are_registered_and_stepped(tmp_path):
+    """A feed-forward with routing and a position encoding of their own, registered from
+    the test, in an architecture with routed and dense layers: portions of two requests
+    against the plain whole-sequence reference.  Tokens whose two best router scores lie too
+    close for 32-bit to tell apart are not compared (none is expected with these weights);
+    every expert is taken by some token."""
+    from celeg_amd.engine import load_model
+    from celeg_amd.weights import write_random_model
+    register_toy_routed()
+    cfg = {"architectures": ["ToyRoutedForCausalLM"], "width": 48, "ff": 40, "experts": 3, "vocab": 91,
+           "stretch": 4.0, "layers": ["routed", "dense", "routed"]}
+    folder = write_random_model(cfg, str(tmp_path / "toy_routed"), seed=9, dtype=torch.float32, std=0.25)
+    _, W = plain.load_model_folder(folder)
+    reqs = {"x": random_tokens(91, 50, 3), "y": random_tokens(91, 37, 4)}
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2,
+                    max_batched_tokens=64)
+    got = EngineDriver(lm).run(portions_schedule(reqs))
+    experts_seen = set()
+    for rid, toks in reqs.items():
+        ref, taken = toy_routed_plain_logits(cfg, W, toks)
+        clear = torch.ones(len(toks), dtype=torch.bool)
+        for choice, scores in taken:
+            top2 = scores.topk(2, dim=1).values
+            clear &= (top2[:, 0] - top2[:, 1]) > 1e-4
+            experts_seen.update(choice.tolist())
+        # a token routed the other way changes the rows after it too
+        first_unclear = int((~clear).nonzero()[0]) if (~clear).any() else len(toks)
+        assert first_unclear > len(toks) // 2, "the weights leave too few tokens with a clear choice"
+        assert_close_f32(got[rid][:first_unclear], ref[:first_unclear], f"toy routed/{rid}")
+    assert experts_seen == {0, 1, 2}
+    # the stretch matters: the same weights with factor 1 give other logits
+    toks = reqs["x"]
+    other, _ = toy_routed_plain_logits(dict(cfg, stretch=1.0), W, toks)
+    ref, _ = toy_routed_plain_logits(cfg, W, toks)
+    assert (other - ref).abs().max() > 1e-3
+
+
 def test_run_order_with_a_layer_twice_and_a_shared_cache(model_folders, tmp_path):
     """LFM2 parts under another run order: layer 1 runs twice (own cache each time) and
     layer 3 reads the keys and values the first run of layer 1 wrote."""
