@@ -11,7 +11,9 @@
 // request, with its state update.
 //
 // Layout.  At these sizes the weights are read once from memory and the rows of A come
-// from cache.  A workgroup owns CT tiles of 16 columns (of every weight stream) over the
+// from cache.  A workgroup owns CT tiles of 16 columns (of every weight stream), for MT tiles
+// of 16 rows (all rows, or a part of them where the columns alone give fewer workgroups
+// than the chip has compute units: the weights are then read once per part, from L2), over the
 // WHOLE of K, which its wavefronts split between them; a wavefront keeps
 // MT x (streams x CT) tiles of 16x16 sums, reads 16 bytes of weights per lane and tile for
 // 32 values of k and the rows of A straight into the instruction's operand layout (whole
@@ -38,6 +40,7 @@ enum { E_STORE = 0, E_STORE_F32 = 1, E_RESIDUAL = 2, E_SWIGLU = 3, E_CONV = 4 };
 #define ROWS_MAX_TAPS 8
 #define ROWS_MAX_STAT_BLOCKS 512
 #define ROWS_MAX_LDS (128 * 1024)
+#define ROWS_COMPUTE_UNITS 256
 
 __device__ __forceinline__ float round_bf16(float x) { return to_float(from_float<bf16>(x)); }
 
@@ -145,13 +148,14 @@ void gemm_rows_kernel(const GemvParams p) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int M = p.M, N = p.N, K = p.K;
     const int n0 = blockIdx.x * COLS;
+    const int row0 = blockIdx.y * ROWS;        // the workgroup's first row
     const int c16 = lane & 15, q = lane >> 4;
 
     // ---- operands: A rows t*16 + c16, W columns n0 + ct*16 + c16 of every stream
     const bf16* arow[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-        const int m = min(t * 16 + c16, M - 1);
+        const int m = min(row0 + t * 16 + c16, M - 1);
         arow[t] = static_cast<const bf16*>(p.a) + static_cast<size_t>(p.rows ? p.rows[m] : m) * p.lda + q * p.a_k8_stride;
     }
     const bf16* wcol[SC];
@@ -193,7 +197,7 @@ void gemm_rows_kernel(const GemvParams p) {
 
     // ---- what the end of this thread's first output needs (asked for behind the first weights)
     const int e0 = min(static_cast<int>(threadIdx.x), ROWS * COLS - 1);
-    const Early<EPI> early0 = early_fetch<EPI>(p, min(e0 / COLS, M - 1), min(n0 + e0 % COLS, N - 1));
+    const Early<EPI> early0 = early_fetch<EPI>(p, min(row0 + e0 / COLS, M - 1), min(n0 + e0 % COLS, N - 1));
 
     // ---- the rows' 1/rms from the partial sums of squares (likewise): LPR neighbouring
     // threads share a row
@@ -201,7 +205,7 @@ void gemm_rows_kernel(const GemvParams p) {
         const int lpr = blockDim.x / ROWS;           // a power of two, 1 .. 32
         const int r = threadIdx.x / lpr, sub = threadIdx.x % lpr;
         const int nb = p.n_stat_blocks;
-        const int m = min(r, M - 1);
+        const int m = min(row0 + r, M - 1);
         const float* srow = p.stats + static_cast<size_t>(p.rows ? p.rows[m] : m) * p.stats_ld;
         float ssq = 0.f;
         for (int b0 = 0; b0 < nb; b0 += 8 * lpr) {   // the same trips for every thread
@@ -236,10 +240,10 @@ void gemm_rows_kernel(const GemvParams p) {
     // ---- thread e takes row e / COLS, column e % COLS of the workgroup's tile
     const int n_threads = blockDim.x;
     for (int e = threadIdx.x; e < ROWS * COLS; e += n_threads) {
-        const int r = e / COLS, j = e % COLS;
-        const int t = r >> 4, rr = r & 15, ct = j >> 4, jj = j & 15;
+        const int rl = e / COLS, j = e % COLS;      // row inside the workgroup's rows
+        const int t = rl >> 4, rr = rl & 15, ct = j >> 4, jj = j & 15;
         const int src = jj + 16 * (rr >> 2), reg = rr & 3;
-        const int n = n0 + j;
+        const int r = row0 + rl, n = n0 + j;
         const bool ok = r < M && n < N;
         const int rc = min(r, M - 1), nc = min(n, N - 1);
         float sum[NS];
@@ -250,7 +254,7 @@ void gemm_rows_kernel(const GemvParams p) {
                 v += red[(((static_cast<size_t>(w) * MT + t) * SC + s * CT + ct) * 4 + reg) * 64 + src];
             sum[s] = v;
         }
-        const float scale = p.stats ? s_scale[r] : 1.f;
+        const float scale = p.stats ? s_scale[rl] : 1.f;
 #pragma unroll
         for (int s = 0; s < NS; ++s) sum[s] *= scale;
         float v = 0.f;
@@ -275,8 +279,8 @@ struct RowsShape {
     int mt, ct, waves;
 };
 
-static int g_force_ct = 0, g_force_waves = 0;   // tuning aids: override the choice below where they fit
-extern "C" void celeg_gemm_rows_force(int ct, int waves) { g_force_ct = ct; g_force_waves = waves; }
+static int g_force_ct = 0, g_force_waves = 0, g_force_mt = 0;   // tuning aids: override the choice below where they fit
+extern "C" void celeg_gemm_rows_force(int ct, int waves, int mt) { g_force_ct = ct; g_force_waves = waves; g_force_mt = mt; }
 
 static RowsShape rows_shape(int M, int N, int K, int streams) {
     RowsShape s;
@@ -285,8 +289,14 @@ static RowsShape rows_shape(int M, int N, int K, int streams) {
     s.ct = 1;
     while (s.ct < max_ct && (N + 32 * s.ct - 1) / (32 * s.ct) >= 1024) s.ct *= 2;
     if (g_force_ct > 0 && g_force_ct <= max_ct) s.ct = g_force_ct;
+    // few columns: the rows are shared out too, until there is a workgroup per compute unit
+    while (s.mt > 1 && ((N + 16 * s.ct - 1) / (16 * s.ct)) * ((M + 16 * s.mt - 1) / (16 * s.mt)) < ROWS_COMPUTE_UNITS)
+        s.mt >>= 1;
+    if ((g_force_mt == 1 || g_force_mt == 2 || g_force_mt == 4) && g_force_mt <= (M <= 16 ? 1 : (M <= 32 ? 2 : 4)))
+        s.mt = g_force_mt;
     const int nkb = K / 32;
     s.waves = rows_max_waves(s.mt, streams * s.ct);
+    if (K <= 2048 && s.waves > 8) s.waves = 8;     // a short K: two workgroups of 8 a compute unit were the faster
     while (s.waves > 1 && s.waves * 2 > nkb) s.waves >>= 1;
     if (g_force_waves > 0 && g_force_waves <= rows_max_waves(s.mt, streams * s.ct)) s.waves = g_force_waves;
     return s;
@@ -303,7 +313,7 @@ static int launch_rows(const GemvParams& p, int waves, hipStream_t stream) {
         if (err != hipSuccess) return static_cast<int>(err);
         raised = true;
     }
-    dim3 grid((p.N + CT * 16 - 1) / (CT * 16)), block(waves * 64);
+    dim3 grid((p.N + CT * 16 - 1) / (CT * 16), (p.M + MT * 16 - 1) / (MT * 16)), block(waves * 64);
     hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p);
     return CELEG_LAUNCH_RESULT();
 }
