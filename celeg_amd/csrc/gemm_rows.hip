@@ -279,7 +279,10 @@ struct RowsShape {
     int mt, ct, waves;
 };
 
-static int g_force_ct = 0, g_force_waves = 0, g_force_mt = 0;   // tuning aids: override the choice below where they fit
+// For tests and tuning: a share of columns (ct: 1, 2 or 4 tiles of 16), a number of
+// wavefronts and a share of rows (mt: 1, 2 or 4 tiles of 16) that override the choice below
+// where they fit; 0 leaves a choice alone.
+static int g_force_ct = 0, g_force_waves = 0, g_force_mt = 0;
 extern "C" void celeg_gemm_rows_force(int ct, int waves, int mt) { g_force_ct = ct; g_force_waves = waves; g_force_mt = mt; }
 
 static RowsShape rows_shape(int M, int N, int K, int streams) {

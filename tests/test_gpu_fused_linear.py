@@ -239,6 +239,26 @@ def test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, M, H, taps
     assert float(state[0].abs().max()) == 0.0          # a slot nobody uses stays zero
 
 
+@pytest.mark.parametrize("mt", [1, 2, 4])
+@pytest.mark.parametrize("ct", [1, 2, 4])
+def test_rows_kernel_with_every_share_of_rows_and_columns(ops, mt, ct):
+    """The kernel for 9 to 64 rows chooses how many rows (16, 32 or 64) and columns (16, 32 or
+    64 of every weight stream) a workgroup takes from the sizes; here every choice is forced in
+    turn (a wider share of columns than an epilogue's streams allow falls back to the kernel's
+    own), for every epilogue, at sizes that leave a part of a share empty."""
+    lib = ops._lib("gemm_rows")
+    lib.celeg_gemm_rows_force(ct, 0, mt)
+    try:
+        test_sliced_products_behind_a_norm(ops, 50, 1000, 352)
+        test_sliced_products_behind_a_norm(ops, 64, 272, 4608)
+        test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, 64, 272, 1024)
+        test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, 33, 1000, 352)
+        test_sliced_swiglu(ops, 40, 352, 128)
+        test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, 62, 96, 4, True)
+    finally:
+        lib.celeg_gemm_rows_force(0, 0, 0)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 64), (4, 1024, 1024), (5, 77, 352), (8, 96, 4608), (16, 272, 1024),
                                    (20, 77, 352), (33, 1024, 1024), (64, 272, 1024)])
 def test_packed_weights_give_the_same_bits(ops, M, N, K):
