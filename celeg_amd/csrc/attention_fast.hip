@@ -467,20 +467,21 @@ extern "C" int celeg_attention_rows_bf16(
 // Decode attention works on rounds of 64 keys.
 #define DEC_KEYS 64
 
-// Joins the rounds of one (request, query head): out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
-// A lane owns an output dimension (and the (m, l) of rounds lane, lane + 64, ..).  The rounds'
+// Joins the parts of one (request, query head), a part being split_rounds rounds of 64 keys:
+// out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
+// A lane owns an output dimension (and the (m, l) of parts lane, lane + 64, ..).  The parts'
 // outputs are asked for 32 at a time without conditions, the first 32 before anything is
-// waited for, so that a context of 2,048 keys costs two trips to memory.
+// waited for, so that a context of 2,048 keys in parts of one round costs two trips to memory.
 template <int HD>
 __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int* __restrict__ positions, bf16* __restrict__ out, int ldo, int q_heads, int n_splits,
-    int window) {
+    int window, int split_rounds) {
     constexpr int DD = HD / 64, CH = 32;
     const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int first = lo / DEC_KEYS, n_all = pos / DEC_KEYS - first + 1;
+    const int first = lo / DEC_KEYS / split_rounds, n_all = pos / DEC_KEYS / split_rounds - first + 1;
     const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits + first;
     const float* __restrict__ op = ws_o + base * HD + lane;
     float o[CH][DD];
@@ -524,9 +525,9 @@ __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
 // forms.  For batches that fill the chip, one workgroup per (request, key/value head, chunk of
 // 16 heads) and no second kernel: its wavefronts take rounds of 64 keys in turn, each keeps
 // a running maximum, sum and output of its own, and they meet in LDS.  For few requests
-// (SPLIT), a workgroup of one wavefront per round of 64 keys, so that a long context spreads
-// over the chip; the rounds' (max, sum, output) go to a workspace and
-// attention_decode_reduce_kernel joins them.
+// (SPLIT), a workgroup per part of the context (1, 4 or 16 rounds of 64 keys, a wavefront
+// per round), so that a long context spreads over the chip; the parts' (max, sum, output) go
+// to a workspace and attention_decode_reduce_kernel joins them.
 //   S^T[key, head] = K Q^T : a lane holds head lane%16, keys 4*(lane/16)..+3 of a 16-key tile;
 //   O^T[dim, head] = V^T P : P's operand wants 8 keys a lane, which are rows 4q..4q+3 of two
 //   tiles: tile 2j holds keys 32j + 8*(row/4) + row%4, tile 2j+1 those + 4, so that a lane's
@@ -537,7 +538,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ token_slot, const int* __restrict__ positions, bf16* __restrict__ out,
     int ldo, int kv_heads, int group, int page_tokens, int page_shift, int n_layers, int layer,
-    float scale, int window, float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits) {
+    float scale, int window, float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
+    int split_rounds) {
     constexpr int KS = HD / 32;   // steps of 32 dims in q.k
     constexpr int DT = HD / 16;   // 16-dim tiles of the output
     extern __shared__ float smem_heads[];
@@ -566,9 +568,13 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    const int r_first = SPLIT ? static_cast<int>(blockIdx.z) : lo / DEC_KEYS + wave;
-    if (SPLIT && (r_first < lo / DEC_KEYS || r_first > pos / DEC_KEYS)) return;     // the whole workgroup
-    for (int r = r_first; r <= pos / DEC_KEYS; r += SPLIT ? (1 << 30) : WAVES) {
+    // the workgroup's rounds: all of the request's, or (SPLIT) part blockIdx.z of them; its
+    // wavefronts take them in turn
+    const int r_begin = SPLIT ? max(lo / DEC_KEYS, static_cast<int>(blockIdx.z) * split_rounds) : lo / DEC_KEYS;
+    const int r_end = SPLIT ? min(pos / DEC_KEYS, static_cast<int>(blockIdx.z) * split_rounds + split_rounds - 1)
+                            : pos / DEC_KEYS;
+    if (SPLIT && r_begin > r_end) return;     // the whole workgroup
+    for (int r = r_begin + wave; r <= r_end; r += WAVES) {
         const int kb = r * DEC_KEYS;
         const int k_lo = max(lo, kb), k_hi = min(pos, kb + DEC_KEYS - 1);
         const int first_page = kb >> page_shift, last_page = k_hi >> page_shift;
@@ -641,7 +647,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt][j], pb, o[dt], 0, 0, 0);
         }
     }
-    if (SPLIT) {
+    if (SPLIT && WAVES == 1) {
         if (c < gp) {
             const size_t idx = (static_cast<size_t>(t) * (kv_heads * group) + h0 + c) * n_splits + blockIdx.z;
             if (qd == 0) { ws_ml[2 * idx] = m_run; ws_ml[2 * idx + 1] = l_run; }
@@ -673,7 +679,13 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             denom += wgt * part_ml[(w * gp + g) * 2 + 1];
             val = fmaf(wgt, part_o[(static_cast<size_t>(w) * gp + g) * HD + d], val);
         }
-        out[static_cast<size_t>(t) * ldo + static_cast<size_t>(h0 + g) * HD + d] = from_float<bf16>(val / denom);
+        if (SPLIT) {       // the part's (max, sum, output) for the second kernel
+            const size_t idx = (static_cast<size_t>(t) * (kv_heads * group) + h0 + g) * n_splits + blockIdx.z;
+            if (d == 0) { ws_ml[2 * idx] = mxw; ws_ml[2 * idx + 1] = denom; }
+            ws_o[idx * HD + d] = val;
+        } else {
+            out[static_cast<size_t>(t) * ldo + static_cast<size_t>(h0 + g) * HD + d] = from_float<bf16>(val / denom);
+        }
     }
 }
 
@@ -697,8 +709,33 @@ static int launch_decode_heads(const void* q, int ldq, const void* k_pool, const
                        dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
                        table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
-                       group, page_tokens, page_shift, n_layers, layer, scale, window, nullptr, nullptr, 0);
+                       group, page_tokens, page_shift, n_layers, layer, scale, window, nullptr, nullptr, 0, 1);
     return CELEG_LAUNCH_RESULT();
+}
+
+template <int HD, int WAVES>
+static int launch_decode_parts(const void* q, int ldq, const void* k_pool, const void* v_pool,
+                               const int* table, int table_stride, const int* token_slot,
+                               const int* positions, float* ws_o, float* ws_ml, int n_splits, void* out,
+                               int ldo, int n_rows, int kv_heads, int group, int page_tokens,
+                               int page_shift, int n_layers, int layer, float scale, int window,
+                               int split_rounds, int n_parts, hipStream_t stream) {
+    const int chunks = (group + 15) / 16;
+    const size_t lds = WAVES == 1 ? 0 : static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
+    static bool raised = false;
+    if (lds > 48 * 1024 && !raised) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, true>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (err != hipSuccess) return static_cast<int>(err);
+        raised = true;
+    }
+    hipLaunchKernelGGL((attention_decode_heads_kernel<HD, WAVES, true>), dim3(kv_heads * chunks, n_rows, n_parts),
+                       dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
+                       static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
+                       table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
+                       group, page_tokens, page_shift, n_layers, layer, scale, window, ws_o, ws_ml,
+                       n_splits, split_rounds);
+    return 0;
 }
 
 extern "C" int celeg_attention_decode_bf16(
@@ -706,7 +743,7 @@ extern "C" int celeg_attention_decode_bf16(
     int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
     int n_splits, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
     int head_dim, int page_tokens, int n_layers, int layer, float scale, int window, int whole,
-    hipStream_t stream) {
+    int split_rounds, int n_parts, hipStream_t stream) {
     if (n_rows <= 0) return 0;
     const int group = q_heads / kv_heads;
     if (q_heads % kv_heads || page_tokens < 16 || (page_tokens & (page_tokens - 1)) || n_splits <= 0 ||
@@ -731,19 +768,30 @@ extern "C" int celeg_attention_decode_bf16(
                                             n_layers, layer, scale, window, stream);
         return static_cast<int>(hipErrorInvalidValue);
     }
-    dim3 sgrid(kv_heads * chunks, n_rows, n_splits);
-#define CELEG_SPLIT_HEADS(HD_)                                                                   \
-    hipLaunchKernelGGL((attention_decode_heads_kernel<HD_, 1, true>), sgrid, dim3(64), 0, stream, \
-                       static_cast<const bf16*>(q), ldq, static_cast<const bf16*>(k_pool),       \
-                       static_cast<const bf16*>(v_pool), table, table_stride, token_slot,        \
-                       positions, static_cast<bf16*>(out), ldo, kv_heads, group, page_tokens,    \
-                       page_shift, n_layers, layer, scale, window, ws_o, ws_ml, n_splits);       \
-    hipLaunchKernelGGL(attention_decode_reduce_kernel<HD_>, dim3(q_heads, n_rows), dim3(64), 0,  \
-                       stream, ws_o, ws_ml, positions, static_cast<bf16*>(out), ldo, q_heads,    \
-                       n_splits, window)
-    if (head_dim == 64) { CELEG_SPLIT_HEADS(64); }
-    else if (head_dim == 128) { CELEG_SPLIT_HEADS(128); }
+    // Parts of split_rounds rounds of 64 keys (1, 4 or 16), one workgroup each with a wavefront per
+    // round (8 at most for heads of 128), n_parts of them per request: the caller chooses both
+    // so that n_parts * split_rounds * 64 keys cover the longest context of the step, and a
+    // longer context gets longer parts instead of more of them.
+    if ((split_rounds != 1 && split_rounds != 4 && split_rounds != 16) || n_parts <= 0 || n_parts > n_splits)
+        return static_cast<int>(hipErrorInvalidValue);
+#define CELEG_SPLIT_ARGS                                                                           \
+    q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions, ws_o, ws_ml, n_splits, out, \
+        ldo, n_rows, kv_heads, group, page_tokens, page_shift, n_layers, layer, scale, window,     \
+        split_rounds, n_parts, stream
+#define CELEG_SPLIT_HEADS(HD_, MOST_)                                                              \
+    {                                                                                              \
+        const int code = split_rounds == 1 ? launch_decode_parts<HD_, 1>(CELEG_SPLIT_ARGS)         \
+                         : split_rounds == 4 ? launch_decode_parts<HD_, 4>(CELEG_SPLIT_ARGS)       \
+                                             : launch_decode_parts<HD_, MOST_>(CELEG_SPLIT_ARGS);  \
+        if (code) return code;                                                                     \
+    }                                                                                              \
+    hipLaunchKernelGGL(attention_decode_reduce_kernel<HD_>, dim3(q_heads, n_rows), dim3(64), 0,   \
+                       stream, ws_o, ws_ml, positions, static_cast<bf16*>(out), ldo, q_heads,     \
+                       n_splits, window, split_rounds)
+    if (head_dim == 64) { CELEG_SPLIT_HEADS(64, 16); }
+    else if (head_dim == 128) { CELEG_SPLIT_HEADS(128, 8); }
     else return static_cast<int>(hipErrorInvalidValue);
+#undef CELEG_SPLIT_ARGS
 #undef CELEG_SPLIT_HEADS
     return CELEG_LAUNCH_RESULT();
 }

@@ -45,6 +45,9 @@ class HipOps:
         self.attention_decode_whole = -1     # -1: chosen from the batch; 0 split-key kernels; 1 one workgroup per request and key/value head
         self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
         self.attention_rows_form = 0         # 0: the kernel chooses; 1, 2 or 3 to force (see attention_fast.hip)
+        # decode attention over few requests: contexts of up to this many rounds of 64 keys are
+        # cut into parts of 1 round, up to that many into parts of 4, longer ones into parts of 16
+        self.decode_part_thresholds = (64, 256)
         self.attention_impl = "auto"
         self._decode_ws = None
         self._retired = []
@@ -381,7 +384,8 @@ class HipOps:
                         _c_int(heads * head_dim), _c_int(heads), _c_int(kv_heads), _c_int(head_dim),
                         _c_int(kv.page_tokens), _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
                         _c_int(window if window else 0), _c_int(self.attention_rows_per_tile),
-                        _c_int(self.attention_rows_form), _c_int(getattr(batch, "max_context_len", 0) or 0),
+                        _c_int(self.attention_rows_form),
+                        _c_int(getattr(batch, "context_bound", 0) or getattr(batch, "max_context_len", 0) or 0),
                         self._stream())
                     self._check(code, "attention over rows (bfloat16)")
                 return
@@ -403,6 +407,14 @@ class HipOps:
             if self._decode_ws is not None:
                 self._retired.append(self._decode_ws)   # recorded graphs may still point at it
             self._decode_ws = torch.empty(need, dtype=torch.float32, device=q.device)
+        # where the context is cut into parts (few requests): parts of 1, 4 or 16 rounds of 64
+        # keys, so that a long context gets longer parts rather than hundreds of them; the
+        # bound is the step's longest context, or what the step's recorded graph is good for
+        bound = getattr(batch, "context_bound", 0) or getattr(batch, "max_context_len", 0) or max_context
+        rounds = (min(bound, max_context) + 63) // 64
+        few, some = self.decode_part_thresholds
+        split_rounds = 1 if rounds <= few else (4 if rounds <= some else 16)
+        n_parts = (rounds + split_rounds - 1) // split_rounds
         ws_o = self._decode_ws[:T * heads * n_splits * head_dim]
         ws_ml = self._decode_ws[T * heads * n_splits * head_dim:need]
         code = self._lib("attention_fast").celeg_attention_decode_bf16(
@@ -411,7 +423,8 @@ class HipOps:
             _ptr(ws_ml), _c_int(n_splits), _ptr(out), _c_int(heads * head_dim),
             _c_int(T), _c_int(heads), _c_int(kv_heads), _c_int(head_dim), _c_int(kv.page_tokens),
             _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
-            _c_int(window if window else 0), _c_int(self.attention_decode_whole), self._stream())
+            _c_int(window if window else 0), _c_int(self.attention_decode_whole),
+            _c_int(split_rounds), _c_int(n_parts), self._stream())
         self._check(code, "attention for decode rows (bfloat16)")
 
     # ------------------------------------------------------------------ sampling

@@ -47,6 +47,7 @@ class StepBatch:
         self.n_real_seqs = 0
         self.max_seg_len = 0
         self.max_context_len = 0
+        self.context_bound = 0    # set by whoever records the step for replay: the longest context the recording must serve
         self.decode_only = False
         self.single_rows = 0      # rows [0, single_rows) are entries of one token each
         self.entry_order: List[int] = []   # which entry each sequence of the layout is

@@ -66,7 +66,7 @@ class ModelRunner:
                                     pin=torch.device(rt.device).type == "cuda")
         self.steps_run = 0
         self.use_graphs = True
-        self._graphs: Dict[int, tuple] = {}
+        self._graphs: Dict[tuple, tuple] = {}
         self._portion_graphs: Dict[tuple, tuple] = {}
         self._portion_seen: Dict[tuple, int] = {}
         self._token_source: Optional[torch.Tensor] = None
@@ -143,13 +143,26 @@ class ModelRunner:
             return False
         return all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
 
+    # A recorded step's launches are fixed, and the attention over few requests sizes its grid
+    # by the context: a graph is therefore good up to a bound on the context, and there is one
+    # per (batch-size bucket, bound).
+    CONTEXT_BOUNDS = (4096, 16384, 65536)
+
+    def _context_bound(self, entries: Sequence[StepEntry]) -> int:
+        longest = max(e.start_pos + len(e.tokens) for e in entries)
+        for bound in self.CONTEXT_BOUNDS:
+            if longest <= bound:
+                return min(bound, self.cache.max_context)
+        return self.cache.max_context
+
     def _step_from_graph(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         S = len(entries)
         bucket = next(b for b in self._buckets if b >= S)
+        bound = self._context_bound(entries)
         caps = [bucket + 8] * len(self.cache.groups)
-        captured = self._graphs.get(bucket)
+        captured = self._graphs.get((bucket, bound))
         if captured is None or captured[2] != self.rt.ws.generation:
-            captured = self._capture(bucket, caps)
+            captured = self._capture(bucket, caps, bound)
         updates = self.cache.drain_table_updates()
         for g, u in enumerate(updates):
             if len(u) > caps[g]:           # a burst (a large reservation): ship it on its own
@@ -162,11 +175,16 @@ class ModelRunner:
         self.steps_run += 1
         return captured[1][:S]
 
-    def _capture(self, bucket: int, caps):
+    def _capture(self, bucket: int, caps, bound: int):
         empty = [[] for _ in self.cache.groups]
-        captured = self._capture_batch(lambda: self.builder.build(
-            [], empty, pad_to=bucket, null_slot=self.cache.null_slot, update_caps=caps))
-        self._graphs[bucket] = captured
+
+        def make_batch():
+            batch = self.builder.build([], empty, pad_to=bucket, null_slot=self.cache.null_slot,
+                                       update_caps=caps)
+            batch.context_bound = bound
+            return batch
+        captured = self._capture_batch(make_batch)
+        self._graphs[(bucket, bound)] = captured
         return captured
 
     # ------------------------------------------------------------------ captured portions
@@ -176,6 +194,7 @@ class ModelRunner:
     # captured for that size, on the null slot like the decode graphs.
     PORTION_GRAPHS = 8          # sizes kept
     PORTION_MIN_TOKENS = 32
+    LONG_CONTEXT = 4096
 
     def _portion_shape(self, entries: Sequence[StepEntry]):
         if not self.use_graphs or torch.device(self.rt.device).type != "cuda" \
@@ -188,7 +207,8 @@ class ModelRunner:
         want = list(e.want)
         if want not in ([], [n - 1]):
             return None
-        shape = (n, len(want))
+        # (the attention over a portion's rows chooses its tiles by the context too: a long one or not)
+        shape = (n, len(want), e.start_pos + n >= self.LONG_CONTEXT)
         if shape not in self._portion_graphs:
             seen = self._portion_seen.get(shape, 0) + 1
             self._portion_seen[shape] = seen
@@ -197,13 +217,18 @@ class ModelRunner:
         return shape
 
     def _portion_from_graph(self, entries: Sequence[StepEntry], shape) -> torch.Tensor:
-        n, n_want = shape
+        n, n_want, long_context = shape
         caps = [n // self.cache.page_tokens + 10] * len(self.cache.groups)
         captured = self._portion_graphs.get(shape)
         if captured is None or captured[2] != self.rt.ws.generation:
             null = [StepEntry(self.cache.null_slot, 0, [0] * n, [n - 1] if n_want else [])]
-            captured = self._capture_batch(lambda: self.builder.build(
-                null, [[] for _ in self.cache.groups], null_slot=self.cache.null_slot, update_caps=caps))
+
+            def make_batch():
+                batch = self.builder.build(null, [[] for _ in self.cache.groups],
+                                           null_slot=self.cache.null_slot, update_caps=caps)
+                batch.context_bound = 2 * self.LONG_CONTEXT if long_context else 0
+                return batch
+            captured = self._capture_batch(make_batch)
             self._portion_graphs[shape] = captured
         updates = self.cache.drain_table_updates()
         for g, u in enumerate(updates):

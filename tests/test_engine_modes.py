@@ -139,6 +139,34 @@ def test_long_decoding(model_folders, name, dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_across_the_bounds_of_recorded_steps(model_folders, dtype):
+    """A recorded decode step serves contexts up to a bound (the attention over few requests
+    cuts the context into parts by it), and a longer context takes another recording.  With
+    the bounds pulled down to 64 and 160 tokens, and parts of 4 rounds from 2 rounds on, two
+    requests decode from 20 to 330 tokens through all three recordings; every position is
+    compared with the plain implementation."""
+    from celeg_amd.engine import load_model
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders("D", storage, WEIGHT_STD)
+    cfg = TINY["D"][0]
+    reqs = {f"bound{i}": random_tokens(cfg["vocab_size"], 330 - 11 * i, seed=940 + i) for i in range(2)}
+    steps = merged_schedule({rid: tail_decode_schedule({rid: toks}, tail=len(toks) - 20)
+                             for rid, toks in reqs.items()})
+    lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16, max_requests=2,
+                    max_batched_tokens=256)
+    lm.runner.CONTEXT_BOUNDS = (64, 160)
+    if hasattr(lm.rt.ops, "decode_part_thresholds"):
+        lm.rt.ops.decode_part_thresholds = (1, 8)
+    got = EngineDriver(lm).run(steps)
+    cfgp, W = plain.load_model_folder(folder)
+    for rid, toks in reqs.items():
+        assert_close(got[rid], plain.model_logits(cfgp, W, toks), dtype, f"D/{dtype}/bounds/{rid}")
+    assert {bound for _, bound in lm.runner._graphs} == {64, 160, lm.cache.max_context}
+    lm.cache.check()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_first_tokens_of_a_sequence(model_folders, name, dtype):
     """Position 0 and its neighbours: requests that start with one, two and three tokens
@@ -189,7 +217,7 @@ def test_portions_of_a_repeated_size_are_replayed(model_folders, name, dtype):
     lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16 + 1,
                     max_requests=4, max_batched_tokens=64)
     got = EngineDriver(lm).run(steps)
-    assert set(lm.runner._portion_graphs) == {(48, 0), (48, 1)}
+    assert set(lm.runner._portion_graphs) == {(48, 0, False), (48, 1, False)}
     cfgp, W = plain.load_model_folder(folder)
     for rid, toks in reqs.items():
         ref = plain.model_logits(cfgp, W, toks)

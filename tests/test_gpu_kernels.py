@@ -395,15 +395,19 @@ def test_attention_rows_tiles_and_forms(ops, rows_per_tile, form, heads, kv_head
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [
     (8, 2, 64, 16), (3, 1, 64, 64), (6, 1, 128, 32), (16, 1, 64, 16), (40, 2, 64, 32), (4, 4, 64, 16),
     (32, 8, 64, 16), (12, 2, 128, 16), (4, 2, 64, 16), (8, 1, 128, 32)])
-@pytest.mark.parametrize("whole", [0, 1])
+@pytest.mark.parametrize("whole", [0, 1, 4, 16])
 def test_attention_decode_one_workgroup_per_request(ops, heads, kv_heads, head_dim, page_tokens, whole):
-    """(whole 0: the same rounds of keys as workgroups of their own, joined by a second kernel.)
+    """(whole 0: the same rounds of keys as workgroups of their own, joined by a second kernel;
+    4 and 16: parts of 4 and of 16 rounds a workgroup, a wavefront per round, joined likewise:
+    contexts that fill a part, leave its end empty, and need several.)
     The decode kernel that walks a request's whole context in one workgroup, the query
     heads of a key/value head being the rows of its matrix instructions (groups of 1 to 20
     heads; more than 16 take two workgroups): long contexts (more rounds of 64 keys than
     wavefronts), a boosted far key, a window that cuts the first round of keys, the last round
     ending inside a page."""
-    ops.attention_decode_whole = whole
+    ops.attention_decode_whole = min(whole, 1) if whole <= 1 else 0
+    if whole > 1:
+        ops.decode_part_thresholds = (0, 1 << 30) if whole == 4 else (0, 0)
     try:
         attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[1300, 150, 70],
                        cuts=[1260] + [1] * 40, boost=(2, 1290), page_tokens=page_tokens)
@@ -415,3 +419,4 @@ def test_attention_decode_one_workgroup_per_request(ops, heads, kv_heads, head_d
                        qk_norm=False, rotary_dim=0, page_tokens=page_tokens)
     finally:
         ops.attention_decode_whole = -1
+        ops.decode_part_thresholds = (64, 256)
