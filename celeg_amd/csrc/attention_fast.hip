@@ -574,7 +574,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     const int r_end = SPLIT ? min(pos / DEC_KEYS, static_cast<int>(blockIdx.z) * split_rounds + split_rounds - 1)
                             : pos / DEC_KEYS;
     if (SPLIT && r_begin > r_end) return;     // the whole workgroup
-    for (int r = r_begin + wave; r <= r_end; r += WAVES) {
+    // (a part of one round: the stride tells the compiler that the loop runs once)
+    for (int r = r_begin + wave; r <= r_end; r += (SPLIT && WAVES == 1) ? (1 << 30) : WAVES) {
         const int kb = r * DEC_KEYS;
         const int k_lo = max(lo, kb), k_hi = min(pos, kb + DEC_KEYS - 1);
         const int first_page = kb >> page_shift, last_page = k_hi >> page_shift;
