@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
     const int tile = tiles - 1 - idx;
     const int start = seq_start[s];
     const int brow0 = tile * ROWS;
-    const int first = ((window > 0 ? max(0, start + brow0 - window + 1) : 0) >> 6) << 6;   // first key of round 0
+    const int first = ((window > 0 ? max(0, start + brow0 - window + 1) : 0) >> 6) << 6;   // first key of the first round
     const int bkmax = start + min(brow0 + ROWS - 1, len - 1);                              // last key the tile sees
     const int total_rounds = ((bkmax - first) >> 6) + 1;
     constexpr int TURNS = SHARE ? 1 : NH;          // halves that take the rounds in turn

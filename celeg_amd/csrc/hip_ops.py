@@ -26,6 +26,11 @@ class KernelError(RuntimeError):
     pass
 
 
+def _raw_stream(device_index: int) -> int:
+    """The raw handle of torch's current stream on a device."""
+    return torch._C._cuda_getCurrentRawStream(device_index)
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return _c_void_p(0 if t is None else t.data_ptr())
 
@@ -43,6 +48,10 @@ class HipOps:
         # "auto": the matrix-core and split-key kernels where they apply; "general": always
         # the general kernel (tests compare the two)
         self.attention_decode_whole = -1     # -1: chosen from the batch; 0 split-key kernels; 1 one workgroup per request and key/value head
+        self.use_blaslt = True               # products of many rows: hipBLASLt called directly
+        self._blaslt = None
+        self._device_index = torch.device(device).index if torch.device(device).index is not None \
+            else torch.cuda.current_device()
         self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
         self.attention_rows_form = 0         # 0: the kernel chooses; 1, 2 or 3 to force (see attention_fast.hip)
         # decode attention over few requests: contexts of up to this many rounds of 64 keys are
@@ -80,7 +89,8 @@ class HipOps:
         return lib
 
     def _stream(self):
-        return _c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        # (the raw handle of torch's current stream, without building a stream object per launch)
+        return _c_void_p(_raw_stream(self._device_index))
 
     def _check(self, code: int, what: str) -> None:
         if code != 0:
@@ -254,17 +264,29 @@ class HipOps:
         if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
             raise KernelError(f"linear: unsupported dtypes {x.dtype} x {w.dtype}")
         if out.dtype == torch.bfloat16:
-            torch.mm(x, w.t(), out=out)
+            self._library_product(x, w, out)
             if bias is not None:
                 self.add_bias(out, bias)
         elif out.dtype == torch.float32:
-            tmp = torch.mm(x, w.t())
+            tmp = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            self._library_product(x, w, tmp)
             self.cast(tmp, out)
             if bias is not None:
                 self.add_bias(out, bias)
         else:
             raise KernelError("linear: out must be bfloat16 or float32")
         return out
+
+    def _library_product(self, x, w, out):
+        """out = x w^T by the library (bfloat16): hipBLASLt called directly where it has a
+        kernel for the sizes, torch's call of the libraries otherwise."""
+        if self.use_blaslt and x.stride(1) == 1 and out.stride(1) == 1:
+            if self._blaslt is None:
+                from .blaslt import BlasLt
+                self._blaslt = BlasLt(self.device)
+            if self._blaslt.matmul(x, w, out, _raw_stream(self._device_index)):
+                return
+        torch.mm(x, w.t(), out=out)
 
     # ------------------------------------------------------------------ short convolution
     def short_conv(self, bcx, weight, bias, state, out, batch):

@@ -118,6 +118,46 @@ def test_linear_bf16_and_stored_f32_matrix(ops):
     torch.testing.assert_close(out32.double().cpu(), ref, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 331, 96), (77, 130, 96), (300, 1000, 352), (129, 48, 40),
+                                   (512, 2048, 1024), (2041, 272, 4608)])
+def test_library_product_called_directly(ops, M, N, K):
+    """The bfloat16 products of many rows go to hipBLASLt directly; where it has a kernel
+    the result is what torch's call of the libraries gives, with rows of x that are not
+    dense and with a 32-bit output too, and a recorded call replays to the same bits."""
+    big = randn(M, K + 8, seed=20, dtype=torch.bfloat16)
+    x = big[:, :K]                                     # rows K + 8 apart
+    w = randn(N, K, seed=21, scale=0.1, dtype=torch.bfloat16)
+    ref = x.double().cpu() @ w.double().cpu().T
+    outs = {}
+    for direct in (True, False):
+        ops.use_blaslt = direct
+        try:
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            ops.linear(x, w, out)
+            out32 = torch.empty(M, N, device=DEV)
+            ops.linear(x, w, out32)
+            outs[direct] = (out, out32)
+        finally:
+            ops.use_blaslt = True
+    bound = 1.6e-2 * max(1.0, float(ref.abs().max()))
+    for out, out32 in outs.values():
+        assert float((out.double().cpu() - ref).abs().max()) <= bound
+        assert torch.equal(out32, out.float())
+    assert float((outs[True][0].float() - outs[False][0].float()).abs().max()) <= bound
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, w, out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.linear(x, w, out)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, outs[True][0])
+
+
 # ---------------------------------------------------------------- cache-backed kernels
 def make_cache(kv_heads, head_dim, n_layers, dtype, n_pages=64, page_tokens=16, slots=4,
                states=(), max_context=512):
