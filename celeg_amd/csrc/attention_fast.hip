@@ -690,13 +690,12 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     }
 }
 
-template <int HD>
+template <int HD, int WAVES>
 static int launch_decode_heads(const void* q, int ldq, const void* k_pool, const void* v_pool,
                                const int* table, int table_stride, const int* token_slot,
                                const int* positions, void* out, int ldo, int n_rows, int kv_heads,
                                int group, int page_tokens, int page_shift, int n_layers, int layer,
                                float scale, int window, hipStream_t stream) {
-    constexpr int WAVES = HD <= 64 ? 16 : 8;   // what the registers of a CU hold of this head size
     const int chunks = (group + 15) / 16;
     const size_t lds = static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
     static bool raised = false;
@@ -759,12 +758,19 @@ extern "C" int celeg_attention_decode_bf16(
     // and 64 requests, a workgroup per round 2 to 5 % faster at 1 to 8).
     if (whole < 0) whole = kv_heads * chunks * n_rows >= 192 ? 1 : 0;
     if (whole) {
+        // 16 wavefronts a workgroup (what the registers of a compute unit hold at this head size),
+        // 8 once there are two workgroups and more for every compute unit: their ends overlap
+        // (64 requests x 8 heads: 4 to 6 % faster at contexts of 1,000 to 4,000; equal at 32 requests)
+        if (head_dim == 64 && kv_heads * chunks * n_rows >= 512)
+            return launch_decode_heads<64, 8>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
+                                              out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
+                                              n_layers, layer, scale, window, stream);
         if (head_dim == 64)
-            return launch_decode_heads<64>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
+            return launch_decode_heads<64, 16>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
                                            out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
                                            n_layers, layer, scale, window, stream);
         if (head_dim == 128)
-            return launch_decode_heads<128>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
+            return launch_decode_heads<128, 8>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
                                             out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
                                             n_layers, layer, scale, window, stream);
         return static_cast<int>(hipErrorInvalidValue);

@@ -283,7 +283,7 @@ def attention_case(ops, dtype, heads, kv_heads, head_dim, lengths, cuts, window=
     total = sum(lengths)
     cache = make_cache(kv_heads, head_dim, n_layers, dtype, page_tokens=page_tokens,
                        n_pages=(total + page_tokens * len(lengths)) // page_tokens + 2,
-                       max_context=max(lengths) + 16)
+                       max_context=max(lengths) + 16, slots=max(4, len(lengths) + 1))
     kv = cache.layer_cache(layer).kv
     qw = 1 + randn(head_dim, seed=20, scale=0.1) if qk_norm else None
     kw = 1 + randn(head_dim, seed=21, scale=0.1) if qk_norm else None
@@ -430,6 +430,13 @@ def test_attention_rows_tiles_and_forms(ops, rows_per_tile, form, heads, kv_head
     finally:
         ops.attention_rows_per_tile = 0
         ops.attention_rows_form = 0
+
+
+def test_attention_decode_of_many_requests_and_heads(ops):
+    """33 requests x 16 key/value heads decoding together: enough workgroups for the form
+    with 8 wavefronts a workgroup (more rounds of keys than wavefronts; a boosted far key)."""
+    attention_case(ops, torch.bfloat16, 32, 16, 64, lengths=[600 + 7 * i for i in range(33)],
+                   cuts=[590] + [1] * 40, boost=(5, 598))
 
 
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [
