@@ -138,6 +138,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--gemm-backend", choices=["library", "tiles"], default="library",
+                    help="products of steps of more than 64 rows (the prefill)")
     ap.add_argument("--batch", type=int, default=BATCH,
                     help="for profiling with --phase decode: another batch size than the headline's 8")
     ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve"], default="all",
@@ -176,7 +178,8 @@ def main() -> int:
         pages_per_request = (need + 15) // 16 + 1
         lm = load_model(folder, dtype="bfloat16", device="cuda:0", page_tokens=16,
                         n_pages=pages_per_request * max_batch, max_requests=max_batch,
-                        max_context=context, max_batched_tokens=PROMPT_TOKENS)
+                        max_context=context, max_batched_tokens=PROMPT_TOKENS,
+                        gemm_backend=args.gemm_backend)
     ff = lm.config.ff_dim
     w_bytes = weight_bytes(lm.model)
     kv_per_token = lm.cache.layout.kv_bytes_per_token(2)

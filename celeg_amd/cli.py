@@ -63,6 +63,9 @@ def build_parser() -> argparse.ArgumentParser:
                     help="cache storage (quantized caches are not built)")
     ap.add_argument("--no-cuda-graph", "--no-graph", dest="no_graph", action="store_true",
                     help="do not replay decode steps from a captured graph")
+    ap.add_argument("--gemm-backend", default="library", choices=["library", "tiles"],
+                    help="bfloat16 steps of more than 64 rows: the library's matrix products, or this "
+                         "package's tiled products with norm, SwiGLU and residual sum folded in")
     ap.add_argument("--device", default="cuda:0")
     return ap
 
@@ -165,7 +168,7 @@ def run(args) -> int:
     pages_per_request = (context + args.page_tokens - 1) // args.page_tokens
     lm = load_model(model_dir, dtype=args.dtype, device=args.device, page_tokens=args.page_tokens,
                     n_pages=args.pages or pages_per_request * batch, max_requests=max(batch, 1),
-                    max_context=context, max_batched_tokens=budget)
+                    max_context=context, max_batched_tokens=budget, gemm_backend=args.gemm_backend)
     lm.runner.use_graphs = not args.no_graph
     if args.memory_report:
         weights = sum(t.numel() * t.element_size() for t in _weight_tensors(lm.model))

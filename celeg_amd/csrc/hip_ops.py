@@ -70,6 +70,8 @@ class HipOps:
         # rows it equals the k-sliced kernels on 1,024-wide layers and is 20 % faster on 2,048-wide
         # ones (1.55 against 1.94 ms at the 2.6B shape); at 8 rows it loses 19 % on the former
         self.rows_kernel_min_rows = 9
+        self.use_tiles = True              # fused bfloat16 products of many rows (gemm_tiles.hip)
+        self.tiles_min_rows = 65
         self.last_stat_blocks = 0
         self.fused_linear_shape = 0        # 0: chosen from the sizes; 1..4 force a workgroup shape
 
@@ -84,6 +86,8 @@ class HipOps:
                 raise KernelError(f"cannot load the built kernels {path}: {err}") from err
             if module == "gemv_slices" and lib.celeg_gemv_params_size() != ctypes.sizeof(_GemvParams):
                 raise KernelError("the argument block of the skinny products does not match the built kernels")
+            if module == "gemm_tiles" and lib.celeg_gemm_tiles_params_size() != ctypes.sizeof(_TileParams):
+                raise KernelError("the argument block of the tiled products does not match the built kernels")
             self._libs[module] = lib
             self.loaded_libraries[module] = path
         return lib
@@ -723,6 +727,98 @@ class HipOps:
             _c_int(self._EPILOGUES[epilogue]), _c_int(self.fused_linear_shape), self._stream())
         self._check(code, f"fused_linear ({epilogue})")
         return out
+
+    # ------------------------------------------------------------------ fused products of many rows
+    def tiled_linear_ok(self, rows: int, n: int, *inner_sizes: int) -> bool:
+        """Whether the fused bfloat16 product for many rows takes these sizes."""
+        return self.use_tiles and rows >= self.tiles_min_rows and n % 4 == 0 \
+            and all(k > 0 and k % 64 == 0 for k in inner_sizes)
+
+    def tiled_stat_blocks(self, rows: int, n: int, k: int) -> int:
+        """Partial sums of squares per row that the "residual" epilogue of ``tiled_linear``
+        leaves for these sizes."""
+        return int(self._lib("gemm_tiles").celeg_gemm_tiles_blocks(_c_int(rows), _c_int(n), _c_int(k)))
+
+    def tiled_linear(self, a, w, out, *, epilogue="store", eps=0.0, stats=None, stat_blocks=0,
+                     bias=None, stats_out=None, out_bf16=None):
+        """out = epilogue(scale * (a w^T) + bias) for many bfloat16 rows (any number; made for
+        more than 64), inner size a multiple of 64, columns a multiple of 4.
+
+        ``a`` [M, K] bfloat16 with dense rows.  With ``stat_blocks`` > 0, ``a`` is the bfloat16
+        copy of the residual stream behind a norm whose weight the caller has folded into
+        ``w``, and ``stats[row, :stat_blocks]`` are partial sums of squares of its rows, from
+        which the rows' 1/rms (with ``eps``) scales the sums.  Epilogues: "store" (bfloat16
+        [M, N]), "residual" (``out`` is the 32-bit stream, added to in place; ``out_bf16``
+        receives its bfloat16 copy and ``stats_out`` [>= M, ``tiled_stat_blocks``] the partial
+        sums of squares of the new rows; ``last_stat_blocks`` says how many a row), "swiglu"
+        (``w`` is [2N, K]: gate rows then up rows)."""
+        if epilogue not in ("store", "residual", "swiglu"):
+            raise KernelError(f"tiled_linear: unknown epilogue '{epilogue}'")
+        self._dev(a, "a", torch.bfloat16, contiguous=False); self._dev(w, "w", torch.bfloat16)
+        streams = 2 if epilogue == "swiglu" else 1
+        if a.dim() != 2 or w.dim() != 2:
+            raise KernelError("tiled_linear: a and w must be 2-D")
+        M, K = a.shape
+        if w.shape[1] != K or w.shape[0] % streams:
+            raise KernelError(f"tiled_linear: a {tuple(a.shape)} and w {tuple(w.shape)} do not fit")
+        N = w.shape[0] // streams
+        if K % 64 or N % 4:
+            raise KernelError(f"tiled_linear: inner size {K} must be a multiple of 64 and {N} columns "
+                              "a multiple of 4")
+        lda = self._rows(a, "a")
+        out_dtype = torch.float32 if epilogue == "residual" else torch.bfloat16
+        self._dev(out, "out", out_dtype, contiguous=False)
+        ldo = self._rows(out, "out")
+        if out.shape != (M, N) or lda % 8 or ldo % 4 or a.data_ptr() % 16 or w.data_ptr() % 16 \
+                or out.data_ptr() % 16:
+            raise KernelError(f"tiled_linear: out must be [{M}, {N}] and the rows aligned")
+        prm = _TileParams()
+        prm.a, prm.lda, prm.w, prm.ldw, prm.stream_rows = a.data_ptr(), lda, w.data_ptr(), K, N
+        if bias is not None:
+            self._dev(bias, "bias", torch.float32)
+            if bias.numel() != streams * N:
+                raise KernelError("tiled_linear: bias does not fit")
+            prm.bias = bias.data_ptr()
+        if stat_blocks > 0:
+            self._dev(stats, "stats", torch.float32)
+            if stats.dim() != 2 or stats.shape[0] < M or stats.shape[1] < stat_blocks or stats.stride(1) != 1:
+                raise KernelError("tiled_linear: stats must be [>= rows, >= stat_blocks]")
+            prm.stats, prm.n_stat_blocks, prm.stats_ld = stats.data_ptr(), stat_blocks, stats.stride(0)
+        prm.eps = eps
+        prm.M, prm.N, prm.K = M, N, K
+        prm.out, prm.ldo = out.data_ptr(), ldo
+        if epilogue == "residual":
+            self.last_stat_blocks = self.tiled_stat_blocks(M, N, K)
+            if out_bf16 is not None:
+                self._dev(out_bf16, "out_bf16", torch.bfloat16, contiguous=False)
+                ldb = self._rows(out_bf16, "out_bf16")
+                if out_bf16.shape != (M, N) or ldb % 4 or out_bf16.data_ptr() % 8:
+                    raise KernelError("tiled_linear: out_bf16 does not fit")
+                prm.out_bf16, prm.ld_bf16 = out_bf16.data_ptr(), ldb
+            if stats_out is not None:
+                self._dev(stats_out, "stats_out", torch.float32)
+                if stats_out.dim() != 2 or stats_out.shape[0] < M or stats_out.shape[1] < self.last_stat_blocks \
+                        or stats_out.stride(1) != 1:
+                    raise KernelError(f"tiled_linear: stats_out must be [>= rows, >= {self.last_stat_blocks}]")
+                prm.stats_out, prm.stats_ld_out = stats_out.data_ptr(), stats_out.stride(0)
+        elif out_bf16 is not None or stats_out is not None:
+            raise KernelError("tiled_linear: out_bf16 and stats_out go with the residual epilogue")
+        code = self._lib("gemm_tiles").celeg_gemm_tiles(
+            ctypes.byref(prm), _c_int(self._EPILOGUES[epilogue]), self._stream())
+        self._check(code, f"tiled_linear ({epilogue})")
+        return out
+
+
+class _TileParams(ctypes.Structure):
+    """Mirror of ``TileParams`` in gemm_tiles.hip (its size is checked when the library loads)."""
+    _fields_ = [
+        ("a", ctypes.c_void_p), ("lda", ctypes.c_int), ("w", ctypes.c_void_p), ("ldw", ctypes.c_int),
+        ("stream_rows", ctypes.c_int), ("bias", ctypes.c_void_p), ("stats", ctypes.c_void_p),
+        ("n_stat_blocks", ctypes.c_int), ("stats_ld", ctypes.c_int), ("eps", ctypes.c_float),
+        ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
+        ("out", ctypes.c_void_p), ("ldo", ctypes.c_int), ("out_bf16", ctypes.c_void_p),
+        ("ld_bf16", ctypes.c_int), ("stats_out", ctypes.c_void_p), ("stats_ld_out", ctypes.c_int),
+    ]
 
 
 class _GemvParams(ctypes.Structure):

@@ -54,10 +54,15 @@ def make_runtime(device, dtype, ops=None) -> Runtime:
 def load_model(model_dir: str, *, dtype="bfloat16", device="cuda:0", page_tokens: int = 16,
                n_pages: Optional[int] = None, max_requests: int = 8,
                max_context: Optional[int] = None, max_batched_tokens: int = 2048,
-               ops=None) -> LoadedModel:
+               ops=None, gemm_backend: str = "library") -> LoadedModel:
     """``n_pages``: pages of the cache pool (per group); by default enough for
     ``max_requests`` requests of ``max_context`` tokens.  ``max_context`` defaults to the
-    model's own maximum and may not exceed it."""
+    model's own maximum and may not exceed it.  ``gemm_backend``: how bfloat16 steps of more
+    than 64 rows multiply: "library" (hipBLASLt, with separate norm and activation kernels)
+    or "tiles" (this package's tiled products with the norm, SwiGLU and the residual sum
+    folded in, where the sizes allow; the library otherwise)."""
+    if gemm_backend not in ("library", "tiles"):
+        raise ValueError(f"gemm_backend must be 'library' or 'tiles', not '{gemm_backend}'")
     dtype = parse_dtype(dtype)
     cfg_dict = read_config_file(model_dir)
     config, spec = spec_from_config(cfg_dict)
@@ -67,6 +72,7 @@ def load_model(model_dir: str, *, dtype="bfloat16", device="cuda:0", page_tokens
         raise ValueError(f"--context {max_context} exceeds model maximum {spec.max_context}")
     model = Model(spec)
     rt = make_runtime(device, dtype, ops)
+    rt.use_tiled_products = gemm_backend == "tiles"
     ckpt = Checkpoint(model_dir)
     try:
         tensors = load_tensors(ckpt, model.expected_tensors(), dtype, device)

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from .base import Embedding, Head, WeightSpec, register_part
-from .fused import _sliced, fused_rows_ok, norm_linear, stream_bf16, stream_stats
+from .fused import _sliced, fused_rows_ok, norm_linear, stream_bf16, stream_stats, tiled_step
 from .norm import RmsNorm
 
 
@@ -34,10 +34,10 @@ class TokenEmbedding(Embedding):
                 and fused_rows_ok(rt, batch, self.width):
             # few rows: leave every row's sum of squares (and the bfloat16 copy of the
             # stream) for the first norm
-            if _sliced(rt, out.shape[0], self.width):
+            if _sliced(rt, out.shape[0], self.width) or tiled_step(rt, out.shape[0]):
                 rt.ops.embed_stream(self.table, token_ids, out,
                                     stream_bf16(rt, out.shape[0], self.width),
-                                    stream_stats(rt, self.width))
+                                    stream_stats(rt, self.width, out.shape[0]))
                 rt.stream_has_bf16 = True
             else:
                 rt.ops.embed_stats(self.table, token_ids, out, stream_stats(rt, self.width))
@@ -91,7 +91,8 @@ def _head_fused(h, norm, batch, out, rt, weight) -> bool:
     """Final norm and output product in one kernel for few wanted rows, 32-bit logits."""
     R = batch.n_logit_rows
     if not (isinstance(norm, RmsNorm) and weight.dtype == torch.bfloat16
-            and fused_rows_ok(rt, batch, h.shape[1]) and 0 < R <= 64):
+            and fused_rows_ok(rt, batch, h.shape[1]) and 0 < R <= 64
+            and not tiled_step(rt, batch.n_tokens)):
         return False
     norm_linear(rt, h, norm, weight, out, epilogue="store_f32", rows=batch.logit_rows, n_rows=R)
     return True

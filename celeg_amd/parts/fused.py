@@ -22,11 +22,27 @@ FUSED_MAX_ROWS = 64
 FUSED_MAX_ROWS_OLD_KERNEL = 32
 
 
+TILED_MAX_STAT_BLOCKS = 128   # partial sums of squares a row of a step of many rows may come with
+
+
+def tiled_step(rt, rows: int) -> bool:
+    """Whether a step of ``rows`` rows is one of many rows that takes the fused path through
+    the tiled products (``rt.use_tiled_products``; otherwise steps of many rows run the
+    library's products with separate norm and activation kernels)."""
+    return rows > FUSED_MAX_ROWS and getattr(rt, "use_tiled_products", False) \
+        and rt.dtype == torch.bfloat16 and getattr(rt, "use_fused", True) \
+        and hasattr(rt.ops, "tiled_linear_ok")
+
+
 def fused_rows_ok(rt, batch, *inner_sizes) -> bool:
     """Whether this step's rows can take the fused path through products with these
     inner sizes."""
     ops = rt.ops
     rows = batch.n_tokens
+    if rows > FUSED_MAX_ROWS:
+        # every inner size is also the width of some product's output
+        return tiled_step(rt, rows) and ops.tiled_linear_ok(rows, 4, *inner_sizes) \
+            and max(inner_sizes) <= 64 * TILED_MAX_STAT_BLOCKS
     if not (rt.dtype == torch.bfloat16 and getattr(ops, "has_fused_linear", False)
             and getattr(rt, "use_fused", True) and ops.fused_linear_ok(rows, *inner_sizes)):
         return False
@@ -42,7 +58,9 @@ SLICED_MAX_STAT_BLOCKS = 512   # partial sums of squares a row may come with
 SLICED_MAX_COLUMNS = 16384   # wider products (the output head) keep their rows in LDS instead
 
 
-def stream_stats(rt, width: int) -> torch.Tensor:
+def stream_stats(rt, width: int, rows: int = 0) -> torch.Tensor:
+    if rows > STAT_COLUMNS:       # a step of many rows: one partial sum per tile of columns
+        return rt.ws.buf("stream_stats_many", (rows, TILED_MAX_STAT_BLOCKS), torch.float32)
     # up to one partial sum per 4 columns (the products for few rows use narrow workgroups)
     return rt.ws.buf("stream_stats", (STAT_COLUMNS, (width + 3) // 4), torch.float32)
 
@@ -60,6 +78,8 @@ def operand_rows(rt, name: str, rows: int, width: int, *producer_inner: int) -> 
     """Room for a bfloat16 operand of the fused products, [rows, width] (up to 16 rows, or
     sizes the kernel for 9 to 64 rows does not take) or the view [rows, width/8, 8] of
     [width/8, 64, 8]."""
+    if rows > STAT_COLUMNS:
+        return rt.ws.buf(name + "_many", (rows, width), torch.bfloat16)
     if _side_by_side(rt, rows, width, *producer_inner):
         return rt.ws.buf(name + "_side_by_side", (width // 8, STAT_COLUMNS, 8), torch.bfloat16).permute(1, 0, 2)[:rows]
     return rt.ws.buf(name, (STAT_COLUMNS, width), torch.bfloat16)[:rows]
@@ -95,6 +115,17 @@ def folded_weight(rt, w: torch.Tensor, norm_weight: torch.Tensor) -> torch.Tenso
     return hit
 
 
+def folded_plain_weight(rt, w: torch.Tensor, norm_weight: torch.Tensor) -> torch.Tensor:
+    """``w`` with the norm's weight multiplied into its columns, rows one after the other (what
+    the tiled products read).  Made once per (weight, norm) pair and kept."""
+    cache = rt.__dict__.setdefault("folded_plain_weights", {})
+    key = (w.data_ptr(), norm_weight.data_ptr())
+    hit = cache.get(key)
+    if hit is None:
+        hit = cache[key] = (w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype).contiguous()
+    return hit
+
+
 def packed_weight(rt, w: torch.Tensor) -> torch.Tensor:
     """A copy of ``w`` in the layout the products for few rows read best; made once."""
     cache = rt.__dict__.setdefault("packed_weights", {})
@@ -108,6 +139,17 @@ def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None
     """out = epilogue(norm(h) w^T), the norm applied while the rows of ``h`` are read."""
     blocks = getattr(rt, "stream_stat_blocks", 0)
     M = n_rows if n_rows is not None else (rows.numel() if rows is not None else h.shape[0])
+    if tiled_step(rt, h.shape[0]):
+        if rows is not None or epilogue not in ("store", "swiglu") or w.dtype != torch.bfloat16:
+            raise RuntimeError("norm_linear: not a product of the path for many rows")
+        stats = stream_stats(rt, h.shape[1], h.shape[0])
+        xb = stream_bf16(rt, h.shape[0], h.shape[1])
+        if not (0 < blocks <= TILED_MAX_STAT_BLOCKS and getattr(rt, "stream_has_bf16", False)):
+            rt.ops.stream_prepare(h, xb, stats)
+            rt.stream_stat_blocks = blocks = 1
+            rt.stream_has_bf16 = True
+        return rt.ops.tiled_linear(xb, folded_plain_weight(rt, w, norm.weight), out, epilogue=epilogue,
+                                   eps=norm.eps, stats=stats, stat_blocks=blocks, bias=kw.get("bias"))
     streams = {"swiglu": 2, "conv": 3}.get(epilogue, 1)
     streamed = hasattr(rt.ops, "rows_kernel_ok") and rt.ops.rows_kernel_ok(M, h.shape[1])
     if _sliced(rt, M, h.shape[1]) and w.dtype == torch.bfloat16 \
@@ -137,6 +179,13 @@ def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None
 def linear_into_stream(rt, a, w, h, bias=None):
     """h += a w^T, leaving the partial sums of squares of the new rows (and, for few rows,
     the stream's bfloat16 copy)."""
+    if tiled_step(rt, h.shape[0]):
+        stats = stream_stats(rt, h.shape[1], h.shape[0])
+        rt.ops.tiled_linear(a, w, h, epilogue="residual", bias=bias, stats_out=stats,
+                            out_bf16=stream_bf16(rt, h.shape[0], h.shape[1]))
+        rt.stream_stat_blocks = rt.ops.last_stat_blocks
+        rt.stream_has_bf16 = True
+        return h
     stats = stream_stats(rt, h.shape[1])
     inner = a.shape[1] * (8 if a.dim() == 3 else 1)
     sliced = _sliced(rt, h.shape[0], inner)

@@ -21,7 +21,7 @@ from __future__ import annotations
 import torch
 
 from .base import Mixer, StateNeed, WeightSpec, register_part
-from .fused import fused_rows_ok, linear_into_stream, norm_linear, operand_rows
+from .fused import fused_rows_ok, linear_into_stream, norm_linear, operand_rows, tiled_step
 
 
 class ShortConv(Mixer):
@@ -79,7 +79,7 @@ class ShortConv(Mixer):
         if not fused_rows_ok(rt, batch, H) or (self.w_in.dtype, self.w_out.dtype) != (rt.dtype,) * 2:
             return False
         T = batch.n_tokens
-        if batch.decode_only and batch.n_seqs == T and self.taps <= 8:   # the fused form holds 8 taps
+        if batch.decode_only and batch.n_seqs == T and self.taps <= 8 and not tiled_step(rt, T):   # the fused form holds 8 taps
             y = operand_rows(rt, "conv_y_fused", T, H, H)
             norm_linear(rt, h, norm, self.w_in, y, epilogue="conv", bias=self.b_in,
                         conv=(self.w_conv, self.b_conv, cache.states["bx"], batch.seq_slot))

@@ -60,7 +60,19 @@ TINY_D = {
     "tie_word_embeddings": False, "norm_eps": 2e-5, "max_position_embeddings": 512,
     "bos_token_id": 0, "eos_token_id": 4, "pad_token_id": 1,
 }
-TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3)}
+# A fifth one whose inner sizes are all multiples of 64 (what the tiled products for steps of
+# many rows take): width 128, 2 query heads of 64, feed-forward 192.
+TINY_E = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "vocab_size": 300, "hidden_size": 128, "num_hidden_layers": 4,
+    "layer_types": ["conv", "full_attention", "conv", "full_attention"],
+    "num_attention_heads": 2, "num_key_value_heads": 1, "head_dim": 64,
+    "intermediate_size": 192, "block_auto_adjust_ff_dim": False,
+    "rope_theta": 20000.0, "conv_L_cache": 3, "conv_bias": True,
+    "tie_word_embeddings": True, "norm_eps": 1e-5, "max_position_embeddings": 512,
+    "bos_token_id": 0, "eos_token_id": 6, "pad_token_id": 1,
+}
+TINY = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2), "D": (TINY_D, 3), "E": (TINY_E, 4)}
 
 
 @pytest.fixture(scope="session")

@@ -14,7 +14,8 @@ from helpers import (WEIGHT_STD, EngineDriver, assert_close, mixed_schedule, pea
                      portions_schedule, random_tokens, tail_decode_schedule, whole_schedule)
 
 LENGTHS = {"A": [40, 57, 90, 128, 65, 33], "B": [45, 200, 64, 100, 256, 33],
-           "C": [70, 33, 150, 97, 48, 260], "D": [300, 66, 129, 40, 210, 77]}
+           "C": [70, 33, 150, 97, 48, 260], "D": [300, 66, 129, 40, 210, 77],
+           "E": [300, 150, 97, 260, 70, 200]}
 SCHEDULES = {"whole": whole_schedule, "tail32": tail_decode_schedule,
              "portions": portions_schedule, "mixed": mixed_schedule}
 
@@ -36,7 +37,7 @@ def plain_logits(folder, name, storage):
     return _plain_cache[key]
 
 
-def run_mode(model_folders, name, dtype, mode, device, ops=None, subset=None):
+def run_mode(model_folders, name, dtype, mode, device, ops=None, subset=None, gemm_backend="library"):
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders(name, storage, WEIGHT_STD)
@@ -47,13 +48,14 @@ def run_mode(model_folders, name, dtype, mode, device, ops=None, subset=None):
     max_tokens = peak_tokens(steps)
     lm = load_model(folder, dtype=dtype, device=device, page_tokens=16,
                     n_pages=max_tokens // 16, max_requests=4,
-                    max_batched_tokens=max(max_tokens, 64), ops=ops)
+                    max_batched_tokens=max(max_tokens, 64), ops=ops, gemm_backend=gemm_backend)
     got = EngineDriver(lm).run(steps)
     ref = plain_logits(folder, name, storage)
     for rid in reqs:
         assert_close(got[rid], ref[rid], dtype, f"{name}/{dtype}/{mode}/{rid}")
     lm.cache.check()
     assert lm.cache.n_free_slots == 4 and lm.cache.free_pages() == [max_tokens // 16]
+    return lm
 
 
 @pytest.mark.gpu
@@ -62,6 +64,19 @@ def run_mode(model_folders, name, dtype, mode, device, ops=None, subset=None):
 @pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_gpu_engine_matches_plain(model_folders, name, dtype, mode):
     run_mode(model_folders, name, dtype, mode, "cuda:0")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", list(SCHEDULES))
+def test_gpu_engine_with_tiled_products_matches_plain(model_folders, mode):
+    """Steps of more than 64 rows through the tiled products (norm, SwiGLU and residual sum
+    folded in) instead of the library's: whole prompts of up to 300 tokens, and portions
+    beside single tokens."""
+    lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles")
+    if mode in ("whole", "tail32"):
+        assert "gemm_tiles" in lm.rt.ops.loaded_libraries
+    # and the same configuration through the library's products
+    run_mode(model_folders, "E", "bfloat16", mode, "cuda:0")
 
 
 @pytest.mark.parametrize("mode", list(SCHEDULES))

@@ -1,0 +1,134 @@
+"""The fused bfloat16 products for many rows (gemm_tiles.hip) alone, against torch: every
+epilogue, every tile shape, at sizes that are no multiple of the tiles."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF = torch.bfloat16
+N_SHAPES = 10
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from celeg_amd.csrc.hip_ops import HipOps
+    ops = HipOps(DEV)
+    yield ops
+    ops._lib("gemm_tiles").celeg_gemm_tiles_force(-1)
+
+
+def randn(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def product(a, w, scale=None, bias=None):
+    y = a.double() @ w.double().T
+    if scale is not None:
+        y = y * scale.double()[:, None]
+    if bias is not None:
+        y = y + bias.double()
+    return y
+
+
+def bf16_round(x):
+    return x.to(torch.float32).to(BF).double()
+
+
+SIZES = [(300, 200, 128), (65, 36, 64), (512, 256, 192), (129, 1024, 1024)]
+
+
+@pytest.mark.parametrize("shape", list(range(N_SHAPES)) + [-1])
+@pytest.mark.parametrize("M,N,K", SIZES)
+def test_store_with_row_scale_and_bias(ops, shape, M, N, K):
+    ops._lib("gemm_tiles").celeg_gemm_tiles_force(shape)
+    a = randn(M, K, seed=1, dtype=BF)
+    w = randn(N, K, seed=2, scale=0.05, dtype=BF)
+    bias = randn(N, seed=3) if shape % 2 else None
+    eps, blocks = 1e-5, 11                       # more partial sums than one round of loads
+    g = torch.Generator().manual_seed(4)
+    stats = (torch.rand(M, blocks + 2, generator=g) * K / blocks).to(DEV)
+    scale = 1.0 / torch.sqrt(stats[:, :blocks].sum(1) / K + eps)
+    out = torch.zeros(M + 1, N, dtype=BF, device=DEV)
+    ops.tiled_linear(a, w, out[:M], bias=bias, stats=stats, stat_blocks=blocks, eps=eps)
+    ref = product(a, w, scale, bias)
+    assert float((out[:M].double() - ref).abs().max()) <= 2 ** -7 * float(ref.abs().max())
+    assert float(out[M].abs().max()) == 0        # nothing behind the last row is written
+    # without statistics the sums are stored as they are
+    ops.tiled_linear(a, w, out[:M], bias=bias)
+    ref = product(a, w, None, bias)
+    assert float((out[:M].double() - ref).abs().max()) <= 2 ** -7 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("shape", list(range(N_SHAPES)) + [-1])
+@pytest.mark.parametrize("M,ff,K", SIZES)
+def test_swiglu(ops, shape, M, ff, K):
+    ops._lib("gemm_tiles").celeg_gemm_tiles_force(shape)
+    a = randn(M, K, seed=5, dtype=BF)
+    w = randn(2 * ff, K, seed=6, scale=0.1, dtype=BF)
+    bias = randn(2 * ff, seed=7, scale=0.1) if shape % 2 else None
+    y = product(a, w, None, bias)
+    gate, up = bf16_round(y[:, :ff]), bf16_round(y[:, ff:])
+    ref = gate / (1 + torch.exp(-gate)) * up
+    out = torch.zeros(M, ff, dtype=BF, device=DEV)
+    ops.tiled_linear(a, w, out, epilogue="swiglu", bias=bias)
+    # a flip of the rounding of gate or up moves the result by one bfloat16 step of it
+    bound = 2 ** -6 * float(ref.abs().max()) + 2 ** -7 * float((up.abs() * (1 + gate.abs())).max())
+    assert float((out.double() - ref).abs().max()) <= bound
+
+
+@pytest.mark.parametrize("shape", list(range(N_SHAPES)) + [-1])
+@pytest.mark.parametrize("M,N,K", SIZES)
+def test_residual_adds_in_place_refreshes_the_copy_and_leaves_partial_sums(ops, shape, M, N, K):
+    ops._lib("gemm_tiles").celeg_gemm_tiles_force(shape)
+    a = randn(M, K, seed=8, dtype=BF)
+    w = randn(N, K, seed=9, scale=0.05, dtype=BF)
+    bias = randn(N, seed=10) if shape % 2 else None
+    h0 = randn(M + 1, N, seed=11)
+    h = h0.clone()
+    blocks = ops.tiled_stat_blocks(M, N, K)
+    copy = torch.zeros(M, N, dtype=BF, device=DEV)
+    sums = torch.zeros(M, blocks + 1, device=DEV)
+    ops.tiled_linear(a, w, h[:M], epilogue="residual", bias=bias, out_bf16=copy, stats_out=sums)
+    assert ops.last_stat_blocks == blocks
+    y = product(a, w, None, bias)
+    ref = h0[:M].double() + bf16_round(y)
+    # the product enters the sum rounded to bfloat16: a flip of that rounding is one step of it
+    assert float((h[:M].double() - ref).abs().max()) <= 2 ** -7 * float(y.abs().max())
+    assert torch.equal(h[M], h0[M])
+    assert torch.equal(copy, h[:M].to(BF))
+    squares = (h[:M].double() ** 2).sum(1)
+    assert float(((sums[:, :blocks].double().sum(1) - squares).abs() / squares).max()) < 1e-5
+    assert float(sums[:, blocks].abs().max()) == 0
+
+
+def test_a_row_does_not_depend_on_the_other_rows(ops):
+    """The same row in a step of 70 rows and in one of 700 gives the same bits where the tile
+    shape is the same (the sums of a row are formed in an order that K alone fixes)."""
+    ops._lib("gemm_tiles").celeg_gemm_tiles_force(7)
+    K, N = 192, 128
+    a = randn(700, K, seed=12, dtype=BF)
+    w = randn(N, K, seed=13, scale=0.05, dtype=BF)
+    big = torch.empty(700, N, dtype=BF, device=DEV)
+    small = torch.empty(70, N, dtype=BF, device=DEV)
+    ops.tiled_linear(a, w, big)
+    ops.tiled_linear(a[330:400], w, small)
+    assert torch.equal(big[330:400], small)
+
+
+def test_unsupported_sizes_are_refused(ops):
+    from celeg_amd.csrc.hip_ops import KernelError
+    ops._lib("gemm_tiles").celeg_gemm_tiles_force(-1)
+    a = randn(80, 96, dtype=BF)
+    with pytest.raises(KernelError):             # inner size no multiple of 64
+        ops.tiled_linear(a, randn(64, 96, dtype=BF), torch.empty(80, 64, dtype=BF, device=DEV))
+    a = randn(80, 128, dtype=BF)
+    with pytest.raises(KernelError):             # columns no multiple of 4
+        ops.tiled_linear(a, randn(66, 128, dtype=BF), torch.empty(80, 66, dtype=BF, device=DEV))
+    with pytest.raises(KernelError):             # a 32-bit output goes with the residual epilogue only
+        ops.tiled_linear(a, randn(64, 128, dtype=BF), torch.empty(80, 64, device=DEV))
+    with pytest.raises(KernelError):
+        ops.tiled_linear(a, randn(64, 128, dtype=BF), torch.empty(80, 64, dtype=BF, device=DEV),
+                         stats_out=torch.empty(80, 4, device=DEV))
+    assert not ops.tiled_linear_ok(80, 64, 96)
+    assert ops.tiled_linear_ok(80, 64, 128, 4608)
