@@ -85,7 +85,7 @@ def prefill_flops(cfg, tokens: int, ff: int) -> float:
     return per_token * tokens + attention + 2.0 * H * cfg["vocab_size"]   # head for one row
 
 
-def serve(shape: str) -> int:
+def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1) -> int:
     """The whole engine on a serving workload: every request submitted at once, the scheduler
     cuts the prompts into portions beside the decoding requests, sampling is greedy on the
     device.  Prints one JSON line: generated tokens a second over the whole run."""
@@ -96,6 +96,7 @@ def serve(shape: str) -> int:
     from celeg_amd.weights import write_random_model
 
     cfg, load = SHAPES[shape]
+    load = dict(load, chunk=chunk or load["chunk"], budget=budget or load["budget"])
     rng = random.Random(0)
     lengths = [rng.randint(*load["prompt"]) for _ in range(load["requests"])]
     prompts = [[rng.randrange(cfg["vocab_size"]) for _ in range(n)] for n in lengths]
@@ -105,12 +106,14 @@ def serve(shape: str) -> int:
         engine = Engine.from_folder(folder, dtype="bfloat16", device="cuda:0", page_tokens=16,
                                     n_pages=pages, max_active_requests=load["requests"],
                                     max_batched_tokens=load["budget"],
-                                    prefill_chunk_tokens=load["chunk"],
+                                    prefill_chunk_tokens=load["chunk"], portion_granule=granule,
                                     context=cfg["max_position_embeddings"])
     # a short run first: kernels loaded, graphs captured for the decode batch sizes
     engine.generate(prompts[:2], max_new_tokens=4, generation=GREEDY, eos_token_ids=[])
     for key in engine.metrics:
         engine.metrics[key] = type(engine.metrics[key])()
+    runner = engine.loaded.runner
+    runner.captures, runner.capture_seconds = 0, 0.0
     torch.cuda.synchronize()
     start = time.perf_counter()
     out = engine.generate(prompts, max_new_tokens=load["new_tokens"], generation=GREEDY, eos_token_ids=[])
@@ -125,8 +128,9 @@ def serve(shape: str) -> int:
         "all_tokens_per_second": round((generated + sum(lengths)) / seconds, 1),
         "requests": load["requests"], "prompt_lengths": list(load["prompt"]),
         "new_tokens": load["new_tokens"], "prefill_chunk": load["chunk"],
-        "step_token_budget": load["budget"], "context": cfg["max_position_embeddings"],
+        "step_token_budget": load["budget"], "portion_granule": granule, "context": cfg["max_position_embeddings"],
         "engine_steps": engine.metrics["steps"], "steps_launched_ahead": engine.metrics["steps_ahead"],
+        "graphs_recorded": runner.captures, "recording_seconds": round(runner.capture_seconds, 3),
         "dtype": "bf16", "data": "synthetic"}))
     return 0
 
@@ -142,6 +146,12 @@ def main() -> int:
                     help="products of steps of more than 64 rows (the prefill)")
     ap.add_argument("--batch", type=int, default=BATCH,
                     help="for profiling with --phase decode: another batch size than the headline's 8")
+    ap.add_argument("--prefill-chunk", type=int, default=0,
+                    help="serve phase: most tokens of a prompt in one step (default: the workload's)")
+    ap.add_argument("--portion-granule", type=int, default=1,
+                    help="serve phase: portions cut by the budget keep to multiples of this")
+    ap.add_argument("--token-budget", type=int, default=0,
+                    help="serve phase: most tokens of a step (default: the workload's)")
     ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
                          "decode measurement (the line printed then holds only that part); "
@@ -155,7 +165,7 @@ def main() -> int:
         return 2
 
     if args.phase == "serve":
-        return serve(args.shape)
+        return serve(args.shape, args.prefill_chunk, args.token_budget, args.portion_granule)
 
     import torch
     import celeg_amd  # noqa: F401

@@ -96,30 +96,43 @@ class BatchBuilder:
 
     def build(self, entries: Sequence[StepEntry], updates: Sequence[Sequence[Tuple[int, int, int]]],
               pad_to: Optional[int] = None, null_slot: int = 0,
-              update_caps: Optional[Sequence[int]] = None) -> StepBatch:
+              update_caps: Optional[Sequence[int]] = None,
+              pad_singles_to: Optional[int] = None, last_rows_too: bool = False) -> StepBatch:
         """``pad_to``: for batches of single rows, the fixed number of rows of a captured
         graph; missing rows are filled with the null slot at position 0, and logits are
-        produced for every row (wanted or not), so that the layout is the same every time."""
+        produced for every row (wanted or not), so that the layout is the same every time.
+        ``pad_singles_to``: for batches that hold portions (beside single rows or without),
+        the fixed number of single rows of a captured graph; the missing ones are filled
+        likewise, between the real single rows and the portions, and their logits come
+        behind the wanted ones.  ``last_rows_too``: a portion that wants nothing gets the
+        logits of its last row all the same, behind the wanted ones (a captured graph has a
+        fixed number of logit rows)."""
         seg_lens = [len(e.tokens) for e in entries]
         S_real = len(entries)
         decode_only = all(n == 1 for n in seg_lens)
         if pad_to is not None and (not decode_only or pad_to < S_real):
             raise ValueError("only batches of single rows can be padded, and only upwards")
+        n_single = sum(1 for n in seg_lens if n == 1)
+        if pad_singles_to is not None and (decode_only or pad_to is not None or pad_singles_to < n_single):
+            raise ValueError("pad_singles_to goes with batches that hold portions, and only upwards")
+        n_pad = 0 if pad_singles_to is None else pad_singles_to - n_single
         T_real = S_real if decode_only else int(sum(seg_lens))
-        S = S_real if pad_to is None else pad_to
-        T = T_real if pad_to is None else pad_to
+        S = (S_real if pad_to is None else pad_to) + n_pad
+        T = (T_real if pad_to is None else pad_to) + n_pad
         # Rows are laid out with the entries of a single token first (their order kept), so
         # that kernels made for single rows can take them as one range also beside portions
         # of prompts; logits still come back in the order of the entries.
         order = list(range(S_real)) if decode_only else \
             sorted(range(S_real), key=lambda i: seg_lens[i] != 1)
-        single_rows = S_real if decode_only else sum(1 for n in seg_lens if n == 1)
+        single_rows = S_real if decode_only else n_single
         if pad_to is not None:
             want_rows = list(range(T))
         else:
             first_row = [0] * S_real
             row = 0
             for i in order:
+                if seg_lens[i] != 1 and row == n_single:
+                    row += n_pad                 # the padding rows lie behind the real single rows
                 first_row[i] = row
                 row += seg_lens[i]
             want_rows = []
@@ -128,6 +141,10 @@ class BatchBuilder:
                     if not 0 <= int(w) < n:
                         raise ValueError(f"wanted place {w} is outside the entry's {n} tokens")
                     want_rows.append(first_row[i] + int(w))
+            if last_rows_too:
+                want_rows.extend(first_row[i] + n - 1 for i, (e, n) in enumerate(zip(entries, seg_lens))
+                                 if n != 1 and not e.want)
+            want_rows.extend(range(n_single, n_single + n_pad))
         R = len(want_rows)
         if update_caps is None:
             update_caps = [len(u) for u in updates]
@@ -171,7 +188,20 @@ class BatchBuilder:
         else:
             row = 0
             cu[0] = 0
-            for i, (e, n) in enumerate((entries[j], seg_lens[j]) for j in order):
+            seq = 0
+            for e, n in ((entries[j], seg_lens[j]) for j in order):
+                if n != 1 and n_pad and row == n_single:
+                    token_ids[row:row + n_pad] = 0
+                    positions[row:row + n_pad] = 0
+                    token_seq[row:row + n_pad] = self._iota[seq:seq + n_pad]
+                    token_slot[row:row + n_pad] = null_slot
+                    seq_slot[seq:seq + n_pad] = null_slot
+                    seq_start[seq:seq + n_pad] = 0
+                    cu[seq + 1:seq + n_pad + 1] = self._iota[row + 1:row + n_pad + 1]
+                    row += n_pad
+                    seq += n_pad
+                i = seq
+                seq += 1
                 token_ids[row:row + n] = e.tokens
                 positions[row:row + n] = self._iota[e.start_pos:e.start_pos + n] \
                     if e.start_pos + n <= self._iota.size else np.arange(e.start_pos, e.start_pos + n)
@@ -199,7 +229,7 @@ class BatchBuilder:
         b.max_seg_len = max(seg_lens) if seg_lens else 0
         b.max_context_len = max((e.start_pos + n for e, n in zip(entries, seg_lens)), default=0)
         b.decode_only = decode_only
-        b.single_rows = S if decode_only else single_rows
+        b.single_rows = S if decode_only else single_rows + n_pad
         b.entry_order = order
 
         def dev(name):       # the same views of the device buffer for the same layout
@@ -215,7 +245,10 @@ class BatchBuilder:
         b.logit_rows = dev("logit_rows")
         b.table_updates = [dev(f"updates{g}") for g in range(len(updates))]
         b.table_update_caps = list(update_caps)
-        b.host = {"seg_lens": np.asarray([seg_lens[j] for j in order] + [1] * (S - S_real), dtype=np.int32),
+        host_lens = [seg_lens[j] for j in order]
+        host_lens = host_lens[:n_single] + [1] * n_pad + host_lens[n_single:] if n_pad \
+            else host_lens + [1] * (S - S_real)
+        b.host = {"seg_lens": np.asarray(host_lens, dtype=np.int32),
                   "seq_slot": seq_slot.copy(), "seq_start": seq_start.copy(),
                   "cu_seqlens": cu.copy(), "want_rows": np.asarray(want_rows, dtype=np.int32)}
         return b

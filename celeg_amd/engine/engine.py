@@ -50,13 +50,13 @@ class Engine:
                     max_active_requests: int = 8, max_batched_tokens: int = 512,
                     prefill_chunk_tokens: int = 256, context: Optional[int] = None,
                     policy: str = "max_utilization", ops=None,
-                    gemm_backend: str = "library") -> "Engine":
+                    gemm_backend: str = "library", portion_granule: int = 1) -> "Engine":
         loaded = load_model(model_dir, dtype=dtype, device=device, page_tokens=page_tokens,
                             n_pages=n_pages, max_requests=max_active_requests,
                             max_context=context, max_batched_tokens=max_batched_tokens, ops=ops,
                             gemm_backend=gemm_backend)
         return cls(loaded, SchedulerOptions(max_active_requests, max_batched_tokens,
-                                            prefill_chunk_tokens, policy))
+                                            prefill_chunk_tokens, policy, portion_granule))
 
     # ------------------------------------------------------------------ requests
     def submit(self, prompt: Sequence[int], options: Optional[RequestOptions] = None) -> int:

@@ -12,6 +12,8 @@ from __future__ import annotations
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
+import time
+
 import torch
 
 from ..cache.manager import CacheManager
@@ -68,6 +70,10 @@ class ModelRunner:
         self.use_graphs = True
         self._graphs: Dict[tuple, tuple] = {}
         self._portion_graphs: Dict[tuple, tuple] = {}
+        self._mixed_graphs: Dict[tuple, tuple] = {}
+        self.captures = 0              # recordings made, and the time they took
+        self._weights = None           # number of weights, counted at first need
+        self.capture_seconds = 0.0
         self._portion_seen: Dict[tuple, int] = {}
         self._token_source: Optional[torch.Tensor] = None
         self._buckets = sorted({min(1 << i, S) for i in range(0, 12)})
@@ -120,6 +126,9 @@ class ModelRunner:
         portion = self._portion_shape(entries)
         if portion is not None:
             return self._portion_from_graph(entries, portion)
+        mixed = self._mixed_shape(entries)
+        if mixed is not None:
+            return self._mixed_from_graph(entries, mixed)
         updates = self.cache.drain_table_updates()
         batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
         self._begin_step(batch)
@@ -241,9 +250,100 @@ class ModelRunner:
         self.steps_run += 1
         return captured[1]
 
+    # ------------------------------------------------------------------ captured mixed steps
+    # Under a token budget the steady state of serving is a step of a few portions of prompts
+    # (of the portion size) beside the single tokens of the decoding requests: some 150
+    # launches again, several times the GPU's time for them at small model sizes.  Such steps
+    # are replayed from a graph per (bucket of single rows, sizes of the portions in their
+    # order, bound on the context); single rows are padded to the bucket with null-slot rows,
+    # which lie between the real single rows and the portions.  Recording costs several
+    # steps' time, so the shapes are kept few: coarse buckets (a padding row costs little
+    # beside a portion), and every portion's last row gets logits, wanted or not.
+    MIXED_GRAPHS = 16
+    MIXED_MAX_PORTIONS = 4
+    MIXED_BUCKETS = (4, 16, 64, 256)
+    MIXED_SEEN_BEFORE_RECORDING = 8      # shapes of a passing phase are not worth a recording
+    # A recording costs several steps' time and only pays where the host's launches, not the
+    # GPU, bound the step: where the step's products (two operations per row and weight, at
+    # the rate the library reaches on so few rows) take less time than its launches (some ten
+    # a layer).  Measured at the 350M shape: 480 rows 2.4 ms a step eager, 1.8 replayed;
+    # 2,048 rows are bound by the GPU either way, and so are 544 rows at the 2.6B shape.
+    HOST_SECONDS_PER_LAUNCH = 14e-6
+    LAUNCHES_PER_LAYER = 10
+    FEW_ROWS_FLOPS_PER_SECOND = 400e12
+
+    def _bound_by_launches(self, rows: int) -> bool:
+        if self._weights is None:
+            self._weights = sum(int(np.prod(w.shape)) for w in self.model.expected_tensors().values())
+        gpu = 2.0 * rows * self._weights / self.FEW_ROWS_FLOPS_PER_SECOND
+        host = self.HOST_SECONDS_PER_LAUNCH * self.LAUNCHES_PER_LAYER * len(self.model.spec.order)
+        return gpu < host
+
+    def _mixed_shape(self, entries: Sequence[StepEntry]):
+        if not self.use_graphs or torch.device(self.rt.device).type != "cuda" \
+                or not self.model.graph_safe or len(entries) < 2:
+            return None
+        portions = []
+        n_single = 0
+        for e in entries:
+            n = len(e.tokens)
+            want = list(e.want)
+            if n == 1:
+                if want != [0]:
+                    return None
+                n_single += 1
+            else:
+                if n < self.PORTION_MIN_TOKENS or want not in ([], [n - 1]):
+                    return None
+                portions.append(n)
+        limit = self._buckets[-1]
+        if not portions or len(portions) > self.MIXED_MAX_PORTIONS or n_single > limit \
+                or not self._bound_by_launches(n_single + sum(portions)):
+            return None
+        bucket = next((min(b, limit) for b in self.MIXED_BUCKETS if b >= n_single), limit)
+        shape = (bucket, tuple(portions), self._context_bound(entries))
+        if shape not in self._mixed_graphs:
+            seen = self._portion_seen.get(shape, 0) + 1
+            self._portion_seen[shape] = seen
+            if seen < self.MIXED_SEEN_BEFORE_RECORDING or len(self._mixed_graphs) >= self.MIXED_GRAPHS:
+                return None
+        return shape
+
+    def _mixed_from_graph(self, entries: Sequence[StepEntry], shape) -> torch.Tensor:
+        bucket, portions, bound = shape
+        room = bucket + 8 + sum(n // self.cache.page_tokens + 10 for n in portions)
+        caps = [room] * len(self.cache.groups)
+        captured = self._mixed_graphs.get(shape)
+        if captured is None or captured[2] != self.rt.ws.generation:
+            null = [StepEntry(self.cache.null_slot, 0, [0] * n, [n - 1]) for n in portions]
+
+            def make_batch():
+                batch = self.builder.build(null, [[] for _ in self.cache.groups],
+                                           null_slot=self.cache.null_slot, update_caps=caps,
+                                           pad_singles_to=bucket)
+                batch.context_bound = bound
+                return batch
+            captured = self._capture_batch(make_batch)
+            self._mixed_graphs[shape] = captured
+        updates = self.cache.drain_table_updates()
+        for g, u in enumerate(updates):
+            if len(u) > caps[g]:
+                self._ship_table_updates(g, u)
+                updates[g] = []
+        # every portion's last row gets logits, as in the recording; those nobody wants lie
+        # behind the wanted ones
+        batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot, update_caps=caps,
+                                   pad_singles_to=bucket, last_rows_too=True)
+        self.last_batch = batch
+        captured[0].replay()
+        self.steps_run += 1
+        return captured[1][:sum(len(e.want) for e in entries)]
+
     def _capture_batch(self, make_batch):
         """Warm-up run and capture of the model's forward over the batch ``make_batch()``
         builds (of null-slot rows only): (graph, logits, workspace generation)."""
+        started = time.perf_counter()
+        self.captures += 1
         batch = make_batch()
         self._begin_step(batch)
         self.model.forward(batch, self.rt)          # warm-up: buffers, libraries, heuristics
@@ -256,6 +356,8 @@ class ModelRunner:
                 logits = self.model.forward(batch, self.rt)
         finally:
             self.rt.ws.frozen = False
+        torch.cuda.synchronize(self.rt.device)
+        self.capture_seconds += time.perf_counter() - started
         return (graph, logits, self.rt.ws.generation)
 
     # ------------------------------------------------------------------ tokens from the device
@@ -273,6 +375,7 @@ class ModelRunner:
         if tensor is not self._token_source:
             self._graphs.clear()            # recorded steps do or do not hold the lookup
             self._portion_graphs.clear()
+            self._mixed_graphs.clear()
         self._token_source = tensor
 
     def _resolve_tokens(self, batch: StepBatch) -> None:

@@ -276,6 +276,34 @@ def test_priority_then_age_and_end_tokens_and_poll():
     assert sched2.requests[rid].generated[-1] == eos_tok
 
 
+def test_portions_cut_by_the_budget_keep_to_the_granule():
+    """A portion that the budget cuts short is a multiple of the granule or waits for the next
+    step, so that steps repeat few shapes; the prompt's end and the portion size cut as ever,
+    and a step is never left empty for it."""
+    sched, _ = make_scheduler(n_pages=64, slots=4, prefill_chunk_tokens=64, max_batched_tokens=100,
+                              portion_granule=16)
+    fake = FakeStep()
+    a = sched.submit([1] * 70, opts(3))
+    b = sched.submit([2] * 90, opts(3))
+    plan = sched.plan()
+    assert [(e.request.id, e.count) for e in plan] == [(a, 64), (b, 32)]     # 36 left: cut to 32
+    sched.accept(plan, fake.run(plan))
+    plan = sched.plan()
+    assert [(e.request.id, e.count) for e in plan] == [(a, 6), (b, 58)]      # the ends of both prompts
+    sched.accept(plan, fake.run(plan))
+    drive(sched, fake)
+    assert sched.requests[a].generated == expected_output([1] * 70, 3)
+    assert sched.requests[b].generated == expected_output([2] * 90, 3)
+    # a budget below the granule: the first portion of a step is cut at the budget all the same
+    sched2, _ = make_scheduler(prefill_chunk_tokens=64, max_batched_tokens=10, portion_granule=16)
+    c = sched2.submit([3] * 25, opts(2))
+    plan = sched2.plan()
+    assert [(e.request.id, e.count) for e in plan] == [(c, 10)]
+    sched2.accept(plan, fake.run(plan))
+    drive(sched2, fake)
+    assert sched2.requests[c].generated == expected_output([3] * 25, 2)
+
+
 def test_admission_waits_for_pages_and_slots():
     sched, m = make_scheduler(n_pages=4, slots=2, prefill_chunk_tokens=64, max_batched_tokens=64)
     fake = FakeStep()

@@ -240,6 +240,61 @@ def test_portions_of_a_repeated_size_are_replayed(model_folders, name, dtype):
     lm.cache.check()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_mixed_steps_of_a_repeated_shape_are_replayed(model_folders, name, dtype):
+    """The steady state of serving under a token budget: every step holds portions of prompts
+    of the portion size beside the single tokens of the requests that decode.  From the
+    second step of a shape on (bucket of single rows, sizes of the portions) the step is
+    replayed from a graph captured on null-slot rows; the single rows are padded to the
+    bucket, and the entries come in changing order (a portion first, between or behind the
+    single tokens).  Every wanted row is checked against the plain implementation."""
+    from celeg_amd.engine import load_model
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders(name, storage, WEIGHT_STD)
+    vocab = TINY[name][0]["vocab_size"]
+    P, n_portions, n_decode = 40, 2, 9
+    reqs = {f"m{i}": random_tokens(vocab, P * n_portions + n_decode, seed=1200 + i) for i in range(7)}
+    ids = list(reqs)
+    # request i starts at step stride * i: two steps of a portion, then one token a step
+    # (stride 2: one portion a step; stride 1: two portions of different requests a step)
+    stride = 2 if name == "B" else 1
+    steps, k = [], 0
+    while True:
+        entries, end = [], []
+        for i, rid in enumerate(ids):
+            j = k - stride * i
+            toks = reqs[rid]
+            if 0 <= j < n_portions:
+                entries.append({"id": rid, "tokens": toks[P * j:P * j + P],
+                                "want": [P - 1] if j == n_portions - 1 else []})
+            elif n_portions <= j < n_portions + n_decode:
+                pos = P * n_portions + j - n_portions
+                entries.append({"id": rid, "tokens": [toks[pos]], "want": [0]})
+                if pos == len(toks) - 1:
+                    end.append(rid)
+        if not entries:
+            break
+        entries = entries[k % len(entries):] + entries[:k % len(entries)]     # a changing order
+        steps.append({"step": k, "entries": entries, "end": end})
+        k += 1
+    lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16 + 8,
+                    max_requests=8, max_batched_tokens=128)
+    lm.runner.MIXED_SEEN_BEFORE_RECORDING = 2          # (a server waits for the eighth)
+    got = EngineDriver(lm).run(steps)
+    shapes = set(lm.runner._mixed_graphs)
+    # shapes that came twice were captured (up to 4 single rows; more came once at most), with one or two portions
+    assert len(shapes) >= 1 and all(len(portions) == 3 - stride for _, portions, _ in shapes), shapes
+    assert {bucket for bucket, _, _ in shapes} >= {4}
+    cfgp, W = plain.load_model_folder(folder)
+    first = P * n_portions - 1
+    for rid, toks in reqs.items():
+        ref = plain.model_logits(cfgp, W, toks)
+        assert_close(got[rid], ref[first:], dtype, f"{name}/{dtype}/mixed replay/{rid}")
+    lm.cache.check()
+
+
 def many_requests_schedule(requests, tail, join_every=0):
     """Every request's head in a step of its own, then decode steps that hold ALL requests
     (one token each); with ``join_every`` the heads are spread between the decode steps instead,
