@@ -326,21 +326,23 @@ extern "C" void celeg_gemm_tiles_force_dies(int dies_m) { g_force_dies_m = dies_
     X(6, 128, 128, 2, 2, 4) \
     X(7, 64, 64, 2, 2, 4)   \
     X(8, 64, 64, 2, 2, 2)   \
-    X(9, 128, 64, 2, 2, 2)
+    X(9, 128, 64, 2, 2, 2)  \
+    X(10, 128, 128, 4, 2, 2)
 
-static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128};
-static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64};
-#define N_TILE_SHAPES 10
+static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 128};
+static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128};
+#define N_TILE_SHAPES 11
 
 static TileShape tile_shape(int M, int N, int K, int streams) {
     int id = 0;
     if (g_force_shape >= 0 && g_force_shape < N_TILE_SHAPES) id = g_force_shape;
     else {
         // Measured at 2,048 rows (1,024 to 9,216 weight rows, 1,024 and 4,608 values of k):
-        // tiles of 128x128 with two workgroups a compute unit where they give every unit
-        // one and a half or more, else smaller tiles, which fill the chip.
+        // tiles of 128x128 with two workgroups of 8 wavefronts a compute unit where they give
+        // every unit one and a half or more (8 wavefronts: a tenth faster than 4), else
+        // smaller tiles, which fill the chip.
         const long long wide = static_cast<long long>((M + 127) / 128) * ((static_cast<long long>(N) * streams + 127) / 128);
-        id = wide >= 384 ? 4 : (wide >= 192 ? 3 : 7);
+        id = wide >= 384 ? 10 : (wide >= 192 ? 3 : 7);
     }
     return TileShape{id, k_shape_bm[id], k_shape_bn[id]};
 }

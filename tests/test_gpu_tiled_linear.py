@@ -6,7 +6,7 @@ import torch
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 BF = torch.bfloat16
-N_SHAPES = 10
+N_SHAPES = 11
 
 
 @pytest.fixture(scope="module")
