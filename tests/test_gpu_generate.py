@@ -64,6 +64,29 @@ def test_greedy_generation_through_the_entry_point(model_folders, name, dtype):
         assert alone == outs
 
 
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_generation_through_replayed_mixed_steps(model_folders, name):
+    """A steady load through the entry point: ten requests of equal length under a budget that
+    holds one portion and the decoding requests, a granule for the portions the budget cuts.
+    The steps' shapes repeat and are replayed from recorded graphs, with the tokens of the
+    decoding requests taken on the device (steps launched one ahead); every request's tokens
+    equal the plain implementation's greedy ones."""
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY
+    folder = model_folders(name, torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    vocab = cfg["vocab_size"]
+    prompts = [random_tokens(vocab, 96, seed=300 + i) for i in range(10)]
+    engine = Engine.from_folder(folder, dtype="float32", max_active_requests=4, n_pages=64,
+                                max_batched_tokens=52, prefill_chunk_tokens=48, portion_granule=8)
+    engine.loaded.runner.MIXED_SEEN_BEFORE_RECORDING = 2
+    outs = engine.generate(prompts, max_new_tokens=12, generation=GREEDY, eos_token_ids=[])
+    assert engine.loaded.runner._mixed_graphs, "no step of portions beside single tokens was replayed"
+    for prompt, out in zip(prompts, outs):
+        assert out == plain_generate(cfg, W, prompt, 12)
+    assert engine.loaded.cache.free_pages() == [64] and engine.loaded.cache.n_free_slots == 4
+
+
 def test_sampled_generation_mixed_batch_equals_plain_sampler(model_folders):
     """Tiny B's workload: prompts 1, 9, 64, 100, 200 in portions of 32 beside decoding,
     temperature 0.8, seed 7; every request's tokens equal the plain model + plain sampler,
