@@ -33,6 +33,7 @@
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 
 enum { T_STORE = 0, T_RESIDUAL = 2, T_SWIGLU = 3 };   // the numbers of the few-rows products
 
@@ -261,24 +262,24 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
                     sq[tm] += old[i] * old[i];
                 }
                 *reinterpret_cast<floatx4_t*>(h) = old;
-                if (p.out_bf16) {
-                    bf16 o[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) o[i] = from_float<bf16>(old[i]);
-                    *reinterpret_cast<uint2*>(p.out_bf16 + static_cast<size_t>(m) * p.ld_bf16 + n) = *reinterpret_cast<const uint2*>(o);
-                }
+                if (p.out_bf16)     // (the conversion rounds to nearest even, as from_float<bf16>)
+                    *reinterpret_cast<bf16x4_t*>(p.out_bf16 + static_cast<size_t>(m) * p.ld_bf16 + n) =
+                        bf16x4_t{static_cast<__bf16>(old[0]), static_cast<__bf16>(old[1]),
+                                 static_cast<__bf16>(old[2]), static_cast<__bf16>(old[3])};
             } else {
-                bf16 o[4];
+                float o[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     if (EPI == T_SWIGLU) {
                         const float g = round_bf16(v[0][i]), u = round_bf16(v[NS - 1][i]);
-                        o[i] = from_float<bf16>((g / (1.0f + expf(-g))) * u);
+                        o[i] = (g / (1.0f + expf(-g))) * u;
                     } else {
-                        o[i] = from_float<bf16>(v[0][i]);
+                        o[i] = v[0][i];
                     }
                 }
-                *reinterpret_cast<uint2*>(static_cast<bf16*>(p.out) + static_cast<size_t>(m) * p.ldo + n) = *reinterpret_cast<const uint2*>(o);
+                *reinterpret_cast<bf16x4_t*>(static_cast<bf16*>(p.out) + static_cast<size_t>(m) * p.ldo + n) =
+                    bf16x4_t{static_cast<__bf16>(o[0]), static_cast<__bf16>(o[1]),
+                             static_cast<__bf16>(o[2]), static_cast<__bf16>(o[3])};
             }
         }
     }
@@ -333,7 +334,7 @@ static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 
 static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128};
 #define N_TILE_SHAPES 11
 
-static TileShape tile_shape(int M, int N, int K, int streams) {
+static TileShape tile_shape(int M, int N, int streams) {
     int id = 0;
     if (g_force_shape >= 0 && g_force_shape < N_TILE_SHAPES) id = g_force_shape;
     else {
@@ -380,7 +381,7 @@ static int launch_tiles(const TileParams& p, hipStream_t stream) {
 
 template <int EPI>
 static int launch_epilogue(const TileParams& p, hipStream_t stream) {
-    const TileShape s = tile_shape(p.M, p.N, p.K, TileStreams<EPI>::n);
+    const TileShape s = tile_shape(p.M, p.N, TileStreams<EPI>::n);
 #define TILE_CASE(ID, BM, BN, WGM, WGN, STAGES) \
     if (s.id == ID) return launch_tiles<BM, BN, WGM, WGN, STAGES, EPI>(p, stream);
     TILE_SHAPES(TILE_CASE)
@@ -391,7 +392,8 @@ static int launch_epilogue(const TileParams& p, hipStream_t stream) {
 // Number of partial sums of squares a row gets from the "residual" epilogue for these
 // sizes (one per tile column): the caller sizes stats_out [>= M, >= blocks].
 extern "C" int celeg_gemm_tiles_blocks(int M, int N, int K) {
-    const TileShape s = tile_shape(M, N, K, 1);
+    (void)K;
+    const TileShape s = tile_shape(M, N, 1);
     return (N + s.bn - 1) / s.bn;
 }
 
