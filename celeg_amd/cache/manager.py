@@ -240,6 +240,14 @@ class CacheManager:
             g.updates = {}
         return out
 
+    def requeue_table_updates(self, updates: Sequence[Sequence[Tuple[int, int, int]]]) -> None:
+        """Put drained updates back (the step they were to travel with was refused).  A newer
+        update of the same table entry wins."""
+        for g, drained in zip(self.groups, updates):
+            fresh = g.updates
+            g.updates = {(slot, idx): page for slot, idx, page in drained}
+            g.updates.update(fresh)
+
     def layer_cache(self, step: int) -> LayerCache:
         kv = None
         writes = False

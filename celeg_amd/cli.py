@@ -113,8 +113,8 @@ def run(args) -> int:
     import torch
 
     import celeg_amd  # noqa: F401
-    from celeg_amd.config import read_config_file, spec_from_config
-    from celeg_amd.engine import Engine, RequestOptions, SchedulerOptions, StepEntry, load_model
+    from celeg_amd.engine import (Engine, RequestOptions, SchedulerOptions, StepEntry, load_model,
+                                  read_model_folder)
     from celeg_amd.engine.benchmark import DecodeBench, measure_prefill, random_prompt
     from celeg_amd.sampling import GenerationConfig
     from celeg_amd.weights import write_random_model
@@ -126,8 +126,7 @@ def run(args) -> int:
             cfg = json.load(fh)
         tmp = tempfile.TemporaryDirectory(prefix="celeg_random_")
         model_dir = write_random_model(cfg, tmp.name, args.random_weights_seed)
-    cfg_dict = read_config_file(model_dir)
-    config, spec = spec_from_config(cfg_dict)
+    config, spec = read_model_folder(model_dir)
     if args.print_config:
         print(json.dumps({"architecture": spec.architecture,
                           "config": {k: (list(v) if isinstance(v, tuple) else v)

@@ -100,29 +100,48 @@ class Lfm2Config:
 
     # ------------------------------------------------------------------ reading
     @classmethod
-    def from_dict(cls, cfg: Mapping[str, Any]) -> "Lfm2Config":
+    def from_dict(cls, cfg: Mapping[str, Any],
+                  tensor_shapes: Optional[Mapping[str, Tuple[int, ...]]] = None) -> "Lfm2Config":
         """Keys and defaults follow src/model/inference/metadata.cpp: hidden_size
         (353), intermediate_size (355-357), num_hidden_layers (358-360),
         num_attention_heads (364-366), num_key_value_heads (367-369), head_dim
         (370), vocab_size (399), max_position_embeddings (404-406), norm_eps
         (407-409, default 1e-6 at 643), conv_L_cache (425-426), rope_theta
-        (427-429, required 663-666), block_auto_adjust_ff_dim (512-514), tying
-        (630-632), token ids (638-642)."""
+        (427-429: also as ``rope_parameters.rope_theta``; required 663-666),
+        block_auto_adjust_ff_dim (512-514), tying (630-632), token ids (638-642).
+
+        ``tensor_shapes`` (name -> shape of the checkpoint's tensors), when given, fills
+        what config.json leaves out the way the reference does: the kind of every layer
+        from the tensors it has (``conv.in_proj.weight`` or ``self_attn.q_proj.weight``,
+        src/model/inference/rules.cpp:18-26, rules_attention.cpp:138-160) and the
+        feed-forward width from the rows of w1 (global_facts.cpp:127-152); a
+        ``layer_types`` that contradicts the tensors is an error.  The original LFM2 keys
+        ``full_attn_idxs`` (the attention layers; every other layer is a convolution) and
+        ``block_ff_dim`` (= intermediate_size) are read too."""
+        cfg = dict(cfg)
+        nested = cfg.get("rope_parameters")
+        if isinstance(nested, Mapping) and nested.get("rope_theta") is not None:
+            cfg["rope_parameters.rope_theta"] = nested["rope_theta"]
         vocab = _require(cfg, "vocab_size", int)
         hidden = _require(cfg, "hidden_size", int)
         layers = _require(cfg, "num_hidden_layers", int)
         heads = _require(cfg, "num_attention_heads", int)
         kv_heads = _alias(cfg, ("num_key_value_heads",), int, heads)
         head_dim = _alias(cfg, ("head_dim",), int, hidden // heads if heads > 0 else 0)
-        intermediate = _require(cfg, "intermediate_size", int)
-        rope_theta = _require(cfg, "rope_theta", float)
+        rope_theta = _alias(cfg, ("rope_theta", "rope_parameters.rope_theta"), float, None)
+        if rope_theta is None:
+            raise ConfigError("config.json: required key 'rope_theta' is missing")
         conv_l = _require(cfg, "conv_L_cache", int)
         max_pos = _require(cfg, "max_position_embeddings", int)
-        if "layer_types" not in cfg or cfg["layer_types"] is None:
-            raise ConfigError("config.json: required key 'layer_types' is missing")
-        kinds = cfg["layer_types"]
-        if not isinstance(kinds, (list, tuple)) or not all(isinstance(k, str) for k in kinds):
-            raise ConfigError("config.json: 'layer_types' must be a list of strings")
+        auto_adjust = _alias(cfg, ("block_auto_adjust_ff_dim",), bool, False)
+        intermediate = _alias(cfg, ("intermediate_size", "block_ff_dim"), int, None)
+        kinds = cls._layer_kinds(cfg, layers, tensor_shapes)
+        if intermediate is None:
+            w1 = (tensor_shapes or {}).get("model.layers.0.feed_forward.w1.weight")
+            if w1 is None:
+                raise ConfigError("config.json: required key 'intermediate_size' is missing")
+            # the width itself: no adjustment is applied to a size read off the weights
+            intermediate, auto_adjust = int(w1[0]), False
         eos = cfg.get("eos_token_id", 0)
         if isinstance(eos, (list, tuple)):
             eos_ids = tuple(int(e) for e in eos)
@@ -143,7 +162,7 @@ class Lfm2Config:
             rope_theta=rope_theta,
             norm_eps=_alias(cfg, ("norm_eps", "rms_norm_eps"), float, 1e-6),
             max_position_embeddings=max_pos,
-            block_auto_adjust_ff_dim=_alias(cfg, ("block_auto_adjust_ff_dim",), bool, False),
+            block_auto_adjust_ff_dim=auto_adjust,
             block_multiple_of=_alias(cfg, ("block_multiple_of",), int, 256),
             block_ffn_dim_multiplier=multiplier,
             tie_word_embeddings=_alias(cfg, ("tie_word_embeddings", "tie_embedding"), bool, True),
@@ -153,6 +172,46 @@ class Lfm2Config:
         )
         out.validate()
         return out
+
+    @staticmethod
+    def _layer_kinds(cfg, layers: int, tensor_shapes) -> Tuple[str, ...]:
+        """``layer_types`` if given; else from ``full_attn_idxs``; else from the tensors each
+        layer has.  Whatever the source, tensors that say otherwise are an error."""
+        from_tensors = None
+        if tensor_shapes is not None:
+            from_tensors = []
+            for i in range(layers):
+                conv = f"model.layers.{i}.conv.in_proj.weight" in tensor_shapes
+                attn = f"model.layers.{i}.self_attn.q_proj.weight" in tensor_shapes
+                from_tensors.append("conv" if conv and not attn else
+                                    "full_attention" if attn and not conv else None)
+        kinds = cfg.get("layer_types")
+        if kinds is not None:
+            if not isinstance(kinds, (list, tuple)) or not all(isinstance(k, str) for k in kinds):
+                raise ConfigError("config.json: 'layer_types' must be a list of strings")
+            kinds = tuple(kinds)
+        elif cfg.get("full_attn_idxs") is not None:
+            idxs = cfg["full_attn_idxs"]
+            if not isinstance(idxs, (list, tuple)) or \
+                    not all(isinstance(i, int) and not isinstance(i, bool) for i in idxs):
+                raise ConfigError("config.json: 'full_attn_idxs' must be a list of integers")
+            if any(not 0 <= i < layers for i in idxs):
+                raise ConfigError(f"config.json: 'full_attn_idxs' names a layer outside [0, {layers})")
+            kinds = tuple("full_attention" if i in set(idxs) else "conv" for i in range(layers))
+        elif from_tensors is not None:
+            unknown = [i for i, k in enumerate(from_tensors) if k is None]
+            if unknown:
+                raise ConfigError("config.json has no 'layer_types' and the tensors of layer(s) "
+                                  f"{unknown} tell neither a convolution nor an attention layer")
+            return tuple(from_tensors)
+        else:
+            raise ConfigError("config.json: required key 'layer_types' is missing")
+        if from_tensors is not None and len(kinds) == layers:
+            for i, (said, found) in enumerate(zip(kinds, from_tensors)):
+                if found is not None and said in _LAYER_KINDS and said != found:
+                    raise ConfigError(f"config.json: 'layer_types'[{i}] is {said!r} but the "
+                                      f"checkpoint's tensors of layer {i} are those of {found!r}")
+        return kinds
 
     def validate(self) -> None:
         """GQA divisibility, even head size and kv width as in

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_start, int n_seqs, bf16* __restrict__ out, int ldo,
     int q_heads, int kv_heads, int page_tokens, int page_shift, int n_layers, int layer,
-    float scale_log2e, int window) {
+    float scale_log2e, int window, int pages_room) {
     constexpr int ROWS = 64 * RT;   // rows of a workgroup
     constexpr int WROWS = 16 * RT;  // rows of a wavefront
     constexpr int DQ = HD / 4;      // dims a lane quad covers in q.k
@@ -139,15 +139,24 @@ __global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
     const int my_rounds = SHARE ? total_rounds : (total_rounds - half + NH - 1) / NH;   // rounds half, half + NH, ..
     const int n_it = (total_rounds + TURNS - 1) / TURNS;
     // the pages of the tile's rounds; behind the last key's page, that page again (allocated
-    // memory for the positions of the last round that are masked anyway)
+    // memory for the positions of the last round that are masked anyway), and before the
+    // first page that a row of the tile can still see (the first round starts at a multiple of
+    // 64 keys, which may lie in a page that a window has passed and the request has given
+    // back), that page.  They are copied to LDS where they fit its room; a tile with more
+    // pages than that (a context of several ten thousand tokens) looks them up in memory.
     const int page0 = first >> page_shift;
-    {
-        const int* __restrict__ pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
-        const int last_page = bkmax >> page_shift;
-        const int n_fill = ((first + 64 * total_rounds - 1) >> page_shift) - page0 + 1;
-        for (int i = threadIdx.x; i < n_fill; i += 256 * NH) spages[i] = pages[min(page0 + i, last_page)];
-    }
+    const int* __restrict__ const pages = table + static_cast<size_t>(seq_slot[s]) * table_stride;
+    const int last_page = bkmax >> page_shift;
+    const int live_page = (window > 0 ? max(0, start + brow0 - window + 1) : 0) >> page_shift;
+    const int n_fill = ((first + 64 * total_rounds - 1) >> page_shift) - page0 + 1;
+    const bool pages_in_lds = n_fill <= pages_room;
+    if (pages_in_lds)
+        for (int i = threadIdx.x; i < n_fill; i += 256 * NH)
+            spages[i] = pages[min(max(page0 + i, live_page), last_page)];
     __syncthreads();
+    auto page_at = [&](int i) __attribute__((always_inline)) -> unsigned {
+        return pages_in_lds ? spages[i] : pages[min(max(page0 + i, live_page), last_page)];
+    };
     const int c = lane & 15, qd = lane >> 4;
     const int wrow0 = brow0 + wave * WROWS;
     const bool wave_active = wrow0 < len && head_valid;
@@ -215,10 +224,10 @@ __global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
             if (!has_piece[j]) continue;
-            const unsigned kpage = spages[pg + k_pg[j]];
+            const unsigned kpage = page_at(pg + k_pg[j]);
             kstage[j] = *reinterpret_cast<const u32x4_t*>(
                 kbase + (static_cast<unsigned long long>(kpage) * page_stride + static_cast<unsigned>(inp * HD + k_off[j])));
-            const unsigned vpage = spages[pg + v_pg[j]];
+            const unsigned vpage = page_at(pg + v_pg[j]);
             vstage[j] = *reinterpret_cast<const u32x4_t*>(
                 vbase + (static_cast<unsigned long long>(vpage) * page_stride + static_cast<unsigned>(inp + v_off[j])));
         }
@@ -377,15 +386,33 @@ __global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
     }
 }
 
+// Most entries of a block-table row that a workgroup of attention_rows_kernel copies to LDS.
+// celeg_attention_rows_pages_in_lds() lets a test lower it, so that the lookup in memory runs
+// at small sizes too.
+static int ROWS_MAX_PAGES_IN_LDS = 4096;
+extern "C" void celeg_attention_rows_pages_in_lds(int entries) {
+    ROWS_MAX_PAGES_IN_LDS = entries > 0 ? min(entries, 4096) : 4096;
+}
+
+// LDS bytes that a launch with these sizes asks for (what the host-side check of the limit
+// of 160 KB works with): form 1 or 2 = sets of staging buffers.
+extern "C" long long celeg_attention_rows_lds_bytes(int head_dim, int sets, int table_stride) {
+    return static_cast<long long>(sets) * 2 * (64 * (head_dim + 8) + head_dim * (64 + 8)) * 2 +
+           static_cast<long long>(min(table_stride + 8, ROWS_MAX_PAGES_IN_LDS)) * 4;
+}
+
 template <int HD, int RT, int NH, bool SHARE>
 static int launch_attention_rows(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start,
     int n_seqs, int n_tokens, void* out, int ldo, int q_heads, int kv_heads, int page_tokens,
     int n_layers, int layer, float scale, int window, hipStream_t stream) {
-    // staging buffers, and a request's pages with room for a round's worth behind the last
+    // staging buffers, and a tile's pages with room for a round's worth behind the last: the
+    // whole of a request's block-table row where that is at most ROWS_MAX_PAGES_IN_LDS entries
+    // (16 KB; with the largest staging buffers, 143,360 bytes, still inside 160 KB)
+    const int pages_room = min(table_stride + 8, ROWS_MAX_PAGES_IN_LDS);
     const size_t lds = (SHARE ? 1 : NH) * 2 * (64 * (HD + 8) + HD * (64 + 8)) * sizeof(bf16) +
-                       (static_cast<size_t>(table_stride) + 8) * sizeof(int);
+                       static_cast<size_t>(pages_room) * sizeof(int);
     if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
     // the kernel multiplies page numbers by the elements of a page in 32 x 32 -> 64 bits
     if (static_cast<size_t>(n_layers) * kv_heads * page_tokens * HD >= (size_t{1} << 31))
@@ -406,7 +433,8 @@ static int launch_attention_rows(
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
                        table_stride, cu_seqlens, seq_slot, seq_start, n_seqs,
                        static_cast<bf16*>(out), ldo, q_heads, kv_heads, page_tokens,
-                       __builtin_ctz(page_tokens), n_layers, layer, scale * 1.4426950408889634f, window);
+                       __builtin_ctz(page_tokens), n_layers, layer, scale * 1.4426950408889634f, window,
+                       pages_room);
     return CELEG_LAUNCH_RESULT();
 }
 

@@ -4,8 +4,8 @@ pointers and the current HIP stream (so a stream that is capturing a graph captu
 them too).  There is no fallback: if a library cannot be built or loaded, or a tensor
 is not on the GPU, the call fails loudly.
 
-Matrix products in bfloat16 go to the library behind ``torch.mm`` (hipBLASLt /
-rocBLAS), as the reference sends its products to cuBLAS
+Matrix products in bfloat16 of more than 64 rows go to hipBLASLt, called directly
+(``blaslt.py``), as the reference sends its products to cuBLAS
 (src/backend/cuda/runtime/gemm_dispatcher.cpp); products in 32-bit go to our own
 kernel, which uses no reduced-precision matrix mode.
 """

@@ -51,6 +51,17 @@ def make_runtime(device, dtype, ops=None) -> Runtime:
     return Runtime(device, dtype, ops, Workspace(device))
 
 
+def read_model_folder(model_dir: str):
+    """(typed configuration, ModelSpec) of a model folder: config.json (with
+    generation_config.json merged) and, for what it leaves out, the tensors' names and shapes."""
+    cfg_dict = read_config_file(model_dir)
+    ckpt = Checkpoint(model_dir)
+    try:
+        return spec_from_config(cfg_dict, {n: tuple(ckpt.info(n).shape) for n in ckpt.names()})
+    finally:
+        ckpt.close()
+
+
 def load_model(model_dir: str, *, dtype="bfloat16", device="cuda:0", page_tokens: int = 16,
                n_pages: Optional[int] = None, max_requests: int = 8,
                max_context: Optional[int] = None, max_batched_tokens: int = 2048,
@@ -65,16 +76,20 @@ def load_model(model_dir: str, *, dtype="bfloat16", device="cuda:0", page_tokens
         raise ValueError(f"gemm_backend must be 'library' or 'tiles', not '{gemm_backend}'")
     dtype = parse_dtype(dtype)
     cfg_dict = read_config_file(model_dir)
-    config, spec = spec_from_config(cfg_dict)
-    if max_context is None:
-        max_context = spec.max_context
-    if max_context > spec.max_context:
-        raise ValueError(f"--context {max_context} exceeds model maximum {spec.max_context}")
-    model = Model(spec)
-    rt = make_runtime(device, dtype, ops)
-    rt.use_tiled_products = gemm_backend == "tiles"
     ckpt = Checkpoint(model_dir)
     try:
+        config, spec = spec_from_config(cfg_dict, {n: tuple(ckpt.info(n).shape) for n in ckpt.names()})
+    except Exception:
+        ckpt.close()
+        raise
+    if max_context is None:
+        max_context = spec.max_context
+    try:
+        if max_context > spec.max_context:
+            raise ValueError(f"--context {max_context} exceeds model maximum {spec.max_context}")
+        model = Model(spec)
+        rt = make_runtime(device, dtype, ops)
+        rt.use_tiled_products = gemm_backend == "tiles"
         tensors = load_tensors(ckpt, model.expected_tensors(), dtype, device)
     finally:
         ckpt.close()

@@ -62,8 +62,9 @@ class ModelRunner:
         n_groups = len(cache.groups)
         S = cache.max_requests
         # room for the largest step, with as many table updates as rows plus requests
+        self._update_room = max_batched_tokens // cache.page_tokens + 2 * S + 8
         _, ints = packed_layout(max_batched_tokens, S, max_batched_tokens,
-                                [max_batched_tokens // cache.page_tokens + 2 * S + 8] * n_groups)
+                                [self._update_room] * n_groups)
         self.builder = BatchBuilder(rt.device, ints, n_groups,
                                     pin=torch.device(rt.device).type == "cuda")
         self.steps_run = 0
@@ -107,6 +108,9 @@ class ModelRunner:
                 in_range = toks.min() >= 0 and toks.max() < vocab
             if not in_range:
                 raise ValueError(f"step: token id out of range [0, {vocab})")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise ValueError(f"wanted place {w} is outside the entry's {n} tokens")
             if not self.cache.covers(e.slot, e.start_pos, n):
                 raise ValueError(f"step: the pages of slot {e.slot} do not cover positions "
                                  f"[{e.start_pos}, {e.start_pos + n})")
@@ -129,8 +133,8 @@ class ModelRunner:
         mixed = self._mixed_shape(entries)
         if mixed is not None:
             return self._mixed_from_graph(entries, mixed)
-        updates = self.cache.drain_table_updates()
-        batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot)
+        updates = self._drain_updates([self._update_room] * len(self.cache.groups))
+        batch = self._build(entries, updates, null_slot=self.cache.null_slot)
         self._begin_step(batch)
         self.last_batch = batch
         logits = self.model.forward(batch, self.rt)
@@ -172,13 +176,9 @@ class ModelRunner:
         captured = self._graphs.get((bucket, bound))
         if captured is None or captured[2] != self.rt.ws.generation:
             captured = self._capture(bucket, caps, bound)
-        updates = self.cache.drain_table_updates()
-        for g, u in enumerate(updates):
-            if len(u) > caps[g]:           # a burst (a large reservation): ship it on its own
-                self._ship_table_updates(g, u)
-                updates[g] = []
-        batch = self.builder.build(entries, updates, pad_to=bucket,
-                                   null_slot=self.cache.null_slot, update_caps=caps)
+        updates = self._drain_updates(caps)
+        batch = self._build(entries, updates, pad_to=bucket,
+                            null_slot=self.cache.null_slot, update_caps=caps)
         self.last_batch = batch
         captured[0].replay()
         self.steps_run += 1
@@ -239,12 +239,8 @@ class ModelRunner:
                 return batch
             captured = self._capture_batch(make_batch)
             self._portion_graphs[shape] = captured
-        updates = self.cache.drain_table_updates()
-        for g, u in enumerate(updates):
-            if len(u) > caps[g]:
-                self._ship_table_updates(g, u)
-                updates[g] = []
-        batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot, update_caps=caps)
+        updates = self._drain_updates(caps)
+        batch = self._build(entries, updates, null_slot=self.cache.null_slot, update_caps=caps)
         self.last_batch = batch
         captured[0].replay()
         self.steps_run += 1
@@ -325,15 +321,11 @@ class ModelRunner:
                 return batch
             captured = self._capture_batch(make_batch)
             self._mixed_graphs[shape] = captured
-        updates = self.cache.drain_table_updates()
-        for g, u in enumerate(updates):
-            if len(u) > caps[g]:
-                self._ship_table_updates(g, u)
-                updates[g] = []
+        updates = self._drain_updates(caps)
         # every portion's last row gets logits, as in the recording; those nobody wants lie
         # behind the wanted ones
-        batch = self.builder.build(entries, updates, null_slot=self.cache.null_slot, update_caps=caps,
-                                   pad_singles_to=bucket, last_rows_too=True)
+        batch = self._build(entries, updates, null_slot=self.cache.null_slot, update_caps=caps,
+                            pad_singles_to=bucket, last_rows_too=True)
         self.last_batch = batch
         captured[0].replay()
         self.steps_run += 1
@@ -382,6 +374,26 @@ class ModelRunner:
         if self._token_source is not None:
             self.rt.ops.resolve_tokens(batch.token_ids, batch.token_slot, self._token_source,
                                        batch.n_tokens)
+
+    def _drain_updates(self, caps):
+        """The block-table updates since the last step, per group.  A group with more of them
+        than the step's metadata has room for (a large reservation made at once) has them
+        shipped on their own, ahead of the step."""
+        updates = self.cache.drain_table_updates()
+        for g, u in enumerate(updates):
+            if len(u) > caps[g]:
+                self._ship_table_updates(g, u)
+                updates[g] = []
+        return updates
+
+    def _build(self, entries, updates, **how) -> StepBatch:
+        """``builder.build``; if it refuses the step, the drained updates go back to the cache
+        manager, so that the device's block tables still get them with the next step."""
+        try:
+            return self.builder.build(entries, updates, **how)
+        except Exception:
+            self.cache.requeue_table_updates(updates)
+            raise
 
     def _ship_table_updates(self, group: int, updates) -> None:
         flat = torch.tensor([len(updates)] + [v for u in updates for v in u], dtype=torch.int32)

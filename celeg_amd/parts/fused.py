@@ -110,9 +110,11 @@ def folded_weight(rt, w: torch.Tensor, norm_weight: torch.Tensor) -> torch.Tenso
     key = (w.data_ptr(), norm_weight.data_ptr())
     hit = cache.get(key)
     if hit is None:
-        hit = _pack(rt, (w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype))
-        cache[key] = hit
-    return hit
+        # (the entry holds on to both tensors: their addresses cannot pass to other weights
+        # while it exists)
+        hit = cache[key] = (_pack(rt, (w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype)),
+                            w, norm_weight)
+    return hit[0]
 
 
 def folded_plain_weight(rt, w: torch.Tensor, norm_weight: torch.Tensor) -> torch.Tensor:
@@ -122,8 +124,9 @@ def folded_plain_weight(rt, w: torch.Tensor, norm_weight: torch.Tensor) -> torch
     key = (w.data_ptr(), norm_weight.data_ptr())
     hit = cache.get(key)
     if hit is None:
-        hit = cache[key] = (w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype).contiguous()
-    return hit
+        hit = cache[key] = ((w.float() * norm_weight.float().reshape(1, -1)).to(w.dtype).contiguous(),
+                            w, norm_weight)
+    return hit[0]
 
 
 def packed_weight(rt, w: torch.Tensor) -> torch.Tensor:
@@ -131,8 +134,8 @@ def packed_weight(rt, w: torch.Tensor) -> torch.Tensor:
     cache = rt.__dict__.setdefault("packed_weights", {})
     hit = cache.get(w.data_ptr())
     if hit is None:
-        hit = cache[w.data_ptr()] = _pack(rt, w)
-    return hit
+        hit = cache[w.data_ptr()] = (_pack(rt, w), w)
+    return hit[0]
 
 
 def norm_linear(rt, h, norm, w, out, *, epilogue="store", rows=None, n_rows=None, **kw):

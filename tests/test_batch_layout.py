@@ -41,3 +41,18 @@ def test_single_rows_only_and_padding():
 def test_a_portion_alone_has_no_single_rows():
     b = build([StepEntry(0, 0, [1, 2, 3, 4], [3])])
     assert b.single_rows == 0 and b.logit_rows.tolist() == [3]
+
+
+def test_attention_rows_kernel_fits_lds_at_the_longest_context():
+    """What the prefill attention asks of LDS at a block table of 8,000 entries (a context of
+    128,000 tokens in pages of 16) for every head size and form: within the 160 KB of a
+    compute unit, because a tile keeps at most 4,096 entries of its request's table there."""
+    import ctypes
+    from celeg_amd.csrc import build
+    lib = ctypes.CDLL(build.ensure_built("attention_fast"))
+    lib.celeg_attention_rows_lds_bytes.restype = ctypes.c_longlong
+    for head_dim in (32, 64, 96, 128):
+        for sets in (1, 2):
+            for stride in (8, 256, 4096, 8000, 1 << 20):
+                need = lib.celeg_attention_rows_lds_bytes(head_dim, sets, stride)
+                assert 0 < need <= 160 * 1024, (head_dim, sets, stride, need)

@@ -48,6 +48,65 @@ def test_config_defaults_and_aliases():
         Lfm2Config.from_dict(dict(TINY_A, rms_norm_eps=1e-3))
 
 
+def _shapes(cfg):
+    return {n: tuple(w.shape) for n, w in _expected(cfg).items()}
+
+
+def test_keys_the_reference_accepts_in_other_places(tmp_path):
+    """rope_theta under rope_parameters (src/model/inference/metadata.cpp:427-429), the
+    original LFM2 keys full_attn_idxs and block_ff_dim, layer kinds and the feed-forward
+    width from the checkpoint's tensors when config.json is silent
+    (src/model/inference/rules.cpp:18-26, rules_attention.cpp:138-160,
+    global_facts.cpp:127-152), and generation_config.json overriding the end tokens
+    (src/checkpoint/catalog.cpp:94-121)."""
+    from celeg_amd.config import read_config_file
+    from celeg_amd.engine import read_model_folder
+    base = Lfm2Config.from_dict(TINY_B)
+    # a config.json as newer writers lay it out: no top-level rope_theta
+    nested = {k: v for k, v in TINY_B.items() if k != "rope_theta"}
+    nested["rope_parameters"] = {"rope_theta": 1000000.0, "rope_type": "default"}
+    assert Lfm2Config.from_dict(nested) == base
+    with pytest.raises(ConfigError, match="disagree"):
+        Lfm2Config.from_dict(dict(nested, rope_theta=5.0))
+    # the original keys
+    old = {k: v for k, v in TINY_B.items() if k not in ("layer_types", "intermediate_size")}
+    old.update(full_attn_idxs=[2, 4], block_ff_dim=512)
+    assert Lfm2Config.from_dict(old) == base
+    with pytest.raises(ConfigError, match="full_attn_idxs"):
+        Lfm2Config.from_dict(dict(old, full_attn_idxs=[2, 6]))
+    with pytest.raises(ConfigError, match="disagree"):
+        Lfm2Config.from_dict(dict(old, intermediate_size=500))
+    # silent config: kinds and width from the tensors
+    silent = {k: v for k, v in TINY_B.items() if k not in ("layer_types", "intermediate_size")}
+    got = Lfm2Config.from_dict(silent, _shapes(TINY_B))
+    assert got.layer_types == base.layer_types and got.ff_dim == base.ff_dim == 352
+    with pytest.raises(ConfigError, match="layer_types"):
+        Lfm2Config.from_dict(silent)                       # nothing to infer from
+    with pytest.raises(ConfigError, match="intermediate_size"):
+        Lfm2Config.from_dict(dict(silent, layer_types=list(base.layer_types)))
+    shapes = _shapes(TINY_B)
+    del shapes["model.layers.3.conv.in_proj.weight"]
+    with pytest.raises(ConfigError, match=r"layer\(s\) \[3\]"):
+        Lfm2Config.from_dict(silent, shapes)
+    # a layer_types that contradicts the tensors
+    wrong = list(base.layer_types)
+    wrong[0], wrong[2] = wrong[2], wrong[0]
+    with pytest.raises(ConfigError, match=r"'layer_types'\[0\]"):
+        Lfm2Config.from_dict(dict(TINY_B, layer_types=wrong), _shapes(TINY_B))
+    # through a folder: the silent config loads, and generation_config.json wins
+    folder = write_random_model(TINY_B, str(tmp_path / "m"), seed=0, dtype=torch.float32)
+    json.dump(silent, open(os.path.join(folder, "config.json"), "w"))
+    json.dump({"bos_token_id": 9, "eos_token_id": [11, 12, "x"], "temperature": 0.3},
+              open(os.path.join(folder, "generation_config.json"), "w"))
+    config, spec = read_model_folder(folder)
+    assert config.layer_types == base.layer_types and config.ff_dim == 352
+    assert config.eos_token_ids == (11, 12) and config.bos_token_id == 9 and spec.eos_token_ids == (11, 12)
+    json.dump({"eos_token_id": 5}, open(os.path.join(folder, "generation_config.json"), "w"))
+    assert read_config_file(folder)["eos_token_id"] == 5 and read_config_file(folder)["bos_token_id"] == 0
+    open(os.path.join(folder, "generation_config.json"), "w").write("{ not json")
+    assert read_config_file(folder)["eos_token_id"] == [2, 3]     # unreadable: ignored
+
+
 @pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers",
                                  "num_attention_heads", "rope_theta", "conv_L_cache",
                                  "layer_types", "intermediate_size", "max_position_embeddings"])

@@ -363,3 +363,83 @@ def test_many_requests_decoding_together(model_folders, name, n_requests, join_e
         assert_close(got[rid], ref, dtype, f"{name}/{dtype}/{n_requests} together/{rid}")
     lm.cache.check()
     assert lm.cache.n_free_slots == n_requests and lm.cache.free_pages() == [pages]
+
+
+def test_a_large_reservation_and_a_refused_step_keep_the_device_tables_right(model_folders):
+    """Pages reserved thousands at a time (what guaranteed_no_evict does at admission) are
+    more block-table updates than a step's metadata has room for: the eager path ships them on
+    their own.  A step that is refused after the updates were drained (a wanted place outside
+    the entry, metadata that does not fit) leaves them queued for the next step, whose logits
+    are then those of the plain implementation."""
+    from cpu_ops import CpuOps
+    from celeg_amd.engine import StepEntry, load_model
+    folder = model_folders("A", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    lm = load_model(folder, dtype="float32", device="cpu", page_tokens=2, n_pages=300,
+                    max_requests=4, max_context=128, max_batched_tokens=16, ops=CpuOps())
+    room = lm.runner._update_room
+    slots = [lm.cache.open() for _ in range(4)]
+    for s in slots:
+        assert lm.cache.prepare(s, 0, 128)          # 64 pages each, 256 updates pending
+    assert 256 > room
+    prompts = [random_tokens(256, 9 + i, seed=40 + i) for i in range(4)]
+    logits = lm.runner.step([StepEntry(s, 0, p[:3], [2]) for s, p in zip(slots, prompts)])
+    for i, p in enumerate(prompts):
+        assert_close(logits[i], plain.model_logits(cfg, W, p[:3])[-1], "float32", f"burst/{i}")
+    host = torch.from_numpy(lm.cache.groups[0].table_host)
+    assert torch.equal(lm.cache.groups[0].table[:4], host[:4])
+    # a refused step: the updates of new pages stay queued
+    for s in slots:
+        lm.cache.close(s)
+    slots = [lm.cache.open() for _ in range(2)]
+    assert lm.cache.prepare(slots[0], 0, 5) and lm.cache.prepare(slots[1], 0, 4)
+    with pytest.raises(ValueError, match="wanted place"):
+        lm.runner.step([StepEntry(slots[0], 0, prompts[0][:5], [5])])
+    lm.runner.builder.capacity, kept = 8, lm.runner.builder.capacity
+    with pytest.raises(ValueError, match="staging buffer"):
+        lm.runner.step([StepEntry(slots[0], 0, prompts[0][:5], [4])])
+    lm.runner.builder.capacity = kept
+    logits = lm.runner.step([StepEntry(slots[0], 0, prompts[0][:5], [4]),
+                             StepEntry(slots[1], 0, prompts[1][:4], [3])])
+    assert_close(logits[0], plain.model_logits(cfg, W, prompts[0][:5])[-1], "float32", "after refusal/0")
+    assert_close(logits[1], plain.model_logits(cfg, W, prompts[1][:4])[-1], "float32", "after refusal/1")
+    host = torch.from_numpy(lm.cache.groups[0].table_host)
+    live = host >= 0
+    assert torch.equal(lm.cache.groups[0].table[live], host[live])
+
+
+@pytest.mark.gpu
+def test_few_rows_and_many_rows_agree_at_norm_weights_far_from_one(model_folders, tmp_path):
+    """Steps of up to 64 rows multiply the norm's weight into the bfloat16 matrices (one more
+    rounding of every weight); steps of more rows apply it to the rows in 32-bit.  With norm
+    weights between 0.3 and 3 the two still give the same logits within the bfloat16 bound,
+    and each agrees with the plain implementation."""
+    from celeg_amd.engine import load_model
+    from celeg_amd.weights import SafetensorsFile, write_safetensors
+    import json, os, shutil
+    src = model_folders("E", torch.bfloat16, WEIGHT_STD)
+    folder = str(tmp_path / "far_from_one")
+    os.makedirs(folder)
+    shutil.copy(os.path.join(src, "config.json"), folder)
+    f = SafetensorsFile(os.path.join(src, "model.safetensors"))
+    g = torch.Generator().manual_seed(5)
+    tensors = {}
+    for name in f.names():
+        t = f.tensor(name).clone()
+        if name.endswith("norm.weight"):                 # operator_norm, ffn_norm, embedding_norm
+            t = (t.float() * torch.exp(torch.empty(t.shape).uniform_(-1.2, 1.1, generator=g))).to(t.dtype)
+        tensors[name] = t
+    f.close()
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    cfg, W = plain.load_model_folder(folder)
+    toks = random_tokens(TINY["E"][0]["vocab_size"], 200, seed=77)
+    ref = plain.model_logits(cfg, W, toks)
+    reqs = {"r": toks}
+    out = {}
+    for mode, steps in (("many", whole_schedule(reqs)),
+                        ("few", portions_schedule(reqs, sizes=(16, 9, 33, 2, 64, 1)))):
+        lm = load_model(folder, dtype="bfloat16", page_tokens=16, n_pages=16, max_requests=2,
+                        max_batched_tokens=256)
+        out[mode] = EngineDriver(lm).run(steps)["r"]
+        assert_close(out[mode], ref, "bfloat16", f"norm weights far from one/{mode}")
+    assert_close(out["few"], out["many"].double(), "bfloat16", "few rows against many rows")

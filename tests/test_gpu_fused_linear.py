@@ -373,3 +373,38 @@ def test_unsupported_sizes_are_refused(ops):
     with pytest.raises(KernelError, match="not supported"):
         ops.fused_linear(randn(65, 64, dtype=BF), w, torch.empty(65, 32, dtype=BF, device=DEV))
     assert not ops.fused_linear_ok(8, 100) and ops.fused_linear_ok(64, 96)
+
+
+@pytest.mark.parametrize("K", [1024, 2048])
+@pytest.mark.parametrize("R", [1, 8, 17, 64])
+def test_output_head_at_the_real_vocabulary(R, K):
+    """Final norm and output product the way the model's head runs them for few wanted rows
+    (``parts.embedding._head_fused`` -> ``norm_linear``), at 65,536 columns: wider than the
+    k-sliced kernels take, so up to 8 rows go to the kernel that keeps its rows in LDS and 9
+    to 64 rows to the one that streams the weights.  Rows picked out of a longer stream."""
+    from types import SimpleNamespace
+    from celeg_amd.engine import make_runtime
+    from celeg_amd.parts.embedding import _head_fused
+    from celeg_amd.parts.norm import RmsNorm
+    from celeg_amd.config.spec import PartSpec
+    V = 65536
+    rt = make_runtime(DEV, BF)
+    T = R + 5 if R < 64 else 64
+    h = randn(T, K, seed=60)
+    norm = RmsNorm(PartSpec("rmsnorm", {"width": K, "eps": 1e-5}))
+    norm.weight = 1 + randn(K, seed=61, scale=0.1)
+    w = randn(V, K, seed=62, scale=0.05, dtype=BF)
+    picked = [(3 * i + 1) % T for i in range(R)]
+    rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
+    batch = SimpleNamespace(n_tokens=T, n_logit_rows=R, logit_rows=rows)
+    out = torch.full((R, V), float("nan"), device=DEV)
+    rt.stream_stat_blocks = 0
+    assert _head_fused(h, norm, batch, out, rt, w)
+    x = plain.rmsnorm(h.cpu(), norm.weight.cpu(), 1e-5)[picked].to(BF).float()
+    ref = x @ w.float().cpu().T            # exact products of bfloat16 values, summed in 32-bit
+    got = out.cpu()
+    assert torch.isfinite(got).all()
+    bound = 8e-3 * float(ref.abs().max())   # the norm weight folded into bfloat16 weights costs a rounding
+    assert float((got - ref).abs().max()) <= bound, float((got - ref).abs().max())
+    # the last columns and rows are there
+    assert float((got[-1, -64:] - ref[-1, -64:]).abs().max()) <= bound

@@ -272,6 +272,74 @@ def test_short_conv_reference_vector(ops):
     assert out.cpu().tolist() == [[6.0, 12.0]]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_short_conv_vector_tells_the_three_thirds_of_bcx_apart(ops, dtype):
+    # worked by hand from src/backend/cpu/kernels/convolution.cpp:14-27 (see test_plain.py):
+    # rows {2,3,5}, {7,11,13}; taps {1,1} -> {30, 1111} (C and x swapped: 1079; B and C: 1106);
+    # taps {2,1} -> {30, 1221} (the filter reversed: 2112).  In one step, and token by token
+    # through the saved state.  All values are exact in bfloat16 except 1111 and 1221.
+    from celeg_amd.engine import StepEntry
+    from celeg_amd.parts.base import StateNeed
+    rows = torch.tensor([[2., 3., 5.], [7., 11., 13.]], device=DEV).to(dtype)
+    for taps, want in (([1., 1.], [30., 1111.]), ([2., 1.], [30., 1221.])):
+        w = torch.tensor([taps], device=DEV)
+        for cuts in ([2], [1, 1]):
+            cache = make_cache(0, 0, 0, dtype, states=[(0, StateNeed("bx", (2, 1)))])
+            slot = cache.open()
+            got, pos = [], 0
+            for c in cuts:
+                batch, keep = build_batch(ops, cache, [StepEntry(slot, pos, [0] * c)])
+                out = torch.empty(c, 1, dtype=dtype, device=DEV)
+                ops.short_conv(rows[pos:pos + c].contiguous(), w, None,
+                               cache.layer_cache(0).states["bx"], out, batch)
+                got += out.float().cpu().reshape(-1).tolist()
+                pos += c
+            if dtype == torch.float32:
+                assert got == want
+            else:
+                assert got[0] == want[0] and abs(got[1] - want[1]) <= 4.0   # far from 1079, 1106, 2112
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("head_dim", [2, 64])
+def test_q_and_k_are_normalised_before_they_are_rotated(ops, dtype, head_dim):
+    """q = k = {3, 4}, norm weight {1, 2}, eps 0, position 1, one pair of frequency 1: the
+    kernel that normalises, rotates and stores gives {-1.44557, 1.93658}
+    (src/backend/cpu/kernels/rope.cpp:95-108, worked by hand in test_plain.py); rotating
+    before normalising would give {-0.4936, 2.6506}.  With head size 64 the pair lies at
+    places 0 and 32, every other place is zero and every other frequency tiny."""
+    from celeg_amd.engine import StepEntry
+    from test_plain import QK_NORM_THEN_ROPE
+    half = head_dim // 2
+    cache = make_cache(1, head_dim, 1, dtype, n_pages=2)
+    kv = cache.layer_cache(0).kv
+    slot = cache.open()
+    assert cache.prepare(slot, 0, 2)
+    batch, keep = build_batch(ops, cache, [StepEntry(slot, 0, [0, 0])])
+    row = torch.zeros(2, head_dim)
+    row[1, 0], row[1, half] = 3.0, 4.0
+    # (the mean of squares is over head_dim values: scale so that 1/rms is that of {3, 4} alone)
+    row *= math.sqrt(head_dim / 2)
+    q = row.to(dtype).to(DEV)
+    k, v = q.clone(), q.clone()
+    weight = torch.ones(head_dim)
+    weight[half] = 2.0
+    weight = weight.to(DEV)
+    inv_freq = torch.zeros(half)
+    inv_freq[0] = 1.0
+    ops.qk_norm_rope_store(q, k, v, weight, weight, 0.0, inv_freq.to(DEV), head_dim, 1, 1, head_dim,
+                           batch, kv)
+    torch.cuda.synchronize()
+    page = int(cache.groups[0].table_host[slot, 0])
+    stored_k = kv.k[page, 0, 0, 1].float().cpu()            # [page, layer, head, token, :]
+    bound = 1e-5 if dtype == torch.float32 else 2e-2
+    for got in (q[1].float().cpu(), stored_k):
+        assert abs(float(got[0]) - QK_NORM_THEN_ROPE[0]) <= bound
+        assert abs(float(got[half]) - QK_NORM_THEN_ROPE[1]) <= bound
+    # the values are stored as they came (transposed inside the page: [.., head_dim, token])
+    assert float(kv.v[page, 0, 0, half, 1]) == float(v[1, half])
+
+
 def attention_case(ops, dtype, heads, kv_heads, head_dim, lengths, cuts, window=None,
                    qk_norm=True, theta=10000.0, rotary_dim=None, boost=None, page_tokens=16):
     """Runs norm+rope+store and attention for several requests cut into steps (one step
@@ -467,3 +535,63 @@ def test_attention_decode_one_workgroup_per_request(ops, heads, kv_heads, head_d
     finally:
         ops.attention_decode_whole = -1
         ops.decode_part_thresholds = (64, 256)
+
+
+def test_attention_rows_with_the_block_table_looked_up_in_memory(ops):
+    """A tile whose pages do not fit the room that the kernel keeps for them in LDS (contexts
+    of several ten thousand tokens) looks them up in memory instead: forced here at a small
+    size by lowering that room to 8 entries, against the same case with the table in LDS."""
+    lib = ops._lib("attention_fast")
+    lib.celeg_attention_rows_pages_in_lds(8)
+    try:
+        attention_case(ops, torch.bfloat16, 4, 2, 64, lengths=[717, 150, 390], cuts=[330, 61, 200],
+                       boost=(2, 700))
+        attention_case(ops, torch.bfloat16, 2, 1, 128, lengths=[500], cuts=[270, 230], window=150,
+                       boost=(301, 450), qk_norm=False, rotary_dim=0, page_tokens=32)
+    finally:
+        lib.celeg_attention_rows_pages_in_lds(0)
+
+
+@pytest.mark.parametrize("head_dim,page_tokens", [(64, 16), (128, 16), (32, 32)])
+def test_window_attention_never_reads_pages_it_has_given_back(ops, head_dim, page_tokens):
+    """A window group hands back the pages that the window has passed; the device's block
+    table still names them.  Another request takes them and fills them with infinities.  The
+    first round of 64 keys of a tile starts at a multiple of 64, before the window's first
+    key: the kernel must stay on the request's live pages there (a masked key has probability
+    zero, and zero times infinity is not a number)."""
+    from celeg_amd.cache import CacheLayout, CacheManager
+    from celeg_amd.engine import StepEntry
+    from celeg_amd.parts.base import KVNeed
+    window, heads, kv_heads = 40, 2, 1
+    layout = CacheLayout()
+    layout.kv_groups = [KVNeed(kv_heads, head_dim, window)]
+    layout.group_layers = [1]
+    layout.kv_of_step = {0: (0, 0, True)}
+    cache = CacheManager(layout, page_tokens=page_tokens, n_pages=24, max_requests=2, max_context=512,
+                         device=DEV, dtype=torch.bfloat16)
+    kv = cache.layer_cache(0).kv
+    n = 330
+    q = randn(n, heads * head_dim, seed=70, dtype=torch.bfloat16)
+    k = randn(n, kv_heads * head_dim, seed=71, dtype=torch.bfloat16)
+    v = randn(n, kv_heads * head_dim, seed=72, dtype=torch.bfloat16)
+    slot = cache.open()
+    got, pos = [], 0
+    for c in [150, 100, 1, 1, 78]:
+        assert cache.prepare(slot, pos, c)          # gives back what lies before pos - window + 1
+        held = set(cache.pages_held(slot)[0])
+        free = [p for p in range(24) if p not in held]
+        kv.k[free] = float("inf")                   # what another request may have left there
+        kv.v[free] = float("inf")
+        batch, keep = build_batch(ops, cache, [StepEntry(slot, pos, [0] * c)])
+        qs, ks, vs = (t[pos:pos + c].contiguous() for t in (q, k, v))
+        ops.qk_norm_rope_store(qs, ks, vs, None, None, 1e-5, None, 0, heads, kv_heads, head_dim, batch, kv)
+        out = torch.empty_like(qs)
+        ops.paged_attention(qs, out, heads, kv_heads, head_dim, 1 / math.sqrt(head_dim), window, batch, kv)
+        got.append(out.double().cpu())
+        pos += c
+    got = torch.cat(got)
+    assert torch.isfinite(got).all()
+    ref = plain.causal_attention(q.double().cpu().reshape(n, heads, head_dim),
+                                 k.double().cpu().reshape(n, kv_heads, head_dim),
+                                 v.double().cpu().reshape(n, kv_heads, head_dim), window=window).reshape(n, -1)
+    torch.testing.assert_close(got, ref, **tol(torch.bfloat16))

@@ -39,6 +39,44 @@ def test_conv_vector():
     assert y.tolist() == [[6., 12.]]
 
 
+def test_conv_vector_tells_the_three_thirds_of_bcx_apart():
+    # Worked by hand from src/backend/cpu/kernels/convolution.cpp:14-27 (b = bcx[ch],
+    # c = bcx[H + ch], x = bcx[2H + ch]; state = b * x; output = c * conv), H 1, L 2, taps
+    # {1, 1}: rows {2,3,5} and {7,11,13} give bx = {10, 91}, y = {3 * 10, 11 * (10 + 91)}.
+    # C and x swapped would give {30, 1079}; B and C swapped {30, 1106}.
+    y = plain.short_conv(torch.tensor([[2., 3., 5.], [7., 11., 13.]]), torch.tensor([[1., 1.]]))
+    assert y.reshape(-1).tolist() == [30., 1111.]
+    # taps {2, 1}: tap L-1 multiplies the current token, tap 0 the one before
+    # (weight[tap * hidden + channel] with slot (cursor + 1 + tap) % L): 11 * (2 * 10 + 91);
+    # the filter reversed would give 11 * (10 + 2 * 91) = 2112
+    y = plain.short_conv(torch.tensor([[2., 3., 5.], [7., 11., 13.]]), torch.tensor([[2., 1.]]))
+    assert y.reshape(-1).tolist() == [30., 1221.]
+
+
+# q = {3, 4}, norm weight {1, 2}, eps 0, position 1, head size 2 (one pair, frequency 1):
+# src/backend/cpu/kernels/rope.cpp:95-108 normalises first, inv = 1/sqrt(12.5),
+# a = 3 inv, b = 4 inv * 2, and rotates the normalised pair by the angle 1:
+# {a cos1 - b sin1, b cos1 + a sin1}.  Rotating first and normalising after would give
+# {(3 cos1 - 4 sin1) inv, (4 cos1 + 3 sin1) inv * 2} = {-0.4936, 2.6506}.
+QK_NORM_THEN_ROPE = [3 / math.sqrt(12.5) * math.cos(1.0) - 8 / math.sqrt(12.5) * math.sin(1.0),
+                     8 / math.sqrt(12.5) * math.cos(1.0) + 3 / math.sqrt(12.5) * math.sin(1.0)]
+
+
+def test_q_and_k_are_normalised_before_they_are_rotated():
+    assert abs(QK_NORM_THEN_ROPE[0] - (-1.445570)) < 1e-6 and abs(QK_NORM_THEN_ROPE[1] - 1.936577) < 1e-6
+    cfg = {"num_attention_heads": 1, "num_key_value_heads": 1, "head_dim": 2, "norm_eps": 0.0,
+           "rope_theta": 10000.0}
+    eye = torch.eye(2, dtype=torch.float64)
+    W = {"self_attn.q_proj.weight": eye, "self_attn.k_proj.weight": eye, "self_attn.v_proj.weight": eye,
+         "self_attn.q_layernorm.weight": torch.tensor([1., 2.]),
+         "self_attn.k_layernorm.weight": torch.tensor([1., 2.])}
+    n = torch.tensor([[0., 0.], [3., 4.]], dtype=torch.float64)     # the row at position 1 is {3, 4}
+    q, k, v = plain.attention_project(n, W, "", cfg, [0, 1])
+    for got in (q[1, 0], k[1, 0]):
+        assert torch.allclose(got, torch.tensor(QK_NORM_THEN_ROPE, dtype=torch.float64), atol=1e-6)
+    assert v[1, 0].tolist() == [3., 4.]
+
+
 def test_attention_vector():
     # tests/reference_test.cpp:40-53: 2 query heads share 1 kv head; both heads equal and
     # strictly between the two values
