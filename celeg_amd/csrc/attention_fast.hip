@@ -830,3 +830,4 @@ extern "C" int celeg_attention_decode_bf16(
 #undef CELEG_SPLIT_HEADS
     return CELEG_LAUNCH_RESULT();
 }
+

@@ -318,8 +318,10 @@ def test_q_and_k_are_normalised_before_they_are_rotated(ops, dtype, head_dim):
     batch, keep = build_batch(ops, cache, [StepEntry(slot, 0, [0, 0])])
     row = torch.zeros(2, head_dim)
     row[1, 0], row[1, half] = 3.0, 4.0
-    # (the mean of squares is over head_dim values: scale so that 1/rms is that of {3, 4} alone)
-    row *= math.sqrt(head_dim / 2)
+    # (the mean of squares is over head_dim values: scaled by s = sqrt(head_dim / 2), the row's
+    # 1/rms is that of {3, 4} alone and the result is s times the hand-worked one)
+    s = math.sqrt(head_dim / 2)
+    row *= s
     q = row.to(dtype).to(DEV)
     k, v = q.clone(), q.clone()
     weight = torch.ones(head_dim)
@@ -332,10 +334,10 @@ def test_q_and_k_are_normalised_before_they_are_rotated(ops, dtype, head_dim):
     torch.cuda.synchronize()
     page = int(cache.groups[0].table_host[slot, 0])
     stored_k = kv.k[page, 0, 0, 1].float().cpu()            # [page, layer, head, token, :]
-    bound = 1e-5 if dtype == torch.float32 else 2e-2
+    bound = (1e-5 if dtype == torch.float32 else 2e-2) * s
     for got in (q[1].float().cpu(), stored_k):
-        assert abs(float(got[0]) - QK_NORM_THEN_ROPE[0]) <= bound
-        assert abs(float(got[half]) - QK_NORM_THEN_ROPE[1]) <= bound
+        assert abs(float(got[0]) - s * QK_NORM_THEN_ROPE[0]) <= bound
+        assert abs(float(got[half]) - s * QK_NORM_THEN_ROPE[1]) <= bound
     # the values are stored as they came (transposed inside the page: [.., head_dim, token])
     assert float(kv.v[page, 0, 0, half, 1]) == float(v[1, half])
 
@@ -575,13 +577,17 @@ def test_window_attention_never_reads_pages_it_has_given_back(ops, head_dim, pag
     k = randn(n, kv_heads * head_dim, seed=71, dtype=torch.bfloat16)
     v = randn(n, kv_heads * head_dim, seed=72, dtype=torch.bfloat16)
     slot = cache.open()
-    got, pos = [], 0
+    got, pos, before = [], 0, set()
     for c in [150, 100, 1, 1, 78]:
         assert cache.prepare(slot, pos, c)          # gives back what lies before pos - window + 1
         held = set(cache.pages_held(slot)[0])
         free = [p for p in range(24) if p not in held]
-        kv.k[free] = float("inf")                   # what another request may have left there
+        kv.k[free] = float("inf")                   # what another request may be writing there
         kv.v[free] = float("inf")
+        fresh = sorted(held - before)               # pages handed out now hold someone's old, finite values
+        kv.k[fresh] = randn(len(fresh), *kv.k.shape[1:], seed=73, dtype=torch.bfloat16)
+        kv.v[fresh] = randn(len(fresh), *kv.v.shape[1:], seed=74, dtype=torch.bfloat16)
+        before = held
         batch, keep = build_batch(ops, cache, [StepEntry(slot, pos, [0] * c)])
         qs, ks, vs = (t[pos:pos + c].contiguous() for t in (q, k, v))
         ops.qk_norm_rope_store(qs, ks, vs, None, None, 1e-5, None, 0, heads, kv_heads, head_dim, batch, kv)
