@@ -16,6 +16,8 @@
 // form src/backend/cuda/kernels/attention_gemm.cuh:15-200; split-key CUDA form
 // src/backend/cuda/kernels/attention_paged.cuh:287-487.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -831,3 +833,57 @@ extern "C" int celeg_attention_decode_bf16(
     return CELEG_LAUNCH_RESULT();
 }
 
+// ================================================================ without allocation
+// (declared in no_alloc.h: no counterpart in the reference; for callers that cannot allocate)
+static __device__ __align__(256) float scratch[CELEG_NO_ALLOC_SCRATCH_BYTES / sizeof(float)];
+
+namespace {
+constexpr int NO_ALLOC_MAX_DEVICES = 64;
+float* scratch_of_device[NO_ALLOC_MAX_DEVICES];     // the array's address on each device, once looked up
+std::mutex scratch_lock;
+
+// The address of `scratch` on the current device.  In host code the array's name is only a
+// handle for hipGetSymbolAddress; kernels and copies get the address it returns.
+int scratch_address(float** ptr) {
+    int device = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return static_cast<int>(err);
+    if (device < 0 || device >= NO_ALLOC_MAX_DEVICES) return static_cast<int>(hipErrorInvalidDevice);
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (scratch_of_device[device] == nullptr) {
+        void* address = nullptr;
+        err = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return static_cast<int>(err);
+        if (address == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+        scratch_of_device[device] = static_cast<float*>(address);
+    }
+    *ptr = scratch_of_device[device];
+    return 0;
+}
+}  // namespace
+
+extern "C" int celeg_attention_decode_no_alloc_init(void) {
+    float* ptr = nullptr;
+    return scratch_address(&ptr);
+}
+
+extern "C" int celeg_attention_decode_bf16_no_alloc(
+    const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+    int table_stride, const int* token_slot, const int* positions, void* out, int ldo,
+    int n_rows, int q_heads, int kv_heads, int head_dim, int page_tokens, int n_layers, int layer,
+    float scale, int window, int split_rounds, int n_parts, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (q_heads <= 0 || kv_heads <= 0 || n_parts <= 0 || (head_dim != 64 && head_dim != 128))
+        return static_cast<int>(hipErrorInvalidValue);
+    // partial outputs [rows, heads, parts, head_dim] then (maximum, sum) [rows, heads, parts, 2]
+    const unsigned long long parts = static_cast<unsigned long long>(n_rows) * q_heads * n_parts;
+    if (parts * (head_dim + 2) > CELEG_NO_ALLOC_SCRATCH_BYTES / sizeof(float))
+        return static_cast<int>(hipErrorInvalidValue);
+    float* ws = nullptr;
+    const int code = scratch_address(&ws);
+    if (code) return code;
+    return celeg_attention_decode_bf16(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
+                                       ws, ws + parts * head_dim, n_parts, out, ldo, n_rows, q_heads,
+                                       kv_heads, head_dim, page_tokens, n_layers, layer, scale, window,
+                                       /*whole=*/0, split_rounds, n_parts, stream);
+}
