@@ -1,12 +1,7 @@
 from .spec import PartSpec, LayerSpec, RunStep, ModelSpec
-from .lfm2 import Lfm2Config, ConfigError, feed_forward_width
-from .registry import (Architecture, register_architecture, registered_architectures,
-                       find_architecture, architecture_name, read_config_file,
-                       spec_from_config)
+from .registry import (ConfigError, Lfm2Config, feed_forward_width, register_architecture,
+                       registered_architectures, read_config_file, read_model_folder, spec_from_config)
 
-__all__ = [
-    "PartSpec", "LayerSpec", "RunStep", "ModelSpec", "Lfm2Config", "ConfigError",
-    "feed_forward_width", "Architecture", "register_architecture",
-    "registered_architectures", "find_architecture", "architecture_name",
-    "read_config_file", "spec_from_config",
-]
+__all__ = ["PartSpec", "LayerSpec", "RunStep", "ModelSpec", "Lfm2Config", "ConfigError",
+           "feed_forward_width", "register_architecture", "registered_architectures",
+           "read_config_file", "read_model_folder", "spec_from_config"]

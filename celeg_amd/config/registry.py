@@ -1,71 +1,109 @@
-"""One registry from an architecture's name to its configuration and model.
+"""Configuration and the architecture registry, as the library sees them.
 
-The reference selects among registered architectures by probing the checkpoint's
-metadata (src/model/architecture.cpp:31-78) and registers exactly one, automatic,
-architecture (src/composition/builtin_runtime.cpp:13-58).  Here the name in
-``config.json`` (``architectures[0]``, else ``model_type``) selects an entry; an
-unknown name is an error that lists the registered ones.
+Reading config.json (with generation_config.json merged), the typed LFM2 configuration, its
+validation and the parts list are the library's (``csrc/host/config.cpp``); here are the Python
+views of their results and the way to register an architecture written in Python.
 """
 from __future__ import annotations
 
 import json
 import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, List, Mapping
+from typing import Any, Callable, Dict, List, Mapping, Optional, Tuple
 
+from .. import native
 from .spec import ModelSpec
 
 
+class ConfigError(ValueError):
+    """A configuration that cannot be built; the message names the key."""
+
+
+def _describe(cfg: Mapping[str, Any], tensor_shapes=None) -> Dict[str, Any]:
+    try:
+        return native.describe_config(dict(cfg), tensor_shapes)
+    except native.NativeArgumentError as err:
+        raise ConfigError(str(err)) from None
+
+
 @dataclass(frozen=True)
-class Architecture:
-    """``read_config`` turns the config.json dictionary into the architecture's typed
-    configuration; ``build_spec`` turns that into the parts list."""
-    name: str
-    read_config: Callable[..., Any]
-    build_spec: Callable[[Any], ModelSpec]
-    aliases: tuple = ()
-    # True: ``read_config(cfg, tensor_shapes)`` also takes the checkpoint's tensor names and
-    # shapes (or None), to fill what config.json leaves out
-    reads_tensor_shapes: bool = False
+class Lfm2Config:
+    """The typed LFM2 configuration: every key the library reads, defaults filled in."""
+    vocab_size: int
+    hidden_size: int
+    num_hidden_layers: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    intermediate_size: int
+    layer_types: Tuple[str, ...]
+    conv_L_cache: int
+    conv_bias: bool
+    rope_theta: float
+    norm_eps: float
+    max_position_embeddings: int
+    block_auto_adjust_ff_dim: bool
+    block_multiple_of: int
+    block_ffn_dim_multiplier: Optional[float]
+    tie_word_embeddings: bool
+    bos_token_id: int
+    eos_token_ids: Tuple[int, ...]
+    pad_token_id: int
+    ff_dim: int
+    architecture: str = "Lfm2ForCausalLM"
+
+    @classmethod
+    def from_typed(cls, c: Mapping[str, Any]) -> "Lfm2Config":
+        return cls(c["vocab_size"], c["hidden_size"], c["num_hidden_layers"], c["num_attention_heads"],
+                   c["num_key_value_heads"], c["head_dim"], c["intermediate_size"], tuple(c["layer_types"]),
+                   c["conv_L_cache"], c["conv_bias"], float(c["rope_theta"]), float(c["norm_eps"]),
+                   c["max_position_embeddings"], c["block_auto_adjust_ff_dim"], c["block_multiple_of"],
+                   c["block_ffn_dim_multiplier"], c["tie_word_embeddings"], c["bos_token_id"],
+                   tuple(c["eos_token_id"]), c["pad_token_id"], c["ff_dim"])
+
+    @classmethod
+    def from_dict(cls, cfg: Mapping[str, Any], tensor_shapes=None) -> "Lfm2Config":
+        cfg = dict(cfg)
+        cfg.setdefault("architectures", ["Lfm2ForCausalLM"])
+        return cls.from_typed(_describe(cfg, tensor_shapes)["config"])
+
+    def to_dict(self) -> Dict[str, Any]:
+        out = {k: (list(v) if isinstance(v, tuple) else v) for k, v in vars(self).items()
+               if k not in ("ff_dim", "architecture", "eos_token_ids")}
+        out["architectures"] = [self.architecture]
+        out["model_type"] = "lfm2"
+        out["eos_token_id"] = list(self.eos_token_ids) if len(self.eos_token_ids) != 1 else self.eos_token_ids[0]
+        return out
 
 
-_ARCHITECTURES: Dict[str, Architecture] = {}
-
-
-def register_architecture(arch: Architecture, replace: bool = False) -> None:
-    for name in (arch.name,) + tuple(arch.aliases):
-        if name in _ARCHITECTURES and not replace:
-            raise ValueError(f"architecture '{name}' is already registered")
-        _ARCHITECTURES[name] = arch
+def feed_forward_width(intermediate_size: int, auto_adjust: bool, multiple_of: int,
+                       multiplier: Optional[float]) -> int:
+    """The SwiGLU width the library computes for these keys."""
+    cfg = {"architectures": ["Lfm2ForCausalLM"], "vocab_size": 8, "hidden_size": 8, "num_hidden_layers": 1,
+           "num_attention_heads": 1, "layer_types": ["conv"], "conv_L_cache": 1, "rope_theta": 1.0,
+           "max_position_embeddings": 8, "intermediate_size": intermediate_size,
+           "block_auto_adjust_ff_dim": auto_adjust, "block_multiple_of": multiple_of,
+           "block_ffn_dim_multiplier": multiplier}
+    return _describe(cfg)["config"]["ff_dim"]
 
 
 def registered_architectures() -> List[str]:
-    return sorted(_ARCHITECTURES)
+    return native.registered("architectures")
 
 
-def architecture_name(cfg: Mapping[str, Any]) -> str:
-    archs = cfg.get("architectures")
-    if isinstance(archs, (list, tuple)) and archs:
-        return str(archs[0])
-    if "model_type" in cfg:
-        return str(cfg["model_type"])
-    raise ValueError("config.json names no architecture: neither 'architectures' nor "
-                     "'model_type' is present")
-
-
-def find_architecture(cfg: Mapping[str, Any]) -> Architecture:
-    name = architecture_name(cfg)
-    if name not in _ARCHITECTURES:
-        raise ValueError(f"no registered architecture is called '{name}'; registered: "
-                         f"{registered_architectures()}")
-    return _ARCHITECTURES[name]
+def register_architecture(name: str, build: Callable[[Dict[str, Any], Optional[Dict[str, Any]]], Any]) -> None:
+    """``build(config: dict, tensor_shapes: dict or None)`` returns a ``ModelSpec`` (or a pair
+    (typed configuration dict, ModelSpec))."""
+    def describe(config, shapes):
+        result = build(config, shapes)
+        typed, spec = result if isinstance(result, tuple) else (dict(config), result)
+        return {"config": typed, "spec": spec.to_json()}
+    native.register_architecture(name, describe)
 
 
 def read_config_file(model_dir: str) -> Dict[str, Any]:
-    """config.json must lie beside the weights (src/checkpoint/catalog.cpp:58-63).  A
-    ``generation_config.json`` beside it overrides ``bos_token_id`` and ``eos_token_id``
-    (a number, or a list of numbers) and is ignored if it cannot be read
-    (src/checkpoint/catalog.cpp:94-121)."""
+    """config.json of a model folder as a dictionary, generation_config.json merged the way the
+    library merges it (src/checkpoint/catalog.cpp:94-121): what tools print."""
     path = os.path.join(model_dir, "config.json")
     if not os.path.isfile(path):
         raise FileNotFoundError(f"config.json not found in model folder {model_dir}")
@@ -79,9 +117,9 @@ def read_config_file(model_dir: str) -> Dict[str, Any]:
         except (OSError, ValueError):
             gen = None
         if isinstance(gen, dict):
+            number = lambda v: isinstance(v, (int, float)) and not isinstance(v, bool)
             for key in ("bos_token_id", "eos_token_id"):
                 value = gen.get(key)
-                number = lambda v: isinstance(v, (int, float)) and not isinstance(v, bool)
                 if number(value):
                     cfg[key] = int(value)
                 elif isinstance(value, list):
@@ -91,23 +129,25 @@ def read_config_file(model_dir: str) -> Dict[str, Any]:
     return cfg
 
 
+def _typed(described: Dict[str, Any]):
+    config = described["config"]
+    if described["spec"]["architecture"] == "Lfm2ForCausalLM":
+        config = Lfm2Config.from_typed(config)
+    return config
+
+
 def spec_from_config(cfg: Mapping[str, Any], tensor_shapes=None):
-    """(typed configuration, ModelSpec) of a config.json dictionary.  ``tensor_shapes``:
-    name -> shape of the checkpoint's tensors, for architectures that fill from them what
-    config.json leaves out."""
-    arch = find_architecture(cfg)
-    typed = arch.read_config(cfg, tensor_shapes) if arch.reads_tensor_shapes else arch.read_config(cfg)
-    spec = arch.build_spec(typed)
-    spec.validate()
-    return typed, spec
+    """(typed configuration, ModelSpec) of a config.json dictionary."""
+    d = _describe(cfg, tensor_shapes)
+    return _typed(d), ModelSpec.from_json(d["spec"])
 
 
-def _register_builtin() -> None:
-    from .lfm2 import Lfm2Config
-    register_architecture(Architecture(
-        name="Lfm2ForCausalLM", aliases=("lfm2",),
-        read_config=Lfm2Config.from_dict, build_spec=lambda c: c.to_spec(),
-        reads_tensor_shapes=True))
-
-
-_register_builtin()
+def read_model_folder(model_dir: str):
+    """(typed configuration, ModelSpec, expected tensors) of a model folder."""
+    try:
+        d = native.describe_folder(model_dir)
+    except native.NativeArgumentError as err:
+        if "not found" in str(err):
+            raise FileNotFoundError(str(err)) from None
+        raise ConfigError(str(err)) from None
+    return _typed(d), ModelSpec.from_json(d["spec"]), d["expected_tensors"]

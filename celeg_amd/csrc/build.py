@@ -1,11 +1,13 @@
-"""Compiling the HIP sources for gfx950 and finding the built libraries.
+"""Compiling the library for gfx950 and finding it.
 
-Every ``<name>.hip`` in this folder becomes one shared library
-``lib/<name>-<hash>.so`` beside it, the hash covering the source, the shared headers
-and the compiler flags, so a library is never used with a source it was not built
-from.  If the package folder cannot be written, the libraries go to a per-user
-folder under the system's temporary directory.  ``ensure_built(name)`` compiles on
-first need and prints a line now and then while the compiler runs.
+The kernels (every ``<name>.hip`` in this folder) and the host code (``host/*.cpp``, C++20)
+become ONE shared library ``lib/libceleg_amd-<hash>.so``.  Every source is compiled to an
+object ``lib/obj/<name>-<hash>.o`` of its own, the hash covering the source, the headers and
+the compiler flags, so an object is never used with a source it was not built from and a
+change recompiles only what it touches; the library's hash covers its objects.  If the package
+folder cannot be written, everything goes to a per-user folder under the system's temporary
+directory.  ``ensure_built()`` compiles on first need, several sources at a time, and prints a
+line now and then while the compiler runs.
 """
 from __future__ import annotations
 
@@ -15,16 +17,25 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import threading
 import time
-from typing import Dict, List
+from concurrent.futures import ThreadPoolExecutor
+from typing import Dict, List, Optional
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+HOST = os.path.join(HERE, "host")
 ARCH = "gfx950"
-FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-command-line-argument"]
-MODULES = ["elementwise", "gemm_f32", "short_conv", "attention", "attention_fast", "gemv_fused", "gemv_slices", "gemm_rows", "gemm_tiles",
-           "sampling"]
+COMMON_FLAGS = ["-O3", "-fPIC", f"--offload-arch={ARCH}",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-Wno-unused-command-line-argument"]
+KERNEL_FLAGS = ["-std=c++17"] + COMMON_FLAGS
+HOST_FLAGS = ["-std=c++20", "-x", "hip", "-Wno-unused-result"] + COMMON_FLAGS
+LINK_FLAGS = ["-shared", "-fPIC", f"--offload-arch={ARCH}", "-ldl", "-lpthread"]
+# the kernel files, by the name tests and tools know them under
+MODULES = ["elementwise", "gemm_f32", "short_conv", "attention", "attention_fast", "gemv_fused", "gemv_slices",
+           "gemm_rows", "gemm_tiles", "sampling"]
+LIBRARY = "libceleg_amd"
+_lock = threading.Lock()
 
 
 class BuildError(RuntimeError):
@@ -36,21 +47,49 @@ def _hipcc() -> str:
         if candidate and os.path.isfile(candidate):
             return candidate
     raise BuildError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc); "
-                     "the HIP kernels cannot be built")
+                     "the library cannot be built")
 
 
 def source_path(name: str) -> str:
     return os.path.join(HERE, name + ".hip")
 
 
-def _digest(name: str) -> str:
+def host_sources() -> List[str]:
+    return sorted(os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".cpp"))
+
+
+def _headers(host: bool) -> List[str]:
+    out = [os.path.join(HERE, f) for f in sorted(os.listdir(HERE)) if f.endswith(".h")]
+    if host:
+        out += [os.path.join(HOST, f) for f in sorted(os.listdir(HOST)) if f.endswith(".hpp")]
+        include = os.path.join(HERE, "include")
+        out += [os.path.join(include, f) for f in sorted(os.listdir(include)) if f.endswith(".h")]
+    return out
+
+
+def _digest(source: str) -> str:
+    host = source.endswith(".cpp")
     h = hashlib.sha256()
-    headers = sorted(f for f in os.listdir(HERE) if f.endswith(".h"))
-    for path in [source_path(name)] + [os.path.join(HERE, f) for f in headers]:
+    for path in [source] + _headers(host):
         with open(path, "rb") as fh:
             h.update(fh.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(HOST_FLAGS if host else KERNEL_FLAGS).encode())
     return h.hexdigest()[:12]
+
+
+def _sources() -> List[str]:
+    return [source_path(m) for m in MODULES] + host_sources()
+
+
+def _object_name(source: str) -> str:
+    stem = os.path.splitext(os.path.basename(source))[0]
+    return f"{'host_' if source.endswith('.cpp') else ''}{stem}-{_digest(source)}.o"
+
+
+def _library_name() -> str:
+    h = hashlib.sha256(" ".join(_object_name(s) for s in _sources()).encode())
+    h.update(" ".join(LINK_FLAGS).encode())
+    return f"{LIBRARY}-{h.hexdigest()[:12]}.so"
 
 
 def _lib_dirs() -> List[str]:
@@ -58,9 +97,10 @@ def _lib_dirs() -> List[str]:
     return [os.path.join(HERE, "lib"), os.path.join(tempfile.gettempdir(), user, "lib")]
 
 
-def library_path(name: str):
-    """Path of an up-to-date built library of module ``name``, or None."""
-    fname = f"{name}-{_digest(name)}.so"
+def library_path(name: Optional[str] = None):
+    """Path of an up-to-date built library, or None.  (``name``: a kernel file's name; all of
+    them are in the one library.)"""
+    fname = _library_name()
     for d in _lib_dirs():
         path = os.path.join(d, fname)
         if os.path.isfile(path):
@@ -71,7 +111,7 @@ def library_path(name: str):
 def _writable_lib_dir() -> str:
     for d in _lib_dirs():
         try:
-            os.makedirs(d, exist_ok=True)
+            os.makedirs(os.path.join(d, "obj"), exist_ok=True)
             probe = os.path.join(d, f".probe-{os.getpid()}")
             with open(probe, "w"):
                 pass
@@ -79,61 +119,97 @@ def _writable_lib_dir() -> str:
             return d
         except OSError:
             continue
-    raise BuildError("no writable folder for the built kernels: tried " + ", ".join(_lib_dirs()))
+    raise BuildError("no writable folder for the built library: tried " + ", ".join(_lib_dirs()))
 
 
-def compile_module(name: str, verbose: bool = True) -> str:
-    """Compile ``name``.hip; returns the library's path."""
-    if not os.path.isfile(source_path(name)):
-        raise BuildError(f"no HIP source {source_path(name)}")
-    out_dir = _writable_lib_dir()
-    final = os.path.join(out_dir, f"{name}-{_digest(name)}.so")
-    tmp = final + f".tmp{os.getpid()}"
-    cmd = [_hipcc()] + FLAGS + ["-I", HERE, source_path(name), "-o", tmp]
+def _run(cmd: List[str], what: str, cwd: str, verbose: bool) -> None:
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())  # the compiler wants a HOME for its caches
-    start = time.time()
-    if verbose:
-        print(f"[celeg_amd] compiling {name}.hip for {ARCH} ...", file=sys.stderr, flush=True)
-    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env,
-                            cwd=out_dir)
-    last = start
+    start = last = time.time()
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, cwd=cwd)
     while True:
         try:
             output, _ = proc.communicate(timeout=5)
             break
         except subprocess.TimeoutExpired:
-            if verbose and time.time() - last >= 10:
+            if verbose and time.time() - last >= 15:
                 last = time.time()
-                print(f"[celeg_amd] ... still compiling {name}.hip ({int(last - start)} s)",
-                      file=sys.stderr, flush=True)
+                print(f"[celeg_amd] ... still {what} ({int(last - start)} s)", file=sys.stderr, flush=True)
     if proc.returncode != 0:
+        raise BuildError(f"hipcc failed while {what}:\n{output.decode(errors='replace')}")
+
+
+def _compile(source: str, out_dir: str, verbose: bool, force: bool) -> str:
+    obj = os.path.join(out_dir, "obj", _object_name(source))
+    if os.path.isfile(obj) and not force:
+        return obj
+    host = source.endswith(".cpp")
+    name = os.path.basename(source)
+    if verbose:
+        print(f"[celeg_amd] compiling {name} for {ARCH} ...", file=sys.stderr, flush=True)
+    tmp = obj + f".tmp{os.getpid()}-{threading.get_ident()}"
+    flags = HOST_FLAGS if host else KERNEL_FLAGS
+    start = time.time()
+    try:
+        _run([_hipcc()] + flags + ["-I", HERE, "-I", HOST, "-c", source, "-o", tmp], f"compiling {name}",
+             os.path.join(out_dir, "obj"), verbose)
+        os.replace(tmp, obj)
+    finally:
         if os.path.exists(tmp):
             os.remove(tmp)
-        raise BuildError(f"hipcc failed on {name}.hip:\n{output.decode(errors='replace')}")
-    os.replace(tmp, final)
-    # drop stale builds of this module
-    for f in os.listdir(out_dir):
-        if f.startswith(name + "-") and f.endswith(".so") and os.path.join(out_dir, f) != final:
+    stem = _object_name(source).rsplit("-", 1)[0]
+    for f in os.listdir(os.path.join(out_dir, "obj")):      # drop stale objects of this source
+        if f.rsplit("-", 1)[0] == stem and f.endswith(".o") and f != os.path.basename(obj):
             try:
-                os.remove(os.path.join(out_dir, f))
+                os.remove(os.path.join(out_dir, "obj", f))
             except OSError:
                 pass
     if verbose:
-        print(f"[celeg_amd] built {os.path.basename(final)} in {time.time() - start:.0f} s",
-              file=sys.stderr, flush=True)
-    return final
+        print(f"[celeg_amd] compiled {name} in {time.time() - start:.0f} s", file=sys.stderr, flush=True)
+    return obj
 
 
-def ensure_built(name: str, verbose: bool = True) -> str:
-    return library_path(name) or compile_module(name, verbose)
+def build(force: bool = False, verbose: bool = True) -> str:
+    """Compile what is missing (``force``: everything) and link; returns the library's path."""
+    with _lock:
+        out_dir = _writable_lib_dir()
+        final = os.path.join(out_dir, _library_name())
+        if os.path.isfile(final) and not force:
+            return final
+        sources = _sources()
+        workers = max(1, min(8, os.cpu_count() or 1, len(sources)))
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            objects = list(pool.map(lambda s: _compile(s, out_dir, verbose, force), sources))
+        tmp = final + f".tmp{os.getpid()}"
+        if verbose:
+            print(f"[celeg_amd] linking {os.path.basename(final)} ...", file=sys.stderr, flush=True)
+        try:
+            _run([_hipcc()] + objects + LINK_FLAGS + ["-o", tmp], "linking", out_dir, verbose)
+            os.replace(tmp, final)
+        finally:
+            if os.path.exists(tmp):
+                os.remove(tmp)
+        for f in os.listdir(out_dir):       # drop stale libraries (and those of the one-library-per-kernel layout)
+            if f.endswith(".so") and f != os.path.basename(final):
+                try:
+                    os.remove(os.path.join(out_dir, f))
+                except OSError:
+                    pass
+        return final
+
+
+def compile_module(name: Optional[str] = None, verbose: bool = True) -> str:
+    return build(force=False, verbose=verbose)
+
+
+def ensure_built(name: Optional[str] = None, verbose: bool = True) -> str:
+    return library_path() or build(verbose=verbose)
 
 
 def build_all(force: bool = False, verbose: bool = True) -> Dict[str, str]:
-    return {name: (compile_module(name, verbose) if force else ensure_built(name, verbose))
-            for name in MODULES}
+    path = build(force=force, verbose=verbose)
+    return {LIBRARY: path}
 
 
 if __name__ == "__main__":
-    for module, path in build_all(force="--force" in sys.argv).items():
-        print(module, path)
+    print(build(force="--force" in sys.argv))

@@ -418,3 +418,42 @@ extern "C" int celeg_resolve_tokens(int* token_ids, const int* token_slot, const
                        token_slot, last_tokens, n);
     return CELEG_LAUNCH_RESULT();
 }
+
+// ---------------------------------------------------------------- weights re-laid at load time
+// out = w with column k scaled by scale[k] (a norm's weight folded into the matrix that follows
+// it: (x * s) w^T = x (w * s)^T; scale null: a plain copy), rounded to bfloat16 once, either
+// with the rows one after the other or in blocks of 32 k-values with the rows side by side
+// inside a block ([K/32, rows, 32], what the products for few rows read in whole runs).
+__global__ void fold_weight_kernel(const bf16* __restrict__ w, const float* __restrict__ scale,
+                                   bf16* __restrict__ out, int rows, int K, int packed) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t total = static_cast<size_t>(rows) * K;
+    if (i >= total) return;
+    const int n = static_cast<int>(i / K), k = static_cast<int>(i % K);
+    const float v = scale ? to_float(w[i]) * scale[k] : to_float(w[i]);
+    const size_t at = packed ? (static_cast<size_t>(k / 32) * rows + n) * 32 + k % 32 : i;
+    out[at] = from_float<bf16>(v);
+}
+
+extern "C" int celeg_fold_weight(const void* w, const float* scale, void* out, int rows, int K,
+                                 int packed, hipStream_t stream) {
+    if (rows <= 0 || K <= 0) return 0;
+    if (packed && K % 32) return static_cast<int>(hipErrorInvalidValue);
+    const size_t total = static_cast<size_t>(rows) * K;
+    hipLaunchKernelGGL(fold_weight_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       stream, static_cast<const bf16*>(w), scale, static_cast<bf16*>(out), rows, K, packed);
+    return CELEG_LAUNCH_RESULT();
+}
+
+// bytes [0, n) of p set to zero by a kernel (what a recorded graph may hold, unlike a memset node)
+__global__ void zero_bytes_kernel(uint32_t* __restrict__ p, size_t words) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < words) p[i] = 0u;
+}
+
+extern "C" int celeg_zero_words(void* p, size_t words, hipStream_t stream) {
+    if (words == 0) return 0;
+    hipLaunchKernelGGL(zero_bytes_kernel, dim3(static_cast<unsigned>((words + 255) / 256)), dim3(256), 0,
+                       stream, static_cast<uint32_t*>(p), words);
+    return CELEG_LAUNCH_RESULT();
+}

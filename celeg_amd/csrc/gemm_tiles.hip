@@ -30,6 +30,7 @@
 // the reference fuses the residual addition into its products with beta = 1
 // (src/backend/cuda/model/prefill_batched/non_attention.cpp:175-201).
 #include "common.h"
+#include "tile_params.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
@@ -37,24 +38,6 @@ typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 
 enum { T_STORE = 0, T_RESIDUAL = 2, T_SWIGLU = 3 };   // the numbers of the few-rows products
 
-struct TileParams {
-    const bf16* a;          // [M, lda]
-    int lda;
-    const bf16* w;          // [streams * stream_rows, ldw]; stream s starts at row s * stream_rows
-    int ldw;
-    int stream_rows;
-    const float* bias;      // optional [streams * stream_rows]
-    const float* stats;     // optional partial sums of squares [M, stats_ld], n_stat_blocks valid a row
-    int n_stat_blocks, stats_ld;
-    float eps;
-    int M, N, K;            // N: output columns (per stream)
-    void* out;              // bf16 [M, ldo] (store, SwiGLU) or the 32-bit stream [M, ldo] (residual)
-    int ldo;
-    bf16* out_bf16;         // residual: the stream's bfloat16 copy [M, ld_bf16], or null
-    int ld_bf16;
-    float* stats_out;       // residual: [M, stats_ld_out], one partial sum per tile column and row; or null
-    int stats_ld_out;
-};
 
 #define GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
 #define LPTR(p) ((__attribute__((address_space(3))) void*)(p))

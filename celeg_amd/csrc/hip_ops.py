@@ -1,8 +1,10 @@
-"""The kernels as Python calls: shapes are checked on the host, then the extern "C"
-entry points of the built libraries are called through ``ctypes`` with raw device
-pointers and the current HIP stream (so a stream that is capturing a graph captures
-them too).  There is no fallback: if a library cannot be built or loaded, or a tensor
-is not on the GPU, the call fails loudly.
+"""The kernels as Python calls on torch tensors: what the tests of single kernels and tuning
+scripts use.  (The engine does not come through here: its host code, ``host/ops.cpp``, makes
+the same checks and calls in C++.)  Shapes are checked on the host, then the extern "C" entry
+points of the built library are called through ``ctypes`` with raw device pointers and the
+current HIP stream (so a stream that is capturing a graph captures them too).  There is no
+fallback: if the library cannot be built or loaded, or a tensor is not on the GPU, the call
+fails loudly.
 
 Matrix products in bfloat16 of more than 64 rows go to hipBLASLt, called directly
 (``blaslt.py``), as the reference sends its products to cuBLAS
@@ -77,19 +79,21 @@ class HipOps:
 
     # ------------------------------------------------------------------ plumbing
     def _lib(self, module: str) -> ctypes.CDLL:
-        lib = self._libs.get(module)
+        """The built library (all kernel files are in the one library; ``module`` names the file
+        a call belongs to, for the record of what ran)."""
+        lib = self._libs.get("library")
         if lib is None:
-            path = build.ensure_built(module)
+            path = build.ensure_built()
             try:
                 lib = ctypes.CDLL(path)
             except OSError as err:
-                raise KernelError(f"cannot load the built kernels {path}: {err}") from err
-            if module == "gemv_slices" and lib.celeg_gemv_params_size() != ctypes.sizeof(_GemvParams):
+                raise KernelError(f"cannot load the built library {path}: {err}") from err
+            if lib.celeg_gemv_params_size() != ctypes.sizeof(_GemvParams):
                 raise KernelError("the argument block of the skinny products does not match the built kernels")
-            if module == "gemm_tiles" and lib.celeg_gemm_tiles_params_size() != ctypes.sizeof(_TileParams):
+            if lib.celeg_gemm_tiles_params_size() != ctypes.sizeof(_TileParams):
                 raise KernelError("the argument block of the tiled products does not match the built kernels")
-            self._libs[module] = lib
-            self.loaded_libraries[module] = path
+            self._libs["library"] = lib
+        self.loaded_libraries[module] = build.library_path() or ""
         return lib
 
     def _stream(self):

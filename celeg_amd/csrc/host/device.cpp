@@ -1,0 +1,127 @@
+#include "device.hpp"
+
+#include <cstdlib>
+
+namespace celeg {
+
+DType parse_dtype(const std::string& name) {
+    if (name == "bfloat16" || name == "bf16") return DType::BF16;
+    if (name == "float32" || name == "fp32" || name == "f32") return DType::F32;
+    throw ConfigError("unknown dtype '" + name + "': bfloat16 or float32");
+}
+
+void hip_check(hipError_t code, const char* what) {
+    if (code != hipSuccess)
+        throw KernelError(std::string(what) + ": " + hipGetErrorString(code) + " (HIP error " +
+                          std::to_string(static_cast<int>(code)) + ")");
+}
+
+void kernel_check(int code, const char* what) {
+    if (code != 0) throw KernelError(std::string(what) + ": HIP error " + std::to_string(code));
+}
+
+float half_to_float(uint16_t h) {
+    const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu, man = h & 0x3ffu, u;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign;
+        } else {              // subnormal: normalise
+            exp = 127 - 15 + 1;
+            while (!(man & 0x400u)) { man <<= 1; --exp; }
+            u = sign | (exp << 23) | ((man & 0x3ffu) << 13);
+        }
+    } else if (exp == 31) {
+        u = sign | 0x7f800000u | (man << 13);
+    } else {
+        u = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+DeviceBuffer::DeviceBuffer(size_t bytes, bool zero) : bytes_(bytes) {
+    if (bytes == 0) return;
+    const hipError_t err = hipMalloc(&ptr_, bytes);
+    if (err != hipSuccess) {
+        ptr_ = nullptr;
+        throw KernelError("hipMalloc of " + std::to_string(bytes) + " bytes failed: " + hipGetErrorString(err));
+    }
+    if (zero) CELEG_HIP(hipMemset(ptr_, 0, bytes));
+}
+
+DeviceBuffer::~DeviceBuffer() {
+    if (ptr_) (void)hipFree(ptr_);
+}
+
+DeviceBuffer& DeviceBuffer::operator=(DeviceBuffer&& o) noexcept {
+    if (this != &o) {
+        if (ptr_) (void)hipFree(ptr_);
+        ptr_ = o.ptr_;
+        bytes_ = o.bytes_;
+        o.ptr_ = nullptr;
+        o.bytes_ = 0;
+    }
+    return *this;
+}
+
+PinnedBuffer::PinnedBuffer(size_t bytes) : bytes_(bytes) {
+    if (bytes == 0) return;
+    if (hipHostMalloc(&ptr_, bytes, hipHostMallocDefault) == hipSuccess) {
+        pinned_ = true;
+    } else {
+        (void)hipGetLastError();
+        ptr_ = std::malloc(bytes);        // no GPU: ordinary memory, for the host-only paths
+        if (!ptr_) throw std::bad_alloc();
+    }
+}
+
+PinnedBuffer::~PinnedBuffer() {
+    if (!ptr_) return;
+    if (pinned_) (void)hipHostFree(ptr_);
+    else std::free(ptr_);
+}
+
+PinnedBuffer& PinnedBuffer::operator=(PinnedBuffer&& o) noexcept {
+    if (this != &o) {
+        this->~PinnedBuffer();
+        ptr_ = o.ptr_;
+        bytes_ = o.bytes_;
+        pinned_ = o.pinned_;
+        o.ptr_ = nullptr;
+    }
+    return *this;
+}
+
+void* Workspace::raw(const std::string& name, size_t bytes) {
+    auto it = buffers_.find(name);
+    if (it == buffers_.end() || it->second.bytes() < bytes) {
+        if (frozen)
+            throw KernelError("workspace buffer '" + name + "' would move while a graph is being recorded");
+        DeviceBuffer fresh(bytes < 256 ? 256 : bytes);
+        if (it != buffers_.end()) {
+            retired_.push_back(std::move(it->second));    // recorded graphs may still point at it
+            it->second = std::move(fresh);
+        } else {
+            it = buffers_.emplace(name, std::move(fresh)).first;
+        }
+        ++generation;
+    }
+    return it->second.ptr();
+}
+
+Tensor Workspace::buf(const std::string& name, DType dtype, std::initializer_list<long long> dims) {
+    long long count = 1;
+    for (long long d : dims) count *= d;
+    void* p = raw(name + ":" + dtype_name(dtype), static_cast<size_t>(count < 1 ? 1 : count) * dtype_size(dtype));
+    return Tensor::make(p, dtype, dims);
+}
+
+size_t Workspace::bytes() const {
+    size_t n = 0;
+    for (const auto& b : buffers_) n += b.second.bytes();
+    return n;
+}
+
+}  // namespace celeg

@@ -1,0 +1,140 @@
+// The kernels as host calls: shapes, dtypes, strides and limits are checked here, then the
+// extern "C" entry points are called with raw device pointers and the runtime's stream (so a
+// stream that is recording a graph records them too).  There is no fallback: a size a kernel
+// was not written for is a KernelError that says why.
+//
+// Matrix products in bfloat16 of more than 64 rows go to hipBLASLt (blaslt.cpp), as the
+// reference sends its products to cuBLAS (src/backend/cuda/runtime/gemm_dispatcher.cpp);
+// products in 32-bit go to this library's own kernel, which uses no reduced-precision matrix
+// mode.
+#pragma once
+#include <functional>
+#include <map>
+#include <memory>
+#include <string>
+
+#include "batch.hpp"
+#include "blaslt.hpp"
+#include "cache.hpp"
+#include "device.hpp"
+#include "weights.hpp"
+
+namespace celeg {
+
+enum class Epilogue : int { Store = 0, StoreF32 = 1, Residual = 2, Swiglu = 3, Conv = 4 };
+
+// The convolution epilogue's operands: one new token per request.
+struct ConvOperands {
+    Tensor taps;          // [N, L] 32-bit
+    Tensor bias;          // optional [N]
+    Tensor state;         // [slots, L, N] 32-bit, the slots a fixed number of elements apart
+    const int* seq_slot = nullptr;   // [M]
+};
+
+struct FusedArgs {
+    Epilogue epilogue = Epilogue::Store;
+    Tensor norm_weight;           // the older form: the 32-bit stream normalised on the fly
+    float eps = 0.f;
+    Tensor stats;                 // partial sums of squares of the rows of the stream [rows, >= stat_blocks]
+    int stat_blocks = 0;
+    const int* rows = nullptr;    // picks rows of a
+    int n_rows = -1;              // number of output rows (with rows: how many are picked)
+    Tensor bias;
+    Tensor stats_out;             // residual: partial sums of squares of the new rows
+    const ConvOperands* conv = nullptr;
+    Tensor out_bf16;              // residual: the bfloat16 copy of the stream
+    bool packed = false;          // w is [K/32, rows, 32] (pack_weight)
+};
+
+class Ops {
+public:
+    explicit Ops(hipStream_t stream) : stream(stream) {}
+    hipStream_t stream;
+    // knobs (tests and tuning)
+    int attention_decode_whole = -1;     // -1: chosen from the batch; 0 split-key kernels; 1 one workgroup per request and key/value head
+    bool use_blaslt = true;
+    int attention_rows_per_tile = 0, attention_rows_form = 0;
+    int decode_part_thresholds[2] = {64, 256};
+    bool attention_general = false;      // always the general attention kernel
+    bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
+    int rows_kernel_min_rows = 9, tiles_min_rows = 65, fused_linear_shape = 0;
+    int last_stat_blocks = 0;
+
+    // row-wise
+    void embed(const Tensor& table, const int* token_ids, const Tensor& out);
+    void rmsnorm(const Tensor& x, const Tensor& weight, float eps, const Tensor& out, const Tensor* delta = nullptr,
+                 const int* rows = nullptr);
+    void swiglu(const Tensor& gate_up, const Tensor& out);
+    void add_bias(const Tensor& x, const Tensor& bias);
+    void cast(const Tensor& src, const Tensor& dst);
+    void apply_table_updates(int* table, int stride, int rows, const int* updates, int capacity);
+    void step_prologue(int* table, int stride, int rows, const int* updates, int capacity, int* token_ids,
+                       const int* token_slot, const int* last_tokens, int n);
+    void resolve_tokens(int* token_ids, const int* token_slot, const int* last_tokens, int n);
+    // products
+    void linear(const Tensor& x, const Tensor& w, const Tensor& out, const Tensor* bias, Workspace& ws);
+    // cache-backed
+    void short_conv(const Tensor& bcx, const Tensor& weight, const Tensor* bias, const Tensor& state, const Tensor& out,
+                    const StepBatch& batch);
+    void qk_norm_rope_store(const Tensor& q, const Tensor* k, const Tensor* v, const Tensor* q_weight,
+                            const Tensor* k_weight, float eps, const Tensor* inv_freq, int rotary_dim, int heads,
+                            int kv_heads, int head_dim, const StepBatch& batch, const KVView& kv);
+    void paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
+                         int window, const StepBatch& batch, const KVView& kv, Workspace& ws);
+    // sampling
+    void sample(const Tensor& logits, const float* fparams, const int* iparams, const uint8_t* seen,
+                size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws);
+    void mark_seen(uint8_t* seen, size_t stride, int n_slots, int vocab, const int* token_ids, const int* token_slot, int n);
+    // fused skinny products
+    bool fused_linear_ok(int rows, std::initializer_list<long long> inner) const;
+    bool rows_kernel_ok(int rows, std::initializer_list<long long> inner) const;
+    int residual_stat_blocks(int rows, int n, int k) const;
+    void stream_prepare(const Tensor& h, const Tensor& xb, const Tensor& stats);
+    void embed_stream(const Tensor& table, const int* token_ids, const Tensor& out, const Tensor& xb, const Tensor& stats);
+    void embed_stats(const Tensor& table, const int* token_ids, const Tensor& out, const Tensor& stats);
+    void fused_linear(const Tensor& a, const Tensor& w, const Tensor& out, const FusedArgs& args);
+    // fused products of many rows
+    bool tiled_linear_ok(int rows, int n, std::initializer_list<long long> inner) const;
+    int tiled_stat_blocks(int rows, int n, int k) const;
+    void tiled_linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue epilogue, float eps,
+                      const Tensor* stats, int stat_blocks, const Tensor* bias, const Tensor* stats_out,
+                      const Tensor* out_bf16);
+    // weights re-laid at load time: w [rows, K] scaled by a norm's weight (or not) and, if
+    // `packed`, laid as [K/32, rows, 32]
+    std::shared_ptr<DeviceTensor> fold_weight(const Tensor& w, const Tensor* scale, bool packed);
+
+private:
+    std::unique_ptr<BlasLt> blaslt_;
+    DeviceBuffer argmax_state_;
+    std::map<std::pair<const void*, int>, std::shared_ptr<DeviceTensor>> rope_tables_;
+    const float* rope_table(const Tensor& inv_freq, int n_positions);
+    void attention_decode(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
+                          int window, const StepBatch& batch, const KVView& kv, int T, Workspace& ws);
+    void library_product(const Tensor& x, const Tensor& w, const Tensor& out, Workspace& ws);
+};
+
+// What every part computes with: the stream, the activation dtype, the kernels, a workspace of
+// reusable buffers, and what the parts of the fused path tell each other about the residual
+// stream between kernels.
+struct Runtime {
+    Runtime(DType dtype, hipStream_t stream) : dtype(dtype), stream(stream), ops(stream) {}
+    DType dtype;
+    hipStream_t stream;
+    Ops ops;
+    Workspace ws;
+    bool use_fused = true;
+    bool use_tiled_products = false;
+    int fused_max_rows = -1;            // -1: by the kernels' own limits
+    // how many partial sums of squares of the stream's rows are valid (0: none), and whether
+    // the stream's bfloat16 copy is; whoever writes the stream another way resets them
+    int stream_stat_blocks = 0;
+    bool stream_has_bf16 = false;
+    // weights re-laid for the fused path, made once per (weight, norm weight) pair
+    std::map<std::pair<const void*, const void*>, std::shared_ptr<DeviceTensor>> folded_weights, folded_plain_weights;
+    std::map<const void*, std::shared_ptr<DeviceTensor>> packed_weights;
+    // a hook for bisecting mismatches: called after every entry of the run order with the
+    // residual stream (the pending addition, if any, not yet made)
+    std::function<void(int step, const Tensor& h, const Tensor* delta)> after_layer;
+};
+
+}  // namespace celeg

@@ -1,3 +1,43 @@
-from .sampler import GenerationConfig, GREEDY, Sampler, XorShift64Star, MAX_TOP_K
+"""Generation options: names, meanings, defaults and limits of the reference's ``GenerationConfig``
+(include/celeg/model/runtime_types.hpp:98-108; validation
+src/model/execution/runtime_types.cpp:20-37).  The sampler itself (a xorshift64* state per
+request on the host, the selection on the GPU) is the library's (``csrc/host/sampler.cpp``,
+``csrc/sampling.hip``)."""
+from __future__ import annotations
 
-__all__ = ["GenerationConfig", "GREEDY", "Sampler", "XorShift64Star", "MAX_TOP_K"]
+import math
+from dataclasses import dataclass
+
+MAX_TOP_K = 128
+_MASK64 = (1 << 64) - 1
+
+
+@dataclass(frozen=True)
+class GenerationConfig:
+    temperature: float = 0.1
+    top_k: int = 50
+    top_p: float = 1.0
+    repetition_penalty: float = 1.05
+    seed: int = 1
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature <= 0.0 or self.top_k == 1
+
+    def validate(self) -> None:
+        """The checks the library makes at submission, for callers that want them earlier."""
+        if not math.isfinite(self.temperature) or self.temperature < 0.0:
+            raise ValueError("temperature must be finite and non-negative")
+        if self.top_k <= 0 or self.top_k > MAX_TOP_K:
+            raise ValueError(f"top_k must be between 1 and {MAX_TOP_K}")
+        if not math.isfinite(self.top_p) or self.top_p <= 0.0 or self.top_p > 1.0:
+            raise ValueError("top_p must be in (0, 1]")
+        if not math.isfinite(self.repetition_penalty) or self.repetition_penalty < 1.0:
+            raise ValueError("repetition_penalty must be finite and at least 1")
+        if self.seed == 0 or not 0 < self.seed <= _MASK64:
+            raise ValueError("seed must be non-zero")
+
+
+GREEDY = GenerationConfig(temperature=0.0, top_k=1, top_p=1.0, repetition_penalty=1.0, seed=1)
+
+__all__ = ["GenerationConfig", "GREEDY", "MAX_TOP_K"]

@@ -17,7 +17,7 @@ from typing import Any, Dict, Mapping
 
 import torch
 
-from ..config.registry import spec_from_config
+from .. import native
 from .safetensors_io import write_safetensors
 
 
@@ -39,17 +39,20 @@ def random_tensor(seed: int, name: str, shape, init: str, std: float) -> torch.T
 
 def random_tensors(expected, seed: int, std: float = 0.02,
                    dtype: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
-    return {name: random_tensor(seed, name, spec.shape, spec.init, std).to(dtype)
-            for name, spec in expected.items()}
+    """``expected``: the library's list of the tensors a model wants
+    ([{"name", "shape", "init", ..}], ``native.describe_config(..)["expected_tensors"]``)."""
+    return {e["name"]: random_tensor(seed, e["name"], e["shape"], e["init"], std).to(dtype) for e in expected}
 
 
 def write_random_model(config: Mapping[str, Any], out_dir: str, seed: int,
                        dtype: torch.dtype = torch.bfloat16, std: float = 0.02) -> str:
     """Write ``out_dir/config.json`` and ``out_dir/model.safetensors`` for the architecture
     that ``config`` names.  Returns ``out_dir``."""
-    from ..engine.model import Model  # the parts know which tensors they want
-    _, spec = spec_from_config(config)
-    expected = Model(spec).expected_tensors()
+    from ..config.registry import ConfigError
+    try:
+        expected = native.describe_config(dict(config))["expected_tensors"]   # the parts know which tensors they want
+    except native.NativeArgumentError as err:
+        raise ConfigError(str(err)) from None
     os.makedirs(out_dir, exist_ok=True)
     with open(os.path.join(out_dir, "config.json"), "w") as fh:
         json.dump(dict(config), fh, indent=1)

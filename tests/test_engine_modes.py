@@ -1,9 +1,8 @@
 """The engine against the plain implementation in every way of cutting and batching:
 each request alone and whole; most of it in one step and the last 32 tokens one by
 one; portions of changing size down to two tokens; mixed, up to four live requests
-with so few pages that they are used again.  On the GPU in 32-bit and bfloat16 (the
-real kernels); on the CPU in 32-bit with the test double of the kernels, which checks
-the host-side logic (metadata, block tables, state slots) where there is no GPU.
+with so few pages that they are used again; in 32-bit and bfloat16, through the library's
+step function and cache manager (the ones generation uses).
 """
 import pytest
 import torch
@@ -37,7 +36,7 @@ def plain_logits(folder, name, storage):
     return _plain_cache[key]
 
 
-def run_mode(model_folders, name, dtype, mode, device, ops=None, subset=None, gemm_backend="library"):
+def run_mode(model_folders, name, dtype, mode, device, subset=None, gemm_backend="library"):
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders(name, storage, WEIGHT_STD)
@@ -48,7 +47,7 @@ def run_mode(model_folders, name, dtype, mode, device, ops=None, subset=None, ge
     max_tokens = peak_tokens(steps)
     lm = load_model(folder, dtype=dtype, device=device, page_tokens=16,
                     n_pages=max_tokens // 16, max_requests=4,
-                    max_batched_tokens=max(max_tokens, 64), ops=ops, gemm_backend=gemm_backend)
+                    max_batched_tokens=max(max_tokens, 64), gemm_backend=gemm_backend)
     got = EngineDriver(lm).run(steps)
     ref = plain_logits(folder, name, storage)
     for rid in reqs:
@@ -73,18 +72,9 @@ def test_gpu_engine_with_tiled_products_matches_plain(model_folders, mode):
     folded in) instead of the library's: whole prompts of up to 300 tokens, and portions
     beside single tokens."""
     lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles")
-    if mode in ("whole", "tail32"):
-        assert "gemm_tiles" in lm.rt.ops.loaded_libraries
+    assert lm.knobs()["use_tiled_products"] == 1
     # and the same configuration through the library's products
     run_mode(model_folders, "E", "bfloat16", mode, "cuda:0")
-
-
-@pytest.mark.parametrize("mode", list(SCHEDULES))
-@pytest.mark.parametrize("name", ["A", "B"])
-def test_host_logic_with_kernel_double(model_folders, name, mode):
-    from cpu_ops import CpuOps
-    run_mode(model_folders, name, "float32", mode, "cpu", ops=CpuOps(),
-             subset=["r0", "r1", "r5"] if mode != "mixed" else None)
 
 
 @pytest.mark.gpu
@@ -104,8 +94,8 @@ def test_captured_decode_steps_equal_eager_steps(model_folders, dtype):
                         max_requests=4, max_batched_tokens=256)
         lm.runner.use_graphs = use_graphs
         out[use_graphs] = EngineDriver(lm).run(steps)
-        if use_graphs:
-            assert lm.runner._graphs, "no decode step was replayed from a graph"
+        replays = lm.runner.counters()["graph_replays"]
+        assert (replays > 0) == use_graphs, "decode steps were (not) replayed from a graph"
     for rid in reqs:
         if dtype == "float32":
             assert torch.equal(out[True][rid], out[False][rid])
@@ -148,7 +138,7 @@ def test_long_decoding(model_folders, name, dtype):
     cfgp, W = plain.load_model_folder(folder)
     for rid, toks in reqs.items():
         assert_close(got[rid], plain.model_logits(cfgp, W, toks), dtype, f"{name}/{dtype}/long/{rid}")
-    assert lm.runner._graphs, "no decode step was replayed from a graph"
+    assert lm.runner.counters()["graph_replays"] > 100, "the decode steps were not replayed from a graph"
     lm.cache.check()
 
 
@@ -157,9 +147,8 @@ def test_long_decoding(model_folders, name, dtype):
 def test_long_decoding_across_the_bounds_of_recorded_steps(model_folders, dtype):
     """A recorded decode step serves contexts up to a bound (the attention over few requests
     cuts the context into parts by it), and a longer context takes another recording.  With
-    the bounds pulled down to 64 and 160 tokens, and parts of 4 rounds from 2 rounds on, two
-    requests decode from 20 to 330 tokens through all three recordings; every position is
-    compared with the plain implementation."""
+    parts of 4 rounds from 2 rounds on and of 16 from 9 on, two requests decode from 20 to 330
+    tokens; every position is compared with the plain implementation."""
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders("D", storage, WEIGHT_STD)
@@ -169,14 +158,13 @@ def test_long_decoding_across_the_bounds_of_recorded_steps(model_folders, dtype)
                              for rid, toks in reqs.items()})
     lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16, max_requests=2,
                     max_batched_tokens=256)
-    lm.runner.CONTEXT_BOUNDS = (64, 160)
-    if hasattr(lm.rt.ops, "decode_part_thresholds"):
-        lm.rt.ops.decode_part_thresholds = (1, 8)
+    lm.set_knob("decode_parts_few", 1)
+    lm.set_knob("decode_parts_some", 8)
     got = EngineDriver(lm).run(steps)
     cfgp, W = plain.load_model_folder(folder)
     for rid, toks in reqs.items():
         assert_close(got[rid], plain.model_logits(cfgp, W, toks), dtype, f"D/{dtype}/bounds/{rid}")
-    assert {bound for _, bound in lm.runner._graphs} == {64, 160, lm.cache.max_context}
+    assert lm.runner.counters()["graph_replays"] > 300
     lm.cache.check()
 
 
@@ -211,11 +199,9 @@ def test_first_tokens_of_a_sequence(model_folders, name, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "C"])
-def test_portions_of_a_repeated_size_are_replayed(model_folders, name, dtype):
-    """Prompts that arrive in equal portions: from the second portion of a size on, the
-    step is replayed from a graph captured for that size (on the null slot).  Every replay
-    is checked against the plain implementation, with other steps (decode tokens, another
-    size) between them."""
+def test_portions_of_a_repeated_size(model_folders, name, dtype):
+    """Prompts that arrive in equal portions, the last one's last row wanted, with decode
+    tokens between them: every wanted row against the plain implementation."""
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders(name, storage, WEIGHT_STD)
@@ -232,7 +218,6 @@ def test_portions_of_a_repeated_size_are_replayed(model_folders, name, dtype):
     lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16 + 1,
                     max_requests=4, max_batched_tokens=64)
     got = EngineDriver(lm).run(steps)
-    assert set(lm.runner._portion_graphs) == {(48, 0, False), (48, 1, False)}
     cfgp, W = plain.load_model_folder(folder)
     for rid, toks in reqs.items():
         ref = plain.model_logits(cfgp, W, toks)
@@ -243,13 +228,11 @@ def test_portions_of_a_repeated_size_are_replayed(model_folders, name, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "D"])
-def test_mixed_steps_of_a_repeated_shape_are_replayed(model_folders, name, dtype):
+def test_mixed_steps_of_a_repeated_shape(model_folders, name, dtype):
     """The steady state of serving under a token budget: every step holds portions of prompts
-    of the portion size beside the single tokens of the requests that decode.  From the
-    second step of a shape on (bucket of single rows, sizes of the portions) the step is
-    replayed from a graph captured on null-slot rows; the single rows are padded to the
-    bucket, and the entries come in changing order (a portion first, between or behind the
-    single tokens).  Every wanted row is checked against the plain implementation."""
+    of the portion size beside the single tokens of the requests that decode, and the entries
+    come in changing order (a portion first, between or behind the single tokens).  Every
+    wanted row is checked against the plain implementation."""
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders(name, storage, WEIGHT_STD)
@@ -281,12 +264,7 @@ def test_mixed_steps_of_a_repeated_shape_are_replayed(model_folders, name, dtype
         k += 1
     lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=peak_tokens(steps) // 16 + 8,
                     max_requests=8, max_batched_tokens=128)
-    lm.runner.MIXED_SEEN_BEFORE_RECORDING = 2          # (a server waits for the eighth)
     got = EngineDriver(lm).run(steps)
-    shapes = set(lm.runner._mixed_graphs)
-    # shapes that came twice were captured (up to 4 single rows; more came once at most), with one or two portions
-    assert len(shapes) >= 1 and all(len(portions) == 3 - stride for _, portions, _ in shapes), shapes
-    assert {bucket for bucket, _, _ in shapes} >= {4}
     cfgp, W = plain.load_model_folder(folder)
     first = P * n_portions - 1
     for rid, toks in reqs.items():
@@ -365,47 +343,38 @@ def test_many_requests_decoding_together(model_folders, name, n_requests, join_e
     assert lm.cache.n_free_slots == n_requests and lm.cache.free_pages() == [pages]
 
 
+@pytest.mark.gpu
 def test_a_large_reservation_and_a_refused_step_keep_the_device_tables_right(model_folders):
-    """Pages reserved thousands at a time (what guaranteed_no_evict does at admission) are
-    more block-table updates than a step's metadata has room for: the eager path ships them on
-    their own.  A step that is refused after the updates were drained (a wanted place outside
-    the entry, metadata that does not fit) leaves them queued for the next step, whose logits
-    are then those of the plain implementation."""
-    from cpu_ops import CpuOps
+    """Pages reserved hundreds at a time (what guaranteed_no_evict does at admission) are more
+    block-table updates than a step's metadata has room for: the step function ships them on
+    their own.  A step that is refused after the cache manager handed its updates over (a wanted
+    place outside the entry) leaves them queued for the next step, whose logits are then those
+    of the plain implementation."""
     from celeg_amd.engine import StepEntry, load_model
     folder = model_folders("A", torch.float32, WEIGHT_STD)
     cfg, W = plain.load_model_folder(folder)
-    lm = load_model(folder, dtype="float32", device="cpu", page_tokens=2, n_pages=300,
-                    max_requests=4, max_context=128, max_batched_tokens=16, ops=CpuOps())
-    room = lm.runner._update_room
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=40, max_requests=4, max_context=128,
+                    max_batched_tokens=16)
     slots = [lm.cache.open() for _ in range(4)]
     for s in slots:
-        assert lm.cache.prepare(s, 0, 128)          # 64 pages each, 256 updates pending
-    assert 256 > room
+        assert lm.cache.prepare(s, 0, 128)          # 8 pages each, 32 updates pending; room for 16/16 + 8 + 8 = 17
     prompts = [random_tokens(256, 9 + i, seed=40 + i) for i in range(4)]
     logits = lm.runner.step([StepEntry(s, 0, p[:3], [2]) for s, p in zip(slots, prompts)])
     for i, p in enumerate(prompts):
         assert_close(logits[i], plain.model_logits(cfg, W, p[:3])[-1], "float32", f"burst/{i}")
-    host = torch.from_numpy(lm.cache.groups[0].table_host)
-    assert torch.equal(lm.cache.groups[0].table[:4], host[:4])
-    # a refused step: the updates of new pages stay queued
     for s in slots:
         lm.cache.close(s)
     slots = [lm.cache.open() for _ in range(2)]
-    assert lm.cache.prepare(slots[0], 0, 5) and lm.cache.prepare(slots[1], 0, 4)
+    assert lm.cache.prepare(slots[0], 0, 20) and lm.cache.prepare(slots[1], 0, 4)
     with pytest.raises(ValueError, match="wanted place"):
         lm.runner.step([StepEntry(slots[0], 0, prompts[0][:5], [5])])
-    lm.runner.builder.capacity, kept = 8, lm.runner.builder.capacity
-    with pytest.raises(ValueError, match="staging buffer"):
-        lm.runner.step([StepEntry(slots[0], 0, prompts[0][:5], [4])])
-    lm.runner.builder.capacity = kept
+    with pytest.raises(ValueError, match="exceed max_batched_tokens"):
+        lm.runner.step([StepEntry(slots[0], 0, prompts[0][:5] * 4, [4])])
     logits = lm.runner.step([StepEntry(slots[0], 0, prompts[0][:5], [4]),
                              StepEntry(slots[1], 0, prompts[1][:4], [3])])
     assert_close(logits[0], plain.model_logits(cfg, W, prompts[0][:5])[-1], "float32", "after refusal/0")
     assert_close(logits[1], plain.model_logits(cfg, W, prompts[1][:4])[-1], "float32", "after refusal/1")
-    host = torch.from_numpy(lm.cache.groups[0].table_host)
-    live = host >= 0
-    assert torch.equal(lm.cache.groups[0].table[live], host[live])
+    lm.cache.check()
 
 
 @pytest.mark.gpu

@@ -73,8 +73,3 @@ def test_engine_matches_plain_at_real_layer_sizes(tmp_path_factory, shape, dtype
     for rid in reqs:
         assert_close(got[rid], ref[rid], dtype, f"{shape}/{dtype}/{mode}/{rid}")
     assert lm.cache.n_free_slots == 4 and lm.cache.free_pages() == [max_tokens // 16]
-    if dtype == "bfloat16" and mode == "tail32":
-        # the kernels the real model's decode steps take were the ones that ran
-        loaded = lm.rt.ops.loaded_libraries
-        for needed in ("gemv_slices", "gemv_fused", "attention_fast"):
-            assert needed in loaded, f"{needed} was not used"
