@@ -58,19 +58,6 @@ SHAPES = {
 }
 
 
-def weight_bytes(model) -> int:
-    seen = {}
-    for _, part in model.named_parts():
-        for value in vars(part).values():
-            if hasattr(value, "data_ptr") and hasattr(value, "element_size"):
-                key = value.untyped_storage().data_ptr() if hasattr(value, "untyped_storage") \
-                    else value.data_ptr()
-                size = value.untyped_storage().nbytes() if hasattr(value, "untyped_storage") \
-                    else value.numel() * value.element_size()
-                seen[key] = size
-    return sum(seen.values())
-
-
 def prefill_flops(cfg, tokens: int, ff: int) -> float:
     H, hq, hkv, hd = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     per_token = 0
@@ -108,17 +95,15 @@ def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1) -> int:
                                     max_batched_tokens=load["budget"],
                                     prefill_chunk_tokens=load["chunk"], portion_granule=granule,
                                     context=cfg["max_position_embeddings"])
-    # a short run first: kernels loaded, graphs captured for the decode batch sizes
+    # a short run first: weights re-laid, a graph recorded
     engine.generate(prompts[:2], max_new_tokens=4, generation=GREEDY, eos_token_ids=[])
-    for key in engine.metrics:
-        engine.metrics[key] = type(engine.metrics[key])()
-    runner = engine.loaded.runner
-    runner.captures, runner.capture_seconds = 0, 0.0
-    torch.cuda.synchronize()
+    before = engine.metrics
+    engine.loaded.native.synchronize()
     start = time.perf_counter()
     out = engine.generate(prompts, max_new_tokens=load["new_tokens"], generation=GREEDY, eos_token_ids=[])
-    torch.cuda.synchronize()
+    engine.loaded.native.synchronize()
     seconds = time.perf_counter() - start
+    after = engine.metrics
     generated = sum(len(o) for o in out)
     print(json.dumps({
         "metric": f"serve: generated tok/s (LFM2-{shape.upper()} shape, bf16, whole engine)",
@@ -129,8 +114,11 @@ def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1) -> int:
         "requests": load["requests"], "prompt_lengths": list(load["prompt"]),
         "new_tokens": load["new_tokens"], "prefill_chunk": load["chunk"],
         "step_token_budget": load["budget"], "portion_granule": granule, "context": cfg["max_position_embeddings"],
-        "engine_steps": engine.metrics["steps"], "steps_launched_ahead": engine.metrics["steps_ahead"],
-        "graphs_recorded": runner.captures, "recording_seconds": round(runner.capture_seconds, 3),
+        "engine_steps": after["steps"] - before["steps"],
+        "steps_launched_ahead": after["steps_ahead"] - before["steps_ahead"],
+        "steps_replayed_from_graphs": after["graph_replays"] - before["graph_replays"],
+        "graphs_recorded": after["captures"] - before["captures"],
+        "recording_seconds": round(after["capture_seconds"] - before["capture_seconds"], 3),
         "dtype": "bf16", "data": "synthetic"}))
     return 0
 
@@ -169,7 +157,7 @@ def main() -> int:
 
     import torch
     import celeg_amd  # noqa: F401
-    from celeg_amd.engine import load_model
+    from celeg_amd.engine import Engine
     from celeg_amd.engine.benchmark import DecodeBench, measure_prefill
     from celeg_amd.weights import write_random_model
 
@@ -180,19 +168,20 @@ def main() -> int:
         cfg["layer_types"] = cfg["layer_types"][:args.layers]
     context = cfg["max_position_embeddings"]
     max_batch = max(BATCH, args.batch) if args.no_points or args.phase != "all" else 64
-    need = PROMPT_TOKENS + args.steps + args.warmup + 1
+    need = PROMPT_TOKENS + args.steps + args.warmup + 64 + 3    # (a request decodes along while the others' prompts are fed)
     if need > context:
         raise SystemExit(f"--steps + --warmup exceed the context of {context}")
     with tempfile.TemporaryDirectory(prefix="celeg_bench_") as folder:
         write_random_model(cfg, folder, seed=0, dtype=torch.bfloat16, std=0.02)
         pages_per_request = (need + 15) // 16 + 1
-        lm = load_model(folder, dtype="bfloat16", device="cuda:0", page_tokens=16,
-                        n_pages=pages_per_request * max_batch, max_requests=max_batch,
-                        max_context=context, max_batched_tokens=PROMPT_TOKENS,
-                        gemm_backend=args.gemm_backend)
+        engine = Engine.from_folder(folder, dtype="bfloat16", device="cuda:0", page_tokens=16,
+                                    n_pages=pages_per_request * max_batch, max_active_requests=max_batch,
+                                    context=context, max_batched_tokens=PROMPT_TOKENS,
+                                    prefill_chunk_tokens=PROMPT_TOKENS, gemm_backend=args.gemm_backend)
+    lm = engine.loaded
     ff = lm.config.ff_dim
-    w_bytes = weight_bytes(lm.model)
-    kv_per_token = lm.cache.layout.kv_bytes_per_token(2)
+    w_bytes = lm.native.info["weights"] * 2          # every weight once, bfloat16
+    kv_per_token = lm.native.info["kv_bytes_per_token"]
 
     flops = prefill_flops(cfg, PROMPT_TOKENS, ff)
     if args.phase == "decode":
@@ -207,7 +196,7 @@ def main() -> int:
         return 0
 
     def decode(batch: int):
-        bench = DecodeBench(lm, batch, PROMPT_TOKENS, seed=batch, prefill_chunk=PROMPT_TOKENS)
+        bench = DecodeBench(engine, batch, PROMPT_TOKENS, args.steps + args.warmup + batch + 2, seed=batch)
         result = bench.run(args.steps, args.warmup)
         bench.close()
         return result
@@ -223,7 +212,7 @@ def main() -> int:
     if not args.no_points and args.phase == "all":
         points = {"decode_b1": round(decode(1)["tokens_per_second"], 1),
                   "decode_b64": round(decode(64)["tokens_per_second"], 1)}
-    mean_context = PROMPT_TOKENS + args.warmup + (args.steps + 1) / 2.0
+    mean_context = main_run["mean_context"]
     step_bytes = w_bytes + kv_per_token * mean_context * BATCH
     achieved = step_bytes / (main_run["ms_per_step"] * 1e-3) / 1e9
     line = {

@@ -63,6 +63,13 @@ def build_parser() -> argparse.ArgumentParser:
                     help="cache storage (quantized caches are not built)")
     ap.add_argument("--no-cuda-graph", "--no-graph", dest="no_graph", action="store_true",
                     help="do not replay decode steps from a captured graph")
+    ap.add_argument("--profile", action="store_true",
+                    help="time every step's phases (embedding, each layer's mixer and feed-forward, head) "
+                         "with events and print ms per step by phase; such steps are not replayed from graphs "
+                         "(the reference's CELEG_PROFILE_DECODE / CELEG_PROFILE_PREFILL)")
+    ap.add_argument("--dump-hidden", default="", metavar="DIR",
+                    help="write the 32-bit residual stream after every layer of every step to "
+                         "DIR/step<k>_layer<i>.f32 (the reference's CELEG_DEBUG_HIDDEN_DIR)")
     ap.add_argument("--gemm-backend", default="library", choices=["library", "tiles"],
                     help="bfloat16 steps of more than 64 rows: the library's matrix products, or this "
                          "package's tiled products with norm, SwiGLU and residual sum folded in")
@@ -109,12 +116,8 @@ def main(argv: Optional[List[str]] = None) -> int:
 
 
 def run(args) -> int:
-    import numpy as np
-    import torch
-
     import celeg_amd  # noqa: F401
-    from celeg_amd.engine import (Engine, RequestOptions, SchedulerOptions, StepEntry, load_model,
-                                  read_model_folder)
+    from celeg_amd.engine import Engine, RequestOptions, read_model_folder
     from celeg_amd.engine.benchmark import DecodeBench, measure_prefill, random_prompt
     from celeg_amd.sampling import GenerationConfig
     from celeg_amd.weights import write_random_model
@@ -128,11 +131,11 @@ def run(args) -> int:
         model_dir = write_random_model(cfg, tmp.name, args.random_weights_seed)
     config, spec = read_model_folder(model_dir)
     if args.print_config:
+        typed = config if isinstance(config, dict) else vars(config)
         print(json.dumps({"architecture": spec.architecture,
-                          "config": {k: (list(v) if isinstance(v, tuple) else v)
-                                     for k, v in vars(config).items()},
+                          "config": {k: (list(v) if isinstance(v, tuple) else v) for k, v in typed.items()},
                           "layers": [layer.mixer.kind for layer in spec.layers],
-                          "feed_forward_width": getattr(config, "ff_dim", None)}, indent=1))
+                          "feed_forward_width": typed.get("ff_dim")}, indent=1))
         return 0
     context = min(4096, spec.max_context) if args.context is None else args.context
     if context > spec.max_context:
@@ -157,7 +160,8 @@ def run(args) -> int:
     if args.tokens_only:
         print(" ".join(str(t) for t in prompt))
         return 0
-    if len(prompt) + args.max_new_tokens > context:
+    new_tokens = args.benchmark_decode + args.benchmark_warmup + 2 if args.benchmark_decode > 0 else args.max_new_tokens
+    if len(prompt) + new_tokens > context:
         raise ValueError("prompt plus output exceeds --context")
 
     batch = args.batch if args.benchmark_decode > 0 else 1
@@ -165,16 +169,16 @@ def run(args) -> int:
     if args.benchmark_prefill_tokens > 0:
         budget = max(budget, args.benchmark_prefill_tokens)
     pages_per_request = (context + args.page_tokens - 1) // args.page_tokens
-    lm = load_model(model_dir, dtype=args.dtype, device=args.device, page_tokens=args.page_tokens,
-                    n_pages=args.pages or pages_per_request * batch, max_requests=max(batch, 1),
-                    max_context=context, max_batched_tokens=budget, gemm_backend=args.gemm_backend)
-    lm.runner.use_graphs = not args.no_graph
-    if args.memory_report:
-        weights = sum(t.numel() * t.element_size() for t in _weight_tensors(lm.model))
-        mem = lm.cache.memory_bytes()
-        for key, value in (("weights", weights), ("kv_cache", mem["kv_cache"]),
-                           ("conv_state", mem["state"]), ("activations", lm.rt.ws.bytes())):
-            print(f"memory.{key}={value}", file=sys.stderr)
+    if args.dump_hidden:
+        os.environ["CELEG_DUMP_HIDDEN"] = args.dump_hidden      # read by the library when it loads the model
+    engine = Engine.from_folder(model_dir, dtype=args.dtype, device=args.device, page_tokens=args.page_tokens,
+                                n_pages=args.pages or pages_per_request * batch, max_active_requests=max(batch, 1),
+                                context=context, max_batched_tokens=budget,
+                                prefill_chunk_tokens=min(args.prefill_chunk, budget),
+                                gemm_backend=args.gemm_backend, use_graphs=not args.no_graph)
+    lm = engine.loaded
+    if args.profile:
+        lm.native.time_phases(True)
 
     if args.benchmark_decode > 0:
         if args.benchmark_prefill_tokens > 0:
@@ -182,18 +186,17 @@ def run(args) -> int:
             print(f"benchmark.prefill_tokens={p['tokens']}\nbenchmark.prefill_ms={p['ms']:.3f}\n"
                   f"benchmark.prefill_tokens_per_second={p['tokens_per_second']:.3f}",
                   file=sys.stderr)
-        bench = DecodeBench(lm, batch, len(prompt), seed=args.seed, prefill_chunk=args.prefill_chunk)
+        bench = DecodeBench(engine, batch, len(prompt), new_tokens, seed=args.seed)
         d = bench.run(args.benchmark_decode, args.benchmark_warmup)
         bench.close()
         print(f"benchmark.decode_warmup={args.benchmark_warmup}\n"
-              f"benchmark.decode_tokens={d['steps'] * batch}\n"
+              f"benchmark.decode_tokens={d['tokens']}\n"
               f"benchmark.decode_ms={d['ms_per_step'] * d['steps']:.3f}\n"
               f"benchmark.decode_ms_per_token={d['ms_per_step'] / batch:.4f}\n"
               f"benchmark.decode_tokens_per_second={d['tokens_per_second']:.3f}", file=sys.stderr)
+        _reports(args, engine)
         return 0
 
-    engine = Engine(lm, SchedulerOptions(max_active_requests=1, max_batched_tokens=budget,
-                                         prefill_chunk_tokens=min(args.prefill_chunk, budget)))
     generation = GenerationConfig(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
                                   repetition_penalty=args.repetition_penalty, seed=args.seed)
     rid = engine.submit(prompt, RequestOptions(max_new_tokens=max(args.max_new_tokens, 1),
@@ -206,7 +209,7 @@ def run(args) -> int:
         if tokens and first:
             first = False
             if args.dump_logits or args.print_top > 0:
-                logits = engine.last_logits[0].detach().to("cpu").numpy().astype("<f4")
+                logits = engine.last_logits[0].numpy().astype("<f4")
                 if args.dump_logits:
                     with open(args.dump_logits, "wb") as fh:
                         fh.write(logits.tobytes())
@@ -225,23 +228,39 @@ def run(args) -> int:
     print()
     if args.runtime_tokens:
         print("CELEG_GENERATED_TOKEN_IDS=[" + ",".join(str(t) for t in generated) + "]")
-    if args.runtime_metrics:
-        s = engine.scheduler.stats
-        secs = engine.metrics["step_seconds"]
-        print(f"runtime.prefill_tokens={s['prefill_tokens']}\nruntime.decode_tokens={s['decode_tokens']}\n"
-              f"runtime.steps={s['steps']}\nruntime.seconds={secs:.4f}", file=sys.stderr)
+    _reports(args, engine, rid)
     if tmp is not None:
         tmp.cleanup()
     return 0
 
 
-def _weight_tensors(model):
-    seen = {}
-    for _, part in model.named_parts():
-        for value in vars(part).values():
-            if hasattr(value, "data_ptr") and hasattr(value, "numel"):
-                seen[value.data_ptr()] = value
-    return list(seen.values())
+def _reports(args, engine, request_id=None) -> None:
+    """--memory-report and --runtime-metrics, in the reference's ``key=value`` lines on stderr."""
+    m = engine.metrics
+    if args.profile:
+        times = engine.loaded.native.phase_times() or {"steps": 0, "phases": {}}
+        steps = max(times["steps"], 1)
+        total = sum(p["ms"] for p in times["phases"].values()) or 1.0
+        for name, p in times["phases"].items():
+            print(f"profile.{name.replace(' ', '_')}_ms_per_step={p['ms'] / steps:.4f} ({100 * p['ms'] / total:.1f}%)",
+                  file=sys.stderr)
+        print(f"profile.steps={times['steps']}\nprofile.ms_per_step={total / steps:.4f}", file=sys.stderr)
+    if args.memory_report:
+        info = engine.loaded.native.info
+        weights = info["weights"] * (2 if info["dtype"] == "bfloat16" else 4)
+        for key, value in (("weights", weights), ("kv_cache", m["cache"]["kv_cache"]),
+                           ("conv_state", m["cache"]["state"]), ("activations", m["workspace_bytes"])):
+            print(f"memory.{key}={value}", file=sys.stderr)
+    if args.runtime_metrics:
+        s = m["scheduler"]
+        print(f"runtime.prefill_tokens={s['prefill_tokens']}\nruntime.decode_tokens={s['decode_tokens']}\n"
+              f"runtime.steps={s['steps']}\nruntime.seconds={m['step_seconds']:.4f}\n"
+              f"runtime.graph_replays={m['graph_replays']}", file=sys.stderr)
+        if request_id is not None:
+            r = engine.request_metrics(request_id)
+            for key in ("ttft_seconds", "itl_mean_seconds", "itl_max_seconds"):
+                if r.get(key) is not None:
+                    print(f"runtime.{key}={r[key]:.6f}", file=sys.stderr)
 
 
 if __name__ == "__main__":

@@ -452,6 +452,21 @@ const char* celeg_model_knobs(celeg_model* model) {
     return text(out.dump());
 }
 
+const char* celeg_model_phase_times(celeg_model* model) {
+    if (!model) return nullptr;
+    Runtime& rt = *model->lm->rt;
+    return text(rt.phases ? rt.phases->report().dump() : std::string("null"));
+}
+
+celeg_status celeg_model_time_phases(celeg_model* model, int32_t on) {
+    if (!model) return CELEG_INVALID_ARGUMENT;
+    return guarded([&] {
+        Runtime& rt = *model->lm->rt;
+        if (on && !rt.phases) rt.phases = std::make_unique<PhaseTimer>(model->lm->stream);
+        if (!on) rt.phases.reset();
+    });
+}
+
 void* celeg_model_stream(celeg_model* model) { return model ? model->lm->stream : nullptr; }
 
 celeg_status celeg_model_synchronize(celeg_model* model) {
@@ -463,7 +478,25 @@ celeg_status celeg_model_synchronize(celeg_model* model) {
 const char* celeg_describe_folder(const char* model_dir) {
     if (!model_dir) return nullptr;
     std::string out;
-    if (guarded([&] { out = describe_json(describe_model_folder(model_dir)).dump(); }) != CELEG_OK) return nullptr;
+    if (guarded([&] {
+            Json j = describe_json(describe_model_folder(model_dir));
+            // how every tensor is stored, and how a bfloat16 and a 32-bit engine hold it
+            Checkpoint ckpt(model_dir);
+            Json held = Json::object();
+            for (const Json& e : j["expected_tensors"].items()) {
+                const std::string name = e["name"].as_string();
+                bool there = false;
+                for (const auto& n : ckpt.names()) there = there || n == name;
+                if (!there) continue;
+                const TensorInfo& info = ckpt.info(name);
+                held.set(name, Json::object().set("stored", info.dtype)
+                                   .set("bfloat16", dtype_name(stored_as(info, e["kind"].as_string(), DType::BF16)))
+                                   .set("float32", dtype_name(stored_as(info, e["kind"].as_string(), DType::F32))));
+            }
+            j.set("held_as", held);
+            out = j.dump();
+        }) != CELEG_OK)
+        return nullptr;
     return text(out);
 }
 

@@ -135,6 +135,8 @@ public:
     LayerCache layer_cache(int step) const;
     void check() const;          // no page lost, none held twice; slots free or open, never both
     Json memory_bytes() const;
+    // where, inside a slot's row of bytes, the state `name` of run-order entry `step` lies
+    size_t state_offset(int step, const std::string& name) const { return regions_.at({step, name}).offset; }
     int* device_table(int group) const { return groups_[static_cast<size_t>(group)].table.as<int>(); }
     int table_host(int group, int slot, int logical) const;
     int trash_page(int group) const { return groups_[static_cast<size_t>(group)].trash_page; }

@@ -1,5 +1,6 @@
 #include "device.hpp"
 
+#include <cstdio>
 #include <cstdlib>
 
 namespace celeg {
@@ -122,6 +123,79 @@ size_t Workspace::bytes() const {
     size_t n = 0;
     for (const auto& b : buffers_) n += b.second.bytes();
     return n;
+}
+
+// ---------------------------------------------------------------------------- phase times
+PhaseTimer::~PhaseTimer() {
+    for (hipEvent_t e : events_) (void)hipEventDestroy(e);
+}
+
+hipEvent_t PhaseTimer::event() {
+    if (used_ == events_.size()) {
+        hipEvent_t e;
+        CELEG_HIP(hipEventCreate(&e));
+        events_.push_back(e);
+    }
+    hipEvent_t e = events_[used_++];
+    CELEG_HIP(hipEventRecord(e, stream_));
+    return e;
+}
+
+void PhaseTimer::begin() {
+    used_ = 0;
+    marks_.clear();
+    event();
+}
+
+void PhaseTimer::mark(const std::string& phase) {
+    if (used_ == 0) return;      // outside a step
+    marks_.emplace_back(phase, used_);
+    event();
+}
+
+void PhaseTimer::end(long long tokens) {
+    if (used_ == 0) return;
+    CELEG_HIP(hipStreamSynchronize(stream_));
+    for (const auto& m : marks_) {
+        float ms = 0.0f;
+        CELEG_HIP(hipEventElapsedTime(&ms, events_[m.second - 1], events_[m.second]));
+        auto it = totals_.find(m.first);
+        if (it == totals_.end()) {
+            order_.push_back(m.first);
+            it = totals_.emplace(m.first, std::make_pair(0.0, 0LL)).first;
+        }
+        it->second.first += ms;
+        it->second.second += 1;
+    }
+    ++steps_;
+    tokens_ += tokens;
+    used_ = 0;
+    marks_.clear();
+}
+
+Json PhaseTimer::report() const {
+    Json phases = Json::object();
+    for (const std::string& name : order_) {
+        const auto& t = totals_.at(name);
+        phases.set(name, Json::object().set("ms", t.first).set("calls", t.second));
+    }
+    return Json::object().set("steps", steps_).set("tokens", tokens_).set("phases", phases);
+}
+
+std::string PhaseTimer::table() const {
+    double all = 0.0;
+    for (const auto& t : totals_) all += t.second.first;
+    std::string out = "phase times over " + std::to_string(steps_) + " steps, " + std::to_string(tokens_) + " tokens\n";
+    char line[160];
+    for (const std::string& name : order_) {
+        const auto& t = totals_.at(name);
+        std::snprintf(line, sizeof line, "  %-28s %10.4f ms/step %6.1f %%  (%lld calls)\n", name.c_str(),
+                      steps_ ? t.first / static_cast<double>(steps_) : 0.0, all > 0 ? 100.0 * t.first / all : 0.0, t.second);
+        out += line;
+    }
+    std::snprintf(line, sizeof line, "  %-28s %10.4f ms/step\n", "all phases", steps_ ? all / static_cast<double>(steps_) : 0.0);
+    out += line;
+    return out;
 }
 
 }  // namespace celeg

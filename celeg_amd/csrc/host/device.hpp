@@ -168,4 +168,32 @@ private:
     std::vector<DeviceBuffer> retired_;
 };
 
+// Times of the phases of a step, for finding where a step's time goes: events on the stream at
+// the phase boundaries, read when the step has run.  The reference brackets its phases with
+// events under CELEG_PROFILE_DECODE / CELEG_PROFILE_PREFILL and prints ms per token
+// (include/celeg/backend/cuda/phase_profile.hpp:11-186); like there, a step that is timed is
+// not replayed from a recorded graph.
+class PhaseTimer {
+public:
+    explicit PhaseTimer(hipStream_t stream) : stream_(stream) {}
+    ~PhaseTimer();
+    PhaseTimer(const PhaseTimer&) = delete;
+    void begin();                               // a step begins
+    void mark(const std::string& phase);        // what ran since the last mark belongs to `phase`
+    void end(long long tokens);                 // waits for the step and adds its times up
+    // {"steps", "tokens", "phases": {name: {"ms": total, "calls": n}}}
+    Json report() const;
+    std::string table() const;                  // the same for people: ms per step and share, by phase
+
+private:
+    hipEvent_t event();
+    hipStream_t stream_;
+    std::vector<hipEvent_t> events_;
+    size_t used_ = 0;
+    std::vector<std::pair<std::string, size_t>> marks_;
+    std::vector<std::string> order_;
+    std::map<std::string, std::pair<double, long long>> totals_;
+    long long steps_ = 0, tokens_ = 0;
+};
+
 }  // namespace celeg

@@ -123,7 +123,7 @@ Json call(HostObject& o, const std::string& method, const Json& a) {
                 regions.set(std::to_string(c.layout.states[i].first) + ":" + c.layout.states[i].second.name,
                             Json::object().set("shape", Json::array_of(std::vector<long long>(t.shape, t.shape + t.ndim)))
                                 .set("slot_stride", t.stride[0]).set("dtype", dtype_name(t.dtype))
-                                .set("offset", static_cast<long long>(reinterpret_cast<uintptr_t>(t.data))));
+                                .set("offset", static_cast<long long>(c.state_offset(c.layout.states[i].first, c.layout.states[i].second.name))));
             }
             return Json::object().set("free_slots", c.n_free_slots()).set("free_pages", Json::array_of(c.free_pages()))
                 .set("open_slots", Json::array_of(c.open_slots())).set("null_slot", c.null_slot)

@@ -149,6 +149,7 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
     rt.stream_stat_blocks = 0;
     rt.stream_has_bf16 = false;
     embedding_->forward(batch.token_ids, h, rt, &batch);
+    rt.mark("embedding");
     Tensor delta;
     for (size_t i = 0; i < spec.order.size(); ++i) {
         delta = blocks_[static_cast<size_t>(spec.order[i].layer)]->forward(h, delta, batch, caches_[i], rt);
@@ -157,10 +158,14 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
     Tensor logits = rt.ws.buf("logits", DType::F32, {R, vocab});
     if (R == 0) return logits;
     const Norm::Foldable* fold = final_norm_->foldable();
-    if (!delta.defined() && fold && head_->forward_fused(h, *fold, batch, logits, rt, embedding_.get())) return logits;
+    if (!delta.defined() && fold && head_->forward_fused(h, *fold, batch, logits, rt, embedding_.get())) {
+        rt.mark("head");
+        return logits;
+    }
     Tensor normed = rt.ws.buf("final_normed", rt.dtype, {R, width});
     final_norm_->forward(h, normed, rt, delta.defined() ? &delta : nullptr, batch.logit_rows);
     head_->forward(normed, logits, rt, embedding_.get());
+    rt.mark("head");
     return logits;
 }
 
@@ -292,9 +297,12 @@ Tensor ModelRunner::step(const std::vector<StepEntry>& entries) {
     BuildOptions options;
     options.null_slot = cache.null_slot;
     StepBatch batch = build(entries, updates, options);
+    if (rt.phases) rt.phases->begin();
     begin_step(batch);
+    rt.mark("step metadata");
     last_batch_ = batch;
     Tensor logits = model.forward(batch, rt);
+    if (rt.phases) rt.phases->end(batch.n_tokens);
     ++steps_run;
     return logits;
 }
@@ -306,7 +314,7 @@ Tensor ModelRunner::step(const std::vector<StepEntry>& entries) {
 // request's cache.  Recording and its warm-up run on such padding rows only: a request's state
 // is never advanced twice.
 bool ModelRunner::graph_applies(const std::vector<StepEntry>& entries) const {
-    if (!use_graphs || !model.graph_safe() || rt.after_layer) return false;
+    if (!use_graphs || !model.graph_safe() || rt.after_layer || rt.phases) return false;
     if (static_cast<int>(entries.size()) > buckets_.back()) return false;
     for (const StepEntry& e : entries)
         if (e.tokens.size() != 1 || e.want.size() != 1 || e.want[0] != 0) return false;
@@ -392,6 +400,7 @@ ModelRunner::Captured& ModelRunner::capture(int bucket, const std::vector<int>& 
 // ---------------------------------------------------------------------------- loading
 LoadedModel::~LoadedModel() {
     if (stream) (void)hipStreamSynchronize(stream);
+    if (rt && rt->phases) std::fputs(rt->phases->table().c_str(), stderr);
     runner.reset();
     cache.reset();
     model.reset();
@@ -473,6 +482,8 @@ std::unique_ptr<LoadedModel> load_model(const std::string& model_dir, const Load
     lm->runner->use_graphs = options.use_graphs;
     if (const char* dump = std::getenv("CELEG_DUMP_HIDDEN"))
         if (*dump) install_hidden_dump(*lm->rt, dump);
+    if (const char* timed = std::getenv("CELEG_PROFILE_PHASES"))
+        if (*timed && std::string(timed) != "0") lm->rt->phases = std::make_unique<PhaseTimer>(lm->stream);
     CELEG_HIP(hipStreamSynchronize(lm->stream));
     return lm;
 }

@@ -135,6 +135,11 @@ struct Runtime {
     // a hook for bisecting mismatches: called after every entry of the run order with the
     // residual stream (the pending addition, if any, not yet made)
     std::function<void(int step, const Tensor& h, const Tensor* delta)> after_layer;
+    // set: every step is timed phase by phase (and none is replayed from a recorded graph)
+    std::unique_ptr<PhaseTimer> phases;
+    void mark(const std::string& phase) {
+        if (phases) phases->mark(phase);
+    }
 };
 
 }  // namespace celeg

@@ -666,10 +666,16 @@ public:
             mixer_norm_->forward(h, normed, rt, delta.defined() ? &delta : nullptr, nullptr);
             mixed = mixer_->forward(normed, batch, cache, rt);
         }
-        if (fusable && !mixed.defined() && ffn_->forward_fused(h, *fold2, batch, rt)) return Tensor();
+        rt.mark("mixer " + mixer_->spec.kind);
+        if (fusable && !mixed.defined() && ffn_->forward_fused(h, *fold2, batch, rt)) {
+            rt.mark("ffn " + ffn_->spec.kind);
+            return Tensor();
+        }
         rt.stream_stat_blocks = 0;
         ffn_norm_->forward(h, normed, rt, mixed.defined() ? &mixed : nullptr, nullptr);
-        return ffn_->forward(normed, batch, rt);
+        Tensor out = ffn_->forward(normed, batch, rt);
+        rt.mark("ffn " + ffn_->spec.kind);
+        return out;
     }
 
 private:

@@ -213,11 +213,16 @@ void Scheduler::accept(const std::vector<PlannedEntry>& entries, const std::vect
     ++steps_;
     size_t next = 0;
     const auto now = std::chrono::steady_clock::now();
+    const long long decoded_before = decode_tokens_, prefilled_before = prefill_tokens_;
+    for (const PlannedEntry& e : entries) {
+        Request& req = *e.request;
+        if (e.count == 1 && req.status == RequestStatus::Decoding) ++decode_tokens_;
+        else prefill_tokens_ += e.count;
+    }
+    if (decode_tokens_ > decoded_before && prefill_tokens_ > prefilled_before) ++mixed_steps_;
     for (const PlannedEntry& e : entries) {
         Request& req = *e.request;
         req.fed = e.start + e.count;
-        if (e.count == 1 && req.status == RequestStatus::Decoding) ++decode_tokens_;
-        else prefill_tokens_ += e.count;
         if (!e.samples) continue;
         if (next >= sampled.size()) throw StepError("accept: fewer sampled tokens than sampling entries");
         const int token = sampled[next++];
@@ -246,7 +251,7 @@ void Scheduler::fail(const std::vector<PlannedEntry>& entries, const std::string
 
 Json Scheduler::stats() const {
     return Json::object().set("steps", steps_).set("preemptions", preemptions_).set("stalled_decodes", stalled_decodes_)
-        .set("prefill_tokens", prefill_tokens_).set("decode_tokens", decode_tokens_);
+        .set("prefill_tokens", prefill_tokens_).set("decode_tokens", decode_tokens_).set("mixed_steps", mixed_steps_);
 }
 
 }  // namespace celeg

@@ -134,7 +134,7 @@ private:
     long long next_id_ = 0, admitted_ = 0;
     std::vector<std::pair<int, Request*>> new_slots_;
     std::vector<int> released_slots_;
-    long long steps_ = 0, preemptions_ = 0, stalled_decodes_ = 0, prefill_tokens_ = 0, decode_tokens_ = 0;
+    long long steps_ = 0, preemptions_ = 0, stalled_decodes_ = 0, prefill_tokens_ = 0, decode_tokens_ = 0, mixed_steps_ = 0;
 };
 
 }  // namespace celeg

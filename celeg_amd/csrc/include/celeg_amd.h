@@ -145,6 +145,14 @@ celeg_status celeg_model_step(celeg_model* model, int32_t n_entries, const int32
  * and their values comes back from celeg_model_knobs */
 celeg_status celeg_model_set_knob(celeg_model* model, const char* name, int32_t value);
 const char* celeg_model_knobs(celeg_model* model);
+/* Times of a step's phases (embedding, every layer's mixer and feed-forward, head), taken with events on
+ * the stream: switched on here or by the environment variable CELEG_PROFILE_PHASES=1 at load time; steps
+ * that are timed are not replayed from recorded graphs.  JSON {"steps", "tokens", "phases": {name:
+ * {"ms", "calls"}}}, or "null" when nothing is timed.  With the environment variable set, a table is
+ * also printed to stderr when the model goes.  CELEG_DUMP_HIDDEN=<folder> at load time writes the 32-bit
+ * residual stream after every entry of the run order to <folder>/step<k>_layer<i>.f32 ([rows, width]). */
+celeg_status celeg_model_time_phases(celeg_model* model, int32_t on);
+const char* celeg_model_phase_times(celeg_model* model);
 /* the raw HIP stream the model's work runs on */
 void* celeg_model_stream(celeg_model* model);
 /* waits for everything launched on that stream */

@@ -145,6 +145,8 @@ def lib() -> ctypes.CDLL:
     sig("celeg_model_knobs", c_char_p, c_void_p)
     sig("celeg_model_stream", c_void_p, c_void_p)
     sig("celeg_model_synchronize", c_int, c_void_p)
+    sig("celeg_model_time_phases", c_int, c_void_p, c_int32)
+    sig("celeg_model_phase_times", c_char_p, c_void_p)
     sig("celeg_describe_folder", c_char_p, c_char_p)
     sig("celeg_describe_config", c_char_p, c_char_p, c_char_p)
     sig("celeg_check_folder", c_int, c_char_p)
@@ -305,6 +307,14 @@ class NativeModel:
 
     def synchronize(self) -> None:
         check(lib().celeg_model_synchronize(self.handle))
+
+    def time_phases(self, on: bool = True) -> None:
+        """Time every step's phases with events (such steps are not replayed from graphs)."""
+        check(lib().celeg_model_time_phases(self.handle, int(bool(on))))
+
+    def phase_times(self):
+        """{"steps", "tokens", "phases": {name: {"ms", "calls"}}}, or None when nothing is timed."""
+        return json.loads(_text(lib().celeg_model_phase_times(self.handle)))
 
     @property
     def stream(self) -> int:

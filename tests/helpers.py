@@ -216,3 +216,18 @@ class EngineDriver:
                 self.lm.cache.close(self.live.pop(rid)[0])
             self.lm.cache.check()
         return {rid: torch.stack(rows) for rid, rows in out.items()}
+
+
+def reordered_lfm2():
+    """An architecture registered from the tests: LFM2's parts under the run order that the
+    configuration's "run_order" gives ([layer, kv_from or None] pairs)."""
+    import dataclasses
+    from celeg_amd.config import RunStep, register_architecture, registered_architectures, spec_from_config
+    if "Lfm2Reordered" in registered_architectures():
+        return
+
+    def build(cfg, shapes):
+        _, spec = spec_from_config(dict(cfg, architectures=["Lfm2ForCausalLM"]), shapes)
+        order = tuple(RunStep(layer, kv_from) for layer, kv_from in cfg["run_order"])
+        return dataclasses.replace(spec, architecture="Lfm2Reordered", order=order)
+    register_architecture("Lfm2Reordered", build)

@@ -248,7 +248,7 @@ def normalise_config(cfg: dict) -> dict:
 def model_logits(cfg: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int],
                  order: Optional[List[int]] = None,
                  kv_from: Optional[Dict[int, int]] = None,
-                 first_position: int = 0) -> torch.Tensor:
+                 first_position: int = 0, hidden: Optional[list] = None) -> torch.Tensor:
     """Logits [T, V] of a whole sequence.
 
     Every layer is pre-norm, mixer, add, pre-norm, feed-forward, add
@@ -258,7 +258,8 @@ def model_logits(cfg: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int],
     they run (default 0..N-1) and ``kv_from[i] = j`` lets the i-th entry of the
     order attend over the keys and values that the j-th entry computed; both are
     generalisations used by tests of the engine's layer list, not LFM2 features.
-    ``first_position`` shifts all positions (for the shift invariance test).
+    ``first_position`` shifts all positions (for the shift invariance test).  ``hidden``, a
+    list, receives the residual stream [T, H] after every entry of the order.
     """
     cfg = normalise_config(cfg)
     T = len(tokens)
@@ -282,6 +283,8 @@ def model_logits(cfg: dict, W: Dict[str, torch.Tensor], tokens: Sequence[int],
         h = h + swiglu_ffn(n2, W[prefix + "feed_forward.w1.weight"],
                            W[prefix + "feed_forward.w3.weight"],
                            W[prefix + "feed_forward.w2.weight"])
+        if hidden is not None:
+            hidden.append(h.clone())
     n = rmsnorm(h, W["model.embedding_norm.weight"], cfg["norm_eps"])
     head = W["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else W["lm_head.weight"]
     return linear(n, head)

@@ -1,13 +1,12 @@
-"""The cache manager (no page lost, held twice or freed twice, under random orders of
-requests; windows; state slots) and the scheduler's decisions, on the host."""
+"""The library's cache manager (no page lost, held twice or freed twice, under random orders
+of requests; windows; state slots) and its scheduler's decisions, by themselves, without a GPU
+(the objects live in the library; the tests drive them through its host-object calls)."""
 import random
 
 import pytest
-import torch
 
-from celeg_amd.cache import CacheLayout, CacheManager, PageError, PagePool
-from celeg_amd.engine.scheduler import (RequestOptions, RequestStatus, Scheduler, SchedulerOptions)
-from celeg_amd.parts.base import KVNeed, StateNeed
+from celeg_amd.cache import CacheManager, PageError, PagePool, cache_layout
+from celeg_amd.engine import RequestOptions, RequestStatus, Scheduler, SchedulerOptions
 from celeg_amd.sampling import GREEDY, GenerationConfig
 
 
@@ -37,18 +36,16 @@ def test_pool_behaviour_of_the_reference():
 
 
 def make_manager(n_pages=12, slots=4, window=None, max_context=256, extra_group=False):
-    layout = CacheLayout()
-    layout.kv_groups = [KVNeed(2, 16, None)]
-    layout.group_layers = [2]
-    layout.kv_of_step = {1: (0, 0, True), 3: (0, 1, True)}
+    groups = [(2, 16, None, 2)]
+    uses = {1: (0, 0, True), 3: (0, 1, True)}
     if window or extra_group:
-        layout.kv_groups.append(KVNeed(1, 16, window))
-        layout.group_layers.append(1)
-        layout.kv_of_step[4] = (1, 0, True)
-    layout.states = [(0, StateNeed("bx", (3, 8))), (2, StateNeed("bx", (3, 8))),
-                     (2, StateNeed("count", (1,), torch.int32))]
-    return CacheManager(layout, page_tokens=16, n_pages=n_pages, max_requests=slots,
-                        max_context=max_context, device="cpu", dtype=torch.float32)
+        groups.append((1, 16, window, 1))
+        uses[4] = (1, 0, True)
+    states = [(0, "bx", (3, 8)), (2, "bx", (3, 8)), (2, "count", (1,), "int32")]
+    m = CacheManager(cache_layout(groups, uses, states), page_tokens=16, n_pages=n_pages, max_requests=slots,
+                     max_context=max_context)
+    m.pool_pages = n_pages if isinstance(n_pages, int) else n_pages[0]
+    return m
 
 
 def test_manager_allocates_covers_and_gives_back():
@@ -75,26 +72,22 @@ def test_manager_allocates_covers_and_gives_back():
     m.check()
 
 
-def test_state_slots_are_separate_zeroed_and_typed():
+def test_state_slots_have_regions_of_their_own():
+    """Every (run-order entry, state) has a region of a slot's row of bytes: typed, aligned to
+    16 bytes, not overlapping; one row per request and one for the null slot.  (That a slot is
+    zeroed when a request takes it is checked on the GPU, with a mixer that keeps state.)"""
     m = make_manager()
-    a, b = m.open(), m.open()
-    bx0 = m.layer_cache(0).states["bx"]
-    bx2 = m.layer_cache(2).states["bx"]
-    count = m.layer_cache(2).states["count"]
-    assert bx0.shape == (5, 3, 8) and count.dtype == torch.int32 and count.shape == (5, 1)
-    bx0[a] = 1.0; bx2[a] = 2.0; count[a] = 7; bx0[b] = 3.0
-    assert float(bx2[b].abs().max()) == 0 and float(bx0[a].min()) == 1.0 and int(count[a]) == 7
-    assert float(bx2[a].min()) == 2.0                  # regions do not overlap
-    m.close(a)
-    again = m.open()
-    assert again == a and float(bx0[a].abs().max()) == 0 and int(count[a]) == 0   # zeroed
-    assert float(bx0[b].min()) == 3.0
-    assert m.layer_cache(1).states == {} and m.layer_cache(1).kv.layer == 0
-    assert m.layer_cache(3).kv.layer == 1 and m.layer_cache(3).kv.k.shape == (13, 2, 2, 16, 16)
-    wide = CacheManager(CacheLayout([KVNeed(2, 32)], [1], {0: (0, 0, True)}, []), page_tokens=16,
-                        n_pages=3, max_requests=1, max_context=64, device="cpu", dtype=torch.float32)
-    kv = wide.layer_cache(0).kv         # keys row by row, values transposed inside the page
-    assert kv.k.shape == (4, 1, 2, 16, 32) and kv.v.shape == (4, 1, 2, 32, 16)
+    st = m.state()
+    regions = st["state_regions"]
+    assert set(regions) == {"0:bx", "2:bx", "2:count"}
+    assert regions["0:bx"]["shape"] == [5, 3, 8] and regions["2:count"]["shape"] == [5, 1]
+    assert regions["2:count"]["dtype"] == "int32" and regions["0:bx"]["dtype"] == "float32"
+    spans = sorted((r["offset"], r["offset"] + 4 * r["shape"][1] * (r["shape"][2] if len(r["shape"]) > 2 else 1))
+                   for r in regions.values())
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))           # regions do not overlap
+    assert all(off % 16 == 0 for off, _ in spans)
+    assert st["slot_bytes"] == 96 + 96 + 16 and regions["0:bx"]["slot_stride"] == st["slot_bytes"] // 4
+    assert st["null_slot"] == 4 and st["max_pages_per_request"] == 16 and st["n_groups"] == 1
 
 
 def test_window_group_gives_pages_back_as_the_window_passes():
@@ -112,7 +105,7 @@ def test_window_group_gives_pages_back_as_the_window_passes():
         assert len(win) <= (20 + n + 15) // 16 + 1
         m.check()
     assert held[-1][0] == (pos + 15) // 16 and held[-1][1] <= 3
-    assert m.groups[1].table_host[s, 0] == -1 and m.groups[0].table_host[s, 0] >= 0
+    assert m.table(1, s, 0) == -1 and m.table(0, s, 0) >= 0
     m.close(s)
     assert m.free_pages() == [6, 6]
 
@@ -166,14 +159,15 @@ class FakeStep:
         self.batches = []
 
     def run(self, plan):
-        self.batches.append([(e.request.id, e.start, e.count) for e in plan])
+        self.batches.append([(e["id"], e["start"], e["count"]) for e in plan])
         out = []
         for e in plan:
-            history = self.fed.setdefault(e.request.slot, [])
-            assert e.start <= len(history), "a position was skipped"
-            del history[e.start:]
-            history.extend(e.request.tokens(e.start, e.count))
-            if e.samples:
+            history = self.fed.setdefault(e["slot"], [])
+            assert e["start"] <= len(history), "a position was skipped"
+            del history[e["start"]:]
+            assert len(e["tokens"]) == e["count"]
+            history.extend(e["tokens"])
+            if e["samples"]:
                 out.append(expected_next(history))
         return out
 
@@ -202,13 +196,11 @@ def drive(sched, fake, max_steps=2000):
     steps = 0
     while sched.has_work():
         plan = sched.plan()
-        released, new = sched.drain_slot_events()
-        for slot in released:
+        for slot in sched.slot_events()["released"]:
             fake.fed.pop(slot, None)
         if plan:
-            sched.accept(plan, fake.run(plan))
-        released, _ = sched.drain_slot_events()
-        for slot in released:
+            sched.accept(fake.run(plan))
+        for slot in sched.slot_events()["released"]:
             fake.fed.pop(slot, None)
         steps += 1
         assert steps < max_steps, "the scheduler does not terminate"
@@ -246,8 +238,8 @@ def test_budget_portions_and_decode_first():
     assert second[0] == (b, 9, 1) and second[1] == (a, 20, 20)   # decode token first, then portion
     assert all(sum(c for _, _, c in batch) <= 32 for batch in fake.batches)
     for rid, prompt in ((a, list(range(1, 46))), (b, list(range(3, 12)))):
-        assert sched.requests[rid].generated == expected_output(prompt, 5)
-        assert sched.requests[rid].status == RequestStatus.FINISHED
+        assert sched.request(rid)["generated"] == expected_output(prompt, 5)
+        assert sched.request(rid)["status"] == "finished"
     assert sched.cache.n_free_slots == 4 and sched.cache.free_pages() == [64]
 
 
@@ -258,8 +250,8 @@ def test_priority_then_age_and_end_tokens_and_poll():
     high = sched.submit([4, 5, 6], opts(3, priority=5))
     later = sched.submit([7, 8], opts(3))
     plan = sched.plan()
-    assert [e.request.id for e in plan] == [high]
-    sched.accept(plan, fake.run(plan))
+    assert [e["id"] for e in plan] == [high]
+    sched.accept(fake.run(plan))
     status, tokens, _ = sched.poll(high)
     assert status == RequestStatus.DECODING and tokens == expected_output([4, 5, 6], 1)
     assert sched.poll(high)[1] == []                        # drained
@@ -272,8 +264,8 @@ def test_priority_then_age_and_end_tokens_and_poll():
     eos_tok = expected_output(prompt, 3)[1]
     rid = sched2.submit(prompt, opts(10, eos_token_ids=[eos_tok]))
     drive(sched2, FakeStep())
-    assert sched2.requests[rid].generated == expected_output(prompt, 10, eos=[eos_tok])
-    assert sched2.requests[rid].generated[-1] == eos_tok
+    assert sched2.request(rid)["generated"] == expected_output(prompt, 10, eos=[eos_tok])
+    assert sched2.request(rid)["generated"][-1] == eos_tok
 
 
 def test_portions_cut_by_the_budget_keep_to_the_granule():
@@ -286,22 +278,22 @@ def test_portions_cut_by_the_budget_keep_to_the_granule():
     a = sched.submit([1] * 70, opts(3))
     b = sched.submit([2] * 90, opts(3))
     plan = sched.plan()
-    assert [(e.request.id, e.count) for e in plan] == [(a, 64), (b, 32)]     # 36 left: cut to 32
-    sched.accept(plan, fake.run(plan))
+    assert [(e["id"], e["count"]) for e in plan] == [(a, 64), (b, 32)]     # 36 left: cut to 32
+    sched.accept(fake.run(plan))
     plan = sched.plan()
-    assert [(e.request.id, e.count) for e in plan] == [(a, 6), (b, 58)]      # the ends of both prompts
-    sched.accept(plan, fake.run(plan))
+    assert [(e["id"], e["count"]) for e in plan] == [(a, 6), (b, 58)]      # the ends of both prompts
+    sched.accept(fake.run(plan))
     drive(sched, fake)
-    assert sched.requests[a].generated == expected_output([1] * 70, 3)
-    assert sched.requests[b].generated == expected_output([2] * 90, 3)
+    assert sched.request(a)["generated"] == expected_output([1] * 70, 3)
+    assert sched.request(b)["generated"] == expected_output([2] * 90, 3)
     # a budget below the granule: the first portion of a step is cut at the budget all the same
     sched2, _ = make_scheduler(prefill_chunk_tokens=64, max_batched_tokens=10, portion_granule=16)
     c = sched2.submit([3] * 25, opts(2))
     plan = sched2.plan()
-    assert [(e.request.id, e.count) for e in plan] == [(c, 10)]
-    sched2.accept(plan, fake.run(plan))
+    assert [(e["id"], e["count"]) for e in plan] == [(c, 10)]
+    sched2.accept(fake.run(plan))
     drive(sched2, fake)
-    assert sched2.requests[c].generated == expected_output([3] * 25, 2)
+    assert sched2.request(c)["generated"] == expected_output([3] * 25, 2)
 
 
 def test_admission_waits_for_pages_and_slots():
@@ -310,11 +302,11 @@ def test_admission_waits_for_pages_and_slots():
     a = sched.submit([1] * 40, opts(4))        # 3 pages
     b = sched.submit([2] * 40, opts(4))        # 3 pages: does not fit beside a
     plan = sched.plan()
-    assert [(e.request.id, e.count) for e in plan] == [(a, 40), (b, 16)]   # cut to the free page
-    sched.accept(plan, fake.run(plan))
+    assert [(e["id"], e["count"]) for e in plan] == [(a, 40), (b, 16)]   # cut to the free page
+    sched.accept(fake.run(plan))
     drive(sched, fake)
-    assert sched.requests[a].generated == expected_output([1] * 40, 4)
-    assert sched.requests[b].generated == expected_output([2] * 40, 4)
+    assert sched.request(a)["generated"] == expected_output([1] * 40, 4)
+    assert sched.request(b)["generated"] == expected_output([2] * 40, 4)
 
 
 def test_out_of_pages_stalls_then_preempts_the_youngest_and_still_gives_the_same_tokens():
@@ -325,9 +317,9 @@ def test_out_of_pages_stalls_then_preempts_the_youngest_and_still_gives_the_same
     drive(sched, fake)
     assert sched.stats["preemptions"] > 0 and sched.stats["stalled_decodes"] > 0
     for rid, p in zip(ids, prompts):
-        assert sched.requests[rid].status == RequestStatus.FINISHED
-        assert sched.requests[rid].generated == expected_output(p, 40)
-    assert sched.requests[ids[0]].preemptions == 0           # the oldest is never the victim
+        assert sched.request(rid)["status"] == "finished"
+        assert sched.request(rid)["generated"] == expected_output(p, 40)
+    assert sched.request(ids[0])["preemptions"] == 0           # the oldest is never the victim
     assert m.free_pages() == [6] and m.n_free_slots == 3
 
 
@@ -337,9 +329,9 @@ def test_request_that_can_never_fit_fails_and_others_go_on():
     big = sched.submit([1] * 100, opts(4))                   # 7 pages > 3
     small = sched.submit([2] * 10, opts(4))
     drive(sched, fake)
-    assert sched.requests[big].status == RequestStatus.FAILED
-    assert "more cache pages" in sched.requests[big].error
-    assert sched.requests[small].generated == expected_output([2] * 10, 4)
+    assert sched.request(big)["status"] == "failed"
+    assert "more cache pages" in sched.request(big)["error"]
+    assert sched.request(small)["generated"] == expected_output([2] * 10, 4)
 
 
 def test_guaranteed_policy_reserves_up_front():
@@ -348,11 +340,11 @@ def test_guaranteed_policy_reserves_up_front():
     fake = FakeStep()
     ids = [sched.submit([1 + i] * 30, opts(40)) for i in range(3)]    # 5 pages each
     plan = sched.plan()
-    assert [e.request.id for e in plan] == [ids[0]] and m.free_pages() == [1]
-    sched.accept(plan, fake.run(plan))
+    assert [e["id"] for e in plan] == [ids[0]] and m.free_pages() == [1]
+    sched.accept(fake.run(plan))
     drive(sched, fake)
     assert sched.stats["preemptions"] == 0 and sched.stats["stalled_decodes"] == 0
-    assert all(sched.requests[r].generated == expected_output([1 + i] * 30, 40)
+    assert all(sched.request(r)["generated"] == expected_output([1 + i] * 30, 40)
                for i, r in enumerate(ids))
 
 
@@ -362,12 +354,12 @@ def test_cancel_frees_everything():
     a = sched.submit([1] * 20, opts(50))
     b = sched.submit([2] * 20, opts(5))
     for _ in range(3):
-        plan = sched.plan(); sched.accept(plan, fake.run(plan))
+        plan = sched.plan(); sched.accept(fake.run(plan))
     sched.cancel(a)
     drive(sched, fake)
-    assert sched.requests[a].status == RequestStatus.CANCELLED
-    assert 0 < len(sched.requests[a].generated) < 50
-    assert sched.requests[b].generated == expected_output([2] * 20, 5)
+    assert sched.request(a)["status"] == "cancelled"
+    assert 0 < len(sched.request(a)["generated"]) < 50
+    assert sched.request(b)["generated"] == expected_output([2] * 20, 5)
     assert m.free_pages() == [64] and m.n_free_slots == 4
 
 
@@ -385,5 +377,36 @@ def test_random_workloads_terminate_with_the_right_tokens(seed):
         work.append((sched.submit(prompt, opts(n)), prompt, n))
     drive(sched, fake)
     for rid, prompt, n in work:
-        assert sched.requests[rid].generated == expected_output(prompt, n)
-    assert m.free_pages() == [m.groups[0].pool.n_pages] and m.n_free_slots == m.max_requests
+        assert sched.request(rid)["generated"] == expected_output(prompt, n)
+    assert m.free_pages() == [m.pool_pages] and m.n_free_slots == m.max_requests
+
+
+def test_a_failed_step_fails_its_requests_and_frees_what_they_hold():
+    """What the engine does when launching or completing a step throws: the step's requests
+    become Failed with the message, their pages and slots go back, and the others go on
+    (src/backend/cuda/runtime/request_lifecycle.cpp:200-218)."""
+    sched, m = make_scheduler(n_pages=16, slots=3, prefill_chunk_tokens=64, max_batched_tokens=64)
+    fake = FakeStep()
+    a = sched.submit([1] * 20, opts(5))
+    b = sched.submit([2] * 20, opts(5))
+    plan = sched.plan()
+    assert {e["id"] for e in plan} == {a, b}
+    sched.fail("HIP error 700 in a kernel")
+    for rid in (a, b):
+        status, tokens, error = sched.poll(rid)
+        assert status == RequestStatus.FAILED and tokens == [] and "HIP error 700" in error
+    assert m.free_pages() == [16] and m.n_free_slots == 3 and not sched.has_work()
+    assert sorted(sched.slot_events()["released"]) == [0, 1]
+    c = sched.submit([3] * 10, opts(4))
+    drive(sched, fake)
+    assert sched.request(c)["generated"] == expected_output([3] * 10, 4)
+    m.check()
+
+
+def test_latencies_are_recorded_per_request():
+    sched, _ = make_scheduler()
+    fake = FakeStep()
+    rid = sched.submit([1, 2, 3], opts(4))
+    drive(sched, fake)
+    r = sched.request(rid)
+    assert r["ttft_seconds"] >= 0 and r["itl_count"] == 3

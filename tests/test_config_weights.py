@@ -8,12 +8,12 @@ import torch
 
 import plain_lfm2 as plain
 from conftest import TINY, TINY_A, TINY_B
+from helpers import reordered_lfm2
 
-from celeg_amd.config import (ConfigError, Lfm2Config, ModelSpec, PartSpec, RunStep,
+from celeg_amd import native
+from celeg_amd.config import (ConfigError, Lfm2Config, ModelSpec, PartSpec, RunStep, register_architecture,
                               registered_architectures, spec_from_config)
-from celeg_amd.engine.model import Model
-from celeg_amd.weights import (Checkpoint, SafetensorsError, SafetensorsFile, WeightError,
-                               check_tensors, load_tensors, write_random_model,
+from celeg_amd.weights import (SafetensorsError, SafetensorsFile, WeightError, check_folder, write_random_model,
                                write_safetensors)
 
 
@@ -49,7 +49,7 @@ def test_config_defaults_and_aliases():
 
 
 def _shapes(cfg):
-    return {n: tuple(w.shape) for n, w in _expected(cfg).items()}
+    return {e["name"]: tuple(e["shape"]) for e in _expected(cfg)}
 
 
 def test_keys_the_reference_accepts_in_other_places(tmp_path):
@@ -60,7 +60,7 @@ def test_keys_the_reference_accepts_in_other_places(tmp_path):
     global_facts.cpp:127-152), and generation_config.json overriding the end tokens
     (src/checkpoint/catalog.cpp:94-121)."""
     from celeg_amd.config import read_config_file
-    from celeg_amd.engine import read_model_folder
+    from celeg_amd.config import read_model_folder
     base = Lfm2Config.from_dict(TINY_B)
     # a config.json as newer writers lay it out: no top-level rope_theta
     nested = {k: v for k, v in TINY_B.items() if k != "rope_theta"}
@@ -98,7 +98,7 @@ def test_keys_the_reference_accepts_in_other_places(tmp_path):
     json.dump(silent, open(os.path.join(folder, "config.json"), "w"))
     json.dump({"bos_token_id": 9, "eos_token_id": [11, 12, "x"], "temperature": 0.3},
               open(os.path.join(folder, "generation_config.json"), "w"))
-    config, spec = read_model_folder(folder)
+    config, spec, _ = read_model_folder(folder)
     assert config.layer_types == base.layer_types and config.ff_dim == 352
     assert config.eos_token_ids == (11, 12) and config.bos_token_id == 9 and spec.eos_token_ids == (11, 12)
     json.dump({"eos_token_id": 5}, open(os.path.join(folder, "generation_config.json"), "w"))
@@ -150,23 +150,23 @@ def test_spec_sizes_come_from_the_config_only():
 
 
 def test_run_order_validation():
-    _, spec = spec_from_config(TINY_A)
-    import dataclasses
-    bad = dataclasses.replace(spec, order=(RunStep(0), RunStep(1, kv_from=1)))
-    with pytest.raises(ValueError, match="does not run before"):
-        bad.validate()
-    with pytest.raises(ValueError, match="names layer 9"):
-        dataclasses.replace(spec, order=(RunStep(9),)).validate()
-    conv_reads = dataclasses.replace(spec, order=(RunStep(0), RunStep(1), RunStep(2, kv_from=1)))
-    with pytest.raises(ValueError, match="keys and values"):
-        Model(conv_reads)
+    reordered_lfm2()
+    def describe(order):
+        return native.describe_config(dict(TINY_A, architectures=["Lfm2Reordered"], run_order=order))
+    with pytest.raises(native.NativeArgumentError, match="does not run before"):
+        describe([[0, None], [1, 1]])
+    with pytest.raises(native.NativeArgumentError, match="names layer 9"):
+        describe([[9, None]])
+    with pytest.raises(native.NativeArgumentError, match="keys and values"):
+        describe([[0, None], [1, None], [2, 1]])             # a convolution cannot read a cache
     # a layer named twice and one that reads another's cache
-    shared = dataclasses.replace(spec, order=(RunStep(0), RunStep(1), RunStep(1), RunStep(3, kv_from=1)))
-    layout = Model(shared).cache_layout()
-    assert layout.group_layers == [2]
-    assert layout.kv_of_step == {1: (0, 0, True), 2: (0, 1, True), 3: (0, 0, False)}
-    assert [s for s, _ in layout.states] == [0]
-    assert "model.layers.3.self_attn.k_proj.weight" not in Model(shared).expected_tensors()
+    d = describe([[0, None], [1, None], [1, None], [3, 1]])
+    layout = d["cache_layout"]
+    assert [g["layers"] for g in layout["kv_groups"]] == [2]
+    assert [(u["step"], u["group"], u["layer"], u["writes"]) for u in layout["kv_of_step"]] == \
+        [(1, 0, 0, True), (2, 0, 1, True), (3, 0, 0, False)]
+    assert [st["step"] for st in layout["states"]] == [0]
+    assert "model.layers.3.self_attn.k_proj.weight" not in [e["name"] for e in d["expected_tensors"]]
 
 
 # ---------------------------------------------------------------- safetensors
@@ -194,8 +194,16 @@ def _raw(path, header: dict, data: bytes):
         fh.write(struct.pack("<Q", len(text)) + text + data)
 
 
-def test_malformed_safetensors_files(tmp_path):
-    p = str(tmp_path / "m.safetensors")
+def _native_reader(path):
+    """The library's reader on the same file: a model folder around it."""
+    folder = os.path.dirname(path)
+    json.dump(TINY_A, open(os.path.join(folder, "config.json"), "w"))
+    check_folder(folder)
+
+
+@pytest.mark.parametrize("SafetensorsFile", [SafetensorsFile, _native_reader], ids=["python", "library"])
+def test_malformed_safetensors_files(tmp_path, SafetensorsFile):
+    p = str(tmp_path / "model.safetensors")
     with open(p, "wb") as fh:
         fh.write(b"abc")
     with pytest.raises(SafetensorsError, match="too small"):
@@ -226,7 +234,7 @@ def test_malformed_safetensors_files(tmp_path):
 
 # ---------------------------------------------------------------- weights against a model
 def _expected(cfg):
-    return Model(spec_from_config(cfg)[1]).expected_tensors()
+    return native.describe_config(cfg)["expected_tensors"]
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
@@ -240,11 +248,11 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     tensors["model.layers.9.extra.weight"] = torch.zeros(1)
     write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
     with pytest.raises(WeightError) as info:
-        check_tensors(Checkpoint(folder), _expected(TINY_B))
+        check_folder(folder)
     err = info.value
     assert err.missing == ["lm_head.weight", "model.layers.2.self_attn.q_layernorm.weight"]
     assert err.unexpected == ["model.layers.9.extra.weight"]
-    assert err.wrong_shape == [("model.layers.0.conv.in_proj.weight", (5, 5), (384, 128))]
+    assert err.wrong_shape == ["model.layers.0.conv.in_proj.weight is (5, 5), expected (384, 128)"]
     text = str(err)
     for word in ("missing tensors (2)", "unexpected tensors (1)", "wrong shape",
                  "model.layers.9.extra.weight", "(5, 5)", "(384, 128)"):
@@ -259,11 +267,11 @@ def test_conv_filter_is_accepted_in_both_shapes_and_bias_is_required(tmp_path):
     f.close()
     tensors["model.layers.0.conv.conv.weight"] = tensors["model.layers.0.conv.conv.weight"].reshape(128, 4)
     write_safetensors(path, tensors)
-    check_tensors(Checkpoint(folder), _expected(TINY_B))
+    check_folder(folder)
     del tensors["model.layers.1.conv.conv.bias"]
     write_safetensors(path, tensors)
     with pytest.raises(WeightError, match="model.layers.1.conv.conv.bias"):
-        check_tensors(Checkpoint(folder), _expected(TINY_B))
+        check_folder(folder)
 
 
 def test_dtype_policy(tmp_path):
@@ -275,15 +283,12 @@ def test_dtype_policy(tmp_path):
     kept32 = "model.layers.1.self_attn.out_proj.weight"
     tensors[kept32] = tensors[kept32].float()
     write_safetensors(path, tensors)
-    exp = _expected(TINY_A)
-    bf = load_tensors(Checkpoint(folder), exp, torch.bfloat16, "cpu")
-    assert bf["model.embed_tokens.weight"].dtype == torch.bfloat16
-    assert bf[kept32].dtype == torch.float32                       # stored in 32-bit: stays so
-    assert bf["model.layers.0.operator_norm.weight"].dtype == torch.float32   # vectors widen exactly
-    assert bf["model.layers.0.conv.conv.weight"].dtype == torch.float32
-    f32 = load_tensors(Checkpoint(folder), exp, torch.float32, "cpu")
-    assert all(t.dtype == torch.float32 for t in f32.values())
-    assert torch.equal(f32["model.embed_tokens.weight"], tensors["model.embed_tokens.weight"].float())
+    held = native.describe_folder(folder)["held_as"]
+    assert held["model.embed_tokens.weight"] == {"stored": "BF16", "bfloat16": "bfloat16", "float32": "float32"}
+    assert held[kept32]["bfloat16"] == "float32"                                 # stored in 32-bit: stays so
+    assert held["model.layers.0.operator_norm.weight"]["bfloat16"] == "float32"   # vectors widen exactly
+    assert held["model.layers.0.conv.conv.weight"]["bfloat16"] == "float32"
+    assert all(h["float32"] == "float32" for h in held.values())
 
 
 def test_random_weights_are_keyed_by_seed_and_name(tmp_path):
@@ -296,12 +301,12 @@ def test_random_weights_are_keyed_by_seed_and_name(tmp_path):
     assert not torch.equal(fa.tensor(name), fc.tensor(name))
     assert abs(float(fa.tensor(name).std()) - 0.02) < 0.002
     assert abs(float(fa.tensor("model.layers.0.ffn_norm.weight").mean()) - 1.0) < 0.02
-    assert sorted(fa.names()) == sorted(_expected(TINY_A))
+    assert sorted(fa.names()) == sorted(e["name"] for e in _expected(TINY_A))
     assert json.load(open(os.path.join(a, "config.json")))["hidden_size"] == 64
     # a folder without weights, a folder without config
     os.remove(os.path.join(a, "model.safetensors"))
     with pytest.raises(FileNotFoundError, match="model.safetensors"):
-        Checkpoint(a)
+        check_folder(a)
     from celeg_amd.config import read_config_file
     os.remove(os.path.join(b, "config.json"))
     with pytest.raises(FileNotFoundError, match="config.json"):
@@ -322,9 +327,8 @@ def test_sharded_checkpoint(tmp_path):
     index = {"weight_map": {n: ("s1.safetensors" if i < half else "s2.safetensors")
                             for i, n in enumerate(names)}}
     json.dump(index, open(os.path.join(folder, "model.safetensors.index.json"), "w"))
-    ck = Checkpoint(folder)
-    check_tensors(ck, _expected(TINY_A))
-    assert all(torch.equal(ck.tensor(n), whole[n]) for n in names)
+    check_folder(folder)
+    assert set(native.describe_folder(folder)["held_as"]) == set(whole)
     os.remove(os.path.join(folder, "s2.safetensors"))
     with pytest.raises(SafetensorsError, match="missing safetensors shard"):
-        Checkpoint(folder)
+        check_folder(folder)

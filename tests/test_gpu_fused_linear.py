@@ -377,34 +377,31 @@ def test_unsupported_sizes_are_refused(ops):
 
 @pytest.mark.parametrize("K", [1024, 2048])
 @pytest.mark.parametrize("R", [1, 8, 17, 64])
-def test_output_head_at_the_real_vocabulary(R, K):
-    """Final norm and output product the way the model's head runs them for few wanted rows
-    (``parts.embedding._head_fused`` -> ``norm_linear``), at 65,536 columns: wider than the
-    k-sliced kernels take, so up to 8 rows go to the kernel that keeps its rows in LDS and 9
-    to 64 rows to the one that streams the weights.  Rows picked out of a longer stream."""
-    from types import SimpleNamespace
-    from celeg_amd.engine import make_runtime
-    from celeg_amd.parts.embedding import _head_fused
-    from celeg_amd.parts.norm import RmsNorm
-    from celeg_amd.config.spec import PartSpec
+def test_output_head_at_the_real_vocabulary(tmp_path, R, K):
+    """Final norm and output product the way the model's head runs them for few wanted rows, at
+    65,536 columns: wider than the k-sliced kernels take, so up to 8 rows go to the kernel that
+    keeps its rows in LDS and 9 to 64 rows to the one that streams the weights.  Rows picked out
+    of a longer step, through a model of one convolution layer of that width."""
+    from celeg_amd.engine import StepEntry, load_model
+    from celeg_amd.weights import write_random_model
+    from helpers import assert_close_bf16, random_tokens
     V = 65536
-    rt = make_runtime(DEV, BF)
+    cfg = {"architectures": ["Lfm2ForCausalLM"], "vocab_size": V, "hidden_size": K, "num_hidden_layers": 1,
+           "layer_types": ["conv"], "num_attention_heads": K // 64, "num_key_value_heads": 8, "head_dim": 64,
+           "intermediate_size": 256, "block_auto_adjust_ff_dim": False, "rope_theta": 1e6, "conv_L_cache": 3,
+           "conv_bias": False, "tie_word_embeddings": K == 1024, "norm_eps": 1e-5, "max_position_embeddings": 128}
+    folder = write_random_model(cfg, str(tmp_path / "head"), seed=R, dtype=BF, std=0.05)
+    pcfg, W = plain.load_model_folder(folder)
     T = R + 5 if R < 64 else 64
-    h = randn(T, K, seed=60)
-    norm = RmsNorm(PartSpec("rmsnorm", {"width": K, "eps": 1e-5}))
-    norm.weight = 1 + randn(K, seed=61, scale=0.1)
-    w = randn(V, K, seed=62, scale=0.05, dtype=BF)
-    picked = [(3 * i + 1) % T for i in range(R)]
-    rows = torch.tensor(picked, dtype=torch.int32, device=DEV)
-    batch = SimpleNamespace(n_tokens=T, n_logit_rows=R, logit_rows=rows)
-    out = torch.full((R, V), float("nan"), device=DEV)
-    rt.stream_stat_blocks = 0
-    assert _head_fused(h, norm, batch, out, rt, w)
-    x = plain.rmsnorm(h.cpu(), norm.weight.cpu(), 1e-5)[picked].to(BF).float()
-    ref = x @ w.float().cpu().T            # exact products of bfloat16 values, summed in 32-bit
-    got = out.cpu()
-    assert torch.isfinite(got).all()
-    bound = 8e-3 * float(ref.abs().max())   # the norm weight folded into bfloat16 weights costs a rounding
-    assert float((got - ref).abs().max()) <= bound, float((got - ref).abs().max())
+    tokens = random_tokens(V, T, seed=60 + R)
+    picked = sorted({(3 * i + 1) % T for i in range(R)}) if R < 64 else list(range(64))
+    lm = load_model(folder, dtype="bfloat16", page_tokens=16, n_pages=8, max_requests=1, max_batched_tokens=64)
+    slot = lm.cache.open()
+    assert lm.cache.prepare(slot, 0, T)
+    got = lm.runner.step([StepEntry(slot, 0, tokens, picked)])
+    assert got.shape == (len(picked), V)
+    ref = plain.model_logits(pcfg, W, tokens)[picked]
+    assert_close_bf16(got, ref, f"head R={R} K={K}")
     # the last columns and rows are there
-    assert float((got[-1, -64:] - ref[-1, -64:]).abs().max()) <= bound
+    assert_close_bf16(got[-1:, -64:], ref[-1:, -64:], "head, last columns")
+    lm.close()

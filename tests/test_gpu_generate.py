@@ -65,12 +65,11 @@ def test_greedy_generation_through_the_entry_point(model_folders, name, dtype):
 
 
 @pytest.mark.parametrize("name", ["B", "D"])
-def test_generation_through_replayed_mixed_steps(model_folders, name):
+def test_generation_under_a_steady_load_of_portions_beside_decoding(model_folders, name):
     """A steady load through the entry point: ten requests of equal length under a budget that
     holds one portion and the decoding requests, a granule for the portions the budget cuts.
-    The steps' shapes repeat and are replayed from recorded graphs, with the tokens of the
-    decoding requests taken on the device (steps launched one ahead); every request's tokens
-    equal the plain implementation's greedy ones."""
+    Most steps carry a portion of one prompt beside the single tokens of the decoding requests;
+    every request's tokens equal the plain implementation's greedy ones."""
     from celeg_amd.engine import Engine
     from celeg_amd.sampling import GREEDY
     folder = model_folders(name, torch.float32, WEIGHT_STD)
@@ -79,9 +78,8 @@ def test_generation_through_replayed_mixed_steps(model_folders, name):
     prompts = [random_tokens(vocab, 96, seed=300 + i) for i in range(10)]
     engine = Engine.from_folder(folder, dtype="float32", max_active_requests=4, n_pages=64,
                                 max_batched_tokens=52, prefill_chunk_tokens=48, portion_granule=8)
-    engine.loaded.runner.MIXED_SEEN_BEFORE_RECORDING = 2
     outs = engine.generate(prompts, max_new_tokens=12, generation=GREEDY, eos_token_ids=[])
-    assert engine.loaded.runner._mixed_graphs, "no step of portions beside single tokens was replayed"
+    assert engine.metrics["scheduler"]["mixed_steps"] > 10, "no step held portions beside single tokens"
     for prompt, out in zip(prompts, outs):
         assert out == plain_generate(cfg, W, prompt, 12)
     assert engine.loaded.cache.free_pages() == [64] and engine.loaded.cache.n_free_slots == 4
@@ -113,7 +111,7 @@ def test_generation_with_few_pages_preempts_and_keeps_the_tokens(model_folders):
     engine = Engine.from_folder(folder, dtype="float32", max_active_requests=3, n_pages=6,
                                 max_batched_tokens=64, prefill_chunk_tokens=32)
     outs = engine.generate(prompts, max_new_tokens=40, generation=GREEDY, eos_token_ids=[])
-    assert engine.scheduler.stats["preemptions"] > 0
+    assert engine.metrics["scheduler"]["preemptions"] > 0
     for prompt, out in zip(prompts, outs):
         assert out == plain_generate(cfg, W, prompt, 40)
 
@@ -150,6 +148,16 @@ def test_command_line(model_folders, tmp_path):
 def ops():
     from celeg_amd.csrc.hip_ops import HipOps
     return HipOps(DEV)
+
+
+def sample_with_draw(logits, temperature, top_k, top_p, penalty, seen, u):
+    """The plain sampler with the draw in [0, 1) given instead of taken from its generator."""
+    generator = plain.random_unit
+    plain.random_unit = lambda state: (state, u)
+    try:
+        return plain.sample(logits, temperature, top_k, top_p, penalty, seen, 1)[0]
+    finally:
+        plain.random_unit = generator
 
 
 def run_sample(ops, logits, rows, all_greedy=False):
@@ -191,12 +199,11 @@ def test_sampling_kernel_equals_plain_sampler(ops, vocab):
             (0.5, 17, 0.5, 1.0, 0.999, None), (0.0, 50, 1.0, 1.7, 0.0, seen[3]),
             (2.0, 128, 0.95, 1.1, 0.05, seen[4]), (1.3, 2, 1.0, 1.0, 0.5, None)]
     got = run_sample(ops, logits, rows)
-    import cpu_ops
     for r, (t, k, p, pen, u, s) in enumerate(rows):
         flags = [False] * vocab
         for tok in (s or []):
             flags[tok] = True
-        want = cpu_ops._sample_with_draw(plain, logits[r].tolist(), t, k, p, pen, flags, u)
+        want = sample_with_draw(logits[r].tolist(), t, k, p, pen, flags, u)
         assert got[r] == want, f"row {r}"
 
 
@@ -246,23 +253,28 @@ def test_mark_seen(ops):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_steps_launched_ahead_of_their_tokens_give_the_same_tokens(model_folders, dtype):
     """Decode steps that take their input token on the device from what the previous step
-    sampled, launched before the host has read it, against steps the host feeds one by one."""
-    import torch
-    from celeg_amd.engine import load_model
+    sampled, launched before the host has read it (the loop that the benchmark times), against
+    steps the host feeds one by one."""
+    from celeg_amd.engine import Engine, RequestStatus
     from celeg_amd.engine.benchmark import DecodeBench
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders("B", storage, 0.05)
     runs = {}
-    for pipelined in (False, True):
-        lm = load_model(folder, dtype=dtype, page_tokens=16, n_pages=64, max_requests=4,
-                        max_batched_tokens=64)
-        bench = DecodeBench(lm, 3, 20, seed=5, prefill_chunk=16)
-        bench.run(steps=40, warmup=7, pipelined=pipelined)
-        runs[pipelined] = bench.generated
-        assert len(bench.generated) == 47 and all(len(t) == 3 for t in bench.generated)
+    for ahead in (False, True):
+        engine = Engine.from_folder(folder, dtype=dtype, page_tokens=16, n_pages=64, max_active_requests=4,
+                                    max_batched_tokens=64, prefill_chunk_tokens=16, run_ahead=ahead)
+        bench = DecodeBench(engine, 3, 20, new_tokens=60, seed=5)
+        bench.run(steps=7, warmup=0)
+        result = bench.run(steps=40, warmup=0)
+        assert result["steps"] == 40 and result["tokens"] == 120
+        assert (engine.metrics["steps_ahead"] > 30) == ahead
+        runs[ahead] = [engine.poll(r)[1] for r in bench.ids]
+        assert all(engine.status(r) == RequestStatus.DECODING for r in bench.ids)
+        assert all(len(t) >= 47 for t in runs[ahead])
         bench.close()
-        lm.cache.check()
-    assert runs[True] == runs[False]
+        engine.loaded.cache.check()
+        assert engine.loaded.cache.n_free_slots == 4 and engine.loaded.cache.free_pages() == [64]
+    assert [t[:47] for t in runs[True]] == [t[:47] for t in runs[False]]
 
 
 def test_generation_ahead_of_the_tokens_with_requests_that_end_early(model_folders):
@@ -281,8 +293,7 @@ def test_generation_ahead_of_the_tokens_with_requests_that_end_early(model_folde
     outs = {}
     for ahead in (True, False):
         engine = Engine.from_folder(folder, dtype="float32", max_active_requests=4, n_pages=24,
-                                    max_batched_tokens=64, prefill_chunk_tokens=32)
-        engine.run_ahead = ahead
+                                    max_batched_tokens=64, prefill_chunk_tokens=32, run_ahead=ahead)
         outs[ahead] = engine.generate(prompts, max_new_tokens=24, generation=GREEDY, eos_token_ids=eos)
         assert (engine.metrics["steps_ahead"] > 10) == ahead
         assert engine.loaded.cache.free_pages() == [24] and engine.loaded.cache.n_free_slots == 4

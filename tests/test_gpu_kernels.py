@@ -159,42 +159,20 @@ def test_library_product_called_directly(ops, M, N, K):
 
 
 # ---------------------------------------------------------------- cache-backed kernels
-def make_cache(kv_heads, head_dim, n_layers, dtype, n_pages=64, page_tokens=16, slots=4,
-               states=(), max_context=512):
-    from celeg_amd.cache import CacheLayout, CacheManager
-    from celeg_amd.parts.base import KVNeed
-    layout = CacheLayout()
-    if kv_heads:
-        layout.kv_groups = [KVNeed(kv_heads, head_dim)]
-        layout.group_layers = [n_layers]
-        layout.kv_of_step = {i: (0, i, True) for i in range(n_layers)}
-    layout.states = list(states)
-    return CacheManager(layout, page_tokens=page_tokens, n_pages=n_pages, max_requests=slots,
-                        max_context=max_context, device=DEV, dtype=dtype)
-
-
-def build_batch(ops, cache, entries):
-    from celeg_amd.engine.batch import BatchBuilder
-    builder = BatchBuilder(DEV, 1 << 16, len(cache.groups), pin=True)
-    batch = builder.build(entries, cache.drain_table_updates(), null_slot=cache.null_slot)
-    for g, (upd, cap) in enumerate(zip(batch.table_updates, batch.table_update_caps)):
-        if cap:
-            ops.apply_table_updates(cache.groups[g].table, upd, cap)
-    return batch, builder
+from kernel_harness import build_batch, make_cache  # noqa: E402
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width,taps,bias", [(2, 3, False), (96, 5, True), (1030, 4, False), (64, 1, True)])
 def test_short_conv_whole_chunked_and_token_by_token(ops, dtype, width, taps, bias):
     from celeg_amd.engine import StepEntry
-    from celeg_amd.parts.base import StateNeed
     T = 23
     bcx = randn(T, 3 * width, seed=12, dtype=dtype)
     w = randn(width, taps, seed=13)
     b = randn(width, seed=14) if bias else None
     ref = plain.short_conv(bcx.cpu(), w.cpu(), b.cpu() if bias else None)
     for cuts in ([T], [1] * T, [7, 2, 1, 9, 4], [3, 20], [20, 3], [1, 1, 21]):
-        cache = make_cache(0, 0, 0, dtype, states=[(0, StateNeed("bx", (taps, width)))])
+        cache = make_cache(0, 0, 0, dtype, states=[(0, "bx", (taps, width))])
         slot_other = cache.open()     # a neighbour slot whose state must stay zero
         slot = cache.open()
         state = cache.layer_cache(0).states["bx"]
@@ -222,12 +200,11 @@ def test_short_conv_long_portions_of_several_requests(ops, dtype, width, taps, b
     two requests per step, so that blocks of eight tokens straddle the border between them, begin
     at a request's first token, and continue from its state at positions inside a block."""
     from celeg_amd.engine import StepEntry
-    from celeg_amd.parts.base import StateNeed
     lengths = [131, 77]
     data = [randn(n, 3 * width, seed=60 + i, dtype=dtype) for i, n in enumerate(lengths)]
     w = randn(width, taps, seed=63)
     b = randn(width, seed=64) if bias else None
-    cache = make_cache(0, 0, 0, dtype, states=[(0, StateNeed("bx", (taps, width)))], slots=4)
+    cache = make_cache(0, 0, 0, dtype, states=[(0, "bx", (taps, width))], slots=4)
     slots = [cache.open() for _ in lengths]
     state = cache.layer_cache(0).states["bx"]
     got = [[] for _ in lengths]
@@ -261,8 +238,7 @@ def test_short_conv_reference_vector(ops):
     # tests/reference_test.cpp:68-73: hidden 2, L 3, bcx {1,1 | 1,1 | 2,4}, weights
     # {1,2,3 ; 1,2,3} channel-major, position 0, zero state -> {6, 12}
     from celeg_amd.engine import StepEntry
-    from celeg_amd.parts.base import StateNeed
-    cache = make_cache(0, 0, 0, torch.float32, states=[(0, StateNeed("bx", (3, 2)))])
+    cache = make_cache(0, 0, 0, torch.float32, states=[(0, "bx", (3, 2))])
     slot = cache.open()
     batch, keep = build_batch(ops, cache, [StepEntry(slot, 0, [0])])
     bcx = torch.tensor([[1., 1., 1., 1., 2., 4.]], device=DEV)
@@ -279,12 +255,11 @@ def test_short_conv_vector_tells_the_three_thirds_of_bcx_apart(ops, dtype):
     # taps {2,1} -> {30, 1221} (the filter reversed: 2112).  In one step, and token by token
     # through the saved state.  All values are exact in bfloat16 except 1111 and 1221.
     from celeg_amd.engine import StepEntry
-    from celeg_amd.parts.base import StateNeed
     rows = torch.tensor([[2., 3., 5.], [7., 11., 13.]], device=DEV).to(dtype)
     for taps, want in (([1., 1.], [30., 1111.]), ([2., 1.], [30., 1221.])):
         w = torch.tensor([taps], device=DEV)
         for cuts in ([2], [1, 1]):
-            cache = make_cache(0, 0, 0, dtype, states=[(0, StateNeed("bx", (2, 1)))])
+            cache = make_cache(0, 0, 0, dtype, states=[(0, "bx", (2, 1))])
             slot = cache.open()
             got, pos = [], 0
             for c in cuts:
@@ -332,7 +307,7 @@ def test_q_and_k_are_normalised_before_they_are_rotated(ops, dtype, head_dim):
     ops.qk_norm_rope_store(q, k, v, weight, weight, 0.0, inv_freq.to(DEV), head_dim, 1, 1, head_dim,
                            batch, kv)
     torch.cuda.synchronize()
-    page = int(cache.groups[0].table_host[slot, 0])
+    page = cache.table_host(slot, 0)
     stored_k = kv.k[page, 0, 0, 1].float().cpu()            # [page, layer, head, token, :]
     bound = (1e-5 if dtype == torch.float32 else 2e-2) * s
     for got in (q[1].float().cpu(), stored_k):
@@ -561,16 +536,10 @@ def test_window_attention_never_reads_pages_it_has_given_back(ops, head_dim, pag
     first round of 64 keys of a tile starts at a multiple of 64, before the window's first
     key: the kernel must stay on the request's live pages there (a masked key has probability
     zero, and zero times infinity is not a number)."""
-    from celeg_amd.cache import CacheLayout, CacheManager
     from celeg_amd.engine import StepEntry
-    from celeg_amd.parts.base import KVNeed
     window, heads, kv_heads = 40, 2, 1
-    layout = CacheLayout()
-    layout.kv_groups = [KVNeed(kv_heads, head_dim, window)]
-    layout.group_layers = [1]
-    layout.kv_of_step = {0: (0, 0, True)}
-    cache = CacheManager(layout, page_tokens=page_tokens, n_pages=24, max_requests=2, max_context=512,
-                         device=DEV, dtype=torch.bfloat16)
+    cache = make_cache(kv_heads, head_dim, 1, torch.bfloat16, n_pages=24, page_tokens=page_tokens, slots=2,
+                       max_context=512, window=window)
     kv = cache.layer_cache(0).kv
     n = 330
     q = randn(n, heads * head_dim, seed=70, dtype=torch.bfloat16)

@@ -1,8 +1,15 @@
 """Each part of a layer alone against its plain function, and the generality of the
-assembly: a toy mixer with state of its own and a toy architecture, defined here, are
-registered, built and stepped without touching the framework's files; a run order that
-names a layer twice and lets a layer read another layer's cache."""
-import dataclasses
+assembly: toy parts defined here (a mixer with state of its own, a feed-forward with routing,
+another position encoding) and toy architectures are registered through the library's
+interface, built and stepped without touching the framework's files; a run order that names a
+layer twice and lets a layer read another layer's cache.
+
+A part runs alone inside a block whose other parts are the neutral ones ("identity" norm,
+"none" mixer or feed-forward) under the head "hidden", which gives the rows of the stream
+back: with the inputs as the embedding table and the tokens 0..T-1 the step returns
+x + part(x), cut into steps like any other model.
+"""
+import json
 import os
 
 import pytest
@@ -10,172 +17,172 @@ import torch
 
 import plain_lfm2 as plain
 from conftest import TINY
-from helpers import WEIGHT_STD, EngineDriver, assert_close_f32, portions_schedule, random_tokens
+from helpers import (WEIGHT_STD, EngineDriver, assert_close_f32, portions_schedule, random_tokens,
+                     reordered_lfm2)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def runtime(dtype=torch.float32):
-    from celeg_amd.engine import make_runtime
-    return make_runtime(DEV, dtype)
+def write_folder(folder, cfg, replace=None, seed=0, std=0.2):
+    """A model folder of random 32-bit tensors for ``cfg`` (what the library says the model
+    wants), some of them replaced."""
+    from celeg_amd import native
+    from celeg_amd.weights import random_tensors
+    from celeg_amd.weights.safetensors_io import write_safetensors
+    expected = native.describe_config(cfg)["expected_tensors"]
+    tensors = random_tensors(expected, seed, std, torch.float32)
+    for name, t in (replace or {}).items():
+        assert tensors[name].shape == t.shape
+        tensors[name] = t.float().contiguous()
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(cfg, fh)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    return folder, tensors
 
 
-def one_request_batch(rt, cache, slot, start, n):
-    from celeg_amd.engine.batch import BatchBuilder
-    from celeg_amd.engine import StepEntry
-    assert cache.prepare(slot, start, n)
-    builder = BatchBuilder(DEV, 1 << 14, len(cache.groups), pin=True)
-    batch = builder.build([StepEntry(slot, start, [0] * n)], cache.drain_table_updates(),
-                          null_slot=cache.null_slot)
-    for g, (upd, cap) in enumerate(zip(batch.table_updates, batch.table_update_caps)):
-        if cap:
-            rt.ops.apply_table_updates(cache.groups[g].table, upd, cap)
-    return batch
+def parts_alone_architecture():
+    """"PartsAlone": one block of the parts that the configuration spells out, neutral ones
+    where it says nothing; the embedding table is the input, the head returns the stream."""
+    from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
+    if "PartsAlone" in registered_architectures():
+        return
+
+    def build(cfg, shapes):
+        H, rows = cfg["width"], cfg["rows"]
+        part = lambda key, neutral: PartSpec.from_json(cfg[key]) if cfg.get(key) else neutral
+        layer = LayerSpec(part("mixer", PartSpec("none", {"width": H})), part("mixer_norm", PartSpec("identity")),
+                          part("ffn", PartSpec("none")), part("ffn_norm", PartSpec("identity")))
+        return ModelSpec("PartsAlone", rows, H, 256, PartSpec("embedding", {"vocab": rows, "width": H}, {"table": "x"}),
+                         (layer,), (RunStep(0),), part("final_norm", PartSpec("identity")),
+                         PartSpec("hidden", {"width": H}))
+    register_architecture("PartsAlone", build)
 
 
-def build_mixer(spec, rt, seed=0):
-    """A mixer alone: built from its PartSpec, random tensors, and a cache of its own."""
-    from celeg_amd.cache import CacheLayout, CacheManager
-    from celeg_amd.parts import build_part
-    from celeg_amd.weights import random_tensor
-    mixer = build_part("mixer", spec)
-    tensors = {role: random_tensor(seed, role, w.shape, w.init, 0.2).to(DEV)
-               for role, w in mixer.weight_specs().items()}
-    mixer.load(dict(tensors), rt)
-    layout = CacheLayout()
-    if mixer.kv_need() is not None:
-        layout.kv_groups, layout.group_layers = [mixer.kv_need()], [1]
-        layout.kv_of_step = {0: (0, 0, True)}
-    layout.states = [(0, s) for s in mixer.state_needs()]
-    cache = CacheManager(layout, page_tokens=16, n_pages=16, max_requests=2, max_context=256,
-                         device=DEV, dtype=rt.dtype)
-    return mixer, tensors, cache
-
-
-def run_mixer_in_cuts(mixer, cache, rt, x, cuts):
-    slot = cache.open()
+def run_part_alone(tmp_path, x, cuts, **parts):
+    """x + part(x) (or norm(x)) for the rows of x fed in steps of ``cuts`` rows, and the
+    folder's tensors."""
+    from celeg_amd.engine import StepEntry, load_model
+    parts_alone_architecture()
+    cfg = {"architectures": ["PartsAlone"], "width": x.shape[1], "rows": x.shape[0]}
+    cfg.update({k: v.to_json() for k, v in parts.items()})
+    folder, tensors = write_folder(str(tmp_path / "alone"), cfg, {"x": x})
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=16, max_requests=2, max_batched_tokens=64)
+    slot = lm.cache.open()
     outs, pos = [], 0
     for n in cuts:
-        batch = one_request_batch(rt, cache, slot, pos, n)
-        outs.append(mixer.forward(x[pos:pos + n].contiguous(), batch, cache.layer_cache(0), rt).clone())
+        assert lm.cache.prepare(slot, pos, n)
+        outs.append(lm.runner.step([StepEntry(slot, pos, list(range(pos, pos + n)), list(range(n)))]))
         pos += n
-    cache.close(slot)
-    return torch.cat(outs).double().cpu()
+    lm.cache.close(slot)
+    lm.cache.check()
+    lm.close()
+    return torch.cat(outs).double(), tensors
 
 
-def test_short_conv_mixer_alone():
+def test_short_conv_mixer_alone(tmp_path):
     from celeg_amd.config import PartSpec
-    rt = runtime()
-    spec = PartSpec("short_conv", {"width": 40, "taps": 4, "bias": True})
-    mixer, t, cache = build_mixer(spec, rt)
-    x = torch.randn(29, 40, generator=torch.Generator().manual_seed(1)).to(DEV)
-    W = {"conv.in_proj.weight": t["in_proj"], "conv.in_proj.bias": t["in_proj_bias"],
-         "conv.conv.weight": t["conv"], "conv.conv.bias": t["conv_bias"],
-         "conv.out_proj.weight": t["out_proj"], "conv.out_proj.bias": t["out_proj_bias"]}
-    ref = plain.conv_mixer(x.cpu(), {k: v.cpu() for k, v in W.items()}, "", True)
-    for cuts in ([29], [5, 1, 2, 21]):
-        torch.testing.assert_close(run_mixer_in_cuts(mixer, cache, rt, x, cuts), ref, rtol=1e-4, atol=1e-5)
+    names = {"in_proj": "conv.in_proj.weight", "in_proj_bias": "conv.in_proj.bias", "conv": "conv.conv.weight",
+             "conv_bias": "conv.conv.bias", "out_proj": "conv.out_proj.weight", "out_proj_bias": "conv.out_proj.bias"}
+    spec = PartSpec("short_conv", {"width": 40, "taps": 4, "bias": True}, names)
+    x = torch.randn(29, 40, generator=torch.Generator().manual_seed(1))
+    for i, cuts in enumerate(([29], [5, 1, 2, 21])):
+        got, W = run_part_alone(tmp_path / str(i), x, cuts, mixer=spec)
+        ref = plain.conv_mixer(x, W, "", True)
+        torch.testing.assert_close(got - x.double(), ref, rtol=1e-4, atol=1e-5)
 
 
 @pytest.mark.parametrize("window", [None, 7])
-def test_attention_mixer_alone(window):
+def test_attention_mixer_alone(tmp_path, window):
     from celeg_amd.config import PartSpec
-    rt = runtime()
-    cfg = {"num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 16, "norm_eps": 1e-5,
-           "rope_theta": 1e4}
+    cfg = {"num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 16, "norm_eps": 1e-5, "rope_theta": 1e4}
+    names = {"q_proj": "self_attn.q_proj.weight", "k_proj": "self_attn.k_proj.weight", "v_proj": "self_attn.v_proj.weight",
+             "out_proj": "self_attn.out_proj.weight", "q_norm": "self_attn.q_layernorm.weight",
+             "k_norm": "self_attn.k_layernorm.weight"}
     spec = PartSpec("gqa_attention", {
         "width": 40, "heads": 6, "kv_heads": 2, "head_dim": 16, "qk_norm": True, "eps": 1e-5,
-        "window": window, "position": PartSpec("rope", {"theta": 1e4, "head_dim": 16})})
-    mixer, t, cache = build_mixer(spec, rt)
-    x = torch.randn(37, 40, generator=torch.Generator().manual_seed(2)).to(DEV)
-    W = {"self_attn.q_proj.weight": t["q_proj"], "self_attn.k_proj.weight": t["k_proj"],
-         "self_attn.v_proj.weight": t["v_proj"], "self_attn.out_proj.weight": t["out_proj"],
-         "self_attn.q_layernorm.weight": t["q_norm"], "self_attn.k_layernorm.weight": t["k_norm"]}
-    ref, _ = plain.attention_mixer(x.cpu(), {k: v.cpu() for k, v in W.items()}, "", cfg,
-                                   list(range(37)), window=window)
-    for cuts in ([37], [9, 1, 1, 20, 6]):
-        torch.testing.assert_close(run_mixer_in_cuts(mixer, cache, rt, x, cuts), ref, rtol=1e-4, atol=1e-5)
+        "window": window, "position": PartSpec("rope", {"theta": 1e4, "head_dim": 16})}, names)
+    x = torch.randn(37, 40, generator=torch.Generator().manual_seed(2))
+    for i, cuts in enumerate(([37], [9, 1, 1, 20, 6])):
+        got, W = run_part_alone(tmp_path / str(i), x, cuts, mixer=spec)
+        ref, _ = plain.attention_mixer(x, W, "", cfg, list(range(37)), window=window)
+        torch.testing.assert_close(got - x.double(), ref, rtol=1e-4, atol=1e-5)
 
 
-def test_attention_without_norm_or_rotation_is_library_attention():
+def test_attention_without_norm_or_rotation_is_library_attention(tmp_path):
     import torch.nn.functional as F
     from celeg_amd.config import PartSpec
-    rt = runtime()
-    spec = PartSpec("gqa_attention", {"width": 32, "heads": 2, "kv_heads": 2, "head_dim": 16,
-                                      "qk_norm": False, "position": PartSpec("none")})
-    mixer, t, cache = build_mixer(spec, rt)
-    x = torch.randn(21, 32, generator=torch.Generator().manual_seed(3)).to(DEV)
-    xd = x.double().cpu()
-    q, k, v = (F.linear(xd, t[n].double().cpu()).reshape(21, 2, 16).transpose(0, 1)[None]
-               for n in ("q_proj", "k_proj", "v_proj"))
+    spec = PartSpec("gqa_attention", {"width": 32, "heads": 2, "kv_heads": 2, "head_dim": 16, "qk_norm": False,
+                                      "position": PartSpec("none")},
+                    {"q_proj": "q", "k_proj": "k", "v_proj": "v", "out_proj": "o"})
+    x = torch.randn(21, 32, generator=torch.Generator().manual_seed(3))
+    got, W = run_part_alone(tmp_path, x, [4, 17], mixer=spec)
+    xd = x.double()
+    q, k, v = (F.linear(xd, W[n].double()).reshape(21, 2, 16).transpose(0, 1)[None] for n in ("q", "k", "v"))
     att = F.scaled_dot_product_attention(q, k, v, is_causal=True)[0].transpose(0, 1).reshape(21, 32)
-    ref = F.linear(att, t["out_proj"].double().cpu())
-    torch.testing.assert_close(run_mixer_in_cuts(mixer, cache, rt, x, [4, 17]), ref, rtol=1e-4, atol=1e-5)
+    ref = F.linear(att, W["o"].double())
+    torch.testing.assert_close(got - xd, ref, rtol=1e-4, atol=1e-5)
 
 
-def test_feed_forward_and_norm_alone():
+def test_feed_forward_and_norm_alone(tmp_path):
     from celeg_amd.config import PartSpec
-    from celeg_amd.parts import build_part
-    from celeg_amd.weights import random_tensor
-    rt = runtime()
-    ffn = build_part("ffn", PartSpec("swiglu", {"width": 24, "ff": 50}))
-    t = {r: random_tensor(0, r, w.shape, w.init, 0.3).to(DEV) for r, w in ffn.weight_specs().items()}
-    ffn.load(dict(t), rt)
-    x = torch.randn(9, 24, generator=torch.Generator().manual_seed(4)).to(DEV)
-    ref = plain.swiglu_ffn(x.cpu(), t["gate"].cpu(), t["up"].cpu(), t["down"].cpu())
-    torch.testing.assert_close(ffn.forward(x, None, rt).double().cpu(), ref, rtol=1e-4, atol=1e-5)
-    norm = build_part("norm", PartSpec("rmsnorm", {"width": 24, "eps": 1e-3}))
-    w = (1 + 0.1 * torch.randn(24)).to(DEV)
-    norm.load({"weight": w}, rt)
-    out = torch.empty_like(x)
-    norm.forward(x.clone(), out, rt)
-    torch.testing.assert_close(out.double().cpu(), plain.rmsnorm(x.cpu(), w.cpu(), 1e-3), rtol=1e-5, atol=1e-6)
+    x = torch.randn(9, 24, generator=torch.Generator().manual_seed(4))
+    ffn = PartSpec("swiglu", {"width": 24, "ff": 50}, {"gate": "g", "up": "u", "down": "d"})
+    got, W = run_part_alone(tmp_path / "ffn", x, [9], ffn=ffn)
+    ref = plain.swiglu_ffn(x, W["g"], W["u"], W["d"])
+    torch.testing.assert_close(got - x.double(), ref, rtol=1e-4, atol=1e-5)
+    norm = PartSpec("rmsnorm", {"width": 24, "eps": 1e-3}, {"weight": "w"})
+    got, W = run_part_alone(tmp_path / "norm", x, [4, 5], final_norm=norm)
+    torch.testing.assert_close(got, plain.rmsnorm(x, W["w"], 1e-3), rtol=1e-5, atol=1e-6)
+    # the norm in front of a part: the feed-forward of the normalised rows, added to the rows
+    got, W = run_part_alone(tmp_path / "both", x, [3, 6], ffn=ffn, ffn_norm=norm)
+    ref = x.double() + plain.swiglu_ffn(plain.rmsnorm(x, W["w"], 1e-3), W["g"], W["u"], W["d"])
+    torch.testing.assert_close(got, ref, rtol=1e-4, atol=1e-5)
 
 
 # ---------------------------------------------------------------- a toy mixer and architecture
 def register_toy():
     """A mixer whose state is its own: the running sum of its inputs and their count.
-    out[t] = (sum of x[0..t]) / (t+1) @ W^T.  It is written with torch (a toy may be) and
-    plans on the host from the batch's host arrays."""
-    from celeg_amd.config import (Architecture, LayerSpec, ModelSpec, PartSpec, RunStep,
-                                  register_architecture, registered_architectures)
-    from celeg_amd.parts import Mixer, StateNeed, WeightSpec, register_part, registered_parts
+    out[t] = (sum of x[0..t]) / (t+1) @ W^T.  It is written with torch (a toy may be), on the
+    memory the library hands it, and plans on the host from the step's host arrays."""
+    from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
+    from celeg_amd.parts import as_tensor, on_stream, register_part, registered_parts
 
-    class RunningMean(Mixer):
+    class RunningMean:
         def __init__(self, spec):
-            super().__init__(spec)
-            self.width = int(self.params["width"])
+            self.width = int(spec["params"]["width"])
             self.w = None
 
-        def state_needs(self):
-            return [StateNeed("sum", (self.width,), torch.float32),
-                    StateNeed("count", (1,), torch.float32)]
+        def describe(self):
+            return {"weights": {"proj": {"shape": [self.width, self.width]}},
+                    "states": [{"name": "sum", "shape": [self.width], "dtype": "float32"},
+                               {"name": "count", "shape": [1], "dtype": "float32"}],
+                    "graph_safe": False, "out_width": self.width}
 
-        def weight_specs(self):
-            return {"proj": WeightSpec((self.width, self.width))}
+        def load(self, tensors):
+            self.w = as_tensor(tensors["proj"])
 
-        def load(self, tensors, rt):
-            self.w = tensors["proj"]
-
-        def forward(self, x, batch, cache, rt):
-            out = rt.ws.buf("toy_out", (x.shape[0], self.width), rt.dtype)
-            total, count = cache.states["sum"], cache.states["count"]
-            cu = batch.host["cu_seqlens"]
-            for s in range(batch.n_seqs):
-                slot = int(batch.host["seq_slot"][s])
-                rows = x[cu[s]:cu[s + 1]].float()
-                running = total[slot] + torch.cumsum(rows, dim=0)
-                n = count[slot] + torch.arange(1, rows.shape[0] + 1, device=x.device)[:, None]
-                out[cu[s]:cu[s + 1]] = ((running / n) @ self.w.float().t()).to(rt.dtype)
-                total[slot] = running[-1]
-                count[slot] = n[-1]
-            return out
+        def forward(self, args):
+            with on_stream(args):
+                x, out = as_tensor(args.x), as_tensor(args.out)
+                states = {args.cache.state_names[i].decode(): as_tensor(args.cache.states[i])
+                          for i in range(args.cache.n_states)}
+                total, count = states["sum"], states["count"]
+                step = args.step
+                for s in range(step.n_seqs):
+                    slot, lo, hi = step.host_seq_slot[s], step.host_cu_seqlens[s], step.host_cu_seqlens[s + 1]
+                    rows = x[lo:hi].float()
+                    running = total[slot] + torch.cumsum(rows, dim=0)
+                    n = count[slot] + torch.arange(1, rows.shape[0] + 1, device=x.device)[:, None]
+                    out[lo:hi] = ((running / n) @ self.w.float().t()).to(out.dtype)
+                    total[slot] = running[-1]
+                    count[slot] = n[-1]
 
     if "running_mean" not in registered_parts("mixer"):
         register_part("mixer", "running_mean", RunningMean)
 
-    def build_spec(cfg):
+    def build_spec(cfg, shapes):
         H = cfg["width"]
         norm = lambda name: PartSpec("rmsnorm", {"width": H, "eps": 1e-5}, {"weight": name})
         layers = []
@@ -199,7 +206,7 @@ def register_toy():
                          norm("final"), PartSpec("tied_head", {"vocab": cfg["vocab"], "width": H}))
 
     if "ToyForCausalLM" not in registered_architectures():
-        register_architecture(Architecture("ToyForCausalLM", lambda d: d, build_spec))
+        register_architecture("ToyForCausalLM", build_spec)
 
 
 def toy_plain_logits(cfg, W, tokens):
@@ -235,14 +242,36 @@ def test_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path):
     reqs = {"x": random_tokens(77, 45, 1), "y": random_tokens(77, 30, 2)}
     lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2,
                     max_batched_tokens=64)
-    assert [n.name for _, n in lm.cache.layout.states] == ["sum", "count", "sum", "count"]
-    assert not lm.model.graph_safe      # the toy plans on the host: its steps are never replayed
+    assert [s["name"] for s in lm.cache.layout["states"]] == ["sum", "count", "sum", "count"]
+    assert not lm.graph_safe      # the toy plans on the host: its steps are never replayed
     got = EngineDriver(lm).run(portions_schedule(reqs))
-    got2 = EngineDriver(lm).run(portions_schedule(dict(reversed(list(reqs.items())))))   # slots reused
+    # the slots are used again by other requests: a new request starts from zeroed state
+    got2 = EngineDriver(lm).run(portions_schedule(dict(reversed(list(reqs.items())))))
     for rid, toks in reqs.items():
         ref = toy_plain_logits(cfg, W, toks)
         assert_close_f32(got[rid], ref, f"toy/{rid}")
         assert_close_f32(got2[rid], ref, f"toy again/{rid}")
+    assert lm.runner.counters()["graph_replays"] == 0
+
+
+def test_toy_model_generates_through_the_engine(tmp_path):
+    """The same toy model under the scheduler and the sampler: greedy tokens equal the plain ones."""
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY
+    from celeg_amd.weights import write_random_model
+    register_toy()
+    cfg = {"architectures": ["ToyForCausalLM"], "width": 32, "vocab": 77, "layers": ["attention", "mean"]}
+    folder = write_random_model(cfg, str(tmp_path / "toy"), seed=6, dtype=torch.float32, std=0.2)
+    _, W = plain.load_model_folder(folder)
+    prompts = [random_tokens(77, n, 10 + n) for n in (3, 19, 8)]
+    engine = Engine.from_folder(folder, dtype="float32", max_active_requests=2, n_pages=8, max_batched_tokens=16,
+                                prefill_chunk_tokens=8)
+    outs = engine.generate(prompts, max_new_tokens=6, generation=GREEDY, eos_token_ids=[])
+    for prompt, out in zip(prompts, outs):
+        seq = list(prompt)
+        for _ in range(6):
+            seq.append(int(toy_plain_logits(cfg, W, seq)[-1].argmax()))
+        assert out == seq[len(prompt):]
 
 
 # ---------------------------------------------------------------- a toy routed feed-forward and position encoding
@@ -252,58 +281,56 @@ def register_toy_routed():
     encoding whose frequencies are the usual ones divided by a factor (positions stretched).
     Both are registered here, from outside the framework, with an architecture that mixes
     routed and dense layers."""
-    from celeg_amd.config import (Architecture, LayerSpec, ModelSpec, PartSpec, RunStep,
-                                  register_architecture, registered_architectures)
-    from celeg_amd.parts import (FeedForward, PositionEncoding, WeightSpec, register_part,
-                                 registered_parts)
+    from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
+    from celeg_amd.parts import as_tensor, on_stream, register_part, registered_parts
 
-    class TopOneExperts(FeedForward):
+    class TopOneExperts:
         def __init__(self, spec):
-            super().__init__(spec)
-            self.width, self.ff = int(self.params["width"]), int(self.params["ff"])
-            self.experts = int(self.params["experts"])
+            p = spec["params"]
+            self.width, self.ff, self.experts = int(p["width"]), int(p["ff"]), int(p["experts"])
 
-        def weight_specs(self):
-            specs = {"router": WeightSpec((self.experts, self.width))}
+        def describe(self):
+            weights = {"router": {"shape": [self.experts, self.width]}}
             for e in range(self.experts):
-                specs[f"gate{e}"] = WeightSpec((self.ff, self.width))
-                specs[f"up{e}"] = WeightSpec((self.ff, self.width))
-                specs[f"down{e}"] = WeightSpec((self.width, self.ff))
-            return specs
+                weights[f"gate{e}"] = {"shape": [self.ff, self.width]}
+                weights[f"up{e}"] = {"shape": [self.ff, self.width]}
+                weights[f"down{e}"] = {"shape": [self.width, self.ff]}
+            return {"weights": weights, "graph_safe": False, "out_width": self.width}
 
-        def load(self, tensors, rt):
-            self.w = tensors
+        def load(self, tensors):
+            self.w = {role: as_tensor(view) for role, view in tensors.items()}
 
-        def forward(self, x, batch, rt):
-            xf = x.float()
-            choice = (xf @ self.w["router"].float().t()).argmax(dim=1)
-            out = rt.ws.buf("toy_routed_out", (x.shape[0], self.width), rt.dtype)
-            for e in range(self.experts):
-                rows = (choice == e).nonzero().flatten()
-                if rows.numel() == 0:
-                    continue
-                xe = xf[rows]
-                act = torch.nn.functional.silu(xe @ self.w[f"gate{e}"].float().t()) * (xe @ self.w[f"up{e}"].float().t())
-                out[rows] = (act @ self.w[f"down{e}"].float().t()).to(rt.dtype)
-            return out
+        def forward(self, args):
+            with on_stream(args):
+                x, out = as_tensor(args.x), as_tensor(args.out)
+                xf = x.float()
+                choice = (xf @ self.w["router"].float().t()).argmax(dim=1)
+                for e in range(self.experts):
+                    rows = (choice == e).nonzero().flatten()
+                    if rows.numel() == 0:
+                        continue
+                    xe = xf[rows]
+                    act = torch.nn.functional.silu(xe @ self.w[f"gate{e}"].float().t()) * (xe @ self.w[f"up{e}"].float().t())
+                    out[rows] = (act @ self.w[f"down{e}"].float().t()).to(out.dtype)
 
-    class StretchedRope(PositionEncoding):
+    class StretchedRope:
         def __init__(self, spec):
-            super().__init__(spec)
-            self.theta, self.factor = float(self.params["theta"]), float(self.params["factor"])
-            self.rotary_dim = int(self.params["rotary_dim"])
+            p = spec["params"]
+            self.theta, self.factor, self.rotary_dim = float(p["theta"]), float(p["factor"]), int(p["rotary_dim"])
 
-        def tables(self, rt):
-            freq = [self.theta ** (-2.0 * i / self.rotary_dim) / self.factor for i in range(self.rotary_dim // 2)]
-            return {"inv_freq": torch.tensor(freq, dtype=torch.float64).to(torch.float32).to(rt.device),
-                    "rotary_dim": self.rotary_dim}
+        def describe(self):
+            return {"inv_freq": [self.theta ** (-2.0 * i / self.rotary_dim) / self.factor
+                                 for i in range(self.rotary_dim // 2)], "rotary_dim": self.rotary_dim}
+
+        def forward(self, args):
+            raise RuntimeError("a position encoding gives tables; it is never called")
 
     if "toy_top_one" not in registered_parts("ffn"):
         register_part("ffn", "toy_top_one", TopOneExperts)
     if "toy_stretched_rope" not in registered_parts("position"):
         register_part("position", "toy_stretched_rope", StretchedRope)
 
-    def build_spec(cfg):
+    def build_spec(cfg, shapes):
         H, ff, E = cfg["width"], cfg["ff"], cfg["experts"]
         norm = lambda name: PartSpec("rmsnorm", {"width": H, "eps": 1e-5}, {"weight": name})
         layers = []
@@ -330,7 +357,7 @@ def register_toy_routed():
                          norm("final"), PartSpec("tied_head", {"vocab": cfg["vocab"], "width": H}))
 
     if "ToyRoutedForCausalLM" not in registered_architectures():
-        register_architecture(Architecture("ToyRoutedForCausalLM", lambda d: d, build_spec))
+        register_architecture("ToyRoutedForCausalLM", build_spec)
 
 
 def toy_routed_plain_logits(cfg, W, tokens):
@@ -401,29 +428,122 @@ def test_toy_routed_feed_forward_and_position_encoding_are_registered_and_steppe
     assert (other - ref).abs().max() > 1e-3
 
 
+def register_toy_that_fails():
+    """A feed-forward that copies its input and refuses a step of more than ``limit`` rows, in a
+    model of one block whose head gives the stream back: logits = 2 * embedding row."""
+    from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
+    from celeg_amd.parts import as_tensor, on_stream, register_part, registered_parts
+
+    class FailsOnManyRows:
+        def __init__(self, spec):
+            self.limit = int(spec["params"]["limit"])
+
+        def describe(self):
+            return {"graph_safe": False}
+
+        def forward(self, args):
+            if args.step.n_tokens > self.limit:
+                raise RuntimeError("too many rows for this toy")
+            with on_stream(args):
+                as_tensor(args.out).copy_(as_tensor(args.x))
+
+    if "toy_fails" not in registered_parts("ffn"):
+        register_part("ffn", "toy_fails", FailsOnManyRows)
+
+    def build(cfg, shapes):
+        H, V = cfg["width"], cfg["vocab"]
+        ident = PartSpec("identity")
+        layer = LayerSpec(PartSpec("none", {"width": H}), ident, PartSpec("toy_fails", {"limit": cfg["limit"]}), ident)
+        return ModelSpec("ToyFails", V, H, 64, PartSpec("embedding", {"vocab": V, "width": H}, {"table": "emb"}),
+                         (layer,), (RunStep(0),), ident, PartSpec("hidden", {"width": H}))
+    if "ToyFails" not in registered_architectures():
+        register_architecture("ToyFails", build)
+
+
+def test_a_part_that_fails_fails_the_step_and_nothing_else(tmp_path):
+    """A part whose forward raises: the step is refused with the part's name, the request's
+    slot can be closed, and the model steps other requests afterwards."""
+    from celeg_amd.engine import StepEntry, load_model
+    from celeg_amd.weights import write_random_model
+    register_toy_that_fails()
+    cfg = {"architectures": ["ToyFails"], "width": 16, "vocab": 20, "limit": 4}
+    folder = write_random_model(cfg, str(tmp_path / "fails"), seed=1, dtype=torch.float32, std=0.5)
+    _, W = plain.load_model_folder(folder)
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=4, max_requests=2, max_batched_tokens=32)
+    a, b = lm.cache.open(), lm.cache.open()
+    assert lm.cache.prepare(a, 0, 6) and lm.cache.prepare(b, 0, 3)
+    with pytest.raises(ValueError, match="toy_fails"):
+        lm.runner.step([StepEntry(a, 0, [1, 2, 3, 4, 5, 6], [5])])
+    lm.cache.close(a)
+    got = lm.runner.step([StepEntry(b, 0, [7, 8, 9], [0, 2])])
+    ref = 2 * W["emb"][[7, 9]].double()
+    torch.testing.assert_close(got.double(), ref, rtol=1e-6, atol=1e-6)
+    lm.cache.close(b)
+    lm.cache.check()
+    assert lm.cache.n_free_slots == 2
+
+
+def test_a_failed_step_fails_its_requests_and_the_engine_goes_on(tmp_path):
+    """Through the engine: a request whose step fails ends FAILED with the message, gives its slot
+    back, and requests before and after it finish with the right tokens
+    (src/runtime/concurrency/request_lifecycle.cpp:200-218)."""
+    from celeg_amd.engine import Engine, RequestOptions, RequestStatus
+    from celeg_amd.sampling import GREEDY
+    from celeg_amd.weights import write_random_model
+    register_toy_that_fails()
+    cfg = {"architectures": ["ToyFails"], "width": 16, "vocab": 20, "limit": 4}
+    folder = write_random_model(cfg, str(tmp_path / "fails"), seed=1, dtype=torch.float32, std=0.5)
+    _, W = plain.load_model_folder(folder)
+
+    def plain_tokens(prompt, n):       # greedy over logits = 2 * embedding row of the last token
+        seq = list(prompt)
+        for _ in range(n):
+            seq.append(int(W["emb"][seq[-1]].argmax()))
+        return seq[len(prompt):]
+
+    engine = Engine.from_folder(folder, dtype="float32", max_active_requests=2, n_pages=4, max_batched_tokens=8,
+                                prefill_chunk_tokens=8)
+    options = RequestOptions(max_new_tokens=5, eos_token_ids=[], generation=GREEDY)
+    first = engine.submit([3, 1, 4], options)
+    engine.run()
+    assert engine.poll(first) == (RequestStatus.FINISHED, plain_tokens([3, 1, 4], 5), "")
+    doomed = engine.submit([2, 7, 1, 8, 2, 8, 1], options)      # a portion of 7 rows: more than the toy takes
+    engine.run()
+    status, tokens, error = engine.poll(doomed)
+    assert status == RequestStatus.FAILED and tokens == [] and "toy_fails" in error
+    assert engine.metrics["failed_steps"] == 1
+    assert engine.loaded.cache.n_free_slots == 2
+    after = engine.submit([5, 9], options)
+    beside = engine.submit([6], options)
+    engine.run()
+    assert engine.poll(after) == (RequestStatus.FINISHED, plain_tokens([5, 9], 5), "")
+    assert engine.poll(beside) == (RequestStatus.FINISHED, plain_tokens([6], 5), "")
+    assert engine.loaded.cache.n_free_slots == 2
+    engine.loaded.cache.check()
+
+
 def test_run_order_with_a_layer_twice_and_a_shared_cache(model_folders, tmp_path):
     """LFM2 parts under another run order: layer 1 runs twice (own cache each time) and
     layer 3 reads the keys and values the first run of layer 1 wrote."""
-    from celeg_amd.cache import CacheManager
-    from celeg_amd.config import RunStep, spec_from_config
-    from celeg_amd.engine import Model, ModelRunner, make_runtime
-    from celeg_amd.engine.loading import LoadedModel
-    from celeg_amd.weights import Checkpoint, load_tensors
-    folder = model_folders("A", torch.float32, WEIGHT_STD)
-    cfg, W = plain.load_model_folder(folder)
-    config, spec = spec_from_config(TINY["A"][0])
-    order = (RunStep(0), RunStep(1), RunStep(2), RunStep(1), RunStep(3, kv_from=1))
-    spec = dataclasses.replace(spec, order=order)
-    model = Model(spec)
-    rt = make_runtime(DEV, torch.float32)
-    expected = model.expected_tensors()
-    assert "model.layers.3.self_attn.k_proj.weight" not in expected
-    ck = Checkpoint(folder)
-    tensors = {n: ck.tensor(n).float().to(DEV) for n in expected}
-    model.load(tensors, rt)
-    cache = CacheManager(model.cache_layout(), page_tokens=16, n_pages=8, max_requests=2,
-                         max_context=128, device=DEV, dtype=torch.float32)
-    lm = LoadedModel(config, spec, model, cache, ModelRunner(model, cache, rt, max_batched_tokens=64), rt)
+    from celeg_amd import native
+    from celeg_amd.engine import load_model
+    from celeg_amd.weights.safetensors_io import SafetensorsFile, write_safetensors
+    reordered_lfm2()
+    source = model_folders("A", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(source)
+    config = dict(TINY["A"][0], architectures=["Lfm2Reordered"],
+                  run_order=[[0, None], [1, None], [2, None], [1, None], [3, 1]])
+    wanted = [e["name"] for e in native.describe_config(config)["expected_tensors"]]
+    assert "model.layers.3.self_attn.k_proj.weight" not in wanted
+    folder = str(tmp_path / "reordered")
+    os.makedirs(folder)
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(config, fh)
+    f = SafetensorsFile(os.path.join(source, "model.safetensors"))
+    write_safetensors(os.path.join(folder, "model.safetensors"), {n: f.tensor(n).clone() for n in wanted})
+    f.close()
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2, max_context=128,
+                    max_batched_tokens=64)
     reqs = {"a": random_tokens(256, 50, 8), "b": random_tokens(256, 37, 9)}
     got = EngineDriver(lm).run(portions_schedule(reqs))
     for rid, toks in reqs.items():
