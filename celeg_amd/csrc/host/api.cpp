@@ -474,6 +474,36 @@ celeg_status celeg_model_synchronize(celeg_model* model) {
     return guarded([&] { CELEG_HIP(hipStreamSynchronize(model->lm->stream)); });
 }
 
+// ---------------------------------------------------------------------------- the dispatch alone
+// Ops::linear on raw device pointers: what the tests of the products call, so that they go
+// through the dispatch that the parts use (the 32-bit kernel, the kernels for few rows, the
+// library above 64 rows and what stands in where it has no kernel).
+celeg_status celeg_ops_linear(const void* x, int32_t x_dtype, int64_t x_row_stride, const void* w, int32_t w_dtype,
+                              void* out, int32_t out_dtype, int64_t out_row_stride, const float* bias, int32_t M,
+                              int32_t N, int32_t K, int32_t use_library, void* stream) {
+    if (!x || !w || !out || M <= 0 || N <= 0 || K <= 0) return CELEG_INVALID_ARGUMENT;
+    return guarded([&] {
+        // one dispatcher for the process (its library plans and workspace are made at the first
+        // call of a size, so a call that a graph records finds them there), on the caller's stream
+        static std::mutex lock;
+        static Ops ops(nullptr);
+        static Workspace ws;
+        std::lock_guard<std::mutex> guard(lock);
+        ops.stream = static_cast<hipStream_t>(stream);
+        auto view = [](const void* p, int32_t dtype, long long rows, long long cols, long long row_stride) {
+            Tensor t = Tensor::make(const_cast<void*>(p), static_cast<DType>(dtype), {rows, cols});
+            t.stride[0] = row_stride;
+            return t;
+        };
+        const Tensor xt = view(x, x_dtype, M, K, x_row_stride), wt = view(w, w_dtype, N, K, K);
+        const Tensor ot = view(out, out_dtype, M, N, out_row_stride);
+        Tensor bt;
+        if (bias) bt = Tensor::make(const_cast<float*>(bias), DType::F32, {static_cast<long long>(N)});
+        ops.use_blaslt = use_library != 0;
+        ops.linear(xt, wt, ot, bias ? &bt : nullptr, ws);
+    });
+}
+
 // ---------------------------------------------------------------------------- descriptions
 const char* celeg_describe_folder(const char* model_dir) {
     if (!model_dir) return nullptr;

@@ -158,6 +158,15 @@ void* celeg_model_stream(celeg_model* model);
 /* waits for everything launched on that stream */
 celeg_status celeg_model_synchronize(celeg_model* model);
 
+/* ---- the products' dispatch alone (tests) ----
+ * out [M, N] = x [M, K] w[N, K]^T (+ bias, 32-bit [N]) on `stream` (a hipStream_t), by the kernels the
+ * parts would get for these sizes and dtypes (0 float32, 1 bfloat16); rows of x and out lie
+ * x_row_stride / out_row_stride elements apart.  use_library 0: bfloat16 products of more than 64 rows
+ * never go to hipBLASLt. */
+celeg_status celeg_ops_linear(const void* x, int32_t x_dtype, int64_t x_row_stride, const void* w, int32_t w_dtype,
+                              void* out, int32_t out_dtype, int64_t out_row_stride, const float* bias, int32_t M,
+                              int32_t N, int32_t K, int32_t use_library, void* stream);
+
 /* ---- without a GPU: what a folder holds ---- */
 /* JSON {"config", "spec", "expected_tensors": [{"name", "shape", "kind", "init", "also"}]} of a model
  * folder (config.json, generation_config.json, and the checkpoint's tensor names for what they leave out) */

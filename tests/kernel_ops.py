@@ -1,15 +1,10 @@
-"""The kernels as Python calls on torch tensors: what the tests of single kernels and tuning
-scripts use.  (The engine does not come through here: its host code, ``host/ops.cpp``, makes
-the same checks and calls in C++.)  Shapes are checked on the host, then the extern "C" entry
+"""The kernels as Python calls on torch tensors, for the tests of single kernels.  (The
+engine does not come through here: its host code, ``celeg_amd/csrc/host/ops.cpp``, makes the
+same checks and calls in C++.)  Shapes are checked on the host, then the extern "C" entry
 points of the built library are called through ``ctypes`` with raw device pointers and the
 current HIP stream (so a stream that is capturing a graph captures them too).  There is no
 fallback: if the library cannot be built or loaded, or a tensor is not on the GPU, the call
-fails loudly.
-
-Matrix products in bfloat16 of more than 64 rows go to hipBLASLt, called directly
-(``blaslt.py``), as the reference sends its products to cuBLAS
-(src/backend/cuda/runtime/gemm_dispatcher.cpp); products in 32-bit go to our own
-kernel, which uses no reduced-precision matrix mode.
+fails loudly.  ``linear`` goes through the library's own dispatch (``celeg_ops_linear``).
 """
 from __future__ import annotations
 
@@ -18,7 +13,7 @@ from typing import Dict, Optional
 
 import torch
 
-from . import build
+from celeg_amd.csrc import build
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 _c_int, _c_float, _c_void_p, _c_size_t = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
@@ -51,7 +46,6 @@ class HipOps:
         # the general kernel (tests compare the two)
         self.attention_decode_whole = -1     # -1: chosen from the batch; 0 split-key kernels; 1 one workgroup per request and key/value head
         self.use_blaslt = True               # products of many rows: hipBLASLt called directly
-        self._blaslt = None
         self._device_index = torch.device(device).index if torch.device(device).index is not None \
             else torch.cuda.current_device()
         self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
@@ -240,61 +234,35 @@ class HipOps:
     # ------------------------------------------------------------------ matrix products
     def linear(self, x, w, out, bias=None):
         """out = x w^T (+ bias).  x [M,K] (rows may be strided), w [N,K], out [M,N] in the
-        dtype of x or in 32-bit."""
-        self._dev(x, "x", contiguous=False); self._dev(w, "w"); self._dev(out, "out")
-        M, K = x.shape
-        N = w.shape[0]
-        if w.shape[1] != K or out.shape != (M, N):
-            raise KernelError(f"linear: shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, "
-                              f"out {tuple(out.shape)}")
+        dtype of x or in 32-bit: the library's own dispatch (``Ops::linear``), the one the parts
+        call.  ``use_blaslt`` False keeps bfloat16 products of many rows away from hipBLASLt."""
+        from celeg_amd import native
+        for t, name in ((x, "x"), (w, "w"), (out, "out")):
+            if not t.is_cuda or t.dim() != 2 or t.stride(1) != 1:
+                raise KernelError(f"linear: {name} must be a matrix on the GPU with dense rows")
+        codes = {torch.float32: 0, torch.bfloat16: 1}
+        if x.dtype not in codes or w.dtype not in codes or out.dtype not in codes:
+            raise KernelError(f"linear: unsupported dtypes {x.dtype} x {w.dtype} -> {out.dtype}")
+        if not w.is_contiguous():
+            raise KernelError("linear: w must be contiguous")
         if bias is not None:
             self._dev(bias, "bias", torch.float32)
-            if bias.numel() != N:
-                raise KernelError("linear: bias must have one entry per output column")
-        if x.dtype == torch.float32 and w.dtype == torch.float32:
-            if out.dtype != torch.float32:
-                raise KernelError("linear: a 32-bit product needs a 32-bit output")
-            code = self._lib("gemm_f32").celeg_gemm_f32(
-                _ptr(x), _c_int(self._rows(x, "x")), _ptr(w), _c_int(K), _ptr(bias), _ptr(out),
-                _c_int(N), _c_int(M), _c_int(N), _c_int(K), self._stream())
-            self._check(code, "linear (32-bit)")
-            return out
-        if x.dtype == torch.bfloat16 and w.dtype == torch.float32:
-            # a matrix stored in 32-bit stays 32-bit: widen the rows and use the 32-bit product
-            xf = torch.empty((M, K), dtype=torch.float32, device=x.device)
-            self.cast(x.contiguous(), xf)
-            yf = out if out.dtype == torch.float32 else torch.empty((M, N), dtype=torch.float32,
-                                                                    device=x.device)
-            self.linear(xf, w, yf, bias)
-            if yf is not out:
-                self.cast(yf, out)
-            return out
-        if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-            raise KernelError(f"linear: unsupported dtypes {x.dtype} x {w.dtype}")
-        if out.dtype == torch.bfloat16:
-            self._library_product(x, w, out)
-            if bias is not None:
-                self.add_bias(out, bias)
-        elif out.dtype == torch.float32:
-            tmp = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-            self._library_product(x, w, tmp)
-            self.cast(tmp, out)
-            if bias is not None:
-                self.add_bias(out, bias)
-        else:
-            raise KernelError("linear: out must be bfloat16 or float32")
+        M, K = x.shape
+        if w.shape[1] != K or out.shape != (M, w.shape[0]):
+            raise KernelError(f"linear: shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+        lib = native.lib()
+        lib.celeg_ops_linear.restype = ctypes.c_int
+        lib.celeg_ops_linear.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int32,
+                                         ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p] + \
+            [ctypes.c_int32] * 4 + [ctypes.c_void_p]
+        try:
+            native.check(lib.celeg_ops_linear(
+                x.data_ptr(), codes[x.dtype], x.stride(0) if M > 1 else max(x.stride(0), K), w.data_ptr(), codes[w.dtype],
+                out.data_ptr(), codes[out.dtype], out.stride(0) if M > 1 else max(out.stride(0), out.shape[1]),
+                bias.data_ptr() if bias is not None else None, M, w.shape[0], K, int(self.use_blaslt), _raw_stream(self._device_index)))
+        except (native.NativeError, native.NativeArgumentError) as err:
+            raise KernelError(str(err)) from None
         return out
-
-    def _library_product(self, x, w, out):
-        """out = x w^T by the library (bfloat16): hipBLASLt called directly where it has a
-        kernel for the sizes, torch's call of the libraries otherwise."""
-        if self.use_blaslt and x.stride(1) == 1 and out.stride(1) == 1:
-            if self._blaslt is None:
-                from .blaslt import BlasLt
-                self._blaslt = BlasLt(self.device)
-            if self._blaslt.matmul(x, w, out, _raw_stream(self._device_index)):
-                return
-        torch.mm(x, w.t(), out=out)
 
     # ------------------------------------------------------------------ short convolution
     def short_conv(self, bcx, weight, bias, state, out, batch):

@@ -12,7 +12,7 @@ BF = torch.bfloat16
 
 @pytest.fixture(scope="module")
 def ops():
-    from celeg_amd.csrc.hip_ops import HipOps
+    from kernel_ops import HipOps
     return HipOps(DEV)
 
 
@@ -315,7 +315,7 @@ def test_operands_with_rows_side_by_side_give_the_same_bits(ops, M, N, K):
     assert torch.equal(hh[0], hh[1]) and torch.equal(so[0], so[1])
     assert torch.equal(copies[1].reshape(M, N), copies[0]) and torch.equal(copies[0], hh[0].to(BF))
     # the kernels for up to 16 rows read rows that lie one after the other only
-    from celeg_amd.csrc.hip_ops import KernelError
+    from kernel_ops import KernelError
     with pytest.raises(KernelError, match="side by side"):
         ops.fused_linear(xc[:8], folded, torch.empty(8, N, dtype=BF, device=DEV))
 
@@ -365,7 +365,7 @@ def test_embed_stats(ops):
 
 
 def test_unsupported_sizes_are_refused(ops):
-    from celeg_amd.csrc.hip_ops import KernelError
+    from kernel_ops import KernelError
     w = randn(32, 100, dtype=BF)
     with pytest.raises(KernelError, match="not supported"):
         ops.fused_linear(randn(4, 100, dtype=BF), w, torch.empty(4, 32, dtype=BF, device=DEV))

@@ -146,7 +146,7 @@ def test_command_line(model_folders, tmp_path):
 # ---------------------------------------------------------------- the sampling kernels alone
 @pytest.fixture(scope="module")
 def ops():
-    from celeg_amd.csrc.hip_ops import HipOps
+    from kernel_ops import HipOps
     return HipOps(DEV)
 
 

@@ -15,7 +15,7 @@ DEV = "cuda:0"
 
 @pytest.fixture(scope="module")
 def ops():
-    from celeg_amd.csrc.hip_ops import HipOps
+    from kernel_ops import HipOps
     return HipOps(DEV)
 
 

@@ -11,7 +11,7 @@ N_SHAPES = 11
 
 @pytest.fixture(scope="module")
 def ops():
-    from celeg_amd.csrc.hip_ops import HipOps
+    from kernel_ops import HipOps
     ops = HipOps(DEV)
     yield ops
     ops._lib("gemm_tiles").celeg_gemm_tiles_force(-1)
@@ -117,7 +117,7 @@ def test_a_row_does_not_depend_on_the_other_rows(ops):
 
 
 def test_unsupported_sizes_are_refused(ops):
-    from celeg_amd.csrc.hip_ops import KernelError
+    from kernel_ops import KernelError
     ops._lib("gemm_tiles").celeg_gemm_tiles_force(-1)
     a = randn(80, 96, dtype=BF)
     with pytest.raises(KernelError):             # inner size no multiple of 64
