@@ -140,6 +140,9 @@ def main() -> int:
                     help="serve phase: portions cut by the budget keep to multiples of this")
     ap.add_argument("--token-budget", type=int, default=0,
                     help="serve phase: most tokens of a step (default: the workload's)")
+    ap.add_argument("--context", type=int, default=0,
+                    help="with --phase decode: tokens every request holds when decoding starts "
+                         "(default 2048, the headline's)")
     ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
                          "decode measurement (the line printed then holds only that part); "
@@ -166,9 +169,14 @@ def main() -> int:
     if args.layers and args.layers < full_layers:
         cfg["num_hidden_layers"] = args.layers
         cfg["layer_types"] = cfg["layer_types"][:args.layers]
-    context = cfg["max_position_embeddings"]
+    decode_context = args.context if args.context > 0 and args.phase == "decode" else PROMPT_TOKENS
     max_batch = max(BATCH, args.batch) if args.no_points or args.phase != "all" else 64
-    need = PROMPT_TOKENS + args.steps + args.warmup + 64 + 3    # (a request decodes along while the others' prompts are fed)
+    # (a request decodes along while the others' prompts are fed, a step for every portion of a prompt)
+    portions = (decode_context + PROMPT_TOKENS - 1) // PROMPT_TOKENS
+    need = decode_context + args.steps + args.warmup + max_batch * portions + 3
+    if decode_context != PROMPT_TOKENS:
+        cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], need)
+    context = cfg["max_position_embeddings"]
     if need > context:
         raise SystemExit(f"--steps + --warmup exceed the context of {context}")
     with tempfile.TemporaryDirectory(prefix="celeg_bench_") as folder:
@@ -196,16 +204,21 @@ def main() -> int:
         return 0
 
     def decode(batch: int):
-        bench = DecodeBench(engine, batch, PROMPT_TOKENS, args.steps + args.warmup + batch + 2, seed=batch)
+        bench = DecodeBench(engine, batch, decode_context, args.steps + args.warmup + batch * portions + 2, seed=batch)
         result = bench.run(args.steps, args.warmup)
         bench.close()
         return result
 
-    if args.phase == "decode" and args.batch != BATCH:
+    if args.phase == "decode" and (args.batch != BATCH or decode_context != PROMPT_TOKENS):
         result = decode(args.batch)
-        print(json.dumps({"metric": f"decode tok/s @ batch {args.batch} (LFM2-{args.shape.upper()} shape, bf16)",
+        step_bytes = w_bytes + kv_per_token * result["mean_context"] * args.batch
+        achieved = step_bytes / (result["ms_per_step"] * 1e-3) / 1e9
+        print(json.dumps({"metric": f"decode tok/s @ batch {args.batch}, context {decode_context} "
+                                    f"(LFM2-{args.shape.upper()} shape, bf16)",
                           "value": round(result["tokens_per_second"], 1), "unit": "tokens/s",
-                          "ms_per_step": round(result["ms_per_step"], 4), "phase": "decode"}))
+                          "ms_per_step": round(result["ms_per_step"], 4), "phase": "decode",
+                          "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                                       "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5)}}))
         return 0
     main_run = decode(BATCH)
     points = {}

@@ -14,6 +14,7 @@ using namespace celeg;
 struct celeg_model {
     std::unique_ptr<LoadedModel> owned;
     LoadedModel* lm = nullptr;
+    PinnedBuffer logits_stage;      // few rows of logits come to the host through pinned memory
 };
 struct celeg_engine {
     std::unique_ptr<Engine> engine;
@@ -394,6 +395,16 @@ celeg_status celeg_model_step(celeg_model* model, int32_t n_entries, const int32
         const Tensor out = lm.runner->step(entries);
         const size_t width = static_cast<size_t>(out.shape[1]);
         if (wanted * width > capacity) throw StepError("step: the logits buffer is too small");
+        const size_t bytes = wanted * width * 4;
+        if (wanted && bytes <= (size_t(8) << 20)) {
+            // one asynchronous copy into pinned memory behind the step, one wait
+            if (model->logits_stage.bytes() < bytes) model->logits_stage = PinnedBuffer(std::max(bytes, size_t(1) << 20));
+            CELEG_HIP(hipMemcpy2DAsync(model->logits_stage.ptr(), width * 4, out.data, static_cast<size_t>(out.row_stride()) * 4,
+                                       width * 4, wanted, hipMemcpyDeviceToHost, lm.stream));
+            CELEG_HIP(hipStreamSynchronize(lm.stream));
+            std::memcpy(logits, model->logits_stage.ptr(), bytes);
+            return;
+        }
         CELEG_HIP(hipStreamSynchronize(lm.stream));
         if (wanted)
             CELEG_HIP(hipMemcpy2D(logits, width * 4, out.data, static_cast<size_t>(out.row_stride()) * 4, width * 4, wanted,

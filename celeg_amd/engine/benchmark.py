@@ -79,6 +79,9 @@ class DecodeBench:
         elapsed = time.perf_counter() - start
         after = self.generated()
         tokens = sum(after) - sum(before)
+        if tokens != done * self.batch:
+            raise RuntimeError(f"decode benchmark: {done} steps of {self.batch} requests gave {tokens} tokens "
+                               "(a request ended or waited for pages inside the timed steps)")
         mean_context = self.context + (sum(before) + sum(after)) / (2.0 * self.batch)
         return {"steps": done, "batch": self.batch, "ms_per_step": elapsed / max(done, 1) * 1e3,
                 "tokens_per_second": tokens / elapsed, "tokens": tokens, "mean_context": mean_context}
