@@ -20,15 +20,16 @@ __device__ __forceinline__ size_t cache_offset(int page, int n_layers, int layer
 // ---------------------------------------------------------------- q/k norm + rope + store
 // One wavefront per (row, head); heads [0,Hq) are q, [Hq,Hq+Hkv) are k, the rest are v.
 // Per head: inv = 1/sqrt(mean(x^2)+eps); x = x*inv*w (if a norm weight is given);
-// split-half rotation of pairs (i, i+rot/2) by angle = float(pos)*inv_freq[i] (if a
-// frequency table is given); q goes back in place, k and v go to the cache.
+// rotation of pair i by angle = float(pos)*inv_freq[i] (if a frequency table is given), the
+// pair being (i, i+rot/2) (pairing 0: halves) or (2i, 2i+1) (pairing 1: neighbours); q goes
+// back in place, k and v go to the cache.
 // Reference: src/backend/cpu/kernels/rope.cpp:61-111; CUDA kernels/rope.cuh:333-393.
 #define ROPE_WAVES 4
 template <typename T>
 __global__ __launch_bounds__(ROPE_WAVES * CELEG_WAVE) void qk_norm_rope_store_kernel(
     T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
-    const float* __restrict__ inv_freq, const float* __restrict__ cos_sin, int rotary_dim,
+    const float* __restrict__ inv_freq, const float* __restrict__ cos_sin, int rotary_dim, int pairing,
     const int* __restrict__ positions,
     const int* __restrict__ token_slot, const int* __restrict__ table, int table_stride,
     T* __restrict__ k_pool, T* __restrict__ v_pool, int n_layers, int layer, int page_tokens,
@@ -82,7 +83,9 @@ __global__ __launch_bounds__(ROPE_WAVES * CELEG_WAVE) void qk_norm_rope_store_ke
     for (int d = lane; d < head_dim; d += CELEG_WAVE) {
         float y = vals[d];
         if (inv_freq && d < rotary_dim) {
-            const int i = d < half ? d : d - half;
+            // the pair's number, and whether this value is the pair's first
+            const int i = pairing ? d >> 1 : (d < half ? d : d - half);
+            const bool first = pairing ? !(d & 1) : d < half;
             float c, s;
             if (cos_sin) {       // the table of celeg_rope_table: the same values, computed once
                 const float* cs = cos_sin + (static_cast<size_t>(pos) * half + i) * 2;
@@ -93,8 +96,8 @@ __global__ __launch_bounds__(ROPE_WAVES * CELEG_WAVE) void qk_norm_rope_store_ke
                 c = cosf(angle);
                 s = sinf(angle);
             }
-            const float a = vals[i], b = vals[i + half];
-            y = d < half ? a * c - b * s : b * c + a * s;
+            const float a = pairing ? vals[2 * i] : vals[i], b = pairing ? vals[2 * i + 1] : vals[i + half];
+            y = first ? a * c - b * s : b * c + a * s;
         }
         dst[d] = from_float<T>(y);
     }
@@ -258,13 +261,14 @@ extern "C" int celeg_rope_table(const float* inv_freq, int half, int n_positions
 extern "C" int celeg_qk_norm_rope_store(
     void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype,
     const float* q_weight, const float* k_weight, float eps, const float* inv_freq,
-    const float* cos_sin, int rotary_dim, const int* positions, const int* token_slot, const int* table,
+    const float* cos_sin, int rotary_dim, int pairing, const int* positions, const int* token_slot, const int* table,
     int table_stride, void* k_pool, void* v_pool, int n_layers, int layer, int page_tokens,
     int n_tokens, int q_heads, int kv_heads, int head_dim, int store_kv, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
+    if (pairing != 0 && pairing != 1) return static_cast<int>(hipErrorInvalidValue);
     const int n_heads = q_heads + (store_kv ? 2 * kv_heads : 0);
     const auto aligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    const bool whole_rotation = !inv_freq || (cos_sin && rotary_dim == head_dim);
+    const bool whole_rotation = !inv_freq || (cos_sin && rotary_dim == head_dim && pairing == 0);
     if ((head_dim == 32 || head_dim == 64 || head_dim == 128) && whole_rotation && ldq % 4 == 0 &&
         (!store_kv || (ldk % 4 == 0 && ldv % 4 == 0 && aligned(k) && aligned(v))) && aligned(q) &&
         aligned(k_pool) && (!q_weight || aligned(q_weight)) && (!k_weight || aligned(k_weight)) &&
@@ -286,14 +290,14 @@ extern "C" int celeg_qk_norm_rope_store(
         hipLaunchKernelGGL(qk_norm_rope_store_kernel<float>, grid, block, lds, stream,
                            static_cast<float*>(q), ldq, static_cast<const float*>(k), ldk,
                            static_cast<const float*>(v), ldv, q_weight, k_weight, eps, inv_freq,
-                           cos_sin, rotary_dim, positions, token_slot, table, table_stride,
+                           cos_sin, rotary_dim, pairing, positions, token_slot, table, table_stride,
                            static_cast<float*>(k_pool), static_cast<float*>(v_pool), n_layers,
                            layer, page_tokens, q_heads, kv_heads, head_dim, n_heads);
     else
         hipLaunchKernelGGL(qk_norm_rope_store_kernel<bf16>, grid, block, lds, stream,
                            static_cast<bf16*>(q), ldq, static_cast<const bf16*>(k), ldk,
                            static_cast<const bf16*>(v), ldv, q_weight, k_weight, eps, inv_freq,
-                           cos_sin, rotary_dim, positions, token_slot, table, table_stride,
+                           cos_sin, rotary_dim, pairing, positions, token_slot, table, table_stride,
                            static_cast<bf16*>(k_pool), static_cast<bf16*>(v_pool), n_layers,
                            layer, page_tokens, q_heads, kv_heads, head_dim, n_heads);
     return CELEG_LAUNCH_RESULT();

@@ -631,7 +631,7 @@ struct OutsideDescription {
     bool graph_safe = false;
     long long out_width = 0;
     std::vector<float> inv_freq;
-    int rotary_dim = 0;
+    int rotary_dim = 0, pairing = 0;
 };
 
 class Outside {
@@ -670,6 +670,10 @@ public:
         if (j["inv_freq"].is_array())
             for (const Json& v : j["inv_freq"].items()) d_.inv_freq.push_back(static_cast<float>(v.as_double()));
         d_.rotary_dim = static_cast<int>(j.get_int("rotary_dim", 0));
+        const std::string pairing = j.get_string("pairing", "halves");
+        if (pairing != "halves" && pairing != "neighbours")
+            throw SpecError("part '" + kind + "': pairing is 'halves' or 'neighbours', not '" + pairing + "'");
+        d_.pairing = pairing == "neighbours" ? 1 : 0;
     }
     ~Outside() {
         if (f_.destroy) f_.destroy(f_.self);
@@ -807,7 +811,7 @@ public:
         if (static_cast<int>(d.inv_freq.size()) * 2 != d.rotary_dim)
             throw SpecError("position '" + spec.kind + "': rotary_dim must be twice the number of frequencies");
         if (!table_) table_ = from_host_floats(d.inv_freq, DType::F32, {static_cast<long long>(d.inv_freq.size())});
-        return Tables{table_->view, d.rotary_dim};
+        return Tables{table_->view, d.rotary_dim, d.pairing};
     }
 
 private:

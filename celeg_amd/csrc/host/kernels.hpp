@@ -38,7 +38,7 @@ int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const float* w, con
 int celeg_rope_table(const float* inv_freq, int half, int n_positions, float* out, hipStream_t stream);
 int celeg_qk_norm_rope_store(void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype,
                              const float* q_weight, const float* k_weight, float eps, const float* inv_freq,
-                             const float* cos_sin, int rotary_dim, const int* positions, const int* token_slot,
+                             const float* cos_sin, int rotary_dim, int pairing, const int* positions, const int* token_slot,
                              const int* table, int table_stride, void* k_pool, void* v_pool, int n_layers, int layer,
                              int page_tokens, int n_tokens, int q_heads, int kv_heads, int head_dim, int store_kv,
                              hipStream_t stream);

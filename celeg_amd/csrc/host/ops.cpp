@@ -246,7 +246,7 @@ const float* Ops::rope_table(const Tensor& inv_freq, int n_positions) {
 }
 
 void Ops::qk_norm_rope_store(const Tensor& q, const Tensor* k, const Tensor* v, const Tensor* q_weight,
-                             const Tensor* k_weight, float eps, const Tensor* inv_freq, int rotary_dim, int heads,
+                             const Tensor* k_weight, float eps, const Tensor* inv_freq, int rotary_dim, int pairing, int heads,
                              int kv_heads, int head_dim, const StepBatch& batch, const KVView& kv) {
     dev(q, "q");
     const long long T = q.shape[0];
@@ -273,6 +273,7 @@ void Ops::qk_norm_rope_store(const Tensor& q, const Tensor* k, const Tensor* v, 
         dev(*inv_freq, "inv_freq", DType::F32);
         need(rotary_dim % 2 == 0 && rotary_dim <= head_dim && inv_freq->numel() == rotary_dim / 2,
              "qk_norm_rope_store: rotary_dim and the frequency table disagree");
+        need(pairing == 0 || pairing == 1, "qk_norm_rope_store: pairing is 0 (halves) or 1 (neighbours)");
     }
     const float* cos_sin = nullptr;
     if (inv_freq && rotary_dim > 0 && use_rope_table) cos_sin = rope_table(*inv_freq, kv.table_stride * kv.page_tokens);
@@ -280,7 +281,7 @@ void Ops::qk_norm_rope_store(const Tensor& q, const Tensor* k, const Tensor* v, 
                      q.data, rows_of(q, "q"), store ? k->data : nullptr, store ? rows_of(*k, "k") : 0,
                      store ? v->data : nullptr, store ? rows_of(*v, "v") : 0, dt(q, "q"),
                      q_weight ? q_weight->as<float>() : nullptr, (store && k_weight) ? k_weight->as<float>() : nullptr, eps,
-                     inv_freq ? inv_freq->as<float>() : nullptr, cos_sin, rotary_dim, batch.positions, batch.token_slot,
+                     inv_freq ? inv_freq->as<float>() : nullptr, cos_sin, rotary_dim, pairing, batch.positions, batch.token_slot,
                      kv.table, kv.table_stride, kv.k, kv.v, kv.n_layers, kv.layer, kv.page_tokens, static_cast<int>(T),
                      heads, kv_heads, head_dim, store ? 1 : 0, stream), "qk_norm_rope_store");
 }

@@ -77,7 +77,7 @@ public:
     void short_conv(const Tensor& bcx, const Tensor& weight, const Tensor* bias, const Tensor& state, const Tensor& out,
                     const StepBatch& batch);
     void qk_norm_rope_store(const Tensor& q, const Tensor* k, const Tensor* v, const Tensor* q_weight,
-                            const Tensor* k_weight, float eps, const Tensor* inv_freq, int rotary_dim, int heads,
+                            const Tensor* k_weight, float eps, const Tensor* inv_freq, int rotary_dim, int pairing, int heads,
                             int kv_heads, int head_dim, const StepBatch& batch, const KVView& kv);
     void paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
                          int window, const StepBatch& batch, const KVView& kv, Workspace& ws);

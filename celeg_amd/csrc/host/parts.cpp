@@ -186,9 +186,10 @@ private:
 };
 
 // ---------------------------------------------------------------------------- position encodings
-// rope: rotary encoding with split-half pairing: for i < rotary_dim/2 the pair
-// (x[i], x[i + rotary_dim/2]) is rotated by the angle position * theta^(-2i/rotary_dim)
-// (src/backend/cpu/kernels/rope.cpp:30-36, 95-108).  The frequencies are computed on the host
+// rope: rotary encoding: for i < rotary_dim/2 pair i is rotated by the angle
+// position * theta^(-2i/rotary_dim); the pair is (x[i], x[i + rotary_dim/2]) ("pairing":
+// "halves", the default and the reference's, src/backend/cpu/kernels/rope.cpp:30-36, 95-108)
+// or (x[2i], x[2i+1]) ("neighbours").  The frequencies are computed on the host
 // in double (include/celeg/model/position.hpp:77-78) and handed to the kernel as a 32-bit
 // table; the angle is the 32-bit product float(position) * frequency.
 class Rope final : public PositionEncoding {
@@ -200,6 +201,9 @@ public:
         if (!(theta_ > 0)) throw SpecError("rope: theta must be positive");
         if (rotary_dim_ <= 0 || rotary_dim_ % 2 || rotary_dim_ > head_dim_)
             throw SpecError("rope: rotary_dim must be even, positive and at most head_dim");
+        const std::string pairing = s.params.get_string("pairing", "halves");
+        if (pairing != "halves" && pairing != "neighbours") throw SpecError("rope: pairing is 'halves' or 'neighbours', not '" + pairing + "'");
+        pairing_ = pairing == "neighbours" ? 1 : 0;
     }
     bool graph_safe() const override { return true; }
     Tables tables(Runtime&) override {
@@ -209,12 +213,12 @@ public:
                 freq[static_cast<size_t>(i)] = static_cast<float>(std::pow(theta_, -2.0 * i / rotary_dim_));
             table_ = from_host_floats(freq, DType::F32, {rotary_dim_ / 2});
         }
-        return Tables{table_->view, rotary_dim_};
+        return Tables{table_->view, rotary_dim_, pairing_};
     }
 
 private:
     double theta_;
-    int head_dim_, rotary_dim_;
+    int head_dim_, rotary_dim_, pairing_ = 0;
     std::shared_ptr<DeviceTensor> table_;
 };
 
@@ -343,7 +347,7 @@ private:
         const PositionEncoding::Tables tables = position_->tables(rt);
         rt.ops.qk_norm_rope_store(q, writes ? &k : nullptr, writes ? &v : nullptr, q_norm_ ? &q_norm_->view : nullptr,
                                   k_norm_ ? &k_norm_->view : nullptr, eps_, tables.inv_freq.defined() ? &tables.inv_freq : nullptr,
-                                  tables.rotary_dim, heads_, kv_heads_, head_dim_, batch, *cache.kv);
+                                  tables.rotary_dim, tables.pairing, heads_, kv_heads_, head_dim_, batch, *cache.kv);
         Tensor attended = rt.ws.buf("attn_out", rt.dtype, {T, qw});
         rt.ops.paged_attention(q, attended, heads_, kv_heads_, head_dim_, scale_, window_ ? *window_ : 0, batch, *cache.kv, rt.ws);
         return attended;

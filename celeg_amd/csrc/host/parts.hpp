@@ -67,7 +67,9 @@ public:
 class PositionEncoding : public Part {
 public:
     using Part::Part;
-    struct Tables { Tensor inv_freq; int rotary_dim = 0; };   // inv_freq undefined: no rotation
+    // inv_freq undefined: no rotation.  Pair i of the first rotary_dim values of a head turns by
+    // position * inv_freq[i]; pairing 0: the pair is (i, i + rotary_dim/2), 1: (2i, 2i + 1).
+    struct Tables { Tensor inv_freq; int rotary_dim = 0; int pairing = 0; };
     virtual Tables tables(Runtime& rt) = 0;
 };
 

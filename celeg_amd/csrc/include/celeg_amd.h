@@ -229,7 +229,8 @@ typedef struct celeg_forward_args {
  *   {"weights": {role: {"shape": [..], "kind": "matrix"|"vector", "init": "normal"|"around_one"}},
  *    "kv_need": {"kv_heads", "head_dim", "window"} or null, "states": [{"name", "shape", "dtype"}],
  *    "graph_safe": bool, "out_width": columns of what forward writes (mixer, ffn),
- *    "inv_freq": [..], "rotary_dim": n  (position encodings)}
+ *    "inv_freq": [..], "rotary_dim": n, "pairing": "halves"|"neighbours"  (position encodings: pair i of
+ *    the first n values of a head, (i, i + n/2) or (2i, 2i + 1), turns by position * inv_freq[i])}
  * load() receives the tensors by role; forward() returns 0 or an error code. */
 typedef struct celeg_part_functions {
     void* self;

@@ -314,7 +314,7 @@ class HipOps:
         return table[0]
 
     def qk_norm_rope_store(self, q, k, v, q_weight, k_weight, eps, inv_freq, rotary_dim,
-                           heads, kv_heads, head_dim, batch, kv):
+                           heads, kv_heads, head_dim, batch, kv, pairing=0):
         self._dev(q, "q", contiguous=False)
         T = q.shape[0]
         dtype = q.dtype
@@ -344,7 +344,7 @@ class HipOps:
             _ptr(q), _c_int(self._rows(q, "q")), _ptr(k), _c_int(self._rows(k, "k") if store else 0),
             _ptr(v), _c_int(self._rows(v, "v") if store else 0), _c_int(self._dtype(q, "q")),
             _ptr(q_weight), _ptr(k_weight if store else None), _c_float(eps), _ptr(inv_freq),
-            _ptr(cos_sin), _c_int(rotary_dim), _ptr(batch.positions), _ptr(batch.token_slot), _ptr(kv.table),
+            _ptr(cos_sin), _c_int(rotary_dim), _c_int(pairing), _ptr(batch.positions), _ptr(batch.token_slot), _ptr(kv.table),
             _c_int(kv.table.shape[1]), _ptr(kv.k), _ptr(kv.v), _c_int(kv.n_layers),
             _c_int(kv.layer), _c_int(kv.page_tokens), _c_int(T), _c_int(heads), _c_int(kv_heads),
             _c_int(head_dim), _c_int(1 if store else 0), self._stream())
