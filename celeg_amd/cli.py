@@ -54,6 +54,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--benchmark-warmup", type=int, default=8, metavar="N")
     ap.add_argument("--benchmark-prefill-tokens", type=int, default=0, metavar="N")
     ap.add_argument("--batch", type=int, default=1, help="requests decoded together in benchmarks")
+    ap.add_argument("--max-requests", type=int, default=0,
+                    help="requests the engine holds at a time (default: --batch)")
     ap.add_argument("--prefill-chunk", type=int, default=256)
     ap.add_argument("--max-batched-tokens", type=int, default=0,
                     help="token budget of a step (default: the larger of 512 and --prefill-chunk)")
@@ -172,7 +174,7 @@ def run(args) -> int:
     if args.dump_hidden:
         os.environ["CELEG_DUMP_HIDDEN"] = args.dump_hidden      # read by the library when it loads the model
     engine = Engine.from_folder(model_dir, dtype=args.dtype, device=args.device, page_tokens=args.page_tokens,
-                                n_pages=args.pages or pages_per_request * batch, max_active_requests=max(batch, 1),
+                                n_pages=args.pages or pages_per_request * max(batch, args.max_requests, 1), max_active_requests=max(batch, args.max_requests, 1),
                                 context=context, max_batched_tokens=budget,
                                 prefill_chunk_tokens=min(args.prefill_chunk, budget),
                                 gemm_backend=args.gemm_backend, use_graphs=not args.no_graph)
