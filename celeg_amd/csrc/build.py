@@ -198,6 +198,33 @@ def build(force: bool = False, verbose: bool = True) -> str:
         return final
 
 
+SANITIZE_FLAGS = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined",
+                  "-fno-omit-frame-pointer", "-g1"]
+
+
+def build_sanitized(out_dir: str, verbose: bool = False) -> str:
+    """The library with its HOST code under AddressSanitizer and UndefinedBehaviorSanitizer (the
+    kernels' objects are the ordinary ones; device code is never instrumented), linked into
+    ``out_dir``: what the tests of the host's memory safety run, on the CPU.  Returns its path."""
+    with _lock:
+        lib_dir = _writable_lib_dir()
+        os.makedirs(os.path.join(out_dir, "obj"), exist_ok=True)
+        kernels = [_compile(source_path(m), lib_dir, verbose, False) for m in MODULES]
+
+        def sanitized(source: str) -> str:
+            obj = os.path.join(out_dir, "obj", "san_" + _object_name(source))
+            if not os.path.isfile(obj):
+                flags = [f for f in HOST_FLAGS if f != "-O3"] + ["-O1"] + SANITIZE_FLAGS
+                _run([_hipcc()] + flags + ["-I", HERE, "-I", HOST, "-c", source, "-o", obj],
+                     f"compiling {os.path.basename(source)} with sanitizers", out_dir, verbose)
+            return obj
+        with ThreadPoolExecutor(max_workers=max(1, min(8, os.cpu_count() or 1))) as pool:
+            hosts = list(pool.map(sanitized, host_sources()))
+        final = os.path.join(out_dir, LIBRARY + "-sanitized.so")
+        _run([_hipcc()] + kernels + hosts + LINK_FLAGS + SANITIZE_FLAGS[:4] + ["-o", final], "linking", out_dir, verbose)
+        return final
+
+
 def compile_module(name: Optional[str] = None, verbose: bool = True) -> str:
     return build(force=False, verbose=verbose)
 
