@@ -324,3 +324,34 @@ def test_generation_ahead_of_the_tokens_with_requests_that_end_early(model_folde
     assert engine.metrics["steps_ahead"] > 5
     for prompt, out in zip(prompts, sampled):
         assert out == plain_generate(cfg, W, prompt, 12, generation=gen)
+
+
+def test_cancelling_while_steps_run_ahead(model_folders):
+    """A request cancelled while others decode (steps launched ahead of their tokens): the
+    others' tokens are the plain implementation's, the cancelled one keeps what it had, and
+    everything is given back.  A request that cannot fit the context is refused at the door."""
+    from celeg_amd.engine import Engine, RequestOptions, RequestStatus
+    from celeg_amd.sampling import GREEDY
+    folder = model_folders("B", torch.float32, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=400 + n) for n in (9, 14, 20)]
+    engine = Engine.from_folder(folder, dtype="float32", max_active_requests=3, n_pages=12, context=64,
+                                max_batched_tokens=64, prefill_chunk_tokens=32)
+    options = RequestOptions(max_new_tokens=30, eos_token_ids=[], generation=GREEDY)
+    ids = [engine.submit(p, options) for p in prompts]
+    assert engine.native.run_steps(6) == 6
+    engine.cancel(ids[1])
+    engine.run()
+    assert engine.metrics["steps_ahead"] > 20
+    results = [engine.poll(r) for r in ids]
+    assert [r[0] for r in results] == [RequestStatus.FINISHED, RequestStatus.CANCELLED, RequestStatus.FINISHED]
+    want = [plain_generate(cfg, W, p, 30) for p in prompts]
+    assert results[0][1] == want[0] and results[2][1] == want[2]
+    assert 1 <= len(results[1][1]) <= 8 and results[1][1] == want[1][:len(results[1][1])]
+    assert engine.loaded.cache.free_pages() == [12] and engine.loaded.cache.n_free_slots == 3
+    engine.loaded.cache.check()
+    with pytest.raises(Exception, match="max_context"):
+        engine.submit(list(range(41)), options)
+    after = engine.submit(prompts[0], options)          # the engine goes on
+    engine.run()
+    assert engine.poll(after) == (RequestStatus.FINISHED, want[0], "")
