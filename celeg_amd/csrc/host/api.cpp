@@ -425,6 +425,8 @@ const std::vector<Knob>& knobs() {
 #define OPS_BOOL(field) {#field, [](LoadedModel& m) { return m.rt->ops.field ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->ops.field = v != 0; }}
     static const std::vector<Knob> table = {
         {"use_graphs", [](LoadedModel& m) { return m.runner->use_graphs ? 1 : 0; }, [](LoadedModel& m, int v) { m.runner->use_graphs = v != 0; }},
+        {"portion_graph_min_tokens", [](LoadedModel& m) { return m.runner->portion_graph_min_tokens; },
+         [](LoadedModel& m, int v) { m.runner->portion_graph_min_tokens = v; }},
         {"use_fused", [](LoadedModel& m) { return m.rt->use_fused ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->use_fused = v != 0; }},
         {"use_tiled_products", [](LoadedModel& m) { return m.rt->use_tiled_products ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->use_tiled_products = v != 0; }},
         {"fused_max_rows", [](LoadedModel& m) { return m.rt->fused_max_rows; }, [](LoadedModel& m, int v) { m.rt->fused_max_rows = v; }},

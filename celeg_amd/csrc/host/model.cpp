@@ -193,6 +193,7 @@ void ModelRunner::drop_graphs() {
         if (g.second.graph) (void)hipGraphDestroy(g.second.graph);
     }
     graphs_.clear();
+    n_portion_graphs_ = 0;
 }
 
 void ModelRunner::set_token_source(int* last_tokens) {
@@ -293,6 +294,7 @@ void ModelRunner::begin_step(const StepBatch& batch) {
 Tensor ModelRunner::step(const std::vector<StepEntry>& entries) {
     validate(entries);
     if (graph_applies(entries)) return step_from_graph(entries);
+    if (portion_graph_applies(entries)) return step_from_portion_graph(entries);
     auto updates = drain_updates(std::vector<int>(static_cast<size_t>(cache.n_groups()), update_room_));
     BuildOptions options;
     options.null_slot = cache.null_slot;
@@ -353,14 +355,6 @@ Tensor ModelRunner::step_from_graph(const std::vector<StepEntry>& entries) {
 }
 
 ModelRunner::Captured& ModelRunner::capture(int bucket, const std::vector<int>& caps, int bound) {
-    const auto started = std::chrono::steady_clock::now();
-    ++captures;
-    auto old = graphs_.find({bucket, bound});
-    if (old != graphs_.end()) {
-        if (old->second.exec) (void)hipGraphExecDestroy(old->second.exec);
-        if (old->second.graph) (void)hipGraphDestroy(old->second.graph);
-        graphs_.erase(old);
-    }
     const std::vector<std::vector<TableUpdate>> empty(static_cast<size_t>(cache.n_groups()));
     BuildOptions options;
     options.pad_to = bucket;
@@ -368,8 +362,22 @@ ModelRunner::Captured& ModelRunner::capture(int bucket, const std::vector<int>& 
     options.update_caps = &caps;
     StepBatch batch = builder_->build({}, empty, options);
     batch.context_bound = bound;
+    return record({bucket, bound}, batch);
+}
+
+// Runs `batch` once (buffers, libraries, weights re-laid at first need), then records it.  The
+// batch holds rows of the null slot only, which write to the spare page and the spare state row.
+ModelRunner::Captured& ModelRunner::record(std::pair<int, int> key, const StepBatch& batch) {
+    const auto started = std::chrono::steady_clock::now();
+    ++captures;
+    auto old = graphs_.find(key);
+    if (old != graphs_.end()) {
+        if (old->second.exec) (void)hipGraphExecDestroy(old->second.exec);
+        if (old->second.graph) (void)hipGraphDestroy(old->second.graph);
+        graphs_.erase(old);
+    }
     begin_step(batch);
-    model.forward(batch, rt);            // warm-up: buffers, libraries, weights re-laid at first need
+    model.forward(batch, rt);
     CELEG_HIP(hipStreamSynchronize(rt.stream));
     Captured captured;
     rt.ws.frozen = true;
@@ -394,7 +402,53 @@ ModelRunner::Captured& ModelRunner::capture(int bucket, const std::vector<int>& 
     CELEG_HIP(hipStreamSynchronize(rt.stream));
     captured.generation = rt.ws.generation;
     capture_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - started).count();
-    return graphs_[{bucket, bound}] = captured;
+    return graphs_[key] = captured;
+}
+
+// A step that is one portion of a prompt is some 150 launches with gaps between them: a size
+// that has come before (the portions that a token budget cuts have the same size again and
+// again) is recorded too, per number of rows and per context below or from 4,096 tokens (the
+// attention over rows chooses its tiles by that).
+bool ModelRunner::portion_graph_applies(const std::vector<StepEntry>& entries) {
+    if (!use_graphs || !model.graph_safe() || rt.after_layer || rt.phases || entries.size() != 1) return false;
+    const StepEntry& e = entries[0];
+    const int T = static_cast<int>(e.tokens.size());
+    if (T < portion_graph_min_tokens || e.want.size() != 1 || e.want[0] != T - 1) return false;
+    if (graphs_.count({-T, 0}) || graphs_.count({-T, 1})) return true;
+    if (portion_sizes_seen_.size() >= 64 && !portion_sizes_seen_.count(T)) return false;     // sizes that never repeat
+    return ++portion_sizes_seen_[T] >= 2 && n_portion_graphs_ < 16;
+}
+
+Tensor ModelRunner::step_from_portion_graph(const std::vector<StepEntry>& entries) {
+    const StepEntry& e = entries[0];
+    const int T = static_cast<int>(e.tokens.size());
+    const bool far = e.start_pos + T >= 4096;
+    const int bound = far ? cache.max_context : std::min(4095, cache.max_context);
+    const std::vector<int> caps(static_cast<size_t>(cache.n_groups()), T / cache.page_tokens + 8);
+    BuildOptions options;
+    options.null_slot = cache.null_slot;
+    options.update_caps = &caps;
+    const std::pair<int, int> key{-T, far ? 1 : 0};
+    auto it = graphs_.find(key);
+    if (it == graphs_.end() || it->second.generation != rt.ws.generation) {
+        if (it == graphs_.end()) ++n_portion_graphs_;
+        const std::vector<std::vector<TableUpdate>> empty(static_cast<size_t>(cache.n_groups()));
+        StepEntry spare;
+        spare.slot = cache.null_slot;
+        spare.start_pos = 0;
+        spare.tokens.assign(static_cast<size_t>(T), 0);
+        spare.want = {T - 1};
+        StepBatch batch = builder_->build({spare}, empty, options);
+        batch.context_bound = bound;
+        record(key, batch);
+    }
+    Captured& captured = graphs_.at(key);
+    auto updates = drain_updates(caps);
+    last_batch_ = build(entries, updates, options);
+    CELEG_HIP(hipGraphLaunch(captured.exec, rt.stream));
+    ++steps_run;
+    ++graph_replays;
+    return captured.logits.rows(0, 1);
 }
 
 // ---------------------------------------------------------------------------- loading

@@ -73,6 +73,7 @@ public:
     Runtime& rt;
     const int max_batched_tokens;
     bool use_graphs = true;
+    int portion_graph_min_tokens = 32;      // portions of fewer rows are never recorded
     long long steps_run = 0, graph_replays = 0, captures = 0;
     double capture_seconds = 0.0;
     const StepBatch& last_batch() const { return last_batch_; }
@@ -96,6 +97,9 @@ private:
     int context_bound(const std::vector<StepEntry>& entries) const;
     Tensor step_from_graph(const std::vector<StepEntry>& entries);
     Captured& capture(int bucket, const std::vector<int>& caps, int bound);
+    Captured& record(std::pair<int, int> key, const StepBatch& batch);
+    bool portion_graph_applies(const std::vector<StepEntry>& entries);
+    Tensor step_from_portion_graph(const std::vector<StepEntry>& entries);
     std::vector<std::vector<TableUpdate>> drain_updates(const std::vector<int>& caps);
     StepBatch build(const std::vector<StepEntry>& entries, std::vector<std::vector<TableUpdate>>& updates,
                     const BuildOptions& options);
@@ -104,7 +108,11 @@ private:
     void drop_graphs();
 
     std::unique_ptr<BatchBuilder> builder_;
+    // (batch-size bucket, bound on the context) for steps of single tokens; (-rows, context
+    // from 4,096 tokens or not) for steps of one portion
     std::map<std::pair<int, int>, Captured> graphs_;
+    std::map<int, int> portion_sizes_seen_;
+    int n_portion_graphs_ = 0;
     std::vector<int> buckets_;
     int update_room_ = 0;
     int* token_source_ = nullptr;

@@ -78,10 +78,10 @@ def test_host_code_under_sanitizers(tmp_path):
             pytest.skip(f"the compiler has no sanitizer runtime here: {str(err)[-300:]}")
         raise
     program = os.path.join(work, "host_sanitized")
-    subprocess.run([build._hipcc(), "-std=c++17", "-O1", "-g1", "-fsanitize=address", "-fsanitize=undefined",
-                    "-fno-omit-frame-pointer", "-x", "c++", "-I", os.path.join(ROOT, "celeg_amd", "csrc", "include"),
-                    os.path.join(ROOT, "tests", "c", "host_sanitized.cpp"), "-o", program,
-                    "-L", work, "-l:" + os.path.basename(library), "-Wl,-rpath," + work],
+    subprocess.run([build._hipcc(), "-std=c++17", "-O1", "-g1", "-x", "hip", f"--offload-arch={build.ARCH}"] +
+                   build.SANITIZE_FLAGS + ["-I", os.path.join(ROOT, "celeg_amd", "csrc", "include"),
+                   os.path.join(ROOT, "tests", "c", "host_sanitized.cpp"), "-o", program,
+                   "-L", work, "-l:" + os.path.basename(library), "-Wl,-rpath," + work],
                    check=True, capture_output=True, text=True)
     good = write_random_model(TINY_A, str(tmp_path / "good"), seed=0, dtype=torch.float32, std=0.05)
     broken = broken_folders(str(tmp_path), good)
