@@ -655,6 +655,8 @@ public:
             KVNeed need;
             need.kv_heads = static_cast<int>(j["kv_need"].get_int("kv_heads", 0));
             need.head_dim = static_cast<int>(j["kv_need"].get_int("head_dim", 0));
+            need.v_head_dim = static_cast<int>(j["kv_need"].get_int("v_head_dim", 0));
+            if (need.v_head_dim == need.head_dim) need.v_head_dim = 0;
             if (!j["kv_need"]["window"].is_null()) need.window = static_cast<int>(j["kv_need"]["window"].as_int());
             d_.kv_need = need;
         }
@@ -725,6 +727,8 @@ struct CacheViews {
             view.page_tokens = kv.page_tokens;
             view.kv_heads = kv.kv_heads;
             view.head_dim = kv.head_dim;
+            view.v_head_dim = kv.v_head_dim;
+            view.n_pages = kv.n_pages;
             view.table_stride = kv.table_stride;
             view.table = kv.table;
         }

@@ -61,7 +61,8 @@ void PagePool::check() const {
 long long CacheLayout::kv_bytes_per_token(size_t itemsize) const {
     long long total = 0;
     for (size_t g = 0; g < kv_groups.size(); ++g)
-        total += 2LL * group_layers[g] * kv_groups[g].kv_heads * kv_groups[g].head_dim * static_cast<long long>(itemsize);
+        total += static_cast<long long>(group_layers[g]) * kv_groups[g].kv_heads * (kv_groups[g].head_dim + kv_groups[g].value_dim()) *
+                 static_cast<long long>(itemsize);
     return total;
 }
 
@@ -69,6 +70,7 @@ Json CacheLayout::to_json() const {
     Json groups = Json::array();
     for (size_t g = 0; g < kv_groups.size(); ++g)
         groups.push(Json::object().set("kv_heads", kv_groups[g].kv_heads).set("head_dim", kv_groups[g].head_dim)
+                        .set("v_head_dim", kv_groups[g].value_dim())
                         .set("window", kv_groups[g].window ? Json(*kv_groups[g].window) : Json())
                         .set("layers", group_layers[g]));
     Json uses = Json::array();
@@ -89,6 +91,8 @@ CacheLayout CacheLayout::from_json(const Json& j) {
             KVNeed need;
             need.kv_heads = static_cast<int>(g.get_int("kv_heads", 0));
             need.head_dim = static_cast<int>(g.get_int("head_dim", 0));
+            need.v_head_dim = static_cast<int>(g.get_int("v_head_dim", 0));
+            if (need.v_head_dim == need.head_dim) need.v_head_dim = 0;
             if (!g["window"].is_null()) need.window = static_cast<int>(g["window"].as_int());
             out.kv_groups.push_back(need);
             out.group_layers.push_back(static_cast<int>(g.get_int("layers", 1)));
@@ -142,10 +146,9 @@ CacheManager::CacheManager(CacheLayout layout_, int page_tokens_, std::vector<in
         grp.pages.assign(static_cast<size_t>(max_requests), {});
         grp.first_live.assign(static_cast<size_t>(max_requests), 0);
         if (on_device_) {
-            const size_t bytes = static_cast<size_t>(n_pages[g] + 1) * grp.n_layers * need.kv_heads * page_tokens *
-                                 need.head_dim * itemsize;
-            grp.k = DeviceBuffer(bytes, true);
-            grp.v = DeviceBuffer(bytes, true);
+            const size_t per_dim = static_cast<size_t>(n_pages[g] + 1) * grp.n_layers * need.kv_heads * page_tokens * itemsize;
+            grp.k = DeviceBuffer(per_dim * need.head_dim, true);
+            grp.v = DeviceBuffer(per_dim * need.value_dim(), true);
             grp.table = DeviceBuffer(grp.table_host.size() * sizeof(int));
             CELEG_HIP(hipMemcpy(grp.table.ptr(), grp.table_host.data(), grp.table_host.size() * sizeof(int),
                                 hipMemcpyHostToDevice));
@@ -317,6 +320,7 @@ LayerCache CacheManager::layer_cache(int step) const {
         kv.page_tokens = page_tokens;
         kv.kv_heads = g.need.kv_heads;
         kv.head_dim = g.need.head_dim;
+        kv.v_head_dim = g.need.value_dim();
         kv.group = it->second.group;
         kv.n_pages = g.pool.n_pages() + 1;
         out.kv = kv;

@@ -10,7 +10,7 @@
 // starts, with a region for every layer that declared a need.
 //
 // Storage of a group: K [pages + 1, layers, kv_heads, page_tokens, head_dim] and V
-// [pages + 1, layers, kv_heads, head_dim, page_tokens] (transposed inside a page: the layout
+// [pages + 1, layers, kv_heads, v_head_dim, page_tokens] (transposed inside a page: the layout
 // the matrix-core attention kernel reads without shuffling).  The extra last page is never
 // handed out: rows that pad a batch to a fixed size write there.  Likewise the last slot
 // (null_slot) is never given to a request.
@@ -54,11 +54,16 @@ private:
     std::vector<int> free_, holders_;
 };
 
-// Keys and values of every position, or of a trailing window of positions.
+// Keys and values of every position, or of a trailing window of positions.  Values may have
+// another width than keys (v_head_dim; 0: the keys').
 struct KVNeed {
     int kv_heads = 0, head_dim = 0;
     std::optional<int> window;
-    bool operator==(const KVNeed& o) const { return kv_heads == o.kv_heads && head_dim == o.head_dim && window == o.window; }
+    int v_head_dim = 0;
+    int value_dim() const { return v_head_dim > 0 ? v_head_dim : head_dim; }
+    bool operator==(const KVNeed& o) const {
+        return kv_heads == o.kv_heads && head_dim == o.head_dim && window == o.window && value_dim() == o.value_dim();
+    }
 };
 
 // State of fixed size per request, zero when the request starts.
@@ -90,6 +95,7 @@ struct KVView {
     int* table = nullptr;
     int table_stride = 0, table_rows = 0;
     int page_tokens = 0, kv_heads = 0, head_dim = 0, group = 0, n_pages = 0;
+    int v_head_dim = 0;           // width of a value (the keys' unless the mixer asked for another)
 };
 
 // The cache of one entry of the run order.

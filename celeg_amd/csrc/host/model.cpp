@@ -43,9 +43,9 @@ void Model::resolve_cache_sharing() {
         if (!mine || !theirs)
             throw SpecError("run order entry " + std::to_string(i) + ": only a mixer with keys and values can read " +
                             "another entry's cache, and only from such a mixer");
-        if (mine->kv_heads != theirs->kv_heads || mine->head_dim != theirs->head_dim)
+        if (mine->kv_heads != theirs->kv_heads || mine->head_dim != theirs->head_dim || mine->value_dim() != theirs->value_dim())
             throw SpecError("run order entry " + std::to_string(i) + ": its mixer and the one of entry " +
-                            std::to_string(*step.kv_from) + " differ in kv_heads or head_dim");
+                            std::to_string(*step.kv_from) + " differ in kv_heads, head_dim or the width of the values");
     }
     for (int layer = 0; layer < static_cast<int>(blocks_.size()); ++layer) {
         bool used = false;

@@ -226,6 +226,7 @@ void Ops::short_conv(const Tensor& bcx, const Tensor& weight, const Tensor* bias
 // ---------------------------------------------------------------------------- attention
 static void check_kv(const KVView& kv, int kv_heads, int head_dim, DType dtype) {
     need(kv.kv_heads == kv_heads && kv.head_dim == head_dim, "attention: the cache has other head sizes than the mixer");
+    need(kv.v_head_dim == head_dim, "attention: these kernels take values of the keys' width only");
     need(kv.k && kv.v && kv.table, "attention: the cache has no device memory");
     need(kv.dtype == dtype, std::string("attention: the cache holds ") + dtype_name(kv.dtype) + ", the rows are " + dtype_name(dtype));
     need(kv.layer >= 0 && kv.layer < kv.n_layers, "attention: layer index outside the cache");

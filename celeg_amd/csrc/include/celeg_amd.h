@@ -205,12 +205,13 @@ typedef struct celeg_step_view {
 
 typedef struct celeg_cache_view {
     int32_t has_kv, writes_kv;
-    void *k, *v;                /* [pages + 1, layers, kv_heads, page_tokens, head_dim] and V with the last two swapped */
+    void *k, *v;                /* K [n_pages, layers, kv_heads, page_tokens, head_dim], V [n_pages, layers, kv_heads, v_head_dim, page_tokens] */
     int32_t kv_dtype, layer, n_layers, page_tokens, kv_heads, head_dim, table_stride;
     const int32_t* table;       /* [slots + 1, table_stride] */
     int32_t n_states;
     const char* const* state_names;
     const celeg_tensor_view* states;    /* [slots + 1, shape...] each */
+    int32_t v_head_dim, n_pages;        /* width of a value; pages of the pool, the spare one included */
 } celeg_cache_view;
 
 typedef struct celeg_forward_args {
@@ -227,7 +228,7 @@ typedef struct celeg_forward_args {
 
 /* A part as functions.  describe() returns JSON:
  *   {"weights": {role: {"shape": [..], "kind": "matrix"|"vector", "init": "normal"|"around_one"}},
- *    "kv_need": {"kv_heads", "head_dim", "window"} or null, "states": [{"name", "shape", "dtype"}],
+ *    "kv_need": {"kv_heads", "head_dim", "window", "v_head_dim" (optional: values of another width)} or null, "states": [{"name", "shape", "dtype"}],
  *    "graph_safe": bool, "out_width": columns of what forward writes (mixer, ffn),
  *    "inv_freq": [..], "rotary_dim": n, "pairing": "halves"|"neighbours"  (position encodings: pair i of
  *    the first n values of a head, (i, i + n/2) or (2i, 2i + 1), turns by position * inv_freq[i])}

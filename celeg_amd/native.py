@@ -66,7 +66,7 @@ class CacheView(ctypes.Structure):
     _fields_ = [("has_kv", c_int32), ("writes_kv", c_int32), ("k", c_void_p), ("v", c_void_p), ("kv_dtype", c_int32),
                 ("layer", c_int32), ("n_layers", c_int32), ("page_tokens", c_int32), ("kv_heads", c_int32),
                 ("head_dim", c_int32), ("table_stride", c_int32), ("table", c_void_p), ("n_states", c_int32),
-                ("state_names", P(c_char_p)), ("states", P(TensorView))]
+                ("state_names", P(c_char_p)), ("states", P(TensorView)), ("v_head_dim", c_int32), ("n_pages", c_int32)]
 
 
 class ForwardArgs(ctypes.Structure):
