@@ -1,0 +1,59 @@
+"""The configuration that bench.py measures (LFM2-350M shape: 16 layers, width 1,024, 65,536
+tokens of vocabulary, random weights of the benchmark's own spread), whole depth, in bfloat16:
+the logits of a prompt fed whole, in portions and with its last tokens decoded one by one, and
+greedy tokens through the engine, against the plain implementation."""
+import sys
+
+import pytest
+import torch
+
+import plain_lfm2 as plain
+from helpers import ROOT, EngineDriver, assert_close_bf16, portions_schedule, random_tokens, tail_decode_schedule
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def benchmark_model(tmp_path_factory):
+    sys.path.insert(0, ROOT)
+    from bench import SHAPES
+    from celeg_amd.weights import write_random_model
+    cfg = dict(SHAPES["350m"][0])
+    folder = write_random_model(cfg, str(tmp_path_factory.mktemp("bench_350m")), seed=0, dtype=torch.bfloat16, std=0.02)
+    pcfg, W = plain.load_model_folder(folder)
+    return folder, pcfg, W
+
+
+def test_logits_at_the_benchmarks_configuration(benchmark_model):
+    from celeg_amd.engine import load_model
+    folder, cfg, W = benchmark_model
+    assert len(plain.normalise_config(cfg)["layer_types"]) == 16 and cfg["vocab_size"] == 65536
+    reqs = {"a": random_tokens(cfg["vocab_size"], 100, seed=1), "b": random_tokens(cfg["vocab_size"], 61, seed=2)}
+    ref = {rid: plain.model_logits(cfg, W, toks).float() for rid, toks in reqs.items()}
+    lm = load_model(folder, dtype="bfloat16", page_tokens=16, n_pages=16, max_requests=2, max_context=256,
+                    max_batched_tokens=128)
+    for mode, schedule in (("tail32", tail_decode_schedule), ("portions", portions_schedule)):
+        got = EngineDriver(lm).run(schedule(reqs))
+        for rid in reqs:
+            assert_close_bf16(got[rid], ref[rid], f"benchmark configuration/{mode}/{rid}")
+    assert lm.runner.counters()["graph_replays"] >= 32       # the single tokens went through recorded steps
+    lm.close()
+
+
+def test_greedy_tokens_at_the_benchmarks_configuration(benchmark_model):
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY
+    folder, cfg, W = benchmark_model
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=10 + n) for n in (40, 9)]
+    engine = Engine.from_folder(folder, dtype="bfloat16", max_active_requests=2, n_pages=16, context=256,
+                                max_batched_tokens=64, prefill_chunk_tokens=32)
+    outs = engine.generate(prompts, max_new_tokens=10, generation=GREEDY, eos_token_ids=[])
+    for prompt, out in zip(prompts, outs):
+        seq, exact = list(prompt), 0
+        for token in out:
+            logits = plain.model_logits(cfg, W, seq)[-1]
+            assert float(logits[token]) >= float(logits.max()) - 4e-2 * float(logits.abs().max())
+            exact += int(token == int(logits.argmax()))
+            seq.append(token)
+        assert len(out) == 10 and exact >= 8
+    assert engine.metrics["graph_replays"] > 0
