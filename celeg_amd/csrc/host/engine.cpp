@@ -164,11 +164,18 @@ long long Engine::run_steps(long long limit) {
     bool have = false;
     Launched launched;
     long long done = 0, begun = 0;
+    int idle = 0;
     while (have || (has_work() && (limit < 0 || begun < limit))) {
         if (!have) {
             std::vector<PlannedEntry> plan = scheduler_->plan();
             sync_slots();
-            if (plan.empty()) continue;
+            if (plan.empty()) {
+                // (the scheduler ends or fails what cannot advance, so this does not repeat; a
+                // loop that spins on nothing must still end)
+                if (++idle > 1000) throw StepError("the scheduler has work but plans no step");
+                continue;
+            }
+            idle = 0;
             ++begun;
             if (!launch(plan, false, launched)) continue;
             have = true;

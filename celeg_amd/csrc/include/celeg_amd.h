@@ -6,6 +6,9 @@
  * src/api/options.cpp:7-101), plus the low-level step function that trace replay drives and
  * the hooks through which parts and architectures defined outside this library are registered.
  *
+ * An engine or a model serves one thread at a time: calls on the same handle must not overlap
+ * (different handles are independent; the registries are guarded).
+ *
  * Every function that can fail returns a celeg_status; the message of the last failure on the
  * calling thread is celeg_last_error().  Functions that return text return a pointer that stays
  * valid until the calling thread's next call of a function of this library that returns text.
