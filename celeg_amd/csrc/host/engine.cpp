@@ -93,7 +93,14 @@ bool Engine::launch(const std::vector<PlannedEntry>& plan, bool device_tokens, L
         Tensor logits = loaded_->runner->step(entries);
         last_logits_ = logits;
         steps_ahead_ += device_tokens ? 1 : 0;
-        if (sampler_->uses_seen()) sampler_->mark_seen(loaded_->runner->last_batch());
+        // tokens that count as seen by their request: the sampler's kernels mark what they choose,
+        // so a step that only feeds such tokens back (every entry the one new token of a
+        // decoding request) has nothing to mark; prompts, and what a request that was put back
+        // feeds again, are marked here
+        bool feeds_prompt = false;
+        for (const PlannedEntry& e : plan)
+            feeds_prompt = feeds_prompt || e.count != 1 || e.request->status != RequestStatus::Decoding;
+        if (feeds_prompt && sampler_->uses_seen()) sampler_->mark_seen(loaded_->runner->last_batch());
         if (!slots.empty()) sampler_->launch(logits, slots);
         out.sampled_rows = !slots.empty();
         return true;

@@ -59,10 +59,10 @@ int celeg_attention_decode_bf16(const void* q, int ldq, const void* k_pool, cons
                                 int window, int whole, int split_rounds, int n_parts, hipStream_t stream);
 // sampling.hip
 int celeg_argmax_rows(const float* logits, int ld, int rows, int vocab, const float* fparams, const int* iparams,
-                      const uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens,
+                      uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens,
                       unsigned long long* best, unsigned int* arrived, hipStream_t stream);
 int celeg_sample(const float* logits, int ld, int rows, int vocab, const float* fparams, const int* iparams,
-                 const uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens, hipStream_t stream);
+                 uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens, hipStream_t stream);
 int celeg_mark_seen(uint8_t* seen, size_t stride, int n_slots, int vocab, const int* tokens, const int* slots, int n,
                     hipStream_t stream);
 // gemv_slices.hip, gemm_rows.hip, gemv_fused.hip: the fused products for up to 64 rows

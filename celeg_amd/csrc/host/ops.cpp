@@ -348,7 +348,7 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
 }
 
 // ---------------------------------------------------------------------------- sampling
-void Ops::sample(const Tensor& logits, const float* fparams, const int* iparams, const uint8_t* seen, size_t seen_stride,
+void Ops::sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen, size_t seen_stride,
                  int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws) {
     dev(logits, "logits", DType::F32, false);
     const int R = static_cast<int>(logits.shape[0]), V = static_cast<int>(logits.shape[1]);
@@ -364,6 +364,10 @@ void Ops::sample(const Tensor& logits, const float* fparams, const int* iparams,
                      "argmax of rows");
         return;
     }
+    // (A row of a sampled step cut into parts over many workgroups, the last one to arrive merging
+    // the parts' lists, was measured: 21 against 23 us for one row of 65,536 logits and top_k 50,
+    // slower from 8 rows on and at top_k 128: what the kernel spends lies in the ranking and the
+    // sums, not in reading the logits.)
     kernel_check(celeg_sample(logits.as<float>(), rows_of(logits, "logits"), R, V, fparams, iparams, seen, seen_stride,
                               out_tokens, last_tokens, stream), "sample");
 }

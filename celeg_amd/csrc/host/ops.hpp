@@ -82,7 +82,7 @@ public:
     void paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
                          int window, const StepBatch& batch, const KVView& kv, Workspace& ws);
     // sampling
-    void sample(const Tensor& logits, const float* fparams, const int* iparams, const uint8_t* seen,
+    void sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen,
                 size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws);
     void mark_seen(uint8_t* seen, size_t stride, int n_slots, int vocab, const int* token_ids, const int* token_slot, int n);
     // fused skinny products

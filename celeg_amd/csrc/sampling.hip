@@ -343,12 +343,83 @@ __device__ __forceinline__ bool top_k_ranked(
     return true;
 }
 
+// What one wavefront does with the candidates (cand_score / cand_id [0, SAMPLE_MAX_K) in LDS, the
+// places from top_k on holding (-inf, max id)): sorts them by (score desc, id asc) unless they
+// came so, then softmax, the top-p prefix and the walk with the draw u.  Returns the token
+// (the same value in every lane).
+__device__ __forceinline__ int choose_among(float* cand_score, int* cand_id, int top_k, float top_p, float u,
+                                            bool sorted, int lane) {
+    // ---- bitonic sort of 128 candidates by (score desc, id asc), unless they came in that
+    // order: lane l owns the pair whose lower member is the l-th position with the stride's bit clear
+    for (int size = sorted ? 2 * SAMPLE_MAX_K : 2; size <= SAMPLE_MAX_K; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            const int a = ((lane & ~(stride - 1)) << 1) | (lane & (stride - 1));
+            const int partner = a | stride;
+            const bool ascending_block = (a & size) == 0;  // "best first" blocks
+            const float sa = cand_score[a], sb = cand_score[partner];
+            const int ia = cand_id[a], ib = cand_id[partner];
+            const bool a_first = better(sa, ia, sb, ib);
+            if (ascending_block ? !a_first : a_first) {
+                cand_score[a] = sb; cand_id[a] = ib;
+                cand_score[partner] = sa; cand_id[partner] = ia;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    }
+
+    // ---- softmax, top-p prefix and the walk.  The sums run over the candidates one after
+    // the other, in the reference's order: every lane runs the same loops over the values in
+    // LDS (reads of one address by all lanes, asked for ahead of the additions that need them;
+    // a value handed from lane to lane for every addition cost ten times the addition).
+    const float maximum = cand_score[0];
+    const int id0 = cand_id[lane], id1 = cand_id[lane + 64];
+    const float e0 = expf(cand_score[lane] - maximum), e1 = expf(cand_score[lane + 64] - maximum);
+    auto wave_sync = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    wave_sync();                       // every lane has read the scores it needs
+    float* const prob = cand_score;    // from here on the array holds exp(score - max), then the probabilities
+    prob[lane] = e0;
+    prob[lane + 64] = e1;
+    wave_sync();
+    float total = 0.f;
+    for (int i = 0; i < top_k; ++i) total += prob[i];
+    wave_sync();
+    prob[lane] = e0 / total;
+    prob[lane + 64] = e1 / total;
+    wave_sync();
+    int active = top_k;
+    if (top_p < 1.0f) {
+        float cumulative = 0.f;
+        active = 0;
+        do {
+            cumulative += prob[active++];
+        } while (active < top_k && cumulative < top_p);
+        total = 0.f;
+        for (int i = 0; i < active; ++i) total += prob[i];
+    } else {
+        total = 1.0f;
+    }
+    float target = u * total;
+    int chosen_at = active - 1;
+    for (int i = 0; i < active; ++i) {
+        target -= prob[i];
+        if (target <= 0.0f) { chosen_at = i; break; }
+    }
+    return __shfl(chosen_at < 64 ? id0 : id1, chosen_at & 63, CELEG_WAVE);
+}
+
 // fparams[row] = {temperature, top_p, penalty, u}; iparams[row] = {top_k, seen_row or -1,
 // slot or -1}; the token also goes to last_tokens[slot] (if given and slot >= 0), where the
-// next step can take it from without the host in between.
+// next step can take it from without the host in between, and is marked as seen in the row's
+// seen_row (if any): the step that feeds it back need not mark it.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ fparams,
-    const int* __restrict__ iparams, const uint8_t* __restrict__ seen_all, size_t seen_stride,
+    const int* __restrict__ iparams, uint8_t* __restrict__ seen_all, size_t seen_stride,
     int* __restrict__ out_tokens, int* __restrict__ last_tokens) {
     __shared__ float s_val[SAMPLE_THREADS / CELEG_WAVE];
     __shared__ int s_idx[SAMPLE_THREADS / CELEG_WAVE];
@@ -396,6 +467,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                 }
             out_tokens[r] = best_i;
             if (last_tokens && slot >= 0) last_tokens[slot] = best_i;
+            if (seen_all && seen_row >= 0) seen_all[static_cast<size_t>(seen_row) * seen_stride + best_i] = 1;
         }
         return;
     }
@@ -421,62 +493,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     if (tid >= top_k && tid < SAMPLE_MAX_K) { cand_score[tid] = -INFINITY; cand_id[tid] = 0x7fffffff; }
     __syncthreads();
     if (wave != 0) return;         // one wavefront does the rest: no workgroup barriers from here
-
-    // ---- bitonic sort of 128 candidates by (score desc, id asc), unless they came in that
-    // order: lane l owns the pair whose lower member is the l-th position with the stride's bit clear
-    for (int size = sorted ? 2 * SAMPLE_MAX_K : 2; size <= SAMPLE_MAX_K; size <<= 1) {
-        for (int stride = size >> 1; stride > 0; stride >>= 1) {
-            const int a = ((lane & ~(stride - 1)) << 1) | (lane & (stride - 1));
-            const int partner = a | stride;
-            const bool ascending_block = (a & size) == 0;  // "best first" blocks
-            const float sa = cand_score[a], sb = cand_score[partner];
-            const int ia = cand_id[a], ib = cand_id[partner];
-            const bool a_first = better(sa, ia, sb, ib);
-            if (ascending_block ? !a_first : a_first) {
-                cand_score[a] = sb; cand_id[a] = ib;
-                cand_score[partner] = sa; cand_id[partner] = ia;
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        }
-    }
-
-    // ---- softmax, top-p prefix and the walk.  The sums run over the candidates one after
-    // the other, in the reference's order; a candidate's value comes from the lane that
-    // holds it (lane i % 64, first or second register), so that the loops touch no memory.
-    const float maximum = cand_score[0];
-    float e0 = expf(cand_score[lane] - maximum), e1 = expf(cand_score[lane + 64] - maximum);
-    const int id0 = cand_id[lane], id1 = cand_id[lane + 64];
-    auto value_at = [&](float first, float second, int i) {
-        return __shfl(i < 64 ? first : second, i & 63, CELEG_WAVE);
-    };
-    float total = 0.f;
-    for (int i = 0; i < top_k; ++i) total += value_at(e0, e1, i);
-    e0 /= total;
-    e1 /= total;
-    int active = top_k;
-    if (top_p < 1.0f) {
-        float cumulative = 0.f;
-        active = 0;
-        do {
-            cumulative += value_at(e0, e1, active++);
-        } while (active < top_k && cumulative < top_p);
-        total = 0.f;
-        for (int i = 0; i < active; ++i) total += value_at(e0, e1, i);
-    } else {
-        total = 1.0f;
-    }
-    float target = u * total;
-    int chosen_at = active - 1;
-    for (int i = 0; i < active; ++i) {
-        target -= value_at(e0, e1, i);
-        if (target <= 0.0f) { chosen_at = i; break; }
-    }
-    const int chosen = __shfl(chosen_at < 64 ? id0 : id1, chosen_at & 63, CELEG_WAVE);
+    const int chosen = choose_among(cand_score, cand_id, top_k, top_p, u, sorted, lane);
     if (lane == 0) {
         out_tokens[r] = chosen;
         if (last_tokens && slot >= 0) last_tokens[slot] = chosen;
+        if (seen_all && seen_row >= 0) seen_all[static_cast<size_t>(seen_row) * seen_stride + chosen] = 1;
     }
 }
 
@@ -491,7 +512,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 #define ARGMAX_THREADS 256
 __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(
     const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ fparams,
-    const int* __restrict__ iparams, const uint8_t* __restrict__ seen_all, size_t seen_stride,
+    const int* __restrict__ iparams, uint8_t* __restrict__ seen_all, size_t seen_stride,
     int* __restrict__ out_tokens, int* __restrict__ last_tokens, unsigned long long* __restrict__ best,
     unsigned int* __restrict__ arrived) {
     constexpr int PER = ARGMAX_PART / ARGMAX_THREADS;
@@ -542,13 +563,14 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(
     const int token = static_cast<int>(0xffffffffu - static_cast<unsigned>(winner & 0xffffffffull));
     out_tokens[r] = token;
     if (last_tokens && slot >= 0) last_tokens[slot] = token;
+    if (seen_all && seen_row >= 0) seen_all[static_cast<size_t>(seen_row) * seen_stride + token] = 1;
 }
 
 // rows that are all greedy (temperature <= 0 or top_k == 1): best [rows] and arrived [rows]
 // must hold zeros when the first launch comes (the kernel leaves them so).  Launches that
 // share them must run one after the other.
 extern "C" int celeg_argmax_rows(const float* logits, int ld, int rows, int vocab, const float* fparams,
-                                 const int* iparams, const uint8_t* seen, size_t seen_stride,
+                                 const int* iparams, uint8_t* seen, size_t seen_stride,
                                  int* out_tokens, int* last_tokens, unsigned long long* best,
                                  unsigned int* arrived, hipStream_t stream) {
     if (rows <= 0) return 0;
@@ -560,7 +582,7 @@ extern "C" int celeg_argmax_rows(const float* logits, int ld, int rows, int voca
 }
 
 extern "C" int celeg_sample(const float* logits, int ld, int rows, int vocab,
-                            const float* fparams, const int* iparams, const uint8_t* seen,
+                            const float* fparams, const int* iparams, uint8_t* seen,
                             size_t seen_stride, int* out_tokens, int* last_tokens,
                             hipStream_t stream) {
     if (rows <= 0) return 0;
