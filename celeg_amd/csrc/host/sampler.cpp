@@ -37,7 +37,6 @@ Sampler::Sampler(Runtime& rt, int vocab, int max_requests) : rt_(rt), vocab_(voc
         std::memset(p.ptr(), 0, cap * 7 * 4);
     }
     params_dev_ = DeviceBuffer(cap * 7 * 4, true);
-    tokens_dev_ = DeviceBuffer(cap * 4, true);
     last_tokens_ = DeviceBuffer((cap + 1) * 4, true);
     // sampled tokens come back through two pinned buffers that take turns, so that one step's
     // tokens can still be on their way while the next step is launched
@@ -113,9 +112,10 @@ void Sampler::launch(const Tensor& logits, const std::vector<int>& slots) {
     }
     const float* fdev = params_dev_.as<float>();
     const int* idev = reinterpret_cast<const int*>(fdev + cap * 4);
-    rt_.ops.sample(logits, fdev, idev, seen_.as<uint8_t>(), static_cast<size_t>(vocab_), tokens_dev_.as<int>(),
+    // the kernels write the tokens straight into the turn's pinned buffer (memory of the host that
+    // the device can address): no copy behind them, the event tells when they are there
+    rt_.ops.sample(logits, fdev, idev, seen_.as<uint8_t>(), static_cast<size_t>(vocab_), tokens_host_[turn].as<int>(),
                    last_tokens_.as<int>(), all_greedy, rt_.ws);
-    CELEG_HIP(hipMemcpyAsync(tokens_host_[turn].ptr(), tokens_dev_.ptr(), static_cast<size_t>(R) * 4, hipMemcpyDeviceToHost, rt_.stream));
     CELEG_HIP(hipEventRecord(events_[turn], rt_.stream));
     pending_.emplace_back(turn, R);
 }

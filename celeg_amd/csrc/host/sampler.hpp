@@ -71,7 +71,7 @@ private:
     std::map<int, std::shared_ptr<XorShift64Star>> rng_;
     DeviceBuffer seen_;            // [max_requests, vocab] bytes, made on need
     PinnedBuffer params_[2];       // 4 floats a row, then 3 ints a row
-    DeviceBuffer params_dev_, tokens_dev_, last_tokens_;
+    DeviceBuffer params_dev_, last_tokens_;
     std::vector<uint32_t> uploaded_;
     PinnedBuffer tokens_host_[2];
     hipEvent_t events_[2] = {nullptr, nullptr};
