@@ -44,12 +44,188 @@ enum { T_STORE = 0, T_RESIDUAL = 2, T_SWIGLU = 3 };   // the numbers of the few-
 
 __device__ __forceinline__ float round_bf16(float x) { return to_float(from_float<bf16>(x)); }
 
+#ifdef CELEG_TILES_FAST_SILU
+__device__ __forceinline__ float tile_silu(float g) { return g * __frcp_rn(1.0f + __expf(-g)); }
+#else
+__device__ __forceinline__ float tile_silu(float g) { return g / (1.0f + expf(-g)); }
+#endif
+
 template <int N>
 __device__ __forceinline__ void wait_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
 template <int EPI> struct TileStreams { static constexpr int n = EPI == T_SWIGLU ? 2 : 1; };
+
+// The 1/rms of a lane's rows (first, first + 16, ..) from the partial sums of squares that
+// the producer of the stream left; 1 without a norm.  The four lanes that share a row (q = 0..3)
+// take four partial sums each, as one load where the rows are aligned, and add up over the
+// lanes: a few loads a lane, all in flight at once.  (One lane reading all of a row's sums,
+// eight at a time, cost a product of 2,048 rows 12 us: 64 loads a lane in two trips, queued
+// behind the first blocks of the operands.)
+template <int FM>
+__device__ __forceinline__ void tile_row_scales(const TileParams& p, const int first, const int q, float (&scale)[FM]) {
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) scale[tm] = 1.f;
+    if (!p.stats) return;
+    const int nb = p.n_stat_blocks;
+    const bool aligned = (p.stats_ld & 3) == 0 && (reinterpret_cast<uintptr_t>(p.stats) & 15) == 0;
+    float ssq[FM];
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) ssq[tm] = 0.f;
+    for (int c0 = 0; c0 < nb; c0 += 16) {         // (once, up to 16 partial sums a row)
+        const int b = c0 + 4 * q;
+        floatx4_t part[FM];
+#pragma unroll
+        for (int tm = 0; tm < FM; ++tm) {
+            const float* const srow = p.stats + static_cast<size_t>(min(first + tm * 16, p.M - 1)) * p.stats_ld;
+            if (aligned && b + 4 <= nb) {
+                part[tm] = *reinterpret_cast<const floatx4_t*>(srow + b);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) part[tm][i] = b + i < nb ? srow[b + i] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int tm = 0; tm < FM; ++tm) ssq[tm] += (part[tm][0] + part[tm][1]) + (part[tm][2] + part[tm][3]);
+    }
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) {
+        float t = ssq[tm];
+        t += __shfl_xor(t, 16, 64);
+        t += __shfl_xor(t, 32, 64);
+        scale[tm] = 1.0f / sqrtf(t / static_cast<float>(p.K) + p.eps);
+    }
+}
+
+// What becomes of a wavefront's sums (shared by the kernels below).  The wavefront (wm, wn) of
+// the tile holds rows m0 + wm*WTM .. of `pieces` (<= FNS) column pieces of 16 from column col0 of
+// every stream:  acc[s*FNS + j][tm][i] is row .. + tm*16 + lane%16, column col0 + j*16 + 4*(lane/16) + i.
+// ROWS_VIA_LDS (store and SwiGLU): a lane's pieces of 4 columns go to the wavefront's corner of
+// LDS first and leave in whole rows of the wavefront's tile, 16 bytes a lane; straight from the
+// registers a store instruction would touch 16 rows with 32 bytes each.
+template <int BM, int WGM, int WGN, int FNS, int EPI, bool ROWS_VIA_LDS>
+__device__ __forceinline__ void tile_epilogue(
+    const TileParams& p, floatx4_t (&acc)[TileStreams<EPI>::n * FNS][BM / WGM / 16], const float (&scale)[BM / WGM / 16],
+    const int m0, const int col0, const int pieces, const int tile_n, const int wm, const int wn, const int lane,
+    char* const lds) {
+    constexpr int NW = WGM * WGN;
+    constexpr int NS = TileStreams<EPI>::n;
+    constexpr int WTM = BM / WGM;
+    constexpr int FM = WTM / 16;
+    const int M = p.M, N = p.N;
+    const int r16 = lane & 15, q = lane >> 4;
+    // the residual stream's old values: all asked for at once where the registers hold them
+    // beside the sums, else a row of pieces at a time
+    constexpr bool RES = EPI == T_RESIDUAL;
+    constexpr bool OLD_AT_ONCE = FM * FNS <= 32;
+    floatx4_t old_[RES && OLD_AT_ONCE ? FM : 1][RES ? FNS : 1];
+    auto fetch_old = [&](int tm, floatx4_t (&to)[RES ? FNS : 1]) {
+#pragma unroll
+        for (int j = 0; j < (RES ? FNS : 1); ++j) {
+            const int m = min(m0 + wm * WTM + tm * 16 + r16, M - 1);
+            const int n = min(col0 + j * 16 + 4 * q, N - 4);
+            to[j] = *reinterpret_cast<const floatx4_t*>(static_cast<const float*>(p.out) + static_cast<size_t>(m) * p.ldo + n);
+        }
+    };
+    if (RES && OLD_AT_ONCE) {
+#pragma unroll
+        for (int tm = 0; tm < FM; ++tm) fetch_old(tm, old_[RES && OLD_AT_ONCE ? tm : 0]);
+    }
+    constexpr int PITCH = FNS * 32 + 16;          // bytes between a wavefront's rows in LDS
+    constexpr bool VIA_LDS = ROWS_VIA_LDS && !RES;
+    char* const corner = lds + static_cast<size_t>(wm * WGN + wn) * WTM * PITCH;
+    if (VIA_LDS) __syncthreads();                 // the stages are no longer read
+    float sq[FM];
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) sq[tm] = 0.f;
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) {
+        const int m = m0 + wm * WTM + tm * 16 + r16;
+        if (RES && !OLD_AT_ONCE) fetch_old(tm, old_[0]);
+#pragma unroll
+        for (int j = 0; j < FNS; ++j) {
+            const int n = col0 + j * 16 + 4 * q;
+            if (j >= pieces || m >= M || n >= N) continue;       // N % 4 == 0: a lane's four columns are inside together
+            float v[NS][4];
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    v[s][i] = acc[s * FNS + j][tm][i] * scale[tm] +
+                              (p.bias ? p.bias[static_cast<size_t>(s) * p.stream_rows + n + i] : 0.f);
+            if (EPI == T_RESIDUAL) {
+                float* const h = static_cast<float*>(p.out) + static_cast<size_t>(m) * p.ldo + n;
+                floatx4_t old = old_[RES && OLD_AT_ONCE ? tm : 0][RES ? j : 0];
+                // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    old[i] += round_bf16(v[0][i]);
+                    sq[tm] += old[i] * old[i];
+                }
+                *reinterpret_cast<floatx4_t*>(h) = old;
+                if (p.out_bf16)     // (the conversion rounds to nearest even, as from_float<bf16>)
+                    *reinterpret_cast<bf16x4_t*>(p.out_bf16 + static_cast<size_t>(m) * p.ld_bf16 + n) =
+                        bf16x4_t{static_cast<__bf16>(old[0]), static_cast<__bf16>(old[1]),
+                                 static_cast<__bf16>(old[2]), static_cast<__bf16>(old[3])};
+            } else {
+                float o[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (EPI == T_SWIGLU) {
+                        const float g = round_bf16(v[0][i]), u = round_bf16(v[NS - 1][i]);
+                        o[i] = tile_silu(g) * u;
+                    } else {
+                        o[i] = v[0][i];
+                    }
+                }
+                const bf16x4_t piece = bf16x4_t{static_cast<__bf16>(o[0]), static_cast<__bf16>(o[1]),
+                                                static_cast<__bf16>(o[2]), static_cast<__bf16>(o[3])};
+                if (VIA_LDS) *reinterpret_cast<bf16x4_t*>(corner + (tm * 16 + r16) * PITCH + (j * 16 + 4 * q) * 2) = piece;
+                else *reinterpret_cast<bf16x4_t*>(static_cast<bf16*>(p.out) + static_cast<size_t>(m) * p.ldo + n) = piece;
+            }
+        }
+    }
+    if (VIA_LDS) {
+        // (the wavefront reads what its own lanes wrote: LDS keeps a wavefront's accesses in order)
+        const int cpr = pieces * 2;               // chunks of 8 columns a row
+        const bool wide_stores = (p.ldo % 8) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
+        for (int idx = lane; idx < WTM * cpr; idx += 64) {
+            const int row = idx / cpr, ch = idx % cpr;
+            const int m = m0 + wm * WTM + row, n = col0 + ch * 8;
+            if (m >= M || n >= N) continue;
+            const char* const from = corner + row * PITCH + ch * 16;
+            bf16* const to = static_cast<bf16*>(p.out) + static_cast<size_t>(m) * p.ldo + n;
+            if (wide_stores && n + 8 <= N) {
+                *reinterpret_cast<bf16x8_t*>(to) = *reinterpret_cast<const bf16x8_t*>(from);
+            } else {
+                *reinterpret_cast<bf16x4_t*>(to) = *reinterpret_cast<const bf16x4_t*>(from);
+                if (n + 8 <= N) *reinterpret_cast<bf16x4_t*>(to + 4) = *reinterpret_cast<const bf16x4_t*>(from + 8);
+            }
+        }
+    }
+
+    if (EPI == T_RESIDUAL && p.stats_out) {
+        // a row's squares: over the lane's columns (above), the four lanes that share the
+        // row, then the wavefronts that share it, always in the same order
+        float* const red = reinterpret_cast<float*>(lds);
+        __syncthreads();                          // the stages are no longer read
+#pragma unroll
+        for (int tm = 0; tm < FM; ++tm) {
+            float s = sq[tm];
+            s += __shfl_xor(s, 16, 64);
+            s += __shfl_xor(s, 32, 64);
+            if (q == 0) red[wn * BM + wm * WTM + tm * 16 + r16] = s;
+        }
+        __syncthreads();
+        for (int r = threadIdx.x; r < BM; r += NW * 64) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < WGN; ++w) s += red[w * BM + r];
+            if (m0 + r < M) p.stats_out[static_cast<size_t>(m0 + r) * p.stats_ld_out + tile_n] = s;
+        }
+    }
+}
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, int EPI>
 __global__ __launch_bounds__(WGM * WGN * 64)
@@ -60,8 +236,9 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
     constexpr int FM = WTM / 16, FN = WTN / 16;
     constexpr int STAGE_BYTES = (BM + BN) * 128;
     constexpr int GROUPS = (BM + BN) / 8;          // loads of 1 KB a block of k
-    constexpr int GPW = GROUPS / NW;               // of which a wavefront issues this many
-    static_assert(GROUPS % NW == 0 && FN % NS == 0 && WTM % 16 == 0 && WTN % 16 == 0, "tile shape");
+    constexpr int GPW = (GROUPS + NW - 1) / NW;    // of which a wavefront issues this many (where they do
+                                                   // not divide, the last ones ask for the last group again)
+    static_assert(FN % NS == 0 && WTM % 16 == 0 && WTN % 16 == 0, "tile shape");
     static_assert(GPW * STAGES < 64, "more loads in flight than the counter holds");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -87,7 +264,7 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
     const char* src[GPW];
 #pragma unroll
     for (int i = 0; i < GPW; ++i) {
-        const int g = wave + i * NW;
+        const int g = min(wave + i * NW, GROUPS - 1);
         const int row = 8 * g + (lane >> 3);               // the row whose chunk lands at this lane's place
         const int chunk = (lane & 7) ^ (row & 7);
         if (g < BM / 8) {
@@ -105,7 +282,7 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
 #pragma unroll
         for (int i = 0; i < GPW; ++i)
             __builtin_amdgcn_global_load_lds(GPTR(src[i] + static_cast<size_t>(kb) * 128),
-                                             LPTR(base + (wave + i * NW) * 1024), 16, 0, 0);
+                                             LPTR(base + min(wave + i * NW, GROUPS - 1) * 1024), 16, 0, 0);
     };
 
     // ---- where this lane's operands lie inside a 16-row piece of a stage (k-step 0 and 1)
@@ -121,40 +298,14 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
 #pragma unroll
         for (int tm = 0; tm < FM; ++tm) acc[tn][tm] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
+    // ---- the rows' 1/rms, asked for ahead of the first blocks
+    float scale[FM];
+    tile_row_scales<FM>(p, m0 + wm * WTM + r16, q, scale);
+
     const int nkb = K >> 6;                       // K % 64 == 0 (checked by the host)
 #pragma unroll
     for (int s = 0; s < STAGES; ++s)
         if (s < nkb) issue(s, s);
-
-    // ---- the rows' 1/rms, asked for behind the first blocks
-    float scale[FM];
-#pragma unroll
-    for (int tm = 0; tm < FM; ++tm) scale[tm] = 1.f;
-    if (p.stats) {
-        // eight partial sums of every row in flight at once (a chain of single loads would
-        // cost a trip to memory each)
-        const float* srow[FM];
-        float ssq[FM];
-#pragma unroll
-        for (int tm = 0; tm < FM; ++tm) {
-            srow[tm] = p.stats + static_cast<size_t>(min(m0 + wm * WTM + tm * 16 + r16, M - 1)) * p.stats_ld;
-            ssq[tm] = 0.f;
-        }
-        const int nb = p.n_stat_blocks;
-        for (int b0 = 0; b0 < nb; b0 += 8) {
-            float part[FM][8];
-#pragma unroll
-            for (int tm = 0; tm < FM; ++tm)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) part[tm][i] = srow[tm][min(b0 + i, nb - 1)];
-#pragma unroll
-            for (int tm = 0; tm < FM; ++tm)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) ssq[tm] += b0 + i < nb ? part[tm][i] : 0.f;
-        }
-#pragma unroll
-        for (int tm = 0; tm < FM; ++tm) scale[tm] = 1.0f / sqrtf(ssq[tm] / static_cast<float>(K) + p.eps);
-    }
 
     // Operands of a k-step (32 values of k) travel from LDS to registers one step ahead of
     // the matrix instructions that use them: a wavefront asks for step 1 of a block, then
@@ -203,90 +354,137 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
         stage = next;
     }
 
-    // ---- acc[tn][tm][i]: row m0 + wm*WTM + tm*16 + lane%16, column (of the stream) ... + 4*(lane/16) + i
-    constexpr int FNS = FN / NS;                  // column pieces of 16 per stream
-    // the residual stream's old values, all asked for at once
-    floatx4_t old_[EPI == T_RESIDUAL ? FM : 1][EPI == T_RESIDUAL ? FNS : 1];
-    if (EPI == T_RESIDUAL) {
+    tile_epilogue<BM, WGM, WGN, FN / NS, EPI, false>(p, acc, scale, m0, n0 + wn * (WTN / NS), FN / NS, tile_n, wm, wn, lane, lds);
+}
+
+// The same product with wide tiles (256 rows x up to 288 weight rows a workgroup), for the
+// products whose operands would otherwise cross from the L2 caches to the compute units many
+// times over.  A wavefront's tile is too large to hold a block's operands in registers beside
+// its sums, so the weights' operands stream from LDS a piece at a time while the matrix
+// instructions of the piece before run; blocks are KB = 32 or 64 values of k (rows of 64 or
+// 128 bytes in LDS, a load instruction fills 16 or 8 rows), STAGES of them, with one barrier a
+// block: behind it everybody's loads of this block have landed and nobody reads the block
+// before any more, whose stage the loads of block + STAGES - 1 then fill.  Chunk c (16
+// bytes) of row r lies at chunk c ^ ((r / 4) % 4) (rows of 64 bytes) or c ^ (r % 8) (128), so
+// that the 16 rows that lanes read at one chunk fall on all banks.  Rows of 64 bytes ask
+// memory for half a cache line at a time, and the vector cache fetches the whole line for each
+// half (measured: the loads alone then take twice as long).
+// The tile's column pieces of 16 (per stream) are dealt to the WGN wavefronts of a row of
+// wavefronts; where they do not divide, the first ones take one more, and the wavefronts are
+// numbered so that the two that share a SIMD have one of each kind.
+template <int BM, int BN, int WGM, int WGN, int STAGES, int KB, int EPI>
+__global__ __launch_bounds__(WGM * WGN * 64)
+void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int tiles_n, const int dies_m) {
+    constexpr int NW = WGM * WGN;
+    constexpr int NS = TileStreams<EPI>::n;
+    constexpr int WTM = BM / WGM;
+    constexpr int FM = WTM / 16;
+    constexpr int PIECES = BN / NS / 16;           // column pieces of a stream in the tile
+    constexpr int BASE = PIECES / WGN, EXTRA = PIECES % WGN;
+    constexpr int FNS = BASE + (EXTRA ? 1 : 0);    // the most a wavefront holds per stream
+    constexpr int ROW_BYTES = KB * 2, CPR = ROW_BYTES / 16, RPL = 1024 / ROW_BYTES;   // chunks a row, rows a load
+    constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+    constexpr int GROUPS = (BM + BN) / RPL;        // loads of 1 KB a block of k
+    constexpr int GPW = (GROUPS + NW - 1) / NW;
+    static_assert(BN % (16 * NS) == 0 && WTM % 16 == 0 && (BM + BN) % 16 == 0 && STAGES >= 2 && BASE >= 1 &&
+                  (KB == 32 || KB == 64), "tile shape");
+    static_assert(GPW * STAGES < 64, "more loads in flight than the counter holds");
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int wm = wave / WGN, wn = (wave + wave / 4) % WGN;
+    const int pieces = BASE + (wn < EXTRA ? 1 : 0), piece0 = wn * BASE + min(wn, EXTRA);
+    const int M = p.M, N = p.N, K = p.K;
+
+    // (the dies' rectangles: as in gemm_tiles_kernel)
+    const int dies_n = 8 / dies_m;
+    const int die = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int di = die / dies_n, dj = die % dies_n;
+    const int r0 = di * tiles_m / dies_m, rows = (di + 1) * tiles_m / dies_m - r0;
+    const int c0 = dj * tiles_n / dies_n, cols = (dj + 1) * tiles_n / dies_n - c0;
+    if (local >= rows * cols) return;
+    const int tile_n = c0 + local / rows;
+    const int m0 = (r0 + local % rows) * BM;
+    const int n0 = tile_n * (BN / NS);
+
+    // ---- what this lane asks memory for: group g, rows RPL*g .. of the stage
+    const char* src[GPW];
 #pragma unroll
-        for (int tm = 0; tm < FM; ++tm)
-#pragma unroll
-            for (int j = 0; j < FNS; ++j) {
-                const int m = min(m0 + wm * WTM + tm * 16 + r16, M - 1);
-                const int n = min(n0 + wn * (WTN / NS) + j * 16 + 4 * q, N - 4);
-                old_[EPI == T_RESIDUAL ? tm : 0][EPI == T_RESIDUAL ? j : 0] =
-                    *reinterpret_cast<const floatx4_t*>(static_cast<const float*>(p.out) + static_cast<size_t>(m) * p.ldo + n);
-            }
+    for (int i = 0; i < GPW; ++i) {
+        const int g = min(wave + i * NW, GROUPS - 1);
+        const int row = RPL * g + lane / CPR;
+        const int chunk = (lane % CPR) ^ (KB == 32 ? (row >> 2) & 3 : row & 7);
+        if (row < BM) {
+            const int m = min(m0 + row, M - 1);
+            src[i] = reinterpret_cast<const char*>(p.a + static_cast<size_t>(m) * p.lda) + chunk * 16;
+        } else {
+            const int b = row - BM;
+            const int s = b / (BN / NS), j = b % (BN / NS);
+            const int n = min(n0 + j, N - 1);
+            src[i] = reinterpret_cast<const char*>(p.w + (static_cast<size_t>(s) * p.stream_rows + n) * p.ldw) + chunk * 16;
+        }
     }
-    float sq[FM];
+    auto issue = [&](int stage, int kb) {
+        char* const base = lds + stage * STAGE_BYTES;
 #pragma unroll
-    for (int tm = 0; tm < FM; ++tm) sq[tm] = 0.f;
+        for (int i = 0; i < GPW; ++i)
+            __builtin_amdgcn_global_load_lds(GPTR(src[i] + static_cast<size_t>(kb) * ROW_BYTES),
+                                             LPTR(base + min(wave + i * NW, GROUPS - 1) * 1024), 16, 0, 0);
+    };
+
+    const int r16 = lane & 15, q = lane >> 4;
+    int lane_off[KB / 32];                        // per step of 32 values of k
 #pragma unroll
-    for (int tm = 0; tm < FM; ++tm) {
-        const int m = m0 + wm * WTM + tm * 16 + r16;
+    for (int ks = 0; ks < KB / 32; ++ks)
+        lane_off[ks] = r16 * ROW_BYTES + (((ks * 4 + q) ^ (KB == 32 ? (r16 >> 2) & 3 : r16 & 7)) * 16);
+
+    floatx4_t acc[NS * FNS][FM];
 #pragma unroll
-        for (int j = 0; j < FNS; ++j) {
-            const int n = n0 + wn * (WTN / NS) + j * 16 + 4 * q;
-            if (m >= M || n >= N) continue;       // N % 4 == 0: a lane's four columns are inside together
-            float v[NS][4];
+    for (int tn = 0; tn < NS * FNS; ++tn)
+#pragma unroll
+        for (int tm = 0; tm < FM; ++tm) acc[tn][tm] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    float scale[FM];                              // (asked for ahead of the first blocks)
+    tile_row_scales<FM>(p, m0 + wm * WTM + r16, q, scale);
+
+    const int nkb = K / KB;                       // K % 64 == 0 (checked by the host)
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+        if (s < nkb) issue(s, s);
+
+    int stage = 0;
+    for (int kb = 0; kb < nkb; ++kb) {
+        // this wavefront's loads of block kb have landed when at most the later blocks' are out
+        if (kb + STAGES - 2 < nkb) wait_loads<GPW * (STAGES - 2)>(); else wait_loads<0>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        int refill = stage - 1;
+        if (refill < 0) refill = STAGES - 1;
+        if (kb + STAGES - 1 < nkb) issue(refill, kb + STAGES - 1);
+#pragma unroll
+        for (int ks = 0; ks < KB / 32; ++ks) {
+            const char* const sa = lds + stage * STAGE_BYTES + (wm * WTM) * ROW_BYTES + lane_off[ks];
+            const char* const sw = lds + stage * STAGE_BYTES + (BM + piece0 * 16) * ROW_BYTES + lane_off[ks];
+            bf16x8_t a[FM];
+#pragma unroll
+            for (int tm = 0; tm < FM; ++tm) a[tm] = *reinterpret_cast<const bf16x8_t*>(sa + tm * 16 * ROW_BYTES);
 #pragma unroll
             for (int s = 0; s < NS; ++s)
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    v[s][i] = acc[s * FNS + j][tm][i] * scale[tm] +
-                              (p.bias ? p.bias[static_cast<size_t>(s) * p.stream_rows + n + i] : 0.f);
-            if (EPI == T_RESIDUAL) {
-                float* const h = static_cast<float*>(p.out) + static_cast<size_t>(m) * p.ldo + n;
-                floatx4_t old = old_[EPI == T_RESIDUAL ? tm : 0][EPI == T_RESIDUAL ? j : 0];
-                // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
+                for (int j = 0; j < FNS; ++j) {
+                    if (j >= BASE && wn >= EXTRA) continue;          // (the whole wavefront)
+                    const bf16x8_t w = *reinterpret_cast<const bf16x8_t*>(sw + (s * (BN / NS) + j * 16) * ROW_BYTES);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    old[i] += round_bf16(v[0][i]);
-                    sq[tm] += old[i] * old[i];
+                    for (int tm = 0; tm < FM; ++tm)
+                        acc[s * FNS + j][tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, a[tm], acc[s * FNS + j][tm], 0, 0, 0);
                 }
-                *reinterpret_cast<floatx4_t*>(h) = old;
-                if (p.out_bf16)     // (the conversion rounds to nearest even, as from_float<bf16>)
-                    *reinterpret_cast<bf16x4_t*>(p.out_bf16 + static_cast<size_t>(m) * p.ld_bf16 + n) =
-                        bf16x4_t{static_cast<__bf16>(old[0]), static_cast<__bf16>(old[1]),
-                                 static_cast<__bf16>(old[2]), static_cast<__bf16>(old[3])};
-            } else {
-                float o[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if (EPI == T_SWIGLU) {
-                        const float g = round_bf16(v[0][i]), u = round_bf16(v[NS - 1][i]);
-                        o[i] = (g / (1.0f + expf(-g))) * u;
-                    } else {
-                        o[i] = v[0][i];
-                    }
-                }
-                *reinterpret_cast<bf16x4_t*>(static_cast<bf16*>(p.out) + static_cast<size_t>(m) * p.ldo + n) =
-                    bf16x4_t{static_cast<__bf16>(o[0]), static_cast<__bf16>(o[1]),
-                             static_cast<__bf16>(o[2]), static_cast<__bf16>(o[3])};
-            }
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (++stage == STAGES) stage = 0;
     }
-
-    if (EPI == T_RESIDUAL && p.stats_out) {
-        // a row's squares: over the lane's columns (above), the four lanes that share the
-        // row, then the wavefronts that share it, always in the same order
-        float* const red = reinterpret_cast<float*>(lds);
-        __syncthreads();                          // the stages are no longer read
-#pragma unroll
-        for (int tm = 0; tm < FM; ++tm) {
-            float s = sq[tm];
-            s += __shfl_xor(s, 16, 64);
-            s += __shfl_xor(s, 32, 64);
-            if (q == 0) red[wn * BM + wm * WTM + tm * 16 + r16] = s;
-        }
-        __syncthreads();
-        for (int r = threadIdx.x; r < BM; r += NW * 64) {
-            float s = 0.f;
-#pragma unroll
-            for (int w = 0; w < WGN; ++w) s += red[w * BM + r];
-            if (m0 + r < M) p.stats_out[static_cast<size_t>(m0 + r) * p.stats_ld_out + tile_n] = s;
-        }
-    }
+    // (rows leave through LDS where the stages have room for the whole tile's output)
+    constexpr bool ROWS_FIT = NW * WTM * (FNS * 32 + 16) <= STAGES * STAGE_BYTES;
+    tile_epilogue<BM, WGM, WGN, FNS, EPI, ROWS_FIT>(p, acc, scale, m0, n0 + piece0 * 16, pieces, tile_n, wm, wn, lane, lds);
 }
 
 // ---- the shape of the work for given sizes
@@ -300,22 +498,31 @@ static int g_force_shape = -1, g_force_dies_m = 0;
 extern "C" void celeg_gemm_tiles_force(int shape) { g_force_shape = shape; }
 extern "C" void celeg_gemm_tiles_force_dies(int dies_m) { g_force_dies_m = dies_m; }
 
+// id, rows, weight rows, wavefronts along rows and along weight rows, stages, values of k a block of
+// the wide kernel (0: the kernel with tiles up to 256x128)
 #define TILE_SHAPES(X) \
-    X(0, 128, 128, 2, 2, 3) \
-    X(1, 256, 128, 2, 2, 3) \
-    X(2, 128, 64, 2, 2, 3)  \
-    X(3, 64, 128, 2, 2, 3)  \
-    X(4, 128, 128, 2, 2, 2) \
-    X(5, 256, 128, 4, 2, 3) \
-    X(6, 128, 128, 2, 2, 4) \
-    X(7, 64, 64, 2, 2, 4)   \
-    X(8, 64, 64, 2, 2, 2)   \
-    X(9, 128, 64, 2, 2, 2)  \
-    X(10, 128, 128, 4, 2, 2)
+    X(0, 128, 128, 2, 2, 3, 0) \
+    X(1, 256, 128, 2, 2, 3, 0) \
+    X(2, 128, 64, 2, 2, 3, 0)  \
+    X(3, 64, 128, 2, 2, 3, 0)  \
+    X(4, 128, 128, 2, 2, 2, 0) \
+    X(5, 256, 128, 4, 2, 3, 0) \
+    X(6, 128, 128, 2, 2, 4, 0) \
+    X(7, 64, 64, 2, 2, 4, 0)   \
+    X(8, 64, 64, 2, 2, 2, 0)   \
+    X(9, 128, 64, 2, 2, 2, 0)  \
+    X(10, 128, 128, 4, 2, 2, 0) \
+    X(11, 256, 288, 4, 2, 4, 32) \
+    X(12, 256, 288, 4, 2, 2, 64) \
+    X(13, 256, 160, 4, 2, 3, 64) \
+    X(14, 256, 192, 4, 2, 2, 64) \
+    X(15, 128, 192, 2, 2, 3, 64) \
+    X(16, 128, 128, 2, 2, 4, 64) \
+    X(17, 256, 128, 4, 2, 3, 64)
 
-static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 128};
-static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128};
-#define N_TILE_SHAPES 11
+static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 128, 256, 256, 256, 256, 128, 128, 256};
+static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128, 288, 288, 160, 192, 192, 128, 128};
+#define N_TILE_SHAPES 18
 
 static TileShape tile_shape(int M, int N, int streams) {
     int id = 0;
@@ -325,20 +532,29 @@ static TileShape tile_shape(int M, int N, int streams) {
         // tiles of 128x128 with two workgroups of 8 wavefronts a compute unit where they give
         // every unit one and a half or more (8 wavefronts: a tenth faster than 4), else
         // smaller tiles, which fill the chip.
+        // Tiles of 256x288, one workgroup a compute unit, where a round of them (2.2 times as long
+        // as a round of 128x128 tiles, measured at 1,024 and 2,048 values of k) covers the product
+        // in less time: 2,048 rows by 9,216 weight rows are exactly one round, 44 us with the
+        // SwiGLU against 63 us.
         const long long wide = static_cast<long long>((M + 127) / 128) * ((static_cast<long long>(N) * streams + 127) / 128);
-        id = wide >= 384 ? 10 : (wide >= 192 ? 3 : 7);
+        const long long tiles288 = static_cast<long long>((M + 255) / 256) * ((static_cast<long long>(N) * streams + 287) / 288);
+        const long long rounds288 = (tiles288 + 255) / 256, rounds128 = (wide + 511) / 512;
+        id = wide >= 384 ? (rounds288 * 22 < rounds128 * 10 ? 12 : 10) : (wide >= 192 ? 3 : 7);
     }
     return TileShape{id, k_shape_bm[id], k_shape_bn[id]};
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, int EPI>
+template <int BM, int BN, int WGM, int WGN, int STAGES, int KB, int EPI>
 static int launch_tiles(const TileParams& p, hipStream_t stream) {
     constexpr int NS = TileStreams<EPI>::n;
-    constexpr size_t lds = static_cast<size_t>(STAGES) * (BM + BN) * 128;
+    constexpr size_t lds = static_cast<size_t>(STAGES) * (BM + BN) * (KB == 32 ? 64 : 128);
+    void (*kernel)(const TileParams, const int, const int, const int);
+    if constexpr (KB != 0) kernel = &gemm_tiles_wide_kernel<BM, BN, WGM, WGN, STAGES, KB, EPI>;
+    else kernel = &gemm_tiles_kernel<BM, BN, WGM, WGN, STAGES, EPI>;
     static_assert(lds <= 160 * 1024, "more LDS than a compute unit has");
     static bool raised = false;              // once per instantiation: more LDS than the default limit
     if (lds > 48 * 1024 && !raised) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiles_kernel<BM, BN, WGM, WGN, STAGES, EPI>),
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         if (err != hipSuccess) return static_cast<int>(err);
         raised = true;
@@ -358,15 +574,15 @@ static int launch_tiles(const TileParams& p, hipStream_t stream) {
     const int dies_n = 8 / dies_m;
     const int per_die = ((tiles_m + dies_m - 1) / dies_m) * ((tiles_n + dies_n - 1) / dies_n);
     dim3 grid(per_die * 8), block(WGM * WGN * 64);
-    hipLaunchKernelGGL((gemm_tiles_kernel<BM, BN, WGM, WGN, STAGES, EPI>), grid, block, lds, stream, p, tiles_m, tiles_n, dies_m);
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, p, tiles_m, tiles_n, dies_m);
     return CELEG_LAUNCH_RESULT();
 }
 
 template <int EPI>
 static int launch_epilogue(const TileParams& p, hipStream_t stream) {
     const TileShape s = tile_shape(p.M, p.N, TileStreams<EPI>::n);
-#define TILE_CASE(ID, BM, BN, WGM, WGN, STAGES) \
-    if (s.id == ID) return launch_tiles<BM, BN, WGM, WGN, STAGES, EPI>(p, stream);
+#define TILE_CASE(ID, BM, BN, WGM, WGN, STAGES, KB) \
+    if (s.id == ID) return launch_tiles<BM, BN, WGM, WGN, STAGES, KB, EPI>(p, stream);
     TILE_SHAPES(TILE_CASE)
 #undef TILE_CASE
     return static_cast<int>(hipErrorInvalidValue);

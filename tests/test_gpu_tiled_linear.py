@@ -6,7 +6,7 @@ import torch
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 BF = torch.bfloat16
-N_SHAPES = 11
+N_SHAPES = 18
 
 
 @pytest.fixture(scope="module")
@@ -35,7 +35,7 @@ def bf16_round(x):
     return x.to(torch.float32).to(BF).double()
 
 
-SIZES = [(300, 200, 128), (65, 36, 64), (512, 256, 192), (129, 1024, 1024)]
+SIZES = [(300, 200, 128), (65, 36, 64), (512, 256, 192), (129, 1024, 1024), (520, 648, 192)]
 
 
 @pytest.mark.parametrize("shape", list(range(N_SHAPES)) + [-1])
