@@ -44,11 +44,10 @@ enum { T_STORE = 0, T_RESIDUAL = 2, T_SWIGLU = 3 };   // the numbers of the few-
 
 __device__ __forceinline__ float round_bf16(float x) { return to_float(from_float<bf16>(x)); }
 
-#ifdef CELEG_TILES_FAST_SILU
+// g / (1 + e^-g) with the hardware's exponential and reciprocal (an ulp each, in 32-bit; the
+// result is rounded to bfloat16): the exact division and exponential cost the SwiGLU product
+// of 2,048 rows 3 us.
 __device__ __forceinline__ float tile_silu(float g) { return g * __frcp_rn(1.0f + __expf(-g)); }
-#else
-__device__ __forceinline__ float tile_silu(float g) { return g / (1.0f + expf(-g)); }
-#endif
 
 template <int N>
 __device__ __forceinline__ void wait_loads() {
@@ -357,21 +356,75 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
     tile_epilogue<BM, WGM, WGN, FN / NS, EPI, false>(p, acc, scale, m0, n0 + wn * (WTN / NS), FN / NS, tile_n, wm, wn, lane, lds);
 }
 
+// SwiGLU of a wide tile whose wavefronts each hold columns of one stream only: gate and up
+// (rounded to bfloat16, as where they are tensors of their own) meet in LDS, [stream][row], and
+// leave as whole rows, 16 bytes a lane.
+template <int BM, int BN, int WGM, int WGN>
+__device__ __forceinline__ void wide_swiglu_epilogue(
+    const TileParams& p, floatx4_t (&acc)[BN / 16 / WGN][BM / WGM / 16], const float (&scale)[BM / WGM / 16],
+    const int m0, const int n0, const int wm, const int wn, const int lane, char* const lds) {
+    constexpr int NW = WGM * WGN, WTM = BM / WGM, FM = WTM / 16, FN = BN / 16 / WGN;
+    constexpr int PS = BN / 32;                   // column pieces of a stream
+    constexpr int OC = BN / 2, PITCH = OC * 2 + 16;
+    const int M = p.M, N = p.N;
+    const int r16 = lane & 15, q = lane >> 4;
+    const int s = (wn * FN) / PS, j0 = (wn * FN) % PS;
+    __syncthreads();                              // the stages are no longer read
+    char* const mine = lds + static_cast<size_t>(s) * BM * PITCH;
+    floatx4_t bias[FN];                           // of the lane's columns
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const int n = n0 + (j0 + j) * 16 + 4 * q;
+        bias[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        if (p.bias && n < N) bias[j] = *reinterpret_cast<const floatx4_t*>(p.bias + static_cast<size_t>(s) * p.stream_rows + n);
+    }
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const floatx4_t v = acc[j][tm] * scale[tm] + bias[j];
+            *reinterpret_cast<bf16x4_t*>(mine + (wm * WTM + tm * 16 + r16) * PITCH + ((j0 + j) * 16 + 4 * q) * 2) =
+                bf16x4_t{static_cast<__bf16>(v[0]), static_cast<__bf16>(v[1]), static_cast<__bf16>(v[2]), static_cast<__bf16>(v[3])};
+        }
+    __syncthreads();
+    constexpr int CPR = OC / 8;                   // chunks of 8 columns a row
+    const bool wide_stores = (p.ldo % 8) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
+    for (int idx = threadIdx.x; idx < BM * CPR; idx += NW * 64) {
+        const int row = idx / CPR, ch = idx % CPR;
+        const int m = m0 + row, n = n0 + ch * 8;
+        if (m >= M || n >= N) continue;
+        const bf16x8_t g = *reinterpret_cast<const bf16x8_t*>(lds + row * PITCH + ch * 16);
+        const bf16x8_t u = *reinterpret_cast<const bf16x8_t*>(lds + static_cast<size_t>(BM) * PITCH + row * PITCH + ch * 16);
+        bf16x8_t o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = static_cast<__bf16>(tile_silu(static_cast<float>(g[i])) * static_cast<float>(u[i]));
+        bf16* const to = static_cast<bf16*>(p.out) + static_cast<size_t>(m) * p.ldo + n;
+        if (wide_stores && n + 8 <= N) {
+            *reinterpret_cast<bf16x8_t*>(to) = o;
+        } else {
+            *reinterpret_cast<bf16x4_t*>(to) = bf16x4_t{o[0], o[1], o[2], o[3]};
+            if (n + 8 <= N) *reinterpret_cast<bf16x4_t*>(to + 4) = bf16x4_t{o[4], o[5], o[6], o[7]};
+        }
+    }
+}
+
 // The same product with wide tiles (256 rows x up to 288 weight rows a workgroup), for the
 // products whose operands would otherwise cross from the L2 caches to the compute units many
 // times over.  A wavefront's tile is too large to hold a block's operands in registers beside
-// its sums, so the weights' operands stream from LDS a piece at a time while the matrix
-// instructions of the piece before run; blocks are KB = 32 or 64 values of k (rows of 64 or
-// 128 bytes in LDS, a load instruction fills 16 or 8 rows), STAGES of them, with one barrier a
-// block: behind it everybody's loads of this block have landed and nobody reads the block
-// before any more, whose stage the loads of block + STAGES - 1 then fill.  Chunk c (16
-// bytes) of row r lies at chunk c ^ ((r / 4) % 4) (rows of 64 bytes) or c ^ (r % 8) (128), so
-// that the 16 rows that lanes read at one chunk fall on all banks.  Rows of 64 bytes ask
-// memory for half a cache line at a time, and the vector cache fetches the whole line for each
-// half (measured: the loads alone then take twice as long).
-// The tile's column pieces of 16 (per stream) are dealt to the WGN wavefronts of a row of
-// wavefronts; where they do not divide, the first ones take one more, and the wavefronts are
-// numbered so that the two that share a SIMD have one of each kind.
+// its sums, so the weights' operands stream from LDS a piece (16 weight rows) at a time, two
+// pieces ahead of the matrix instructions that use them, and the rows' operands of the next
+// step of 32 values of k come in between; the order is pinned (sched_barrier), because left
+// alone the compiler reads two pieces into the same registers, waits for them, multiplies, and
+// reads again.  Blocks are KB = 32 or 64 values of k (rows of 64 or 128 bytes in LDS, a load
+// instruction fills 16 or 8 rows), STAGES of them, with one barrier a block: behind it
+// everybody's loads of this block have landed and nobody reads the block before any more,
+// whose stage the loads of block + STAGES - 1 then fill.  Chunk c (16 bytes) of row r lies at
+// chunk c ^ ((r / 4) % 4) (rows of 64 bytes) or c ^ (r % 8) (128), so that the 16 rows that
+// lanes read at one chunk fall on all banks.  Rows of 64 bytes ask memory for half a cache
+// line at a time, and the vector cache fetches the whole line for each half (measured: the
+// loads alone then take a third longer).
+// The tile's BN / 16 column pieces (gate pieces, then up pieces) are dealt evenly to the WGN
+// wavefronts of a row of wavefronts, each within one stream.
 template <int BM, int BN, int WGM, int WGN, int STAGES, int KB, int EPI>
 __global__ __launch_bounds__(WGM * WGN * 64)
 void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int tiles_n, const int dies_m) {
@@ -379,21 +432,20 @@ void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int til
     constexpr int NS = TileStreams<EPI>::n;
     constexpr int WTM = BM / WGM;
     constexpr int FM = WTM / 16;
-    constexpr int PIECES = BN / NS / 16;           // column pieces of a stream in the tile
-    constexpr int BASE = PIECES / WGN, EXTRA = PIECES % WGN;
-    constexpr int FNS = BASE + (EXTRA ? 1 : 0);    // the most a wavefront holds per stream
+    constexpr int FN = BN / 16 / WGN;              // column pieces of a wavefront
+    constexpr int PS = BN / 16 / NS;               // column pieces of a stream in the tile
+    constexpr int KS = KB / 32;                    // steps of 32 values of k a block
     constexpr int ROW_BYTES = KB * 2, CPR = ROW_BYTES / 16, RPL = 1024 / ROW_BYTES;   // chunks a row, rows a load
     constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
     constexpr int GROUPS = (BM + BN) / RPL;        // loads of 1 KB a block of k
     constexpr int GPW = (GROUPS + NW - 1) / NW;
-    static_assert(BN % (16 * NS) == 0 && WTM % 16 == 0 && (BM + BN) % 16 == 0 && STAGES >= 2 && BASE >= 1 &&
-                  (KB == 32 || KB == 64), "tile shape");
+    static_assert(BN % (16 * WGN) == 0 && BN % (16 * NS) == 0 && PS % FN == 0 && WTM % 16 == 0 &&
+                  (BM + BN) % 16 == 0 && STAGES >= 2 && FN >= 2 && (KB == 32 || KB == 64), "tile shape");
     static_assert(GPW * STAGES < 64, "more loads in flight than the counter holds");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int wm = wave / WGN, wn = (wave + wave / 4) % WGN;
-    const int pieces = BASE + (wn < EXTRA ? 1 : 0), piece0 = wn * BASE + min(wn, EXTRA);
+    const int wm = wave / WGN, wn = wave % WGN;
     const int M = p.M, N = p.N, K = p.K;
 
     // (the dies' rectangles: as in gemm_tiles_kernel)
@@ -433,14 +485,14 @@ void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int til
     };
 
     const int r16 = lane & 15, q = lane >> 4;
-    int lane_off[KB / 32];                        // per step of 32 values of k
+    int lane_off[KS];                             // per step of 32 values of k
 #pragma unroll
-    for (int ks = 0; ks < KB / 32; ++ks)
+    for (int ks = 0; ks < KS; ++ks)
         lane_off[ks] = r16 * ROW_BYTES + (((ks * 4 + q) ^ (KB == 32 ? (r16 >> 2) & 3 : r16 & 7)) * 16);
 
-    floatx4_t acc[NS * FNS][FM];
+    floatx4_t acc[FN][FM];
 #pragma unroll
-    for (int tn = 0; tn < NS * FNS; ++tn)
+    for (int tn = 0; tn < FN; ++tn)
 #pragma unroll
         for (int tm = 0; tm < FM; ++tm) acc[tn][tm] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
@@ -461,30 +513,40 @@ void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int til
         int refill = stage - 1;
         if (refill < 0) refill = STAGES - 1;
         if (kb + STAGES - 1 < nkb) issue(refill, kb + STAGES - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const char* const sa = lds + stage * STAGE_BYTES + (wm * WTM) * ROW_BYTES;
+        const char* const sw = lds + stage * STAGE_BYTES + (BM + wn * FN * 16) * ROW_BYTES;
+        // piece t = ks * FN + j of the block: step ks of 32 values of k, column piece j
+        auto weights = [&](int t) {
+            return *reinterpret_cast<const bf16x8_t*>(sw + (t % FN) * 16 * ROW_BYTES + lane_off[t / FN]);
+        };
+        bf16x8_t a[2][FM], w[3];
 #pragma unroll
-        for (int ks = 0; ks < KB / 32; ++ks) {
-            const char* const sa = lds + stage * STAGE_BYTES + (wm * WTM) * ROW_BYTES + lane_off[ks];
-            const char* const sw = lds + stage * STAGE_BYTES + (BM + piece0 * 16) * ROW_BYTES + lane_off[ks];
-            bf16x8_t a[FM];
+        for (int tm = 0; tm < FM; ++tm) a[0][tm] = *reinterpret_cast<const bf16x8_t*>(sa + tm * 16 * ROW_BYTES + lane_off[0]);
+        w[0] = weights(0);
+        w[1] = weights(1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int tm = 0; tm < FM; ++tm) a[tm] = *reinterpret_cast<const bf16x8_t*>(sa + tm * 16 * ROW_BYTES);
+        for (int t = 0; t < KS * FN; ++t) {
+            const int ks = t / FN, j = t % FN;
+            acc[j][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t % 3], a[ks & 1][0], acc[j][0], 0, 0, 0);
+            if (t + 2 < KS * FN) w[(t + 2) % 3] = weights(t + 2);
+            if (ks + 1 < KS && j < FM)            // the rows' operands of the next step, one a piece
+                a[(ks + 1) & 1][j] = *reinterpret_cast<const bf16x8_t*>(sa + j * 16 * ROW_BYTES + lane_off[ks + 1 < KS ? ks + 1 : 0]);
 #pragma unroll
-            for (int s = 0; s < NS; ++s)
-#pragma unroll
-                for (int j = 0; j < FNS; ++j) {
-                    if (j >= BASE && wn >= EXTRA) continue;          // (the whole wavefront)
-                    const bf16x8_t w = *reinterpret_cast<const bf16x8_t*>(sw + (s * (BN / NS) + j * 16) * ROW_BYTES);
-#pragma unroll
-                    for (int tm = 0; tm < FM; ++tm)
-                        acc[s * FNS + j][tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, a[tm], acc[s * FNS + j][tm], 0, 0, 0);
-                }
+            for (int tm = 1; tm < FM; ++tm)
+                acc[j][tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t % 3], a[ks & 1][tm], acc[j][tm], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (++stage == STAGES) stage = 0;
     }
-    // (rows leave through LDS where the stages have room for the whole tile's output)
-    constexpr bool ROWS_FIT = NW * WTM * (FNS * 32 + 16) <= STAGES * STAGE_BYTES;
-    tile_epilogue<BM, WGM, WGN, FNS, EPI, ROWS_FIT>(p, acc, scale, m0, n0 + piece0 * 16, pieces, tile_n, wm, wn, lane, lds);
+    if constexpr (EPI == T_SWIGLU) {
+        wide_swiglu_epilogue<BM, BN, WGM, WGN>(p, acc, scale, m0, n0, wm, wn, lane, lds);
+    } else {
+        // (rows leave through LDS where the stages have room for the whole tile's output)
+        constexpr bool ROWS_FIT = NW * WTM * (FN * 32 + 16) <= STAGES * STAGE_BYTES;
+        tile_epilogue<BM, WGM, WGN, FN, EPI, ROWS_FIT>(p, acc, scale, m0, n0 + wn * FN * 16, FN, tile_n, wm, wn, lane, lds);
+    }
 }
 
 // ---- the shape of the work for given sizes
@@ -512,17 +574,15 @@ extern "C" void celeg_gemm_tiles_force_dies(int dies_m) { g_force_dies_m = dies_
     X(8, 64, 64, 2, 2, 2, 0)   \
     X(9, 128, 64, 2, 2, 2, 0)  \
     X(10, 128, 128, 4, 2, 2, 0) \
-    X(11, 256, 288, 4, 2, 4, 32) \
-    X(12, 256, 288, 4, 2, 2, 64) \
-    X(13, 256, 160, 4, 2, 3, 64) \
-    X(14, 256, 192, 4, 2, 2, 64) \
-    X(15, 128, 192, 2, 2, 3, 64) \
-    X(16, 128, 128, 2, 2, 4, 64) \
-    X(17, 256, 128, 4, 2, 3, 64)
+    X(11, 256, 288, 4, 2, 2, 64) \
+    X(12, 256, 160, 4, 2, 3, 64) \
+    X(13, 256, 192, 4, 2, 2, 64) \
+    X(14, 128, 192, 2, 2, 3, 64) \
+    X(15, 256, 128, 4, 2, 3, 64)
 
-static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 128, 256, 256, 256, 256, 128, 128, 256};
-static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128, 288, 288, 160, 192, 192, 128, 128};
-#define N_TILE_SHAPES 18
+static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 128, 256, 256, 256, 128, 256};
+static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128, 288, 160, 192, 192, 128};
+#define N_TILE_SHAPES 16
 
 static TileShape tile_shape(int M, int N, int streams) {
     int id = 0;
@@ -539,7 +599,7 @@ static TileShape tile_shape(int M, int N, int streams) {
         const long long wide = static_cast<long long>((M + 127) / 128) * ((static_cast<long long>(N) * streams + 127) / 128);
         const long long tiles288 = static_cast<long long>((M + 255) / 256) * ((static_cast<long long>(N) * streams + 287) / 288);
         const long long rounds288 = (tiles288 + 255) / 256, rounds128 = (wide + 511) / 512;
-        id = wide >= 384 ? (rounds288 * 22 < rounds128 * 10 ? 12 : 10) : (wide >= 192 ? 3 : 7);
+        id = wide >= 384 ? (rounds288 * 22 < rounds128 * 10 ? 11 : 10) : (wide >= 192 ? 3 : 7);
     }
     return TileShape{id, k_shape_bm[id], k_shape_bn[id]};
 }
@@ -547,7 +607,10 @@ static TileShape tile_shape(int M, int N, int streams) {
 template <int BM, int BN, int WGM, int WGN, int STAGES, int KB, int EPI>
 static int launch_tiles(const TileParams& p, hipStream_t stream) {
     constexpr int NS = TileStreams<EPI>::n;
-    constexpr size_t lds = static_cast<size_t>(STAGES) * (BM + BN) * (KB == 32 ? 64 : 128);
+    constexpr size_t stages_lds = static_cast<size_t>(STAGES) * (BM + BN) * (KB == 32 ? 64 : 128);
+    // (the wide kernel's SwiGLU lays the tile's gate and up values out in LDS)
+    constexpr size_t swiglu_lds = KB != 0 && EPI == T_SWIGLU ? static_cast<size_t>(2) * BM * (BN + 16) : 0;
+    constexpr size_t lds = stages_lds > swiglu_lds ? stages_lds : swiglu_lds;
     void (*kernel)(const TileParams, const int, const int, const int);
     if constexpr (KB != 0) kernel = &gemm_tiles_wide_kernel<BM, BN, WGM, WGN, STAGES, KB, EPI>;
     else kernel = &gemm_tiles_kernel<BM, BN, WGM, WGN, STAGES, EPI>;
@@ -607,6 +670,7 @@ extern "C" int celeg_gemm_tiles(const TileParams* params, int epi, hipStream_t s
         p.lda < p.K || p.ldw < p.K || p.ldo < p.N)
         return static_cast<int>(hipErrorInvalidValue);
     if (p.stats && p.n_stat_blocks < 1) return static_cast<int>(hipErrorInvalidValue);
+    if (reinterpret_cast<uintptr_t>(p.bias) & 15) return static_cast<int>(hipErrorInvalidValue);
     if (p.out_bf16 && ((p.ld_bf16 % 4) || p.ld_bf16 < p.N)) return static_cast<int>(hipErrorInvalidValue);
     if (epi == T_SWIGLU && p.stream_rows < p.N) return static_cast<int>(hipErrorInvalidValue);
     switch (epi) {

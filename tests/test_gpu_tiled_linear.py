@@ -6,7 +6,7 @@ import torch
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 BF = torch.bfloat16
-N_SHAPES = 18
+N_SHAPES = 16
 
 
 @pytest.fixture(scope="module")
