@@ -130,7 +130,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
-    ap.add_argument("--gemm-backend", choices=["library", "tiles"], default="library",
+    ap.add_argument("--gemm-backend", choices=["auto", "library", "tiles"], default="auto",
                     help="products of steps of more than 64 rows (the prefill)")
     ap.add_argument("--batch", type=int, default=BATCH,
                     help="for profiling with --phase decode: another batch size than the headline's 8")
@@ -241,7 +241,8 @@ def main() -> int:
                    "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "ff": ff, "vocab_size": cfg["vocab_size"], "conv_L_cache": cfg["conv_L_cache"],
-                   "rope_theta": cfg["rope_theta"], "tied_embeddings": True, "page_tokens": 16},
+                   "rope_theta": cfg["rope_theta"], "tied_embeddings": True, "page_tokens": 16,
+                   "prefill_products": lm.native.info["gemm_backend"]},
         "prefill": None if prefill is None else {
             "value": round(prefill["tokens_per_second"], 1), "tokens": PROMPT_TOKENS,
             "ms": round(prefill["ms"], 4),

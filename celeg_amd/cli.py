@@ -72,9 +72,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--dump-hidden", default="", metavar="DIR",
                     help="write the 32-bit residual stream after every layer of every step to "
                          "DIR/step<k>_layer<i>.f32 (the reference's CELEG_DEBUG_HIDDEN_DIR)")
-    ap.add_argument("--gemm-backend", default="library", choices=["library", "tiles"],
-                    help="bfloat16 steps of more than 64 rows: the library's matrix products, or this "
-                         "package's tiled products with norm, SwiGLU and residual sum folded in")
+    ap.add_argument("--gemm-backend", default="auto", choices=["auto", "library", "tiles"],
+                    help="bfloat16 steps of more than 64 rows: the library's matrix products, this "
+                         "package's tiled products with norm, SwiGLU and residual sum folded in, or "
+                         "(auto) the one that was measured faster at the model's width")
     ap.add_argument("--device", default="cuda:0")
     return ap
 

@@ -356,6 +356,39 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
     tile_epilogue<BM, WGM, WGN, FN / NS, EPI, false>(p, acc, scale, m0, n0 + wn * (WTN / NS), FN / NS, tile_n, wm, wn, lane, lds);
 }
 
+// A read of 16 bytes a lane from LDS at `address` + index * STRIDE, and the waits that go with
+// such reads, written as instructions: the compiler does not see the read, so every use of
+// `to` has to come behind a wait that names it (the wait takes the registers in and out, which
+// keeps the uses behind it), with no branch and no indexing by a variable in between (either
+// would let the compiler copy the registers before the data is there).  `left`: how many later
+// reads may still be out.
+template <int STRIDE>
+__device__ __forceinline__ void lds_read(bf16x8_t& to, const unsigned address, const int index) {
+    switch (index) {
+#define CELEG_LDS_READ_CASE(I) \
+    case I: asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(to) : "v"(address), "n"(I * STRIDE)); break;
+        CELEG_LDS_READ_CASE(0) CELEG_LDS_READ_CASE(1) CELEG_LDS_READ_CASE(2) CELEG_LDS_READ_CASE(3)
+        CELEG_LDS_READ_CASE(4) CELEG_LDS_READ_CASE(5) CELEG_LDS_READ_CASE(6) CELEG_LDS_READ_CASE(7)
+        CELEG_LDS_READ_CASE(8) CELEG_LDS_READ_CASE(9) CELEG_LDS_READ_CASE(10) CELEG_LDS_READ_CASE(11)
+#undef CELEG_LDS_READ_CASE
+        default: __builtin_trap();
+    }
+}
+__device__ __forceinline__ void lds_wait(const int left, bf16x8_t& x) {
+    switch (left) {
+        case 0: asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(x)); break;
+        case 1: asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(x)); break;
+        case 2: asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(x)); break;
+        default: asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(x)); break;
+    }
+}
+template <int FM>
+__device__ __forceinline__ void lds_wait_rows(const int left, bf16x8_t& x, bf16x8_t (&rows)[FM]) {
+    lds_wait(left, x);
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) asm volatile("" : "+v"(rows[tm]));     // (behind the wait above: volatile statements keep their order)
+}
+
 // SwiGLU of a wide tile whose wavefronts each hold columns of one stream only: gate and up
 // (rounded to bfloat16, as where they are tensors of their own) meet in LDS, [stream][row], and
 // leave as whole rows, 16 bytes a lane.
@@ -413,9 +446,9 @@ __device__ __forceinline__ void wide_swiglu_epilogue(
 // times over.  A wavefront's tile is too large to hold a block's operands in registers beside
 // its sums, so the weights' operands stream from LDS a piece (16 weight rows) at a time, two
 // pieces ahead of the matrix instructions that use them, and the rows' operands of the next
-// step of 32 values of k come in between; the order is pinned (sched_barrier), because left
-// alone the compiler reads two pieces into the same registers, waits for them, multiplies, and
-// reads again.  Blocks are KB = 32 or 64 values of k (rows of 64 or 128 bytes in LDS, a load
+// step of 32 values of k come in between; the order is pinned (sched_barrier) and the reads and
+// their waits are written as instructions, because left alone the compiler reads two pieces
+// into the same registers, waits for them, multiplies, and reads again.  Blocks are KB = 32 or 64 values of k (rows of 64 or 128 bytes in LDS, a load
 // instruction fills 16 or 8 rows), STAGES of them, with one barrier a block: behind it
 // everybody's loads of this block have landed and nobody reads the block before any more,
 // whose stage the loads of block + STAGES - 1 then fill.  Chunk c (16 bytes) of row r lies at
@@ -440,7 +473,7 @@ void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int til
     constexpr int GROUPS = (BM + BN) / RPL;        // loads of 1 KB a block of k
     constexpr int GPW = (GROUPS + NW - 1) / NW;
     static_assert(BN % (16 * WGN) == 0 && BN % (16 * NS) == 0 && PS % FN == 0 && WTM % 16 == 0 &&
-                  (BM + BN) % 16 == 0 && STAGES >= 2 && FN >= 2 && (KB == 32 || KB == 64), "tile shape");
+                  (BM + BN) % 16 == 0 && STAGES >= 2 && FN >= 2 && FN <= 12 && FM <= 12 && (KB == 32 || KB == 64), "tile shape");
     static_assert(GPW * STAGES < 64, "more loads in flight than the counter holds");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -504,6 +537,7 @@ void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int til
     for (int s = 0; s < STAGES - 1; ++s)
         if (s < nkb) issue(s, s);
 
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(LPTR(lds)));
     int stage = 0;
     for (int kb = 0; kb < nkb; ++kb) {
         // this wavefront's loads of block kb have landed when at most the later blocks' are out
@@ -514,25 +548,38 @@ void gemm_tiles_wide_kernel(const TileParams p, const int tiles_m, const int til
         if (refill < 0) refill = STAGES - 1;
         if (kb + STAGES - 1 < nkb) issue(refill, kb + STAGES - 1);
         __builtin_amdgcn_sched_barrier(0);
-        const char* const sa = lds + stage * STAGE_BYTES + (wm * WTM) * ROW_BYTES;
-        const char* const sw = lds + stage * STAGE_BYTES + (BM + wn * FN * 16) * ROW_BYTES;
-        // piece t = ks * FN + j of the block: step ks of 32 values of k, column piece j
-        auto weights = [&](int t) {
-            return *reinterpret_cast<const bf16x8_t*>(sw + (t % FN) * 16 * ROW_BYTES + lane_off[t / FN]);
-        };
+        // LDS addresses of this lane's operands per step of 32 values of k; pieces are 16 rows apart
+        unsigned at_a[KS], at_w[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            at_a[ks] = lds_base + stage * STAGE_BYTES + (wm * WTM) * ROW_BYTES + lane_off[ks];
+            at_w[ks] = lds_base + stage * STAGE_BYTES + (BM + wn * FN * 16) * ROW_BYTES + lane_off[ks];
+        }
+        // The reads and the waits for them are written out (the compiler, left to count, waits for
+        // every read in flight before each second piece).  Piece t = ks * FN + j of the block: step
+        // ks, column piece j.  In the order of issue: the rows' operands of step 0, weights 0 and 1;
+        // then behind the first matrix instruction of piece t weights t + 2 and, for the first FM
+        // pieces of a step, one of the rows' operands of the next step.  LDS answers in order, so
+        // piece t may start when no more reads are out than were issued behind weights t.
         bf16x8_t a[2][FM], w[3];
 #pragma unroll
-        for (int tm = 0; tm < FM; ++tm) a[0][tm] = *reinterpret_cast<const bf16x8_t*>(sa + tm * 16 * ROW_BYTES + lane_off[0]);
-        w[0] = weights(0);
-        w[1] = weights(1);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int tm = 0; tm < FM; ++tm) lds_read<16 * ROW_BYTES>(a[0][tm], at_a[0], tm);
+        lds_read<16 * ROW_BYTES>(w[0], at_w[0], 0);
+        lds_read<16 * ROW_BYTES>(w[1], at_w[1 / FN < KS ? 1 / FN : 0], 1 % FN);
 #pragma unroll
         for (int t = 0; t < KS * FN; ++t) {
             const int ks = t / FN, j = t % FN;
+            // reads issued behind weights t: weights t + 1 (if any) and the rows' operands that went
+            // with weights t and t + 1 (issued in pieces t - 2 and t - 1)
+            constexpr auto rows_with = [](int piece) {      // does piece `piece` issue one of the next step's rows' operands?
+                return piece >= 0 && piece / FN + 1 < KS && piece % FN < FM ? 1 : 0;
+            };
+            const int behind = (t + 1 < KS * FN ? 1 : 0) + (t >= 2 ? rows_with(t - 2) : 0) + (t >= 1 ? rows_with(t - 1) : 0);
+            if (j == 0) lds_wait_rows(behind, w[t % 3], a[ks & 1]);
+            else lds_wait(behind, w[t % 3]);
             acc[j][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t % 3], a[ks & 1][0], acc[j][0], 0, 0, 0);
-            if (t + 2 < KS * FN) w[(t + 2) % 3] = weights(t + 2);
-            if (ks + 1 < KS && j < FM)            // the rows' operands of the next step, one a piece
-                a[(ks + 1) & 1][j] = *reinterpret_cast<const bf16x8_t*>(sa + j * 16 * ROW_BYTES + lane_off[ks + 1 < KS ? ks + 1 : 0]);
+            if (t + 2 < KS * FN) lds_read<16 * ROW_BYTES>(w[(t + 2) % 3], at_w[(t + 2) / FN < KS ? (t + 2) / FN : 0], (t + 2) % FN);
+            if (rows_with(t)) lds_read<16 * ROW_BYTES>(a[(ks + 1) & 1][j < FM ? j : 0], at_a[ks + 1 < KS ? ks + 1 : 0], j);
 #pragma unroll
             for (int tm = 1; tm < FM; ++tm)
                 acc[j][tm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[t % 3], a[ks & 1][tm], acc[j][tm], 0, 0, 0);

@@ -69,7 +69,7 @@ LoadOptions load_options(const celeg_engine_options& o) {
     l.max_requests = o.max_active_requests;
     l.max_context = o.context > 0 ? o.context : -1;
     l.max_batched_tokens = o.max_batched_tokens;
-    l.gemm_backend = o.gemm_backend == CELEG_GEMM_TILES ? "tiles" : "library";
+    l.gemm_backend = o.gemm_backend == CELEG_GEMM_TILES ? "tiles" : o.gemm_backend == CELEG_GEMM_LIBRARY ? "library" : "auto";
     l.use_graphs = o.use_graphs != 0;
     return l;
 }
@@ -134,7 +134,7 @@ void celeg_engine_options_init(celeg_engine_options* o, size_t struct_size) {
     full.logical_kv_pages = 0;
     full.scheduler_policy = CELEG_POLICY_MAX_UTILIZATION;
     full.context = 0;
-    full.gemm_backend = CELEG_GEMM_LIBRARY;
+    full.gemm_backend = CELEG_GEMM_AUTO;
     full.use_graphs = 1;
     full.run_ahead = 1;
     full.portion_granule = 1;
@@ -326,7 +326,8 @@ const char* celeg_model_describe(celeg_model* model) {
                 .set("max_batched_tokens", lm.runner->max_batched_tokens).set("graph_safe", lm.model->graph_safe())
                 .set("dtype", dtype_name(lm.rt->dtype)).set("weights", lm.model->weight_count())
                 .set("kv_bytes_per_token", lm.cache->layout.kv_bytes_per_token(dtype_size(lm.rt->dtype)))
-                .set("eos_token_ids", Json::array_of(lm.model->spec.eos_token_ids));
+                .set("eos_token_ids", Json::array_of(lm.model->spec.eos_token_ids))
+                .set("gemm_backend", lm.rt->use_tiled_products ? "tiles" : "library");
             out = j.dump();
         }) != CELEG_OK)
         return nullptr;

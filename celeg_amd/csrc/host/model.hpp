@@ -127,7 +127,7 @@ struct LoadOptions {
     int max_requests = 8;
     int max_context = -1;           // -1: the model's own maximum; may not exceed it
     int max_batched_tokens = 2048;
-    std::string gemm_backend = "library";   // how bfloat16 steps of more than 64 rows multiply: "library" or "tiles"
+    std::string gemm_backend = "auto";      // how bfloat16 steps of more than 64 rows multiply: "library", "tiles" or "auto"
     bool use_graphs = true;
 };
 

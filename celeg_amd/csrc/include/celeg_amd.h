@@ -43,7 +43,10 @@ typedef enum celeg_request_status {
 } celeg_request_status;
 
 enum { CELEG_POLICY_MAX_UTILIZATION = 0, CELEG_POLICY_GUARANTEED_NO_EVICT = 1 };
-enum { CELEG_GEMM_LIBRARY = 0, CELEG_GEMM_TILES = 1 };
+/* how bfloat16 steps of more than 64 rows multiply: the library's products, this library's tiled
+ * products with norm, SwiGLU and residual sum folded in, or (the default) whichever was measured
+ * faster at the model's width */
+enum { CELEG_GEMM_LIBRARY = 0, CELEG_GEMM_TILES = 1, CELEG_GEMM_AUTO = 2 };
 
 /* temperature 0.1, top_k 50, top_p 1, repetition_penalty 1.05, seed 1
  * (include/celeg/model/runtime_types.hpp:98-108); greedy when temperature <= 0 or top_k == 1 */
@@ -128,7 +131,8 @@ celeg_model* celeg_engine_model(celeg_engine* engine);
 celeg_status celeg_model_create(const char* model_dir, const celeg_engine_options* options, celeg_model** out);
 void celeg_model_destroy(celeg_model* model);
 /* JSON: {"config": typed configuration, "spec": model description, "cache_layout": .., "vocab_size", "max_context",
- *        "page_tokens", "max_requests", "graph_safe", "logit_width"} */
+ *        "page_tokens", "max_requests", "graph_safe", "logit_width", "gemm_backend": "library" | "tiles" (what
+ *        CELEG_GEMM_AUTO became)} */
 const char* celeg_model_describe(celeg_model* model);
 celeg_status celeg_model_open_slot(celeg_model* model, int32_t* slot);      /* -1: every slot is taken */
 celeg_status celeg_model_close_slot(celeg_model* model, int32_t slot);

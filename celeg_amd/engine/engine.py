@@ -180,12 +180,13 @@ class LoadedModel:
 
 def load_model(model_dir: str, *, dtype="bfloat16", device="cuda:0", page_tokens: int = 16,
                n_pages: Optional[int] = None, max_requests: int = 8, max_context: Optional[int] = None,
-               max_batched_tokens: int = 2048, gemm_backend: str = "library", use_graphs: bool = True) -> LoadedModel:
+               max_batched_tokens: int = 2048, gemm_backend: str = "auto", use_graphs: bool = True) -> LoadedModel:
     """``n_pages``: pages of the cache pool (per group); by default enough for ``max_requests``
     requests of ``max_context`` tokens.  ``max_context`` defaults to the model's own maximum and
     may not exceed it.  ``gemm_backend``: how bfloat16 steps of more than 64 rows multiply:
-    "library" (hipBLASLt, with separate norm and activation kernels) or "tiles" (the library's own
-    tiled products with the norm, SwiGLU and the residual sum folded in, where the sizes allow)."""
+    "library" (hipBLASLt, with separate norm and activation kernels), "tiles" (the library's own
+    tiled products with the norm, SwiGLU and the residual sum folded in, where the sizes allow) or
+    "auto" (the one that was measured faster at the model's width; ``describe()`` says which)."""
     options = native.engine_options(dtype=parse_dtype(dtype), device=native.device_index(device),
                                     max_active_requests=max_requests, max_batched_tokens=max_batched_tokens,
                                     page_tokens=page_tokens, n_pages=n_pages, context=max_context,
@@ -206,7 +207,7 @@ class Engine:
                     n_pages: Optional[int] = None, max_active_requests: int = 8,
                     max_batched_tokens: int = 2048, prefill_chunk_tokens: int = 1024,
                     context: Optional[int] = None, policy: str = "max_utilization",
-                    gemm_backend: str = "library", portion_granule: int = 1, use_graphs: bool = True,
+                    gemm_backend: str = "auto", portion_granule: int = 1, use_graphs: bool = True,
                     run_ahead: bool = True) -> "Engine":
         # (Steps of 2,048 tokens and portions of 1,024: on an MI355X a step of a few hundred rows
         # leaves most of the chip idle; the reference's 512 / 256 are ``SchedulerOptions``'.)

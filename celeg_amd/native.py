@@ -206,12 +206,12 @@ def registered(what: str) -> List[str]:
 # ------------------------------------------------------------------ options
 def engine_options(*, dtype="bfloat16", device=0, max_active_requests=8, max_batched_tokens=2048,
                    prefill_chunk_tokens=1024, page_tokens=16, n_pages=None, policy="max_utilization",
-                   context=None, gemm_backend="library", use_graphs=True, run_ahead=True,
+                   context=None, gemm_backend="auto", use_graphs=True, run_ahead=True,
                    portion_granule=1) -> EngineOptions:
     if policy not in ("max_utilization", "guaranteed_no_evict"):
         raise NativeArgumentError("policy must be max_utilization or guaranteed_no_evict")
-    if gemm_backend not in ("library", "tiles"):
-        raise NativeArgumentError(f"gemm_backend must be 'library' or 'tiles', not '{gemm_backend}'")
+    if gemm_backend not in ("library", "tiles", "auto"):
+        raise NativeArgumentError(f"gemm_backend must be 'library', 'tiles' or 'auto', not '{gemm_backend}'")
     o = EngineOptions()
     lib().celeg_engine_options_init(ctypes.byref(o), ctypes.sizeof(o))
     o.dtype = str(dtype).replace("torch.", "").encode()
@@ -221,7 +221,7 @@ def engine_options(*, dtype="bfloat16", device=0, max_active_requests=8, max_bat
     o.logical_kv_pages = int(n_pages) if n_pages else 0
     o.scheduler_policy = 1 if policy == "guaranteed_no_evict" else 0
     o.context = int(context) if context else 0
-    o.gemm_backend = 1 if gemm_backend == "tiles" else 0
+    o.gemm_backend = {"library": 0, "tiles": 1, "auto": 2}[gemm_backend]
     o.use_graphs, o.run_ahead, o.portion_granule = int(bool(use_graphs)), int(bool(run_ahead)), int(portion_granule)
     return o
 
