@@ -36,7 +36,7 @@ def plain_logits(folder, name, storage):
     return _plain_cache[key]
 
 
-def run_mode(model_folders, name, dtype, mode, device, subset=None, gemm_backend="library"):
+def run_mode(model_folders, name, dtype, mode, device, subset=None, gemm_backend="auto"):
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders(name, storage, WEIGHT_STD)
@@ -72,9 +72,25 @@ def test_gpu_engine_with_tiled_products_matches_plain(model_folders, mode):
     folded in) instead of the library's: whole prompts of up to 300 tokens, and portions
     beside single tokens."""
     lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles")
-    assert lm.knobs()["use_tiled_products"] == 1
+    assert lm.knobs()["use_tiled_products"] == 1 and lm.native.info["gemm_backend"] == "tiles"
     # and the same configuration through the library's products
-    run_mode(model_folders, "E", "bfloat16", mode, "cuda:0")
+    lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="library")
+    assert lm.knobs()["use_tiled_products"] == 0 and lm.native.info["gemm_backend"] == "library"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_gpu_engine_through_the_library_products_matches_plain(model_folders, name):
+    """The other tests take the products that the width of their models selects (the tiled
+    ones); here every configuration's prompts go through the library's products."""
+    lm = run_mode(model_folders, name, "bfloat16", "whole", "cuda:0", gemm_backend="library")
+    assert lm.native.info["gemm_backend"] == "library"
+
+
+@pytest.mark.gpu
+def test_the_products_of_long_steps_follow_the_width_of_the_model(model_folders):
+    lm = run_mode(model_folders, "A", "bfloat16", "whole", "cuda:0")
+    assert lm.native.info["gemm_backend"] == "tiles"          # a width up to 1,024
 
 
 @pytest.mark.gpu

@@ -393,6 +393,66 @@ def attention_case(ops, dtype, heads, kv_heads, head_dim, lengths, cuts, window=
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(16, 8, 64), (4, 2, 128), (10, 5, 32)])
+def test_norm_rope_store_of_a_long_step_equals_short_steps(ops, dtype, heads, kv_heads, head_dim):
+    """A step of thousands of rows takes four rows a thread (values of four neighbouring rows
+    leave as one store); the same rows in steps of a few hundred take one row a thread.  Three
+    requests whose portions start at positions 0, 5 and 1, so that runs of four rows start on a
+    multiple of four, in the middle of one, and straddle the border between two requests: the
+    queries and both caches must come out the same bit for bit."""
+    from celeg_amd.engine import StepEntry
+    starts, lengths = [0, 5, 1], [2503, 1202, 650]
+    n_layers, layer, page_tokens = 2, 1, 16
+    qw = 1 + randn(head_dim, seed=20, scale=0.1)
+    kw = 1 + randn(head_dim, seed=21, scale=0.1)
+    inv_freq = torch.tensor(plain.rope_inverse_frequencies(10000.0, head_dim), dtype=torch.float64).float().to(DEV)
+    total = sum(lengths)
+    q0 = randn(total, heads * head_dim, seed=1, dtype=dtype)
+    k0 = randn(total, kv_heads * head_dim, seed=2, dtype=dtype)
+    v0 = randn(total, kv_heads * head_dim, seed=3, dtype=dtype)
+    results = []
+    for pieces in (1, 17):                       # the whole step, then steps of at most 260 rows
+        cache = make_cache(kv_heads, head_dim, n_layers, dtype, page_tokens=page_tokens,
+                           n_pages=(total + sum(starts)) // page_tokens + 8, max_context=max(lengths) + 16, slots=4)
+        kv = cache.layer_cache(layer).kv
+        slots = [cache.open() for _ in lengths]
+        for slot, start in zip(slots, starts):   # what lies before the portions is of no interest here
+            if start:
+                assert cache.prepare(slot, 0, start)
+        q_out = torch.empty_like(q0)
+        done = [0] * len(lengths)
+        for piece in range(pieces):
+            entries, rows = [], []
+            row0 = 0
+            for i, n in enumerate(lengths):
+                c = n if pieces == 1 else min((n + pieces - 1) // pieces, n - done[i])
+                if c > 0:
+                    assert cache.prepare(slots[i], starts[i] + done[i], c)
+                    entries.append(StepEntry(slots[i], starts[i] + done[i], [0] * c))
+                    rows.append((row0 + done[i], c))
+                    done[i] += c
+                row0 += n
+            if not entries:
+                continue
+            batch, keep = build_batch(ops, cache, entries)
+            rows = [rows[j] for j in batch.entry_order]
+            index = torch.cat([torch.arange(r, r + c) for r, c in rows]).to(DEV)
+            q, k, v = q0[index].contiguous(), k0[index].contiguous(), v0[index].contiguous()
+            ops.qk_norm_rope_store(q, k, v, qw, kw, 1e-5, inv_freq, head_dim, heads, kv_heads, head_dim, batch, kv)
+            q_out[index] = q
+        torch.cuda.synchronize()
+        # the pools page by page in the order of the requests' tables (the page numbers may differ)
+        table = kv.table.cpu()
+        pages = [int(table[slot, p]) for slot, start, n in zip(slots, starts, lengths)
+                 for p in range((start + n + page_tokens - 1) // page_tokens)]
+        results.append((q_out.clone(), kv.k[pages].clone(), kv.v[pages].clone(), [int(x) for x in starts]))
+    (qa, ka, va, _), (qb, kb, vb, _) = results
+    assert torch.equal(qa, qb)
+    assert torch.equal(ka, kb) and torch.equal(va, vb)
+    assert float(ka.float().abs().max()) > 0 and float(va.float().abs().max()) > 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kv_heads,head_dim", [
     (6, 3, 48), (5, 5, 16), (8, 1, 128), (4, 2, 80), (16, 8, 64), (3, 3, 64), (6, 2, 96),
     (8, 2, 32), (12, 4, 128)])
