@@ -72,7 +72,7 @@ def prefill_flops(cfg, tokens: int, ff: int) -> float:
     return per_token * tokens + attention + 2.0 * H * cfg["vocab_size"]   # head for one row
 
 
-def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1) -> int:
+def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1, gemm_backend: str = "auto") -> int:
     """The whole engine on a serving workload: every request submitted at once, the scheduler
     cuts the prompts into portions beside the decoding requests, sampling is greedy on the
     device.  Prints one JSON line: generated tokens a second over the whole run."""
@@ -94,7 +94,7 @@ def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1) -> int:
                                     n_pages=pages, max_active_requests=load["requests"],
                                     max_batched_tokens=load["budget"],
                                     prefill_chunk_tokens=load["chunk"], portion_granule=granule,
-                                    context=cfg["max_position_embeddings"])
+                                    context=cfg["max_position_embeddings"], gemm_backend=gemm_backend)
     # a short run first: weights re-laid, a graph recorded
     engine.generate(prompts[:2], max_new_tokens=4, generation=GREEDY, eos_token_ids=[])
     before = engine.metrics
@@ -119,7 +119,7 @@ def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1) -> int:
         "steps_replayed_from_graphs": after["graph_replays"] - before["graph_replays"],
         "graphs_recorded": after["captures"] - before["captures"],
         "recording_seconds": round(after["capture_seconds"] - before["capture_seconds"], 3),
-        "dtype": "bf16", "data": "synthetic"}))
+        "prefill_products": engine.loaded.native.info["gemm_backend"], "dtype": "bf16", "data": "synthetic"}))
     return 0
 
 
@@ -156,7 +156,7 @@ def main() -> int:
         return 2
 
     if args.phase == "serve":
-        return serve(args.shape, args.prefill_chunk, args.token_budget, args.portion_granule)
+        return serve(args.shape, args.prefill_chunk, args.token_budget, args.portion_granule, args.gemm_backend)
 
     import torch
     import celeg_amd  # noqa: F401
