@@ -81,6 +81,7 @@ GenerationConfig generation_of(const celeg_generation_options& g) {
     c.top_p = g.top_p;
     c.repetition_penalty = g.repetition_penalty;
     c.seed = g.seed;
+    if (g.forced_prefix && g.n_forced_prefix > 0) c.forced_prefix.assign(g.forced_prefix, g.forced_prefix + g.n_forced_prefix);
     return c;
 }
 

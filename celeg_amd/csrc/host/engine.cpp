@@ -34,6 +34,9 @@ long long Engine::submit(const std::vector<int>& prompt, const RequestOptions& o
     for (int t : prompt)
         if (t < 0 || t >= vocab)
             throw ConfigError("token id " + std::to_string(t) + " out of range [0, " + std::to_string(vocab) + ")");
+    for (int t : options.generation.forced_prefix)
+        if (t < 0 || t >= vocab)
+            throw ConfigError("forced_prefix: token id " + std::to_string(t) + " out of range [0, " + std::to_string(vocab) + ")");
     return scheduler_->submit(prompt, options);
 }
 
@@ -53,7 +56,7 @@ void Engine::sync_slots() {
     for (const auto& b : bound) {
         Request& req = *b.second;
         if (!req.rng) req.rng = std::make_shared<XorShift64Star>(req.options.generation.seed);
-        sampler_->begin(b.first, req.options.generation, req.rng);
+        sampler_->begin(b.first, req.options.generation, req.rng, req.generated.size());
     }
 }
 

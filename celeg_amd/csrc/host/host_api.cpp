@@ -55,6 +55,9 @@ GenerationConfig generation_from(const Json& j) {
     g.top_p = static_cast<float>(j.get_double("top_p", g.top_p));
     g.repetition_penalty = static_cast<float>(j.get_double("repetition_penalty", g.repetition_penalty));
     g.seed = static_cast<uint64_t>(j.get_int("seed", 1));
+    const Json& forced = j["forced_prefix"];
+    if (forced.is_array())
+        for (const Json& t : forced.items()) g.forced_prefix.push_back(static_cast<int>(t.as_int()));
     return g;
 }
 

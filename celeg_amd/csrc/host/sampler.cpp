@@ -12,6 +12,8 @@ void GenerationConfig::validate() const {
     if (!std::isfinite(repetition_penalty) || repetition_penalty < 1.0f)
         throw ConfigError("repetition_penalty must be finite and at least 1");
     if (seed == 0) throw ConfigError("seed must be non-zero");
+    for (int t : forced_prefix)
+        if (t < 0) throw ConfigError("forced_prefix holds a negative token id");
 }
 
 XorShift64Star::XorShift64Star(uint64_t seed) : state(seed) {
@@ -49,9 +51,12 @@ Sampler::~Sampler() {
         if (e) (void)hipEventDestroy(e);
 }
 
-void Sampler::begin(int slot, const GenerationConfig& config, std::shared_ptr<XorShift64Star> rng) {
+void Sampler::begin(int slot, const GenerationConfig& config, std::shared_ptr<XorShift64Star> rng, size_t generated) {
     config.validate();
+    for (int t : config.forced_prefix)
+        if (t >= vocab_) throw ConfigError("forced_prefix: token id " + std::to_string(t) + " out of range [0, " + std::to_string(vocab_) + ")");
     configs_[slot] = config;
+    forced_used_[slot] = std::min(generated, config.forced_prefix.size());
     rng_[slot] = rng ? std::move(rng) : std::make_shared<XorShift64Star>(config.seed);
     if (config.repetition_penalty > 1.0f && !seen_.ptr()) {
         seen_ = DeviceBuffer(static_cast<size_t>(cap_) * vocab_, true);
@@ -63,6 +68,7 @@ void Sampler::begin(int slot, const GenerationConfig& config, std::shared_ptr<Xo
 void Sampler::end(int slot) {
     configs_.erase(slot);
     rng_.erase(slot);
+    forced_used_.erase(slot);
 }
 
 bool Sampler::uses_seen() const {
@@ -95,11 +101,15 @@ void Sampler::launch(const Tensor& logits, const std::vector<int>& slots) {
         f[4 * r] = c.temperature;
         f[4 * r + 1] = c.top_p;
         f[4 * r + 2] = c.repetition_penalty;
-        f[4 * r + 3] = c.greedy() ? 0.0f : rng_[slots[static_cast<size_t>(r)]]->next_unit();
-        iv[3 * r] = c.top_k;
+        size_t& forced_used = forced_used_[slots[static_cast<size_t>(r)]];
+        const bool forced = forced_used < c.forced_prefix.size();
+        f[4 * r + 3] = (c.greedy() || forced) ? 0.0f : rng_[slots[static_cast<size_t>(r)]]->next_unit();
+        // a forced token travels in the place of top_k as -(token + 1): the kernel gives it out
+        // (and marks it as seen, and leaves it for the next step) instead of choosing one
+        iv[3 * r] = forced ? -(c.forced_prefix[forced_used++] + 1) : c.top_k;
         iv[3 * r + 1] = (c.repetition_penalty > 1.0f && seen_.ptr()) ? slots[static_cast<size_t>(r)] : -1;
         iv[3 * r + 2] = slots[static_cast<size_t>(r)];
-        all_greedy = all_greedy && c.greedy();
+        all_greedy = all_greedy && c.greedy() && !forced;
     }
     // greedy rows have nothing that changes from step to step: ship only what differs from what
     // the device holds

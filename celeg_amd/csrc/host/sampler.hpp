@@ -26,6 +26,9 @@ struct GenerationConfig {
     float top_p = 1.0f;
     float repetition_penalty = 1.05f;
     uint64_t seed = 1;
+    // given out as the first generated tokens instead of sampled ones, without a draw from the
+    // generator (include/celeg/model/runtime_types.hpp:93-104; src/backend/cpu/sampler.cpp:31-34)
+    std::vector<int> forced_prefix;
     bool greedy() const { return temperature <= 0.0f || top_k == 1; }
     void validate() const;     // throws ConfigError
 };
@@ -46,8 +49,9 @@ public:
     ~Sampler();
     Sampler(const Sampler&) = delete;
     // Bind a request to `slot`.  rng continues an existing generator (a request that was
-    // preempted and comes back); null: a fresh one is seeded.
-    void begin(int slot, const GenerationConfig& config, std::shared_ptr<XorShift64Star> rng = nullptr);
+    // preempted and comes back); null: a fresh one is seeded.  `generated`: how many tokens the
+    // request has been given already (as many of its forced prefix are used up).
+    void begin(int slot, const GenerationConfig& config, std::shared_ptr<XorShift64Star> rng = nullptr, size_t generated = 0);
     void end(int slot);
     bool uses_seen() const;
     // every token a step feeds (prompt portions and decoded tokens) counts as seen by its request
@@ -69,6 +73,7 @@ private:
     int vocab_, cap_;
     std::map<int, GenerationConfig> configs_;
     std::map<int, std::shared_ptr<XorShift64Star>> rng_;
+    std::map<int, size_t> forced_used_;      // of the slot's forced prefix
     DeviceBuffer seen_;            // [max_requests, vocab] bytes, made on need
     PinnedBuffer params_[2];       // 4 floats a row, then 3 ints a row
     DeviceBuffer params_dev_, last_tokens_;

@@ -57,6 +57,12 @@ typedef struct celeg_generation_options {
     float top_p;
     float repetition_penalty;
     uint64_t seed;
+    /* tokens given out as the request's first generated tokens instead of sampled ones (they are
+     * polled, counted and checked against the end tokens like sampled ones; the request's generator
+     * is not advanced for them): ForcedTokenPrefix, include/celeg/model/runtime_types.hpp:93-104,
+     * src/backend/cpu/sampler.cpp:31-34.  Copied at submission; null or 0: none. */
+    const int32_t* forced_prefix;
+    int32_t n_forced_prefix;
 } celeg_generation_options;
 
 /* max_active_requests 8, page_tokens 16, logical_kv_pages 0 (= enough for every request at the

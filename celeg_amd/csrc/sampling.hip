@@ -413,8 +413,8 @@ __device__ __forceinline__ int choose_among(float* cand_score, int* cand_id, int
     return __shfl(chosen_at < 64 ? id0 : id1, chosen_at & 63, CELEG_WAVE);
 }
 
-// fparams[row] = {temperature, top_p, penalty, u}; iparams[row] = {top_k, seen_row or -1,
-// slot or -1}; the token also goes to last_tokens[slot] (if given and slot >= 0), where the
+// fparams[row] = {temperature, top_p, penalty, u}; iparams[row] = {top_k (or -(token + 1): that
+// token is given out, nothing is chosen), seen_row or -1, slot or -1}; the token also goes to last_tokens[slot] (if given and slot >= 0), where the
 // next step can take it from without the host in between, and is marked as seen in the row's
 // seen_row (if any): the step that feeds it back need not mark it.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
@@ -443,6 +443,17 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const uint8_t* seen = (seen_all && seen_row >= 0)
                               ? seen_all + static_cast<size_t>(seen_row) * seen_stride : nullptr;
 
+    if (top_k < 0) {
+        // ---- a token that the caller forces: -(token + 1) in the place of top_k
+        // (src/backend/cuda/model/sampler.cu:44-54: the forced token is copied in and marked as seen)
+        if (tid == 0) {
+            const int token = min(-(top_k + 1), vocab - 1);
+            out_tokens[r] = token;
+            if (last_tokens && slot >= 0) last_tokens[slot] = token;
+            if (seen_all && seen_row >= 0) seen_all[static_cast<size_t>(seen_row) * seen_stride + token] = 1;
+        }
+        return;
+    }
     if (temperature <= 0.0f || top_k == 1) {
         // ---- penalised argmax, lowest index wins ties
         float best = -INFINITY;

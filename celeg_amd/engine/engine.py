@@ -230,7 +230,8 @@ class Engine:
         try:
             return self.native.submit(prompt, max_new_tokens=o.max_new_tokens, eos_token_ids=o.eos_token_ids,
                                       priority=o.priority, temperature=g.temperature, top_k=g.top_k, top_p=g.top_p,
-                                      repetition_penalty=g.repetition_penalty, seed=g.seed)
+                                      repetition_penalty=g.repetition_penalty, seed=g.seed,
+                                      forced_prefix=g.forced_prefix)
         except native.NativeArgumentError as err:
             raise ValueError(str(err)) from None
 
@@ -307,7 +308,7 @@ class Scheduler:
         return self._host._call("submit", [int(t) for t in prompt],
                                 {"max_new_tokens": o.max_new_tokens, "priority": o.priority,
                                  "eos_token_ids": None if o.eos_token_ids is None else list(o.eos_token_ids),
-                                 "generation": vars(o.generation)})
+                                 "generation": dict(vars(o.generation), forced_prefix=list(o.generation.forced_prefix))})
 
     def cancel(self, request_id: int) -> None:
         self._host._call("cancel", request_id)

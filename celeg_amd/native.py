@@ -33,7 +33,8 @@ class NativeArgumentError(ValueError):
 
 class GenerationOptions(ctypes.Structure):
     _fields_ = [("struct_size", c_size_t), ("temperature", c_float), ("top_k", c_int32), ("top_p", c_float),
-                ("repetition_penalty", c_float), ("seed", ctypes.c_uint64)]
+                ("repetition_penalty", c_float), ("seed", ctypes.c_uint64),
+                ("forced_prefix", P(c_int32)), ("n_forced_prefix", c_int32)]
 
 
 class EngineOptions(ctypes.Structure):
@@ -342,7 +343,7 @@ class NativeEngine:
             pass
 
     def submit(self, tokens: Sequence[int], *, max_new_tokens=128, eos_token_ids=None, priority=0,
-               temperature=0.1, top_k=50, top_p=1.0, repetition_penalty=1.05, seed=1) -> int:
+               temperature=0.1, top_k=50, top_p=1.0, repetition_penalty=1.05, seed=1, forced_prefix=()) -> int:
         o = RequestOptionsStruct()
         lib().celeg_request_options_init(ctypes.byref(o), ctypes.sizeof(o))
         o.max_new_tokens, o.priority = int(max_new_tokens), int(priority)
@@ -357,6 +358,11 @@ class NativeEngine:
         if not 0 <= int(seed) < (1 << 64):
             raise NativeArgumentError("seed must be non-zero")
         g.seed = int(seed)
+        forced = None
+        if forced_prefix:
+            forced = _ints([int(t) for t in forced_prefix])        # (kept alive until the call has copied it)
+            g.forced_prefix = ctypes.cast(forced, P(c_int32))
+            g.n_forced_prefix = len(forced_prefix)
         request_id = c_int64()
         toks = [int(t) for t in tokens]
         check(lib().celeg_engine_submit(self.handle, _ints(toks), len(toks), ctypes.byref(o), ctypes.byref(request_id)))

@@ -7,6 +7,7 @@ from __future__ import annotations
 
 import math
 from dataclasses import dataclass
+from typing import Tuple
 
 MAX_TOP_K = 128
 _MASK64 = (1 << 64) - 1
@@ -19,6 +20,10 @@ class GenerationConfig:
     top_p: float = 1.0
     repetition_penalty: float = 1.05
     seed: int = 1
+    # given out as the request's first generated tokens instead of sampled ones; the generator is
+    # not advanced for them (ForcedTokenPrefix, include/celeg/model/runtime_types.hpp:93-104;
+    # src/backend/cpu/sampler.cpp:31-34)
+    forced_prefix: Tuple[int, ...] = ()
 
     @property
     def greedy(self) -> bool:
@@ -36,6 +41,8 @@ class GenerationConfig:
             raise ValueError("repetition_penalty must be finite and at least 1")
         if self.seed == 0 or not 0 < self.seed <= _MASK64:
             raise ValueError("seed must be non-zero")
+        if any(int(t) < 0 for t in self.forced_prefix):
+            raise ValueError("forced_prefix holds a negative token id")
 
 
 GREEDY = GenerationConfig(temperature=0.0, top_k=1, top_p=1.0, repetition_penalty=1.0, seed=1)
