@@ -160,6 +160,24 @@ const char* celeg_last_error(void) { return g_error.c_str(); }
 void celeg_set_last_error_(const char* message) { g_error = message ? message : ""; }   // for host_api.cpp
 const char* celeg_version(void) { return "celeg_amd 0.2 (gfx950)"; }
 
+const char* celeg_backend_capabilities(void) {
+    std::string out = "HIP backend for gfx950 (one GPU; bfloat16 and a true float32 path; paged keys and values, "
+                      "state slots, portions beside decoding requests in one step; no CPU path): ";
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        out += "no device is visible";
+    } else {
+        out += std::to_string(count) + (count == 1 ? " device" : " devices") + " visible";
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, 0) == hipSuccess)
+            out += std::string(", device 0 is ") + prop.name + " (" + prop.gcnArchName + ")";
+        else
+            (void)hipGetLastError();
+    }
+    return text(out);
+}
+
 // ---------------------------------------------------------------------------- the engine
 celeg_status celeg_engine_create(const char* model_dir, const celeg_engine_options* options, celeg_engine** out) {
     if (!model_dir || !out) {

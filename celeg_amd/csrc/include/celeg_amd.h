@@ -103,6 +103,9 @@ void celeg_request_options_init(celeg_request_options* options, size_t struct_si
 
 const char* celeg_last_error(void);
 const char* celeg_version(void);
+/* what this build can run and on what, in a sentence (the reference's celeg_backend_capabilities,
+ * include/celeg/api.h:150, answers likewise for a backend's name; here there is one backend) */
+const char* celeg_backend_capabilities(void);
 
 /* ---- the engine ---- */
 celeg_status celeg_engine_create(const char* model_dir, const celeg_engine_options* options, celeg_engine** out);

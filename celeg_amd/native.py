@@ -113,6 +113,7 @@ def lib() -> ctypes.CDLL:
 
     sig("celeg_last_error", c_char_p)
     sig("celeg_version", c_char_p)
+    sig("celeg_backend_capabilities", c_char_p)
     sig("celeg_generation_options_init", None, P(GenerationOptions), c_size_t)
     sig("celeg_engine_options_init", None, P(EngineOptions), c_size_t)
     sig("celeg_request_options_init", None, P(RequestOptionsStruct), c_size_t)
@@ -187,6 +188,11 @@ def _ints(values: Sequence[int]):
 
 
 # ------------------------------------------------------------------ descriptions
+def backend_capabilities() -> str:
+    """What this build can run and on what, in a sentence."""
+    return _text(lib().celeg_backend_capabilities())
+
+
 def describe_folder(model_dir: str) -> Dict[str, Any]:
     return json.loads(_text(lib().celeg_describe_folder(model_dir.encode())))
 

@@ -40,6 +40,8 @@ static int describe(const char* dir) {
     celeg_request_options_init(&ro, sizeof ro);
     celeg_generation_options_init(&go, sizeof go);
     printf("version %s\n", celeg_version());
+    printf("capabilities %s\n", celeg_backend_capabilities());
+    printf("forced_prefix_default %d %d\n", go.forced_prefix == NULL, go.n_forced_prefix);
     printf("engine_defaults %s %d %d %d %d %d\n", eo.dtype, eo.max_active_requests, eo.max_batched_tokens,
            eo.prefill_chunk_tokens, eo.page_tokens, eo.scheduler_policy);
     printf("request_defaults %d %d %d\n", ro.max_new_tokens, ro.n_eos_token_ids, ro.priority);

@@ -38,6 +38,8 @@ def test_defaults_and_descriptions_from_c(program, model_folders):
     assert lines["engine_defaults"] == "bfloat16 8 2048 1024 16 0"
     assert lines["request_defaults"] == "128 -1 0"
     assert lines["generation_defaults"] == "0.10 50 1.00 1.05 1"
+    assert lines["forced_prefix_default"] == "1 0"
+    assert "gfx950" in lines["capabilities"] and ("visible" in lines["capabilities"])
     assert "\nchecked\n" in proc.stdout
     assert "config.json" in lines["missing:"]
     assert "must not be null" in lines["refused:"]
