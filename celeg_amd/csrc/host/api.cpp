@@ -81,7 +81,9 @@ GenerationConfig generation_of(const celeg_generation_options& g) {
     c.top_p = g.top_p;
     c.repetition_penalty = g.repetition_penalty;
     c.seed = g.seed;
-    if (g.forced_prefix && g.n_forced_prefix > 0) c.forced_prefix.assign(g.forced_prefix, g.forced_prefix + g.n_forced_prefix);
+    if (g.n_forced_prefix < 0 || (g.n_forced_prefix > 0 && !g.forced_prefix))
+        throw ConfigError("forced_prefix: a count without tokens (or a negative count)");
+    if (g.n_forced_prefix > 0) c.forced_prefix.assign(g.forced_prefix, g.forced_prefix + g.n_forced_prefix);
     return c;
 }
 
@@ -213,7 +215,9 @@ celeg_status celeg_engine_submit(celeg_engine* engine, const int32_t* tokens, in
         RequestOptions ro;
         ro.max_new_tokens = o.max_new_tokens;
         ro.priority = o.priority;
-        if (o.n_eos_token_ids >= 0) ro.eos_token_ids = std::vector<int>(o.eos_token_ids, o.eos_token_ids + o.n_eos_token_ids);
+        if (o.n_eos_token_ids > 0 && !o.eos_token_ids) throw ConfigError("eos_token_ids: a count without tokens");
+        if (o.n_eos_token_ids == 0) ro.eos_token_ids = std::vector<int>();
+        if (o.n_eos_token_ids > 0) ro.eos_token_ids = std::vector<int>(o.eos_token_ids, o.eos_token_ids + o.n_eos_token_ids);
         ro.generation = generation_of(o.generation);
         const long long id = engine->engine->submit(std::vector<int>(tokens, tokens + n_tokens), ro);
         if (request_id) *request_id = id;
@@ -276,6 +280,12 @@ celeg_status celeg_engine_status(celeg_engine* engine, int64_t request_id, int32
 
 celeg_status celeg_engine_cancel(celeg_engine* engine, int64_t request_id) {
     return with_request(engine, [&] { engine->engine->cancel(request_id); });
+}
+
+celeg_status celeg_engine_release(celeg_engine* engine, int64_t request_id) {
+    return with_request(engine, [&] {
+        if (!engine->engine->release(request_id)) throw ConfigError("request " + std::to_string(request_id) + " has not ended: cancel it first");
+    });
 }
 
 const char* celeg_engine_request_error(celeg_engine* engine, int64_t request_id) {
@@ -412,6 +422,9 @@ celeg_status celeg_model_step(celeg_model* model, int32_t n_entries, const int32
             wanted += static_cast<size_t>(n_want[i]);
         }
         LoadedModel& lm = *model->lm;
+        // (checked before the step runs: a step that has run has advanced its requests)
+        if (wanted && !logits) throw StepError("step: logits are wanted and there is no buffer for them");
+        if (wanted * static_cast<size_t>(lm.model->logit_width()) > capacity) throw StepError("step: the logits buffer is too small");
         const Tensor out = lm.runner->step(entries);
         const size_t width = static_cast<size_t>(out.shape[1]);
         if (wanted * width > capacity) throw StepError("step: the logits buffer is too small");

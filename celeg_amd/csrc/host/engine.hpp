@@ -35,6 +35,7 @@ public:
 
     long long submit(const std::vector<int>& prompt, const RequestOptions& options);
     void cancel(long long id) { scheduler_->cancel(id); }
+    bool release(long long id) { return scheduler_->release_request(id); }
     RequestStatus status(long long id) { return scheduler_->request(id).status; }
     // drains the tokens generated since the last poll (src/backend/cuda/runtime/request_lifecycle.cpp:57-73)
     RequestStatus poll(long long id, std::vector<int>& tokens, std::string& error);

@@ -12,6 +12,7 @@
 //   "cache"     {"layout": cache layout JSON, "page_tokens", "n_pages": n or [n per group], "max_requests", "max_context"}
 //   "scheduler" {"cache": handle, "options": {..SchedulerOptions..}, "max_context", "default_eos": [..]}
 //   "batch"     {"capacity", "n_groups"}
+#include <algorithm>
 #include <map>
 #include <mutex>
 
@@ -145,6 +146,15 @@ Json call(HostObject& o, const std::string& method, const Json& a) {
             return Json(s.submit(ints(a[0]), ro));
         }
         if (method == "cancel") { s.cancel(a[0].as_int()); return Json(true); }
+        if (method == "release") {
+            const long long id = a[0].as_int();
+            const bool ended = is_done(s.request(id).status);
+            if (ended)      // the plan kept for accept / fail must not name a record that goes
+                o.last_plan.erase(std::remove_if(o.last_plan.begin(), o.last_plan.end(),
+                                                 [&](const PlannedEntry& e) { return e.request->id == id; }),
+                                  o.last_plan.end());
+            return Json(s.release_request(id));
+        }
         if (method == "has_work") return Json(s.has_work());
         if (method == "plan") {
             o.last_plan = s.plan();

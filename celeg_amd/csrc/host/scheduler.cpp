@@ -66,6 +66,18 @@ void Scheduler::cancel(long long request_id) {
     if (!is_done(req.status)) req.cancel_requested = true;
 }
 
+bool Scheduler::release_request(long long request_id) {
+    Request& req = request(request_id);
+    if (!is_done(req.status)) return false;
+    // (a request that has ended is in no list any more; a slot event of this very step may
+    // still name it)
+    new_slots_.erase(std::remove_if(new_slots_.begin(), new_slots_.end(),
+                                    [&](const std::pair<int, Request*>& b) { return b.second == &req; }),
+                     new_slots_.end());
+    requests_.erase(request_id);
+    return true;
+}
+
 // ---------------------------------------------------------------------------- planning
 Request* Scheduler::best_queued() const {
     Request* best = nullptr;

@@ -101,6 +101,10 @@ public:
     Scheduler(CacheManager& cache, SchedulerOptions options, int max_context, std::vector<int> default_eos);
     long long submit(const std::vector<int>& prompt, const RequestOptions& options);
     void cancel(long long request_id);
+    // Forgets a request that has ended (finished, cancelled or failed): its record, tokens that
+    // were not polled and its metrics go.  False, and nothing happens, while it is queued or
+    // running (the reference's release, src/backend/cuda/runtime/request_lifecycle.cpp:47-55).
+    bool release_request(long long request_id);
     bool has_work() const { return !queue_.empty() || !active_.empty(); }
     // decide this step's entries; pages for them are taken here
     std::vector<PlannedEntry> plan();

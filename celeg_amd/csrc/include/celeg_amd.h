@@ -124,6 +124,9 @@ celeg_status celeg_engine_poll(celeg_engine* engine, int64_t request_id, int32_t
                                int32_t* n_tokens, int32_t* status);
 celeg_status celeg_engine_status(celeg_engine* engine, int64_t request_id, int32_t* status);
 celeg_status celeg_engine_cancel(celeg_engine* engine, int64_t request_id);
+/* forgets a request that has ended (its id is unknown afterwards); a request that is queued or running
+ * is refused with CELEG_INVALID_ARGUMENT.  An engine keeps the record of every request until this call. */
+celeg_status celeg_engine_release(celeg_engine* engine, int64_t request_id);
 /* the message of a Failed request ("" otherwise) */
 const char* celeg_engine_request_error(celeg_engine* engine, int64_t request_id);
 const char* celeg_engine_last_error(celeg_engine* engine);

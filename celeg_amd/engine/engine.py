@@ -238,6 +238,14 @@ class Engine:
     def cancel(self, request_id: int) -> None:
         self.native.cancel(request_id)
 
+    def release(self, request_id: int) -> None:
+        """Forgets a request that has ended; the engine keeps every request's record until then.
+        ValueError while it is queued or running, KeyError-like ValueError for an unknown id."""
+        try:
+            self.native.release(request_id)
+        except native.NativeArgumentError as err:
+            raise ValueError(str(err)) from None
+
     def status(self, request_id: int) -> RequestStatus:
         return RequestStatus(self.native.status(request_id))
 
@@ -283,10 +291,13 @@ class Engine:
         out = []
         for rid in ids:
             status, tokens, error = self.poll(rid)
+            out.append((status, tokens, error))
+        for rid in ids:
+            self.release(rid)
+        for rid, (status, tokens, error) in zip(ids, out):
             if status == RequestStatus.FAILED:
                 raise RuntimeError(f"request {rid} failed: {error}")
-            out.append(tokens)
-        return out
+        return [tokens for _, tokens, _ in out]
 
     def close(self) -> None:
         self.native.close()
@@ -312,6 +323,10 @@ class Scheduler:
 
     def cancel(self, request_id: int) -> None:
         self._host._call("cancel", request_id)
+
+    def release(self, request_id: int) -> bool:
+        """Forgets a request that has ended; False (and nothing happens) while it has not."""
+        return self._host._call("release", request_id)
 
     def has_work(self) -> bool:
         return self._host._call("has_work")

@@ -127,6 +127,7 @@ def lib() -> ctypes.CDLL:
     sig("celeg_engine_poll", c_int, c_void_p, c_int64, P(c_int32), c_int32, P(c_int32), P(c_int32))
     sig("celeg_engine_status", c_int, c_void_p, c_int64, P(c_int32))
     sig("celeg_engine_cancel", c_int, c_void_p, c_int64)
+    sig("celeg_engine_release", c_int, c_void_p, c_int64)
     sig("celeg_engine_request_error", c_char_p, c_void_p, c_int64)
     sig("celeg_engine_last_error", c_char_p, c_void_p)
     sig("celeg_engine_metrics", c_char_p, c_void_p)
@@ -412,6 +413,9 @@ class NativeEngine:
 
     def cancel(self, request_id: int) -> None:
         check(lib().celeg_engine_cancel(self.handle, request_id))
+
+    def release(self, request_id: int) -> None:
+        check(lib().celeg_engine_release(self.handle, request_id))
 
     def metrics(self) -> Dict[str, Any]:
         return json.loads(_text(lib().celeg_engine_metrics(self.handle)))

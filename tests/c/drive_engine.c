@@ -119,6 +119,17 @@ static int generate(int argc, char** argv) {
     }
     int32_t status = 0;
     if (celeg_engine_status(engine, 123456, &status) != CELEG_NOT_FOUND) return 1;
+    /* records go when they are released: a running request is refused, an ended one is unknown afterwards */
+    int64_t late;
+    int32_t one_token[1] = {1};
+    if (celeg_engine_submit(engine, one_token, 1, &ro, &late) != CELEG_OK) return fail("submit");
+    if (celeg_engine_release(engine, late) != CELEG_INVALID_ARGUMENT) return 1;
+    if (celeg_engine_cancel(engine, late) != CELEG_OK || celeg_engine_run(engine) != CELEG_OK) return fail("cancel");
+    if (celeg_engine_release(engine, late) != CELEG_OK) return fail("release");
+    for (int r = 0; r < n_requests; ++r)
+        if (celeg_engine_release(engine, ids[r]) != CELEG_OK) return fail("release");
+    if (celeg_engine_status(engine, ids[0], &status) != CELEG_NOT_FOUND) return 1;
+    if (celeg_engine_release(engine, ids[0]) != CELEG_NOT_FOUND) return 1;
     printf("metrics %s\n", celeg_engine_metrics(engine));
     celeg_engine_destroy(engine);
     return 0;

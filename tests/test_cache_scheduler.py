@@ -363,6 +363,34 @@ def test_cancel_frees_everything():
     assert m.free_pages() == [64] and m.n_free_slots == 4
 
 
+def test_release_forgets_an_ended_request_and_no_other():
+    """The record of a request stays until it is released (the reference's release,
+    src/backend/cuda/runtime/request_lifecycle.cpp:47-55): refused while the request is queued or
+    running, and the others go on as if nothing had happened."""
+    sched, m = make_scheduler()
+    fake = FakeStep()
+    a = sched.submit([1] * 20, opts(3))
+    b = sched.submit([2] * 20, opts(30))
+    assert sched.release(a) is False                 # queued
+    plan = sched.plan(); sched.accept(fake.run(plan))
+    assert sched.release(a) is False                 # running
+    while sched.request(a)["status"] != "finished":
+        plan = sched.plan(); sched.accept(fake.run(plan))
+    assert sched.poll(a)[1] == expected_output([1] * 20, 3)
+    assert sched.release(a) is True
+    with pytest.raises(ValueError, match="unknown request id"):
+        sched.request(a)
+    with pytest.raises(ValueError, match="unknown request id"):
+        sched.release(a)
+    c = sched.submit([3] * 10, opts(4))              # ids are not given out again
+    assert c not in (a, b)
+    drive(sched, fake)
+    assert sched.request(b)["generated"] == expected_output([2] * 20, 30)
+    assert sched.request(c)["generated"] == expected_output([3] * 10, 4)
+    assert sched.release(b) and sched.release(c)
+    assert m.free_pages() == [64] and m.n_free_slots == 4
+
+
 @pytest.mark.parametrize("seed", range(4))
 def test_random_workloads_terminate_with_the_right_tokens(seed):
     rng = random.Random(seed)

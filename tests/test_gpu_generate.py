@@ -353,5 +353,11 @@ def test_cancelling_while_steps_run_ahead(model_folders):
     with pytest.raises(Exception, match="max_context"):
         engine.submit(list(range(41)), options)
     after = engine.submit(prompts[0], options)          # the engine goes on
+    with pytest.raises(ValueError, match="has not ended"):
+        engine.release(after)                           # queued: a record goes only once its request has ended
     engine.run()
     assert engine.poll(after) == (RequestStatus.FINISHED, want[0], "")
+    for rid in ids + [after]:
+        engine.release(rid)
+    with pytest.raises(Exception, match="unknown request id"):
+        engine.status(after)
