@@ -625,13 +625,15 @@ extern "C" void celeg_gemm_tiles_force_dies(int dies_m) { g_force_dies_m = dies_
     X(12, 256, 160, 4, 2, 3, 64) \
     X(13, 256, 192, 4, 2, 2, 64) \
     X(14, 128, 192, 2, 2, 3, 64) \
-    X(15, 256, 128, 4, 2, 3, 64)
+    X(15, 256, 128, 4, 2, 3, 64) \
+    X(16, 128, 64, 4, 2, 4, 0) \
+    X(17, 64, 128, 2, 4, 4, 0)
 
-static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 128, 256, 256, 256, 128, 256};
-static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128, 288, 160, 192, 192, 128};
-#define N_TILE_SHAPES 16
+static const int k_shape_bm[] = {128, 256, 128, 64, 128, 256, 128, 64, 64, 128, 128, 256, 256, 256, 128, 256, 128, 64};
+static const int k_shape_bn[] = {128, 128, 64, 128, 128, 128, 128, 64, 64, 64, 128, 288, 160, 192, 192, 128, 64, 128};
+#define N_TILE_SHAPES 18
 
-static TileShape tile_shape(int M, int N, int streams) {
+static TileShape tile_shape(int M, int N, int K, int streams) {
     int id = 0;
     if (g_force_shape >= 0 && g_force_shape < N_TILE_SHAPES) id = g_force_shape;
     else {
@@ -646,7 +648,19 @@ static TileShape tile_shape(int M, int N, int streams) {
         const long long wide = static_cast<long long>((M + 127) / 128) * ((static_cast<long long>(N) * streams + 127) / 128);
         const long long tiles288 = static_cast<long long>((M + 255) / 256) * ((static_cast<long long>(N) * streams + 287) / 288);
         const long long rounds288 = (tiles288 + 255) / 256, rounds128 = (wide + 511) / 512;
-        id = wide >= 384 ? (rounds288 * 22 < rounds128 * 10 ? 11 : 10) : (wide >= 192 ? 3 : 7);
+        // Few weight rows (w2, out_proj: 1,024 of them by 2,048 rows): what a compute unit pulls
+        // from L2 bounds the product, so tiles of 128x64 or 64x128 on 8 wavefronts, one a compute
+        // unit and 4 blocks of k in flight, beat 64x64 where they still give nearly every unit
+        // one (w2 at K = 4,608: 34.8 us as 128x64, 36.0 as 64x128, 40.3 as 64x64; out_proj at
+        // K = 1,024: 14.1, 13.6, 14.5).
+        const long long tall = static_cast<long long>((M + 127) / 128) * ((static_cast<long long>(N) * streams + 63) / 64);
+        const long long flat = static_cast<long long>((M + 63) / 64) * ((static_cast<long long>(N) * streams + 127) / 128);
+        id = wide >= 384   ? (rounds288 * 22 < rounds128 * 10 ? 11 : 10)
+             : wide >= 256 ? 10
+             : wide >= 192 ? 3
+             : tall >= 224 && K >= 2048 ? 16
+             : flat >= 224 ? 17
+                           : 7;
     }
     return TileShape{id, k_shape_bm[id], k_shape_bn[id]};
 }
@@ -690,7 +704,7 @@ static int launch_tiles(const TileParams& p, hipStream_t stream) {
 
 template <int EPI>
 static int launch_epilogue(const TileParams& p, hipStream_t stream) {
-    const TileShape s = tile_shape(p.M, p.N, TileStreams<EPI>::n);
+    const TileShape s = tile_shape(p.M, p.N, p.K, TileStreams<EPI>::n);
 #define TILE_CASE(ID, BM, BN, WGM, WGN, STAGES, KB) \
     if (s.id == ID) return launch_tiles<BM, BN, WGM, WGN, STAGES, KB, EPI>(p, stream);
     TILE_SHAPES(TILE_CASE)
@@ -701,8 +715,7 @@ static int launch_epilogue(const TileParams& p, hipStream_t stream) {
 // Number of partial sums of squares a row gets from the "residual" epilogue for these
 // sizes (one per tile column): the caller sizes stats_out [>= M, >= blocks].
 extern "C" int celeg_gemm_tiles_blocks(int M, int N, int K) {
-    (void)K;
-    const TileShape s = tile_shape(M, N, 1);
+    const TileShape s = tile_shape(M, N, K, 1);
     return (N + s.bn - 1) / s.bn;
 }
 

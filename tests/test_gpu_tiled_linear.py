@@ -6,7 +6,7 @@ import torch
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 BF = torch.bfloat16
-N_SHAPES = 16
+N_SHAPES = 18
 
 
 @pytest.fixture(scope="module")
@@ -100,6 +100,29 @@ def test_residual_adds_in_place_refreshes_the_copy_and_leaves_partial_sums(ops, 
     squares = (h[:M].double() ** 2).sum(1)
     assert float(((sums[:, :blocks].double().sum(1) - squares).abs() / squares).max()) < 1e-5
     assert float(sums[:, blocks].abs().max()) == 0
+
+
+@pytest.mark.parametrize("M,N,K,blocks", [(2000, 1024, 2304, 16), (2000, 1024, 1024, 8), (2048, 2048, 1024, 16),
+                                          (2048, 3072, 1024, 24)])
+def test_the_shapes_chosen_for_a_prefill(ops, M, N, K, blocks):
+    """What the choice of shape gives at the sizes of a prefill of some 2,000 rows (few weight
+    rows with a long and a short K, q/k/v, in_proj), against torch, with the residual epilogue;
+    the number of tile columns says which shape it was."""
+    ops._lib("gemm_tiles").celeg_gemm_tiles_force(-1)
+    assert ops.tiled_stat_blocks(M, N, K) == blocks
+    a = randn(M, K, seed=20, dtype=BF)
+    w = randn(N, K, seed=21, scale=0.03, dtype=BF)
+    h0 = randn(M, N, seed=22)
+    h = h0.clone()
+    copy = torch.zeros(M, N, dtype=BF, device=DEV)
+    sums = torch.zeros(M, blocks, device=DEV)
+    ops.tiled_linear(a, w, h, epilogue="residual", out_bf16=copy, stats_out=sums)
+    y = product(a, w)
+    ref = h0.double() + bf16_round(y)
+    assert float((h.double() - ref).abs().max()) <= 2 ** -7 * float(y.abs().max())
+    assert torch.equal(copy, h.to(BF))
+    squares = (h.double() ** 2).sum(1)
+    assert float(((sums.double().sum(1) - squares).abs() / squares).max()) < 1e-5
 
 
 def test_a_row_does_not_depend_on_the_other_rows(ops):
