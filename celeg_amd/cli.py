@@ -76,6 +76,15 @@ def build_parser() -> argparse.ArgumentParser:
                     help="bfloat16 steps of more than 64 rows: the library's matrix products, this "
                          "package's tiled products with norm, SwiGLU and residual sum folded in, or "
                          "(auto) the one that was measured faster at the model's width")
+    ap.add_argument("--attention-mode", default="auto", choices=["single", "segmented", "auto"],
+                    help="attention of a decoding request: one workgroup per request and key/value head "
+                         "over the whole context (single), the context cut into parts that workgroups of "
+                         "their own take and a second kernel joins (segmented), or (auto) segmented for few "
+                         "requests and single for batches that fill the chip by themselves (the reference's "
+                         "flag of this name, src/app/cuda/main.cpp:129; its auto goes by the position)")
+    ap.add_argument("--attention-chunk-tokens", type=int, default=0, metavar="N",
+                    help="keys of a part of segmented attention: 64, 256 or 1024 (default: by the context, "
+                         "64 up to 4,096 tokens, 256 up to 16,384, 1024 above)")
     ap.add_argument("--device", default="cuda:0")
     return ap
 
@@ -105,6 +114,8 @@ def validate(args, ap) -> None:
             or args.benchmark_warmup < 0 or args.benchmark_prefill_tokens < 0 \
             or args.prefill_chunk <= 0 or args.batch <= 0 or args.page_tokens <= 0:
         ap.error("invalid numeric argument")
+    if args.attention_chunk_tokens not in (0, 64, 256, 1024):
+        ap.error("--attention-chunk-tokens must be 64, 256 or 1024")
 
 
 def main(argv: Optional[List[str]] = None) -> int:
@@ -182,6 +193,14 @@ def run(args) -> int:
     lm = engine.loaded
     if args.profile:
         lm.native.time_phases(True)
+    if args.attention_mode != "auto":
+        lm.set_knob("attention_decode_whole", 1 if args.attention_mode == "single" else 0)
+    if args.attention_chunk_tokens:
+        # parts of 1, 4 or 16 rounds of 64 keys: the two bounds on the context's rounds choose
+        big = 1 << 30
+        few, some = {64: (big, big), 256: (0, big), 1024: (0, 0)}[args.attention_chunk_tokens]
+        lm.set_knob("decode_parts_few", few)
+        lm.set_knob("decode_parts_some", some)
 
     if args.benchmark_decode > 0:
         if args.benchmark_prefill_tokens > 0:

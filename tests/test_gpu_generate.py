@@ -156,6 +156,36 @@ def test_command_line(model_folders, tmp_path):
     assert bad.returncode == 1 and "prompt plus output exceeds --context" in bad.stderr
 
 
+@pytest.mark.parametrize("flags", [["--attention-mode", "single"], ["--attention-mode", "segmented"],
+                                   ["--attention-mode", "segmented", "--attention-chunk-tokens", "256"],
+                                   ["--attention-chunk-tokens", "1024", "--no-cuda-graph"]])
+def test_command_line_attention_modes(model_folders, flags):
+    """--attention-mode / --attention-chunk-tokens (bfloat16, heads of 64: the kernels they choose
+    between): every token is the plain model's most likely one given the tokens so far, or within
+    bfloat16's rounding of it."""
+    folder = model_folders("D", torch.bfloat16, WEIGHT_STD)
+    cfg, W = plain.load_model_folder(folder)
+    prompt = random_tokens(cfg["vocab_size"], 70, seed=8)
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "celeg-run"), "--model", folder, "--prompt",
+         ",".join(map(str, prompt)), "--max-new-tokens", "10", "--repetition-penalty", "1.0", "--runtime-tokens"] + flags,
+        capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    line = [l for l in proc.stdout.splitlines() if l.startswith("CELEG_GENERATED_TOKEN_IDS=")][0]
+    out = json.loads(line.split("=", 1)[1])
+    assert 1 <= len(out) <= 10
+    seq, exact = list(prompt), 0
+    for token in out:
+        logits = plain.model_logits(cfg, W, seq)[-1]
+        assert float(logits[token]) >= float(logits.max()) - 4e-2 * float(logits.abs().max())
+        exact += int(token == int(logits.argmax()))
+        seq.append(token)
+    assert exact >= len(out) - 2
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "celeg-run"), "--model", folder, "--prompt", "1 2 3",
+                          "--attention-chunk-tokens", "100"], capture_output=True, text=True, timeout=300)
+    assert bad.returncode == 2 and "must be 64, 256 or 1024" in bad.stderr
+
+
 # ---------------------------------------------------------------- the sampling kernels alone
 @pytest.fixture(scope="module")
 def ops():
