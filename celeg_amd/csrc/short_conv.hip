@@ -7,10 +7,11 @@
 // ragged CUDA form src/backend/cuda/kernels/shortconv.cuh:34-64.
 //
 // State per request [taps, width] in 32-bit: entry j holds bx at position
-// (tokens seen) - taps + j.  The forward kernel reads only the OLD state and the rows
-// of the step; the update kernel runs after it on the same stream.  bx is kept as the
-// unrounded 32-bit product both in the state and when read from rows, so cutting a
-// sequence into steps changes nothing.
+// (tokens seen) - taps + j.  The forward kernels read only the OLD state and the rows
+// of the step; the update kernel runs after them on the same stream, except behind the
+// kernel for long steps, which updates the state itself (the thread that read a request's
+// old state writes its new one).  bx is kept as the unrounded 32-bit product both in the
+// state and when read from rows, so cutting a sequence into steps changes nothing.
 #include "common.h"
 
 template <typename T>
@@ -68,7 +69,7 @@ template <> struct ConvVec<bf16> {
 template <typename T>
 __device__ __forceinline__ void short_conv_token_vec(
     int t, int ch, const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
-    const float* __restrict__ bias, const float* __restrict__ state, size_t state_slot_stride,
+    const float* __restrict__ bias, const float* state, size_t state_slot_stride,
     T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_seqlens, int width, int taps) {
@@ -137,15 +138,60 @@ __global__ void short_conv_fwd_vec_kernel(
                             token_seq, seq_start, seq_slot, cu_seqlens, width, taps);
 }
 
+// The state update for VEC neighbouring channels of one request, by the thread that has just
+// read the old state for the request's first tokens: entry j becomes bx at position
+// end - taps + j, from the step's rows where they reach that far back, else from the old state.
+template <typename T>
+__device__ __forceinline__ void short_conv_state_vec(
+    int s, int ch, const T* __restrict__ bcx, int ld_bcx, float* state, size_t state_slot_stride,
+    const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
+    const int* __restrict__ cu_seqlens, int width, int taps) {
+    constexpr int VEC = ConvVec<T>::n;
+    typedef typename ConvVec<T>::raw raw;
+    const int start = seq_start[s];
+    const int row0 = cu_seqlens[s];
+    const int n = cu_seqlens[s + 1] - row0;
+    const int end = start + n;
+    float* st = state + static_cast<size_t>(seq_slot[s]) * state_slot_stride + ch;
+    float v[CONV_VEC_MAX_TAPS][VEC];
+#pragma unroll
+    for (int j = 0; j < CONV_VEC_MAX_TAPS; ++j) {
+        if (j >= taps) break;
+        const int q = end - taps + j;
+        if (q >= start) {
+            const T* row = bcx + static_cast<size_t>(row0 + (q - start)) * ld_bcx;
+            const raw bv = *reinterpret_cast<const raw*>(row + ch);
+            const raw xv = *reinterpret_cast<const raw*>(row + 2 * width + ch);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[j][i] = ConvVec<T>::at(bv, i) * ConvVec<T>::at(xv, i);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[j][i] = q >= 0 ? st[static_cast<size_t>(q - start + taps) * width + i] : 0.f;
+        }
+    }
+    // every old entry has been read: now the new ones
+#pragma unroll
+    for (int j = 0; j < CONV_VEC_MAX_TAPS; ++j) {
+        if (j >= taps) break;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) st[static_cast<size_t>(j) * width + i] = v[j][i];
+    }
+}
+
 // The same for TT tokens in a row per thread: where they all belong to one request and every
 // tap lies in rows of this step, a row's B and x are read once for all the tokens that use it
 // (a window that slides down the rows) instead of once per tap.  The sums are formed in the
-// same order as above, so the results are the same bits.
+// same order as above, so the results are the same bits.  The rows are asked for before it is
+// known whether the block is of that kind (their addresses do not depend on it).
+// This kernel also updates the state, with no kernel behind it: the first taps-1 tokens of a
+// request's rows, the only ones that read the old state, are all computed by the block that
+// holds the request's first row (also those that lie in the next block, which skips them), and
+// the same thread then writes the new state for its channels.
 #define CONV_BLOCK_TOKENS 4     // (2,048 tokens of 1,024 channels: 9.3 us with 4, 11.3 with 8, 15.6 with 16 a thread)
 template <typename T, int TAPS>
 __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
     const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
-    const float* __restrict__ bias, const float* __restrict__ state, size_t state_slot_stride,
+    const float* __restrict__ bias, float* state, size_t state_slot_stride,
     T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_seqlens, int width, int n_tokens) {
@@ -156,24 +202,39 @@ __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
     if (ch >= width) return;
     const int t0 = blockIdx.x * TT;
     const int n = min(TT, n_tokens - t0);
-    const int s = token_seq[t0];
-    // the same for the whole workgroup
-    if (n < TT || token_seq[t0 + TT - 1] != s || t0 - (TAPS - 1) < cu_seqlens[s]) {
-        for (int j = 0; j < n; ++j)
-            short_conv_token_vec<T>(t0 + j, ch, bcx, ld_bcx, w, bias, state, state_slot_stride, out,
-                                    positions, token_seq, seq_start, seq_slot, cu_seqlens, width, TAPS);
-        return;
-    }
     raw bv[TT + TAPS - 1], xv[TT + TAPS - 1], cv[TT];
 #pragma unroll
     for (int j = 0; j < TT + TAPS - 1; ++j) {
-        const T* row = bcx + static_cast<size_t>(t0 - (TAPS - 1) + j) * ld_bcx;
+        const T* row = bcx + static_cast<size_t>(min(max(t0 - (TAPS - 1) + j, 0), n_tokens - 1)) * ld_bcx;
         bv[j] = *reinterpret_cast<const raw*>(row + ch);
         xv[j] = *reinterpret_cast<const raw*>(row + 2 * width + ch);
     }
 #pragma unroll
     for (int j = 0; j < TT; ++j)
-        cv[j] = *reinterpret_cast<const raw*>(bcx + static_cast<size_t>(t0 + j) * ld_bcx + width + ch);
+        cv[j] = *reinterpret_cast<const raw*>(bcx + static_cast<size_t>(min(t0 + j, n_tokens - 1)) * ld_bcx + width + ch);
+    const int s = token_seq[t0];
+    // the same for the whole workgroup
+    if (n < TT || token_seq[t0 + TT - 1] != s || t0 - (TAPS - 1) < cu_seqlens[s]) {
+        for (int j = 0; j < n; ++j) {
+            const int t = t0 + j;
+            const int first = cu_seqlens[token_seq[t]];
+            if (t - first < TAPS - 1 && first < t0) continue;      // the block of the request's first row has it
+            short_conv_token_vec<T>(t, ch, bcx, ld_bcx, w, bias, state, state_slot_stride, out,
+                                    positions, token_seq, seq_start, seq_slot, cu_seqlens, width, TAPS);
+        }
+        for (int j = 0; j < n; ++j) {
+            const int t = t0 + j;
+            const int sj = token_seq[t];
+            if (cu_seqlens[sj] != t) continue;                     // requests that begin in this block:
+            const int last = min(t + TAPS - 1, cu_seqlens[sj + 1]);
+            for (int u = t0 + n; u < last; ++u)                    // their tokens in the next block that read the old state,
+                short_conv_token_vec<T>(u, ch, bcx, ld_bcx, w, bias, state, state_slot_stride, out,
+                                        positions, token_seq, seq_start, seq_slot, cu_seqlens, width, TAPS);
+            short_conv_state_vec<T>(sj, ch, bcx, ld_bcx, state, state_slot_stride, seq_start, seq_slot,      // then the new one
+                                    cu_seqlens, width, TAPS);
+        }
+        return;
+    }
     float wt[VEC][TAPS], b0[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -244,10 +305,7 @@ extern "C" int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const fl
     hipLaunchKernelGGL((short_conv_fwd_block_kernel<T_, TAPS_>), bgrid, vblock, 0, stream,          \
                        static_cast<const T_*>(bcx), ld_bcx, w, bias, state, state_slot_stride,      \
                        static_cast<T_*>(out), positions, token_seq, seq_start, seq_slot, cu_seqlens, \
-                       width, n_tokens);                                                           \
-    hipLaunchKernelGGL(short_conv_state_kernel<T_>, grid_state, block, 0, stream,                   \
-                       static_cast<const T_*>(bcx), ld_bcx, state, state_slot_stride, seq_start,    \
-                       seq_slot, cu_seqlens, width, taps)
+                       width, n_tokens)
 #define CELEG_CONV_BLOCK_T(T_)                                                                     \
     if (taps == 2) { CELEG_CONV_BLOCK(T_, 2); } else if (taps == 3) { CELEG_CONV_BLOCK(T_, 3); }     \
     else { CELEG_CONV_BLOCK(T_, 4); }

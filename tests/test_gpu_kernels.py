@@ -234,6 +234,50 @@ def test_short_conv_long_portions_of_several_requests(ops, dtype, width, taps, b
         torch.testing.assert_close(state[slots[i]], bx[-taps:], rtol=0, atol=0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width,taps", [(128, 3), (264, 4), (96, 2)])
+def test_short_conv_long_steps_with_single_tokens_and_short_portions(ops, dtype, width, taps):
+    """The kernel for long steps updates the state itself: steps that hold a long portion beside
+    requests that bring one, two or three tokens (several requests begin inside one block of
+    tokens; portions shorter than the taps keep part of the old state).  Outputs and every
+    request's state after every step against the plain convolution."""
+    from celeg_amd.engine import StepEntry
+    plans = [[66, 1, 1, 2, 3, 1], [65, 1, 2, 1, 1, 3], [70, 3, 1, 1, 2, 1], [64, 1, 1, 1, 1, 1]]
+    n_req = len(plans[0])
+    lengths = [sum(plan[i] for plan in plans) for i in range(n_req)]
+    data = [randn(n, 3 * width, seed=80 + i, dtype=dtype) for i, n in enumerate(lengths)]
+    w = randn(width, taps, seed=90)
+    cache = make_cache(0, 0, 0, dtype, states=[(0, "bx", (taps, width))], slots=n_req + 1)
+    idle = cache.open()
+    slots = [cache.open() for _ in range(n_req)]
+    state = cache.layer_cache(0).states["bx"]
+    got = [[] for _ in range(n_req)]
+    pos = [0] * n_req
+    for plan in plans:
+        entries = [StepEntry(slots[i], pos[i], [0] * n) for i, n in enumerate(plan)]
+        batch, keep = build_batch(ops, cache, entries)
+        parts = [(i, pos[i], plan[i]) for i in batch.entry_order]
+        bcx = torch.cat([data[i][p:p + n] for i, p, n in parts]).contiguous()
+        assert bcx.shape[0] >= 64
+        out = torch.empty(bcx.shape[0], width, dtype=dtype, device=DEV)
+        ops.short_conv(bcx, w, None, state, out, batch)
+        torch.cuda.synchronize()
+        row = 0
+        for i, p, n in parts:
+            got[i].append(out[row:row + n].double().cpu())
+            row += n
+            pos[i] += n
+        for i in range(n_req):
+            bx = data[i][:pos[i], :width].float() * data[i][:pos[i], 2 * width:].float()
+            want = torch.zeros(taps, width, device=DEV)
+            want[max(0, taps - pos[i]):] = bx[max(0, pos[i] - taps):]
+            torch.testing.assert_close(state[slots[i]], want, rtol=0, atol=0)
+        assert float(state[idle].abs().max()) == 0.0
+    for i in range(n_req):
+        ref = plain.short_conv(data[i].cpu(), w.cpu(), None)
+        torch.testing.assert_close(torch.cat(got[i]), ref, **tol(dtype))
+
+
 def test_short_conv_reference_vector(ops):
     # tests/reference_test.cpp:68-73: hidden 2, L 3, bcx {1,1 | 1,1 | 2,4}, weights
     # {1,2,3 ; 1,2,3} channel-major, position 0, zero state -> {6, 12}
