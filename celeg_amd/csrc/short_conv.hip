@@ -187,8 +187,8 @@ __device__ __forceinline__ void short_conv_state_vec(
 // request's rows, the only ones that read the old state, are all computed by the block that
 // holds the request's first row (also those that lie in the next block, which skips them), and
 // the same thread then writes the new state for its channels.
-#define CONV_BLOCK_TOKENS 4     // (2,048 tokens of 1,024 channels: 9.3 us with 4, 11.3 with 8, 15.6 with 16 a thread)
-template <typename T, int TAPS>
+#define CONV_BLOCK_TOKENS 2     // (2,048 tokens of 1,024 channels, with the state update: 9.2 us with 2, 10.0 with 4 a thread; more were slower)
+template <typename T, int TAPS, int TT>
 __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
     const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
     const float* __restrict__ bias, float* state, size_t state_slot_stride,
@@ -196,12 +196,13 @@ __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ cu_seqlens, int width, int n_tokens) {
     constexpr int VEC = ConvVec<T>::n;
-    constexpr int TT = CONV_BLOCK_TOKENS;
     typedef typename ConvVec<T>::raw raw;
     const int ch = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
     if (ch >= width) return;
     const int t0 = blockIdx.x * TT;
     const int n = min(TT, n_tokens - t0);
+    // (asked for ahead of the rows; what depends on it is asked for while the rows are on their way)
+    const int s = token_seq[t0], s_end = token_seq[min(t0 + TT - 1, n_tokens - 1)];
     raw bv[TT + TAPS - 1], xv[TT + TAPS - 1], cv[TT];
 #pragma unroll
     for (int j = 0; j < TT + TAPS - 1; ++j) {
@@ -212,9 +213,15 @@ __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
 #pragma unroll
     for (int j = 0; j < TT; ++j)
         cv[j] = *reinterpret_cast<const raw*>(bcx + static_cast<size_t>(min(t0 + j, n_tokens - 1)) * ld_bcx + width + ch);
-    const int s = token_seq[t0];
+    float wt[VEC][TAPS], b0[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        b0[i] = bias ? bias[ch + i] : 0.f;
+#pragma unroll
+        for (int tap = 0; tap < TAPS; ++tap) wt[i][tap] = w[static_cast<size_t>(ch + i) * TAPS + tap];
+    }
     // the same for the whole workgroup
-    if (n < TT || token_seq[t0 + TT - 1] != s || t0 - (TAPS - 1) < cu_seqlens[s]) {
+    if (n < TT || s_end != s || t0 - (TAPS - 1) < cu_seqlens[s]) {
         for (int j = 0; j < n; ++j) {
             const int t = t0 + j;
             const int first = cu_seqlens[token_seq[t]];
@@ -234,13 +241,6 @@ __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
                                     cu_seqlens, width, TAPS);
         }
         return;
-    }
-    float wt[VEC][TAPS], b0[VEC];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-        b0[i] = bias ? bias[ch + i] : 0.f;
-#pragma unroll
-        for (int tap = 0; tap < TAPS; ++tap) wt[i][tap] = w[static_cast<size_t>(ch + i) * TAPS + tap];
     }
 #pragma unroll
     for (int j = 0; j < TT; ++j) {
@@ -284,6 +284,10 @@ __global__ void short_conv_state_kernel(
     }
 }
 
+// For tests and tuning: 4 tokens a thread in the kernel for long steps instead of CONV_BLOCK_TOKENS (0: the default).
+static int g_force_block_tokens = 0;
+extern "C" void celeg_short_conv_force_block_tokens(int tokens) { g_force_block_tokens = tokens; }
+
 extern "C" int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const float* w,
                                 const float* bias, float* state, size_t state_slot_stride,
                                 void* out, const int* positions, const int* token_seq,
@@ -299,10 +303,13 @@ extern "C" int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const fl
         aligned(bcx) && aligned(out)) {
         const int threads = min(256, (width / vec + 63) / 64 * 64);
         dim3 vblock(threads), vgrid(n_tokens, (width / vec + threads - 1) / threads);
-        if (n_tokens >= 64 && taps >= 2 && taps <= 4) {
-            dim3 bgrid((n_tokens + CONV_BLOCK_TOKENS - 1) / CONV_BLOCK_TOKENS, vgrid.y);
+        if (taps >= 2 && taps <= 4) {      // (n_tokens >= 16 here)
+            const int tt = g_force_block_tokens == 4 ? 4 : CONV_BLOCK_TOKENS;
+            dim3 bgrid((n_tokens + tt - 1) / tt, vgrid.y);
 #define CELEG_CONV_BLOCK(T_, TAPS_)                                                                \
-    hipLaunchKernelGGL((short_conv_fwd_block_kernel<T_, TAPS_>), bgrid, vblock, 0, stream,          \
+    if (tt == 4) CELEG_CONV_BLOCK_TT(T_, TAPS_, 4); else CELEG_CONV_BLOCK_TT(T_, TAPS_, CONV_BLOCK_TOKENS)
+#define CELEG_CONV_BLOCK_TT(T_, TAPS_, TT_)                                                        \
+    hipLaunchKernelGGL((short_conv_fwd_block_kernel<T_, TAPS_, TT_>), bgrid, vblock, 0, stream,     \
                        static_cast<const T_*>(bcx), ld_bcx, w, bias, state, state_slot_stride,      \
                        static_cast<T_*>(out), positions, token_seq, seq_start, seq_slot, cu_seqlens, \
                        width, n_tokens)
@@ -311,6 +318,7 @@ extern "C" int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const fl
     else { CELEG_CONV_BLOCK(T_, 4); }
             if (dtype == CELEG_F32) { CELEG_CONV_BLOCK_T(float) } else { CELEG_CONV_BLOCK_T(bf16) }
 #undef CELEG_CONV_BLOCK_T
+#undef CELEG_CONV_BLOCK_TT
 #undef CELEG_CONV_BLOCK
             return CELEG_LAUNCH_RESULT();
         }

@@ -234,14 +234,17 @@ def test_short_conv_long_portions_of_several_requests(ops, dtype, width, taps, b
         torch.testing.assert_close(state[slots[i]], bx[-taps:], rtol=0, atol=0)
 
 
+@pytest.mark.parametrize("block_tokens", [0, 4])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("width,taps", [(128, 3), (264, 4), (96, 2)])
-def test_short_conv_long_steps_with_single_tokens_and_short_portions(ops, dtype, width, taps):
+def test_short_conv_long_steps_with_single_tokens_and_short_portions(ops, dtype, width, taps, block_tokens):
     """The kernel for long steps updates the state itself: steps that hold a long portion beside
     requests that bring one, two or three tokens (several requests begin inside one block of
     tokens; portions shorter than the taps keep part of the old state).  Outputs and every
     request's state after every step against the plain convolution."""
     from celeg_amd.engine import StepEntry
+    force = ops._lib("short_conv").celeg_short_conv_force_block_tokens
+    force(block_tokens)          # tokens a thread: the default, or 4
     plans = [[66, 1, 1, 2, 3, 1], [65, 1, 2, 1, 1, 3], [70, 3, 1, 1, 2, 1], [64, 1, 1, 1, 1, 1]]
     n_req = len(plans[0])
     lengths = [sum(plan[i] for plan in plans) for i in range(n_req)]
@@ -273,6 +276,7 @@ def test_short_conv_long_steps_with_single_tokens_and_short_portions(ops, dtype,
             want[max(0, taps - pos[i]):] = bx[max(0, pos[i] - taps):]
             torch.testing.assert_close(state[slots[i]], want, rtol=0, atol=0)
         assert float(state[idle].abs().max()) == 0.0
+    force(0)
     for i in range(n_req):
         ref = plain.short_conv(data[i].cpu(), w.cpu(), None)
         torch.testing.assert_close(torch.cat(got[i]), ref, **tol(dtype))
