@@ -93,7 +93,8 @@ StepBatch BatchBuilder::build(const std::vector<StepEntry>& entries,
     } else {
         for (const auto& u : updates) caps.push_back(static_cast<int>(u.size()));
     }
-    if (caps.size() != updates.size()) throw StepError("one list of block-table updates per cache group is needed");
+    if (caps.size() != updates.size() || static_cast<int>(updates.size()) != n_groups_)
+        throw StepError("one list of block-table updates per cache group is needed");
     for (size_t g = 0; g < updates.size(); ++g)
         if (static_cast<int>(updates[g].size()) > caps[g])
             throw StepError("more block-table updates than the step has room for");
