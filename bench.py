@@ -147,6 +147,9 @@ def main() -> int:
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
                          "decode measurement (the line printed then holds only that part); "
                          "serve: the whole engine on the serving workload of --shape")
+    ap.add_argument("--knob", action="append", default=[], metavar="NAME=VALUE",
+                    help="set a knob of the step function or the kernels' dispatch before measuring "
+                         "(tuning runs; the names are those of celeg_model_knobs)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="350m",
                     help="the LFM2 shape (the headline line is the 350m one)")
     args = ap.parse_args()
@@ -187,6 +190,9 @@ def main() -> int:
                                     context=context, max_batched_tokens=PROMPT_TOKENS,
                                     prefill_chunk_tokens=PROMPT_TOKENS, gemm_backend=args.gemm_backend)
     lm = engine.loaded
+    for knob in args.knob:
+        name, _, value = knob.partition("=")
+        lm.set_knob(name, int(value))
     ff = lm.config.ff_dim
     w_bytes = lm.native.info["weights"] * 2          # every weight once, bfloat16
     kv_per_token = lm.native.info["kv_bytes_per_token"]
