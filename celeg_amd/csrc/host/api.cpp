@@ -11,10 +11,25 @@
 
 using namespace celeg;
 
+// One request at a time, driven by prefill / decode calls.
+struct ModelSession {
+    int slot = -1;
+    int position = 0;               // tokens fed so far
+    bool ready = false;             // a prefill has succeeded: `logits` are those of its last token
+    Tensor logits;                  // [1, width] on the device, the last step's
+    std::unique_ptr<Sampler> sampler;
+    GenerationConfig generation;
+    double prefill_ms = 0.0, decode_ms = 0.0;
+    unsigned long long prefill_tokens = 0, decode_tokens = 0;
+};
+
 struct celeg_model {
     std::unique_ptr<LoadedModel> owned;
     LoadedModel* lm = nullptr;
     PinnedBuffer logits_stage;      // few rows of logits come to the host through pinned memory
+    std::unique_ptr<ModelSession> session;
+    // (the session's sampler points into the model's runtime: it goes first)
+    ~celeg_model() { session.reset(); }
 };
 struct celeg_engine {
     std::unique_ptr<Engine> engine;
@@ -442,6 +457,121 @@ celeg_status celeg_model_step(celeg_model* model, int32_t n_entries, const int32
         if (wanted)
             CELEG_HIP(hipMemcpy2D(logits, width * 4, out.data, static_cast<size_t>(out.row_stride()) * 4, width * 4, wanted,
                                   hipMemcpyDeviceToHost));
+    });
+}
+
+// ---------------------------------------------------------------------------- one request at a time
+static ModelSession& session_of(celeg_model* model) {
+    if (!model->owned) throw ConfigError("the prefill / decode calls need a model of its own, not an engine's");
+    if (!model->session) {
+        auto s = std::make_unique<ModelSession>();
+        LoadedModel& lm = *model->lm;
+        s->sampler = std::make_unique<Sampler>(*lm.rt, lm.model->logit_width(), lm.cache->max_requests);
+        model->session = std::move(s);
+    }
+    return *model->session;
+}
+
+celeg_status celeg_model_set_generation(celeg_model* model, const celeg_generation_options* options) {
+    if (!model) return CELEG_INVALID_ARGUMENT;
+    return guarded([&] {
+        const celeg_generation_options o = options_from(options, celeg_generation_options_init);
+        GenerationConfig c = generation_of(o);
+        c.validate();
+        session_of(model).generation = c;        // from the next prefill on
+    });
+}
+
+celeg_status celeg_model_prefill(celeg_model* model, const int32_t* tokens, size_t count) {
+    if (!model || !tokens || count == 0) {
+        g_error = "celeg_model_prefill: model and tokens must not be null, and at least one token is needed";
+        return CELEG_INVALID_ARGUMENT;
+    }
+    return guarded([&] {
+        ModelSession& s = session_of(model);
+        LoadedModel& lm = *model->lm;
+        if (count > static_cast<size_t>(lm.cache->max_context)) throw ConfigError("prefill exceeds max_context");
+        s.ready = false;
+        if (s.slot >= 0) {                       // an earlier sequence: what it held goes back
+            s.sampler->end(s.slot);
+            lm.cache->close(s.slot);
+            s.slot = -1;
+        }
+        s.slot = lm.cache->open();
+        if (s.slot < 0) throw StepError("prefill: every slot of the cache is taken");
+        s.position = 0;
+        s.sampler->begin(s.slot, s.generation);
+        const auto begun = std::chrono::steady_clock::now();
+        const size_t portion = static_cast<size_t>(lm.runner->max_batched_tokens);
+        for (size_t done = 0; done < count; done += portion) {
+            const size_t n = std::min(portion, count - done);
+            if (!lm.cache->prepare(s.slot, static_cast<int>(done), static_cast<int>(n)))
+                throw StepError("prefill: the cache has too few pages for the prompt");
+            StepEntry e;
+            e.slot = s.slot;
+            e.start_pos = static_cast<int>(done);
+            e.tokens.assign(tokens + done, tokens + done + n);
+            if (done + n == count) e.want = {static_cast<int>(n) - 1};
+            s.logits = lm.runner->step({e});
+            if (s.sampler->uses_seen()) s.sampler->mark_seen(lm.runner->last_batch());
+            s.position = static_cast<int>(done + n);
+        }
+        CELEG_HIP(hipStreamSynchronize(lm.stream));
+        s.prefill_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - begun).count();
+        s.prefill_tokens = count;
+        s.decode_ms = 0.0;
+        s.decode_tokens = 0;
+        s.ready = true;
+    });
+}
+
+celeg_status celeg_model_decode(celeg_model* model, int32_t* token) {
+    if (!model || !token) return CELEG_INVALID_ARGUMENT;
+    return guarded([&] {
+        ModelSession& s = session_of(model);
+        LoadedModel& lm = *model->lm;
+        if (!s.ready) throw StepError("decode requires a successful prefill");
+        if (s.position >= lm.cache->max_context) throw StepError("context limit reached");
+        const auto begun = std::chrono::steady_clock::now();
+        const int chosen = s.sampler->sample(s.logits, {s.slot}).at(0);
+        s.ready = false;                         // until the token has been fed
+        if (!lm.cache->prepare(s.slot, s.position, 1)) throw StepError("decode: the cache has no page left");
+        StepEntry e;
+        e.slot = s.slot;
+        e.start_pos = s.position;
+        e.tokens = {chosen};
+        e.want = {0};
+        s.logits = lm.runner->step({e});
+        CELEG_HIP(hipStreamSynchronize(lm.stream));
+        ++s.position;
+        ++s.decode_tokens;
+        s.decode_ms += std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - begun).count();
+        s.ready = true;
+        *token = chosen;
+    });
+}
+
+celeg_status celeg_model_copy_logits(celeg_model* model, float* output, size_t capacity, size_t* required) {
+    if (!model || !required) return CELEG_INVALID_ARGUMENT;
+    return guarded([&] {
+        ModelSession& s = session_of(model);
+        if (!s.ready) throw StepError("copy_logits requires a successful prefill");
+        const size_t width = static_cast<size_t>(s.logits.shape[1]);
+        *required = width;
+        if (!output || capacity < width) throw StepError("logit output buffer is too small");
+        CELEG_HIP(hipStreamSynchronize(model->lm->stream));
+        CELEG_HIP(hipMemcpy(output, s.logits.data, width * sizeof(float), hipMemcpyDeviceToHost));
+    });
+}
+
+celeg_status celeg_model_get_metrics(celeg_model* model, celeg_metrics* metrics) {
+    if (!model || !metrics || metrics->struct_size < sizeof(*metrics)) return CELEG_INVALID_ARGUMENT;
+    return guarded([&] {
+        const ModelSession& s = session_of(model);
+        metrics->prefill_ms = s.prefill_ms;
+        metrics->prefill_tokens = s.prefill_tokens;
+        metrics->decode_ms = s.decode_ms;
+        metrics->decode_tokens = s.decode_tokens;
     });
 }
 

@@ -160,6 +160,27 @@ const char* celeg_model_cache_state(celeg_model* model);
 celeg_status celeg_model_step(celeg_model* model, int32_t n_entries, const int32_t* slot, const int32_t* start_pos,
                               const int32_t* n_tokens, const int32_t* tokens, const int32_t* n_want,
                               const int32_t* want, float* logits, size_t capacity);
+/* ---- one request at a time on a model of its own (the reference's celeg_model_prefill / decode /
+ * copy_logits / get_metrics, include/celeg/api.h:158-164, src/api/model.cpp:32-77): prefill starts a new
+ * sequence with a prompt (what the model held of an earlier one is given back); decode chooses the next
+ * token from the logits of the last step (by the generation options: celeg_generation_options_init's
+ * defaults unless set), feeds it, and returns it; copy_logits gives the logits the next decode will
+ * choose from.  Not for a model that belongs to an engine. ---- */
+typedef struct celeg_metrics {
+    size_t struct_size;
+    double prefill_ms;          /* the last prefill */
+    uint64_t prefill_tokens;
+    double decode_ms;           /* all decode calls since that prefill */
+    uint64_t decode_tokens;
+} celeg_metrics;
+/* the options of the sequences that later prefills start (null: the defaults) */
+celeg_status celeg_model_set_generation(celeg_model* model, const celeg_generation_options* options);
+celeg_status celeg_model_prefill(celeg_model* model, const int32_t* tokens, size_t count);
+celeg_status celeg_model_decode(celeg_model* model, int32_t* token);
+/* *required: the number of logits; CELEG_ERROR if output is null or capacity is smaller */
+celeg_status celeg_model_copy_logits(celeg_model* model, float* output, size_t capacity, size_t* required);
+celeg_status celeg_model_get_metrics(celeg_model* model, celeg_metrics* metrics);
+
 /* knobs of the runner and the kernels' dispatch, by name (tests and tuning); JSON of the known names
  * and their values comes back from celeg_model_knobs */
 celeg_status celeg_model_set_knob(celeg_model* model, const char* name, int32_t value);

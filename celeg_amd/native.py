@@ -37,6 +37,11 @@ class GenerationOptions(ctypes.Structure):
                 ("forced_prefix", P(c_int32)), ("n_forced_prefix", c_int32)]
 
 
+class SessionMetrics(ctypes.Structure):
+    _fields_ = [("struct_size", c_size_t), ("prefill_ms", ctypes.c_double), ("prefill_tokens", ctypes.c_uint64),
+                ("decode_ms", ctypes.c_double), ("decode_tokens", ctypes.c_uint64)]
+
+
 class EngineOptions(ctypes.Structure):
     _fields_ = [("struct_size", c_size_t), ("dtype", c_char_p), ("device", c_int32),
                 ("max_active_requests", c_int32), ("max_batched_tokens", c_int32),
@@ -148,6 +153,11 @@ def lib() -> ctypes.CDLL:
     sig("celeg_model_knobs", c_char_p, c_void_p)
     sig("celeg_model_stream", c_void_p, c_void_p)
     sig("celeg_model_synchronize", c_int, c_void_p)
+    sig("celeg_model_set_generation", c_int, c_void_p, P(GenerationOptions))
+    sig("celeg_model_prefill", c_int, c_void_p, P(c_int32), c_size_t)
+    sig("celeg_model_decode", c_int, c_void_p, P(c_int32))
+    sig("celeg_model_copy_logits", c_int, c_void_p, P(c_float), c_size_t, P(c_size_t))
+    sig("celeg_model_get_metrics", c_int, c_void_p, P(SessionMetrics))
     sig("celeg_model_time_phases", c_int, c_void_p, c_int32)
     sig("celeg_model_phase_times", c_char_p, c_void_p)
     sig("celeg_describe_folder", c_char_p, c_char_p)
@@ -315,6 +325,45 @@ class NativeModel:
 
     def synchronize(self) -> None:
         check(lib().celeg_model_synchronize(self.handle))
+
+    # ---- one request at a time (celeg_model_prefill / decode / copy_logits / get_metrics)
+    def set_generation(self, *, temperature=0.1, top_k=50, top_p=1.0, repetition_penalty=1.05, seed=1,
+                       forced_prefix=()) -> None:
+        g = GenerationOptions()
+        lib().celeg_generation_options_init(ctypes.byref(g), ctypes.sizeof(g))
+        g.temperature, g.top_k, g.top_p = float(temperature), int(top_k), float(top_p)
+        g.repetition_penalty, g.seed = float(repetition_penalty), int(seed)
+        forced = None
+        if forced_prefix:
+            forced = _ints([int(t) for t in forced_prefix])        # (kept alive until the call has copied it)
+            g.forced_prefix = ctypes.cast(forced, P(c_int32))
+            g.n_forced_prefix = len(forced_prefix)
+        check(lib().celeg_model_set_generation(self.handle, ctypes.byref(g)))
+
+    def prefill(self, tokens: Sequence[int]) -> None:
+        """Starts a new sequence with this prompt (the model's earlier one is given back)."""
+        toks = [int(t) for t in tokens]
+        check(lib().celeg_model_prefill(self.handle, _ints(toks), len(toks)))
+
+    def decode(self) -> int:
+        """Chooses the next token from the last step's logits, feeds it, returns it."""
+        token = c_int32()
+        check(lib().celeg_model_decode(self.handle, ctypes.byref(token)))
+        return token.value
+
+    def copy_logits(self) -> np.ndarray:
+        """The logits the next ``decode`` chooses from."""
+        out = np.empty(self.logit_width, dtype=np.float32)
+        required = c_size_t()
+        check(lib().celeg_model_copy_logits(self.handle, out.ctypes.data_as(P(c_float)), out.size, ctypes.byref(required)))
+        return out[:required.value]
+
+    def session_metrics(self) -> Dict[str, float]:
+        m = SessionMetrics()
+        m.struct_size = ctypes.sizeof(m)
+        check(lib().celeg_model_get_metrics(self.handle, ctypes.byref(m)))
+        return {"prefill_ms": m.prefill_ms, "prefill_tokens": int(m.prefill_tokens), "decode_ms": m.decode_ms,
+                "decode_tokens": int(m.decode_tokens)}
 
     def time_phases(self, on: bool = True) -> None:
         """Time every step's phases with events (such steps are not replayed from graphs)."""
