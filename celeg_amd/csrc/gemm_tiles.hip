@@ -36,7 +36,7 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 
-enum { T_STORE = 0, T_RESIDUAL = 2, T_SWIGLU = 3 };   // the numbers of the few-rows products
+enum { T_STORE = 0, T_RESIDUAL = 2, T_SWIGLU = 3, T_QKV = 5 };   // (0, 2, 3: the numbers of the few-rows products)
 
 
 #define GPTR(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -226,6 +226,178 @@ __device__ __forceinline__ void tile_epilogue(
     }
 }
 
+// ---- the q/k/v epilogue (heads of 64 columns: a wavefront of a 128x128 tile on 4x2 wavefronts
+// holds 32 rows of one head)
+#define QKV_HD 64
+// What it needs from memory, asked for before the product: the positions of the lane's rows
+// and the head's norm weight at the lane's columns; and, lanes 0 .. rows-1 of the wavefront, the
+// position and the slot of one row each (whose page is looked up once they have arrived).
+template <int FM>
+struct QkvEarly {
+    int pos[FM];
+    floatx4_t weight[4];
+    int row_pos, row_slot, row_page;
+};
+
+template <int BM, int WGM, int WGN>
+__device__ __forceinline__ void qkv_early_rows(const TileParams& p, QkvEarly<BM / WGM / 16>& e, const int m0, const int col0,
+                                               const int wm, const int lane) {
+    constexpr int WTM = BM / WGM, FM = WTM / 16;
+    const int r16 = lane & 15, q = lane >> 4;
+    const int head = min(col0, p.N - QKV_HD) / QKV_HD;
+    const float* const weight = head < p.q_heads ? p.q_weight : (head < p.q_heads + p.kv_heads ? p.k_weight : nullptr);
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) e.pos[tm] = p.positions[min(m0 + wm * WTM + tm * 16 + r16, p.M - 1)];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        e.weight[j] = weight ? *reinterpret_cast<const floatx4_t*>(weight + j * 16 + 4 * q) : floatx4_t{1.f, 1.f, 1.f, 1.f};
+    const int row = min(m0 + wm * WTM + min(lane, WTM - 1), p.M - 1);
+    e.row_pos = p.positions[row];
+    e.row_slot = p.token_slot[row];
+    e.row_page = 0;
+}
+
+// (behind the first blocks' loads: the page of the lane's row)
+template <int BM, int WGM, int WGN>
+__device__ __forceinline__ void qkv_early_pages(const TileParams& p, QkvEarly<BM / WGM / 16>& e, const int col0) {
+    const int head = min(col0, p.N - QKV_HD) / QKV_HD;
+    if (head >= p.q_heads)
+        e.row_page = p.table[static_cast<size_t>(e.row_slot) * p.table_stride + e.row_pos / p.page_tokens];
+}
+
+// acc[j][tm][i]: row .. + tm*16 + lane%16, column col0 + j*16 + 4*(lane/16) + i of the head at col0.
+// The sums are rounded to bfloat16 first, as where the product is a tensor of its own; norm,
+// rotation (split halves: pair (c, c + 32)) as qk_norm_rope_store makes them.  The head's rows
+// go to the wavefront's corner of LDS and leave from there: query rows to `out`, key rows to
+// their places in the pages, values by groups of four tokens that lie side by side in a page.
+template <int BM, int WGM, int WGN>
+__device__ __forceinline__ void qkv_epilogue(const TileParams& p, floatx4_t (&acc)[4][BM / WGM / 16],
+                                             const float (&scale)[BM / WGM / 16], const QkvEarly<BM / WGM / 16>& e,
+                                             const int m0, const int col0, const int wm, const int wn, const int lane,
+                                             char* const lds) {
+    constexpr int WTM = BM / WGM, FM = WTM / 16;
+    constexpr int PITCH = QKV_HD * 2 + 16;            // bytes between a wavefront's rows in LDS
+    constexpr int CORNER = WTM * PITCH + WTM * 16;    // the rows, then (position, slot, page, -) of every row
+    const int M = p.M;
+    const int r16 = lane & 15, q = lane >> 4;
+    char* const corner = lds + static_cast<size_t>(wm * WGN + wn) * CORNER;
+    int* const rowinfo = reinterpret_cast<int*>(corner + WTM * PITCH);
+    const int head = min(col0, p.N - QKV_HD) / QKV_HD;
+    const bool is_q = head < p.q_heads, is_k = !is_q && head < p.q_heads + p.kv_heads;
+    const int kv_head = is_q ? 0 : (is_k ? head - p.q_heads : head - p.q_heads - p.kv_heads);
+    const bool normed = is_q ? p.q_weight != nullptr : (is_k && p.k_weight != nullptr);
+    const bool rotate = p.cos_sin && (is_q || is_k);
+    // (cos, sin) of the lane's 2 x 4 column pairs for each of its rows: asked for only now (the
+    // registers they take would cost the product a wavefront a SIMD), ahead of the barrier
+    floatx4_t cs[FM][4];
+    if (rotate) {
+#pragma unroll
+        for (int tm = 0; tm < FM; ++tm) {
+            const float* const c = p.cos_sin + static_cast<size_t>(e.pos[tm]) * QKV_HD;     // 32 pairs of two
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                cs[tm][2 * j] = *reinterpret_cast<const floatx4_t*>(c + (j * 16 + 4 * q) * 2);
+                cs[tm][2 * j + 1] = *reinterpret_cast<const floatx4_t*>(c + (j * 16 + 4 * q) * 2 + 4);
+            }
+        }
+    }
+    __syncthreads();                                  // the stages are no longer read
+    if (col0 >= p.N) return;                          // (a tile that hangs over the last head)
+#pragma unroll
+    for (int tm = 0; tm < FM; ++tm) {
+        float x[4][4];
+        float ssq = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                x[j][i] = round_bf16(acc[j][tm][i] * scale[tm] + (p.bias ? p.bias[col0 + j * 16 + 4 * q + i] : 0.f));
+                ssq += x[j][i] * x[j][i];
+            }
+        if (normed) {
+            ssq += __shfl_xor(ssq, 16, 64);
+            ssq += __shfl_xor(ssq, 32, 64);
+            const float inv = 1.0f / sqrtf(ssq / static_cast<float>(QKV_HD) + p.qk_eps);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) x[j][i] = x[j][i] * inv * e.weight[j][i];
+        }
+        if (rotate) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    // (cos, sin) of pair j*16 + 4q + i: four pairs are two loads of four floats
+                    const float c = i < 2 ? cs[tm][2 * j][2 * i] : cs[tm][2 * j + 1][2 * (i - 2)];
+                    const float s = i < 2 ? cs[tm][2 * j][2 * i + 1] : cs[tm][2 * j + 1][2 * (i - 2) + 1];
+                    const float a = x[j][i], b = x[j + 2][i];
+                    x[j][i] = a * c - b * s;
+                    x[j + 2][i] = b * c + a * s;
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<bf16x4_t*>(corner + (tm * 16 + r16) * PITCH + (j * 16 + 4 * q) * 2) =
+                bf16x4_t{static_cast<__bf16>(x[j][0]), static_cast<__bf16>(x[j][1]), static_cast<__bf16>(x[j][2]),
+                         static_cast<__bf16>(x[j][3])};
+    }
+    if (lane < WTM) {
+        rowinfo[4 * lane] = e.row_pos;
+        rowinfo[4 * lane + 1] = e.row_slot;
+        rowinfo[4 * lane + 2] = e.row_page;
+    }
+    // (the wavefront reads what its own lanes wrote: LDS keeps a wavefront's accesses in order)
+    const int page_mask = p.page_tokens - 1;
+    const int row_base = m0 + wm * WTM;
+    if (is_q || is_k) {
+        for (int idx = lane; idx < WTM * 8; idx += 64) {
+            const int row = idx >> 3, ch = idx & 7;
+            if (row_base + row >= M) continue;
+            const bf16x8_t piece = *reinterpret_cast<const bf16x8_t*>(corner + row * PITCH + ch * 16);
+            bf16* to;
+            if (is_q) {
+                to = static_cast<bf16*>(p.out) + static_cast<size_t>(row_base + row) * p.ldo + col0 + ch * 8;
+            } else {
+                const int pos = rowinfo[4 * row], page = rowinfo[4 * row + 2];
+                to = p.k_pool + (((static_cast<size_t>(page) * p.n_layers + p.layer) * p.kv_heads + kv_head) * p.page_tokens +
+                                 (pos & page_mask)) * QKV_HD + ch * 8;
+            }
+            *reinterpret_cast<bf16x8_t*>(to) = piece;
+        }
+        return;
+    }
+    // values: [dimension][token] inside a page
+    for (int u = lane; u < (WTM / 4) * QKV_HD; u += 64) {
+        const int g = u % (WTM / 4), d = u / (WTM / 4);
+        const int r0 = 4 * g;
+        const int pos0 = rowinfo[4 * r0], slot0 = rowinfo[4 * r0 + 1];
+        bool together = row_base + r0 + 3 < M && (pos0 & 3) == 0;
+        unsigned short val[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            together = together && rowinfo[4 * (r0 + k)] == pos0 + k && rowinfo[4 * (r0 + k) + 1] == slot0;
+            val[k] = *reinterpret_cast<const unsigned short*>(corner + (r0 + k) * PITCH + d * 2);
+        }
+        if (together) {
+            bf16* const to = p.v_pool + ((static_cast<size_t>(rowinfo[4 * r0 + 2]) * p.n_layers + p.layer) * p.kv_heads + kv_head) *
+                                            p.page_tokens * QKV_HD + static_cast<size_t>(d) * p.page_tokens + (pos0 & page_mask);
+            *reinterpret_cast<uint2*>(to) = uint2{static_cast<unsigned>(val[0]) | (static_cast<unsigned>(val[1]) << 16),
+                                                  static_cast<unsigned>(val[2]) | (static_cast<unsigned>(val[3]) << 16)};
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                if (row_base + r0 + k >= M) continue;
+                const int pos = rowinfo[4 * (r0 + k)], page = rowinfo[4 * (r0 + k) + 2];
+                unsigned short* const to = reinterpret_cast<unsigned short*>(
+                    p.v_pool + ((static_cast<size_t>(page) * p.n_layers + p.layer) * p.kv_heads + kv_head) * p.page_tokens * QKV_HD +
+                    static_cast<size_t>(d) * p.page_tokens + (pos & page_mask));
+                *to = val[k];
+            }
+        }
+    }
+}
+
 template <int BM, int BN, int WGM, int WGN, int STAGES, int EPI>
 __global__ __launch_bounds__(WGM * WGN * 64)
 void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n, const int dies_m) {
@@ -300,11 +472,14 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
     // ---- the rows' 1/rms, asked for ahead of the first blocks
     float scale[FM];
     tile_row_scales<FM>(p, m0 + wm * WTM + r16, q, scale);
+    QkvEarly<EPI == T_QKV ? FM : 1> qkv_early;
+    if constexpr (EPI == T_QKV) qkv_early_rows<BM, WGM, WGN>(p, qkv_early, m0, n0 + wn * WTN, wm, lane);
 
     const int nkb = K >> 6;                       // K % 64 == 0 (checked by the host)
 #pragma unroll
     for (int s = 0; s < STAGES; ++s)
         if (s < nkb) issue(s, s);
+    if constexpr (EPI == T_QKV) qkv_early_pages<BM, WGM, WGN>(p, qkv_early, n0 + wn * WTN);
 
     // Operands of a k-step (32 values of k) travel from LDS to registers one step ahead of
     // the matrix instructions that use them: a wavefront asks for step 1 of a block, then
@@ -353,7 +528,12 @@ void gemm_tiles_kernel(const TileParams p, const int tiles_m, const int tiles_n,
         stage = next;
     }
 
-    tile_epilogue<BM, WGM, WGN, FN / NS, EPI, false>(p, acc, scale, m0, n0 + wn * (WTN / NS), FN / NS, tile_n, wm, wn, lane, lds);
+    if constexpr (EPI == T_QKV) {
+        static_assert(EPI != T_QKV || (WTN == QKV_HD && FN == 4), "a wavefront holds one head of 64 columns");
+        qkv_epilogue<BM, WGM, WGN>(p, acc, scale, qkv_early, m0, n0 + wn * WTN, wm, wn, lane, lds);
+    } else {
+        tile_epilogue<BM, WGM, WGN, FN / NS, EPI, false>(p, acc, scale, m0, n0 + wn * (WTN / NS), FN / NS, tile_n, wm, wn, lane, lds);
+    }
 }
 
 // A read of 16 bytes a lane from LDS at `address` + index * STRIDE, and the waits that go with
@@ -737,6 +917,18 @@ extern "C" int celeg_gemm_tiles(const TileParams* params, int epi, hipStream_t s
         case T_STORE: return launch_epilogue<T_STORE>(p, stream);
         case T_RESIDUAL: return launch_epilogue<T_RESIDUAL>(p, stream);
         case T_SWIGLU: return launch_epilogue<T_SWIGLU>(p, stream);
+        case T_QKV: {
+            const auto misaligned = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) != 0; };
+            const long long heads = static_cast<long long>(p.q_heads) + 2LL * p.kv_heads;
+            if (p.q_heads <= 0 || p.kv_heads <= 0 || p.N != heads * QKV_HD || p.ldo % 8 || misaligned(p.out) ||
+                !p.positions || !p.token_slot || !p.table || p.table_stride <= 0 || !p.k_pool || !p.v_pool ||
+                misaligned(p.k_pool) || misaligned(p.v_pool) || p.page_tokens < 4 || (p.page_tokens & (p.page_tokens - 1)) ||
+                p.n_layers <= 0 || p.layer < 0 || p.layer >= p.n_layers || misaligned(p.q_weight) || misaligned(p.k_weight) ||
+                misaligned(p.cos_sin))
+                return static_cast<int>(hipErrorInvalidValue);
+            // a wavefront of the 128x128 tile on 4x2 wavefronts holds 32 rows of one head
+            return launch_tiles<128, 128, 4, 2, 2, 0, T_QKV>(p, stream);
+        }
         default: return static_cast<int>(hipErrorInvalidValue);
     }
 }

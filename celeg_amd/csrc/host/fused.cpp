@@ -95,6 +95,8 @@ std::shared_ptr<DeviceTensor> packed_weight(Runtime& rt, const Tensor& w) {
 }
 }  // namespace
 
+bool qkv_tail_ok(const Runtime& rt, int rows) { return tiled_step(rt, rows); }
+
 void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const Tensor& w, const Tensor& out,
                  Epilogue epilogue, const LinearExtras& extras) {
     int blocks = rt.stream_stat_blocks;
@@ -112,9 +114,10 @@ void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const
             rt.stream_has_bf16 = true;
         }
         rt.ops.tiled_linear(xb, folded_plain_weight(rt, w, norm.weight)->view, out, epilogue, norm.eps, &stats, blocks,
-                            extras.bias.defined() ? &extras.bias : nullptr, nullptr, nullptr);
+                            extras.bias.defined() ? &extras.bias : nullptr, nullptr, nullptr, extras.qkv);
         return;
     }
+    if (extras.qkv) throw KernelError("norm_linear: the q/k/v tail goes with steps of many rows");
     const int streams = epilogue == Epilogue::Swiglu ? 2 : epilogue == Epilogue::Conv ? 3 : 1;
     const bool streamed = rt.ops.rows_kernel_ok(M, {width});
     FusedArgs args;

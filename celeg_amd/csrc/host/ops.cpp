@@ -582,9 +582,18 @@ int Ops::tiled_stat_blocks(int rows, int n, int k) const { return celeg_gemm_til
 // 1/rms (with eps) scales the sums.  Epilogues: Store (bfloat16 [M, N]), Residual (out is the
 // 32-bit stream, added to in place; out_bf16 receives its bfloat16 copy and stats_out the partial
 // sums of squares of the new rows; last_stat_blocks says how many a row), Swiglu (w is [2N, K]).
+bool Ops::tiled_qkv_ok(int head_dim, const Tensor* inv_freq, int rotary_dim, int pairing, const KVView& kv) const {
+    if (!use_qkv_tail) return false;
+    if (head_dim != 64 || kv.dtype != DType::BF16 || kv.head_dim != 64 || (kv.v_head_dim && kv.v_head_dim != 64)) return false;
+    if (kv.page_tokens < 4 || (kv.page_tokens & (kv.page_tokens - 1))) return false;
+    // the rotation: none, or of the whole head by split halves from the table of cosines and sines
+    return !inv_freq || (rotary_dim == head_dim && pairing == 0 && use_rope_table);
+}
+
 void Ops::tiled_linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue epi, float eps, const Tensor* stats,
-                       int stat_blocks, const Tensor* bias, const Tensor* stats_out, const Tensor* out_bf16) {
+                       int stat_blocks, const Tensor* bias, const Tensor* stats_out, const Tensor* out_bf16, const QkvTail* qkv) {
     need(epi == Epilogue::Store || epi == Epilogue::Residual || epi == Epilogue::Swiglu, "tiled_linear: unknown epilogue");
+    need(!qkv || epi == Epilogue::Store, "tiled_linear: the q/k/v tail goes with the store epilogue");
     dev(a, "a", DType::BF16, false);
     dev(w, "w", DType::BF16);
     const int streams = epi == Epilogue::Swiglu ? 2 : 1;
@@ -647,7 +656,41 @@ void Ops::tiled_linear(const Tensor& a, const Tensor& w, const Tensor& out, Epil
     } else {
         need(!out_bf16 && !stats_out, "tiled_linear: out_bf16 and stats_out go with the residual epilogue");
     }
-    kernel_check(celeg_gemm_tiles(&prm, static_cast<int>(epi), stream), "tiled_linear");
+    int kernel_epilogue = static_cast<int>(epi);
+    if (qkv) {
+        need(qkv->batch && qkv->kv, "tiled_linear: the q/k/v tail needs the step and the cache");
+        const KVView& kv = *qkv->kv;
+        need(tiled_qkv_ok(qkv->head_dim, qkv->inv_freq, qkv->head_dim, 0, kv), "tiled_linear: the q/k/v tail does not take these sizes");
+        check_kv(kv, qkv->kv_heads, qkv->head_dim, DType::BF16);
+        need(N == (static_cast<long long>(qkv->heads) + 2LL * qkv->kv_heads) * qkv->head_dim && M == qkv->batch->n_tokens,
+             "tiled_linear: the q/k/v tail needs all heads of every row of the step");
+        for (const Tensor* wt : {qkv->q_weight, qkv->k_weight})
+            if (wt) {
+                dev(*wt, "q/k norm weight", DType::F32);
+                need(wt->numel() == qkv->head_dim, "tiled_linear: a norm weight must have head_dim entries");
+            }
+        prm.positions = qkv->batch->positions;
+        prm.token_slot = qkv->batch->token_slot;
+        prm.table = kv.table;
+        prm.table_stride = kv.table_stride;
+        prm.k_pool = static_cast<bf16*>(kv.k);
+        prm.v_pool = static_cast<bf16*>(kv.v);
+        prm.n_layers = kv.n_layers;
+        prm.layer = kv.layer;
+        prm.page_tokens = kv.page_tokens;
+        prm.q_heads = qkv->heads;
+        prm.kv_heads = qkv->kv_heads;
+        prm.q_weight = qkv->q_weight ? qkv->q_weight->as<float>() : nullptr;
+        prm.k_weight = qkv->k_weight ? qkv->k_weight->as<float>() : nullptr;
+        prm.qk_eps = qkv->eps;
+        if (qkv->inv_freq) {
+            dev(*qkv->inv_freq, "inv_freq", DType::F32);
+            need(qkv->inv_freq->numel() == qkv->head_dim / 2, "tiled_linear: the frequency table must have head_dim / 2 entries");
+            prm.cos_sin = rope_table(*qkv->inv_freq, kv.table_stride * kv.page_tokens);
+        }
+        kernel_epilogue = 5;
+    }
+    kernel_check(celeg_gemm_tiles(&prm, kernel_epilogue, stream), "tiled_linear");
 }
 
 std::shared_ptr<DeviceTensor> Ops::fold_weight(const Tensor& w, const Tensor* scale, bool packed) {

@@ -23,6 +23,19 @@ namespace celeg {
 
 enum class Epilogue : int { Store = 0, StoreF32 = 1, Residual = 2, Swiglu = 3, Conv = 4 };
 
+// What follows a q/k/v product of many rows inside its kernel (heads of 64 columns): the norm of
+// query and key heads, their rotation by the rows' positions, and the write of keys and values
+// into the pages of the rows' requests; the query heads alone reach `out`.
+struct QkvTail {
+    int heads = 0, kv_heads = 0, head_dim = 0;
+    const Tensor* q_weight = nullptr;      // [head_dim] 32-bit, or null: no norm
+    const Tensor* k_weight = nullptr;
+    float eps = 0.f;
+    const Tensor* inv_freq = nullptr;      // [head_dim / 2], or null: no rotation
+    const StepBatch* batch = nullptr;
+    const KVView* kv = nullptr;
+};
+
 // The convolution epilogue's operands: one new token per request.
 struct ConvOperands {
     Tensor taps;          // [N, L] 32-bit
@@ -57,6 +70,7 @@ public:
     int decode_part_thresholds[2] = {64, 256};
     bool attention_general = false;      // always the general attention kernel
     bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
+    bool use_qkv_tail = true;          // q/k/v products of many rows take norm, rotation and cache write along
     int rows_kernel_min_rows = 9, tiles_min_rows = 65, fused_linear_shape = 0;
     int last_stat_blocks = 0;
 
@@ -98,7 +112,9 @@ public:
     int tiled_stat_blocks(int rows, int n, int k) const;
     void tiled_linear(const Tensor& a, const Tensor& w, const Tensor& out, Epilogue epilogue, float eps,
                       const Tensor* stats, int stat_blocks, const Tensor* bias, const Tensor* stats_out,
-                      const Tensor* out_bf16);
+                      const Tensor* out_bf16, const QkvTail* qkv = nullptr);
+    // whether the q/k/v product of many rows can take what follows it (norm, rotation, cache write) along
+    bool tiled_qkv_ok(int head_dim, const Tensor* inv_freq, int rotary_dim, int pairing, const KVView& kv) const;
     // weights re-laid at load time: w [rows, K] scaled by a norm's weight (or not) and, if
     // `packed`, laid as [K/32, rows, 32]
     std::shared_ptr<DeviceTensor> fold_weight(const Tensor& w, const Tensor* scale, bool packed);

@@ -333,10 +333,31 @@ private:
             if (norm) fused::norm_linear(rt, x, *norm, w->view, out, Epilogue::Store);
             else rt.ops.linear(x, w->view, out, nullptr, rt.ws);
         };
+        const PositionEncoding::Tables tables = position_->tables(rt);
+        const Tensor* inv_freq = tables.inv_freq.defined() ? &tables.inv_freq : nullptr;
         Tensor q, k, v;
+        bool finished = false;      // norm, rotation and cache write made by the product's own kernel
         if (writes) {
             Tensor qkv = rt.ws.buf("attn_qkv", rt.dtype, {T, qw + 2 * kvw});
-            project(w_qkv_, qkv);
+            if (norm && fused::qkv_tail_ok(rt, static_cast<int>(T)) && T == batch.n_tokens &&
+                rt.ops.tiled_qkv_ok(head_dim_, inv_freq, tables.rotary_dim, tables.pairing, *cache.kv)) {
+                QkvTail tail;
+                tail.heads = heads_;
+                tail.kv_heads = kv_heads_;
+                tail.head_dim = head_dim_;
+                tail.q_weight = q_norm_ ? &q_norm_->view : nullptr;
+                tail.k_weight = k_norm_ ? &k_norm_->view : nullptr;
+                tail.eps = eps_;
+                tail.inv_freq = inv_freq;
+                tail.batch = &batch;
+                tail.kv = &*cache.kv;
+                fused::LinearExtras extras;
+                extras.qkv = &tail;
+                fused::norm_linear(rt, x, *norm, w_qkv_->view, qkv, Epilogue::Store, extras);
+                finished = true;
+            } else {
+                project(w_qkv_, qkv);
+            }
             q = qkv.cols(0, qw);
             k = qkv.cols(qw, kvw);
             v = qkv.cols(qw + kvw, kvw);
@@ -344,10 +365,10 @@ private:
             q = rt.ws.buf("attn_q", rt.dtype, {T, qw});
             project(w_q_, q);
         }
-        const PositionEncoding::Tables tables = position_->tables(rt);
-        rt.ops.qk_norm_rope_store(q, writes ? &k : nullptr, writes ? &v : nullptr, q_norm_ ? &q_norm_->view : nullptr,
-                                  k_norm_ ? &k_norm_->view : nullptr, eps_, tables.inv_freq.defined() ? &tables.inv_freq : nullptr,
-                                  tables.rotary_dim, tables.pairing, heads_, kv_heads_, head_dim_, batch, *cache.kv);
+        if (!finished)
+            rt.ops.qk_norm_rope_store(q, writes ? &k : nullptr, writes ? &v : nullptr, q_norm_ ? &q_norm_->view : nullptr,
+                                      k_norm_ ? &k_norm_->view : nullptr, eps_, inv_freq,
+                                      tables.rotary_dim, tables.pairing, heads_, kv_heads_, head_dim_, batch, *cache.kv);
         Tensor attended = rt.ws.buf("attn_out", rt.dtype, {T, qw});
         rt.ops.paged_attention(q, attended, heads_, kv_heads_, head_dim_, scale_, window_ ? *window_ : 0, batch, *cache.kv, rt.ws);
         return attended;

@@ -170,7 +170,10 @@ struct LinearExtras {
     int n_rows = -1;
     Tensor bias;
     const ConvOperands* conv = nullptr;
+    const QkvTail* qkv = nullptr;          // steps of many rows: what follows a q/k/v product, inside its kernel
 };
+// whether norm_linear would take a q/k/v tail for a step of this many rows
+bool qkv_tail_ok(const Runtime& rt, int rows);
 // out = epilogue(norm(h) w^T), the norm applied while the rows of h are read
 void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const Tensor& w, const Tensor& out,
                  Epilogue epilogue, const LinearExtras& extras = {});

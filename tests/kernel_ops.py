@@ -712,7 +712,7 @@ class HipOps:
         return int(self._lib("gemm_tiles").celeg_gemm_tiles_blocks(_c_int(rows), _c_int(n), _c_int(k)))
 
     def tiled_linear(self, a, w, out, *, epilogue="store", eps=0.0, stats=None, stat_blocks=0,
-                     bias=None, stats_out=None, out_bf16=None):
+                     bias=None, stats_out=None, out_bf16=None, qkv=None):
         """out = epilogue(scale * (a w^T) + bias) for many bfloat16 rows (any number; made for
         more than 64), inner size a multiple of 64, columns a multiple of 4.
 
@@ -723,7 +723,12 @@ class HipOps:
         [M, N]), "residual" (``out`` is the 32-bit stream, added to in place; ``out_bf16``
         receives its bfloat16 copy and ``stats_out`` [>= M, ``tiled_stat_blocks``] the partial
         sums of squares of the new rows; ``last_stat_blocks`` says how many a row), "swiglu"
-        (``w`` is [2N, K]: gate rows then up rows)."""
+        (``w`` is [2N, K]: gate rows then up rows).
+
+        ``qkv`` (with "store"): a dict ``heads, kv_heads, q_weight, k_weight, eps, cos_sin
+        ([positions, 32, 2] 32-bit or None), batch, kv``: the columns are heads of 64; query heads
+        are normalised, turned and stored to ``out``, key heads likewise and stored to their rows'
+        pages, value heads stored to the pages (what ``qk_norm_rope_store`` does behind a product)."""
         if epilogue not in ("store", "residual", "swiglu"):
             raise KernelError(f"tiled_linear: unknown epilogue '{epilogue}'")
         self._dev(a, "a", torch.bfloat16, contiguous=False); self._dev(w, "w", torch.bfloat16)
@@ -759,6 +764,26 @@ class HipOps:
         prm.eps = eps
         prm.M, prm.N, prm.K = M, N, K
         prm.out, prm.ldo = out.data_ptr(), ldo
+        code = {"store": 0, "residual": 2, "swiglu": 3}[epilogue]
+        if qkv is not None:
+            if epilogue != "store":
+                raise KernelError("tiled_linear: the q/k/v tail goes with the store epilogue")
+            kv, batch = qkv["kv"], qkv["batch"]
+            self._check_kv(kv, qkv["kv_heads"], 64, torch.bfloat16)
+            if N != (qkv["heads"] + 2 * qkv["kv_heads"]) * 64 or M != batch.n_tokens:
+                raise KernelError("tiled_linear: the q/k/v tail needs all heads of every row of the step")
+            prm.positions, prm.token_slot = _ptr(batch.positions).value, _ptr(batch.token_slot).value
+            prm.table, prm.table_stride = kv.table.data_ptr(), kv.table.stride(0)
+            prm.k_pool, prm.v_pool = kv.k.data_ptr(), kv.v.data_ptr()
+            prm.n_layers, prm.layer, prm.page_tokens = kv.n_layers, kv.layer, kv.page_tokens
+            prm.q_heads, prm.kv_heads = qkv["heads"], qkv["kv_heads"]
+            for name in ("q_weight", "k_weight", "cos_sin"):
+                t = qkv.get(name)
+                if t is not None:
+                    self._dev(t, name, torch.float32)
+                    setattr(prm, name, t.data_ptr())
+            prm.qk_eps = qkv.get("eps", 0.0)
+            code = 5
         if epilogue == "residual":
             self.last_stat_blocks = self.tiled_stat_blocks(M, N, K)
             if out_bf16 is not None:
@@ -775,9 +800,8 @@ class HipOps:
                 prm.stats_out, prm.stats_ld_out = stats_out.data_ptr(), stats_out.stride(0)
         elif out_bf16 is not None or stats_out is not None:
             raise KernelError("tiled_linear: out_bf16 and stats_out go with the residual epilogue")
-        code = self._lib("gemm_tiles").celeg_gemm_tiles(
-            ctypes.byref(prm), _c_int(self._EPILOGUES[epilogue]), self._stream())
-        self._check(code, f"tiled_linear ({epilogue})")
+        status = self._lib("gemm_tiles").celeg_gemm_tiles(ctypes.byref(prm), _c_int(code), self._stream())
+        self._check(status, f"tiled_linear ({epilogue})")
         return out
 
 
@@ -790,6 +814,11 @@ class _TileParams(ctypes.Structure):
         ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int),
         ("out", ctypes.c_void_p), ("ldo", ctypes.c_int), ("out_bf16", ctypes.c_void_p),
         ("ld_bf16", ctypes.c_int), ("stats_out", ctypes.c_void_p), ("stats_ld_out", ctypes.c_int),
+        ("positions", ctypes.c_void_p), ("token_slot", ctypes.c_void_p), ("table", ctypes.c_void_p),
+        ("table_stride", ctypes.c_int), ("k_pool", ctypes.c_void_p), ("v_pool", ctypes.c_void_p),
+        ("n_layers", ctypes.c_int), ("layer", ctypes.c_int), ("page_tokens", ctypes.c_int),
+        ("q_heads", ctypes.c_int), ("kv_heads", ctypes.c_int), ("q_weight", ctypes.c_void_p),
+        ("k_weight", ctypes.c_void_p), ("qk_eps", ctypes.c_float), ("cos_sin", ctypes.c_void_p),
     ]
 
 

@@ -36,7 +36,7 @@ def plain_logits(folder, name, storage):
     return _plain_cache[key]
 
 
-def run_mode(model_folders, name, dtype, mode, device, subset=None, gemm_backend="auto"):
+def run_mode(model_folders, name, dtype, mode, device, subset=None, gemm_backend="auto", knobs=None):
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders(name, storage, WEIGHT_STD)
@@ -48,6 +48,8 @@ def run_mode(model_folders, name, dtype, mode, device, subset=None, gemm_backend
     lm = load_model(folder, dtype=dtype, device=device, page_tokens=16,
                     n_pages=max_tokens // 16, max_requests=4,
                     max_batched_tokens=max(max_tokens, 64), gemm_backend=gemm_backend)
+    for knob, value in (knobs or {}).items():
+        lm.set_knob(knob, value)
     got = EngineDriver(lm).run(steps)
     ref = plain_logits(folder, name, storage)
     for rid in reqs:
@@ -73,6 +75,9 @@ def test_gpu_engine_with_tiled_products_matches_plain(model_folders, mode):
     beside single tokens."""
     lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles")
     assert lm.knobs()["use_tiled_products"] == 1 and lm.native.info["gemm_backend"] == "tiles"
+    assert lm.knobs()["use_qkv_tail"] == 1     # q/k norm, rotation and cache write inside the q/k/v product's kernel
+    # the same with the q/k norm, the rotation and the cache write as a kernel of their own
+    run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles", knobs={"use_qkv_tail": 0})
     # and the same configuration through the library's products
     lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="library")
     assert lm.knobs()["use_tiled_products"] == 0 and lm.native.info["gemm_backend"] == "library"

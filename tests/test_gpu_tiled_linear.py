@@ -155,3 +155,68 @@ def test_unsupported_sizes_are_refused(ops):
                          stats_out=torch.empty(80, 4, device=DEV))
     assert not ops.tiled_linear_ok(80, 64, 96)
     assert ops.tiled_linear_ok(80, 64, 128, 4608)
+
+
+# ---------------------------------------------------------------- the q/k/v product with its tail
+@pytest.mark.parametrize("heads,kv_heads,K,rotate,normed", [(16, 8, 1024, True, True), (6, 2, 192, True, False),
+                                                            (4, 4, 128, False, True), (3, 1, 64, True, True)])
+def test_qkv_product_with_norm_rotation_and_cache_write(ops, heads, kv_heads, K, rotate, normed):
+    """The product of the q, k and v projections that normalises and turns the query and key
+    heads and writes keys and values into the pages inside its own kernel, against the product
+    followed by qk_norm_rope_store: a step of three requests (portions that start at positions
+    0, 5 and 130, so that groups of four rows start on a multiple of four, in the middle of one,
+    and straddle the border between two requests; one request brings a single row).  Values must
+    come out bit for bit; queries and keys may differ by a rounding (the sums of squares are
+    added in another order)."""
+    import plain_lfm2 as plain
+    from celeg_amd.engine import StepEntry
+    from kernel_harness import build_batch, make_cache
+    hd, n_layers, layer, page_tokens = 64, 2, 1, 16
+    starts, lengths = [0, 5, 130, 77], [203, 131, 1, 66]
+    total = sum(lengths)
+    N = (heads + 2 * kv_heads) * hd
+    a = randn(total, K, seed=30, dtype=BF)
+    w = randn(N, K, seed=31, scale=0.05, dtype=BF)
+    bias = randn(N, seed=32) if not normed else None
+    qw = (1 + randn(hd, seed=33, scale=0.2)) if normed else None
+    kw = (1 + randn(hd, seed=34, scale=0.2)) if normed else None
+    inv_freq = torch.tensor(plain.rope_inverse_frequencies(10000.0, hd), dtype=torch.float64).float().to(DEV) if rotate else None
+    eps, blocks = 1e-5, 5
+    g = torch.Generator().manual_seed(35)
+    stats = (torch.rand(total, blocks, generator=g) * K / blocks).to(DEV)
+    results = []
+    for fused in (False, True):
+        cache = make_cache(kv_heads, hd, n_layers, BF, page_tokens=page_tokens, n_pages=64, max_context=512, slots=4)
+        kv = cache.layer_cache(layer).kv
+        slots = [cache.open() for _ in lengths]
+        entries = []
+        for slot, start, n in zip(slots, starts, lengths):
+            assert cache.prepare(slot, 0, start + n)
+            entries.append(StepEntry(slot, start, [0] * n))
+        batch, keep = build_batch(ops, cache, entries)
+        qkv = torch.zeros(total + 1, N, dtype=BF, device=DEV)
+        if fused:
+            cos_sin = ops._rope_table(inv_freq, kv.table.shape[1] * page_tokens) if rotate else None
+            ops.tiled_linear(a, w, qkv[:total], stats=stats, stat_blocks=blocks, eps=eps, bias=bias,
+                             qkv=dict(heads=heads, kv_heads=kv_heads, q_weight=qw, k_weight=kw, eps=1e-6, cos_sin=cos_sin,
+                                      batch=batch, kv=kv))
+        else:
+            ops.tiled_linear(a, w, qkv[:total], stats=stats, stat_blocks=blocks, eps=eps, bias=bias)
+            q, k, v = qkv[:total, :heads * hd], qkv[:total, heads * hd:(heads + kv_heads) * hd], qkv[:total, (heads + kv_heads) * hd:]
+            ops.qk_norm_rope_store(q, k, v, qw, kw, 1e-6, inv_freq, hd, heads, kv_heads, hd, batch, kv)
+        torch.cuda.synchronize()
+        assert float(qkv[total].abs().max()) == 0
+        table = kv.table.cpu()
+        pages = [int(table[slot, p]) for slot, start, n in zip(slots, starts, lengths)
+                 for p in range((start + n + page_tokens - 1) // page_tokens)]
+        others = sorted(set(range(kv.k.shape[0])) - set(pages))
+        assert float(kv.k[others].float().abs().max()) == 0 and float(kv.v[others].float().abs().max()) == 0
+        assert float(kv.k[:, 0].float().abs().max()) == 0          # the other layer's pages
+        results.append((qkv[:total, :heads * hd].float().clone(), kv.k[pages].float().clone(), kv.v[pages].clone()))
+    (qa, ka, va), (qb, kb, vb) = results
+    assert torch.equal(va, vb) and float(va.float().abs().max()) > 0
+    for x, y in ((qa, qb), (ka, kb)):
+        assert float(x.abs().max()) > 0
+        # a rounding of bfloat16 where the two differ at all
+        assert float(((x - y).abs() / (x.abs() + y.abs() + 1e-3)).max()) <= 2 ** -7
+        assert float((x != y).float().mean()) < 0.02
