@@ -340,14 +340,16 @@ __global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
         __syncthreads();
         buf ^= 1;
     }
-    // half 1 hands over: register by register, a lane to the same lane (the halves' wavefronts
-    // of one number own the same rows).  The staging buffers are free after the last barrier.
+    // the sets behind the first hand over: register by register, a lane to the same lane (the
+    // sets' wavefronts of one number own the same rows; a set that had no round hands over
+    // nothing: maximum -inf, sum and output 0).  The staging buffers are free after the last barrier.
+    constexpr int XSET = 4 * RT * (4 * DT + 2) * 64;      // floats a set hands over
     float* const xch = reinterpret_cast<float*>(smem) + wave * (RT * (4 * DT + 2) * 64) + lane;
     if (TURNS > 1 && total_rounds > 1) {
-        if (half == 1 && wave_active) {
+        if (half >= 1 && wave_active) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                float* x = xch + rt * (4 * DT + 2) * 64;
+                float* x = xch + (half - 1) * XSET + rt * (4 * DT + 2) * 64;
                 x[0] = m[rt];
                 x[64] = l[rt];
 #pragma unroll
@@ -358,16 +360,19 @@ __global__ __launch_bounds__(256 * NH) void attention_rows_kernel(
         }
         __syncthreads();
     }
-    if ((TURNS > 1 && half == 1) || !wave_active) return;
+    if ((TURNS > 1 && half >= 1) || !wave_active) return;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        if (TURNS > 1 && total_rounds > 1) {
-            const float* x = xch + rt * (4 * DT + 2) * 64;
+#pragma unroll
+        for (int other = 1; other < TURNS; ++other) {
+            if (total_rounds <= 1) break;
+            const float* x = xch + (other - 1) * XSET + rt * (4 * DT + 2) * 64;
             const float m1 = x[0];
             const float m_new = fmaxf(m[rt], m1);
             const float m_use = m_new == neg_inf ? 0.f : m_new;
             const float a0 = __builtin_amdgcn_exp2f(m[rt] - m_use), a1 = __builtin_amdgcn_exp2f(m1 - m_use);
             l[rt] = l[rt] * a0 + x[64] * a1;
+            m[rt] = m_new;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -399,8 +404,9 @@ extern "C" void celeg_attention_rows_pages_in_lds(int entries) {
 // LDS bytes that a launch with these sizes asks for (what the host-side check of the limit
 // of 160 KB works with): form 1 or 2 = sets of staging buffers.
 extern "C" long long celeg_attention_rows_lds_bytes(int head_dim, int sets, int table_stride) {
-    return static_cast<long long>(sets) * 2 * (64 * (head_dim + 8) + head_dim * (64 + 8)) * 2 +
-           static_cast<long long>(min(table_stride + 8, ROWS_MAX_PAGES_IN_LDS)) * 4;
+    const long long staging = static_cast<long long>(sets) * 2 * (64 * (head_dim + 8) + head_dim * (64 + 8)) * 2;
+    const long long room = staging < 160 * 1024 ? (160 * 1024 - staging) / 4 : 0;
+    return staging + min(static_cast<long long>(min(table_stride + 8, ROWS_MAX_PAGES_IN_LDS)), room) * 4;
 }
 
 template <int HD, int RT, int NH, bool SHARE>
@@ -412,9 +418,13 @@ static int launch_attention_rows(
     // staging buffers, and a tile's pages with room for a round's worth behind the last: the
     // whole of a request's block-table row where that is at most ROWS_MAX_PAGES_IN_LDS entries
     // (16 KB; with the largest staging buffers, 143,360 bytes, still inside 160 KB)
-    const int pages_room = min(table_stride + 8, ROWS_MAX_PAGES_IN_LDS);
-    const size_t lds = (SHARE ? 1 : NH) * 2 * (64 * (HD + 8) + HD * (64 + 8)) * sizeof(bf16) +
-                       static_cast<size_t>(pages_room) * sizeof(int);
+    const size_t staging = static_cast<size_t>(SHARE ? 1 : NH) * 2 * (64 * (HD + 8) + HD * (64 + 8)) * sizeof(bf16);
+    const int pages_room = min(min(table_stride + 8, ROWS_MAX_PAGES_IN_LDS),
+                               staging < 160 * 1024 ? static_cast<int>((160 * 1024 - staging) / sizeof(int)) : 0);
+    const size_t lds = staging + static_cast<size_t>(pages_room) * sizeof(int);
+    static_assert(SHARE || static_cast<size_t>(NH - 1) * 4 * RT * (4 * (HD / 16) + 2) * 64 * sizeof(float) <=
+                               static_cast<size_t>(NH) * 2 * (64 * (HD + 8) + HD * (64 + 8)) * sizeof(bf16),
+                  "what the sets hand over fits the staging buffers");
     if (lds > 160 * 1024) return static_cast<int>(hipErrorInvalidValue);
     // the kernel multiplies page numbers by the elements of a page in 32 x 32 -> 64 bits
     if (static_cast<size_t>(n_layers) * kv_heads * page_tokens * HD >= (size_t{1} << 31))
@@ -444,7 +454,12 @@ static int launch_attention_rows(
 // rounds of keys of its tile for one query head; 2, two such sets take the rounds in turn and
 // join at the end (more workgroups in flight and half as long a way for a tile with many
 // keys: for few rows); 3, two sets take a query head each of those that share a key/value
-// head, and the staged keys and values with it (half the traffic: for many rows).  0 leaves
+// head, and the staged keys and values with it (half the traffic: for many rows); 4, four
+// sets take the rounds in turn (tiles of 64 rows, heads of 32 or 64; never chosen here: a
+// prompt of 2,048 tokens gives about as many tiles as the chip holds workgroups, so its time
+// is that of the tile with the most rounds, which four sets walk in half as many steps as
+// two, but one workgroup of 16 wavefronts a compute unit instead of two of 8 made the six
+// attention layers of such a prefill 40 us slower, not faster).  0 leaves
 // a choice to this function, which then goes by the number of rows and by context_hint, the
 // longest context among the step's requests (0: not known).
 extern "C" int celeg_attention_rows_bf16(
@@ -472,7 +487,8 @@ extern "C" int celeg_attention_rows_bf16(
         const long long shared = static_cast<long long>(n_tokens / rows_per_tile + n_seqs) * kv_heads * ((group + 1) / 2);
         form = group >= 2 && shared >= 1024 ? 3 : 2;
     }
-    if (form < 1 || form > 3) return static_cast<int>(hipErrorInvalidValue);
+    if (form < 1 || form > 4) return static_cast<int>(hipErrorInvalidValue);
+    if (form == 4 && (rows_per_tile != 64 || head_dim > 64)) return static_cast<int>(hipErrorInvalidValue);
 #define CELEG_ROWS_ARGS                                                                            \
     q, ldq, k_pool, v_pool, table, table_stride, cu_seqlens, seq_slot, seq_start, n_seqs, n_tokens, \
         out, ldo, q_heads, kv_heads, page_tokens, n_layers, layer, scale, window, stream
@@ -481,6 +497,9 @@ extern "C" int celeg_attention_rows_bf16(
      : form == 2 ? launch_attention_rows<HD_, RT_, 2, false>(CELEG_ROWS_ARGS)                 \
                  : launch_attention_rows<HD_, RT_, 2, true>(CELEG_ROWS_ARGS))
 #define CELEG_ROWS(HD_) return rows_per_tile == 64 ? CELEG_ROWS_RT(HD_, 1) : CELEG_ROWS_RT(HD_, 2)
+    if (form == 4)
+        return head_dim == 32 ? launch_attention_rows<32, 1, 4, false>(CELEG_ROWS_ARGS)
+                              : launch_attention_rows<64, 1, 4, false>(CELEG_ROWS_ARGS);
     switch (head_dim) {
         case 32: CELEG_ROWS(32);
         case 64: CELEG_ROWS(64);

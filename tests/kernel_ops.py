@@ -49,7 +49,7 @@ class HipOps:
         self._device_index = torch.device(device).index if torch.device(device).index is not None \
             else torch.cuda.current_device()
         self.attention_rows_per_tile = 0     # 0: the kernel chooses; 64 or 128 to force
-        self.attention_rows_form = 0         # 0: the kernel chooses; 1, 2 or 3 to force (see attention_fast.hip)
+        self.attention_rows_form = 0         # 0: the kernel chooses; 1 to 4 to force (see attention_fast.hip)
         # decode attention over few requests: contexts of up to this many rounds of 64 keys are
         # cut into parts of 1 round, up to that many into parts of 4, longer ones into parts of 16
         self.decode_part_thresholds = (64, 256)

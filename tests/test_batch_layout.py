@@ -60,7 +60,7 @@ def test_attention_rows_kernel_fits_lds_at_the_longest_context():
     lib = ctypes.CDLL(library.ensure_built())
     lib.celeg_attention_rows_lds_bytes.restype = ctypes.c_longlong
     for head_dim in (32, 64, 96, 128):
-        for sets in (1, 2):
+        for sets in (1, 2) + ((4,) if head_dim <= 64 else ()):      # (four sets: heads up to 64)
             for stride in (8, 256, 4096, 8000, 1 << 20):
                 need = lib.celeg_attention_rows_lds_bytes(head_dim, sets, stride)
                 assert 0 < need <= 160 * 1024, (head_dim, sets, stride, need)

@@ -558,7 +558,7 @@ def test_attention_window_fast_kernels(ops):
 
 
 @pytest.mark.parametrize("rows_per_tile", [64, 128])
-@pytest.mark.parametrize("form", [1, 2, 3])
+@pytest.mark.parametrize("form", [1, 2, 3, 4])
 @pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [
     (4, 2, 64, 16), (2, 1, 128, 32), (3, 3, 96, 16), (4, 1, 32, 64), (2, 2, 64, 128), (6, 2, 64, 16),
     (3, 1, 96, 32)])
@@ -567,8 +567,19 @@ def test_attention_rows_tiles_and_forms(ops, rows_per_tile, form, heads, kv_head
     so that the wavefronts that take the rounds in turn get equal and unequal shares),
     continued at a position inside a tile, at either tile size, with the rounds of keys taken
     by one set of wavefronts, shared between two, or by two sets that each take a query head
-    of a group (groups of 1, 2, 3 and 4 heads); then the same with a window that ends inside a
-    round of keys.  Pages shorter and longer than a round."""
+    of a group (groups of 1, 2, 3 and 4 heads), or shared between four sets (tiles of 64 rows and
+    heads up to 64 only: some sets then have no round at all in the first tiles); then the same
+    with a window that ends inside a round of keys.  Pages shorter and longer than a round."""
+    if form == 4 and (rows_per_tile != 64 or head_dim > 64):
+        from kernel_ops import KernelError
+        ops.attention_rows_per_tile, ops.attention_rows_form = rows_per_tile, form
+        try:
+            with pytest.raises(KernelError):
+                attention_case(ops, torch.bfloat16, heads, kv_heads, head_dim, lengths=[130], cuts=[130],
+                               page_tokens=page_tokens)
+        finally:
+            ops.attention_rows_per_tile = ops.attention_rows_form = 0
+        return
     ops.attention_rows_per_tile = rows_per_tile
     ops.attention_rows_form = form
     try:
