@@ -6,7 +6,7 @@ import torch
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 BF = torch.bfloat16
-N_SHAPES = 18
+N_SHAPES = 19
 
 
 @pytest.fixture(scope="module")
@@ -103,7 +103,7 @@ def test_residual_adds_in_place_refreshes_the_copy_and_leaves_partial_sums(ops, 
 
 
 @pytest.mark.parametrize("M,N,K,blocks", [(2000, 1024, 2304, 16), (2000, 1024, 1024, 8), (2048, 2048, 1024, 16),
-                                          (2048, 3072, 1024, 24)])
+                                          (2048, 3072, 1024, 16), (1024, 3072, 1024, 24)])
 def test_the_shapes_chosen_for_a_prefill(ops, M, N, K, blocks):
     """What the choice of shape gives at the sizes of a prefill of some 2,000 rows (few weight
     rows with a long and a short K, q/k/v, in_proj), against torch, with the residual epilogue;
