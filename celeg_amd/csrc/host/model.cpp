@@ -521,7 +521,7 @@ std::unique_ptr<LoadedModel> load_model(const std::string& model_dir, const Load
     CELEG_HIP(hipStreamCreate(&lm->stream));
     lm->rt = std::make_unique<Runtime>(dtype, lm->stream);
     // "auto": measured on 2,048 rows, whole prefill.  At a width of 1,024 (K of most products) the
-    // tiled products with their folded norms and SwiGLU take 2.40 ms against 2.77 ms through the
+    // tiled products with their folded norms and SwiGLU take 2.33 ms against 2.72 ms through the
     // library and the separate kernels it needs; at 2,048 the library's products run at 1.2
     // PFLOP/s and win (5.5 against 6.2 ms, 9.3 against 11.0 ms at the two larger shapes).
     lm->rt->use_tiled_products = options.gemm_backend == "tiles" ||
