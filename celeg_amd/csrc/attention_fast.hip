@@ -581,14 +581,101 @@ __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
 //   O^T[dim, head] = V^T P : P's operand wants 8 keys a lane, which are rows 4q..4q+3 of two
 //   tiles: tile 2j holds keys 32j + 8*(row/4) + row%4, tile 2j+1 those + 4, so that a lane's
 //   eight p are eight keys in a row and V (stored [dim][key] in a page) is read 16 bytes a lane.
-template <int HD, int WAVES, bool SPLIT>
+// The step's own token where its key and value are not in the cache yet (k set): q and k come
+// as the q/k/v product left them; the kernel then normalises and turns the query heads itself,
+// takes the rounds of keys up to the position before the token's, and the workgroup (and
+// wavefront) whose part holds the token's position prepares the new key, adds it and the new
+// value to its running sums as one more key, and writes both into the request's page: what
+// qk_norm_rope_store does as a kernel of its own before the attention.
+struct DecodeFresh {
+    const bf16* k;            // [rows, ldk] or null: the cache holds the step's keys and values already
+    const bf16* v;            // [rows, ldv]
+    int ldk, ldv;
+    const float* q_weight;    // [HD] or null: no norm
+    const float* k_weight;
+    float eps;
+    const float* cos_sin;     // [positions, HD / 2, 2] or null: no rotation
+    bf16* k_pool;             // the pools again, to write to
+    bf16* v_pool;
+};
+
+// A head's HD values spread over the four lanes qd = 0..3 of a head's lane group as the matrix
+// instruction wants them (x[s][e] is dimension 32 s + 8 qd + e): norm (weight w in the same
+// layout; null: none) and rotation by split halves (cs: (cos, sin) of pair 32 s + 8 qd + e for
+// s < KS / 2; null: none), as qk_norm_rope_store makes them.
+// What decode_prepare_head needs from memory, asked for early: the weight at the lane's
+// dimensions and the (cos, sin) of its pairs.
+template <int KS>
+struct DecodeHeadOperands {
+    floatx4_t w[KS][2];
+    floatx4_t cs[KS / 2][4];
+};
+template <int KS>
+__device__ __forceinline__ void decode_head_operands(DecodeHeadOperands<KS>& o, const float* __restrict__ w,
+                                                     const float* __restrict__ cs, const int qd) {
+    if (w) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            o.w[s][0] = *reinterpret_cast<const floatx4_t*>(w + 32 * s + 8 * qd);
+            o.w[s][1] = *reinterpret_cast<const floatx4_t*>(w + 32 * s + 8 * qd + 4);
+        }
+    }
+    if (cs) {
+#pragma unroll
+        for (int s = 0; s < KS / 2; ++s)
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) o.cs[s][e4] = *reinterpret_cast<const floatx4_t*>(cs + (32 * s + 8 * qd) * 2 + 4 * e4);
+    }
+}
+
+template <int KS>
+__device__ __forceinline__ void decode_prepare_head(float (&x)[KS][8], const bool normed, const bool rotate,
+                                                    const floatx4_t (&w)[KS][2], const floatx4_t (&cs)[KS / 2][4], const float eps) {
+    constexpr int HD = 32 * KS;
+    if (normed) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ssq += x[s][e] * x[s][e];
+        ssq += __shfl_xor(ssq, 16, 64);
+        ssq += __shfl_xor(ssq, 32, 64);
+        const float inv = 1.0f / sqrtf(ssq / static_cast<float>(HD) + eps);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                x[s][e] = x[s][e] * inv * w[s][0][e];
+                x[s][4 + e] = x[s][4 + e] * inv * w[s][1][e];
+            }
+        }
+    }
+    if (rotate) {
+#pragma unroll
+        for (int s = 0; s < KS / 2; ++s) {
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {          // two pairs a load
+                const floatx4_t t = cs[s][e4];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int e = 2 * e4 + h;
+                    const float a = x[s][e], b = x[s + KS / 2][e];
+                    x[s][e] = a * t[2 * h] - b * t[2 * h + 1];
+                    x[s + KS / 2][e] = b * t[2 * h] + a * t[2 * h + 1];
+                }
+            }
+        }
+    }
+}
+
+template <int HD, int WAVES, bool SPLIT, bool FRESH>
 __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
     const int* __restrict__ token_slot, const int* __restrict__ positions, bf16* __restrict__ out,
     int ldo, int kv_heads, int group, int page_tokens, int page_shift, int n_layers, int layer,
     float scale, int window, float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
-    int split_rounds) {
+    int split_rounds, const DecodeFresh fresh) {
     constexpr int KS = HD / 32;   // steps of 32 dims in q.k
     constexpr int DT = HD / 16;   // 16-dim tiles of the output
     extern __shared__ float smem_heads[];
@@ -612,6 +699,27 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
 #pragma unroll
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8_t*>(qrow + s * 32);
     }
+    // The query heads as the product left them: norm and rotation here, once the first round's
+    // keys have been asked for (what that needs from memory is asked for now).
+    const float* const fresh_cs = FRESH && fresh.cos_sin ? fresh.cos_sin + static_cast<size_t>(pos) * HD : nullptr;
+    DecodeHeadOperands<KS> q_operands;
+    if (FRESH) decode_head_operands<KS>(q_operands, fresh.q_weight, fresh_cs, qd);
+    bool q_ready = !FRESH;
+    auto prepare_q = [&]() {
+        float x[KS][8];
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[s][e] = static_cast<float>(qf[s][e]);
+        decode_prepare_head<KS>(x, fresh.q_weight != nullptr, fresh_cs != nullptr, q_operands.w, q_operands.cs, fresh.eps);
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<__bf16>(x[s][e]);
+        q_ready = true;
+    };
+    // (with a fresh token the rounds end at the position before it)
+    const int last_key = FRESH ? pos - 1 : pos;
     float m_run = -INFINITY, l_run = 0.f;
     floatx4_t o[DT];
 #pragma unroll
@@ -620,13 +728,30 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     // the workgroup's rounds: all of the request's, or (SPLIT) part blockIdx.z of them; its
     // wavefronts take them in turn
     const int r_begin = SPLIT ? max(lo / DEC_KEYS, static_cast<int>(blockIdx.z) * split_rounds) : lo / DEC_KEYS;
-    const int r_end = SPLIT ? min(pos / DEC_KEYS, static_cast<int>(blockIdx.z) * split_rounds + split_rounds - 1)
-                            : pos / DEC_KEYS;
-    if (SPLIT && r_begin > r_end) return;     // the whole workgroup
+    const int last_round = last_key < 0 ? -1 : last_key / DEC_KEYS;
+    const int r_end = SPLIT ? min(last_round, static_cast<int>(blockIdx.z) * split_rounds + split_rounds - 1) : last_round;
+    // the fresh token belongs to the part that holds its position (which may hold no other key)
+    const bool adds_fresh = FRESH && wave == 0 && (!SPLIT || static_cast<int>(blockIdx.z) == pos / DEC_KEYS / split_rounds);
+    const bool part_of_fresh = FRESH && (!SPLIT || static_cast<int>(blockIdx.z) == pos / DEC_KEYS / split_rounds);
+    if (SPLIT && r_begin > r_end && !part_of_fresh) return;     // the whole workgroup
+    // the new key and value of the wavefront that adds them: asked for ahead of the rounds
+    bf16x8_t k_raw[KS];
+    bf16x4_t v_raw[DT];
+    DecodeHeadOperands<KS> k_operands;
+    if (adds_fresh) {
+        const bf16* krow = fresh.k + static_cast<size_t>(t) * fresh.ldk + static_cast<size_t>(kvh) * HD + qd * 8;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) k_raw[s] = *reinterpret_cast<const bf16x8_t*>(krow + s * 32);
+        const bf16* vrow = fresh.v + static_cast<size_t>(t) * fresh.ldv + static_cast<size_t>(kvh) * HD + 4 * qd;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v_raw[dt] = *reinterpret_cast<const bf16x4_t*>(vrow + 16 * dt);
+        decode_head_operands<KS>(k_operands, fresh.k_weight, nullptr, qd);
+    }
     // (a part of one round: the stride tells the compiler that the loop runs once)
     for (int r = r_begin + wave; r <= r_end; r += (SPLIT && WAVES == 1) ? (1 << 30) : WAVES) {
         const int kb = r * DEC_KEYS;
-        const int k_lo = max(lo, kb), k_hi = min(pos, kb + DEC_KEYS - 1);
+        const int k_lo = max(lo, kb), k_hi = min(last_key, kb + DEC_KEYS - 1);
+        if (k_lo > k_hi) continue;            // (a window of one key with a fresh token: nothing before it)
         const int first_page = kb >> page_shift, last_page = k_hi >> page_shift;
         const int my_page = pages[min(first_page + lane, last_page)];
         bf16x8_t kf[4][KS], vf[DT][2];
@@ -650,6 +775,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             for (int dt = 0; dt < DT; ++dt)
                 vf[dt][j] = *reinterpret_cast<const bf16x8_t*>(vbase + static_cast<size_t>(16 * dt + c) * page_tokens);
         }
+        if (FRESH && !q_ready) prepare_q();   // (the round's keys and values are on their way)
         float sc[4][4];
         float mx = -INFINITY;
 #pragma unroll
@@ -695,6 +821,51 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt][j], pb, o[dt], 0, 0, 0);
+        }
+    }
+    if (adds_fresh) {
+        if (!q_ready) prepare_q();            // (a part that holds no other key)
+        // the new key in the layout of a query head (every head's lanes prepare it alike)
+        float kx[KS][8];
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) kx[s][e] = static_cast<float>(k_raw[s][e]);
+        decode_prepare_head<KS>(kx, fresh.k_weight != nullptr, fresh_cs != nullptr, k_operands.w, q_operands.cs, fresh.eps);
+        const int page = pages[pos >> page_shift];
+        const size_t block = kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD);
+        float dot = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            bf16x8_t kb16;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                kb16[e] = static_cast<__bf16>(kx[s][e]);
+                dot = fmaf(static_cast<float>(qf[s][e]), static_cast<float>(kb16[e]), dot);
+            }
+            if (chunk == 0 && c == 0)        // one copy into the page
+                *reinterpret_cast<bf16x8_t*>(fresh.k_pool + block + static_cast<size_t>(pos & page_mask) * HD + s * 32 + qd * 8) = kb16;
+        }
+        dot += __shfl_xor(dot, 16, 64);
+        dot += __shfl_xor(dot, 32, 64);
+        const float s_new = dot * scale;
+        const float m_new = fmaxf(m_run, s_new);
+        const float keep = expf(m_run - m_new);         // e^(-inf) = 0 where the part holds no other key
+        const float p_exact = expf(s_new - m_new);
+        const float p_new = static_cast<float>(static_cast<__bf16>(p_exact));     // as the rounds round theirs for the output
+        l_run = l_run * keep + p_exact;
+        m_run = m_new;
+        // the new value: this lane's dimensions of the output, 16 dt + 4 qd + i
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x4_t vv = v_raw[dt];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[dt][i] = o[dt][i] * keep + p_new * static_cast<float>(vv[i]);
+            if (chunk == 0 && c == 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    reinterpret_cast<__bf16*>(fresh.v_pool)[block + static_cast<size_t>(16 * dt + 4 * qd + i) * page_tokens + (pos & page_mask)] = vv[i];
+            }
         }
     }
     if (SPLIT && WAVES == 1) {
@@ -744,21 +915,25 @@ static int launch_decode_heads(const void* q, int ldq, const void* k_pool, const
                                const int* table, int table_stride, const int* token_slot,
                                const int* positions, void* out, int ldo, int n_rows, int kv_heads,
                                int group, int page_tokens, int page_shift, int n_layers, int layer,
-                               float scale, int window, hipStream_t stream) {
+                               float scale, int window, const DecodeFresh& fresh, hipStream_t stream) {
     const int chunks = (group + 15) / 16;
     const size_t lds = static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, false>),
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, false, false>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (err == hipSuccess)
+            err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, false, true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (err != hipSuccess) return static_cast<int>(err);
         raised = true;
     }
-    hipLaunchKernelGGL((attention_decode_heads_kernel<HD, WAVES, false>), dim3(kv_heads * chunks, n_rows),
+    auto kernel = fresh.k ? &attention_decode_heads_kernel<HD, WAVES, false, true> : &attention_decode_heads_kernel<HD, WAVES, false, false>;
+    hipLaunchKernelGGL(kernel, dim3(kv_heads * chunks, n_rows),
                        dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
                        table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
-                       group, page_tokens, page_shift, n_layers, layer, scale, window, nullptr, nullptr, 0, 1);
+                       group, page_tokens, page_shift, n_layers, layer, scale, window, nullptr, nullptr, 0, 1, fresh);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -768,31 +943,35 @@ static int launch_decode_parts(const void* q, int ldq, const void* k_pool, const
                                const int* positions, float* ws_o, float* ws_ml, int n_splits, void* out,
                                int ldo, int n_rows, int kv_heads, int group, int page_tokens,
                                int page_shift, int n_layers, int layer, float scale, int window,
-                               int split_rounds, int n_parts, hipStream_t stream) {
+                               int split_rounds, int n_parts, const DecodeFresh& fresh, hipStream_t stream) {
     const int chunks = (group + 15) / 16;
     const size_t lds = WAVES == 1 ? 0 : static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, true>),
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, true, false>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (err == hipSuccess)
+            err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, true, true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (err != hipSuccess) return static_cast<int>(err);
         raised = true;
     }
-    hipLaunchKernelGGL((attention_decode_heads_kernel<HD, WAVES, true>), dim3(kv_heads * chunks, n_rows, n_parts),
+    auto kernel = fresh.k ? &attention_decode_heads_kernel<HD, WAVES, true, true> : &attention_decode_heads_kernel<HD, WAVES, true, false>;
+    hipLaunchKernelGGL(kernel, dim3(kv_heads * chunks, n_rows, n_parts),
                        dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
                        table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
                        group, page_tokens, page_shift, n_layers, layer, scale, window, ws_o, ws_ml,
-                       n_splits, split_rounds);
+                       n_splits, split_rounds, fresh);
     return 0;
 }
 
-extern "C" int celeg_attention_decode_bf16(
+static int attention_decode(
     const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
     int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
     int n_splits, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
     int head_dim, int page_tokens, int n_layers, int layer, float scale, int window, int whole,
-    int split_rounds, int n_parts, hipStream_t stream) {
+    int split_rounds, int n_parts, const DecodeFresh& fresh, hipStream_t stream) {
     if (n_rows <= 0) return 0;
     const int group = q_heads / kv_heads;
     if (q_heads % kv_heads || page_tokens < 16 || (page_tokens & (page_tokens - 1)) || n_splits <= 0 ||
@@ -813,15 +992,15 @@ extern "C" int celeg_attention_decode_bf16(
         if (head_dim == 64 && kv_heads * chunks * n_rows >= 512)
             return launch_decode_heads<64, 8>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
                                               out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
-                                              n_layers, layer, scale, window, stream);
+                                              n_layers, layer, scale, window, fresh, stream);
         if (head_dim == 64)
             return launch_decode_heads<64, 16>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
                                            out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
-                                           n_layers, layer, scale, window, stream);
+                                           n_layers, layer, scale, window, fresh, stream);
         if (head_dim == 128)
             return launch_decode_heads<128, 8>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
                                             out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
-                                            n_layers, layer, scale, window, stream);
+                                            n_layers, layer, scale, window, fresh, stream);
         return static_cast<int>(hipErrorInvalidValue);
     }
     // Parts of split_rounds rounds of 64 keys (1, 4 or 16), one workgroup each with a wavefront per
@@ -833,7 +1012,7 @@ extern "C" int celeg_attention_decode_bf16(
 #define CELEG_SPLIT_ARGS                                                                           \
     q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions, ws_o, ws_ml, n_splits, out, \
         ldo, n_rows, kv_heads, group, page_tokens, page_shift, n_layers, layer, scale, window,     \
-        split_rounds, n_parts, stream
+        split_rounds, n_parts, fresh, stream
 #define CELEG_SPLIT_HEADS(HD_, MOST_)                                                              \
     {                                                                                              \
         const int code = split_rounds == 1 ? launch_decode_parts<HD_, 1>(CELEG_SPLIT_ARGS)         \
@@ -850,6 +1029,48 @@ extern "C" int celeg_attention_decode_bf16(
 #undef CELEG_SPLIT_ARGS
 #undef CELEG_SPLIT_HEADS
     return CELEG_LAUNCH_RESULT();
+}
+
+extern "C" int celeg_attention_decode_bf16(
+    const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table,
+    int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
+    int n_splits, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
+    int head_dim, int page_tokens, int n_layers, int layer, float scale, int window, int whole,
+    int split_rounds, int n_parts, hipStream_t stream) {
+    return attention_decode(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions, ws_o, ws_ml, n_splits, out,
+                            ldo, n_rows, q_heads, kv_heads, head_dim, page_tokens, n_layers, layer, scale, window, whole,
+                            split_rounds, n_parts, DecodeFresh{}, stream);
+}
+
+// The same for a step whose own keys and values are not in the cache yet: q, k and v as the
+// q/k/v product left them ([rows, ld..]); the kernel normalises (weights of head_dim 32-bit
+// values, or null) and turns (cos_sin [positions, head_dim / 2, 2], or null) the query heads
+// and the new key itself and writes the new key and value into the pages (DecodeFresh).
+extern "C" int celeg_attention_decode_fresh_bf16(
+    const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* q_weight,
+    const float* k_weight, float eps, const float* cos_sin, void* k_pool, void* v_pool, const int* table,
+    int table_stride, const int* token_slot, const int* positions, float* ws_o, float* ws_ml,
+    int n_splits, void* out, int ldo, int n_rows, int q_heads, int kv_heads,
+    int head_dim, int page_tokens, int n_layers, int layer, float scale, int window, int whole,
+    int split_rounds, int n_parts, hipStream_t stream) {
+    const auto misaligned = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+    if (!k || !v || (ldk % 8) || (ldv % 4) || misaligned(k) || (reinterpret_cast<uintptr_t>(v) & 7) || misaligned(q_weight) ||
+        misaligned(k_weight) || misaligned(cos_sin) || misaligned(k_pool))
+        return static_cast<int>(hipErrorInvalidValue);
+    DecodeFresh fresh{};
+    fresh.k = static_cast<const bf16*>(k);
+    fresh.v = static_cast<const bf16*>(v);
+    fresh.ldk = ldk;
+    fresh.ldv = ldv;
+    fresh.q_weight = q_weight;
+    fresh.k_weight = k_weight;
+    fresh.eps = eps;
+    fresh.cos_sin = cos_sin;
+    fresh.k_pool = static_cast<bf16*>(k_pool);
+    fresh.v_pool = static_cast<bf16*>(v_pool);
+    return attention_decode(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions, ws_o, ws_ml, n_splits, out,
+                            ldo, n_rows, q_heads, kv_heads, head_dim, page_tokens, n_layers, layer, scale, window, whole,
+                            split_rounds, n_parts, fresh, stream);
 }
 
 // ================================================================ without allocation

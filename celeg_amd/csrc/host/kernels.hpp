@@ -57,6 +57,13 @@ int celeg_attention_decode_bf16(const void* q, int ldq, const void* k_pool, cons
                                 float* ws_ml, int n_splits, void* out, int ldo, int n_rows, int q_heads,
                                 int kv_heads, int head_dim, int page_tokens, int n_layers, int layer, float scale,
                                 int window, int whole, int split_rounds, int n_parts, hipStream_t stream);
+int celeg_attention_decode_fresh_bf16(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv,
+                                      const float* q_weight, const float* k_weight, float eps, const float* cos_sin,
+                                      void* k_pool, void* v_pool, const int* table, int table_stride, const int* token_slot,
+                                      const int* positions, float* ws_o, float* ws_ml, int n_splits, void* out, int ldo,
+                                      int n_rows, int q_heads, int kv_heads, int head_dim, int page_tokens, int n_layers,
+                                      int layer, float scale, int window, int whole, int split_rounds, int n_parts,
+                                      hipStream_t stream);
 // sampling.hip
 int celeg_argmax_rows(const float* logits, int ld, int rows, int vocab, const float* fparams, const int* iparams,
                       uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens,

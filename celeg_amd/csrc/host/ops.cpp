@@ -287,8 +287,30 @@ void Ops::qk_norm_rope_store(const Tensor& q, const Tensor* k, const Tensor* v, 
                      heads, kv_heads, head_dim, store ? 1 : 0, stream), "qk_norm_rope_store");
 }
 
+// The conditions under which paged_attention hands a decode-only step to the kernels for single
+// rows, and those can prepare the step's own keys and values (the rotation: none, or of the whole
+// head by split halves from the table).
+bool Ops::attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, int rotary_dim, int pairing, const StepBatch& batch,
+                             const KVView& kv, DType dtype) const {
+    if (!use_fresh_decode || dtype != DType::BF16 || kv.dtype != DType::BF16 || attention_general) return false;
+    if (kv.page_tokens < 16 || (kv.page_tokens & (kv.page_tokens - 1))) return false;
+    if ((head_dim != 64 && head_dim != 128) || kv.head_dim != head_dim || (kv.v_head_dim && kv.v_head_dim != head_dim)) return false;
+    if (!batch.decode_only || batch.n_seqs != batch.n_tokens) return false;
+    // Only where the kernel that takes a round of 64 keys a workgroup runs (few requests, contexts up
+    // to 4,096 tokens, heads of 64): the forms with many wavefronts a workgroup have no registers
+    // left for the new token's operands.
+    if (head_dim != 64 || attention_decode_whole > 0) return false;
+    const int max_context = kv.table_stride * kv.page_tokens;
+    const int hint = batch.context_hint();
+    const int rounds = ((hint ? std::min(hint, max_context) : max_context) + 63) / 64;
+    if (rounds > decode_part_thresholds[0]) return false;
+    const int chunks = (heads / kv.kv_heads + 15) / 16;
+    if (attention_decode_whole < 0 && static_cast<long long>(kv.kv_heads) * chunks * batch.n_tokens >= 192) return false;
+    return !inv_freq || (rotary_dim == head_dim && pairing == 0 && use_rope_table);
+}
+
 void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
-                          int window, const StepBatch& batch, const KVView& kv, Workspace& ws) {
+                          int window, const StepBatch& batch, const KVView& kv, Workspace& ws, const FreshKV* fresh) {
     dev(q, "q");
     dev(out, "out", q.dtype);
     const long long T = q.shape[0], qw = static_cast<long long>(heads) * head_dim;
@@ -302,9 +324,10 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
         (kv.page_tokens & (kv.page_tokens - 1)) == 0 && ldq % 8 == 0) {
         const bool decode_hd = head_dim == 64 || head_dim == 128;
         if (batch.decode_only && decode_hd && batch.n_seqs == T) {
-            attention_decode(q, out, heads, kv_heads, head_dim, scale, window, batch, kv, static_cast<int>(T), ws);
+            attention_decode(q, out, heads, kv_heads, head_dim, scale, window, batch, kv, static_cast<int>(T), ws, fresh);
             return;
         }
+        need(!fresh, "paged_attention: fresh keys and values go with decode-only steps");
         if (head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128) {
             // entries of one token lie first: they go to the kernel for single rows (a tile of
             // the rows kernel would hold one row), the portions to the rows kernel
@@ -320,6 +343,7 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
             return;
         }
     }
+    need(!fresh, "paged_attention: fresh keys and values go with the kernels for single rows");
     kernel_check(celeg_paged_attention(q.data, ldq, kv.k, kv.v, dt(q, "q"), kv.table, kv.table_stride, batch.token_slot,
                                        batch.positions, out.data, static_cast<int>(qw), static_cast<int>(T), heads,
                                        kv_heads, head_dim, kv.page_tokens, kv.n_layers, kv.layer, scale, window, stream),
@@ -328,7 +352,7 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
 
 // The first T rows of the step, each the one new token of its request.
 void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
-                           int window, const StepBatch& batch, const KVView& kv, int T, Workspace& ws) {
+                           int window, const StepBatch& batch, const KVView& kv, int T, Workspace& ws, const FreshKV* fresh) {
     const int max_context = kv.table_stride * kv.page_tokens;
     // where the context is cut into parts (few requests): parts of 1, 4 or 16 rounds of 64 keys,
     // so that a long context gets longer parts rather than hundreds of them; the bound is the
@@ -340,6 +364,33 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
     const int n_parts = (rounds + split_rounds - 1) / split_rounds;
     const size_t parts = static_cast<size_t>(T) * heads * n_parts;
     float* workspace = static_cast<float*>(ws.raw("attention_decode_parts", parts * (head_dim + 2) * sizeof(float)));
+    if (fresh) {
+        need(fresh->k && fresh->v, "attention_decode: fresh keys and values are missing");
+        const long long kvw = static_cast<long long>(kv_heads) * head_dim;
+        for (const Tensor* t : {fresh->k, fresh->v}) {
+            dev(*t, "fresh k/v", DType::BF16, false);
+            need(t->ndim == 2 && t->shape[0] == T && t->shape[1] == kvw, "attention_decode: fresh k and v must be [rows, kv_heads*head_dim]");
+        }
+        for (const Tensor* wt : {fresh->q_weight, fresh->k_weight})
+            if (wt) {
+                dev(*wt, "q/k norm weight", DType::F32);
+                need(wt->numel() == head_dim, "attention_decode: a norm weight must have head_dim entries");
+            }
+        const float* cos_sin = nullptr;
+        if (fresh->inv_freq) {
+            dev(*fresh->inv_freq, "inv_freq", DType::F32);
+            need(fresh->inv_freq->numel() == head_dim / 2, "attention_decode: the frequency table must have head_dim / 2 entries");
+            cos_sin = rope_table(*fresh->inv_freq, kv.table_stride * kv.page_tokens);
+        }
+        kernel_check(celeg_attention_decode_fresh_bf16(
+                         q.data, rows_of(q, "q"), fresh->k->data, rows_of(*fresh->k, "k"), fresh->v->data, rows_of(*fresh->v, "v"),
+                         fresh->q_weight ? fresh->q_weight->as<float>() : nullptr, fresh->k_weight ? fresh->k_weight->as<float>() : nullptr,
+                         fresh->eps, cos_sin, kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot, batch.positions, workspace,
+                         workspace + parts * head_dim, n_parts, out.data, heads * head_dim, T, heads, kv_heads, head_dim,
+                         kv.page_tokens, kv.n_layers, kv.layer, scale, window, attention_decode_whole, split_rounds, n_parts, stream),
+                     "attention for decode rows with fresh keys (bfloat16)");
+        return;
+    }
     kernel_check(celeg_attention_decode_bf16(q.data, rows_of(q, "q"), kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot,
                                              batch.positions, workspace, workspace + parts * head_dim, n_parts, out.data,
                                              heads * head_dim, T, heads, kv_heads, head_dim, kv.page_tokens, kv.n_layers,

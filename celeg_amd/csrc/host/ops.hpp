@@ -36,6 +36,17 @@ struct QkvTail {
     const KVView* kv = nullptr;
 };
 
+// A decode-only step's own keys and values as the q/k/v product left them, for an attention
+// that normalises and turns q and the new keys itself and writes keys and values into the pages.
+struct FreshKV {
+    const Tensor* k = nullptr;             // [rows, kv_heads * head_dim]
+    const Tensor* v = nullptr;
+    const Tensor* q_weight = nullptr;      // [head_dim] 32-bit, or null: no norm
+    const Tensor* k_weight = nullptr;
+    float eps = 0.f;
+    const Tensor* inv_freq = nullptr;      // [head_dim / 2], or null: no rotation
+};
+
 // The convolution epilogue's operands: one new token per request.
 struct ConvOperands {
     Tensor taps;          // [N, L] 32-bit
@@ -71,6 +82,7 @@ public:
     bool attention_general = false;      // always the general attention kernel
     bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
     bool use_qkv_tail = true;          // q/k/v products of many rows take norm, rotation and cache write along
+    bool use_fresh_decode = true;      // decode-only steps: the attention prepares and writes the new keys and values
     int rows_kernel_min_rows = 9, tiles_min_rows = 65, fused_linear_shape = 0;
     int last_stat_blocks = 0;
 
@@ -94,7 +106,10 @@ public:
                             const Tensor* k_weight, float eps, const Tensor* inv_freq, int rotary_dim, int pairing, int heads,
                             int kv_heads, int head_dim, const StepBatch& batch, const KVView& kv);
     void paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
-                         int window, const StepBatch& batch, const KVView& kv, Workspace& ws);
+                         int window, const StepBatch& batch, const KVView& kv, Workspace& ws, const FreshKV* fresh = nullptr);
+    // whether a decode-only step's attention can prepare and write the step's own keys and values itself
+    bool attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, int rotary_dim, int pairing, const StepBatch& batch,
+                            const KVView& kv, DType dtype) const;
     // sampling
     void sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen,
                 size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws);
@@ -125,7 +140,7 @@ private:
     std::map<std::pair<const void*, int>, std::shared_ptr<DeviceTensor>> rope_tables_;
     const float* rope_table(const Tensor& inv_freq, int n_positions);
     void attention_decode(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
-                          int window, const StepBatch& batch, const KVView& kv, int T, Workspace& ws);
+                          int window, const StepBatch& batch, const KVView& kv, int T, Workspace& ws, const FreshKV* fresh = nullptr);
     void library_product(const Tensor& x, const Tensor& w, const Tensor& out, Workspace& ws);
 };
 

@@ -365,11 +365,25 @@ private:
             q = rt.ws.buf("attn_q", rt.dtype, {T, qw});
             project(w_q_, q);
         }
+        Tensor attended = rt.ws.buf("attn_out", rt.dtype, {T, qw});
+        // a decode-only step: the attention kernel prepares and writes the step's own keys and values
+        if (!finished && writes && T == batch.n_tokens &&
+            rt.ops.attention_fresh_ok(heads_, head_dim_, inv_freq, tables.rotary_dim, tables.pairing, batch, *cache.kv, rt.dtype)) {
+            FreshKV fresh;
+            fresh.k = &k;
+            fresh.v = &v;
+            fresh.q_weight = q_norm_ ? &q_norm_->view : nullptr;
+            fresh.k_weight = k_norm_ ? &k_norm_->view : nullptr;
+            fresh.eps = eps_;
+            fresh.inv_freq = inv_freq;
+            rt.ops.paged_attention(q, attended, heads_, kv_heads_, head_dim_, scale_, window_ ? *window_ : 0, batch, *cache.kv, rt.ws,
+                                   &fresh);
+            return attended;
+        }
         if (!finished)
             rt.ops.qk_norm_rope_store(q, writes ? &k : nullptr, writes ? &v : nullptr, q_norm_ ? &q_norm_->view : nullptr,
                                       k_norm_ ? &k_norm_->view : nullptr, eps_, inv_freq,
                                       tables.rotary_dim, tables.pairing, heads_, kv_heads_, head_dim_, batch, *cache.kv);
-        Tensor attended = rt.ws.buf("attn_out", rt.dtype, {T, qw});
         rt.ops.paged_attention(q, attended, heads_, kv_heads_, head_dim_, scale_, window_ ? *window_ : 0, batch, *cache.kv, rt.ws);
         return attended;
     }

@@ -396,7 +396,16 @@ class HipOps:
             _c_int(window if window else 0), self._stream())
         self._check(code, "paged_attention")
 
-    def _attention_decode(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv, T):
+    def attention_decode_fresh(self, q, k, v, out, q_weight, k_weight, eps, inv_freq, heads, kv_heads, head_dim,
+                               scale, window, batch, kv):
+        """A decode-only step whose new keys and values are not in the cache yet: q, k and v as
+        the q/k/v product left them; the attention kernel normalises and turns q and the new
+        key, adds the new key and value as one more key and writes them into the pages."""
+        cos_sin = self._rope_table(inv_freq, kv.table.shape[1] * kv.page_tokens) if inv_freq is not None else None
+        self._attention_decode(q, out, heads, kv_heads, head_dim, scale, window, batch, kv, q.shape[0],
+                               fresh=(k, v, q_weight, k_weight, eps, cos_sin))
+
+    def _attention_decode(self, q, out, heads, kv_heads, head_dim, scale, window, batch, kv, T, fresh=None):
         """The first ``T`` rows of the step, each the one new token of its request."""
         max_context = kv.table.shape[1] * kv.page_tokens
         n_splits = (max_context + 63) // 64          # the kernel takes 64 keys a wavefront
@@ -415,6 +424,19 @@ class HipOps:
         n_parts = (rounds + split_rounds - 1) // split_rounds
         ws_o = self._decode_ws[:T * heads * n_splits * head_dim]
         ws_ml = self._decode_ws[T * heads * n_splits * head_dim:need]
+        if fresh is not None:
+            k, v, q_weight, k_weight, eps, cos_sin = fresh
+            code = self._lib("attention_fast").celeg_attention_decode_fresh_bf16(
+                _ptr(q), _c_int(self._rows(q, "q")), _ptr(k), _c_int(self._rows(k, "k")), _ptr(v), _c_int(self._rows(v, "v")),
+                _ptr(q_weight), _ptr(k_weight), _c_float(eps), _ptr(cos_sin), _ptr(kv.k), _ptr(kv.v), _ptr(kv.table),
+                _c_int(kv.table.shape[1]), _ptr(batch.token_slot), _ptr(batch.positions), _ptr(ws_o),
+                _ptr(ws_ml), _c_int(n_splits), _ptr(out), _c_int(heads * head_dim),
+                _c_int(T), _c_int(heads), _c_int(kv_heads), _c_int(head_dim), _c_int(kv.page_tokens),
+                _c_int(kv.n_layers), _c_int(kv.layer), _c_float(scale),
+                _c_int(window if window else 0), _c_int(self.attention_decode_whole),
+                _c_int(split_rounds), _c_int(n_parts), self._stream())
+            self._check(code, "attention for decode rows with fresh keys (bfloat16)")
+            return
         code = self._lib("attention_fast").celeg_attention_decode_bf16(
             _ptr(q), _c_int(self._rows(q, "q")), _ptr(kv.k), _ptr(kv.v), _ptr(kv.table),
             _c_int(kv.table.shape[1]), _ptr(batch.token_slot), _ptr(batch.positions), _ptr(ws_o),

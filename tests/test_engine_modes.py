@@ -75,9 +75,12 @@ def test_gpu_engine_with_tiled_products_matches_plain(model_folders, mode):
     beside single tokens."""
     lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles")
     assert lm.knobs()["use_tiled_products"] == 1 and lm.native.info["gemm_backend"] == "tiles"
-    assert lm.knobs()["use_qkv_tail"] == 1     # q/k norm, rotation and cache write inside the q/k/v product's kernel
+    # (q/k norm, rotation and cache write inside the q/k/v product's kernel for long steps, inside the
+    # attention kernel for decode-only steps)
+    assert lm.knobs()["use_qkv_tail"] == 1 and lm.knobs()["use_fresh_decode"] == 1
     # the same with the q/k norm, the rotation and the cache write as a kernel of their own
-    run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles", knobs={"use_qkv_tail": 0})
+    run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles",
+             knobs={"use_qkv_tail": 0, "use_fresh_decode": 0})
     # and the same configuration through the library's products
     lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="library")
     assert lm.knobs()["use_tiled_products"] == 0 and lm.native.info["gemm_backend"] == "library"

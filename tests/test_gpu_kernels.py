@@ -689,3 +689,71 @@ def test_window_attention_never_reads_pages_it_has_given_back(ops, head_dim, pag
                                  k.double().cpu().reshape(n, kv_heads, head_dim),
                                  v.double().cpu().reshape(n, kv_heads, head_dim), window=window).reshape(n, -1)
     torch.testing.assert_close(got, ref, **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("whole,parts", [(0, (64, 256)), (0, (0, 1 << 30)), (0, (0, 0)), (1, (64, 256))])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,rotate,normed", [(16, 8, 64, True, True), (4, 1, 128, True, True),
+                                                                   (6, 2, 64, False, True), (40, 2, 64, True, False)])
+def test_attention_decode_that_prepares_and_writes_the_new_token_itself(ops, whole, parts, heads, kv_heads, head_dim,
+                                                                        rotate, normed):
+    """Decode steps whose attention kernel normalises and turns q and the new key, takes the new
+    key and value as one more key and writes them into the pages, against qk_norm_rope_store
+    followed by the attention: requests at positions 0, 1, 63, 64, 65 and further (a part that
+    holds nothing but the new token; the first key of a round), parts of 1, 4 and 16 rounds and
+    one workgroup a request, three steps in a row so that later steps read what earlier ones
+    wrote; a window of 40 keys too.  Values must be written bit for bit; outputs and keys may
+    differ by a rounding."""
+    from celeg_amd.engine import StepEntry
+    n_layers, layer, page_tokens = 2, 1, 16
+    starts = [0, 1, 63, 64, 65, 200, 331]
+    n = len(starts)
+    qw = (1 + randn(head_dim, seed=40, scale=0.2)) if normed else None
+    kw = (1 + randn(head_dim, seed=41, scale=0.2)) if normed else None
+    inv_freq = torch.tensor(plain.rope_inverse_frequencies(10000.0, head_dim), dtype=torch.float64).float().to(DEV) if rotate else None
+    scale = head_dim ** -0.5
+    N = (heads + 2 * kv_heads) * head_dim
+    ops.attention_decode_whole = whole
+    saved = ops.decode_part_thresholds
+    ops.decode_part_thresholds = parts
+    try:
+        for window in (None, 40):
+            results = []
+            for fused in (False, True):
+                cache = make_cache(kv_heads, head_dim, n_layers, torch.bfloat16, page_tokens=page_tokens, n_pages=n * 24 + 4,
+                                   max_context=352, slots=n, window=window)
+                kv = cache.layer_cache(layer).kv
+                slots = [cache.open() for _ in starts]
+                # what lies before the first step: the same keys and values for both runs
+                for i, (slot, start) in enumerate(zip(slots, starts)):
+                    assert cache.prepare(slot, 0, start + 3)
+                batch, keep = build_batch(ops, cache, [StepEntry(s, 0, [0]) for s in slots])      # (applies the tables)
+                table = kv.table.cpu()
+                g = torch.Generator().manual_seed(50)
+                kv.k.copy_((torch.randn(kv.k.shape, generator=g) * 0.5).to(torch.bfloat16))
+                kv.v.copy_((torch.randn(kv.v.shape, generator=g) * 0.5).to(torch.bfloat16))
+                outs = []
+                for step in range(3):
+                    batch, keep = build_batch(ops, cache, [StepEntry(s, st + step, [0]) for s, st in zip(slots, starts)])
+                    qkv = randn(n, N, seed=60 + step, dtype=torch.bfloat16)
+                    q, k, v = qkv[:, :heads * head_dim], qkv[:, heads * head_dim:(heads + kv_heads) * head_dim], qkv[:, (heads + kv_heads) * head_dim:]
+                    out = torch.zeros(n, heads * head_dim, dtype=torch.bfloat16, device=DEV)
+                    if fused:
+                        ops.attention_decode_fresh(q, k, v, out, qw, kw, 1e-6, inv_freq, heads, kv_heads, head_dim, scale,
+                                                   window, batch, kv)
+                    else:
+                        ops.qk_norm_rope_store(q, k, v, qw, kw, 1e-6, inv_freq, head_dim if rotate else 0, heads, kv_heads,
+                                               head_dim, batch, kv)
+                        ops.paged_attention(q, out, heads, kv_heads, head_dim, scale, window, batch, kv)
+                    torch.cuda.synchronize()
+                    outs.append(out.float().clone())
+                results.append((torch.stack(outs), kv.k.float().clone(), kv.v.clone()))
+            (oa, ka, va), (ob, kb, vb) = results
+            assert torch.equal(va, vb)
+            assert float(oa.abs().max()) > 0 and not torch.isnan(ob).any()
+            assert float(((ka - kb).abs() / (ka.abs() + kb.abs() + 1e-3)).max()) <= 2 ** -7
+            assert float((ka != kb).float().mean()) < 0.01
+            assert float((oa - ob).abs().max()) <= 2e-2 * float(oa.abs().max())
+            assert float((oa - ob).abs().mean()) <= 2e-3 * float(oa.abs().max())
+    finally:
+        ops.attention_decode_whole = -1
+        ops.decode_part_thresholds = saved
