@@ -699,8 +699,13 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
 #pragma unroll
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8_t*>(qrow + s * 32);
     }
-    // The query heads as the product left them: norm and rotation here, once the first round's
-    // keys have been asked for (what that needs from memory is asked for now).
+    // The query heads as the product left them: norm and rotation here.  A workgroup of one
+    // wavefront (one round of keys) asks for what that needs now, does the arithmetic once its
+    // round's keys have been asked for, and asks for the new key and value ahead of the round
+    // too (LAZY).  Wavefronts with many rounds have no registers to hold all that meanwhile:
+    // they prepare q at once, each of them the same, which a compute unit that runs many such
+    // workgroups in turn pays every time (the host sends it launches of few workgroups only).
+    constexpr bool LAZY = WAVES == 1;
     const float* const fresh_cs = FRESH && fresh.cos_sin ? fresh.cos_sin + static_cast<size_t>(pos) * HD : nullptr;
     DecodeHeadOperands<KS> q_operands;
     if (FRESH) decode_head_operands<KS>(q_operands, fresh.q_weight, fresh_cs, qd);
@@ -718,6 +723,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<__bf16>(x[s][e]);
         q_ready = true;
     };
+    if (FRESH && !LAZY) prepare_q();
     // (with a fresh token the rounds end at the position before it)
     const int last_key = FRESH ? pos - 1 : pos;
     float m_run = -INFINITY, l_run = 0.f;
@@ -738,7 +744,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     bf16x8_t k_raw[KS];
     bf16x4_t v_raw[DT];
     DecodeHeadOperands<KS> k_operands;
-    if (adds_fresh) {
+    if (adds_fresh && LAZY) {
         const bf16* krow = fresh.k + static_cast<size_t>(t) * fresh.ldk + static_cast<size_t>(kvh) * HD + qd * 8;
 #pragma unroll
         for (int s = 0; s < KS; ++s) k_raw[s] = *reinterpret_cast<const bf16x8_t*>(krow + s * 32);
@@ -747,11 +753,68 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
         for (int dt = 0; dt < DT; ++dt) v_raw[dt] = *reinterpret_cast<const bf16x4_t*>(vrow + 16 * dt);
         decode_head_operands<KS>(k_operands, fresh.k_weight, nullptr, qd);
     }
-    // (a part of one round: the stride tells the compiler that the loop runs once)
-    for (int r = r_begin + wave; r <= r_end; r += (SPLIT && WAVES == 1) ? (1 << 30) : WAVES) {
+    // The new token as one more key: before the rounds where the wavefront has many (what it
+    // needs from memory arrives with q), after its one round otherwise.
+    auto add_fresh = [&]() {
+        if (!q_ready) prepare_q();            // (a part that holds no other key)
+        if (!LAZY) {
+            const bf16* krow = fresh.k + static_cast<size_t>(t) * fresh.ldk + static_cast<size_t>(kvh) * HD + qd * 8;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) k_raw[s] = *reinterpret_cast<const bf16x8_t*>(krow + s * 32);
+            const bf16* vrow = fresh.v + static_cast<size_t>(t) * fresh.ldv + static_cast<size_t>(kvh) * HD + 4 * qd;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) v_raw[dt] = *reinterpret_cast<const bf16x4_t*>(vrow + 16 * dt);
+            decode_head_operands<KS>(k_operands, fresh.k_weight, fresh_cs, qd);
+        }
+        // the new key in the layout of a query head (every head's lanes prepare it alike)
+        float kx[KS][8];
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) kx[s][e] = static_cast<float>(k_raw[s][e]);
+        decode_prepare_head<KS>(kx, fresh.k_weight != nullptr, fresh_cs != nullptr, k_operands.w, LAZY ? q_operands.cs : k_operands.cs,
+                                fresh.eps);
+        const int page = pages[pos >> page_shift];
+        const size_t block = kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD);
+        float dot = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            bf16x8_t kb16;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                kb16[e] = static_cast<__bf16>(kx[s][e]);
+                dot = fmaf(static_cast<float>(qf[s][e]), static_cast<float>(kb16[e]), dot);
+            }
+            if (chunk == 0 && c == 0)        // one copy into the page
+                *reinterpret_cast<bf16x8_t*>(fresh.k_pool + block + static_cast<size_t>(pos & page_mask) * HD + s * 32 + qd * 8) = kb16;
+        }
+        dot += __shfl_xor(dot, 16, 64);
+        dot += __shfl_xor(dot, 32, 64);
+        const float s_new = dot * scale;
+        const float m_new = fmaxf(m_run, s_new);
+        const float keep = expf(m_run - m_new);         // e^(-inf) = 0 where the part holds no other key
+        const float p_exact = expf(s_new - m_new);
+        const float p_new = static_cast<float>(static_cast<__bf16>(p_exact));     // as the rounds round theirs for the output
+        l_run = l_run * keep + p_exact;
+        m_run = m_new;
+        // the new value: this lane's dimensions of the output, 16 dt + 4 qd + i
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x4_t vv = v_raw[dt];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[dt][i] = o[dt][i] * keep + p_new * static_cast<float>(vv[i]);
+            if (chunk == 0 && c == 0) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    reinterpret_cast<__bf16*>(fresh.v_pool)[block + static_cast<size_t>(16 * dt + 4 * qd + i) * page_tokens + (pos & page_mask)] = vv[i];
+            }
+        }
+    };
+    // One round of 64 keys; after_loads runs once the round's keys and values have been asked for.
+    auto one_round = [&](const int r, auto&& after_loads) {
         const int kb = r * DEC_KEYS;
         const int k_lo = max(lo, kb), k_hi = min(last_key, kb + DEC_KEYS - 1);
-        if (k_lo > k_hi) continue;            // (a window of one key with a fresh token: nothing before it)
+        if (k_lo > k_hi) return;              // (a window of one key with a fresh token: no round holds a key)
         const int first_page = kb >> page_shift, last_page = k_hi >> page_shift;
         const int my_page = pages[min(first_page + lane, last_page)];
         bf16x8_t kf[4][KS], vf[DT][2];
@@ -775,7 +838,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             for (int dt = 0; dt < DT; ++dt)
                 vf[dt][j] = *reinterpret_cast<const bf16x8_t*>(vbase + static_cast<size_t>(16 * dt + c) * page_tokens);
         }
-        if (FRESH && !q_ready) prepare_q();   // (the round's keys and values are on their way)
+        after_loads();
         float sc[4][4];
         float mx = -INFINITY;
 #pragma unroll
@@ -822,52 +885,14 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             for (int dt = 0; dt < DT; ++dt)
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt][j], pb, o[dt], 0, 0, 0);
         }
+    };
+    if (adds_fresh && !LAZY) add_fresh();
+    if constexpr (SPLIT && WAVES == 1) {       // a part of one round
+        if (r_begin <= r_end) one_round(r_begin, [&]() { if (FRESH) prepare_q(); });
+    } else {
+        for (int r = r_begin + wave; r <= r_end; r += WAVES) one_round(r, []() {});
     }
-    if (adds_fresh) {
-        if (!q_ready) prepare_q();            // (a part that holds no other key)
-        // the new key in the layout of a query head (every head's lanes prepare it alike)
-        float kx[KS][8];
-#pragma unroll
-        for (int s = 0; s < KS; ++s)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) kx[s][e] = static_cast<float>(k_raw[s][e]);
-        decode_prepare_head<KS>(kx, fresh.k_weight != nullptr, fresh_cs != nullptr, k_operands.w, q_operands.cs, fresh.eps);
-        const int page = pages[pos >> page_shift];
-        const size_t block = kv_block(page, n_layers, layer, kv_heads, kvh, page_tokens, HD);
-        float dot = 0.f;
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            bf16x8_t kb16;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                kb16[e] = static_cast<__bf16>(kx[s][e]);
-                dot = fmaf(static_cast<float>(qf[s][e]), static_cast<float>(kb16[e]), dot);
-            }
-            if (chunk == 0 && c == 0)        // one copy into the page
-                *reinterpret_cast<bf16x8_t*>(fresh.k_pool + block + static_cast<size_t>(pos & page_mask) * HD + s * 32 + qd * 8) = kb16;
-        }
-        dot += __shfl_xor(dot, 16, 64);
-        dot += __shfl_xor(dot, 32, 64);
-        const float s_new = dot * scale;
-        const float m_new = fmaxf(m_run, s_new);
-        const float keep = expf(m_run - m_new);         // e^(-inf) = 0 where the part holds no other key
-        const float p_exact = expf(s_new - m_new);
-        const float p_new = static_cast<float>(static_cast<__bf16>(p_exact));     // as the rounds round theirs for the output
-        l_run = l_run * keep + p_exact;
-        m_run = m_new;
-        // the new value: this lane's dimensions of the output, 16 dt + 4 qd + i
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const bf16x4_t vv = v_raw[dt];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) o[dt][i] = o[dt][i] * keep + p_new * static_cast<float>(vv[i]);
-            if (chunk == 0 && c == 0) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    reinterpret_cast<__bf16*>(fresh.v_pool)[block + static_cast<size_t>(16 * dt + 4 * qd + i) * page_tokens + (pos & page_mask)] = vv[i];
-            }
-        }
-    }
+    if (adds_fresh && LAZY) add_fresh();
     if (SPLIT && WAVES == 1) {
         if (c < gp) {
             const size_t idx = (static_cast<size_t>(t) * (kv_heads * group) + h0 + c) * n_splits + blockIdx.z;

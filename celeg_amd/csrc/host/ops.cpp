@@ -296,16 +296,25 @@ bool Ops::attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, in
     if (kv.page_tokens < 16 || (kv.page_tokens & (kv.page_tokens - 1))) return false;
     if ((head_dim != 64 && head_dim != 128) || kv.head_dim != head_dim || (kv.v_head_dim && kv.v_head_dim != head_dim)) return false;
     if (!batch.decode_only || batch.n_seqs != batch.n_tokens) return false;
-    // Only where the kernel that takes a round of 64 keys a workgroup runs (few requests, contexts up
-    // to 4,096 tokens, heads of 64): the forms with many wavefronts a workgroup have no registers
-    // left for the new token's operands.
-    if (head_dim != 64 || attention_decode_whole > 0) return false;
-    const int max_context = kv.table_stride * kv.page_tokens;
-    const int hint = batch.context_hint();
-    const int rounds = ((hint ? std::min(hint, max_context) : max_context) + 63) / 64;
-    if (rounds > decode_part_thresholds[0]) return false;
+    // (measured with heads of 64 only)
+    if (head_dim != 64) return false;
+    // Which kernel attention_decode will take: one workgroup a (request, key/value head), or parts
+    // of 1, 4 or 16 rounds.  In parts of many rounds every wavefront prepares q before it asks for
+    // its keys, which pays where a compute unit runs one such workgroup and costs more than the
+    // kernel it saves where it runs many in turn (8 requests at 8,192 and 32,768 tokens: 1 and 5 us
+    // a layer slower; 1 request at 16,384: 4 us a layer faster).
     const int chunks = (heads / kv.kv_heads + 15) / 16;
-    if (attention_decode_whole < 0 && static_cast<long long>(kv.kv_heads) * chunks * batch.n_tokens >= 192) return false;
+    const long long groups = static_cast<long long>(kv.kv_heads) * chunks * batch.n_tokens;
+    const bool whole = attention_decode_whole < 0 ? groups >= 192 : attention_decode_whole > 0;
+    if (!whole) {
+        const int max_context = kv.table_stride * kv.page_tokens;
+        const int hint = batch.context_hint();
+        const int rounds = ((hint ? std::min(hint, max_context) : max_context) + 63) / 64;
+        if (rounds > decode_part_thresholds[0]) {
+            const int split_rounds = rounds <= decode_part_thresholds[1] ? 4 : 16;
+            if (groups * ((rounds + split_rounds - 1) / split_rounds) > 256) return false;
+        }
+    }
     return !inv_freq || (rotary_dim == head_dim && pairing == 0 && use_rope_table);
 }
 

@@ -167,12 +167,14 @@ def test_long_decoding(model_folders, name, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("whole", [-1, 1])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_decoding_across_the_bounds_of_recorded_steps(model_folders, dtype):
+def test_long_decoding_across_the_bounds_of_recorded_steps(model_folders, dtype, whole):
     """A recorded decode step serves contexts up to a bound (the attention over few requests
     cuts the context into parts by it), and a longer context takes another recording.  With
     parts of 4 rounds from 2 rounds on and of 16 from 9 on, two requests decode from 20 to 330
-    tokens; every position is compared with the plain implementation."""
+    tokens; every position is compared with the plain implementation.  Once more with the
+    kernel of many requests (one workgroup a request and key/value head) forced."""
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders("D", storage, WEIGHT_STD)
@@ -184,6 +186,7 @@ def test_long_decoding_across_the_bounds_of_recorded_steps(model_folders, dtype)
                     max_batched_tokens=256)
     lm.set_knob("decode_parts_few", 1)
     lm.set_knob("decode_parts_some", 8)
+    lm.set_knob("attention_decode_whole", whole)
     got = EngineDriver(lm).run(steps)
     cfgp, W = plain.load_model_folder(folder)
     for rid, toks in reqs.items():
