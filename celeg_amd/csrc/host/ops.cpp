@@ -301,19 +301,23 @@ bool Ops::attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, in
     // Which kernel attention_decode will take: one workgroup a (request, key/value head), or parts
     // of 1, 4 or 16 rounds.  In parts of many rounds every wavefront prepares q before it asks for
     // its keys, which pays where a compute unit runs one such workgroup and costs more than the
-    // kernel it saves where it runs many in turn (8 requests at 8,192 and 32,768 tokens: 1 and 5 us
-    // a layer slower; 1 request at 16,384: 4 us a layer faster).
+    // kernel it saves where it runs many in turn (8 requests at 8,192 and 32,768 tokens, 2,112
+    // workgroups: 1 and 5 us a layer slower; 1 request at 16,384, 136 workgroups: 4 us a layer
+    // faster; 264 workgroups: 1 us a layer faster).
     const int chunks = (heads / kv.kv_heads + 15) / 16;
     const long long groups = static_cast<long long>(kv.kv_heads) * chunks * batch.n_tokens;
     const bool whole = attention_decode_whole < 0 ? groups >= 192 : attention_decode_whole > 0;
-    if (!whole) {
-        const int max_context = kv.table_stride * kv.page_tokens;
-        const int hint = batch.context_hint();
-        const int rounds = ((hint ? std::min(hint, max_context) : max_context) + 63) / 64;
-        if (rounds > decode_part_thresholds[0]) {
-            const int split_rounds = rounds <= decode_part_thresholds[1] ? 4 : 16;
-            if (groups * ((rounds + split_rounds - 1) / split_rounds) > 256) return false;
-        }
+    const int max_context = kv.table_stride * kv.page_tokens;
+    const int hint = batch.context_hint();
+    const int rounds = ((hint ? std::min(hint, max_context) : max_context) + 63) / 64;
+    if (whole) {
+        // the kernel's loop over the rounds runs 1.7 % slower in this form, which outweighs the
+        // kernel saved from about 8,192 tokens for each of 64 requests on (at 32,768: 4.94 against
+        // 4.86 ms a step; at 2,048: 0.906 against 0.916)
+        if (static_cast<long long>(batch.n_tokens) * rounds > 4096) return false;
+    } else if (rounds > decode_part_thresholds[0]) {
+        const int split_rounds = rounds <= decode_part_thresholds[1] ? 4 : 16;
+        if (groups * ((rounds + split_rounds - 1) / split_rounds) > 512) return false;
     }
     return !inv_freq || (rotary_dim == head_dim && pairing == 0 && use_rope_table);
 }
