@@ -24,18 +24,27 @@ def random_prompt(vocab: int, n: int, seed: int) -> List[int]:
 
 
 def measure_prefill(lm: LoadedModel, n_tokens: int, repeats: int = 5, warmup: int = 2,
-                    seed: int = 0) -> Dict[str, float]:
+                    seed: int = 0, offset: int = 0) -> Dict[str, float]:
     """One prompt of ``n_tokens`` in one step, logits for the last row (brought to the host);
-    median of ``repeats`` after ``warmup`` runs."""
-    prompt = random_prompt(lm.spec.vocab_size, n_tokens, seed)
+    median of ``repeats`` after ``warmup`` runs.  With ``offset`` the step is a later portion of
+    a long prompt: the ``offset`` tokens before it are fed first, in portions of ``n_tokens``,
+    outside the timing."""
+    prompt = random_prompt(lm.spec.vocab_size, offset + n_tokens, seed)
     times = []
     for i in range(warmup + repeats):
         slot = lm.cache.open()
-        if slot is None or not lm.cache.prepare(slot, 0, n_tokens):
+        if slot is None:
+            raise RuntimeError("measure_prefill: no free request slot")
+        for at in range(0, offset, n_tokens):
+            n = min(n_tokens, offset - at)
+            if not lm.cache.prepare(slot, at, n):
+                raise RuntimeError("measure_prefill: the cache pool is too small for the prompt")
+            lm.runner.step([StepEntry(slot, at, prompt[at:at + n], [])])
+        if not lm.cache.prepare(slot, offset, n_tokens):
             raise RuntimeError("measure_prefill: the cache pool is too small for the prompt")
         lm.native.synchronize()
         start = time.perf_counter()
-        lm.runner.step([StepEntry(slot, 0, prompt, [n_tokens - 1])])     # returns when the logits are on the host
+        lm.runner.step([StepEntry(slot, offset, prompt[offset:], [n_tokens - 1])])     # returns when the logits are on the host
         elapsed = time.perf_counter() - start
         lm.cache.close(slot)
         if i >= warmup:
