@@ -348,6 +348,62 @@ __global__ void embed_stream_kernel(const bf16* __restrict__ table, const int* _
     if (threadIdx.x == 0) stats[static_cast<size_t>(row) * stats_ld] = s;
 }
 
+// The same with what a step begins with taken along (one kernel fewer in a step that is bound by
+// its number of kernels): a row whose token id is negative takes the token its request sampled
+// last and leaves it in ids, and the blocks behind the rows' write the step's block-table
+// updates (count, then (slot, logical page, page) triples).
+__global__ void embed_stream_prologue_kernel(const bf16* __restrict__ table, int* __restrict__ ids,
+                                             float* __restrict__ out, bf16* __restrict__ xb, int ldx,
+                                             long long xb_k8, float* __restrict__ stats, int stats_ld,
+                                             int width, int vocab, int rows,
+                                             int* __restrict__ block_table, int stride, int n_slots,
+                                             const int* __restrict__ updates, int capacity,
+                                             const int* __restrict__ token_slot,
+                                             const int* __restrict__ last_tokens) {
+    __shared__ float scratch[16];
+    if (static_cast<int>(blockIdx.x) >= rows) {
+        const int i = (static_cast<int>(blockIdx.x) - rows) * blockDim.x + threadIdx.x;
+        if (i < min(updates[0], capacity)) {
+            const int slot = updates[1 + 3 * i], logical = updates[2 + 3 * i], page = updates[3 + 3 * i];
+            if (slot >= 0 && slot < n_slots && logical >= 0 && logical < stride)
+                block_table[static_cast<size_t>(slot) * stride + logical] = page;
+        }
+        return;
+    }
+    const int row = blockIdx.x;
+    int id = ids[row];
+    if (id < 0 && last_tokens) {
+        // (a thread that reads ids[row] after thread 0 has written it finds the same token there)
+        id = last_tokens[token_slot[row]];
+        if (threadIdx.x == 0) ids[row] = id;
+    }
+    const bool ok = id >= 0 && id < vocab;
+    const bf16* src = table + static_cast<size_t>(ok ? id : 0) * width;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const bf16 raw = ok ? src[i] : bf16{0};
+        const float v = to_float(raw);
+        out[static_cast<size_t>(row) * width + i] = v;
+        xb[static_cast<size_t>(row) * ldx + static_cast<size_t>(i >> 3) * xb_k8 + (i & 7)] = raw;
+        s += v * v;
+    }
+    s = block_sum(s, scratch);
+    if (threadIdx.x == 0) stats[static_cast<size_t>(row) * stats_ld] = s;
+}
+
+extern "C" int celeg_embed_stream_prologue(const void* table, int* ids, float* out, void* xb, int ldx,
+                                           long long xb_k8, float* stats, int stats_ld, int rows, int width,
+                                           int vocab, int* block_table, int stride, int n_slots,
+                                           const int* updates, int capacity, const int* token_slot,
+                                           const int* last_tokens, hipStream_t stream) {
+    if (rows <= 0 || capacity <= 0 || !updates || !block_table) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(embed_stream_prologue_kernel, dim3(rows + (capacity + 255) / 256), dim3(256), 0, stream,
+                       static_cast<const bf16*>(table), ids, out, static_cast<bf16*>(xb), ldx, xb_k8,
+                       stats, stats_ld, width, vocab, rows, block_table, stride, n_slots, updates, capacity,
+                       token_slot, last_tokens);
+    return CELEG_LAUNCH_RESULT();
+}
+
 extern "C" int celeg_embed_stream(const void* table, const int* ids, float* out, void* xb, int ldx,
                                   long long xb_k8, float* stats, int stats_ld, int rows, int width,
                                   int vocab, hipStream_t stream) {

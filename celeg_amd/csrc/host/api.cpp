@@ -591,6 +591,7 @@ const std::vector<Knob>& knobs() {
         {"portion_graph_min_tokens", [](LoadedModel& m) { return m.runner->portion_graph_min_tokens; },
          [](LoadedModel& m, int v) { m.runner->portion_graph_min_tokens = v; }},
         {"use_fused", [](LoadedModel& m) { return m.rt->use_fused ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->use_fused = v != 0; }},
+        {"defer_prologue", [](LoadedModel& m) { return m.rt->defer_prologue ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->defer_prologue = v != 0; }},
         {"use_tiled_products", [](LoadedModel& m) { return m.rt->use_tiled_products ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->use_tiled_products = v != 0; }},
         {"fused_max_rows", [](LoadedModel& m) { return m.rt->fused_max_rows; }, [](LoadedModel& m, int v) { m.rt->fused_max_rows = v; }},
         OPS_INT(attention_decode_whole), OPS_BOOL(use_blaslt), OPS_INT(attention_rows_per_tile), OPS_INT(attention_rows_form),

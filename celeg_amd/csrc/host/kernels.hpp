@@ -80,6 +80,10 @@ int celeg_stream_prepare(const float* h, int ldh, void* xb, int ldx, long long x
                          int rows, int width, hipStream_t stream);
 int celeg_embed_stream(const void* table, const int* ids, float* out, void* xb, int ldx, long long xb_k8, float* stats,
                        int stats_ld, int rows, int width, int vocab, hipStream_t stream);
+int celeg_embed_stream_prologue(const void* table, int* ids, float* out, void* xb, int ldx, long long xb_k8, float* stats,
+                                int stats_ld, int rows, int width, int vocab, int* block_table, int stride, int n_slots,
+                                const int* updates, int capacity, const int* token_slot, const int* last_tokens,
+                                hipStream_t stream);
 int celeg_gemm_rows_blocks(int M, int N, int K, int epi);
 int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t stream);
 int celeg_gemv_fused(const GemvParams* params, int amode, int epi, int shape, hipStream_t stream);

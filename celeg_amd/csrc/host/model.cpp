@@ -148,7 +148,9 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
     Tensor h = rt.ws.buf("hidden", DType::F32, {T, width});
     rt.stream_stat_blocks = 0;
     rt.stream_has_bf16 = false;
+    if (!embedding_->takes_step_prologue()) rt.flush_prologue();
     embedding_->forward(batch.token_ids, h, rt, &batch);
+    rt.flush_prologue();      // (an embedding that said it would and did not)
     rt.mark("embedding");
     Tensor delta;
     for (size_t i = 0; i < spec.order.size(); ++i) {
@@ -280,8 +282,19 @@ void ModelRunner::ship_table_updates(int group, const std::vector<TableUpdate>& 
 void ModelRunner::begin_step(const StepBatch& batch) {
     const auto& caps = batch.table_update_caps;
     if (caps.size() == 1 && caps[0] > 0) {
-        rt.ops.step_prologue(cache.device_table(0), cache.max_pages_per_request, cache.max_requests + 1,
-                             batch.table_updates[0], caps[0], batch.token_ids, batch.token_slot, token_source_, batch.n_tokens);
+        StepPrologue& p = rt.prologue;
+        p.table = cache.device_table(0);
+        p.stride = cache.max_pages_per_request;
+        p.n_slots = cache.max_requests + 1;
+        p.updates = batch.table_updates[0];
+        p.capacity = caps[0];
+        p.token_ids = batch.token_ids;
+        p.token_slot = batch.token_slot;
+        p.last_tokens = token_source_;
+        p.n = batch.n_tokens;
+        p.pending = true;
+        // left to the embedding's kernel (one kernel fewer a step), or run now
+        if (!rt.defer_prologue || rt.phases) rt.flush_prologue();
         return;
     }
     for (size_t g = 0; g < caps.size(); ++g)

@@ -473,7 +473,8 @@ void Ops::stream_prepare(const Tensor& h, const Tensor& xb, const Tensor& stats)
                                       static_cast<int>(width), stream), "stream_prepare");
 }
 
-void Ops::embed_stream(const Tensor& table, const int* token_ids, const Tensor& out, const Tensor& xb, const Tensor& stats) {
+void Ops::embed_stream(const Tensor& table, const int* token_ids, const Tensor& out, const Tensor& xb, const Tensor& stats,
+                       const StepPrologue* prologue) {
     dev(table, "table", DType::BF16);
     dev(out, "out", DType::F32);
     dev(xb, "xb", DType::BF16, false);
@@ -481,6 +482,16 @@ void Ops::embed_stream(const Tensor& table, const int* token_ids, const Tensor& 
     const long long rows = out.shape[0], width = out.shape[1];
     const Operand o = operand(xb, "xb");
     need(table.shape[1] == width && stats.shape[0] >= rows && o.rows == rows && o.width == width, "embed_stream: shapes do not fit");
+    if (prologue) {
+        need(prologue->token_ids == token_ids && prologue->n == rows && prologue->capacity > 0 && prologue->table && prologue->updates,
+             "embed_stream: the step's prologue is not for these rows");
+        kernel_check(celeg_embed_stream_prologue(table.data, prologue->token_ids, out.as<float>(), xb.data, static_cast<int>(o.ld), o.k8,
+                                                 stats.as<float>(), static_cast<int>(stats.stride[0]), static_cast<int>(rows),
+                                                 static_cast<int>(width), static_cast<int>(table.shape[0]), prologue->table,
+                                                 prologue->stride, prologue->n_slots, prologue->updates, prologue->capacity,
+                                                 prologue->token_slot, prologue->last_tokens, stream), "embed_stream with the step's prologue");
+        return;
+    }
     kernel_check(celeg_embed_stream(table.data, token_ids, out.as<float>(), xb.data, static_cast<int>(o.ld), o.k8,
                                     stats.as<float>(), static_cast<int>(stats.stride[0]), static_cast<int>(rows),
                                     static_cast<int>(width), static_cast<int>(table.shape[0]), stream), "embed_stream");

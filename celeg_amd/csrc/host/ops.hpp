@@ -70,6 +70,20 @@ struct FusedArgs {
     bool packed = false;          // w is [K/32, rows, 32] (pack_weight)
 };
 
+// What a step begins with, when the runner leaves it to the step's first kernel: the block-table
+// updates of the (one) cache group and the rows whose token is on the device.
+struct StepPrologue {
+    int* table = nullptr;
+    int stride = 0, n_slots = 0;
+    const int* updates = nullptr;
+    int capacity = 0;
+    int* token_ids = nullptr;
+    const int* token_slot = nullptr;
+    const int* last_tokens = nullptr;
+    int n = 0;
+    bool pending = false;
+};
+
 class Ops {
 public:
     explicit Ops(hipStream_t stream) : stream(stream) {}
@@ -119,7 +133,9 @@ public:
     bool rows_kernel_ok(int rows, std::initializer_list<long long> inner) const;
     int residual_stat_blocks(int rows, int n, int k) const;
     void stream_prepare(const Tensor& h, const Tensor& xb, const Tensor& stats);
-    void embed_stream(const Tensor& table, const int* token_ids, const Tensor& out, const Tensor& xb, const Tensor& stats);
+    // (with `prologue`: the step's block-table updates and token ids from the device in the same launch)
+    void embed_stream(const Tensor& table, const int* token_ids, const Tensor& out, const Tensor& xb, const Tensor& stats,
+                      const StepPrologue* prologue = nullptr);
     void embed_stats(const Tensor& table, const int* token_ids, const Tensor& out, const Tensor& stats);
     void fused_linear(const Tensor& a, const Tensor& w, const Tensor& out, const FusedArgs& args);
     // fused products of many rows
@@ -160,6 +176,16 @@ struct Runtime {
     // the stream's bfloat16 copy is; whoever writes the stream another way resets them
     int stream_stat_blocks = 0;
     bool stream_has_bf16 = false;
+    // the step's prologue, left by the runner for the embedding's kernel to take along
+    // (defer_prologue); whoever cannot take it along calls flush_prologue() before its own work
+    bool defer_prologue = true;
+    StepPrologue prologue;
+    void flush_prologue() {
+        if (!prologue.pending) return;
+        prologue.pending = false;
+        ops.step_prologue(prologue.table, prologue.stride, prologue.n_slots, prologue.updates, prologue.capacity,
+                          prologue.token_ids, prologue.token_slot, prologue.last_tokens, prologue.n);
+    }
     // weights re-laid for the fused path, made once per (weight, norm weight) pair
     std::map<std::pair<const void*, const void*>, std::shared_ptr<DeviceTensor>> folded_weights, folded_plain_weights;
     std::map<const void*, std::shared_ptr<DeviceTensor>> packed_weights;

@@ -579,21 +579,28 @@ public:
     WeightSpecs weight_specs() const override { return {{"table", matrix(vocab_, width_)}}; }
     void load(const PartTensors& t, Runtime&) override { table_ = get(t, "table"); }
     Tensor table() const override { return table_->view; }
+    bool takes_step_prologue() const override { return true; }
     void forward(const int* token_ids, const Tensor& out, Runtime& rt, const StepBatch* batch) override {
         const int rows = static_cast<int>(out.shape[0]);
         if (batch && table_->view.dtype == DType::BF16 && fused::fused_rows_ok(rt, *batch, {width_})) {
             // few rows: leave every row's sum of squares (and the bfloat16 copy of the stream)
             // for the first norm
             if (fused::sliced(rt, rows, width_) || fused::tiled_step(rt, rows)) {
+                // (the step's prologue rides along where it is for these rows)
+                const bool along = rt.prologue.pending && rt.prologue.token_ids == token_ids && rt.prologue.n == rows;
+                if (!along) rt.flush_prologue();
                 rt.ops.embed_stream(table_->view, token_ids, out, fused::stream_bf16(rt, rows, width_),
-                                    fused::stream_stats(rt, width_, rows));
+                                    fused::stream_stats(rt, width_, rows), along ? &rt.prologue : nullptr);
+                rt.prologue.pending = false;
                 rt.stream_has_bf16 = true;
             } else {
+                rt.flush_prologue();
                 rt.ops.embed_stats(table_->view, token_ids, out, fused::stream_stats(rt, width_));
                 rt.stream_has_bf16 = false;
             }
             rt.stream_stat_blocks = 1;
         } else {
+            rt.flush_prologue();
             rt.ops.embed(table_->view, token_ids, out);
         }
     }

@@ -101,6 +101,9 @@ public:
     using Part::Part;
     virtual void forward(const int* token_ids, const Tensor& out, Runtime& rt, const StepBatch* batch) = 0;
     virtual Tensor table() const { return Tensor(); }     // what a tied head multiplies with
+    // true: forward looks at rt.prologue itself (its kernel takes the step's prologue along, or
+    // it calls rt.flush_prologue() first); false: the model runs the prologue before forward
+    virtual bool takes_step_prologue() const { return false; }
 };
 
 class Head : public Part {

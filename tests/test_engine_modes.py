@@ -81,6 +81,10 @@ def test_gpu_engine_with_tiled_products_matches_plain(model_folders, mode):
     # the same with the q/k norm, the rotation and the cache write as a kernel of their own
     run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles",
              knobs={"use_qkv_tail": 0, "use_fresh_decode": 0})
+    # and with the step's prologue (block-table updates, tokens from the device) as a kernel of its
+    # own instead of inside the embedding's
+    assert lm.knobs()["defer_prologue"] == 1
+    run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="tiles", knobs={"defer_prologue": 0})
     # and the same configuration through the library's products
     lm = run_mode(model_folders, "E", "bfloat16", mode, "cuda:0", gemm_backend="library")
     assert lm.knobs()["use_tiled_products"] == 0 and lm.native.info["gemm_backend"] == "library"
