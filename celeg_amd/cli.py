@@ -85,6 +85,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--attention-chunk-tokens", type=int, default=0, metavar="N",
                     help="keys of a part of segmented attention: 64, 256 or 1024 (default: by the context, "
                          "64 up to 4,096 tokens, 256 up to 16,384, 1024 above)")
+    ap.add_argument("--strict-weights", action="store_true",
+                    help="refuse a checkpoint that holds tensors the model has no use for (default: a warning)")
     ap.add_argument("--device", default="cuda:0")
     return ap
 
@@ -189,7 +191,8 @@ def run(args) -> int:
                                 n_pages=args.pages or pages_per_request * max(batch, args.max_requests, 1), max_active_requests=max(batch, args.max_requests, 1),
                                 context=context, max_batched_tokens=budget,
                                 prefill_chunk_tokens=min(args.prefill_chunk, budget),
-                                gemm_backend=args.gemm_backend, use_graphs=not args.no_graph)
+                                gemm_backend=args.gemm_backend, use_graphs=not args.no_graph,
+                                strict_weights=args.strict_weights)
     lm = engine.loaded
     if args.profile:
         lm.native.time_phases(True)

@@ -186,7 +186,10 @@ __global__ __launch_bounds__(ROPE_WAVES * CELEG_WAVE) void qk_norm_rope_store_qu
     // (the page holds a dimension's keys side by side) instead of sixteen of two bytes
     if (TOKENS == 4 && !is_q && !is_k) {
         const int slot0 = token_slot[t[0]];
-        bool together = static_cast<int>(blockIdx.x) * TOKENS + 3 < n_tokens && (pos[0] & 3) == 0;
+        // a page whose size is a multiple of four holds positions 4n .. 4n+3 side by side, at an
+        // address the store of four may take; any other page size goes row by row
+        bool together = static_cast<int>(blockIdx.x) * TOKENS + 3 < n_tokens && (pos[0] & 3) == 0 &&
+                        (page_tokens & 3) == 0;
 #pragma unroll
         for (int i = 1; i < TOKENS; ++i) together = together && pos[i] == pos[0] + i && token_slot[t[i]] == slot0;
         if (together) {

@@ -5,6 +5,8 @@
 
 #include <cstring>
 #include <mutex>
+#include <set>
+#include <algorithm>
 
 #include "engine.hpp"
 #include "model.hpp"
@@ -86,6 +88,7 @@ LoadOptions load_options(const celeg_engine_options& o) {
     l.max_batched_tokens = o.max_batched_tokens;
     l.gemm_backend = o.gemm_backend == CELEG_GEMM_TILES ? "tiles" : o.gemm_backend == CELEG_GEMM_LIBRARY ? "library" : "auto";
     l.use_graphs = o.use_graphs != 0;
+    l.strict_weights = o.strict_weights != 0;
     return l;
 }
 
@@ -156,6 +159,7 @@ void celeg_engine_options_init(celeg_engine_options* o, size_t struct_size) {
     full.use_graphs = 1;
     full.run_ahead = 1;
     full.portion_granule = 1;
+    full.strict_weights = 0;
     std::memcpy(o, &full, std::min(struct_size ? struct_size : sizeof(full), sizeof(full)));
     o->struct_size = std::min(struct_size ? struct_size : sizeof(full), sizeof(full));
 }
@@ -371,7 +375,8 @@ const char* celeg_model_describe(celeg_model* model) {
                 .set("dtype", dtype_name(lm.rt->dtype)).set("weights", lm.model->weight_count())
                 .set("kv_bytes_per_token", lm.cache->layout.kv_bytes_per_token(dtype_size(lm.rt->dtype)))
                 .set("eos_token_ids", Json::array_of(lm.model->spec.eos_token_ids))
-                .set("gemm_backend", lm.rt->use_tiled_products ? "tiles" : "library");
+                .set("gemm_backend", lm.rt->use_tiled_products ? "tiles" : "library")
+                .set("unused_tensors", Json::array_of(lm.unused_tensors));
             out = j.dump();
         }) != CELEG_OK)
         return nullptr;
@@ -626,6 +631,7 @@ const char* celeg_model_knobs(celeg_model* model) {
     for (const Knob& k : knobs()) out.set(k.name, k.get(*model->lm));
     ModelRunner& r = *model->lm->runner;
     out.set("steps_run", r.steps_run).set("graph_replays", r.graph_replays).set("captures", r.captures);
+    out.set("paths", model->lm->rt->ops.paths_json());
     return text(out.dump());
 }
 
@@ -701,6 +707,14 @@ const char* celeg_describe_folder(const char* model_dir) {
                                    .set("float32", dtype_name(stored_as(info, e["kind"].as_string(), DType::F32))));
             }
             j.set("held_as", held);
+            // tensors that no part asks for (no error by themselves; loading warns about them)
+            std::set<std::string> wanted;
+            for (const Json& e : j["expected_tensors"].items()) wanted.insert(e["name"].as_string());
+            std::vector<std::string> unused;
+            for (const auto& n : ckpt.names())
+                if (!wanted.count(n)) unused.push_back(n);
+            std::sort(unused.begin(), unused.end());
+            j.set("unused_tensors", Json::array_of(unused));
             out = j.dump();
         }) != CELEG_OK)
         return nullptr;
@@ -735,13 +749,15 @@ const char* celeg_describe_config(const char* config_json, const char* shapes_js
     return text(out);
 }
 
-celeg_status celeg_check_folder(const char* model_dir) {
+celeg_status celeg_check_folder(const char* model_dir) { return celeg_check_folder_strict(model_dir, 0); }
+
+celeg_status celeg_check_folder_strict(const char* model_dir, int32_t strict) {
     if (!model_dir) return CELEG_INVALID_ARGUMENT;
     return guarded([&] {
         const Described d = describe_model_folder(model_dir);
         Model model(d.spec);
         Checkpoint ckpt(model_dir);
-        check_tensors(ckpt, model.expected_tensors());
+        check_tensors(ckpt, model.expected_tensors(), strict != 0);
     });
 }
 

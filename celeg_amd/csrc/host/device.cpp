@@ -17,8 +17,23 @@ void hip_check(hipError_t code, const char* what) {
                           std::to_string(static_cast<int>(code)) + ")");
 }
 
+bool sync_launches() {
+    static const bool on = [] {
+        const char* v = std::getenv("CELEG_SYNC_LAUNCHES");
+        return v && *v && std::string(v) != "0";
+    }();
+    return on;
+}
+
 void kernel_check(int code, const char* what) {
     if (code != 0) throw KernelError(std::string(what) + ": HIP error " + std::to_string(code));
+    if (!sync_launches()) return;
+    // the launch is waited for, so that a fault while the kernel ran is reported under the
+    // kernel's name and not by whatever call comes next
+    const hipError_t ran = hipDeviceSynchronize();
+    if (ran != hipSuccess)
+        throw KernelError(std::string(what) + ": failed while it ran: " + hipGetErrorString(ran) + " (" +
+                          std::to_string(static_cast<int>(ran)) + ")");
 }
 
 float half_to_float(uint16_t h) {

@@ -41,6 +41,11 @@ void hip_check(hipError_t code, const char* what);
 #define CELEG_HIP(expr) ::celeg::hip_check((expr), #expr)
 // the return value of a kernel's entry point (0 or a hipError_t)
 void kernel_check(int code, const char* what);
+// CELEG_SYNC_LAUNCHES=1 in the environment: kernel_check also waits for the kernel and checks how
+// it ended, so that an asynchronous fault is named by the launch that caused it, and no step is
+// recorded into or replayed from a graph (the reference's CELEG_DEBUG_SYNC build,
+// include/celeg/backend/cuda/utils.cuh:109-116, synchronises the stream behind every launch)
+bool sync_launches();
 
 // bfloat16 <-> float on the host (round to nearest even, like the device's conversion)
 inline uint16_t float_to_bf16(float f) {

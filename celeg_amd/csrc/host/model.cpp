@@ -329,7 +329,7 @@ Tensor ModelRunner::step(const std::vector<StepEntry>& entries) {
 // request's cache.  Recording and its warm-up run on such padding rows only: a request's state
 // is never advanced twice.
 bool ModelRunner::graph_applies(const std::vector<StepEntry>& entries) const {
-    if (!use_graphs || !model.graph_safe() || rt.after_layer || rt.phases) return false;
+    if (!use_graphs || !model.graph_safe() || rt.after_layer || rt.phases || sync_launches()) return false;
     if (static_cast<int>(entries.size()) > buckets_.back()) return false;
     for (const StepEntry& e : entries)
         if (e.tokens.size() != 1 || e.want.size() != 1 || e.want[0] != 0) return false;
@@ -423,7 +423,7 @@ ModelRunner::Captured& ModelRunner::record(std::pair<int, int> key, const StepBa
 // again) is recorded too, per number of rows and per context below or from 4,096 tokens (the
 // attention over rows chooses its tiles by that).
 bool ModelRunner::portion_graph_applies(const std::vector<StepEntry>& entries) {
-    if (!use_graphs || !model.graph_safe() || rt.after_layer || rt.phases || entries.size() != 1) return false;
+    if (!use_graphs || !model.graph_safe() || rt.after_layer || rt.phases || sync_launches() || entries.size() != 1) return false;
     const StepEntry& e = entries[0];
     const int T = static_cast<int>(e.tokens.size());
     if (T < portion_graph_min_tokens || e.want.size() != 1 || e.want[0] != T - 1) return false;
@@ -541,7 +541,15 @@ std::unique_ptr<LoadedModel> load_model(const std::string& model_dir, const Load
                                  (options.gemm_backend == "auto" && described.spec.hidden_size <= 1024);
     lm->model = std::make_unique<Model>(described.spec);
     {
-        WeightMap tensors = load_tensors(ckpt, lm->model->expected_tensors(), dtype);
+        WeightMap tensors = load_tensors(ckpt, lm->model->expected_tensors(), dtype, options.strict_weights,
+                                         &lm->unused_tensors);
+        if (!lm->unused_tensors.empty()) {
+            std::string names;
+            for (size_t i = 0; i < lm->unused_tensors.size() && i < 8; ++i) names += (i ? ", " : "") + lm->unused_tensors[i];
+            if (lm->unused_tensors.size() > 8) names += ", ...";
+            std::fprintf(stderr, "[celeg_amd] warning: %zu tensor(s) of %s are not used by the model: %s\n",
+                         lm->unused_tensors.size(), model_dir.c_str(), names.c_str());
+        }
         lm->model->load(tensors, *lm->rt);
     }
     const int pages_per_request = (max_context + options.page_tokens - 1) / options.page_tokens;

@@ -129,6 +129,7 @@ struct LoadOptions {
     int max_batched_tokens = 2048;
     std::string gemm_backend = "auto";      // how bfloat16 steps of more than 64 rows multiply: "library", "tiles" or "auto"
     bool use_graphs = true;
+    bool strict_weights = false;    // tensors of the checkpoint that the model has no use for are an error
 };
 
 // From a model folder to a ready step function.  The reference's path: open the checkpoint,
@@ -143,6 +144,7 @@ struct LoadedModel {
     std::unique_ptr<CacheManager> cache;
     std::unique_ptr<ModelRunner> runner;
     int device = 0;
+    std::vector<std::string> unused_tensors;   // in the checkpoint, asked for by no part
     ~LoadedModel();
 };
 

@@ -45,6 +45,30 @@ Operand operand(const Tensor& t, const char* name) {
 }
 }  // namespace
 
+const char* path_name(Path p) {
+    switch (p) {
+        case Path::AttentionDecode: return "attention_decode";
+        case Path::AttentionDecodeFresh: return "attention_decode_fresh";
+        case Path::AttentionRows: return "attention_rows";
+        case Path::AttentionGeneral: return "attention_general";
+        case Path::LinearF32: return "linear_f32";
+        case Path::LinearLibrary: return "linear_library";
+        case Path::LinearStandIn: return "linear_stand_in";
+        case Path::FusedSliced: return "fused_sliced";
+        case Path::FusedRows: return "fused_rows";
+        case Path::FusedStaged: return "fused_staged";
+        case Path::Tiled: return "tiled";
+        case Path::TiledQkv: return "tiled_qkv";
+        default: return "?";
+    }
+}
+
+Json Ops::paths_json() const {
+    Json out = Json::object();
+    for (int i = 0; i < static_cast<int>(Path::Count); ++i) out.set(path_name(static_cast<Path>(i)), path_count[i]);
+    return out;
+}
+
 // ---------------------------------------------------------------------------- row-wise
 void Ops::embed(const Tensor& table, const int* token_ids, const Tensor& out) {
     dev(table, "table");
@@ -118,7 +142,10 @@ void Ops::library_product(const Tensor& x, const Tensor& w, const Tensor& out, W
     const int M = static_cast<int>(x.shape[0]), K = static_cast<int>(x.shape[1]), N = static_cast<int>(w.shape[0]);
     if (use_blaslt) {
         if (!blaslt_) blaslt_ = std::make_unique<BlasLt>();
-        if (blaslt_->matmul(x.data, rows_of(x, "x"), w.data, out.data, rows_of(out, "out"), M, N, K, stream)) return;
+        if (blaslt_->matmul(x.data, rows_of(x, "x"), w.data, out.data, rows_of(out, "out"), M, N, K, stream)) {
+            took(Path::LinearLibrary);
+            return;
+        }
     }
     // sizes the library has no kernel for: the tiled product where the sizes fit it, else the
     // 32-bit product on widened copies
@@ -134,6 +161,7 @@ void Ops::library_product(const Tensor& x, const Tensor& w, const Tensor& out, W
         for (int m = 0; m < M; ++m) cast(x.rows(m, 1), xf.rows(m, 1));
     }
     cast(w, wf);
+    took(Path::LinearStandIn);
     kernel_check(celeg_gemm_f32(xf.as<float>(), K, wf.as<float>(), K, nullptr, yf.as<float>(), N, M, N, K, stream),
                  "linear (32-bit stand-in)");
     if (out.contiguous()) {
@@ -161,6 +189,7 @@ void Ops::linear(const Tensor& x, const Tensor& w, const Tensor& out, const Tens
     if (M == 0) return;
     if (x.dtype == DType::F32 && w.dtype == DType::F32) {
         need(out.dtype == DType::F32, "linear: a 32-bit product needs a 32-bit output");
+        took(Path::LinearF32);
         kernel_check(celeg_gemm_f32(x.as<float>(), rows_of(x, "x"), w.as<float>(), static_cast<int>(K),
                                     bias ? bias->as<float>() : nullptr, out.as<float>(), rows_of(out, "out"),
                                     static_cast<int>(M), static_cast<int>(N), static_cast<int>(K), stream), "linear (32-bit)");
@@ -346,6 +375,7 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
             // the rows kernel would hold one row), the portions to the rows kernel
             const int single = decode_hd ? batch.single_rows : 0;
             if (single) attention_decode(q, out, heads, kv_heads, head_dim, scale, window, batch, kv, single, ws);
+            if (single < batch.n_seqs) took(Path::AttentionRows);
             if (single < batch.n_seqs)
                 kernel_check(celeg_attention_rows_bf16(
                                  q.data, ldq, kv.k, kv.v, kv.table, kv.table_stride, batch.cu_seqlens + single,
@@ -357,6 +387,7 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
         }
     }
     need(!fresh, "paged_attention: fresh keys and values go with the kernels for single rows");
+    took(Path::AttentionGeneral);
     kernel_check(celeg_paged_attention(q.data, ldq, kv.k, kv.v, dt(q, "q"), kv.table, kv.table_stride, batch.token_slot,
                                        batch.positions, out.data, static_cast<int>(qw), static_cast<int>(T), heads,
                                        kv_heads, head_dim, kv.page_tokens, kv.n_layers, kv.layer, scale, window, stream),
@@ -395,6 +426,7 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
             need(fresh->inv_freq->numel() == head_dim / 2, "attention_decode: the frequency table must have head_dim / 2 entries");
             cos_sin = rope_table(*fresh->inv_freq, kv.table_stride * kv.page_tokens);
         }
+        took(Path::AttentionDecodeFresh);
         kernel_check(celeg_attention_decode_fresh_bf16(
                          q.data, rows_of(q, "q"), fresh->k->data, rows_of(*fresh->k, "k"), fresh->v->data, rows_of(*fresh->v, "v"),
                          fresh->q_weight ? fresh->q_weight->as<float>() : nullptr, fresh->k_weight ? fresh->k_weight->as<float>() : nullptr,
@@ -404,6 +436,7 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
                      "attention for decode rows with fresh keys (bfloat16)");
         return;
     }
+    took(Path::AttentionDecode);
     kernel_check(celeg_attention_decode_bf16(q.data, rows_of(q, "q"), kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot,
                                              batch.positions, workspace, workspace + parts * head_dim, n_parts, out.data,
                                              heads * head_dim, T, heads, kv_heads, head_dim, kv.page_tokens, kv.n_layers,
@@ -631,6 +664,7 @@ void Ops::fused_linear(const Tensor& a, const Tensor& w, const Tensor& out, cons
         prm.seq_slot = c.seq_slot;
         prm.taps = static_cast<int>(L);
     }
+    took(sliced ? Path::FusedSliced : streamed ? Path::FusedRows : Path::FusedStaged);
     if (sliced) {
         kernel_check(celeg_gemv_slices(&prm, static_cast<int>(epi), stream), "fused_linear (k-sliced)");
     } else if (streamed) {
@@ -765,6 +799,7 @@ void Ops::tiled_linear(const Tensor& a, const Tensor& w, const Tensor& out, Epil
         }
         kernel_epilogue = 5;
     }
+    took(qkv ? Path::TiledQkv : Path::Tiled);
     kernel_check(celeg_gemm_tiles(&prm, kernel_epilogue, stream), "tiled_linear");
 }
 

@@ -84,10 +84,22 @@ struct StepPrologue {
     bool pending = false;
 };
 
+// Which kernel a call was handed to (counted per Ops at the time of the launch, also while a
+// graph records; a replay counts nothing): what tests and tools ask to see that a size took the
+// path it was meant to take.
+enum class Path : int {
+    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, LinearF32, LinearLibrary, LinearStandIn,
+    FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, Count
+};
+const char* path_name(Path p);
+
 class Ops {
 public:
     explicit Ops(hipStream_t stream) : stream(stream) {}
     hipStream_t stream;
+    long long path_count[static_cast<int>(Path::Count)] = {};
+    void took(Path p) { ++path_count[static_cast<int>(p)]; }
+    Json paths_json() const;
     // knobs (tests and tuning)
     int attention_decode_whole = -1;     // -1: chosen from the batch; 0 split-key kernels; 1 one workgroup per request and key/value head
     bool use_blaslt = true;

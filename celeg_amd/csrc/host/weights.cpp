@@ -191,7 +191,7 @@ TensorShapes Checkpoint::shapes() const {
 }
 
 // ---------------------------------------------------------------------------- checking
-void check_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected) {
+std::vector<std::string> check_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected, bool strict) {
     std::set<std::string> have;
     for (const auto& n : ckpt.names()) have.insert(n);
     std::set<std::string> wanted;
@@ -211,7 +211,12 @@ void check_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected) {
         if (!wanted.count(n)) unexpected.push_back(n);
     std::sort(missing.begin(), missing.end());
     missing.erase(std::unique(missing.begin(), missing.end()), missing.end());
-    if (missing.empty() && unexpected.empty() && wrong.empty()) return;
+    std::sort(unexpected.begin(), unexpected.end());
+    // Tensors are bound by name and what nobody asks for is left alone, as the reference does
+    // (include/celeg/checkpoint/weight_repository.hpp:14-20: a repository answers requests by
+    // name; src/checkpoint/formats/safetensors.cpp:283-297 fails on a missing tensor only): a tied
+    // model that still carries lm_head.weight, or an exported buffer, loads.  `strict` refuses them.
+    if (missing.empty() && wrong.empty() && (unexpected.empty() || !strict)) return unexpected;
     auto join = [](const std::vector<std::string>& v) {
         std::string out;
         for (size_t i = 0; i < v.size(); ++i) out += (i ? ", " : "") + v[i];
@@ -297,8 +302,10 @@ static std::shared_ptr<DeviceTensor> upload(const Checkpoint& ckpt, const std::s
     return t;
 }
 
-WeightMap load_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected, DType engine_dtype) {
-    check_tensors(ckpt, expected);
+WeightMap load_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected, DType engine_dtype, bool strict,
+                       std::vector<std::string>* unused) {
+    std::vector<std::string> left = check_tensors(ckpt, expected, strict);
+    if (unused) *unused = std::move(left);
     WeightMap out;
     for (const auto& e : expected)
         if (!out.count(e.first)) out[e.first] = upload(ckpt, e.first, e.second.kind, engine_dtype);

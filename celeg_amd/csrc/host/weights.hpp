@@ -89,8 +89,10 @@ struct WeightSpec {
 using ExpectedTensors = std::vector<std::pair<std::string, WeightSpec>>;   // checkpoint name -> spec
 
 // One WeightError that lists every missing tensor, every tensor the model has no use for and
-// every wrong shape.
-void check_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected);
+// every wrong shape, if a tensor is missing or has a wrong shape or dtype.  Tensors that the model
+// has no use for are no error by themselves unless `strict`: their names are returned (sorted),
+// for the caller to warn about.
+std::vector<std::string> check_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected, bool strict = false);
 
 struct DeviceTensor {
     DeviceBuffer buffer;
@@ -100,7 +102,8 @@ using WeightMap = std::map<std::string, std::shared_ptr<DeviceTensor>>;
 
 DType stored_as(const TensorInfo& info, const std::string& kind, DType engine_dtype);
 // check_tensors, then every expected tensor converted and copied to the device
-WeightMap load_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected, DType engine_dtype);
+WeightMap load_tensors(const Checkpoint& ckpt, const ExpectedTensors& expected, DType engine_dtype, bool strict = false,
+                       std::vector<std::string>* unused = nullptr);
 
 // device-side helpers parts use while they re-lay their weights at load time
 std::shared_ptr<DeviceTensor> device_tensor(DType dtype, std::initializer_list<long long> dims);

@@ -84,6 +84,10 @@ typedef struct celeg_engine_options {
     int32_t use_graphs;          /* 1: decode steps are replayed from recorded HIP graphs */
     int32_t run_ahead;           /* 1: celeg_engine_run launches decode steps one ahead of their tokens */
     int32_t portion_granule;
+    /* 0 (the default): tensors of the checkpoint that the model has no use for are named in a
+     * warning on stderr and in celeg_model_describe ("unused_tensors"), as the reference binds by
+     * name and leaves the rest alone; 1: they are an error */
+    int32_t strict_weights;
 } celeg_engine_options;
 
 /* max_new_tokens 128, priority 0 (include/celeg/runtime/request_types.hpp:16-26);
@@ -214,8 +218,10 @@ const char* celeg_describe_folder(const char* model_dir);
 /* the same from a config.json text alone (shapes_json: {"name": [dims]} or null) */
 const char* celeg_describe_config(const char* config_json, const char* shapes_json);
 /* checks the folder's checkpoint against the model: CELEG_OK, or CELEG_ERROR with one message that lists
- * missing and unexpected tensors and wrong shapes */
+ * missing and unexpected tensors and wrong shapes.  A checkpoint that only holds tensors the model has no
+ * use for passes (celeg_describe_folder names them under "unused_tensors") unless `strict`. */
 celeg_status celeg_check_folder(const char* model_dir);
+celeg_status celeg_check_folder_strict(const char* model_dir, int32_t strict);
 const char* celeg_registered(const char* what);   /* "architectures", or a role of parts: JSON list of names */
 
 /* ---- the host-side objects by themselves, without a GPU, by JSON calls (tests of the bookkeeping) ----

@@ -174,23 +174,33 @@ class LoadedModel:
     def knobs(self) -> Dict[str, int]:
         return self.native.knobs()
 
+    def paths(self) -> Dict[str, int]:
+        """How many launches each kernel family has taken so far (attention_decode,
+        attention_decode_fresh, attention_rows, attention_general, linear_f32, linear_library,
+        fused_sliced, fused_rows, fused_staged, tiled, tiled_qkv ...), counted when the host
+        launches (also while a graph records; a replay counts nothing)."""
+        return dict(self.native.knobs()["paths"])
+
     def close(self) -> None:
         self.native.close()
 
 
 def load_model(model_dir: str, *, dtype="bfloat16", device="cuda:0", page_tokens: int = 16,
                n_pages: Optional[int] = None, max_requests: int = 8, max_context: Optional[int] = None,
-               max_batched_tokens: int = 2048, gemm_backend: str = "auto", use_graphs: bool = True) -> LoadedModel:
+               max_batched_tokens: int = 2048, gemm_backend: str = "auto", use_graphs: bool = True,
+               strict_weights: bool = False) -> LoadedModel:
     """``n_pages``: pages of the cache pool (per group); by default enough for ``max_requests``
     requests of ``max_context`` tokens.  ``max_context`` defaults to the model's own maximum and
     may not exceed it.  ``gemm_backend``: how bfloat16 steps of more than 64 rows multiply:
     "library" (hipBLASLt, with separate norm and activation kernels), "tiles" (the library's own
     tiled products with the norm, SwiGLU and the residual sum folded in, where the sizes allow) or
-    "auto" (the one that was measured faster at the model's width; ``describe()`` says which)."""
+    "auto" (the one that was measured faster at the model's width; ``describe()`` says which).
+    ``strict_weights``: tensors of the checkpoint that the model has no use for are an error
+    instead of a warning (``describe()["unused_tensors"]`` names them)."""
     options = native.engine_options(dtype=parse_dtype(dtype), device=native.device_index(device),
                                     max_active_requests=max_requests, max_batched_tokens=max_batched_tokens,
                                     page_tokens=page_tokens, n_pages=n_pages, context=max_context,
-                                    gemm_backend=gemm_backend, use_graphs=use_graphs)
+                                    gemm_backend=gemm_backend, use_graphs=use_graphs, strict_weights=strict_weights)
     try:
         return LoadedModel(native.NativeModel.load(model_dir, options))
     except (native.NativeError, native.NativeArgumentError) as err:
@@ -208,7 +218,7 @@ class Engine:
                     max_batched_tokens: int = 2048, prefill_chunk_tokens: int = 1024,
                     context: Optional[int] = None, policy: str = "max_utilization",
                     gemm_backend: str = "auto", portion_granule: int = 1, use_graphs: bool = True,
-                    run_ahead: bool = True) -> "Engine":
+                    run_ahead: bool = True, strict_weights: bool = False) -> "Engine":
         # (Steps of 2,048 tokens and portions of 1,024: on an MI355X a step of a few hundred rows
         # leaves most of the chip idle; the reference's 512 / 256 are ``SchedulerOptions``'.)
         options = native.engine_options(dtype=parse_dtype(dtype), device=native.device_index(device),
@@ -217,7 +227,7 @@ class Engine:
                                         prefill_chunk_tokens=prefill_chunk_tokens, page_tokens=page_tokens,
                                         n_pages=n_pages, policy=policy, context=context,
                                         gemm_backend=gemm_backend, use_graphs=use_graphs, run_ahead=run_ahead,
-                                        portion_granule=portion_granule)
+                                        portion_granule=portion_granule, strict_weights=strict_weights)
         try:
             return cls(native.NativeEngine(model_dir, options))
         except (native.NativeError, native.NativeArgumentError) as err:

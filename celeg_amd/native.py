@@ -47,7 +47,8 @@ class EngineOptions(ctypes.Structure):
                 ("max_active_requests", c_int32), ("max_batched_tokens", c_int32),
                 ("prefill_chunk_tokens", c_int32), ("page_tokens", c_int32), ("logical_kv_pages", c_int32),
                 ("scheduler_policy", c_int32), ("context", c_int32), ("gemm_backend", c_int32),
-                ("use_graphs", c_int32), ("run_ahead", c_int32), ("portion_granule", c_int32)]
+                ("use_graphs", c_int32), ("run_ahead", c_int32), ("portion_granule", c_int32),
+                ("strict_weights", c_int32)]
 
 
 class RequestOptionsStruct(ctypes.Structure):
@@ -163,6 +164,7 @@ def lib() -> ctypes.CDLL:
     sig("celeg_describe_folder", c_char_p, c_char_p)
     sig("celeg_describe_config", c_char_p, c_char_p, c_char_p)
     sig("celeg_check_folder", c_int, c_char_p)
+    sig("celeg_check_folder_strict", c_int, c_char_p, c_int32)
     sig("celeg_registered", c_char_p, c_char_p)
     sig("celeg_host_new", ctypes.c_longlong, c_char_p, c_char_p)
     sig("celeg_host_call", c_char_p, ctypes.c_longlong, c_char_p, c_char_p)
@@ -213,8 +215,8 @@ def describe_config(config: Dict[str, Any], tensor_shapes: Optional[Dict[str, Se
     return json.loads(_text(lib().celeg_describe_config(json.dumps(config).encode(), shapes)))
 
 
-def check_folder(model_dir: str) -> None:
-    check(lib().celeg_check_folder(model_dir.encode()))
+def check_folder(model_dir: str, strict: bool = False) -> None:
+    check(lib().celeg_check_folder_strict(model_dir.encode(), int(bool(strict))))
 
 
 def registered(what: str) -> List[str]:
@@ -225,7 +227,7 @@ def registered(what: str) -> List[str]:
 def engine_options(*, dtype="bfloat16", device=0, max_active_requests=8, max_batched_tokens=2048,
                    prefill_chunk_tokens=1024, page_tokens=16, n_pages=None, policy="max_utilization",
                    context=None, gemm_backend="auto", use_graphs=True, run_ahead=True,
-                   portion_granule=1) -> EngineOptions:
+                   portion_granule=1, strict_weights=False) -> EngineOptions:
     if policy not in ("max_utilization", "guaranteed_no_evict"):
         raise NativeArgumentError("policy must be max_utilization or guaranteed_no_evict")
     if gemm_backend not in ("library", "tiles", "auto"):
@@ -241,6 +243,7 @@ def engine_options(*, dtype="bfloat16", device=0, max_active_requests=8, max_bat
     o.context = int(context) if context else 0
     o.gemm_backend = {"library": 0, "tiles": 1, "auto": 2}[gemm_backend]
     o.use_graphs, o.run_ahead, o.portion_granule = int(bool(use_graphs)), int(bool(run_ahead)), int(portion_granule)
+    o.strict_weights = int(bool(strict_weights))
     return o
 
 

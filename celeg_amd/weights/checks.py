@@ -2,7 +2,10 @@
 
 Opening the container (one file or a sharded index), its validation, the check and the way to
 the device are the library's (``csrc/host/weights.cpp``).  ALL problems of a checkpoint come as
-one error: missing tensors, tensors nobody asked for, and wrong shapes.
+one error: missing tensors, tensors nobody asked for, and wrong shapes.  Tensors nobody asked
+for are no problem by themselves (the reference binds tensors by name and leaves the rest alone,
+include/celeg/checkpoint/weight_repository.hpp:14-20): loading warns about them, and ``strict``
+makes them an error.
 """
 from __future__ import annotations
 
@@ -39,12 +42,12 @@ def translate(err: Exception) -> Exception:
     return err
 
 
-def check_folder(model_dir: str) -> None:
+def check_folder(model_dir: str, strict: bool = False) -> None:
     """Raises ``WeightError`` (the checkpoint does not fit), ``SafetensorsError`` (a malformed
     container), ``FileNotFoundError`` or ``ConfigError``; returns None if the folder loads."""
     from ..config.registry import ConfigError
     try:
-        native.check_folder(model_dir)
+        native.check_folder(model_dir, strict)
     except native.NativeArgumentError as err:
         translated = translate(err)
         raise (translated if translated is not err else ConfigError(str(err))) from None

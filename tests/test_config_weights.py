@@ -259,6 +259,34 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert word in text
 
 
+def test_tensors_nobody_asks_for_are_a_warning_unless_strict(tmp_path):
+    """The reference binds tensors by name and leaves the rest alone
+    (include/celeg/checkpoint/weight_repository.hpp:14-20; src/checkpoint/formats/safetensors.cpp:283-297
+    fails on a missing tensor only): a tied model whose checkpoint still carries lm_head.weight, or an
+    exported buffer, is no error.  The description names what is left over; a strict check refuses it."""
+    folder = write_random_model(TINY_A, str(tmp_path / "m"), seed=3, dtype=torch.float32)
+    path = os.path.join(folder, "model.safetensors")
+    f = SafetensorsFile(path)
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    f.close()
+    assert "lm_head.weight" not in tensors                     # Tiny A ties its head to the embedding
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    tensors["model.rotary_emb.inv_freq"] = torch.zeros(8)
+    write_safetensors(path, tensors)
+    check_folder(folder)
+    assert native.describe_folder(folder)["unused_tensors"] == ["lm_head.weight", "model.rotary_emb.inv_freq"]
+    with pytest.raises(WeightError) as info:
+        check_folder(folder, strict=True)
+    assert info.value.unexpected == ["lm_head.weight", "model.rotary_emb.inv_freq"] and not info.value.missing
+    # beside a real fault they are still listed, in the one error
+    del tensors["model.layers.0.operator_norm.weight"]
+    write_safetensors(path, tensors)
+    with pytest.raises(WeightError) as info:
+        check_folder(folder)
+    assert info.value.missing == ["model.layers.0.operator_norm.weight"]
+    assert info.value.unexpected == ["lm_head.weight", "model.rotary_emb.inv_freq"]
+
+
 def test_conv_filter_is_accepted_in_both_shapes_and_bias_is_required(tmp_path):
     folder = write_random_model(TINY_B, str(tmp_path / "m"), seed=3, dtype=torch.float32)
     path = os.path.join(folder, "model.safetensors")

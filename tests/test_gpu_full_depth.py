@@ -40,6 +40,24 @@ def test_logits_at_the_benchmarks_configuration(benchmark_model):
     lm.close()
 
 
+def test_32bit_logits_at_the_benchmarks_depth(benchmark_model):
+    """All 16 layers in true 32-bit (the same folder, its bfloat16 weights widened exactly):
+    two short requests, most in one step and the last tokens one by one, then in portions,
+    against the plain implementation at the 32-bit bound."""
+    from celeg_amd.engine import load_model
+    from helpers import assert_close_f32
+    folder, cfg, W = benchmark_model
+    reqs = {"a": random_tokens(cfg["vocab_size"], 64, seed=5), "b": random_tokens(cfg["vocab_size"], 41, seed=6)}
+    ref = {rid: plain.model_logits(cfg, W, toks) for rid, toks in reqs.items()}
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2, max_context=128,
+                    max_batched_tokens=64)
+    for mode, schedule in (("tail", lambda r: tail_decode_schedule(r, tail=12)), ("portions", portions_schedule)):
+        got = EngineDriver(lm).run(schedule(reqs))
+        for rid in reqs:
+            assert_close_f32(got[rid], ref[rid], f"benchmark depth, 32-bit/{mode}/{rid}")
+    lm.close()
+
+
 def test_greedy_tokens_at_the_benchmarks_configuration(benchmark_model):
     from celeg_amd.engine import Engine
     from celeg_amd.sampling import GREEDY

@@ -391,3 +391,36 @@ def test_cancelling_while_steps_run_ahead(model_folders):
         engine.release(rid)
     with pytest.raises(Exception, match="unknown request id"):
         engine.status(after)
+
+
+def test_a_checkpoint_with_tensors_nobody_asks_for_loads_and_generates(model_folders, tmp_path, capfd):
+    """A tied model whose checkpoint still carries lm_head.weight (filled with other values) and an
+    exported buffer: the reference binds tensors by name and leaves the rest alone
+    (include/celeg/checkpoint/weight_repository.hpp:14-20), and so does loading here: a warning
+    names them, the description lists them, and the tokens are those of the folder without them.
+    With strict_weights the same folder is refused."""
+    import shutil
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY
+    from celeg_amd.weights import SafetensorsFile, WeightError, write_safetensors
+    src = model_folders("A", torch.float32, WEIGHT_STD)
+    folder = str(tmp_path / "extra")
+    os.makedirs(folder)
+    shutil.copy(os.path.join(src, "config.json"), folder)
+    f = SafetensorsFile(os.path.join(src, "model.safetensors"))
+    tensors = {n: f.tensor(n).clone() for n in f.names()}
+    f.close()
+    tensors["lm_head.weight"] = torch.randn_like(tensors["model.embed_tokens.weight"])
+    tensors["model.rotary_emb.inv_freq"] = torch.zeros(8)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    prompts = [random_tokens(256, n, seed=70 + n) for n in (9, 21)]
+    outs = {}
+    for name, where in (("plain", src), ("extra", folder)):
+        engine = Engine.from_folder(where, dtype="float32", max_active_requests=2, n_pages=8, max_batched_tokens=32)
+        outs[name] = engine.generate(prompts, max_new_tokens=8, generation=GREEDY, eos_token_ids=[])
+        if name == "extra":
+            assert engine.loaded.native.info["unused_tensors"] == ["lm_head.weight", "model.rotary_emb.inv_freq"]
+    assert outs["extra"] == outs["plain"]
+    assert "lm_head.weight" in capfd.readouterr().err
+    with pytest.raises(WeightError, match="unexpected tensors"):
+        Engine.from_folder(folder, dtype="float32", max_active_requests=2, n_pages=8, strict_weights=True)

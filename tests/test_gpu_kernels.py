@@ -441,16 +441,20 @@ def attention_case(ops, dtype, heads, kv_heads, head_dim, lengths, cuts, window=
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,kv_heads,head_dim", [(16, 8, 64), (4, 2, 128), (10, 5, 32)])
-def test_norm_rope_store_of_a_long_step_equals_short_steps(ops, dtype, heads, kv_heads, head_dim):
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page_tokens", [(16, 8, 64, 16), (4, 2, 128, 16), (10, 5, 32, 16),
+                                                                 (16, 8, 64, 2), (10, 5, 32, 6), (4, 2, 128, 1)])
+def test_norm_rope_store_of_a_long_step_equals_short_steps(ops, dtype, heads, kv_heads, head_dim, page_tokens):
     """A step of thousands of rows takes four rows a thread (values of four neighbouring rows
     leave as one store); the same rows in steps of a few hundred take one row a thread.  Three
     requests whose portions start at positions 0, 5 and 1, so that runs of four rows start on a
     multiple of four, in the middle of one, and straddle the border between two requests: the
-    queries and both caches must come out the same bit for bit."""
+    queries and both caches must come out the same bit for bit.  With pages of 1, 2 and 6 tokens
+    four neighbouring rows do not lie side by side in one page (or not at an address that a store
+    of four takes): they must go row by row, and what the pages hold is compared with the rows
+    themselves."""
     from celeg_amd.engine import StepEntry
     starts, lengths = [0, 5, 1], [2503, 1202, 650]
-    n_layers, layer, page_tokens = 2, 1, 16
+    n_layers, layer = 2, 1
     qw = 1 + randn(head_dim, seed=20, scale=0.1)
     kw = 1 + randn(head_dim, seed=21, scale=0.1)
     inv_freq = torch.tensor(plain.rope_inverse_frequencies(10000.0, head_dim), dtype=torch.float64).float().to(DEV)
@@ -494,6 +498,13 @@ def test_norm_rope_store_of_a_long_step_equals_short_steps(ops, dtype, heads, kv
         pages = [int(table[slot, p]) for slot, start, n in zip(slots, starts, lengths)
                  for p in range((start + n + page_tokens - 1) // page_tokens)]
         results.append((q_out.clone(), kv.k[pages].clone(), kv.v[pages].clone(), [int(x) for x in starts]))
+        # the values are stored as they came: position p of a request in page p // page_tokens, place p % page_tokens
+        row0 = 0
+        for slot, start, n in zip(slots, starts, lengths):
+            mine = table[slot, :(start + n + page_tokens - 1) // page_tokens].long().to(DEV)
+            held = kv.v[mine, layer].permute(1, 2, 0, 3).reshape(kv_heads, head_dim, -1)[:, :, start:start + n]
+            assert torch.equal(held.permute(2, 0, 1).reshape(n, -1), v0[row0:row0 + n])
+            row0 += n
     (qa, ka, va, _), (qb, kb, vb, _) = results
     assert torch.equal(qa, qb)
     assert torch.equal(ka, kb) and torch.equal(va, vb)

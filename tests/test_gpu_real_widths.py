@@ -1,8 +1,9 @@
-"""The engine against the plain implementation at the real layer sizes: three-layer slices
-(convolution, attention, convolution) with the widths, head counts, feed-forward sizes and
-the vocabulary of 65,536 of the LFM2-350M shape and of the LFM2-1.2B / 2.6B shape, so that
+"""The engine against the plain implementation at the real layer sizes: slices of three or four
+layers with the widths, head counts, feed-forward sizes and the vocabulary of 65,536 of the
+LFM2-350M, LFM2-1.2B and LFM2-2.6B shapes (the last with its own feed-forward of 7,168 columns
+and an attention layer followed by three convolution layers, as that model orders them), so that
 every product runs through the kernel (and the tiles of it) that the real model takes: the
-output head through the wide-product kernels, the feed-forward at 4,608 and 8,192 columns.
+output head through the wide-product kernels, the feed-forward at 4,608, 8,192 and 7,168 columns.
 Requests are short (up to 128 tokens) so that the float64 plain implementation stays fast."""
 import pytest
 import torch
@@ -25,7 +26,10 @@ BASE = {
 WIDTHS = {
     "350m": dict(BASE, hidden_size=1024, num_attention_heads=16, intermediate_size=6656),    # ff 4608
     "1.2b": dict(BASE, hidden_size=2048, num_attention_heads=32, intermediate_size=12288),   # ff 8192
+    "2.6b": dict(BASE, hidden_size=2048, num_attention_heads=32, intermediate_size=10752,    # ff 7168
+                 num_hidden_layers=4, layer_types=["full_attention", "conv", "conv", "conv"]),
 }
+FF = {"350m": 4608, "1.2b": 8192, "2.6b": 7168}
 LENGTHS = [128, 70, 100, 45, 33]
 SCHEDULES = {"whole": whole_schedule, "tail32": tail_decode_schedule,
              "portions": portions_schedule, "mixed": mixed_schedule}
@@ -49,18 +53,16 @@ def folder_of(tmp_path_factory, shape, storage):
 def plain_logits(folder, key):
     if key not in _plain:
         cfg, W = plain.load_model_folder(folder)
-        assert plain.ff_dim(cfg["intermediate_size"], True, 256) == W["model.layers.0.feed_forward.w1.weight"].shape[0]
+        assert plain.ff_dim(cfg["intermediate_size"], True, 256) == W["model.layers.0.feed_forward.w1.weight"].shape[0] == FF[key[0]]
         _plain[key] = {rid: plain.model_logits(cfg, W, toks).float() for rid, toks in requests().items()}
     return _plain[key]
 
 
 @pytest.mark.parametrize("mode", list(SCHEDULES))
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", ["350m", "1.2b"])
+@pytest.mark.parametrize("shape", ["350m", "1.2b", "2.6b"])
 def test_engine_matches_plain_at_real_layer_sizes(tmp_path_factory, shape, dtype, mode):
     from celeg_amd.engine import load_model
-    if shape == "1.2b" and mode in ("tail32", "portions"):
-        pytest.skip("the wider shape runs the whole and the mixed schedule (time)")
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = folder_of(tmp_path_factory, shape, storage)
     reqs = requests()
