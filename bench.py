@@ -195,7 +195,7 @@ def main() -> int:
     for knob in args.knob:
         name, _, value = knob.partition("=")
         lm.set_knob(name, int(value))
-    ff = lm.config.ff_dim
+    ff = int(lm.native.info["spec"]["layers"][0]["ffn"]["params"]["ff"])      # from the parts list, whatever the architecture
     w_bytes = lm.native.info["weights"] * 2          # every weight once, bfloat16
     kv_per_token = lm.native.info["kv_bytes_per_token"]
 

@@ -26,6 +26,21 @@ def _describe(cfg: Mapping[str, Any], tensor_shapes=None) -> Dict[str, Any]:
         raise ConfigError(str(err)) from None
 
 
+# Typed views of configurations, by architecture: a function from the library's typed configuration
+# (a dictionary) to whatever Python object stands for it.  An architecture without a view is seen
+# as the dictionary itself.  The generic code below and the engine ask this table only.
+_typed_views: Dict[str, Callable[[Mapping[str, Any]], Any]] = {}
+
+
+def register_typed_view(architecture: str, view: Callable[[Mapping[str, Any]], Any]) -> None:
+    _typed_views[architecture] = view
+
+
+def typed_config(architecture: str, config: Mapping[str, Any]):
+    view = _typed_views.get(architecture)
+    return view(config) if view else config
+
+
 @dataclass(frozen=True)
 class Lfm2Config:
     """The typed LFM2 configuration: every key the library reads, defaults filled in."""
@@ -64,7 +79,7 @@ class Lfm2Config:
     @classmethod
     def from_dict(cls, cfg: Mapping[str, Any], tensor_shapes=None) -> "Lfm2Config":
         cfg = dict(cfg)
-        cfg.setdefault("architectures", ["Lfm2ForCausalLM"])
+        cfg.setdefault("architectures", [cls.architecture])
         return cls.from_typed(_describe(cfg, tensor_shapes)["config"])
 
     def to_dict(self) -> Dict[str, Any]:
@@ -76,10 +91,13 @@ class Lfm2Config:
         return out
 
 
+register_typed_view(Lfm2Config.architecture, Lfm2Config.from_typed)
+
+
 def feed_forward_width(intermediate_size: int, auto_adjust: bool, multiple_of: int,
                        multiplier: Optional[float]) -> int:
     """The SwiGLU width the library computes for these keys."""
-    cfg = {"architectures": ["Lfm2ForCausalLM"], "vocab_size": 8, "hidden_size": 8, "num_hidden_layers": 1,
+    cfg = {"architectures": [Lfm2Config.architecture], "vocab_size": 8, "hidden_size": 8, "num_hidden_layers": 1,
            "num_attention_heads": 1, "layer_types": ["conv"], "conv_L_cache": 1, "rope_theta": 1.0,
            "max_position_embeddings": 8, "intermediate_size": intermediate_size,
            "block_auto_adjust_ff_dim": auto_adjust, "block_multiple_of": multiple_of,
@@ -130,10 +148,7 @@ def read_config_file(model_dir: str) -> Dict[str, Any]:
 
 
 def _typed(described: Dict[str, Any]):
-    config = described["config"]
-    if described["spec"]["architecture"] == "Lfm2ForCausalLM":
-        config = Lfm2Config.from_typed(config)
-    return config
+    return typed_config(described["spec"]["architecture"], described["config"])
 
 
 def spec_from_config(cfg: Mapping[str, Any], tensor_shapes=None):

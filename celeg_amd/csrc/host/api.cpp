@@ -375,7 +375,8 @@ const char* celeg_model_describe(celeg_model* model) {
                 .set("dtype", dtype_name(lm.rt->dtype)).set("weights", lm.model->weight_count())
                 .set("kv_bytes_per_token", lm.cache->layout.kv_bytes_per_token(dtype_size(lm.rt->dtype)))
                 .set("eos_token_ids", Json::array_of(lm.model->spec.eos_token_ids))
-                .set("gemm_backend", lm.rt->use_tiled_products ? "tiles" : "library")
+                .set("gemm_backend", lm.model->spec.hidden_size <= lm.rt->tiled_max_width ? "tiles" : "library")
+                .set("tiled_max_width", lm.rt->tiled_max_width)
                 .set("unused_tensors", Json::array_of(lm.unused_tensors));
             out = j.dump();
         }) != CELEG_OK)
@@ -597,7 +598,11 @@ const std::vector<Knob>& knobs() {
          [](LoadedModel& m, int v) { m.runner->portion_graph_min_tokens = v; }},
         {"use_fused", [](LoadedModel& m) { return m.rt->use_fused ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->use_fused = v != 0; }},
         {"defer_prologue", [](LoadedModel& m) { return m.rt->defer_prologue ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->defer_prologue = v != 0; }},
-        {"use_tiled_products", [](LoadedModel& m) { return m.rt->use_tiled_products ? 1 : 0; }, [](LoadedModel& m, int v) { m.rt->use_tiled_products = v != 0; }},
+        // (use_tiled_products: 1 = always, 0 = never; tiled_max_width is the rule itself)
+        {"use_tiled_products", [](LoadedModel& m) { return m.model->spec.hidden_size <= m.rt->tiled_max_width ? 1 : 0; },
+         [](LoadedModel& m, int v) { m.rt->tiled_max_width = v ? (1LL << 40) : 0; }},
+        {"tiled_max_width", [](LoadedModel& m) { return static_cast<int>(std::min<long long>(m.rt->tiled_max_width, 1 << 30)); },
+         [](LoadedModel& m, int v) { m.rt->tiled_max_width = v; }},
         {"fused_max_rows", [](LoadedModel& m) { return m.rt->fused_max_rows; }, [](LoadedModel& m, int v) { m.rt->fused_max_rows = v; }},
         OPS_INT(attention_decode_whole), OPS_BOOL(use_blaslt), OPS_INT(attention_rows_per_tile), OPS_INT(attention_rows_form),
         OPS_BOOL(attention_general), OPS_BOOL(use_rope_table), OPS_BOOL(use_argmax_parts), OPS_BOOL(use_sliced),
@@ -655,36 +660,6 @@ void* celeg_model_stream(celeg_model* model) { return model ? model->lm->stream 
 celeg_status celeg_model_synchronize(celeg_model* model) {
     if (!model) return CELEG_INVALID_ARGUMENT;
     return guarded([&] { CELEG_HIP(hipStreamSynchronize(model->lm->stream)); });
-}
-
-// ---------------------------------------------------------------------------- the dispatch alone
-// Ops::linear on raw device pointers: what the tests of the products call, so that they go
-// through the dispatch that the parts use (the 32-bit kernel, the kernels for few rows, the
-// library above 64 rows and what stands in where it has no kernel).
-celeg_status celeg_ops_linear(const void* x, int32_t x_dtype, int64_t x_row_stride, const void* w, int32_t w_dtype,
-                              void* out, int32_t out_dtype, int64_t out_row_stride, const float* bias, int32_t M,
-                              int32_t N, int32_t K, int32_t use_library, void* stream) {
-    if (!x || !w || !out || M <= 0 || N <= 0 || K <= 0) return CELEG_INVALID_ARGUMENT;
-    return guarded([&] {
-        // one dispatcher for the process (its library plans and workspace are made at the first
-        // call of a size, so a call that a graph records finds them there), on the caller's stream
-        static std::mutex lock;
-        static Ops ops(nullptr);
-        static Workspace ws;
-        std::lock_guard<std::mutex> guard(lock);
-        ops.stream = static_cast<hipStream_t>(stream);
-        auto view = [](const void* p, int32_t dtype, long long rows, long long cols, long long row_stride) {
-            Tensor t = Tensor::make(const_cast<void*>(p), static_cast<DType>(dtype), {rows, cols});
-            t.stride[0] = row_stride;
-            return t;
-        };
-        const Tensor xt = view(x, x_dtype, M, K, x_row_stride), wt = view(w, w_dtype, N, K, K);
-        const Tensor ot = view(out, out_dtype, M, N, out_row_stride);
-        Tensor bt;
-        if (bias) bt = Tensor::make(const_cast<float*>(bias), DType::F32, {static_cast<long long>(N)});
-        ops.use_blaslt = use_library != 0;
-        ops.linear(xt, wt, ot, bias ? &bt : nullptr, ws);
-    });
 }
 
 // ---------------------------------------------------------------------------- descriptions

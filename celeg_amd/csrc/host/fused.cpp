@@ -5,11 +5,12 @@
 namespace celeg {
 namespace fused {
 
-// Whether a step of `rows` rows is one of many rows that takes the fused path through the
-// tiled products (Runtime::use_tiled_products; otherwise steps of many rows run the library's
-// products with separate norm and activation kernels).
-bool tiled_step(const Runtime& rt, int rows) {
-    return rows > FUSED_MAX_ROWS && rt.use_tiled_products && rt.dtype == DType::BF16 && rt.use_fused;
+// Whether products of `rows` rows that read a stream of this width take the fused path through
+// the tiled products (otherwise they run the library's products with separate norm and activation
+// kernels).  The choice is by the sizes of the products, not by the model: Runtime::tiled_max_width
+// holds the widest stream for which the tiled products were measured faster.
+bool tiled_step(const Runtime& rt, int rows, long long width) {
+    return rows > FUSED_MAX_ROWS && width <= rt.tiled_max_width && rt.dtype == DType::BF16 && rt.use_fused;
 }
 
 // Whether this step's rows can take the fused path through products with these inner sizes.
@@ -19,7 +20,9 @@ bool fused_rows_ok(const Runtime& rt, const StepBatch& batch, std::initializer_l
     for (long long k : inner) widest = std::max(widest, k);
     if (rows > FUSED_MAX_ROWS)
         // every inner size is also the width of some product's output
-        return tiled_step(rt, rows) && rt.ops.tiled_linear_ok(rows, 4, inner) && widest <= 64 * TILED_MAX_STAT_BLOCKS;
+        // (the first inner size is the width of the stream)
+        return inner.size() > 0 && tiled_step(rt, rows, *inner.begin()) && rt.ops.tiled_linear_ok(rows, 4, inner) &&
+               widest <= 64 * TILED_MAX_STAT_BLOCKS;
     if (!(rt.dtype == DType::BF16 && rt.use_fused && rt.ops.fused_linear_ok(rows, inner))) return false;
     int limit = rt.fused_max_rows;
     if (limit < 0) limit = rt.ops.rows_kernel_ok(rows, inner) ? FUSED_MAX_ROWS : FUSED_MAX_ROWS_OLD_KERNEL;
@@ -95,7 +98,7 @@ std::shared_ptr<DeviceTensor> packed_weight(Runtime& rt, const Tensor& w) {
 }
 }  // namespace
 
-bool qkv_tail_ok(const Runtime& rt, int rows) { return tiled_step(rt, rows); }
+bool qkv_tail_ok(const Runtime& rt, int rows, long long width) { return tiled_step(rt, rows, width); }
 
 void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const Tensor& w, const Tensor& out,
                  Epilogue epilogue, const LinearExtras& extras) {
@@ -103,7 +106,7 @@ void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const
     const int T = static_cast<int>(h.shape[0]);
     const long long width = h.shape[1];
     const int M = extras.n_rows >= 0 ? extras.n_rows : T;
-    if (tiled_step(rt, T)) {
+    if (tiled_step(rt, T, width)) {
         if (extras.rows || (epilogue != Epilogue::Store && epilogue != Epilogue::Swiglu) || w.dtype != DType::BF16)
             throw KernelError("norm_linear: not a product of the path for many rows");
         Tensor stats = stream_stats(rt, width, T);
@@ -160,7 +163,7 @@ void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const
 void linear_into_stream(Runtime& rt, const Tensor& a, const Tensor& w, const Tensor& h, const Tensor* bias) {
     const int T = static_cast<int>(h.shape[0]);
     const long long width = h.shape[1];
-    if (tiled_step(rt, T)) {
+    if (tiled_step(rt, T, width)) {
         Tensor stats = stream_stats(rt, width, T);
         Tensor xb = stream_bf16(rt, T, width);
         rt.ops.tiled_linear(a, w, h, Epilogue::Residual, 0.f, nullptr, 0, bias, &stats, &xb);

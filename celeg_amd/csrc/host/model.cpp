@@ -533,12 +533,9 @@ std::unique_ptr<LoadedModel> load_model(const std::string& model_dir, const Load
     lm->config = described.config;
     CELEG_HIP(hipStreamCreate(&lm->stream));
     lm->rt = std::make_unique<Runtime>(dtype, lm->stream);
-    // "auto": measured on 2,048 rows, whole prefill.  At a width of 1,024 (K of most products) the
-    // tiled products with their folded norms and SwiGLU take 2.33 ms against 2.72 ms through the
-    // library and the separate kernels it needs; at 2,048 the library's products run at 1.2
-    // PFLOP/s and win (5.5 against 6.2 ms, 9.3 against 11.0 ms at the two larger shapes).
-    lm->rt->use_tiled_products = options.gemm_backend == "tiles" ||
-                                 (options.gemm_backend == "auto" && described.spec.hidden_size <= 1024);
+    // "auto" keeps the runtime's own rule, which goes by the sizes of the products
+    if (options.gemm_backend == "tiles") lm->rt->tiled_max_width = 1LL << 40;
+    if (options.gemm_backend == "library") lm->rt->tiled_max_width = 0;
     lm->model = std::make_unique<Model>(described.spec);
     {
         WeightMap tensors = load_tensors(ckpt, lm->model->expected_tensors(), dtype, options.strict_weights,

@@ -275,6 +275,17 @@ const float* Ops::rope_table(const Tensor& inv_freq, int n_positions) {
     return it->second->view.as<float>();
 }
 
+void Ops::forget_rope_tables(const void* inv_freq) {
+    for (auto it = rope_tables_.begin(); it != rope_tables_.end();) {
+        if (it->first.first == inv_freq) {
+            retired_rope_tables_.push_back(it->second);
+            it = rope_tables_.erase(it);
+        } else {
+            ++it;
+        }
+    }
+}
+
 void Ops::qk_norm_rope_store(const Tensor& q, const Tensor* k, const Tensor* v, const Tensor* q_weight,
                              const Tensor* k_weight, float eps, const Tensor* inv_freq, int rotary_dim, int pairing, int heads,
                              int kv_heads, int head_dim, const StepBatch& batch, const KVView& kv) {

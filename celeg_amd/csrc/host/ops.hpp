@@ -161,11 +161,17 @@ public:
     // weights re-laid at load time: w [rows, K] scaled by a norm's weight (or not) and, if
     // `packed`, laid as [K/32, rows, 32]
     std::shared_ptr<DeviceTensor> fold_weight(const Tensor& w, const Tensor* scale, bool packed);
+    // The tables of cosines and sines are kept by the address of their frequencies, which a model's
+    // position encoding owns for as long as the dispatcher lives.  A caller whose frequency tensors
+    // come and go (an address may then name other frequencies later) says so here: the tables made
+    // for this address are set aside (not freed: a recorded graph may still read them) and made anew.
+    void forget_rope_tables(const void* inv_freq);
 
 private:
     std::unique_ptr<BlasLt> blaslt_;
     DeviceBuffer argmax_state_;
     std::map<std::pair<const void*, int>, std::shared_ptr<DeviceTensor>> rope_tables_;
+    std::vector<std::shared_ptr<DeviceTensor>> retired_rope_tables_;
     const float* rope_table(const Tensor& inv_freq, int n_positions);
     void attention_decode(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
                           int window, const StepBatch& batch, const KVView& kv, int T, Workspace& ws, const FreshKV* fresh = nullptr);
@@ -182,7 +188,14 @@ struct Runtime {
     Ops ops;
     Workspace ws;
     bool use_fused = true;
-    bool use_tiled_products = false;
+    // Steps of more than 64 bfloat16 rows: products that read a stream of up to this width go
+    // through the tiled products with the norm, SwiGLU and residual sum folded in, wider ones
+    // through the library's products with separate norm and activation kernels.  The default is
+    // what was measured on whole prefills of 2,048 tokens: at a width of 1,024 the tiled path
+    // takes 2.33 ms against 2.72 ms, at 2,048 the library's products run at 1.2 PFLOP/s and win
+    // (5.5 against 6.2 ms and 9.3 against 11.0 ms for 16 and 30 layers).  0: always the library;
+    // a large number: always the tiles.
+    long long tiled_max_width = 1024;
     int fused_max_rows = -1;            // -1: by the kernels' own limits
     // how many partial sums of squares of the stream's rows are valid (0: none), and whether
     // the stream's bfloat16 copy is; whoever writes the stream another way resets them

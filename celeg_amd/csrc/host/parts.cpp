@@ -339,7 +339,7 @@ private:
         bool finished = false;      // norm, rotation and cache write made by the product's own kernel
         if (writes) {
             Tensor qkv = rt.ws.buf("attn_qkv", rt.dtype, {T, qw + 2 * kvw});
-            if (norm && fused::qkv_tail_ok(rt, static_cast<int>(T)) && T == batch.n_tokens &&
+            if (norm && fused::qkv_tail_ok(rt, static_cast<int>(T), width_) && T == batch.n_tokens &&
                 rt.ops.tiled_qkv_ok(head_dim_, inv_freq, tables.rotary_dim, tables.pairing, *cache.kv)) {
                 QkvTail tail;
                 tail.heads = heads_;
@@ -466,7 +466,7 @@ public:
         fused::LinearExtras extras;
         if (b_in_) extras.bias = b_in_->view;
         Tensor y;
-        if (batch.decode_only && batch.n_seqs == T && taps_ <= 8 && !fused::tiled_step(rt, T)) {   // the fused form holds 8 taps
+        if (batch.decode_only && batch.n_seqs == T && taps_ <= 8 && !fused::tiled_step(rt, T, width_)) {   // the fused form holds 8 taps
             y = fused::operand_rows(rt, "conv_y_fused", T, width_, {width_});
             ConvOperands conv;
             conv.taps = taps_view_;
@@ -585,7 +585,7 @@ public:
         if (batch && table_->view.dtype == DType::BF16 && fused::fused_rows_ok(rt, *batch, {width_})) {
             // few rows: leave every row's sum of squares (and the bfloat16 copy of the stream)
             // for the first norm
-            if (fused::sliced(rt, rows, width_) || fused::tiled_step(rt, rows)) {
+            if (fused::sliced(rt, rows, width_) || fused::tiled_step(rt, rows, width_)) {
                 // (the step's prologue rides along where it is for these rows)
                 const bool along = rt.prologue.pending && rt.prologue.token_ids == token_ids && rt.prologue.n == rows;
                 if (!along) rt.flush_prologue();
@@ -615,7 +615,7 @@ bool head_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& ba
                 const Tensor& weight) {
     const int R = batch.n_logit_rows;
     if (!(weight.defined() && weight.dtype == DType::BF16 && fused::fused_rows_ok(rt, batch, {h.shape[1]}) && R > 0 && R <= 64 &&
-          !fused::tiled_step(rt, batch.n_tokens)))
+          !fused::tiled_step(rt, batch.n_tokens, h.shape[1])))
         return false;
     fused::LinearExtras extras;
     extras.rows = batch.logit_rows;

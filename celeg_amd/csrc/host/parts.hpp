@@ -161,7 +161,7 @@ constexpr int FUSED_MAX_ROWS_OLD_KERNEL = 32;  // else; above it the library's p
 constexpr int TILED_MAX_STAT_BLOCKS = 128;
 constexpr int SLICED_MAX_ROWS = 16, SLICED_MAX_STAT_BLOCKS = 512, SLICED_MAX_COLUMNS = 16384;
 
-bool tiled_step(const Runtime& rt, int rows);
+bool tiled_step(const Runtime& rt, int rows, long long width);
 bool fused_rows_ok(const Runtime& rt, const StepBatch& batch, std::initializer_list<long long> inner);
 Tensor stream_stats(Runtime& rt, long long width, int rows = 0);
 Tensor operand_rows(Runtime& rt, const std::string& name, int rows, long long width, std::initializer_list<long long> producer_inner);
@@ -176,7 +176,7 @@ struct LinearExtras {
     const QkvTail* qkv = nullptr;          // steps of many rows: what follows a q/k/v product, inside its kernel
 };
 // whether norm_linear would take a q/k/v tail for a step of this many rows
-bool qkv_tail_ok(const Runtime& rt, int rows);
+bool qkv_tail_ok(const Runtime& rt, int rows, long long width);
 // out = epilogue(norm(h) w^T), the norm applied while the rows of h are read
 void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const Tensor& w, const Tensor& out,
                  Epilogue epilogue, const LinearExtras& extras = {});

@@ -202,14 +202,21 @@ void* celeg_model_stream(celeg_model* model);
 /* waits for everything launched on that stream */
 celeg_status celeg_model_synchronize(celeg_model* model);
 
-/* ---- the products' dispatch alone (tests) ----
- * out [M, N] = x [M, K] w[N, K]^T (+ bias, 32-bit [N]) on `stream` (a hipStream_t), by the kernels the
- * parts would get for these sizes and dtypes (0 float32, 1 bfloat16); rows of x and out lie
- * x_row_stride / out_row_stride elements apart.  use_library 0: bfloat16 products of more than 64 rows
- * never go to hipBLASLt. */
-celeg_status celeg_ops_linear(const void* x, int32_t x_dtype, int64_t x_row_stride, const void* w, int32_t w_dtype,
-                              void* out, int32_t out_dtype, int64_t out_row_stride, const float* bias, int32_t M,
-                              int32_t N, int32_t K, int32_t use_library, void* stream);
+/* ---- the kernels' dispatcher alone (tests of single kernels) ----
+ * A dispatcher of its own (workspace, library plans, tables of cosines and sines): the same class the parts
+ * of a model call, with its shape checks and its choice of kernel.  celeg_ops_call runs the method that `op`
+ * names ("linear", "rmsnorm", "short_conv", "qk_norm_rope_store", "paged_attention", "fused_linear",
+ * "tiled_linear", "sample", ...; "state" runs nothing) on `stream` (a hipStream_t) with the arguments in
+ * args_json: tensors as {"data": address, "dtype": "float32" | "bfloat16" | "int32" | "uint8", "shape": [...],
+ * "stride": [...]} (strides in elements), arrays of a step as addresses, a step and a cache view as objects of
+ * addresses and counts, and optionally "knobs": {name: value} set before the call.  It returns JSON
+ * ({"last_stat_blocks": n, ...}; "state" adds "paths", the launches counted by kernel family) that stays
+ * valid until the next call on the same handle, or NULL with the reason in celeg_last_error(): a size that a
+ * kernel does not take is refused here, before anything is launched. */
+typedef struct celeg_ops celeg_ops;
+celeg_status celeg_ops_create(celeg_ops** out);
+void celeg_ops_destroy(celeg_ops* ops);
+const char* celeg_ops_call(celeg_ops* ops, const char* op, const char* args_json, void* stream);
 
 /* ---- without a GPU: what a folder holds ---- */
 /* JSON {"config", "spec", "expected_tensors": [{"name", "shape", "kind", "init", "also"}]} of a model

@@ -157,12 +157,11 @@ class LoadedModel:
 
     def __init__(self, model: native.NativeModel):
         from ..config.spec import ModelSpec
-        from ..config.registry import Lfm2Config
+        from ..config.registry import typed_config
         self.native = model
         info = model.info
         self.spec = ModelSpec.from_json(info["spec"])
-        self.config = Lfm2Config.from_typed(info["config"]) if self.spec.architecture == "Lfm2ForCausalLM" \
-            else info["config"]
+        self.config = typed_config(self.spec.architecture, info["config"])
         self.cache = _CacheFacade(model)
         self.runner = _RunnerFacade(model)
         self.dtype = info["dtype"]

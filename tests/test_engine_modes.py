@@ -100,9 +100,17 @@ def test_gpu_engine_through_the_library_products_matches_plain(model_folders, na
 
 
 @pytest.mark.gpu
-def test_the_products_of_long_steps_follow_the_width_of_the_model(model_folders):
-    lm = run_mode(model_folders, "A", "bfloat16", "whole", "cuda:0")
-    assert lm.native.info["gemm_backend"] == "tiles"          # a width up to 1,024
+def test_the_products_of_long_steps_follow_the_sizes_of_the_products(model_folders):
+    """Steps of many rows take the tiled products where the stream is at most ``tiled_max_width`` wide
+    (1,024 as measured) and the library's above; the rule looks at the products, and the knob moves it."""
+    lm = run_mode(model_folders, "E", "bfloat16", "whole", "cuda:0")
+    assert lm.native.info["gemm_backend"] == "tiles" and lm.native.info["tiled_max_width"] == 1024
+    paths = lm.paths()
+    heads = len(LENGTHS["E"])          # the output head over all rows of a whole prompt is the library's in either case
+    assert paths["tiled"] > 0 and paths["tiled_qkv"] > 0 and paths["linear_library"] == heads, paths
+    lm = run_mode(model_folders, "E", "bfloat16", "whole", "cuda:0", knobs={"tiled_max_width": 127})
+    paths = lm.paths()
+    assert paths["tiled"] == 0 and paths["tiled_qkv"] == 0 and paths["linear_library"] > 10 * heads, paths
 
 
 @pytest.mark.gpu
@@ -173,12 +181,15 @@ def test_long_decoding(model_folders, name, dtype):
 @pytest.mark.gpu
 @pytest.mark.parametrize("whole", [-1, 1])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_long_decoding_across_the_bounds_of_recorded_steps(model_folders, dtype, whole):
-    """A recorded decode step serves contexts up to a bound (the attention over few requests
-    cuts the context into parts by it), and a longer context takes another recording.  With
-    parts of 4 rounds from 2 rounds on and of 16 from 9 on, two requests decode from 20 to 330
-    tokens; every position is compared with the plain implementation.  Once more with the
-    kernel of many requests (one workgroup a request and key/value head) forced."""
+def test_long_decoding_with_the_context_cut_into_parts_of_several_rounds(model_folders, dtype, whole):
+    """The decode attention over few requests cuts a context into parts, and a recorded decode step
+    fixes how: by the longest context the recording serves (here the model's 512 positions, 8 rounds
+    of 64 keys).  With the thresholds lowered to 1 and 8 rounds the recording takes parts of 4
+    rounds instead of one round a part, so that two requests decoding from 20 to 330 tokens run
+    through parts that are empty at first, half full later and full at the end; every position is
+    compared with the plain implementation.  Once more with the kernel of many requests (one
+    workgroup a request and key/value head) forced.  (Contexts that cross the bounds between
+    recordings, 4,096 tokens and up, are in test_gpu_long_context.py, with the thresholds as shipped.)"""
     from celeg_amd.engine import load_model
     storage = torch.float32 if dtype == "float32" else torch.bfloat16
     folder = model_folders("D", storage, WEIGHT_STD)

@@ -196,9 +196,8 @@ def test_qkv_product_with_norm_rotation_and_cache_write(ops, heads, kv_heads, K,
         batch, keep = build_batch(ops, cache, entries)
         qkv = torch.zeros(total + 1, N, dtype=BF, device=DEV)
         if fused:
-            cos_sin = ops._rope_table(inv_freq, kv.table.shape[1] * page_tokens) if rotate else None
             ops.tiled_linear(a, w, qkv[:total], stats=stats, stat_blocks=blocks, eps=eps, bias=bias,
-                             qkv=dict(heads=heads, kv_heads=kv_heads, q_weight=qw, k_weight=kw, eps=1e-6, cos_sin=cos_sin,
+                             qkv=dict(heads=heads, kv_heads=kv_heads, q_weight=qw, k_weight=kw, eps=1e-6, inv_freq=inv_freq,
                                       batch=batch, kv=kv))
         else:
             ops.tiled_linear(a, w, qkv[:total], stats=stats, stat_blocks=blocks, eps=eps, bias=bias)
