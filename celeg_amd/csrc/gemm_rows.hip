@@ -22,7 +22,14 @@
 // the next 32 values in flight while it multiplies.  The wavefronts' tiles meet in LDS;
 // every thread then finishes outputs of one row, always adding in the same order, so a
 // result does not depend on what else is in the batch.  No workgroup needs another one's
-// sums.  (Cutting K across workgroups, with a second kernel that adds the slices, was
+// sums.  The columns a workgroup owns need not fill its tiles: where whole tiles would give a
+// number of workgroups that the compute units do not share out evenly (4,608 columns are 288
+// tiles of 16 for 256 compute units: 32 of them get twice the work, and the product lasts as
+// long as they do), a workgroup owns fewer columns than its tiles hold (18 of 32) and the lanes
+// of the others repeat an address that is loaded anyway.  What these products wait for is what a
+// compute unit pulls through its vector cache, rows of A and weights alike (about 45 GB/s a compute
+// unit when the weights come from memory), so they last as long as the compute unit with the most
+// workgroups.  (Cutting K across workgroups, with a second kernel that adds the slices, was
 // measured and gained nothing: narrow tiles and many wavefronts a workgroup were as fast
 // or faster at every size tried, 1024 to 14336 columns and 1024 to 7168 values of k.)
 //
@@ -30,6 +37,8 @@
 // SwiGLU elementwise.cpp:101-119, short convolution src/backend/cpu/kernels/convolution.cpp:7-28,
 // projections y = x W^T src/model/weight_plan.cpp:82-130; the reference fuses the residual
 // addition into its products with beta = 1 (src/backend/cuda/model/prefill_batched/non_attention.cpp:175-201).
+#include <algorithm>
+
 #include "common.h"
 #include "gemv_params.h"
 
@@ -134,10 +143,10 @@ __device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n
 // wavefronts split K.  LDS: [waves][MT][streams * CT][4][64] floats, then MT*16 scales.
 template <int MT, int CT, int EPI>
 __global__ __launch_bounds__(64 * rows_max_waves(MT, Streams<EPI>::n * CT))
-void gemm_rows_kernel(const GemvParams p) {
+void gemm_rows_kernel(const GemvParams p, const int cols) {
     constexpr int NS = Streams<EPI>::n;
     constexpr int SC = NS * CT;
-    constexpr int COLS = CT * 16;
+    constexpr int COLS = CT * 16;          // columns the tiles hold; the workgroup owns the first `cols` of them
     constexpr int ROWS = MT * 16;
     extern __shared__ float smem[];
     const int n_waves = blockDim.x >> 6;
@@ -147,7 +156,7 @@ void gemm_rows_kernel(const GemvParams p) {
     // ones (the matrix instructions do not honour a lane mask)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int M = p.M, N = p.N, K = p.K;
-    const int n0 = blockIdx.x * COLS;
+    const int n0 = blockIdx.x * cols;
     const int row0 = blockIdx.y * ROWS;        // the workgroup's first row
     const int c16 = lane & 15, q = lane >> 4;
 
@@ -162,8 +171,12 @@ void gemm_rows_kernel(const GemvParams p) {
 #pragma unroll
     for (int s = 0; s < NS; ++s)
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-            wcol[s * CT + ct] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + ct * 16 + c16, N - 1)) * p.w_row_stride + q * p.w_q_stride;
+        for (int ct = 0; ct < CT; ++ct) {
+            // a lane whose column is not the workgroup's repeats the first column's address (no memory traffic of its own)
+            const int jn = ct * 16 + c16;
+            const int n = jn < cols && n0 + jn < N ? n0 + jn : n0;
+            wcol[s * CT + ct] = p.w + (static_cast<size_t>(s) * p.stream_rows + n) * p.w_row_stride + q * p.w_q_stride;
+        }
     const int nkb = K >> 5;                    // K % 32 == 0 (checked by the host)
     const int kb_begin = wave * nkb / n_waves, kb_end = (wave + 1) * nkb / n_waves;
 
@@ -244,7 +257,7 @@ void gemm_rows_kernel(const GemvParams p) {
         const int t = rl >> 4, rr = rl & 15, ct = j >> 4, jj = j & 15;
         const int src = jj + 16 * (rr >> 2), reg = rr & 3;
         const int r = row0 + rl, n = n0 + j;
-        const bool ok = r < M && n < N;
+        const bool ok = r < M && n < N && j < cols;
         const int rc = min(r, M - 1), nc = min(n, N - 1);
         float sum[NS];
 #pragma unroll
@@ -274,20 +287,28 @@ void gemm_rows_kernel(const GemvParams p) {
 
 // The shape of the work for these sizes: narrow tiles, so that there are many workgroups
 // (wide ones only where even they give thousands, as for an output head), and as many
-// wavefronts as LDS holds tiles of and as still have two blocks of 32 each.
+// wavefronts as LDS holds tiles of and as still have two blocks of 32 each.  Then the columns a
+// workgroup owns: all its tiles hold, or fewer (a) where that leaves compute units without a
+// workgroup (1,024 columns of a product of 16 rows are 64 tiles: 4 columns a workgroup give 256
+// workgroups, 6.9 against 8.4 us for K = 4,608) and (b) where the last round of workgroups would
+// be far from full (4,608 columns of two streams are 288 tiles, a round of 256 and one of 32 that
+// takes as long: tiles twice as wide of which a workgroup owns 18 columns are two full rounds,
+// 10.7 against 12.2 us at 64 rows, 9.0 against 9.4 at 32, 7.5 against 7.8 at 16).
 struct RowsShape {
-    int mt, ct, waves;
+    int mt, ct, waves, cols;
 };
 
-// For tests and tuning: a share of columns (ct: 1, 2 or 4 tiles of 16), a number of
+// For tests and tuning: a share of columns (ct: 1, 2 or 4 tiles of 16, owned whole), a number of
 // wavefronts and a share of rows (mt: 1, 2 or 4 tiles of 16) that override the choice below
-// where they fit; 0 leaves a choice alone.
-static int g_force_ct = 0, g_force_waves = 0, g_force_mt = 0;
+// where they fit; 0 leaves a choice alone.  celeg_gemm_rows_force_cols: the columns a workgroup owns.
+static int g_force_ct = 0, g_force_waves = 0, g_force_mt = 0, g_force_cols = 0;
 extern "C" void celeg_gemm_rows_force(int ct, int waves, int mt) { g_force_ct = ct; g_force_waves = waves; g_force_mt = mt; }
+extern "C" void celeg_gemm_rows_force_cols(int cols) { g_force_cols = cols; }
 
 static RowsShape rows_shape(int M, int N, int K, int streams) {
     RowsShape s;
-    s.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    const int max_mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    s.mt = max_mt;
     const int max_ct = streams == 1 ? 4 : (streams == 2 ? 2 : 1);
     s.ct = 1;
     while (s.ct < max_ct && (N + 32 * s.ct - 1) / (32 * s.ct) >= 1024) s.ct *= 2;
@@ -295,8 +316,33 @@ static RowsShape rows_shape(int M, int N, int K, int streams) {
     // few columns: the rows are shared out too, until there is a workgroup per compute unit
     while (s.mt > 1 && ((N + 16 * s.ct - 1) / (16 * s.ct)) * ((M + 16 * s.mt - 1) / (16 * s.mt)) < ROWS_COMPUTE_UNITS)
         s.mt >>= 1;
-    if ((g_force_mt == 1 || g_force_mt == 2 || g_force_mt == 4) && g_force_mt <= (M <= 16 ? 1 : (M <= 32 ? 2 : 4)))
-        s.mt = g_force_mt;
+    if ((g_force_mt == 1 || g_force_mt == 2 || g_force_mt == 4) && g_force_mt <= max_mt) s.mt = g_force_mt;
+    s.cols = 16 * s.ct;
+    const bool forced = g_force_ct > 0 || g_force_mt > 0 || g_force_cols > 0;
+    if (!forced) {
+        const auto row_groups = [&](int mt) { return (M + 16 * mt - 1) / (16 * mt); };
+        // (a) compute units without a workgroup
+        if (s.ct == 1)
+            while (s.cols > 4 && row_groups(s.mt) * ((N + s.cols - 1) / s.cols) < ROWS_COMPUTE_UNITS) s.cols >>= 1;
+        // (b) a last round of workgroups that is less than three quarters full
+        const long long groups = static_cast<long long>(row_groups(s.mt)) * ((N + s.cols - 1) / s.cols);
+        const long long rounds = (groups + ROWS_COMPUTE_UNITS - 1) / ROWS_COMPUTE_UNITS;
+        if (s.cols == 16 * s.ct && groups > ROWS_COMPUTE_UNITS && rounds * ROWS_COMPUTE_UNITS - groups > ROWS_COMPUTE_UNITS / 4 &&
+            2 * s.ct <= max_ct) {
+            const int mt = std::min(s.mt, 2), wide = 32 * s.ct;
+            for (int k = 1; k <= 8; ++k) {
+                const long long want = static_cast<long long>(ROWS_COMPUTE_UNITS) * k;      // workgroups: whole rounds
+                const int cols = static_cast<int>((static_cast<long long>(N) * row_groups(mt) + want - 1) / want);
+                if (cols > wide) continue;
+                if (cols > 16 * s.ct) s.mt = mt, s.ct *= 2, s.cols = cols;
+                break;
+            }
+        }
+    }
+    if (g_force_cols >= 1 && g_force_cols <= 16 * max_ct) {
+        s.cols = g_force_cols;
+        s.ct = s.cols <= 16 ? 1 : (s.cols <= 32 ? 2 : 4);
+    }
     const int nkb = K / 32;
     s.waves = rows_max_waves(s.mt, streams * s.ct);
     if (K <= 2048 && s.waves > 8) s.waves = 8;     // a short K: two workgroups of 8 a compute unit were the faster
@@ -309,7 +355,7 @@ static RowsShape rows_shape(int M, int N, int K, int streams) {
 }
 
 template <int MT, int CT, int EPI>
-static int launch_rows(const GemvParams& p, int waves, hipStream_t stream) {
+static int launch_rows(const GemvParams& p, int waves, int cols, hipStream_t stream) {
     constexpr int NS = Streams<EPI>::n;
     const size_t lds = static_cast<size_t>(waves) * MT * NS * CT * 1024 + MT * 16 * sizeof(float);
     static bool raised = false;              // once per instantiation: more LDS than the default limit
@@ -319,8 +365,8 @@ static int launch_rows(const GemvParams& p, int waves, hipStream_t stream) {
         if (err != hipSuccess) return static_cast<int>(err);
         raised = true;
     }
-    dim3 grid((p.N + CT * 16 - 1) / (CT * 16), (p.M + MT * 16 - 1) / (MT * 16)), block(waves * 64);
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p);
+    dim3 grid((p.N + cols - 1) / cols, (p.M + MT * 16 - 1) / (MT * 16)), block(waves * 64);
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p, cols);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -329,7 +375,7 @@ static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
     constexpr int NS = Streams<EPI>::n;
     const RowsShape s = rows_shape(p.M, p.N, p.K, NS);
 #define ROWS_CASE(MT_, CT_) \
-    if (s.mt == MT_ && s.ct == CT_) return launch_rows<MT_, CT_, EPI>(p, s.waves, stream);
+    if (s.mt == MT_ && s.ct == CT_) return launch_rows<MT_, CT_, EPI>(p, s.waves, s.cols, stream);
     ROWS_CASE(1, 1) ROWS_CASE(2, 1) ROWS_CASE(4, 1)
     if constexpr (NS <= 2) { ROWS_CASE(1, 2) ROWS_CASE(2, 2) ROWS_CASE(4, 2) }
     if constexpr (NS == 1) { ROWS_CASE(1, 4) ROWS_CASE(2, 4) ROWS_CASE(4, 4) }
@@ -343,7 +389,7 @@ static int streams_of(int epi) { return epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3
 // squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
 extern "C" int celeg_gemm_rows_blocks(int M, int N, int K, int epi) {
     const RowsShape s = rows_shape(M, N, K, streams_of(epi));
-    return (N + s.ct * 16 - 1) / (s.ct * 16);
+    return (N + s.cols - 1) / s.cols;
 }
 
 // M <= 64 (made for 17 and more; fewer rows work too), K % 32 == 0, bfloat16 a and

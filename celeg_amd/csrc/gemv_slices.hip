@@ -53,14 +53,14 @@ template <> struct Streams<E_CONV> { static constexpr int n = 3; };
 // products are under way, wait at the barrier, and finish.
 template <int G, int KW, int U, int EPI>
 __global__ __launch_bounds__((KW + (16 / G) * (16 / G) / 64 + ((16 / G) * (16 / G) % 64 ? 1 : 0)) * 64)
-void gemv_slices_kernel(const GemvParams p) {
+void gemv_slices_kernel(const GemvParams p, const int cols) {
     constexpr int MP = 16 / G;
     constexpr int NS = Streams<EPI>::n;
     constexpr int ROWS_FW = MP * MP >= 64 ? 64 / MP : MP;   // rows a finishing wavefront holds
     __shared__ floatx4_t red[NS][KW][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int M = p.M, N = p.N, K = p.K;
-    const int n0 = blockIdx.x * MP;
+    const int n0 = blockIdx.x * cols;       // the workgroup owns `cols` <= MP columns
 
     if (wave < KW) {
         // ---- the products
@@ -72,7 +72,8 @@ void gemv_slices_kernel(const GemvParams p) {
         const bf16* wrow[NS];
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(n0 + idx, N - 1)) * p.w_row_stride;
+            // (a lane whose column is not the workgroup's repeats its first column: no memory traffic of its own)
+            wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + (idx < cols && n0 + idx < N ? n0 + idx : n0)) * p.w_row_stride;
         const int k_slice = slice * Ks;
         const int chunks = (Ks + 63) >> 6;
         const int c_begin = wave * chunks / KW, c_end = (wave + 1) * chunks / KW;
@@ -115,7 +116,7 @@ void gemv_slices_kernel(const GemvParams p) {
     const int fw = wave - KW;
     const int t = fw * 64 + lane;
     const int em = (t / MP) & (MP - 1), ej = t % MP;
-    const bool e_ok = t < MP * MP && em < M && n0 + ej < N;
+    const bool e_ok = t < MP * MP && em < M && ej < cols && n0 + ej < N;
     const int en = min(n0 + ej, N - 1), emc = min(em, M - 1);
     float old = 0.f, taps[EPI == E_CONV ? SLICES_MAX_TAPS : 1], state[EPI == E_CONV ? SLICES_MAX_TAPS - 1 : 1];
     float bias[NS];
@@ -226,16 +227,16 @@ void gemv_slices_kernel(const GemvParams p) {
 }
 
 template <int G, int KW, int EPI>
-static int launch_slices(const GemvParams& p, int chunks_per_wave, hipStream_t stream) {
+static int launch_slices(const GemvParams& p, int chunks_per_wave, int cols, hipStream_t stream) {
     constexpr int MP = 16 / G;
-    dim3 grid((p.N + MP - 1) / MP), block((KW + (MP * MP + 63) / 64) * 64);
+    dim3 grid((p.N + cols - 1) / cols), block((KW + (MP * MP + 63) / 64) * 64);
     constexpr int NS = Streams<EPI>::n;
     if (chunks_per_wave <= 2)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, EPI>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, EPI>), grid, block, 0, stream, p, cols);
     else if (chunks_per_wave <= 4 || NS > 1)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, EPI>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, EPI>), grid, block, 0, stream, p, cols);
     else
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), EPI>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), EPI>), grid, block, 0, stream, p, cols);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -252,15 +253,32 @@ static int slices_for(int M, int N, int K) {
     return g;
 }
 
+// The columns a workgroup owns: all that its tile holds (16 / g), or fewer where that gives fewer
+// workgroups than the chip has compute units.  What these products wait for is what a compute unit
+// pulls through its vector cache (its share of the weights and, every workgroup anew, the rows of A),
+// so a product is the faster the more compute units share it; the lanes of the columns that a
+// workgroup does not own load nothing.
+static int g_force_cols = 0;     // a tuning aid: the columns a workgroup owns (where they fit its tile)
+extern "C" void celeg_gemv_slices_force_cols(int cols) { g_force_cols = cols; }
+
+static int cols_for(int g, int N) {
+    const int mp = 16 / g;
+    int cols = mp;
+    while (cols > 4 && (N + cols - 1) / cols < 256) cols >>= 1;
+    if (g_force_cols > 0 && g_force_cols <= mp) cols = g_force_cols;
+    return cols;
+}
+
 template <int EPI>
 static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
     const int g = slices_for(p.M, p.N, p.K);
     const int chunks = (p.K / g + 63) / 64;
     const int kw = chunks >= 24 ? 8 : 4;
     const int cpw = (chunks + kw - 1) / kw;
-    if (g == 4) return kw == 8 ? launch_slices<4, 8, EPI>(p, cpw, stream) : launch_slices<4, 4, EPI>(p, cpw, stream);
-    if (g == 2) return kw == 8 ? launch_slices<2, 8, EPI>(p, cpw, stream) : launch_slices<2, 4, EPI>(p, cpw, stream);
-    return kw == 8 ? launch_slices<1, 8, EPI>(p, cpw, stream) : launch_slices<1, 4, EPI>(p, cpw, stream);
+    const int cols = cols_for(g, p.N);
+    if (g == 4) return kw == 8 ? launch_slices<4, 8, EPI>(p, cpw, cols, stream) : launch_slices<4, 4, EPI>(p, cpw, cols, stream);
+    if (g == 2) return kw == 8 ? launch_slices<2, 8, EPI>(p, cpw, cols, stream) : launch_slices<2, 4, EPI>(p, cpw, cols, stream);
+    return kw == 8 ? launch_slices<1, 8, EPI>(p, cpw, cols, stream) : launch_slices<1, 4, EPI>(p, cpw, cols, stream);
 }
 
 extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvParams)); }
@@ -268,8 +286,8 @@ extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvPar
 // Number of workgroups for these sizes, which is also the number of partial sums of
 // squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
 extern "C" int celeg_gemv_slices_blocks(int M, int N, int K) {
-    const int mp = 16 / slices_for(M, N, K);
-    return (N + mp - 1) / mp;
+    const int cols = cols_for(slices_for(M, N, K), N);
+    return (N + cols - 1) / cols;
 }
 
 // M <= 16, K % 8 == 0, bfloat16 a and w (w in either layout that w_row_stride and

@@ -47,7 +47,7 @@ def test_plain_rows_store_and_32bit_store_with_bias(ops, M, N, K):
     # which the wavefronts' partial sums are added (their number depends on the rows)
     one = torch.empty(1, N, device=DEV)
     ops.fused_linear(a[M // 2:M // 2 + 1], w, one, epilogue="store_f32", bias=b)
-    if ops.residual_stat_blocks(M, N, K) == ops.residual_stat_blocks(1, N, K):   # the same layout
+    if M <= 4:   # up to four rows share a layout (the same cut of the matrix instruction's tile into k-slices)
         assert torch.equal(one[0], out32[M // 2])
     close(one[0], out32[M // 2], rel=1e-5)
 
