@@ -78,3 +78,34 @@ def test_phase_times_cover_the_step(model_folders):
     lm.native.time_phases(False)
     assert lm.native.phase_times() is None
     lm.close()
+
+
+def test_sync_launches_flag_checks_every_kernel_and_records_no_graph(model_folders, tmp_path):
+    """CELEG_SYNC_LAUNCHES=1 (read when the library first launches a kernel, so a process of its own):
+    every launch is waited for and checked, which names the kernel behind an asynchronous fault, and no
+    step is recorded into or replayed from a graph (the reference's CELEG_DEBUG_SYNC build,
+    include/celeg/backend/cuda/utils.cuh:109-116).  The tokens are those of an ordinary run."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from helpers import ROOT
+    folder = model_folders("D", torch.bfloat16, WEIGHT_STD)
+    script = tmp_path / "run.py"
+    script.write_text(
+        "import json, sys\n"
+        f"sys.path.insert(0, {ROOT!r})\n"
+        "from celeg_amd.engine import Engine\n"
+        "from celeg_amd.sampling import GREEDY\n"
+        f"e = Engine.from_folder({folder!r}, dtype='bfloat16', max_active_requests=2, n_pages=16, max_batched_tokens=64)\n"
+        "out = e.generate([[5, 17, 3, 200, 41], list(range(10, 27))], max_new_tokens=12, generation=GREEDY, eos_token_ids=[])\n"
+        "print(json.dumps({'tokens': out, 'replays': e.metrics['graph_replays'], 'captures': e.loaded.runner.counters()['captures']}))\n")
+    results = {}
+    for flag in ("0", "1"):
+        env = dict(os.environ, CELEG_SYNC_LAUNCHES=flag)
+        done = subprocess.run([sys.executable, str(script)], env=env, capture_output=True, text=True, timeout=300)
+        assert done.returncode == 0, done.stderr[-2000:]
+        results[flag] = json.loads(done.stdout.strip().splitlines()[-1])
+    assert results["0"]["replays"] > 0 and results["0"]["captures"] > 0
+    assert results["1"]["replays"] == 0 and results["1"]["captures"] == 0
+    assert results["1"]["tokens"] == results["0"]["tokens"]

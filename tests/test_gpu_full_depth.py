@@ -40,6 +40,33 @@ def test_logits_at_the_benchmarks_configuration(benchmark_model):
     lm.close()
 
 
+def test_logits_at_the_benchmarks_context(benchmark_model):
+    """What bench.py times, with its logits checked: prompts of 2,048 tokens fed in one step each (the
+    tiled products, the attention over 2,048 rows), then eight requests decoding together from position
+    2,048 on (the recorded step of a batch of 8, keys cut into 33 parts and joined).  Two different
+    prompts, four requests each; the last row of every prompt and every decoded token against the plain
+    implementation."""
+    from celeg_amd.engine import load_model
+    folder, cfg, W = benchmark_model
+    prompts = [random_tokens(cfg["vocab_size"], 2048 + 8, seed=21 + i) for i in range(2)]
+    reqs = {f"b{i}": prompts[i % 2] for i in range(8)}
+    steps = [{"step": i, "entries": [{"id": rid, "tokens": toks[:2048], "want": [2047]}], "end": []}
+             for i, (rid, toks) in enumerate(reqs.items())]
+    for k in range(8):
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [toks[2048 + k]], "want": [0]} for rid, toks in reqs.items()],
+                      "end": list(reqs) if k == 7 else []})
+    lm = load_model(folder, dtype="bfloat16", page_tokens=16, n_pages=8 * 129, max_requests=8, max_context=4096,
+                    max_batched_tokens=2048)
+    got = EngineDriver(lm).run(steps)
+    assert lm.runner.counters()["graph_replays"] >= 8
+    paths = lm.paths()
+    assert paths["tiled"] > 0 and paths["tiled_qkv"] > 0 and paths["attention_rows"] > 0 and paths["attention_decode_fresh"] > 0, paths
+    ref = [plain.model_logits(cfg, W, toks)[2047:].float() for toks in prompts]
+    for i, rid in enumerate(reqs):
+        assert_close_bf16(got[rid], ref[i % 2], f"benchmark context/{rid}")
+    lm.close()
+
+
 def test_32bit_logits_at_the_benchmarks_depth(benchmark_model):
     """All 16 layers in true 32-bit (the same folder, its bfloat16 weights widened exactly):
     two short requests, most in one step and the last tokens one by one, then in portions,
