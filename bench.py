@@ -115,6 +115,9 @@ def serve(shape: str, chunk: int = 0, budget: int = 0, granule: int = 1, gemm_ba
         "new_tokens": load["new_tokens"], "prefill_chunk": load["chunk"],
         "step_token_budget": load["budget"], "portion_granule": granule, "context": cfg["max_position_embeddings"],
         "engine_steps": after["steps"] - before["steps"],
+        "decode_steps": after["decode_steps"] - before["decode_steps"],
+        "portion_steps": after["portion_steps"] - before["portion_steps"],
+        "mixed_steps": after["mixed_steps"] - before["mixed_steps"],
         "steps_launched_ahead": after["steps_ahead"] - before["steps_ahead"],
         "steps_replayed_from_graphs": after["graph_replays"] - before["graph_replays"],
         "graphs_recorded": after["captures"] - before["captures"],

@@ -96,6 +96,10 @@ bool Engine::launch(const std::vector<PlannedEntry>& plan, bool device_tokens, L
         Tensor logits = loaded_->runner->step(entries);
         last_logits_ = logits;
         steps_ahead_ += device_tokens ? 1 : 0;
+        // what kind of step it was: single tokens only, portions only, or both side by side
+        bool singles = false, portions = false;
+        for (const PlannedEntry& e : plan) (e.count == 1 ? singles : portions) = true;
+        (singles && portions ? mixed_steps_ : singles ? decode_steps_ : portion_steps_) += 1;
         // tokens that count as seen by their request: the sampler's kernels mark what they choose,
         // so a step that only feeds such tokens back (every entry the one new token of a
         // decoding request) has nothing to mark; prompts, and what a request that was put back
@@ -206,6 +210,7 @@ Json Engine::metrics() const {
     const ModelRunner& r = *loaded_->runner;
     Json out = Json::object();
     out.set("steps", steps_).set("steps_ahead", steps_ahead_).set("failed_steps", failed_steps_)
+        .set("decode_steps", decode_steps_).set("portion_steps", portion_steps_).set("mixed_steps", mixed_steps_)
         .set("step_seconds", step_seconds_).set("graph_replays", r.graph_replays).set("captures", r.captures)
         .set("capture_seconds", r.capture_seconds).set("steps_run", r.steps_run)
         .set("scheduler", scheduler_->stats()).set("cache", loaded_->cache->memory_bytes())

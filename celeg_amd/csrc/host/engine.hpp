@@ -73,6 +73,7 @@ private:
     bool run_ahead_ = true;
     Tensor last_logits_;
     long long steps_ = 0, steps_ahead_ = 0, failed_steps_ = 0;
+    long long decode_steps_ = 0, portion_steps_ = 0, mixed_steps_ = 0;      // launched steps by kind
     double step_seconds_ = 0.0;
 };
 

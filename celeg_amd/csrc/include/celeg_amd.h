@@ -218,6 +218,14 @@ celeg_status celeg_ops_create(celeg_ops** out);
 void celeg_ops_destroy(celeg_ops* ops);
 const char* celeg_ops_call(celeg_ops* ops, const char* op, const char* args_json, void* stream);
 
+/* ---- plain C++ functions for what the kernels compute, on host memory (tests) ----
+ * One beside each kernel (host/reference.cpp: loops in 32-bit floats over the same layouts of the cache pages
+ * and the state slots): "embed", "rmsnorm", "linear", "swiglu", "short_conv", "qk_norm_rope", "kv_store",
+ * "paged_attention", "sample".  args_json holds host addresses (as integers) and sizes under the functions'
+ * parameter names.  Returns JSON ("sample": {"token": n}) or NULL with the reason in celeg_last_error().
+ * Needs no GPU. */
+const char* celeg_reference_call(const char* op, const char* args_json);
+
 /* ---- without a GPU: what a folder holds ---- */
 /* JSON {"config", "spec", "expected_tensors": [{"name", "shape", "kind", "init", "also"}]} of a model
  * folder (config.json, generation_config.json, and the checkpoint's tensor names for what they leave out) */
