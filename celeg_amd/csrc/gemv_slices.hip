@@ -51,16 +51,24 @@ template <> struct Streams<E_CONV> { static constexpr int n = 3; };
 // the end needs - the old value of the stream, or the convolution's state through the
 // request's slot, and the partial sums of squares for the rows' 1/rms - while the
 // products are under way, wait at the barrier, and finish.
-template <int G, int KW, int U, int EPI>
-__global__ __launch_bounds__((KW + (16 / G) * (16 / G) / 64 + ((16 / G) * (16 / G) % 64 ? 1 : 0)) * 64)
+// CT: tiles of MP columns a workgroup takes one after the other with the same rows of A in its
+// registers (wide products, where MP columns a workgroup would be thousands of workgroups that the
+// compute units cannot share out evenly: 4,608 columns of two streams at 8 rows are 576 workgroups of
+// 8 columns, 2 on some compute units and 3 on others, but 256 of 18 in three tiles).
+template <int G, int KW, int U, int CT, int EPI>
+__global__ __launch_bounds__((KW + ((16 / G) * (16 / G) * CT + 63) / 64) * 64)
 void gemv_slices_kernel(const GemvParams p, const int cols) {
     constexpr int MP = 16 / G;
     constexpr int NS = Streams<EPI>::n;
-    constexpr int ROWS_FW = MP * MP >= 64 ? 64 / MP : MP;   // rows a finishing wavefront holds
-    __shared__ floatx4_t red[NS][KW][64];
+    // rows a finishing wavefront holds the sums of squares of: its own share of the rows where one tile
+    // fills several wavefronts (MP = 16), else all MP rows
+    constexpr int ROWS_FW = MP * MP > 64 ? 64 / MP : MP;
+    constexpr bool ROWS_BY_WAVE = MP * MP > 64;
+    static_assert(CT == 1 || !ROWS_BY_WAVE, "several tiles of columns go with tiles of up to 64 outputs");
+    __shared__ floatx4_t red[NS][CT][KW][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int M = p.M, N = p.N, K = p.K;
-    const int n0 = blockIdx.x * cols;       // the workgroup owns `cols` <= MP columns
+    const int n0 = blockIdx.x * cols;       // the workgroup owns `cols` <= CT * MP columns
 
     if (wave < KW) {
         // ---- the products
@@ -69,19 +77,25 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
         const int Ks = K / G;                   // K % (8 G) == 0 (checked by the host)
         const size_t a_row = static_cast<size_t>(p.rows ? p.rows[min(idx, M - 1)] : min(idx, M - 1));
         const bf16* arow = static_cast<const bf16*>(p.a) + a_row * p.lda + slice * Ks;
-        const bf16* wrow[NS];
+        const bf16* wrow[NS][CT];
 #pragma unroll
         for (int s = 0; s < NS; ++s)
-            // (a lane whose column is not the workgroup's repeats its first column: no memory traffic of its own)
-            wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + (idx < cols && n0 + idx < N ? n0 + idx : n0)) * p.w_row_stride;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                // (a lane whose column is not the workgroup's repeats its first column: no memory traffic of its own)
+                const int j = ct * MP + idx;
+                wrow[s][ct] = p.w + (static_cast<size_t>(s) * p.stream_rows + (j < cols && n0 + j < N ? n0 + j : n0)) * p.w_row_stride;
+            }
         const int k_slice = slice * Ks;
         const int chunks = (Ks + 63) >> 6;
         const int c_begin = wave * chunks / KW, c_end = (wave + 1) * chunks / KW;
-        floatx4_t acc[NS];
+        floatx4_t acc[NS][CT];
 #pragma unroll
-        for (int s = 0; s < NS; ++s) acc[s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[s][ct] = floatx4_t{0.f, 0.f, 0.f, 0.f};
         for (int c0 = c_begin; c0 < c_end; c0 += U) {
-            Frag2 wv[U][NS][2], av[U][2];
+            Frag2 wv[U][NS][CT][2], av[U][2];
 #pragma unroll
             for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -93,30 +107,37 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
                     av[u][v] = in ? *reinterpret_cast<const Frag2*>(arow + k) : Frag2{};
 #pragma unroll
                     for (int s = 0; s < NS; ++s)
-                        wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + w_off) : Frag2{};
+#pragma unroll
+                        for (int ct = 0; ct < CT; ++ct)
+                            wv[u][s][ct][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s][ct] + w_off) : Frag2{};
                 }
 #pragma unroll
             for (int u = 0; u < U; ++u)
 #pragma unroll
                 for (int v = 0; v < 2; ++v)
 #pragma unroll
-                    for (int s = 0; s < NS; ++s) {
-                        acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].lo, wv[u][s][v].lo, acc[s], 0, 0, 0);
-                        acc[s] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].hi, wv[u][s][v].hi, acc[s], 0, 0, 0);
-                    }
+                    for (int s = 0; s < NS; ++s)
+#pragma unroll
+                        for (int ct = 0; ct < CT; ++ct) {
+                            acc[s][ct] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].lo, wv[u][s][ct][v].lo, acc[s][ct], 0, 0, 0);
+                            acc[s][ct] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[u][v].hi, wv[u][s][ct][v].hi, acc[s][ct], 0, 0, 0);
+                        }
         }
         // acc: lane l holds column l%16 of rows 4*(l/16)..+3 of the 16x16 tile
 #pragma unroll
-        for (int s = 0; s < NS; ++s) red[s][wave][lane] = acc[s];
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) red[s][ct][wave][lane] = acc[s][ct];
         __syncthreads();
         return;
     }
 
-    // ---- the finishing wavefronts: thread t finishes row em, column n0 + ej
+    // ---- the finishing wavefronts: thread t finishes row em, column n0 + ej of tile tile_ct
     const int fw = wave - KW;
     const int t = fw * 64 + lane;
-    const int em = (t / MP) & (MP - 1), ej = t % MP;
-    const bool e_ok = t < MP * MP && em < M && ej < cols && n0 + ej < N;
+    const int tile_ct = CT == 1 ? 0 : min(t / (MP * MP), CT - 1);
+    const int em = (t / MP) & (MP - 1), ej = (CT == 1 ? 0 : tile_ct * MP) + t % MP;
+    const bool e_ok = t < MP * MP * CT && em < M && ej < cols && n0 + ej < N;
     const int en = min(n0 + ej, N - 1), emc = min(em, M - 1);
     float old = 0.f, taps[EPI == E_CONV ? SLICES_MAX_TAPS : 1], state[EPI == E_CONV ? SLICES_MAX_TAPS - 1 : 1];
     float bias[NS];
@@ -132,7 +153,7 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
     float ssq = 0.f;
     if (p.stats) {
         const int nb = p.n_stat_blocks;
-        const int sm = min(fw * ROWS_FW + lane / LPR, M - 1), sj = lane % LPR;
+        const int sm = min((ROWS_BY_WAVE ? fw * ROWS_FW : 0) + lane / LPR, M - 1), sj = lane % LPR;
         const float* srow = p.stats + static_cast<size_t>(p.rows ? p.rows[sm] : sm) * p.stats_ld;
         float part[NFIRST];
 #pragma unroll
@@ -163,7 +184,7 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
 #pragma unroll
         for (int off = LPR / 2; off > 0; off >>= 1) ssq += __shfl_xor(ssq, off, 64);
         // the lanes of row em - fw * ROWS_FW hold its sum
-        const float total = __shfl(ssq, ((em - fw * ROWS_FW) & (ROWS_FW - 1)) * LPR, 64);
+        const float total = __shfl(ssq, ((em - (ROWS_BY_WAVE ? fw * ROWS_FW : 0)) & (ROWS_FW - 1)) * LPR, 64);
         scale = 1.0f / sqrtf(total / static_cast<float>(K) + p.eps);
     }
     __syncthreads();
@@ -173,10 +194,10 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
         sum[s] = 0.f;
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            const int r = g * MP + em, c = g * MP + ej;
+            const int r = g * MP + em, c = g * MP + t % MP;
             const int src = c + 16 * (r >> 2), reg = r & 3;
 #pragma unroll
-            for (int w = 0; w < KW; ++w) sum[s] += red[s][w][src][reg];
+            for (int w = 0; w < KW; ++w) sum[s] += red[s][tile_ct][w][src][reg];
         }
         sum[s] = sum[s] * scale + bias[s];
     }
@@ -193,11 +214,12 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
             if (p.out_bf16) static_cast<bf16*>(p.out_bf16)[static_cast<size_t>(em) * p.ld_bf16 + en] = from_float<bf16>(v);
         }
         if (p.stats_out) {
-            float sq = v * v;                   // the MP columns of a row sit in MP neighbouring lanes
+            float sq = v * v;                   // the MP columns of a row and tile sit in MP neighbouring lanes
 #pragma unroll
             for (int off = MP / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
-            if (ej == 0 && em < M && t < MP * MP)
-                p.stats_out[static_cast<size_t>(em) * p.stats_ld_out + blockIdx.x] = sq;
+            // (one partial sum a tile: CT of them a workgroup)
+            if (t % MP == 0 && em < M && t < MP * MP * CT)
+                p.stats_out[static_cast<size_t>(em) * p.stats_ld_out + blockIdx.x * CT + tile_ct] = sq;
         }
     } else if (EPI == E_SWIGLU) {
         if (e_ok) {
@@ -226,59 +248,84 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
     }
 }
 
-template <int G, int KW, int EPI>
+template <int G, int KW, int CT, int EPI>
 static int launch_slices(const GemvParams& p, int chunks_per_wave, int cols, hipStream_t stream) {
     constexpr int MP = 16 / G;
-    dim3 grid((p.N + cols - 1) / cols), block((KW + (MP * MP + 63) / 64) * 64);
+    dim3 grid((p.N + cols - 1) / cols), block((KW + (MP * MP * CT + 63) / 64) * 64);
     constexpr int NS = Streams<EPI>::n;
-    if (chunks_per_wave <= 2)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, EPI>), grid, block, 0, stream, p, cols);
+    if (CT > 1 || chunks_per_wave <= 2 || (NS == 3 && KW == 8 && G == 1))   // (or the weights in flight fill the registers)
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, CT, EPI>), grid, block, 0, stream, p, cols);
     else if (chunks_per_wave <= 4 || NS > 1)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, EPI>), grid, block, 0, stream, p, cols);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, 1, EPI>), grid, block, 0, stream, p, cols);
     else
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), EPI>), grid, block, 0, stream, p, cols);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), 1, EPI>), grid, block, 0, stream, p, cols);
     return CELEG_LAUNCH_RESULT();
 }
 
-// How many k-slices share the matrix instruction's tile for this many rows and this K.
-static int g_force_slices = 0;     // a tuning aid: 1, 2 or 4 overrides the choice below where it fits
+// The shape of the work: how many k-slices share the matrix instruction's tile (g: 4 for up to 4
+// rows, 2 for up to 8, else 1; a tile then holds 16 / g columns), how many columns a workgroup owns and
+// in how many tiles.  What these products wait for is what a compute unit pulls through its vector
+// cache (its share of the weights and, every workgroup anew, the rows of A), so a product lasts as long
+// as the compute unit with the most workgroups.  Few columns: a workgroup owns fewer than its tile holds
+// (the lanes of the others load nothing), so that every compute unit has one.  The widest product (w1
+// with w3) at 5 to 8 rows: the columns are shared out so that the workgroups are as many as the compute
+// units, each with up to three tiles that share the rows of A in its registers (4,608 columns: 6.5 us
+// instead of 6.9).  Measured and left: several tiles for the other epilogues and for 4 k-slices (the
+// same or slower).
+struct SlicesShape {
+    int g, cols, ct;
+};
+static int g_force_slices = 0;     // tuning aids: 1, 2 or 4 k-slices; the columns a workgroup owns (where they fit)
+static int g_force_cols = 0;
 extern "C" void celeg_gemv_slices_force(int g) { g_force_slices = g; }
+extern "C" void celeg_gemv_slices_force_cols(int cols) { g_force_cols = cols; }
+#define SLICES_COMPUTE_UNITS 256
+#define SLICES_MAX_TILES 3
 
-static int slices_for(int M, int N, int K) {
-    int g = M <= 4 ? 4 : (M <= 8 ? 2 : 1);
-    if (g_force_slices > 0 && g_force_slices <= g) g = g_force_slices;
-    while (g > 1 && K % (8 * g)) g >>= 1;
+static SlicesShape slices_shape(int M, int N, int K, int epi) {
+    SlicesShape s;
+    s.g = M <= 4 ? 4 : (M <= 8 ? 2 : 1);
+    if (g_force_slices > 0 && g_force_slices <= s.g) s.g = g_force_slices;
+    while (s.g > 1 && K % (8 * s.g)) s.g >>= 1;
     // more than about a thousand workgroups gain nothing (measured on 4,608 columns)
-    while (g > 1 && g_force_slices == 0 && (N + 16 / g - 1) / (16 / g) > 1024) g >>= 1;
-    return g;
+    while (s.g > 1 && g_force_slices == 0 && N / (16 / s.g) > 1024) s.g >>= 1;
+    const int mp = 16 / s.g;
+    const int max_tiles = s.g == 2 && epi == E_SWIGLU ? SLICES_MAX_TILES : 1;
+    s.cols = mp, s.ct = 1;
+    if ((N + mp - 1) / mp < SLICES_COMPUTE_UNITS) {
+        while (s.cols > 4 && (N + s.cols - 1) / s.cols < SLICES_COMPUTE_UNITS) s.cols >>= 1;
+    } else if (max_tiles > 1 && M > 4) {
+        for (int k = 1; k <= 16; ++k) {
+            const int cols = (N + SLICES_COMPUTE_UNITS * k - 1) / (SLICES_COMPUTE_UNITS * k);
+            if (cols > mp * max_tiles) continue;
+            if (cols > mp) s.cols = cols;
+            break;
+        }
+    }
+    if (g_force_cols > 0 && g_force_cols <= mp * max_tiles) s.cols = g_force_cols;
+    s.ct = (s.cols + mp - 1) / mp;
+    return s;
 }
 
-// The columns a workgroup owns: all that its tile holds (16 / g), or fewer where that gives fewer
-// workgroups than the chip has compute units.  What these products wait for is what a compute unit
-// pulls through its vector cache (its share of the weights and, every workgroup anew, the rows of A),
-// so a product is the faster the more compute units share it; the lanes of the columns that a
-// workgroup does not own load nothing.
-static int g_force_cols = 0;     // a tuning aid: the columns a workgroup owns (where they fit its tile)
-extern "C" void celeg_gemv_slices_force_cols(int cols) { g_force_cols = cols; }
-
-static int cols_for(int g, int N) {
-    const int mp = 16 / g;
-    int cols = mp;
-    while (cols > 4 && (N + cols - 1) / cols < 256) cols >>= 1;
-    if (g_force_cols > 0 && g_force_cols <= mp) cols = g_force_cols;
-    return cols;
+template <int G, int KW, int EPI>
+static int launch_tiles(const GemvParams& p, int cpw, const SlicesShape& s, hipStream_t stream) {
+    if constexpr (G == 2 && EPI == E_SWIGLU) {
+        if (s.ct == 2) return launch_slices<G, KW, 2, EPI>(p, cpw, s.cols, stream);
+        if (s.ct == 3) return launch_slices<G, KW, 3, EPI>(p, cpw, s.cols, stream);
+    }
+    if (s.ct != 1) return static_cast<int>(hipErrorInvalidValue);
+    return launch_slices<G, KW, 1, EPI>(p, cpw, s.cols, stream);
 }
 
 template <int EPI>
 static int launch_epilogue(const GemvParams& p, hipStream_t stream) {
-    const int g = slices_for(p.M, p.N, p.K);
-    const int chunks = (p.K / g + 63) / 64;
+    const SlicesShape s = slices_shape(p.M, p.N, p.K, EPI);
+    const int chunks = (p.K / s.g + 63) / 64;
     const int kw = chunks >= 24 ? 8 : 4;
     const int cpw = (chunks + kw - 1) / kw;
-    const int cols = cols_for(g, p.N);
-    if (g == 4) return kw == 8 ? launch_slices<4, 8, EPI>(p, cpw, cols, stream) : launch_slices<4, 4, EPI>(p, cpw, cols, stream);
-    if (g == 2) return kw == 8 ? launch_slices<2, 8, EPI>(p, cpw, cols, stream) : launch_slices<2, 4, EPI>(p, cpw, cols, stream);
-    return kw == 8 ? launch_slices<1, 8, EPI>(p, cpw, cols, stream) : launch_slices<1, 4, EPI>(p, cpw, cols, stream);
+    if (s.g == 4) return kw == 8 ? launch_tiles<4, 8, EPI>(p, cpw, s, stream) : launch_tiles<4, 4, EPI>(p, cpw, s, stream);
+    if (s.g == 2) return kw == 8 ? launch_tiles<2, 8, EPI>(p, cpw, s, stream) : launch_tiles<2, 4, EPI>(p, cpw, s, stream);
+    return kw == 8 ? launch_tiles<1, 8, EPI>(p, cpw, s, stream) : launch_tiles<1, 4, EPI>(p, cpw, s, stream);
 }
 
 extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvParams)); }
@@ -286,8 +333,8 @@ extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvPar
 // Number of workgroups for these sizes, which is also the number of partial sums of
 // squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
 extern "C" int celeg_gemv_slices_blocks(int M, int N, int K) {
-    const int cols = cols_for(slices_for(M, N, K), N);
-    return (N + cols - 1) / cols;
+    const SlicesShape s = slices_shape(M, N, K, E_RESIDUAL);
+    return (N + s.cols - 1) / s.cols * s.ct;
 }
 
 // M <= 16, K % 8 == 0, bfloat16 a and w (w in either layout that w_row_stride and

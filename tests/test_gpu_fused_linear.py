@@ -192,7 +192,8 @@ def test_sliced_products_behind_a_norm(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M,ff,K", [(1, 192, 64), (8, 4608, 1024), (7, 352, 128), (16, 200, 96), (4, 100, 1160),
-                                    (19, 352, 128), (40, 4608, 1024), (64, 200, 96), (33, 7200, 64)])
+                                    (19, 352, 128), (40, 4608, 1024), (64, 200, 96), (33, 7200, 64),
+                                    (5, 2300, 352), (6, 5000, 96), (8, 7000, 64)])
 def test_sliced_swiglu(ops, M, ff, K):
     h, xb, stats, nw, w, folded, rows, x = scaled_case(M, ff, K, 2, 50)
     g = (x @ w[:ff].double().cpu().T).to(BF).double()
@@ -237,6 +238,21 @@ def test_sliced_conv_token_by_token_equals_the_whole_convolution(ops, M, H, taps
         ref = plain.short_conv(bcx.to(BF), cw.cpu(), cb.cpu() if bias else None)
         close(got[:, m], ref, rel=2.5e-2)
     assert float(state[0].abs().max()) == 0.0          # a slot nobody uses stays zero
+
+
+@pytest.mark.parametrize("cols", [4, 7, 8, 9, 13, 16, 17, 24])
+def test_sliced_swiglu_with_every_share_of_columns(ops, cols):
+    """At 5 to 8 rows a workgroup of the SwiGLU product owns up to three tiles of 8 columns of each
+    weight stream, as many as make the workgroups a whole number of rounds of the compute units; here
+    the number of columns is forced, at widths that leave the last workgroup and its last tile partly
+    empty."""
+    lib = ops._lib("gemv_slices")
+    lib.celeg_gemv_slices_force_cols(cols)
+    try:
+        test_sliced_swiglu(ops, 8, 1000, 128)
+        test_sliced_swiglu(ops, 5, 333, 352)
+    finally:
+        lib.celeg_gemv_slices_force_cols(0)
 
 
 @pytest.mark.parametrize("mt", [1, 2, 4])
