@@ -96,7 +96,7 @@ __device__ __forceinline__ Early<EPI> early_fetch(const GemvParams& p, int r, in
 }
 
 // Finishes one output from the scaled sums of its weight streams.  Returns the new value of
-// the residual stream (E_RESIDUAL).
+// the residual stream (E_RESIDUAL) or the value stored (E_STORE_F32).
 template <int EPI>
 __device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n, const float* scaled,
                                                const Early<EPI>& early) {
@@ -109,6 +109,7 @@ __device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n
         static_cast<bf16*>(p.out)[ob] = from_float<bf16>(sum[0]);
     } else if (EPI == E_STORE_F32) {
         static_cast<float*>(p.out)[o] = sum[0];
+        return sum[0];
     } else if (EPI == E_RESIDUAL) {
         // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
         const float v = early.old + round_bf16(sum[0]);
@@ -152,6 +153,8 @@ void gemm_rows_kernel(const GemvParams p, const int cols) {
     const int n_waves = blockDim.x >> 6;
     float* const red = smem;
     float* const s_scale = smem + static_cast<size_t>(n_waves) * MT * SC * 256;
+    // (E_STORE_F32 with row_best: the best logit of every 16 columns of a row, [ROWS][CT])
+    unsigned long long* const s_best = reinterpret_cast<unsigned long long*>(s_scale + ROWS);
     // the wavefront's number as a scalar: the branches on its range of k are then uniform
     // ones (the matrix instructions do not honour a lane mask)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -282,6 +285,23 @@ void gemm_rows_kernel(const GemvParams p, const int cols) {
             for (int off = COLS / 2; off > 0; off >>= 1) sq += __shfl_xor(sq, off, 64);
             if (j == 0 && r < M) p.stats_out[static_cast<size_t>(r) * p.stats_ld_out + blockIdx.x] = sq;
         }
+        if (EPI == E_STORE_F32 && p.row_best) {
+            // the best (logit, index) of the tile's 16 columns of this row (no trip through LDS, which
+            // this loop's reads of the partial sums would wait behind); the tiles meet below
+            const unsigned long long b = group_best_logit<16>(v, ok, n0 + (j & ~15));
+            if (jj == 0) s_best[rl * CT + ct] = b;
+        }
+    }
+    if (EPI == E_STORE_F32 && p.row_best) {
+        // one part a row and workgroup: the best of its tiles
+        __syncthreads();
+        const int rl = threadIdx.x;
+        if (rl < ROWS && row0 + rl < M) {
+            unsigned long long b = 0ull;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) b = max(b, s_best[rl * CT + ct]);
+            p.row_best[static_cast<size_t>(blockIdx.x) * p.row_best_ld + row0 + rl] = b;
+        }
     }
 }
 
@@ -357,7 +377,8 @@ static RowsShape rows_shape(int M, int N, int K, int streams) {
 template <int MT, int CT, int EPI>
 static int launch_rows(const GemvParams& p, int waves, int cols, hipStream_t stream) {
     constexpr int NS = Streams<EPI>::n;
-    const size_t lds = static_cast<size_t>(waves) * MT * NS * CT * 1024 + MT * 16 * sizeof(float);
+    const size_t lds = static_cast<size_t>(waves) * MT * NS * CT * 1024 + MT * 16 * sizeof(float) +
+                       (p.row_best ? static_cast<size_t>(MT) * 16 * CT * sizeof(unsigned long long) : 0);
     static bool raised = false;              // once per instantiation: more LDS than the default limit
     if (lds > 48 * 1024 && !raised) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_kernel<MT, CT, EPI>),
@@ -408,6 +429,8 @@ extern "C" int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t st
     if (p.stats && (p.n_stat_blocks < 1 || p.n_stat_blocks > ROWS_MAX_STAT_BLOCKS))
         return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.taps > ROWS_MAX_TAPS || p.stream_rows != p.N))
+        return static_cast<int>(hipErrorInvalidValue);
+    if (p.row_best && (epi != E_STORE_F32 || p.row_best_ld < p.M || p.row_best_parts < celeg_gemm_rows_blocks(p.M, p.N, p.K, epi)))
         return static_cast<int>(hipErrorInvalidValue);
     switch (epi) {
         case E_STORE: return launch_epilogue<E_STORE>(p, stream);

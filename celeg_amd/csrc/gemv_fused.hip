@@ -99,12 +99,14 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&a
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         float sq[4] = {0.f, 0.f, 0.f, 0.f};
+        unsigned long long best[4] = {0ull, 0ull, 0ull, 0ull};
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int m = mt * 16 + 4 * q + r;
             const bool ok = col_ok && m < M;
             if (EPI == E_STORE || EPI == E_STORE_F32) {
                 const float v = acc[mt][0][r] + (p.bias && ok ? p.bias[n] : 0.f);
+                if (EPI == E_STORE_F32 && p.row_best) best[r] = group_best_logit<16>(v, ok, tile * 16);
                 if (ok) {
                     if (EPI == E_STORE) static_cast<bf16*>(p.out)[static_cast<size_t>(m) * p.ldo + n] = from_float<bf16>(v);
                     else static_cast<float*>(p.out)[static_cast<size_t>(m) * p.ldo + n] = v;
@@ -148,6 +150,14 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&a
                     if (p.conv_b) conv += p.conv_b[n];
                     static_cast<bf16*>(p.out)[static_cast<size_t>(m) * p.ldo + n] = from_float<bf16>(cc * conv);
                 }
+            }
+        }
+        if (EPI == E_STORE_F32 && p.row_best) {
+            // the best of the tile's 16 columns, row by row: one part of the row
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = mt * 16 + 4 * q + r;
+                if (c16 == 0 && m < M) p.row_best[static_cast<size_t>(tile) * p.row_best_ld + m] = best[r];
             }
         }
         if (EPI == E_RESIDUAL && p.stats_out) {
@@ -460,6 +470,7 @@ extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, in
     if (epi == E_CONV && (p.taps < 1 || p.taps > CONV_PREFETCH_TAPS || p.stream_rows != p.N))
         return static_cast<int>(hipErrorInvalidValue);
     const int tiles = (p.N + 15) / 16, chunks = (p.K + 63) / 64;
+    if (p.row_best && (epi != E_STORE_F32 || p.row_best_ld < p.M || p.row_best_parts < tiles)) return static_cast<int>(hipErrorInvalidValue);
     const int streams = epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3 : 1);
     const int mt = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
     const size_t limit = 144 * 1024;

@@ -44,4 +44,10 @@ struct GemvParams {
     // bf16_k8_stride, and element (n, k) of w at
     //   n * w_row_stride + (k / 32) * w_kb_stride + (k % 32 / 8) * w_q_stride + k % 8
     long long a_k8_stride, out_k8_stride, bf16_k8_stride, w_q_stride;
+    // 32-bit store of an output head (the kernels for staged rows and for 9 to 64 rows): beside the
+    // logits, the best (logit, index) of every workgroup's (or wavefront's) columns, packed as
+    // packed_logit packs them: [parts, row_best_ld >= rows], part j from the j-th share of columns
+    // (the rows of a part side by side: a workgroup's values are one run of memory); or null
+    unsigned long long* row_best;
+    int row_best_ld, row_best_parts;     // (room for row_best_parts parts: a launch that would leave more is refused)
 };

@@ -206,6 +206,13 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
         if (e_ok) static_cast<bf16*>(p.out)[o] = from_float<bf16>(sum[0]);
     } else if (EPI == E_STORE_F32) {
         if (e_ok) static_cast<float*>(p.out)[o] = sum[0];
+        if (p.row_best) {
+            // an output head: the best (logit, index) of the tile's columns, row by row (they sit in MP
+            // neighbouring lanes): one part of the row
+            const unsigned long long b = group_best_logit<MP>(sum[0], e_ok, n0 + tile_ct * MP);
+            if (t % MP == 0 && em < M && t < MP * MP * CT)
+                p.row_best[static_cast<size_t>(blockIdx.x * CT + tile_ct) * p.row_best_ld + em] = b;
+        }
     } else if (EPI == E_RESIDUAL) {
         // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
         const float v = e_ok ? old + round_bf16(sum[0]) : 0.f;
@@ -351,6 +358,8 @@ extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t 
     if (p.stats && (p.n_stat_blocks < 1 || p.n_stat_blocks > SLICES_MAX_STAT_BLOCKS))
         return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.taps > SLICES_MAX_TAPS || p.stream_rows != p.N))
+        return static_cast<int>(hipErrorInvalidValue);
+    if (p.row_best && (epi != E_STORE_F32 || p.row_best_ld < p.M || p.row_best_parts < celeg_gemv_slices_blocks(p.M, p.N, p.K)))
         return static_cast<int>(hipErrorInvalidValue);
     switch (epi) {
         case E_STORE: return launch_epilogue<E_STORE>(p, stream);

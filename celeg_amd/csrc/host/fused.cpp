@@ -130,6 +130,10 @@ void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const
     args.n_rows = extras.n_rows;
     args.bias = extras.bias;
     args.conv = extras.conv;
+    args.row_best = extras.row_best;
+    args.row_best_ld = extras.row_best_ld;
+    args.row_best_parts = extras.row_best_parts;
+    rt.ops.last_best_parts = 0;
     if (sliced(rt, M, width) && w.dtype == DType::BF16 && (streamed || w.shape[0] / streams <= SLICED_MAX_COLUMNS)) {
         // the stream's bfloat16 copy times the weight with the norm's weight folded in, scaled
         // by the rows' 1/rms at the end

@@ -68,6 +68,8 @@ int celeg_attention_decode_fresh_bf16(const void* q, int ldq, const void* k, int
 int celeg_argmax_rows(const float* logits, int ld, int rows, int vocab, const float* fparams, const int* iparams,
                       uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens,
                       unsigned long long* best, unsigned int* arrived, hipStream_t stream);
+int celeg_argmax_merge(const unsigned long long* best, int ld, int parts, int rows, const int* iparams, int* out_tokens,
+                       int* last_tokens, hipStream_t stream);
 int celeg_sample(const float* logits, int ld, int rows, int vocab, const float* fparams, const int* iparams,
                  uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens, hipStream_t stream);
 int celeg_mark_seen(uint8_t* seen, size_t stride, int n_slots, int vocab, const int* tokens, const int* slots, int n,

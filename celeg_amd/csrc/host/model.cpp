@@ -148,6 +148,7 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
     Tensor h = rt.ws.buf("hidden", DType::F32, {T, width});
     rt.stream_stat_blocks = 0;
     rt.stream_has_bf16 = false;
+    rt.head_best = HeadBest{};
     if (!embedding_->takes_step_prologue()) rt.flush_prologue();
     embedding_->forward(batch.token_ids, h, rt, &batch);
     rt.flush_prologue();      // (an embedding that said it would and did not)
@@ -362,6 +363,7 @@ Tensor ModelRunner::step_from_graph(const std::vector<StepEntry>& entries) {
     options.update_caps = &caps;
     last_batch_ = build(entries, updates, options);
     CELEG_HIP(hipGraphLaunch(captured.exec, rt.stream));
+    rt.head_best = captured.head_best;
     ++steps_run;
     ++graph_replays;
     return captured.logits.rows(0, S);
@@ -402,6 +404,7 @@ ModelRunner::Captured& ModelRunner::record(std::pair<int, int> key, const StepBa
     try {
         begin_step(batch);
         captured.logits = model.forward(batch, rt);
+        captured.head_best = rt.head_best;
     } catch (...) {
         hipGraph_t broken = nullptr;
         (void)hipStreamEndCapture(rt.stream, &broken);
@@ -459,6 +462,7 @@ Tensor ModelRunner::step_from_portion_graph(const std::vector<StepEntry>& entrie
     auto updates = drain_updates(caps);
     last_batch_ = build(entries, updates, options);
     CELEG_HIP(hipGraphLaunch(captured.exec, rt.stream));
+    rt.head_best = captured.head_best;
     ++steps_run;
     ++graph_replays;
     return captured.logits.rows(0, 1);

@@ -90,6 +90,7 @@ private:
         hipGraph_t graph = nullptr;
         hipGraphExec_t exec = nullptr;
         Tensor logits;
+        HeadBest head_best;           // what the recorded head leaves beside the logits
         unsigned long long generation = 0;
     };
     void validate(const std::vector<StepEntry>& entries) const;

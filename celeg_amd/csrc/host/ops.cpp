@@ -57,6 +57,7 @@ const char* path_name(Path p) {
         case Path::FusedSliced: return "fused_sliced";
         case Path::FusedRows: return "fused_rows";
         case Path::FusedStaged: return "fused_staged";
+        case Path::ArgmaxMerged: return "argmax_merged";
         case Path::Tiled: return "tiled";
         case Path::TiledQkv: return "tiled_qkv";
         default: return "?";
@@ -457,10 +458,19 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
 
 // ---------------------------------------------------------------------------- sampling
 void Ops::sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen, size_t seen_stride,
-                 int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws) {
+                 int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws, const HeadBest* head_best) {
     dev(logits, "logits", DType::F32, false);
     const int R = static_cast<int>(logits.shape[0]), V = static_cast<int>(logits.shape[1]);
     if (R == 0) return;
+    if (all_greedy && use_head_argmax && head_best && head_best->logits == logits.data && head_best->rows >= R &&
+        head_best->parts > 0) {
+        // greedy rows without a penalty (the caller's word): the head's kernel left the best of every
+        // share of a row's columns, so the logits need not be read again
+        took(Path::ArgmaxMerged);
+        kernel_check(celeg_argmax_merge(head_best->best, head_best->ld, head_best->parts, R, iparams, out_tokens, last_tokens,
+                                        stream), "argmax from the head's parts");
+        return;
+    }
     if (all_greedy && use_argmax_parts && R <= 16) {     // (64 rows: 23 us against 12 us, one workgroup a row)
         // per row: the best (value, index) so far and a count of the parts that have arrived;
         // zero at first, and the kernel leaves both at zero for its next launch
@@ -674,6 +684,19 @@ void Ops::fused_linear(const Tensor& a, const Tensor& w, const Tensor& out, cons
         prm.state_slot_stride = static_cast<size_t>(c.state.stride[0]);
         prm.seq_slot = c.seq_slot;
         prm.taps = static_cast<int>(L);
+    }
+    last_best_parts = 0;
+    if (args.row_best) {
+        need(epi == Epilogue::StoreF32, "fused_linear: row_best goes with the 32-bit store");
+        last_best_parts = streamed ? celeg_gemm_rows_blocks(M, static_cast<int>(N), static_cast<int>(K), static_cast<int>(epi))
+                          : sliced ? celeg_gemv_slices_blocks(M, static_cast<int>(N), static_cast<int>(K))
+                                   : static_cast<int>((N + 15) / 16);
+        need(args.row_best_parts >= last_best_parts && args.row_best_ld >= M,
+             "fused_linear: row_best has room for " + std::to_string(args.row_best_parts) + " parts of " +
+                 std::to_string(args.row_best_ld) + " rows, the kernel leaves " + std::to_string(last_best_parts) + " of " + std::to_string(M));
+        prm.row_best = args.row_best;
+        prm.row_best_ld = args.row_best_ld;
+        prm.row_best_parts = args.row_best_parts;
     }
     took(sliced ? Path::FusedSliced : streamed ? Path::FusedRows : Path::FusedStaged);
     if (sliced) {

@@ -68,6 +68,19 @@ struct FusedArgs {
     const ConvOperands* conv = nullptr;
     Tensor out_bf16;              // residual: the bfloat16 copy of the stream
     bool packed = false;          // w is [K/32, rows, 32] (pack_weight)
+    // 32-bit store of an output head: beside the logits, the best (logit, index) of every share of
+    // columns [row_best_parts, row_best_ld >= rows]; Ops::last_best_parts then says how many parts
+    // were written
+    unsigned long long* row_best = nullptr;
+    int row_best_ld = 0, row_best_parts = 0;
+};
+
+// What an output head left beside its logits for greedy rows: the best (logit, index) of every
+// share of a row's columns [parts, ld >= rows], for the first `rows` rows of `logits`.
+struct HeadBest {
+    const void* logits = nullptr;
+    const unsigned long long* best = nullptr;
+    int ld = 0, parts = 0, rows = 0;
 };
 
 // What a step begins with, when the runner leaves it to the step's first kernel: the block-table
@@ -89,7 +102,7 @@ struct StepPrologue {
 // path it was meant to take.
 enum class Path : int {
     AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, LinearF32, LinearLibrary, LinearStandIn,
-    FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, Count
+    FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, ArgmaxMerged, Count
 };
 const char* path_name(Path p);
 
@@ -109,8 +122,9 @@ public:
     bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
     bool use_qkv_tail = true;          // q/k/v products of many rows take norm, rotation and cache write along
     bool use_fresh_decode = true;      // decode-only steps: the attention prepares and writes the new keys and values
+    bool use_head_argmax = true;       // greedy rows without a penalty: the token from what the head left beside the logits
     int rows_kernel_min_rows = 9, tiles_min_rows = 65, fused_linear_shape = 0;
-    int last_stat_blocks = 0;
+    int last_stat_blocks = 0, last_best_parts = 0;
 
     // row-wise
     void embed(const Tensor& table, const int* token_ids, const Tensor& out);
@@ -138,7 +152,11 @@ public:
                             const KVView& kv, DType dtype) const;
     // sampling
     void sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen,
-                size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws);
+                size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws,
+                const HeadBest* head_best = nullptr);
+    // the most parts a row of an output head of n columns can have (for the caller's buffer): one
+    // per 16 columns, or per 4 where the columns are few (narrow tiles, or less than a tile a workgroup)
+    static int head_best_parts(long long n) { return static_cast<int>(std::max((n + 15) / 16, std::min<long long>((n + 3) / 4, 4096))); }
     void mark_seen(uint8_t* seen, size_t stride, int n_slots, int vocab, const int* token_ids, const int* token_slot, int n);
     // fused skinny products
     bool fused_linear_ok(int rows, std::initializer_list<long long> inner) const;
@@ -204,6 +222,9 @@ struct Runtime {
     // the step's prologue, left by the runner for the embedding's kernel to take along
     // (defer_prologue); whoever cannot take it along calls flush_prologue() before its own work
     bool defer_prologue = true;
+    // what the step's output head left for greedy rows (none: logits == nullptr); every forward
+    // pass and every replay of a recorded one sets it anew
+    HeadBest head_best;
     StepPrologue prologue;
     void flush_prologue() {
         if (!prologue.pending) return;

@@ -159,6 +159,7 @@ void set_knobs(Ops& ops, const Json& knobs) {
         else if (name == "attention_general") ops.attention_general = v != 0;
         else if (name == "use_rope_table") ops.use_rope_table = v != 0;
         else if (name == "use_argmax_parts") ops.use_argmax_parts = v != 0;
+        else if (name == "use_head_argmax") ops.use_head_argmax = v != 0;
         else if (name == "use_sliced") ops.use_sliced = v != 0;
         else if (name == "use_rows_kernel") ops.use_rows_kernel = v != 0;
         else if (name == "use_tiles") ops.use_tiles = v != 0;
@@ -240,9 +241,18 @@ Json call(celeg_ops& h, const std::string& op, const Json& a) {
                                 h.ws, has_fresh ? &fresh : nullptr);
         }
     } else if (op == "sample") {
-        ops.sample(must(a, "logits"), address<float>(a, "fparams"), address<int>(a, "iparams"), address<uint8_t>(a, "seen"),
+        const Tensor logits = must(a, "logits");
+        HeadBest best;
+        best.best = address<unsigned long long>(a, "row_best");
+        if (best.best) {
+            best.logits = logits.data;
+            best.ld = static_cast<int>(a.get_int("row_best_ld", 0));
+            best.parts = static_cast<int>(a.get_int("row_best_parts", 0));
+            best.rows = static_cast<int>(logits.shape[0]);
+        }
+        ops.sample(logits, address<float>(a, "fparams"), address<int>(a, "iparams"), address<uint8_t>(a, "seen"),
                    static_cast<size_t>(a.get_int("seen_stride", 0)), address<int>(a, "out_tokens"), address<int>(a, "last_tokens"),
-                   a.get_bool("all_greedy", false), h.ws);
+                   a.get_bool("all_greedy", false), h.ws, best.best ? &best : nullptr);
     } else if (op == "mark_seen") {
         const Tensor seen = must(a, "seen");
         ops.mark_seen(seen.as<uint8_t>(), static_cast<size_t>(seen.stride[0]), static_cast<int>(seen.shape[0]),
@@ -291,6 +301,9 @@ Json call(celeg_ops& h, const std::string& op, const Json& a) {
             conv.seq_slot = address<int>(c, "seq_slot");
             args.conv = &conv;
         }
+        args.row_best = address<unsigned long long>(a, "row_best");
+        args.row_best_ld = static_cast<int>(a.get_int("row_best_ld", 0));
+        args.row_best_parts = static_cast<int>(a.get_int("row_best_parts", 0));
         ops.fused_linear(must(a, "a"), must(a, "w"), must(a, "out"), args);
     } else if (op == "tiled_linear") {
         const Maybe stats = maybe(a, "stats"), bias = maybe(a, "bias"), stats_out = maybe(a, "stats_out"), out_bf16 = maybe(a, "out_bf16");
@@ -338,6 +351,7 @@ Json call(celeg_ops& h, const std::string& op, const Json& a) {
         throw KernelError("unknown operation '" + op + "'");
     }
     out.set("last_stat_blocks", ops.last_stat_blocks);
+    out.set("last_best_parts", ops.last_best_parts);
     if (op == "state") out.set("paths", ops.paths_json());
     return out;
 }

@@ -93,7 +93,7 @@ void Sampler::launch(const Tensor& logits, const std::vector<int>& slots) {
     const size_t cap = static_cast<size_t>(cap_);
     float* f = params_[turn].as<float>();
     int* iv = reinterpret_cast<int*>(f + cap * 4);
-    bool all_greedy = true;
+    bool all_greedy = true, penalised = false;
     for (int r = 0; r < R; ++r) {
         auto cit = configs_.find(slots[static_cast<size_t>(r)]);
         if (cit == configs_.end()) throw StepError("sample: slot " + std::to_string(slots[static_cast<size_t>(r)]) + " has no request");
@@ -110,6 +110,7 @@ void Sampler::launch(const Tensor& logits, const std::vector<int>& slots) {
         iv[3 * r + 1] = (c.repetition_penalty > 1.0f && seen_.ptr()) ? slots[static_cast<size_t>(r)] : -1;
         iv[3 * r + 2] = slots[static_cast<size_t>(r)];
         all_greedy = all_greedy && c.greedy() && !forced;
+        penalised = penalised || iv[3 * r + 1] >= 0;
     }
     // greedy rows have nothing that changes from step to step: ship only what differs from what
     // the device holds
@@ -125,7 +126,7 @@ void Sampler::launch(const Tensor& logits, const std::vector<int>& slots) {
     // the kernels write the tokens straight into the turn's pinned buffer (memory of the host that
     // the device can address): no copy behind them, the event tells when they are there
     rt_.ops.sample(logits, fdev, idev, seen_.as<uint8_t>(), static_cast<size_t>(vocab_), tokens_host_[turn].as<int>(),
-                   last_tokens_.as<int>(), all_greedy, rt_.ws);
+                   last_tokens_.as<int>(), all_greedy, rt_.ws, penalised ? nullptr : &rt_.head_best);
     CELEG_HIP(hipEventRecord(events_[turn], rt_.stream));
     pending_.emplace_back(turn, R);
 }

@@ -14,12 +14,6 @@
 #define SAMPLE_HIST_COPIES 16
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
-// larger float <-> larger key
-__device__ __forceinline__ uint32_t order_key(float f) {
-    const uint32_t u = __float_as_uint(f);
-    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
 __device__ __forceinline__ bool better(float sa, int ia, float sb, int ib) {
     return sa == sb ? ia < ib : sa > sb;
 }
@@ -550,10 +544,7 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(
         const int i = lo + tid + ARGMAX_THREADS * j;
         float x = v[j];
         if (sn[j]) x = x >= 0.0f ? x / penalty : x * penalty;
-        x += 0.0f;                                                       // -0 and +0 are one value
-        const unsigned long long packed = (static_cast<unsigned long long>(order_key(x)) << 32) |
-                                          (0xffffffffu - static_cast<unsigned>(i));
-        if (i < vocab) mine = max(mine, packed);
+        if (i < vocab) mine = max(mine, packed_logit(x, i));
     }
 #pragma unroll
     for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) {
@@ -571,7 +562,7 @@ __global__ __launch_bounds__(ARGMAX_THREADS) void argmax_parts_kernel(
     __threadfence();
     const unsigned long long winner = atomicExch(&best[r], 0ull);
     atomicExch(&arrived[r], 0u);
-    const int token = static_cast<int>(0xffffffffu - static_cast<unsigned>(winner & 0xffffffffull));
+    const int token = packed_logit_index(winner);
     out_tokens[r] = token;
     if (last_tokens && slot >= 0) last_tokens[slot] = token;
     if (seen_all && seen_row >= 0) seen_all[static_cast<size_t>(seen_row) * seen_stride + token] = 1;
@@ -589,6 +580,50 @@ extern "C" int celeg_argmax_rows(const float* logits, int ld, int rows, int voca
     hipLaunchKernelGGL(argmax_parts_kernel, dim3((vocab + ARGMAX_PART - 1) / ARGMAX_PART, rows),
                        dim3(ARGMAX_THREADS), 0, stream, logits, ld, vocab, fparams, iparams, seen,
                        seen_stride, out_tokens, last_tokens, best, arrived);
+    return CELEG_LAUNCH_RESULT();
+}
+
+// The greedy tokens of rows whose output head left the best (logit, index) of every workgroup's
+// columns beside the logits (best [parts, ld >= rows], packed as packed_logit packs them): the
+// largest of a row's parts is its token.  No repetition penalty: the head
+// knows nothing of what a request has seen.  One workgroup a row; the token also goes to
+// last_tokens[slot] as with the other kernels.
+#define MERGE_THREADS 256
+__global__ __launch_bounds__(MERGE_THREADS) void argmax_merge_kernel(
+    const unsigned long long* __restrict__ best, int ld, int parts, const int* __restrict__ iparams,
+    int* __restrict__ out_tokens, int* __restrict__ last_tokens) {
+    __shared__ unsigned long long s_best[MERGE_THREADS / CELEG_WAVE];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int lane = tid & (CELEG_WAVE - 1), wave = tid / CELEG_WAVE;
+    const unsigned long long* row = best + r;
+    unsigned long long mine = 0ull;
+    for (int j0 = 0; j0 < parts; j0 += 8 * MERGE_THREADS) {         // eight loads of a thread under way at a time
+        unsigned long long v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)      // (a part twice changes nothing)
+            v[j] = row[static_cast<size_t>(min(j0 + tid + MERGE_THREADS * j, parts - 1)) * ld];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mine = max(mine, v[j]);
+    }
+#pragma unroll
+    for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) mine = max(mine, __shfl_xor(mine, off, CELEG_WAVE));
+    if (lane == 0) s_best[wave] = mine;
+    __syncthreads();
+    if (tid != 0) return;
+#pragma unroll
+    for (int w = 1; w < MERGE_THREADS / CELEG_WAVE; ++w) mine = max(mine, s_best[w]);
+    const int token = packed_logit_index(mine);
+    const int slot = iparams[3 * r + 2];
+    out_tokens[r] = token;
+    if (last_tokens && slot >= 0) last_tokens[slot] = token;
+}
+
+extern "C" int celeg_argmax_merge(const unsigned long long* best, int ld, int parts, int rows, const int* iparams,
+                                  int* out_tokens, int* last_tokens, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (parts <= 0 || ld < rows) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(MERGE_THREADS), 0, stream, best, ld, parts, iparams,
+                       out_tokens, last_tokens);
     return CELEG_LAUNCH_RESULT();
 }
 

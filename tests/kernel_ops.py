@@ -112,6 +112,7 @@ class HipOps:
         self.use_fresh_decode = True
         self.fused_linear_shape = 0
         self.last_stat_blocks = 0
+        self.last_best_parts = 0
         handle = ctypes.c_void_p()
         lib = self._lib("host")
         if lib.celeg_ops_create(ctypes.byref(handle)) != 0:
@@ -161,6 +162,7 @@ class HipOps:
             raise KernelError(self._library.celeg_last_error().decode())
         out = json.loads(answer.decode())
         self.last_stat_blocks = out.get("last_stat_blocks", self.last_stat_blocks)
+        self.last_best_parts = out.get("last_best_parts", 0)
         return out
 
     def paths(self) -> Dict[str, int]:
@@ -259,9 +261,13 @@ class HipOps:
                                fresh={"inv_freq": _tensor(inv_freq, "inv_freq")}, dtype=_NAMES[dtype])["ok"])
 
     # ------------------------------------------------------------------ sampling
-    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None, all_greedy=False):
+    def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None, all_greedy=False, row_best=None,
+               row_best_parts=0):
         """One token per row.  ``all_greedy``: the caller knows that every row takes its
-        (penalised) largest logit; the rows are then cut into parts over many workgroups."""
+        (penalised) largest logit; the rows are then cut into parts over many workgroups.
+        ``row_best`` [>= row_best_parts, >= rows] (int64): what the head's product left beside these
+        logits (``fused_linear(..., row_best=...)``); greedy rows without a penalty then take their
+        token from it."""
         R, V = logits.shape
         if out_tokens.numel() != R or fparams.numel() < 4 * R or iparams.numel() < 3 * R:
             raise KernelError("sample: parameter arrays do not fit the rows")
@@ -270,7 +276,9 @@ class HipOps:
         self._call("sample", logits=_tensor(logits, "logits"), fparams=_address(fparams, "fparams", torch.float32),
                    iparams=_address(iparams, "iparams"), seen=_address(seen, "seen", torch.uint8),
                    seen_stride=int(seen.stride(0)) if seen is not None else 0, out_tokens=_address(out_tokens, "out_tokens"),
-                   last_tokens=_address(last_tokens, "last_tokens"), all_greedy=bool(all_greedy))
+                   last_tokens=_address(last_tokens, "last_tokens"), all_greedy=bool(all_greedy),
+                   row_best=_address(row_best, "row_best", torch.int64),
+                   row_best_ld=int(row_best.stride(0)) if row_best is not None else 0, row_best_parts=int(row_best_parts))
 
     def mark_seen(self, seen, token_ids, token_slot, n):
         if token_ids.numel() < n or token_slot.numel() < n:
@@ -333,8 +341,10 @@ class HipOps:
 
     def fused_linear(self, a, w, out, *, epilogue="store", norm_weight=None, eps=0.0, stats=None,
                      stat_blocks=0, rows=None, bias=None, stats_out=None, conv=None, n_rows=None,
-                     out_bf16=None):
+                     out_bf16=None, row_best=None):
         """out = epilogue(prologue(a) w^T) for up to 64 rows, bfloat16 weights (``Ops::fused_linear``).
+        ``row_best`` (int64 [parts, >= rows], with "store_f32"): receives the best (logit, index) of every
+        share of a row's columns; ``last_best_parts`` says how many parts were written.
 
         ``a``: bfloat16 rows [M, K], or, with ``norm_weight``, the 32-bit residual stream,
         normalised on the fly (``stats[row, :stat_blocks]`` holding partial sums of squares
@@ -356,7 +366,10 @@ class HipOps:
                    norm_weight=_tensor(norm_weight, "norm_weight"), eps=float(eps), stats=_tensor(stats, "stats"),
                    stat_blocks=int(stat_blocks), rows=_address(rows, "rows"), n_rows=-1 if n_rows is None else int(n_rows),
                    bias=_tensor(bias, "bias"), stats_out=_tensor(stats_out, "stats_out"), conv=conv_json,
-                   out_bf16=_tensor(out_bf16, "out_bf16"), packed=w.dim() == 3)
+                   out_bf16=_tensor(out_bf16, "out_bf16"), packed=w.dim() == 3,
+                   row_best=_address(row_best, "row_best", torch.int64),
+                   row_best_ld=int(row_best.stride(0)) if row_best is not None else 0,
+                   row_best_parts=int(row_best.shape[0]) if row_best is not None else 0)
         return out
 
     # ------------------------------------------------------------------ fused products of many rows

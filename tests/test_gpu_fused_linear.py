@@ -103,6 +103,55 @@ def test_residual_epilogue_adds_in_place_and_leaves_partial_sums(ops, M, N, K):
     assert float(stats[M:].max()) == -1.0 if M < 64 else True
 
 
+@pytest.mark.parametrize("M,N,K,form", [(1, 4100, 64, "norm"), (8, 65536, 256, "norm"), (16, 333, 96, "norm"), (5, 24, 40, "norm"),
+                                        (9, 4100, 64, "rows"), (64, 65536, 64, "rows"), (33, 1000, 96, "rows"),
+                                        (17, 20, 32, "rows"), (64, 4608, 1024, "rows"),
+                                        (1, 4100, 64, "rows"), (4, 333, 96, "rows"), (8, 16384, 32, "rows"), (16, 1000, 40, "rows")])
+def test_the_32bit_store_leaves_the_best_of_every_share_of_a_row(ops, M, N, K, form):
+    """An output head's product writes, beside the logits, the best (logit, index) of the columns of
+    every workgroup (or wavefront): their maximum over a row is the row's largest logit at its
+    lowest index, and the merging kernel gives that token.  Two equal weight rows make equal logits:
+    the lower index wins, wherever the two lie."""
+    h = randn(M, K, seed=21)
+    nw = 1 + randn(K, seed=22, scale=0.1)
+    w = randn(N, K, seed=23, scale=0.1, dtype=BF)
+    for r, (lo, hi) in enumerate([(N // 3, N - 1), (0, N // 2), (N - 2, N - 1), (1, 17 % N)]):
+        boost = randn(K, seed=30 + r, scale=0.5, dtype=BF)      # a direction that some row likes most, twice
+        w[lo] = boost
+        w[hi] = boost
+    room = max((N + 15) // 16, min((N + 3) // 4, 4096))
+    best = torch.full((room, M + 3), -1, dtype=torch.int64, device=DEV)
+    out = torch.empty(M, N, device=DEV)
+    if form == "norm":
+        ops.fused_linear(h, w, out, epilogue="store_f32", norm_weight=nw, eps=1e-5, row_best=best)
+    else:
+        xb = torch.empty(M, K, dtype=BF, device=DEV)
+        stats = torch.zeros(64, 1, device=DEV)
+        ops.stream_prepare(h, xb, stats)
+        ops.fused_linear(xb, ops.fold_weight(w, nw), out, epilogue="store_f32", eps=1e-5, stats=stats, stat_blocks=1,
+                         row_best=best)
+    parts = ops.last_best_parts
+    assert 0 < parts <= room
+    assert bool((best[parts:] == -1).all()) and bool((best[:, M:] == -1).all())
+    top = best[:parts, :M].cpu().numpy().view("uint64").max(axis=0)
+    index = (0xffffffff - (top & 0xffffffff)).astype("int64")
+    logits = out.cpu()
+    want = [int((logits[m] == logits[m].max()).nonzero()[0]) for m in range(M)]
+    assert index.tolist() == want
+    tokens = torch.full((M,), -1, dtype=torch.int32, device=DEV)
+    last = torch.full((M + 1,), -1, dtype=torch.int32, device=DEV)
+    f = torch.tensor([[0.0, 1.0, 1.0, 0.0]] * M, dtype=torch.float32, device=DEV).reshape(-1)
+    i = torch.tensor([[1, -1, m + 1 if m % 2 else -1] for m in range(M)], dtype=torch.int32, device=DEV).reshape(-1)
+    before = ops.paths().get("argmax_merged", 0)
+    ops.sample(out, f, i, None, tokens, last_tokens=last, all_greedy=True, row_best=best, row_best_parts=parts)
+    assert ops.paths()["argmax_merged"] == before + 1
+    assert tokens.tolist() == want
+    assert last.tolist() == [-1] + [want[m] if m % 2 else -1 for m in range(M)]
+    # the other greedy kernels give the same tokens from the logits
+    ops.sample(out, f, i, None, tokens, all_greedy=True)
+    assert tokens.tolist() == want
+
+
 @pytest.mark.parametrize("M,ff,K", [(1, 192, 64), (8, 4608, 1024), (19, 352, 128), (64, 200, 96)])
 def test_swiglu_epilogue(ops, M, ff, K):
     h = randn(M, K, seed=11)

@@ -320,6 +320,37 @@ def test_steps_launched_ahead_of_their_tokens_give_the_same_tokens(model_folders
     assert [t[:47] for t in runs[True]] == [t[:47] for t in runs[False]]
 
 
+@pytest.mark.parametrize("name,dtype", [("B", "bfloat16"), ("A", "bfloat16"), ("B", "float32")])
+def test_greedy_tokens_from_what_the_head_leaves_beside_the_logits(model_folders, name, dtype):
+    """In bfloat16 the head's product of up to 64 rows leaves the best logit of every share of a row's
+    columns, and greedy rows without a penalty take their token from that instead of reading the
+    logits again: the same tokens as with that switched off, in recorded and in eager steps; a request
+    with a repetition penalty in the batch sends the whole batch to the kernels that read the logits."""
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GREEDY, GenerationConfig
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = model_folders(name, storage, 0.05)
+    vocab = plain.load_model_folder(folder)[0]["vocab_size"]
+    prompts = [random_tokens(vocab, n, seed=70 + n) for n in (9, 20, 3)]
+    outs, merged = {}, {}
+    for head_argmax in (1, 0):
+        engine = Engine.from_folder(folder, dtype=dtype, max_active_requests=4, n_pages=32, page_tokens=16,
+                                    max_batched_tokens=64, prefill_chunk_tokens=16)
+        engine.loaded.set_knob("use_head_argmax", head_argmax)
+        outs[head_argmax] = engine.generate(prompts, max_new_tokens=24, generation=GREEDY, eos_token_ids=[])
+        merged[head_argmax] = engine.loaded.paths()["argmax_merged"]
+        if head_argmax:
+            penalised = GenerationConfig(temperature=0.0, top_k=1, top_p=1.0, repetition_penalty=1.3)
+            before = engine.loaded.paths()["argmax_merged"]
+            both = engine.generate(prompts[:2], max_new_tokens=8, generations=[GREEDY, penalised], eos_token_ids=[])
+            assert both[0] == outs[1][0][:8]
+            # (the first request decodes alone while the other's prompt is still fed: those steps may merge)
+            assert engine.loaded.paths()["argmax_merged"] - before <= 4
+    assert outs[1] == outs[0]
+    assert merged[0] == 0
+    assert (merged[1] >= 20) == (dtype == "bfloat16")
+
+
 def test_generation_ahead_of_the_tokens_with_requests_that_end_early(model_folders):
     """``generate`` launches decode steps before it has read the previous step's tokens.
     With end tokens chosen so that requests end at different steps (a request that ends
