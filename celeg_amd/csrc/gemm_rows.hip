@@ -144,7 +144,8 @@ __device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n
 // wavefronts split K.  LDS: [waves][MT][streams * CT][4][64] floats, then MT*16 scales.
 template <int MT, int CT, int EPI>
 __global__ __launch_bounds__(64 * rows_max_waves(MT, Streams<EPI>::n * CT))
-void gemm_rows_kernel(const GemvParams p, const int cols) {
+void gemm_rows_kernel(const GemvParams p) {
+    const int cols = p.cols;
     constexpr int NS = Streams<EPI>::n;
     constexpr int SC = NS * CT;
     constexpr int COLS = CT * 16;          // columns the tiles hold; the workgroup owns the first `cols` of them
@@ -375,8 +376,10 @@ static RowsShape rows_shape(int M, int N, int K, int streams) {
 }
 
 template <int MT, int CT, int EPI>
-static int launch_rows(const GemvParams& p, int waves, int cols, hipStream_t stream) {
+static int launch_rows(const GemvParams& params, int waves, int cols, hipStream_t stream) {
     constexpr int NS = Streams<EPI>::n;
+    GemvParams p = params;
+    p.cols = cols;
     const size_t lds = static_cast<size_t>(waves) * MT * NS * CT * 1024 + MT * 16 * sizeof(float) +
                        (p.row_best ? static_cast<size_t>(MT) * 16 * CT * sizeof(unsigned long long) : 0);
     static bool raised = false;              // once per instantiation: more LDS than the default limit
@@ -387,7 +390,7 @@ static int launch_rows(const GemvParams& p, int waves, int cols, hipStream_t str
         raised = true;
     }
     dim3 grid((p.N + cols - 1) / cols, (p.M + MT * 16 - 1) / (MT * 16)), block(waves * 64);
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p, cols);
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p);
     return CELEG_LAUNCH_RESULT();
 }
 

@@ -57,7 +57,8 @@ template <> struct Streams<E_CONV> { static constexpr int n = 3; };
 // 8 columns, 2 on some compute units and 3 on others, but 256 of 18 in three tiles).
 template <int G, int KW, int U, int CT, int EPI>
 __global__ __launch_bounds__((KW + ((16 / G) * (16 / G) * CT + 63) / 64) * 64)
-void gemv_slices_kernel(const GemvParams p, const int cols) {
+void gemv_slices_kernel(const GemvParams p) {
+    const int cols = p.cols;
     constexpr int MP = 16 / G;
     constexpr int NS = Streams<EPI>::n;
     // rows a finishing wavefront holds the sums of squares of: its own share of the rows where one tile
@@ -256,16 +257,18 @@ void gemv_slices_kernel(const GemvParams p, const int cols) {
 }
 
 template <int G, int KW, int CT, int EPI>
-static int launch_slices(const GemvParams& p, int chunks_per_wave, int cols, hipStream_t stream) {
+static int launch_slices(const GemvParams& params, int chunks_per_wave, int cols, hipStream_t stream) {
     constexpr int MP = 16 / G;
+    GemvParams p = params;
+    p.cols = cols;
     dim3 grid((p.N + cols - 1) / cols), block((KW + (MP * MP * CT + 63) / 64) * 64);
     constexpr int NS = Streams<EPI>::n;
     if (CT > 1 || chunks_per_wave <= 2 || (NS == 3 && KW == 8 && G == 1))   // (or the weights in flight fill the registers)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, CT, EPI>), grid, block, 0, stream, p, cols);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, CT, EPI>), grid, block, 0, stream, p);
     else if (chunks_per_wave <= 4 || NS > 1)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, 1, EPI>), grid, block, 0, stream, p, cols);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, 1, EPI>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), 1, EPI>), grid, block, 0, stream, p, cols);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), 1, EPI>), grid, block, 0, stream, p);
     return CELEG_LAUNCH_RESULT();
 }
 
