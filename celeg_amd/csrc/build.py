@@ -28,7 +28,9 @@ ARCH = "gfx950"
 COMMON_FLAGS = ["-O3", "-fPIC", f"--offload-arch={ARCH}",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                 "-Wno-unused-command-line-argument"]
-KERNEL_FLAGS = ["-std=c++17"] + COMMON_FLAGS
+# the first 14 words of a kernel's arguments (what fits the registers a launch can fill) arrive with
+# the launch instead of being fetched by every wavefront
+KERNEL_FLAGS = ["-std=c++17", "-mllvm", "-amdgpu-kernarg-preload-count=14"] + COMMON_FLAGS
 HOST_FLAGS = ["-std=c++20", "-x", "hip", "-Wno-unused-result"] + COMMON_FLAGS
 LINK_FLAGS = ["-shared", "-fPIC", f"--offload-arch={ARCH}", "-ldl", "-lpthread"]
 # the kernel files, by the name tests and tools know them under

@@ -57,8 +57,12 @@ template <> struct Streams<E_CONV> { static constexpr int n = 3; };
 // 8 columns, 2 on some compute units and 3 on others, but 256 of 18 in three tiles).
 template <int G, int KW, int U, int CT, int EPI>
 __global__ __launch_bounds__((KW + ((16 / G) * (16 / G) * CT + 63) / 64) * 64)
-void gemv_slices_kernel(const GemvParams p) {
-    const int cols = p.cols;
+void gemv_slices_kernel(const void* const a_, const bf16* const w_, const int* const rows_, const int M, const int N, const int K,
+                        const int cols, const int lda_, const int stream_rows_, const int w_row_stride_, const int w_kb_stride_,
+                        const GemvParams p) {
+    // (What the first loads need comes as arguments of its own, ahead of the struct that holds it too:
+    // the first 14 words of a kernel's arguments arrive in registers with the launch, the rest is
+    // fetched by the wavefronts.)
     constexpr int MP = 16 / G;
     constexpr int NS = Streams<EPI>::n;
     // rows a finishing wavefront holds the sums of squares of: its own share of the rows where one tile
@@ -68,7 +72,6 @@ void gemv_slices_kernel(const GemvParams p) {
     static_assert(CT == 1 || !ROWS_BY_WAVE, "several tiles of columns go with tiles of up to 64 outputs");
     __shared__ floatx4_t red[NS][CT][KW][64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int M = p.M, N = p.N, K = p.K;
     const int n0 = blockIdx.x * cols;       // the workgroup owns `cols` <= CT * MP columns
 
     if (wave < KW) {
@@ -76,8 +79,8 @@ void gemv_slices_kernel(const GemvParams p) {
         const int c16 = lane & 15, q = lane >> 4;
         const int idx = c16 & (MP - 1), slice = c16 / MP;
         const int Ks = K / G;                   // K % (8 G) == 0 (checked by the host)
-        const size_t a_row = static_cast<size_t>(p.rows ? p.rows[min(idx, M - 1)] : min(idx, M - 1));
-        const bf16* arow = static_cast<const bf16*>(p.a) + a_row * p.lda + slice * Ks;
+        const size_t a_row = static_cast<size_t>(rows_ ? rows_[min(idx, M - 1)] : min(idx, M - 1));
+        const bf16* arow = static_cast<const bf16*>(a_) + a_row * lda_ + slice * Ks;
         const bf16* wrow[NS][CT];
 #pragma unroll
         for (int s = 0; s < NS; ++s)
@@ -85,7 +88,7 @@ void gemv_slices_kernel(const GemvParams p) {
             for (int ct = 0; ct < CT; ++ct) {
                 // (a lane whose column is not the workgroup's repeats its first column: no memory traffic of its own)
                 const int j = ct * MP + idx;
-                wrow[s][ct] = p.w + (static_cast<size_t>(s) * p.stream_rows + (j < cols && n0 + j < N ? n0 + j : n0)) * p.w_row_stride;
+                wrow[s][ct] = w_ + (static_cast<size_t>(s) * stream_rows_ + (j < cols && n0 + j < N ? n0 + j : n0)) * w_row_stride_;
             }
         const int k_slice = slice * Ks;
         const int chunks = (Ks + 63) >> 6;
@@ -104,7 +107,7 @@ void gemv_slices_kernel(const GemvParams p) {
                     const int k = (c0 + u) * 64 + v * 32 + q * 8;
                     const bool in = c0 + u < c_end && k + 8 <= Ks;
                     const int kw_ = k_slice + k;      // 8 values from here never leave a block of 32
-                    const size_t w_off = static_cast<size_t>(kw_ >> 5) * p.w_kb_stride + (kw_ & 31);
+                    const size_t w_off = static_cast<size_t>(kw_ >> 5) * w_kb_stride_ + (kw_ & 31);
                     av[u][v] = in ? *reinterpret_cast<const Frag2*>(arow + k) : Frag2{};
 #pragma unroll
                     for (int s = 0; s < NS; ++s)
@@ -155,7 +158,7 @@ void gemv_slices_kernel(const GemvParams p) {
     if (p.stats) {
         const int nb = p.n_stat_blocks;
         const int sm = min((ROWS_BY_WAVE ? fw * ROWS_FW : 0) + lane / LPR, M - 1), sj = lane % LPR;
-        const float* srow = p.stats + static_cast<size_t>(p.rows ? p.rows[sm] : sm) * p.stats_ld;
+        const float* srow = p.stats + static_cast<size_t>(rows_ ? rows_[sm] : sm) * p.stats_ld;
         float part[NFIRST];
 #pragma unroll
         for (int i = 0; i < NFIRST; ++i) part[i] = srow[min(sj + LPR * i, nb - 1)];
@@ -172,7 +175,7 @@ void gemv_slices_kernel(const GemvParams p) {
     if (EPI == E_RESIDUAL)
         old = static_cast<const float*>(p.out)[static_cast<size_t>(emc) * p.ldo + en];
 #pragma unroll
-    for (int s = 0; s < NS; ++s) bias[s] = p.bias ? p.bias[static_cast<size_t>(s) * p.stream_rows + en] : 0.f;
+    for (int s = 0; s < NS; ++s) bias[s] = p.bias ? p.bias[static_cast<size_t>(s) * stream_rows_ + en] : 0.f;
     if (EPI == E_CONV) {
 #pragma unroll
         for (int i = 0; i < SLICES_MAX_TAPS; ++i) taps[i] = p.conv_w[static_cast<size_t>(en) * p.taps + min(i, p.taps - 1)];
@@ -264,11 +267,14 @@ static int launch_slices(const GemvParams& params, int chunks_per_wave, int cols
     dim3 grid((p.N + cols - 1) / cols), block((KW + (MP * MP * CT + 63) / 64) * 64);
     constexpr int NS = Streams<EPI>::n;
     if (CT > 1 || chunks_per_wave <= 2 || (NS == 3 && KW == 8 && G == 1))   // (or the weights in flight fill the registers)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, CT, EPI>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 2, CT, EPI>), grid, block, 0, stream, p.a, p.w, p.rows, p.M, p.N, p.K, cols, p.lda, p.stream_rows,
+                           static_cast<int>(p.w_row_stride), static_cast<int>(p.w_kb_stride), p);
     else if (chunks_per_wave <= 4 || NS > 1)
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, 1, EPI>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, 1, EPI>), grid, block, 0, stream, p.a, p.w, p.rows, p.M, p.N, p.K, cols, p.lda, p.stream_rows,
+                           static_cast<int>(p.w_row_stride), static_cast<int>(p.w_kb_stride), p);
     else
-        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), 1, EPI>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), 1, EPI>), grid, block, 0, stream, p.a, p.w, p.rows, p.M, p.N, p.K, cols, p.lda, p.stream_rows,
+                           static_cast<int>(p.w_row_stride), static_cast<int>(p.w_kb_stride), p);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -356,7 +362,8 @@ extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t 
     const GemvParams& p = *params;
     if (p.M <= 0 || p.N <= 0) return 0;
     if (p.M > 16 || p.K <= 0 || (p.K % 8) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
-    if ((p.w_row_stride % 8) || (p.w_kb_stride % 8) || p.w_row_stride <= 0 || p.w_kb_stride <= 0)
+    if ((p.w_row_stride % 8) || (p.w_kb_stride % 8) || p.w_row_stride <= 0 || p.w_kb_stride <= 0 ||
+        p.w_row_stride > 0x7fffffffLL || p.w_kb_stride > 0x7fffffffLL)
         return static_cast<int>(hipErrorInvalidValue);
     if (p.stats && (p.n_stat_blocks < 1 || p.n_stat_blocks > SLICES_MAX_STAT_BLOCKS))
         return static_cast<int>(hipErrorInvalidValue);
