@@ -670,10 +670,11 @@ __device__ __forceinline__ void decode_prepare_head(float (&x)[KS][8], const boo
 
 template <int HD, int WAVES, bool SPLIT, bool FRESH>
 __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
-    const bf16* __restrict__ q, int ldq, const bf16* __restrict__ k_pool,
-    const bf16* __restrict__ v_pool, const int* __restrict__ table, int table_stride,
-    const int* __restrict__ token_slot, const int* __restrict__ positions, bf16* __restrict__ out,
-    int ldo, int kv_heads, int group, int page_tokens, int page_shift, int n_layers, int layer,
+    // (the pointers that the first loads go through first: the leading 14 words of the arguments
+    // arrive in registers with the launch)
+    const bf16* __restrict__ q, const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
+    const int* __restrict__ table, const int* __restrict__ token_slot, const int* __restrict__ positions,
+    int ldq, int table_stride, bf16* __restrict__ out, int ldo, int kv_heads, int group, int page_tokens, int page_shift, int n_layers, int layer,
     float scale, int window, float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
     int split_rounds, const DecodeFresh fresh) {
     constexpr int KS = HD / 32;   // steps of 32 dims in q.k
@@ -955,9 +956,9 @@ static int launch_decode_heads(const void* q, int ldq, const void* k_pool, const
     }
     auto kernel = fresh.k ? &attention_decode_heads_kernel<HD, WAVES, false, true> : &attention_decode_heads_kernel<HD, WAVES, false, false>;
     hipLaunchKernelGGL(kernel, dim3(kv_heads * chunks, n_rows),
-                       dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
+                       dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q),
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
-                       table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
+                       token_slot, positions, ldq, table_stride, static_cast<bf16*>(out), ldo, kv_heads,
                        group, page_tokens, page_shift, n_layers, layer, scale, window, nullptr, nullptr, 0, 1, fresh);
     return CELEG_LAUNCH_RESULT();
 }
@@ -983,9 +984,9 @@ static int launch_decode_parts(const void* q, int ldq, const void* k_pool, const
     }
     auto kernel = fresh.k ? &attention_decode_heads_kernel<HD, WAVES, true, true> : &attention_decode_heads_kernel<HD, WAVES, true, false>;
     hipLaunchKernelGGL(kernel, dim3(kv_heads * chunks, n_rows, n_parts),
-                       dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q), ldq,
+                       dim3(WAVES * 64), lds, stream, static_cast<const bf16*>(q),
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
-                       table_stride, token_slot, positions, static_cast<bf16*>(out), ldo, kv_heads,
+                       token_slot, positions, ldq, table_stride, static_cast<bf16*>(out), ldo, kv_heads,
                        group, page_tokens, page_shift, n_layers, layer, scale, window, ws_o, ws_ml,
                        n_splits, split_rounds, fresh);
     return 0;

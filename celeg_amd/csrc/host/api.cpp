@@ -605,7 +605,7 @@ const std::vector<Knob>& knobs() {
          [](LoadedModel& m, int v) { m.rt->tiled_max_width = v; }},
         {"fused_max_rows", [](LoadedModel& m) { return m.rt->fused_max_rows; }, [](LoadedModel& m, int v) { m.rt->fused_max_rows = v; }},
         OPS_INT(attention_decode_whole), OPS_BOOL(use_blaslt), OPS_INT(attention_rows_per_tile), OPS_INT(attention_rows_form),
-        OPS_BOOL(attention_general), OPS_BOOL(use_rope_table), OPS_BOOL(use_argmax_parts), OPS_BOOL(use_head_argmax), OPS_BOOL(use_sliced),
+        OPS_BOOL(attention_general), OPS_BOOL(use_rope_table), OPS_BOOL(use_argmax_parts), OPS_BOOL(use_head_argmax), OPS_BOOL(decode_parts_fill), OPS_BOOL(use_sliced),
         OPS_BOOL(use_rows_kernel), OPS_BOOL(use_tiles), OPS_BOOL(use_qkv_tail), OPS_BOOL(use_fresh_decode), OPS_INT(rows_kernel_min_rows), OPS_INT(tiles_min_rows),
         OPS_INT(fused_linear_shape),
         {"decode_parts_few", [](LoadedModel& m) { return m.rt->ops.decode_part_thresholds[0]; }, [](LoadedModel& m, int v) { m.rt->ops.decode_part_thresholds[0] = v; }},

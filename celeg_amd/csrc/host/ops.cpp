@@ -356,9 +356,9 @@ bool Ops::attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, in
         // kernel saved from about 8,192 tokens for each of 64 requests on (at 32,768: 4.94 against
         // 4.86 ms a step; at 2,048: 0.906 against 0.916)
         if (static_cast<long long>(batch.n_tokens) * rounds > 4096) return false;
-    } else if (rounds > decode_part_thresholds[0]) {
-        const int split_rounds = rounds <= decode_part_thresholds[1] ? 4 : 16;
-        if (groups * ((rounds + split_rounds - 1) / split_rounds) > 512) return false;
+    } else {
+        const int split_rounds = decode_split_rounds(groups, rounds);
+        if (split_rounds > 1 && groups * ((rounds + split_rounds - 1) / split_rounds) > 512) return false;
     }
     return !inv_freq || (rotary_dim == head_dim && pairing == 0 && use_rope_table);
 }
@@ -406,6 +406,18 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
                  "paged_attention");
 }
 
+// Where the context of few requests is cut into parts: how many rounds of 64 keys a part (a
+// workgroup) takes, a wavefront per round.  Long parts where they give every compute unit just one
+// workgroup of 16 wavefronts (8 requests of 8 key/value heads at up to 4,096 tokens, 2 at up to
+// 16,384: 1.4 and 3 % of a decode step faster than the next best); else by the length alone, so
+// that a long context gets longer parts rather than hundreds of them (measured at 2 to 16 requests,
+// 2,048 and 8,192 tokens).
+int Ops::decode_split_rounds(long long groups, int rounds) const {
+    const long long long_parts = groups * ((rounds + 15) / 16);
+    if (decode_parts_fill && rounds > 16 && long_parts >= 192 && long_parts <= 256) return 16;
+    return rounds <= decode_part_thresholds[0] ? 1 : (rounds <= decode_part_thresholds[1] ? 4 : 16);
+}
+
 // The first T rows of the step, each the one new token of its request.
 void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv_heads, int head_dim, float scale,
                            int window, const StepBatch& batch, const KVView& kv, int T, Workspace& ws, const FreshKV* fresh) {
@@ -416,7 +428,8 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
     const int hint = batch.context_hint();
     const int bound = hint ? std::min(hint, max_context) : max_context;
     const int rounds = (bound + 63) / 64;
-    const int split_rounds = rounds <= decode_part_thresholds[0] ? 1 : (rounds <= decode_part_thresholds[1] ? 4 : 16);
+    const int chunks = (heads / kv_heads + 15) / 16;
+    const int split_rounds = decode_split_rounds(static_cast<long long>(kv_heads) * chunks * T, rounds);
     const int n_parts = (rounds + split_rounds - 1) / split_rounds;
     const size_t parts = static_cast<size_t>(T) * heads * n_parts;
     float* workspace = static_cast<float*>(ws.raw("attention_decode_parts", parts * (head_dim + 2) * sizeof(float)));

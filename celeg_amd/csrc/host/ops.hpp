@@ -118,6 +118,8 @@ public:
     bool use_blaslt = true;
     int attention_rows_per_tile = 0, attention_rows_form = 0;
     int decode_part_thresholds[2] = {64, 256};
+    bool decode_parts_fill = true;       // parts of 16 rounds where they are one workgroup a compute unit
+    int decode_split_rounds(long long groups, int rounds) const;
     bool attention_general = false;      // always the general attention kernel
     bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
     bool use_qkv_tail = true;          // q/k/v products of many rows take norm, rotation and cache write along

@@ -160,6 +160,7 @@ void set_knobs(Ops& ops, const Json& knobs) {
         else if (name == "use_rope_table") ops.use_rope_table = v != 0;
         else if (name == "use_argmax_parts") ops.use_argmax_parts = v != 0;
         else if (name == "use_head_argmax") ops.use_head_argmax = v != 0;
+        else if (name == "decode_parts_fill") ops.decode_parts_fill = v != 0;
         else if (name == "use_sliced") ops.use_sliced = v != 0;
         else if (name == "use_rows_kernel") ops.use_rows_kernel = v != 0;
         else if (name == "use_tiles") ops.use_tiles = v != 0;
