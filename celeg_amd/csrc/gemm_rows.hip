@@ -144,14 +144,21 @@ __device__ __forceinline__ float finish_output(const GemvParams& p, int r, int n
 // wavefronts split K.  LDS: [waves][MT][streams * CT][4][64] floats, then MT*16 scales.
 template <int MT, int CT, int EPI>
 __global__ __launch_bounds__(64 * rows_max_waves(MT, Streams<EPI>::n * CT))
-void gemm_rows_kernel(const GemvParams p) {
-    const int cols = p.cols;
+void gemm_rows_kernel(const void* const a_, const bf16* const w_, const int* const rows_, const int N, const int K, const int M,
+                      const int shape_, const int stream_rows_, const int w_row_stride_, const int w_kb_stride_,
+                      const int a_strides_, const GemvParams p) {
+    // (What the first loads need comes as arguments of its own, ahead of the struct that holds it too:
+    // the first 14 words of a kernel's arguments arrive in registers with the launch, the rest is
+    // fetched by the wavefronts.  shape_: the columns the workgroup owns, its wavefronts << 8,
+    // w_q_stride << 16; a_strides_: lda, a_k8_stride << 20.)
+    const int cols = shape_ & 0xff;
+    const int w_q_stride_ = shape_ >> 16, lda_ = a_strides_ & 0xfffff, a_k8_stride_ = a_strides_ >> 20;
     constexpr int NS = Streams<EPI>::n;
     constexpr int SC = NS * CT;
     constexpr int COLS = CT * 16;          // columns the tiles hold; the workgroup owns the first `cols` of them
     constexpr int ROWS = MT * 16;
     extern __shared__ float smem[];
-    const int n_waves = blockDim.x >> 6;
+    const int n_waves = (shape_ >> 8) & 0xff;
     float* const red = smem;
     float* const s_scale = smem + static_cast<size_t>(n_waves) * MT * SC * 256;
     // (E_STORE_F32 with row_best: the best logit of every 16 columns of a row, [ROWS][CT])
@@ -159,7 +166,6 @@ void gemm_rows_kernel(const GemvParams p) {
     // the wavefront's number as a scalar: the branches on its range of k are then uniform
     // ones (the matrix instructions do not honour a lane mask)
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int M = p.M, N = p.N, K = p.K;
     const int n0 = blockIdx.x * cols;
     const int row0 = blockIdx.y * ROWS;        // the workgroup's first row
     const int c16 = lane & 15, q = lane >> 4;
@@ -169,7 +175,7 @@ void gemm_rows_kernel(const GemvParams p) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int m = min(row0 + t * 16 + c16, M - 1);
-        arow[t] = static_cast<const bf16*>(p.a) + static_cast<size_t>(p.rows ? p.rows[m] : m) * p.lda + q * p.a_k8_stride;
+        arow[t] = static_cast<const bf16*>(a_) + static_cast<size_t>(rows_ ? rows_[m] : m) * lda_ + q * a_k8_stride_;
     }
     const bf16* wcol[SC];
 #pragma unroll
@@ -179,7 +185,7 @@ void gemm_rows_kernel(const GemvParams p) {
             // a lane whose column is not the workgroup's repeats the first column's address (no memory traffic of its own)
             const int jn = ct * 16 + c16;
             const int n = jn < cols && n0 + jn < N ? n0 + jn : n0;
-            wcol[s * CT + ct] = p.w + (static_cast<size_t>(s) * p.stream_rows + n) * p.w_row_stride + q * p.w_q_stride;
+            wcol[s * CT + ct] = w_ + (static_cast<size_t>(s) * stream_rows_ + n) * w_row_stride_ + q * w_q_stride_;
         }
     const int nkb = K >> 5;                    // K % 32 == 0 (checked by the host)
     const int kb_begin = wave * nkb / n_waves, kb_end = (wave + 1) * nkb / n_waves;
@@ -196,10 +202,10 @@ void gemm_rows_kernel(const GemvParams p) {
     auto fetch = [&](int kb, bf16x8_t (&av)[MT], bf16x8_t (&wv)[SC]) {
 #pragma unroll
         for (int s = 0; s < SC; ++s)
-            wv[s] = *reinterpret_cast<const bf16x8_t*>(wcol[s] + static_cast<size_t>(kb) * p.w_kb_stride);
+            wv[s] = *reinterpret_cast<const bf16x8_t*>(wcol[s] + static_cast<size_t>(kb) * w_kb_stride_);
 #pragma unroll
         for (int t = 0; t < MT; ++t)
-            av[t] = *reinterpret_cast<const bf16x8_t*>(arow[t] + static_cast<size_t>(kb) * 4 * p.a_k8_stride);
+            av[t] = *reinterpret_cast<const bf16x8_t*>(arow[t] + static_cast<size_t>(kb) * 4 * a_k8_stride_);
     };
     auto multiply = [&](const bf16x8_t (&av)[MT], const bf16x8_t (&wv)[SC]) {
 #pragma unroll
@@ -219,11 +225,11 @@ void gemm_rows_kernel(const GemvParams p) {
     // ---- the rows' 1/rms from the partial sums of squares (likewise): LPR neighbouring
     // threads share a row
     if (p.stats) {
-        const int lpr = blockDim.x / ROWS;           // a power of two, 1 .. 32
+        const int lpr = n_waves * 64 / ROWS;         // a power of two, 1 .. 32
         const int r = threadIdx.x / lpr, sub = threadIdx.x % lpr;
         const int nb = p.n_stat_blocks;
         const int m = min(row0 + r, M - 1);
-        const float* srow = p.stats + static_cast<size_t>(p.rows ? p.rows[m] : m) * p.stats_ld;
+        const float* srow = p.stats + static_cast<size_t>(rows_ ? rows_[m] : m) * p.stats_ld;
         float ssq = 0.f;
         for (int b0 = 0; b0 < nb; b0 += 8 * lpr) {   // the same trips for every thread
             float part[8];
@@ -255,7 +261,7 @@ void gemm_rows_kernel(const GemvParams p) {
     __syncthreads();
 
     // ---- thread e takes row e / COLS, column e % COLS of the workgroup's tile
-    const int n_threads = blockDim.x;
+    const int n_threads = n_waves * 64;
     for (int e = threadIdx.x; e < ROWS * COLS; e += n_threads) {
         const int rl = e / COLS, j = e % COLS;      // row inside the workgroup's rows
         const int t = rl >> 4, rr = rl & 15, ct = j >> 4, jj = j & 15;
@@ -390,7 +396,10 @@ static int launch_rows(const GemvParams& params, int waves, int cols, hipStream_
         raised = true;
     }
     dim3 grid((p.N + cols - 1) / cols, (p.M + MT * 16 - 1) / (MT * 16)), block(waves * 64);
-    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p);
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, CT, EPI>), grid, block, lds, stream, p.a, p.w, p.rows, p.N, p.K, p.M,
+                       cols | (waves << 8) | (static_cast<int>(p.w_q_stride) << 16), p.stream_rows,
+                       static_cast<int>(p.w_row_stride), static_cast<int>(p.w_kb_stride),
+                       p.lda | (static_cast<int>(p.a_k8_stride) << 20), p);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -424,7 +433,8 @@ extern "C" int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t st
     if (p.M <= 0 || p.N <= 0) return 0;
     if (p.M > 64 || p.K <= 0 || (p.K % 32) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
     if ((p.w_row_stride % 8) || (p.w_kb_stride % 8) || (p.w_q_stride % 8) || p.w_row_stride <= 0 ||
-        p.w_kb_stride <= 0 || p.w_q_stride <= 0)
+        p.w_kb_stride <= 0 || p.w_q_stride <= 0 || p.w_row_stride > 0x7fffffffLL || p.w_kb_stride > 0x7fffffffLL ||
+        p.w_q_stride > 0x7fffLL || p.a_k8_stride > 0x7ffLL || p.lda > 0xfffff)      // (they travel in packed words)
         return static_cast<int>(hipErrorInvalidValue);
     if ((p.a_k8_stride % 8) || p.a_k8_stride <= 0 || (p.out_k8_stride % 8) || p.out_k8_stride <= 0 ||
         (p.out_bf16 && ((p.bf16_k8_stride % 8) || p.bf16_k8_stride <= 0)))
