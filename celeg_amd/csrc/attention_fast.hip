@@ -516,7 +516,7 @@ extern "C" int celeg_attention_rows_bf16(
 // Decode attention works on rounds of 64 keys.
 #define DEC_KEYS 64
 
-// Joins the parts of one (request, query head), a part being split_rounds rounds of 64 keys:
+// Joins the parts of one (request, query head), a part being some rounds of 64 keys:
 // out = sum_i e^(m_i - m) o_i / sum_i e^(m_i - m) l_i.
 // A lane owns an output dimension (and the (m, l) of parts lane, lane + 64, ..).  The parts'
 // outputs are asked for 32 at a time without conditions, the first 32 before anything is
@@ -525,13 +525,15 @@ template <int HD>
 __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
     const float* __restrict__ ws_o, const float* __restrict__ ws_ml,
     const int* __restrict__ positions, bf16* __restrict__ out, int ldo, int q_heads, int n_splits,
-    int window, int split_rounds) {
+    int window, int n_parts) {
     constexpr int DD = HD / 64, CH = 32;
     const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int first = lo / DEC_KEYS / split_rounds, n_all = pos / DEC_KEYS / split_rounds - first + 1;
-    const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits + first;
+    // the request's rounds were shared out evenly over the parts (see decode_part_rounds)
+    const int total = pos / DEC_KEYS - lo / DEC_KEYS + 1, per = (total + n_parts - 1) / n_parts;
+    const int n_all = (total + per - 1) / per;
+    const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits;
     const float* __restrict__ op = ws_o + base * HD + lane;
     float o[CH][DD];
     auto fetch = [&](int j0) {
@@ -676,7 +678,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     const int* __restrict__ table, const int* __restrict__ token_slot, const int* __restrict__ positions,
     int ldq, int table_stride, bf16* __restrict__ out, int ldo, int kv_heads, int group, int page_tokens, int page_shift, int n_layers, int layer,
     float scale, int window, float* __restrict__ ws_o, float* __restrict__ ws_ml, int n_splits,
-    int split_rounds, const DecodeFresh fresh) {
+    int n_parts, const DecodeFresh fresh) {
     constexpr int KS = HD / 32;   // steps of 32 dims in q.k
     constexpr int DT = HD / 16;   // 16-dim tiles of the output
     extern __shared__ float smem_heads[];
@@ -734,12 +736,17 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
 
     // the workgroup's rounds: all of the request's, or (SPLIT) part blockIdx.z of them; its
     // wavefronts take them in turn
-    const int r_begin = SPLIT ? max(lo / DEC_KEYS, static_cast<int>(blockIdx.z) * split_rounds) : lo / DEC_KEYS;
+    // (SPLIT: the request's rounds, from the first of its window to the one of its own position, are
+    // shared out evenly over the n_parts workgroups, so that a context well below what the launch was
+    // sized for still keeps all of them busy: `per` rounds each, the last parts none)
+    const int first_round = lo / DEC_KEYS;
+    const int total = pos / DEC_KEYS - first_round + 1, per = SPLIT ? (total + n_parts - 1) / n_parts : 0;
+    const int r_begin = SPLIT ? first_round + static_cast<int>(blockIdx.z) * per : first_round;
     const int last_round = last_key < 0 ? -1 : last_key / DEC_KEYS;
-    const int r_end = SPLIT ? min(last_round, static_cast<int>(blockIdx.z) * split_rounds + split_rounds - 1) : last_round;
+    const int r_end = SPLIT ? min(last_round, r_begin + per - 1) : last_round;
     // the fresh token belongs to the part that holds its position (which may hold no other key)
-    const bool adds_fresh = FRESH && wave == 0 && (!SPLIT || static_cast<int>(blockIdx.z) == pos / DEC_KEYS / split_rounds);
-    const bool part_of_fresh = FRESH && (!SPLIT || static_cast<int>(blockIdx.z) == pos / DEC_KEYS / split_rounds);
+    const bool part_of_fresh = FRESH && (!SPLIT || static_cast<int>(blockIdx.z) == (pos / DEC_KEYS - first_round) / per);
+    const bool adds_fresh = part_of_fresh && wave == 0;
     if (SPLIT && r_begin > r_end && !part_of_fresh) return;     // the whole workgroup
     // the new key and value of the wavefront that adds them: asked for ahead of the rounds
     bf16x8_t k_raw[KS];
@@ -888,8 +895,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
         }
     };
     if (adds_fresh && !LAZY) add_fresh();
-    if constexpr (SPLIT && WAVES == 1) {       // a part of one round
-        if (r_begin <= r_end) one_round(r_begin, [&]() { if (FRESH) prepare_q(); });
+    if constexpr (SPLIT && WAVES == 1) {       // a part of one round (more, if the caller gave fewer parts than rounds)
+        for (int r = r_begin; r <= r_end; ++r) one_round(r, [&]() { if (FRESH && !q_ready) prepare_q(); });
     } else {
         for (int r = r_begin + wave; r <= r_end; r += WAVES) one_round(r, []() {});
     }
@@ -988,7 +995,7 @@ static int launch_decode_parts(const void* q, int ldq, const void* k_pool, const
                        static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table,
                        token_slot, positions, ldq, table_stride, static_cast<bf16*>(out), ldo, kv_heads,
                        group, page_tokens, page_shift, n_layers, layer, scale, window, ws_o, ws_ml,
-                       n_splits, split_rounds, fresh);
+                       n_splits, n_parts, fresh);
     return 0;
 }
 
@@ -1029,10 +1036,11 @@ static int attention_decode(
                                             n_layers, layer, scale, window, fresh, stream);
         return static_cast<int>(hipErrorInvalidValue);
     }
-    // Parts of split_rounds rounds of 64 keys (1, 4 or 16), one workgroup each with a wavefront per
-    // round (8 at most for heads of 128), n_parts of them per request: the caller chooses both
-    // so that n_parts * split_rounds * 64 keys cover the longest context of the step, and a
-    // longer context gets longer parts instead of more of them.
+    // n_parts workgroups per request and key/value head, of 1, 4 or 16 wavefronts (split_rounds; 8
+    // at most for heads of 128) that take a round of 64 keys each at a time: the caller chooses both
+    // so that n_parts * split_rounds * 64 keys cover the longest context the launch is meant for, and
+    // a longer context gets longer parts instead of more of them.  A request's rounds are shared
+    // out evenly over its workgroups, whatever its context.
     if ((split_rounds != 1 && split_rounds != 4 && split_rounds != 16) || n_parts <= 0 || n_parts > n_splits)
         return static_cast<int>(hipErrorInvalidValue);
 #define CELEG_SPLIT_ARGS                                                                           \
@@ -1048,7 +1056,7 @@ static int attention_decode(
     }                                                                                              \
     hipLaunchKernelGGL(attention_decode_reduce_kernel<HD_>, dim3(q_heads, n_rows), dim3(64), 0,   \
                        stream, ws_o, ws_ml, positions, static_cast<bf16*>(out), ldo, q_heads,     \
-                       n_splits, window, split_rounds)
+                       n_splits, window, n_parts)
     if (head_dim == 64) { CELEG_SPLIT_HEADS(64, 16); }
     else if (head_dim == 128) { CELEG_SPLIT_HEADS(128, 8); }
     else return static_cast<int>(hipErrorInvalidValue);

@@ -406,16 +406,19 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
                  "paged_attention");
 }
 
-// Where the context of few requests is cut into parts: how many rounds of 64 keys a part (a
-// workgroup) takes, a wavefront per round.  Long parts where they give every compute unit just one
-// workgroup of 16 wavefronts (8 requests of 8 key/value heads at up to 4,096 tokens, 2 at up to
-// 16,384: 1.4 and 3 % of a decode step faster than the next best); else by the length alone, so
-// that a long context gets longer parts rather than hundreds of them (measured at 2 to 16 requests,
-// 2,048 and 8,192 tokens).
+// Where the context of few requests is cut into parts: how many wavefronts a part's workgroup has
+// (1, 4 or 16: as many rounds of 64 keys does it take at a time; a request's rounds are shared out
+// evenly over its parts).  Workgroups of 16 where they give every compute unit just one (8 requests
+// of 8 key/value heads at up to 4,096 tokens: 0.463 against 0.475 and 0.479 ms a decode step; 2
+// requests at up to 16,384: 3 % faster); else by the length, so that a long context gets longer
+// parts rather than hundreds of them, and at short lengths workgroups of 4 once there are enough
+// of them for every compute unit (2, 4 and 16 requests at 2,048 tokens: 0.5 to 1.4 % faster than
+// single wavefronts; 1 request: slower).  Measured at 1 to 16 requests, 2,048 and 8,192 tokens.
 int Ops::decode_split_rounds(long long groups, int rounds) const {
     const long long long_parts = groups * ((rounds + 15) / 16);
     if (decode_parts_fill && rounds > 16 && long_parts >= 192 && long_parts <= 256) return 16;
-    return rounds <= decode_part_thresholds[0] ? 1 : (rounds <= decode_part_thresholds[1] ? 4 : 16);
+    if (rounds <= decode_part_thresholds[0]) return decode_parts_fill && rounds > 4 && groups * ((rounds + 3) / 4) >= 256 ? 4 : 1;
+    return rounds <= decode_part_thresholds[1] ? 4 : 16;
 }
 
 // The first T rows of the step, each the one new token of its request.
