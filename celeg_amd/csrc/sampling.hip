@@ -597,13 +597,13 @@ __global__ __launch_bounds__(MERGE_THREADS) void argmax_merge_kernel(
     const int lane = tid & (CELEG_WAVE - 1), wave = tid / CELEG_WAVE;
     const unsigned long long* row = best + r;
     unsigned long long mine = 0ull;
-    for (int j0 = 0; j0 < parts; j0 += 8 * MERGE_THREADS) {         // eight loads of a thread under way at a time
-        unsigned long long v[8];
+    for (int j0 = 0; j0 < parts; j0 += 16 * MERGE_THREADS) {        // sixteen loads of a thread under way at a time:
+        unsigned long long v[16];                                   // one trip to memory for 65,536 columns in tiles of 16
 #pragma unroll
-        for (int j = 0; j < 8; ++j)      // (a part twice changes nothing)
+        for (int j = 0; j < 16; ++j)     // (a part twice changes nothing)
             v[j] = row[static_cast<size_t>(min(j0 + tid + MERGE_THREADS * j, parts - 1)) * ld];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) mine = max(mine, v[j]);
+        for (int j = 0; j < 16; ++j) mine = max(mine, v[j]);
     }
 #pragma unroll
     for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) mine = max(mine, __shfl_xor(mine, off, CELEG_WAVE));
