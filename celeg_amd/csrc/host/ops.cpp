@@ -412,12 +412,12 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
 // of 8 key/value heads at up to 4,096 tokens: 0.463 against 0.475 and 0.479 ms a decode step; 2
 // requests at up to 16,384: 3 % faster); else by the length, so that a long context gets longer
 // parts rather than hundreds of them, and at short lengths workgroups of 4 once there are enough
-// of them for every compute unit (2, 4 and 16 requests at 2,048 tokens: 0.5 to 1.4 % faster than
-// single wavefronts; 1 request: slower).  Measured at 1 to 16 requests, 2,048 and 8,192 tokens.
+// of them for half the compute units (1, 2, 4 and 16 requests at 2,048 tokens: 0.5 to 1.4 % faster
+// than single wavefronts).  Measured at 1 to 16 requests, 2,048 and 8,192 tokens.
 int Ops::decode_split_rounds(long long groups, int rounds) const {
     const long long long_parts = groups * ((rounds + 15) / 16);
     if (decode_parts_fill && rounds > 16 && long_parts >= 192 && long_parts <= 256) return 16;
-    if (rounds <= decode_part_thresholds[0]) return decode_parts_fill && rounds > 4 && groups * ((rounds + 3) / 4) >= 256 ? 4 : 1;
+    if (rounds <= decode_part_thresholds[0]) return decode_parts_fill && rounds > 4 && groups * ((rounds + 3) / 4) >= 128 ? 4 : 1;
     return rounds <= decode_part_thresholds[1] ? 4 : 16;
 }
 
