@@ -530,7 +530,7 @@ __global__ __launch_bounds__(64) void attention_decode_reduce_kernel(
     const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-    // the request's rounds were shared out evenly over the parts (see decode_part_rounds)
+    // the request's rounds were shared out evenly over the parts (the same arithmetic as in attention_decode_heads_kernel)
     const int total = pos / DEC_KEYS - lo / DEC_KEYS + 1, per = (total + n_parts - 1) / n_parts;
     const int n_all = (total + per - 1) / per;
     const size_t base = (static_cast<size_t>(t) * q_heads + h) * n_splits;

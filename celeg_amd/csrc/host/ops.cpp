@@ -70,6 +70,14 @@ Json Ops::paths_json() const {
     return out;
 }
 
+// the bound on the context that a step's decode attention is launched for: the step's longest
+// context, or what the step's recorded graph is good for
+static int hint_of(const StepBatch& batch, const KVView& kv) {
+    const int max_context = kv.table_stride * kv.page_tokens;
+    const int hint = batch.context_hint();
+    return hint ? std::min(hint, max_context) : max_context;
+}
+
 // ---------------------------------------------------------------------------- row-wise
 void Ops::embed(const Tensor& table, const int* token_ids, const Tensor& out) {
     dev(table, "table");
@@ -347,10 +355,8 @@ bool Ops::attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, in
     // faster; 264 workgroups: 1 us a layer faster).
     const int chunks = (heads / kv.kv_heads + 15) / 16;
     const long long groups = static_cast<long long>(kv.kv_heads) * chunks * batch.n_tokens;
-    const bool whole = attention_decode_whole < 0 ? groups >= 192 : attention_decode_whole > 0;
-    const int max_context = kv.table_stride * kv.page_tokens;
-    const int hint = batch.context_hint();
-    const int rounds = ((hint ? std::min(hint, max_context) : max_context) + 63) / 64;
+    const int rounds = (hint_of(batch, kv) + 63) / 64;
+    const bool whole = decode_whole(groups, rounds);
     if (whole) {
         // the kernel's loop over the rounds runs 1.7 % slower in this form, which outweighs the
         // kernel saved from about 8,192 tokens for each of 64 requests on (at 32,768: 4.94 against
@@ -414,6 +420,15 @@ void Ops::paged_attention(const Tensor& q, const Tensor& out, int heads, int kv_
 // parts rather than hundreds of them, and at short lengths workgroups of 4 once there are enough
 // of them for half the compute units (1, 2, 4 and 16 requests at 2,048 tokens: 0.5 to 1.4 % faster
 // than single wavefronts).  Measured at 1 to 16 requests, 2,048 and 8,192 tokens.
+// One workgroup a (request, key/value head), its wavefronts taking the rounds in turn and no second
+// kernel, once there are enough of them: 192 (24 requests of 8 key/value heads) at any length, 96 at
+// contexts up to 4,096 tokens (12 and 16 requests at 2,048 tokens: 1 and 3 % of a decode step
+// faster than in parts; 16 requests at 8,192: 3 % slower).
+bool Ops::decode_whole(long long groups, int rounds) const {
+    if (attention_decode_whole >= 0) return attention_decode_whole > 0;
+    return groups >= 192 || (groups >= 96 && rounds <= 64);
+}
+
 int Ops::decode_split_rounds(long long groups, int rounds) const {
     const long long long_parts = groups * ((rounds + 15) / 16);
     if (decode_parts_fill && rounds > 16 && long_parts >= 192 && long_parts <= 256) return 16;
@@ -432,6 +447,7 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
     const int bound = hint ? std::min(hint, max_context) : max_context;
     const int rounds = (bound + 63) / 64;
     const int chunks = (heads / kv_heads + 15) / 16;
+    const int whole = decode_whole(static_cast<long long>(kv_heads) * chunks * T, rounds) ? 1 : 0;
     const int split_rounds = decode_split_rounds(static_cast<long long>(kv_heads) * chunks * T, rounds);
     const int n_parts = (rounds + split_rounds - 1) / split_rounds;
     const size_t parts = static_cast<size_t>(T) * heads * n_parts;
@@ -460,7 +476,7 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
                          fresh->q_weight ? fresh->q_weight->as<float>() : nullptr, fresh->k_weight ? fresh->k_weight->as<float>() : nullptr,
                          fresh->eps, cos_sin, kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot, batch.positions, workspace,
                          workspace + parts * head_dim, n_parts, out.data, heads * head_dim, T, heads, kv_heads, head_dim,
-                         kv.page_tokens, kv.n_layers, kv.layer, scale, window, attention_decode_whole, split_rounds, n_parts, stream),
+                         kv.page_tokens, kv.n_layers, kv.layer, scale, window, whole, split_rounds, n_parts, stream),
                      "attention for decode rows with fresh keys (bfloat16)");
         return;
     }
@@ -468,7 +484,7 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
     kernel_check(celeg_attention_decode_bf16(q.data, rows_of(q, "q"), kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot,
                                              batch.positions, workspace, workspace + parts * head_dim, n_parts, out.data,
                                              heads * head_dim, T, heads, kv_heads, head_dim, kv.page_tokens, kv.n_layers,
-                                             kv.layer, scale, window, attention_decode_whole, split_rounds, n_parts, stream),
+                                             kv.layer, scale, window, whole, split_rounds, n_parts, stream),
                  "attention for decode rows (bfloat16)");
 }
 

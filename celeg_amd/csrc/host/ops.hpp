@@ -120,6 +120,7 @@ public:
     int decode_part_thresholds[2] = {64, 256};
     bool decode_parts_fill = true;       // parts of 16 rounds where they are one workgroup a compute unit
     int decode_split_rounds(long long groups, int rounds) const;
+    bool decode_whole(long long groups, int rounds) const;
     bool attention_general = false;      // always the general attention kernel
     bool use_rope_table = true, use_argmax_parts = true, use_sliced = true, use_rows_kernel = true, use_tiles = true;
     bool use_qkv_tail = true;          // q/k/v products of many rows take norm, rotation and cache write along
