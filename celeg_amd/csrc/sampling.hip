@@ -263,8 +263,33 @@ __device__ __forceinline__ bool top_k_ranked(
     const int lane = tid & (CELEG_WAVE - 1), wave = tid / CELEG_WAVE;
     const bool pen = seen && penalty > 1.0f;
     const float inv_penalty = 1.0f / penalty;
+    // Place j of a thread holds element tid + SAMPLE_THREADS * j, or, where the row can be read 16
+    // bytes a lane (and the seen marks 4), element 4 * (tid + SAMPLE_THREADS * (j / 4)) + j % 4: a
+    // load of one logit or one mark a lane costs the vector cache as much as one of four (a row of
+    // 65,536 logits with its marks: 2,048 loads of a wavefront instead of 512).
+    const bool by_fours = (vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0 &&
+                          (!pen || (reinterpret_cast<uintptr_t>(seen) & 3) == 0);
+    auto index_of = [&](int j) { return by_fours ? 4 * (tid + SAMPLE_THREADS * (j >> 2)) + (j & 3) : tid + SAMPLE_THREADS * j; };
     uint32_t keys[KPT];
-    {
+    if (by_fours) {
+        floatx4_t v[KPT / 4];
+        unsigned sn[KPT / 4];
+        const int n4 = vocab >> 2;
+#pragma unroll
+        for (int jj = 0; jj < KPT / 4; ++jj) {
+            const int g = min(tid + SAMPLE_THREADS * jj, n4 - 1);       // clamped, masked below
+            v[jj] = reinterpret_cast<const floatx4_t*>(row)[g];
+            sn[jj] = pen ? reinterpret_cast<const unsigned*>(seen)[g] : 0u;
+        }
+#pragma unroll
+        for (int jj = 0; jj < KPT / 4; ++jj)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float x0 = v[jj][e];
+                const float x = ((sn[jj] >> (8 * e)) & 0xffu) ? (x0 >= 0.0f ? x0 * inv_penalty : x0 * penalty) : x0;
+                keys[4 * jj + e] = tid + SAMPLE_THREADS * jj < n4 ? order_key(x) : 0u;
+            }
+    } else {
         float v[KPT];
         unsigned char sn[KPT];
 #pragma unroll
@@ -303,9 +328,9 @@ __device__ __forceinline__ bool top_k_ranked(
     lower = lower > 8u ? lower - 8u : 0u;
 #pragma unroll
     for (int j = 0; j < KPT; ++j)
-        if (tid + SAMPLE_THREADS * j < vocab && keys[j] >= lower) {
+        if (index_of(j) < vocab && keys[j] >= lower) {
             const unsigned int p = atomicAdd(&sel[1], 1u);
-            if (p < SAMPLE_RANK_CAP) gathered[p].y = static_cast<unsigned>(tid + SAMPLE_THREADS * j);
+            if (p < SAMPLE_RANK_CAP) gathered[p].y = static_cast<unsigned>(index_of(j));
         }
     __syncthreads();
     const int n = static_cast<int>(sel[1]);
