@@ -373,9 +373,11 @@ static RowsShape rows_shape(int M, int N, int K, int streams) {
     const int nkb = K / 32;
     s.waves = rows_max_waves(s.mt, streams * s.ct);
     if (K <= 2048 && s.waves > 8) s.waves = 8;     // a short K: two workgroups of 8 a compute unit were the faster
-    // tiles of 64 columns (an output head): 4 wavefronts (65,536 columns by 1,024: 32.4 against 36.6 us at
-    // 32 rows, 31.9 against 34.7 at 16; at 64 rows LDS holds no more than 4 anyway)
-    if (s.ct == 4 && s.waves > 4) s.waves = 4;
+    // tiles of 64 columns (an output head): 2 wavefronts, so that a compute unit holds four such
+    // workgroups and their ends overlap (65,536 columns by 1,024: 36.6 against 42.3 us with 4 wavefronts at
+    // 64 rows, 29.5 against 30.7 at 32, 26.8 against 31.0 at 16; by 2,048: 60.3 against 64.0 at 64 rows;
+    // one wavefront and eight are slower)
+    if (s.ct == 4 && s.waves > 2) s.waves = 2;
     while (s.waves > 1 && s.waves * 2 > nkb) s.waves >>= 1;
     if (g_force_waves > 0 && g_force_waves <= rows_max_waves(s.mt, streams * s.ct)) s.waves = g_force_waves;
     return s;
