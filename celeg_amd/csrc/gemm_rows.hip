@@ -307,7 +307,7 @@ void gemm_rows_kernel(const void* const a_, const bf16* const w_, const int* con
             unsigned long long b = 0ull;
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) b = max(b, s_best[rl * CT + ct]);
-            p.row_best[static_cast<size_t>(blockIdx.x) * p.row_best_ld + row0 + rl] = b;
+            p.row_best[static_cast<size_t>(row0 + rl) * p.row_best_ld + blockIdx.x] = b;
         }
     }
 }
@@ -422,6 +422,7 @@ static int streams_of(int epi) { return epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3
 
 // Number of workgroups for these sizes, which is also the number of partial sums of
 // squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
+extern "C" int celeg_gemm_rows_cols(int M, int N, int K, int epi) { return rows_shape(M, N, K, streams_of(epi)).cols; }
 extern "C" int celeg_gemm_rows_blocks(int M, int N, int K, int epi) {
     const RowsShape s = rows_shape(M, N, K, streams_of(epi));
     return (N + s.cols - 1) / s.cols;
@@ -445,7 +446,7 @@ extern "C" int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t st
         return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.taps > ROWS_MAX_TAPS || p.stream_rows != p.N))
         return static_cast<int>(hipErrorInvalidValue);
-    if (p.row_best && (epi != E_STORE_F32 || p.row_best_ld < p.M || p.row_best_parts < celeg_gemm_rows_blocks(p.M, p.N, p.K, epi)))
+    if (p.row_best && (epi != E_STORE_F32 || p.row_best_rows < p.M || p.row_best_ld < celeg_gemm_rows_blocks(p.M, p.N, p.K, epi)))
         return static_cast<int>(hipErrorInvalidValue);
     switch (epi) {
         case E_STORE: return launch_epilogue<E_STORE>(p, stream);

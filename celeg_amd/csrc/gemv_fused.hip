@@ -157,7 +157,7 @@ __device__ __forceinline__ void gemv_epilogue(const GemvParams& p, floatx4_t (&a
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = mt * 16 + 4 * q + r;
-                if (c16 == 0 && m < M) p.row_best[static_cast<size_t>(tile) * p.row_best_ld + m] = best[r];
+                if (c16 == 0 && m < M) p.row_best[static_cast<size_t>(m) * p.row_best_ld + tile] = best[r];
             }
         }
         if (EPI == E_RESIDUAL && p.stats_out) {
@@ -470,7 +470,7 @@ extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, in
     if (epi == E_CONV && (p.taps < 1 || p.taps > CONV_PREFETCH_TAPS || p.stream_rows != p.N))
         return static_cast<int>(hipErrorInvalidValue);
     const int tiles = (p.N + 15) / 16, chunks = (p.K + 63) / 64;
-    if (p.row_best && (epi != E_STORE_F32 || p.row_best_ld < p.M || p.row_best_parts < tiles)) return static_cast<int>(hipErrorInvalidValue);
+    if (p.row_best && (epi != E_STORE_F32 || p.row_best_rows < p.M || p.row_best_ld < tiles)) return static_cast<int>(hipErrorInvalidValue);
     const int streams = epi == E_SWIGLU ? 2 : (epi == E_CONV ? 3 : 1);
     const int mt = p.M <= 16 ? 1 : (p.M <= 32 ? 2 : 4);
     const size_t limit = 144 * 1024;

@@ -48,9 +48,9 @@ struct GemvParams {
     int reserved_;
     const float* norm_w;    // A_NORM: [K]
     // 32-bit store of an output head: beside the logits, the best (logit, index) of every
-    // workgroup's (or wavefront's) columns, packed as packed_logit packs them: [parts, row_best_ld >=
-    // rows], part j from the j-th share of columns (the rows of a part side by side: a workgroup's
-    // values are one run of memory); or null
+    // workgroup's (or wavefront's) columns, packed as packed_logit packs them: [rows, row_best_ld >=
+    // parts], part j from the j-th share of columns (the parts of a row one after the other: what
+    // picks a row's token afterwards reads one run of memory); or null
     unsigned long long* row_best;
     // ---- bytes 192..
     // layouts that only the kernel for 9 to 64 rows reads: element (m, k) of a lies at
@@ -60,7 +60,7 @@ struct GemvParams {
     // bf16_k8_stride, and element (n, k) of w at
     //   n * w_row_stride + (k / 32) * w_kb_stride + (k % 32 / 8) * w_q_stride + k % 8
     long long a_k8_stride, out_k8_stride, bf16_k8_stride, w_q_stride;
-    int row_best_ld, row_best_parts;     // (room for row_best_parts parts: a launch that would leave more is refused)
+    int row_best_ld, row_best_rows;     // (room for row_best_rows rows of row_best_ld parts: a launch that would leave more is refused)
 };
 static_assert(offsetof(GemvParams, M) == 64 && offsetof(GemvParams, conv_w) == 128 && offsetof(GemvParams, a_k8_stride) == 192,
               "the fields of GemvParams are grouped by 64-byte lines");

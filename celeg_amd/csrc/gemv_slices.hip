@@ -215,7 +215,7 @@ void gemv_slices_kernel(const void* const a_, const bf16* const w_, const int* c
             // neighbouring lanes): one part of the row
             const unsigned long long b = group_best_logit<MP>(sum[0], e_ok, n0 + tile_ct * MP);
             if (t % MP == 0 && em < M && t < MP * MP * CT)
-                p.row_best[static_cast<size_t>(blockIdx.x * CT + tile_ct) * p.row_best_ld + em] = b;
+                p.row_best[static_cast<size_t>(em) * p.row_best_ld + blockIdx.x * CT + tile_ct] = b;
         }
     } else if (EPI == E_RESIDUAL) {
         // the product enters the sum rounded to bfloat16, as where it is a tensor of its own
@@ -348,6 +348,7 @@ extern "C" int celeg_gemv_params_size() { return static_cast<int>(sizeof(GemvPar
 
 // Number of workgroups for these sizes, which is also the number of partial sums of
 // squares a row gets from the "residual" epilogue: the caller sizes stats_out [>= M, >= blocks].
+extern "C" int celeg_gemv_slices_cols(int M, int N, int K) { return slices_shape(M, N, K, E_RESIDUAL).cols; }
 extern "C" int celeg_gemv_slices_blocks(int M, int N, int K) {
     const SlicesShape s = slices_shape(M, N, K, E_RESIDUAL);
     return (N + s.cols - 1) / s.cols * s.ct;
@@ -369,7 +370,7 @@ extern "C" int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t 
         return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.taps > SLICES_MAX_TAPS || p.stream_rows != p.N))
         return static_cast<int>(hipErrorInvalidValue);
-    if (p.row_best && (epi != E_STORE_F32 || p.row_best_ld < p.M || p.row_best_parts < celeg_gemv_slices_blocks(p.M, p.N, p.K)))
+    if (p.row_best && (epi != E_STORE_F32 || p.row_best_rows < p.M || p.row_best_ld < celeg_gemv_slices_blocks(p.M, p.N, p.K)))
         return static_cast<int>(hipErrorInvalidValue);
     switch (epi) {
         case E_STORE: return launch_epilogue<E_STORE>(p, stream);

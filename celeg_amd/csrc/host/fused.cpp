@@ -132,7 +132,7 @@ void norm_linear(Runtime& rt, const Tensor& h, const Norm::Foldable& norm, const
     args.conv = extras.conv;
     args.row_best = extras.row_best;
     args.row_best_ld = extras.row_best_ld;
-    args.row_best_parts = extras.row_best_parts;
+    args.row_best_rows = extras.row_best_rows;
     rt.ops.last_best_parts = 0;
     if (sliced(rt, M, width) && w.dtype == DType::BF16 && (streamed || w.shape[0] / streams <= SLICED_MAX_COLUMNS)) {
         // the stream's bfloat16 copy times the weight with the norm's weight folded in, scaled

@@ -71,12 +71,14 @@ int celeg_argmax_rows(const float* logits, int ld, int rows, int vocab, const fl
 int celeg_argmax_merge(const unsigned long long* best, int ld, int parts, int rows, const int* iparams, int* out_tokens,
                        int* last_tokens, hipStream_t stream);
 int celeg_sample(const float* logits, int ld, int rows, int vocab, const float* fparams, const int* iparams,
-                 uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens, hipStream_t stream);
+                 uint8_t* seen, size_t seen_stride, int* out_tokens, int* last_tokens, const unsigned long long* best,
+                 int best_ld, int best_parts, int best_cols, hipStream_t stream);
 int celeg_mark_seen(uint8_t* seen, size_t stride, int n_slots, int vocab, const int* tokens, const int* slots, int n,
                     hipStream_t stream);
 // gemv_slices.hip, gemm_rows.hip, gemv_fused.hip: the fused products for up to 64 rows
 int celeg_gemv_params_size();
 int celeg_gemv_slices_blocks(int M, int N, int K);
+int celeg_gemv_slices_cols(int M, int N, int K);
 int celeg_gemv_slices(const GemvParams* params, int epi, hipStream_t stream);
 int celeg_stream_prepare(const float* h, int ldh, void* xb, int ldx, long long xb_k8, float* stats, int stats_ld,
                          int rows, int width, hipStream_t stream);
@@ -87,6 +89,7 @@ int celeg_embed_stream_prologue(const void* table, int* ids, float* out, void* x
                                 const int* updates, int capacity, const int* token_slot, const int* last_tokens,
                                 hipStream_t stream);
 int celeg_gemm_rows_blocks(int M, int N, int K, int epi);
+int celeg_gemm_rows_cols(int M, int N, int K, int epi);
 int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t stream);
 int celeg_gemv_fused(const GemvParams* params, int amode, int epi, int shape, hipStream_t stream);
 int celeg_embed_stats(const void* table, const int* ids, float* out, float* stats, int stats_ld, int rows, int width,

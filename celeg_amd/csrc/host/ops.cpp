@@ -490,12 +490,14 @@ void Ops::attention_decode(const Tensor& q, const Tensor& out, int heads, int kv
 
 // ---------------------------------------------------------------------------- sampling
 void Ops::sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen, size_t seen_stride,
-                 int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws, const HeadBest* head_best) {
+                 int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws, const HeadBest* head_best, bool penalised) {
     dev(logits, "logits", DType::F32, false);
     const int R = static_cast<int>(logits.shape[0]), V = static_cast<int>(logits.shape[1]);
     if (R == 0) return;
-    if (all_greedy && use_head_argmax && head_best && head_best->logits == logits.data && head_best->rows >= R &&
-        head_best->parts > 0) {
+    // what the head's product left beside these very logits, if it did
+    const bool left = use_head_argmax && head_best && head_best->logits == logits.data && head_best->rows >= R &&
+                      head_best->parts > 0 && head_best->cols > 0;
+    if (all_greedy && !penalised && left) {
         // greedy rows without a penalty (the caller's word): the head's kernel left the best of every
         // share of a row's columns, so the logits need not be read again
         took(Path::ArgmaxMerged);
@@ -518,8 +520,11 @@ void Ops::sample(const Tensor& logits, const float* fparams, const int* iparams,
     // the parts' lists, was measured: 21 against 23 us for one row of 65,536 logits and top_k 50,
     // slower from 8 rows on and at top_k 128: what the kernel spends lies in the ranking and the
     // sums, not in reading the logits.)
+    // (sampled rows find their candidates among the columns of the parts whose best logit is large enough,
+    // without reading the row, where the head left such parts)
     kernel_check(celeg_sample(logits.as<float>(), rows_of(logits, "logits"), R, V, fparams, iparams, seen, seen_stride,
-                              out_tokens, last_tokens, stream), "sample");
+                              out_tokens, last_tokens, left ? head_best->best : nullptr, left ? head_best->ld : 0,
+                              left ? head_best->parts : 0, left ? head_best->cols : 0, stream), "sample");
 }
 
 void Ops::mark_seen(uint8_t* seen, size_t stride, int n_slots, int vocab, const int* token_ids, const int* token_slot, int n) {
@@ -718,17 +723,21 @@ void Ops::fused_linear(const Tensor& a, const Tensor& w, const Tensor& out, cons
         prm.taps = static_cast<int>(L);
     }
     last_best_parts = 0;
+    last_best_cols = 0;
     if (args.row_best) {
         need(epi == Epilogue::StoreF32, "fused_linear: row_best goes with the 32-bit store");
         last_best_parts = streamed ? celeg_gemm_rows_blocks(M, static_cast<int>(N), static_cast<int>(K), static_cast<int>(epi))
                           : sliced ? celeg_gemv_slices_blocks(M, static_cast<int>(N), static_cast<int>(K))
                                    : static_cast<int>((N + 15) / 16);
-        need(args.row_best_parts >= last_best_parts && args.row_best_ld >= M,
-             "fused_linear: row_best has room for " + std::to_string(args.row_best_parts) + " parts of " +
-                 std::to_string(args.row_best_ld) + " rows, the kernel leaves " + std::to_string(last_best_parts) + " of " + std::to_string(M));
+        need(args.row_best_ld >= last_best_parts && args.row_best_rows >= M,
+             "fused_linear: row_best has room for " + std::to_string(args.row_best_rows) + " rows of " +
+                 std::to_string(args.row_best_ld) + " parts, the kernel leaves " + std::to_string(M) + " of " + std::to_string(last_best_parts));
+        last_best_cols = streamed ? celeg_gemm_rows_cols(M, static_cast<int>(N), static_cast<int>(K), static_cast<int>(epi))
+                         : sliced ? celeg_gemv_slices_cols(M, static_cast<int>(N), static_cast<int>(K))
+                                  : 16;
         prm.row_best = args.row_best;
         prm.row_best_ld = args.row_best_ld;
-        prm.row_best_parts = args.row_best_parts;
+        prm.row_best_rows = args.row_best_rows;
     }
     took(sliced ? Path::FusedSliced : streamed ? Path::FusedRows : Path::FusedStaged);
     if (sliced) {

@@ -69,18 +69,19 @@ struct FusedArgs {
     Tensor out_bf16;              // residual: the bfloat16 copy of the stream
     bool packed = false;          // w is [K/32, rows, 32] (pack_weight)
     // 32-bit store of an output head: beside the logits, the best (logit, index) of every share of
-    // columns [row_best_parts, row_best_ld >= rows]; Ops::last_best_parts then says how many parts
-    // were written
+    // columns [row_best_rows, row_best_ld >= parts]; Ops::last_best_parts then says how many parts
+    // of every row were written
     unsigned long long* row_best = nullptr;
-    int row_best_ld = 0, row_best_parts = 0;
+    int row_best_ld = 0, row_best_rows = 0;
 };
 
 // What an output head left beside its logits for greedy rows: the best (logit, index) of every
-// share of a row's columns [parts, ld >= rows], for the first `rows` rows of `logits`.
+// share of a row's columns [rows, ld >= parts], for the first `rows` rows of `logits`.
 struct HeadBest {
     const void* logits = nullptr;
     const unsigned long long* best = nullptr;
     int ld = 0, parts = 0, rows = 0;
+    int cols = 0;        // columns a part stands for: part p is the best of columns p * cols .. + cols - 1
 };
 
 // What a step begins with, when the runner leaves it to the step's first kernel: the block-table
@@ -127,7 +128,7 @@ public:
     bool use_fresh_decode = true;      // decode-only steps: the attention prepares and writes the new keys and values
     bool use_head_argmax = true;       // greedy rows without a penalty: the token from what the head left beside the logits
     int rows_kernel_min_rows = 9, tiles_min_rows = 65, fused_linear_shape = 0;
-    int last_stat_blocks = 0, last_best_parts = 0;
+    int last_stat_blocks = 0, last_best_parts = 0, last_best_cols = 0;
 
     // row-wise
     void embed(const Tensor& table, const int* token_ids, const Tensor& out);
@@ -156,7 +157,7 @@ public:
     // sampling
     void sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen,
                 size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws,
-                const HeadBest* head_best = nullptr);
+                const HeadBest* head_best = nullptr, bool penalised = false);
     // the most parts a row of an output head of n columns can have (for the caller's buffer): one
     // per 16 columns, or per 4 where the columns are few (narrow tiles, or less than a tile a workgroup)
     static int head_best_parts(long long n) { return static_cast<int>(std::max((n + 15) / 16, std::min<long long>((n + 3) / 4, 4096))); }

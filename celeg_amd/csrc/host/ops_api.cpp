@@ -250,10 +250,11 @@ Json call(celeg_ops& h, const std::string& op, const Json& a) {
             best.ld = static_cast<int>(a.get_int("row_best_ld", 0));
             best.parts = static_cast<int>(a.get_int("row_best_parts", 0));
             best.rows = static_cast<int>(logits.shape[0]);
+            best.cols = static_cast<int>(a.get_int("row_best_cols", 0));
         }
         ops.sample(logits, address<float>(a, "fparams"), address<int>(a, "iparams"), address<uint8_t>(a, "seen"),
                    static_cast<size_t>(a.get_int("seen_stride", 0)), address<int>(a, "out_tokens"), address<int>(a, "last_tokens"),
-                   a.get_bool("all_greedy", false), h.ws, best.best ? &best : nullptr);
+                   a.get_bool("all_greedy", false), h.ws, best.best ? &best : nullptr, a.get_bool("penalised", false));
     } else if (op == "mark_seen") {
         const Tensor seen = must(a, "seen");
         ops.mark_seen(seen.as<uint8_t>(), static_cast<size_t>(seen.stride[0]), static_cast<int>(seen.shape[0]),
@@ -304,7 +305,7 @@ Json call(celeg_ops& h, const std::string& op, const Json& a) {
         }
         args.row_best = address<unsigned long long>(a, "row_best");
         args.row_best_ld = static_cast<int>(a.get_int("row_best_ld", 0));
-        args.row_best_parts = static_cast<int>(a.get_int("row_best_parts", 0));
+        args.row_best_rows = static_cast<int>(a.get_int("row_best_rows", 0));
         ops.fused_linear(must(a, "a"), must(a, "w"), must(a, "out"), args);
     } else if (op == "tiled_linear") {
         const Maybe stats = maybe(a, "stats"), bias = maybe(a, "bias"), stats_out = maybe(a, "stats_out"), out_bf16 = maybe(a, "out_bf16");
@@ -353,6 +354,7 @@ Json call(celeg_ops& h, const std::string& op, const Json& a) {
     }
     out.set("last_stat_blocks", ops.last_stat_blocks);
     out.set("last_best_parts", ops.last_best_parts);
+    out.set("last_best_cols", ops.last_best_cols);
     if (op == "state") out.set("paths", ops.paths_json());
     return out;
 }

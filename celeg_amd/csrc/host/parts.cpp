@@ -625,8 +625,8 @@ bool head_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& ba
     const int room = Ops::head_best_parts(weight.shape[0]);
     if (rt.ops.use_head_argmax) {
         extras.row_best = static_cast<unsigned long long*>(rt.ws.raw("head_best", static_cast<size_t>(64) * room * sizeof(unsigned long long)));
-        extras.row_best_ld = (R + 7) / 8 * 8;     // the rows of a part side by side (R <= 64)
-        extras.row_best_parts = room;
+        extras.row_best_ld = room;     // the parts of a row one after the other (R <= 64 rows)
+        extras.row_best_rows = 64;
     }
     fused::norm_linear(rt, h, norm, weight, out, Epilogue::StoreF32, extras);
     if (extras.row_best && rt.ops.last_best_parts > 0) {
@@ -634,6 +634,7 @@ bool head_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& ba
         rt.head_best.best = extras.row_best;
         rt.head_best.ld = extras.row_best_ld;
         rt.head_best.parts = rt.ops.last_best_parts;
+        rt.head_best.cols = rt.ops.last_best_cols;
         rt.head_best.rows = R;
     }
     return true;

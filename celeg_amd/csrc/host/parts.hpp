@@ -175,7 +175,7 @@ struct LinearExtras {
     const ConvOperands* conv = nullptr;
     const QkvTail* qkv = nullptr;          // steps of many rows: what follows a q/k/v product, inside its kernel
     unsigned long long* row_best = nullptr;   // an output head's 32-bit store: see FusedArgs
-    int row_best_ld = 0, row_best_parts = 0;
+    int row_best_ld = 0, row_best_rows = 0;
 };
 // whether norm_linear would take a q/k/v tail for a step of this many rows
 bool qkv_tail_ok(const Runtime& rt, int rows, long long width);

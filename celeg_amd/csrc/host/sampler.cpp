@@ -126,7 +126,7 @@ void Sampler::launch(const Tensor& logits, const std::vector<int>& slots) {
     // the kernels write the tokens straight into the turn's pinned buffer (memory of the host that
     // the device can address): no copy behind them, the event tells when they are there
     rt_.ops.sample(logits, fdev, idev, seen_.as<uint8_t>(), static_cast<size_t>(vocab_), tokens_host_[turn].as<int>(),
-                   last_tokens_.as<int>(), all_greedy, rt_.ws, penalised ? nullptr : &rt_.head_best);
+                   last_tokens_.as<int>(), all_greedy, rt_.ws, &rt_.head_best, penalised);
     CELEG_HIP(hipEventRecord(events_[turn], rt_.stream));
     pending_.emplace_back(turn, R);
 }

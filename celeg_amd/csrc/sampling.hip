@@ -254,6 +254,9 @@ __device__ __forceinline__ void top_k_candidates(
 // Five workgroup barriers instead of about forty, and two divisions per gathered logit
 // instead of per logit.
 #define SAMPLE_RANK_CAP 2048
+__device__ __forceinline__ void rank_gathered(const float* __restrict__ row, const uint8_t* __restrict__ seen, bool pen,
+                                              float penalty, float temperature, int top_k, int n, uint2* gathered,
+                                              float* cand_score, int* cand_id);
 template <int KPT>
 __device__ __forceinline__ bool top_k_ranked(
     const float* __restrict__ row, const uint8_t* __restrict__ seen, float penalty, float temperature,
@@ -335,7 +338,17 @@ __device__ __forceinline__ bool top_k_ranked(
     __syncthreads();
     const int n = static_cast<int>(sel[1]);
     if (n > SAMPLE_RANK_CAP) return false;       // the same for every thread
-    // the exact scores of the gathered logits, as the reference computes them
+    rank_gathered(row, seen, pen, penalty, temperature, top_k, n, gathered, cand_score, cand_id);
+    return true;
+}
+
+// The last steps of the ranking: the exact scores of the n gathered logits (gathered[e].y: their
+// indices), as the reference computes them, and every one's place among them; the first top_k places
+// go to cand_score / cand_id.  All threads call it; n is the same for all.
+__device__ __forceinline__ void rank_gathered(const float* __restrict__ row, const uint8_t* __restrict__ seen, bool pen,
+                                              float penalty, float temperature, int top_k, int n, uint2* gathered,
+                                              float* cand_score, int* cand_id) {
+    const int tid = threadIdx.x;
     for (int e = tid; e < n; e += SAMPLE_THREADS) {
         const int id = static_cast<int>(gathered[e].y);
         float x = row[id];
@@ -359,6 +372,98 @@ __device__ __forceinline__ bool top_k_ranked(
         if (place < top_k) { cand_score[place] = score; cand_id[place] = id; }
     }
     __syncthreads();
+}
+
+// The same candidates without reading the row: an output head left, beside the logits, the best
+// (logit, index) of every `cols` columns (best[p]: part p of this row, packed as packed_logit
+// packs them).  A penalised logit is never above the logit itself, so:
+//   1. every thread takes up to SAMPLE_PARTS_PER_THREAD parts' maxima; the c-th largest thread maximum
+//      of each wavefront, c = ceil(top_k / 16), bounds the top_k-th largest maximum from below as in
+//      top_k_ranked; the threads whose maximum reaches it (top_k different logits at least) apply the
+//      penalty to theirs, and the smallest of these penalised values, less eight units in the last
+//      place, is a bound from below for the top_k-th largest penalised logit;
+//   2. only parts whose maximum reaches that bound can hold a logit that does: their columns are read
+//      (a few hundred logits instead of the row), and what reaches the bound is gathered and ranked
+//      as in top_k_ranked.
+// false (nothing written that matters) if the parts are too many for the threads, too few to bound
+// anything, or more parts or logits reach the bound than there is room for: the caller then reads the row.
+#define SAMPLE_PARTS_PER_THREAD 4
+#define SAMPLE_PART_LIST 1024
+__device__ __forceinline__ bool top_k_from_parts(
+    const float* __restrict__ row, const uint8_t* __restrict__ seen, float penalty, float temperature, int vocab, int top_k,
+    const unsigned long long* __restrict__ best, int n_parts, int cols, uint32_t* wave_bound, uint2* gathered,
+    unsigned int* sel, unsigned int* part_list, float* cand_score, int* cand_id) {
+    const int tid = threadIdx.x;
+    const int lane = tid & (CELEG_WAVE - 1), wave = tid / CELEG_WAVE;
+    if (n_parts > SAMPLE_THREADS * SAMPLE_PARTS_PER_THREAD || cols <= 0) return false;
+    const bool pen = seen && penalty > 1.0f;
+    const float inv_penalty = 1.0f / penalty;
+    auto stand_in = [&](float x, unsigned seen_byte) { return seen_byte ? (x >= 0.0f ? x * inv_penalty : x * penalty) : x; };
+    uint32_t part_key[SAMPLE_PARTS_PER_THREAD];
+    unsigned long long my_best = 0ull;
+    {
+        unsigned long long v[SAMPLE_PARTS_PER_THREAD];
+#pragma unroll
+        for (int j = 0; j < SAMPLE_PARTS_PER_THREAD; ++j)
+            v[j] = best[min(tid + SAMPLE_THREADS * j, n_parts - 1)];     // clamped, masked below
+#pragma unroll
+        for (int j = 0; j < SAMPLE_PARTS_PER_THREAD; ++j) {
+            const bool valid = tid + SAMPLE_THREADS * j < n_parts;
+            part_key[j] = valid ? static_cast<uint32_t>(v[j] >> 32) : 0u;
+            my_best = valid ? max(my_best, v[j]) : my_best;
+        }
+    }
+    const uint32_t my_max = static_cast<uint32_t>(my_best >> 32);
+    const int c = (top_k + SAMPLE_THREADS / CELEG_WAVE - 1) / (SAMPLE_THREADS / CELEG_WAVE);
+    uint32_t left = my_max, cth = 0u;
+    for (int round = 0; round < c; ++round) {
+        uint32_t m = left;
+#pragma unroll
+        for (int off = CELEG_WAVE / 2; off > 0; off >>= 1)
+            m = max(m, static_cast<uint32_t>(__shfl_xor(static_cast<int>(m), off, CELEG_WAVE)));
+        cth = m;
+        const unsigned long long holders = __ballot(left == m);
+        if (lane == __ffsll(static_cast<long long>(holders)) - 1) left = 0u;
+    }
+    if (lane == 0) wave_bound[wave] = cth;
+    if (tid == 0) { sel[0] = 0u; sel[1] = 0u; sel[2] = 0xffffffffu; }
+    __syncthreads();
+    uint32_t lower_max = wave_bound[0];
+#pragma unroll
+    for (int w = 1; w < SAMPLE_THREADS / CELEG_WAVE; ++w) lower_max = min(lower_max, wave_bound[w]);
+    if (lower_max == 0u) return false;           // (some wavefront has fewer than c parts: nothing is bounded)
+    if (my_max >= lower_max) {
+        // this thread's best logit is one of top_k different logits at least: its penalised value
+        const int index = packed_logit_index(my_best);
+        const float x = stand_in(key_score(my_max), pen ? seen[index] : 0u);
+        atomicMin(&sel[2], order_key(x));
+    }
+    __syncthreads();
+    const uint32_t lowest = sel[2];
+    const uint32_t lower = lowest > 8u ? lowest - 8u : 0u;
+#pragma unroll
+    for (int j = 0; j < SAMPLE_PARTS_PER_THREAD; ++j)
+        if (tid + SAMPLE_THREADS * j < n_parts && part_key[j] >= lower) {
+            const unsigned int p = atomicAdd(&sel[0], 1u);
+            if (p < SAMPLE_PART_LIST) part_list[p] = static_cast<unsigned>(tid + SAMPLE_THREADS * j);
+        }
+    __syncthreads();
+    const int n_listed = static_cast<int>(sel[0]);
+    if (n_listed > SAMPLE_PART_LIST) return false;
+    for (int e = tid; e < n_listed * cols; e += SAMPLE_THREADS) {
+        const int i = static_cast<int>(part_list[e / cols]) * cols + e % cols;
+        if (i < vocab) {
+            const float x = stand_in(row[i], pen ? seen[i] : 0u);
+            if (order_key(x) >= lower) {
+                const unsigned int p = atomicAdd(&sel[1], 1u);
+                if (p < SAMPLE_RANK_CAP) gathered[p].y = static_cast<unsigned>(i);
+            }
+        }
+    }
+    __syncthreads();
+    const int n = static_cast<int>(sel[1]);
+    if (n > SAMPLE_RANK_CAP || n < top_k) return false;
+    rank_gathered(row, seen, pen, penalty, temperature, top_k, n, gathered, cand_score, cand_id);
     return true;
 }
 
@@ -439,7 +544,9 @@ __device__ __forceinline__ int choose_among(float* cand_score, int* cand_id, int
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int ld, int vocab, const float* __restrict__ fparams,
     const int* __restrict__ iparams, uint8_t* __restrict__ seen_all, size_t seen_stride,
-    int* __restrict__ out_tokens, int* __restrict__ last_tokens) {
+    int* __restrict__ out_tokens, int* __restrict__ last_tokens, const unsigned long long* __restrict__ best, int best_ld,
+    int best_parts, int best_cols) {
+    __shared__ unsigned int part_list[SAMPLE_PART_LIST];
     __shared__ float s_val[SAMPLE_THREADS / CELEG_WAVE];
     __shared__ int s_idx[SAMPLE_THREADS / CELEG_WAVE];
     __shared__ __attribute__((aligned(16))) unsigned int hist[256 * SAMPLE_HIST_COPIES];   // or SAMPLE_RANK_CAP gathered (key, id)
@@ -508,7 +615,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     static_assert(sizeof(hist) >= SAMPLE_RANK_CAP * sizeof(uint2), "the gathered scores share the histograms' room");
     uint2* gathered = reinterpret_cast<uint2*>(hist);
     bool sorted = false;
-    if (vocab <= SAMPLE_THREADS * 64)
+    if (best) {
+        // what the output head left beside the logits: the candidates without reading the row
+        sorted = top_k_from_parts(row, seen, penalty, temperature, vocab, top_k, best + static_cast<size_t>(r) * best_ld, best_parts, best_cols, maxes,
+                                  gathered, sel, part_list, cand_score, cand_id);
+        __syncthreads();        // (before what follows reuses the counters)
+    }
+    if (sorted) {
+    } else if (vocab <= SAMPLE_THREADS * 64)
         sorted = top_k_ranked<64>(row, seen, penalty, temperature, vocab, top_k, maxes, gathered, sel, cand_score, cand_id);
     else if (vocab <= SAMPLE_THREADS * 128)
         sorted = top_k_ranked<128>(row, seen, penalty, temperature, vocab, top_k, maxes, gathered, sel, cand_score, cand_id);
@@ -609,7 +723,7 @@ extern "C" int celeg_argmax_rows(const float* logits, int ld, int rows, int voca
 }
 
 // The greedy tokens of rows whose output head left the best (logit, index) of every workgroup's
-// columns beside the logits (best [parts, ld >= rows], packed as packed_logit packs them): the
+// columns beside the logits (best [rows, ld >= parts], packed as packed_logit packs them): the
 // largest of a row's parts is its token.  No repetition penalty: the head
 // knows nothing of what a request has seen.  One workgroup a row; the token also goes to
 // last_tokens[slot] as with the other kernels.
@@ -620,13 +734,13 @@ __global__ __launch_bounds__(MERGE_THREADS) void argmax_merge_kernel(
     __shared__ unsigned long long s_best[MERGE_THREADS / CELEG_WAVE];
     const int r = blockIdx.x, tid = threadIdx.x;
     const int lane = tid & (CELEG_WAVE - 1), wave = tid / CELEG_WAVE;
-    const unsigned long long* row = best + r;
+    const unsigned long long* row = best + static_cast<size_t>(r) * ld;
     unsigned long long mine = 0ull;
     for (int j0 = 0; j0 < parts; j0 += 16 * MERGE_THREADS) {        // sixteen loads of a thread under way at a time:
         unsigned long long v[16];                                   // one trip to memory for 65,536 columns in tiles of 16
 #pragma unroll
         for (int j = 0; j < 16; ++j)     // (a part twice changes nothing)
-            v[j] = row[static_cast<size_t>(min(j0 + tid + MERGE_THREADS * j, parts - 1)) * ld];
+            v[j] = row[min(j0 + tid + MERGE_THREADS * j, parts - 1)];
 #pragma unroll
         for (int j = 0; j < 16; ++j) mine = max(mine, v[j]);
     }
@@ -646,20 +760,27 @@ __global__ __launch_bounds__(MERGE_THREADS) void argmax_merge_kernel(
 extern "C" int celeg_argmax_merge(const unsigned long long* best, int ld, int parts, int rows, const int* iparams,
                                   int* out_tokens, int* last_tokens, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (parts <= 0 || ld < rows) return static_cast<int>(hipErrorInvalidValue);
+    if (parts <= 0 || ld < parts) return static_cast<int>(hipErrorInvalidValue);
     hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(MERGE_THREADS), 0, stream, best, ld, parts, iparams,
                        out_tokens, last_tokens);
     return CELEG_LAUNCH_RESULT();
 }
 
+// best (or null): what an output head left beside these logits, [rows, best_ld >= best_parts], part p of a row
+// the best (logit, index) of its columns p * best_cols .. + best_cols - 1 (packed_logit).
 extern "C" int celeg_sample(const float* logits, int ld, int rows, int vocab,
                             const float* fparams, const int* iparams, uint8_t* seen,
                             size_t seen_stride, int* out_tokens, int* last_tokens,
+                            const unsigned long long* best, int best_ld, int best_parts, int best_cols,
                             hipStream_t stream) {
     if (rows <= 0) return 0;
     if (vocab <= 0) return static_cast<int>(hipErrorInvalidValue);
+    if (best && (best_ld < best_parts || best_parts <= 0 || best_cols <= 0 ||
+                 static_cast<long long>(best_parts) * best_cols < vocab))
+        return static_cast<int>(hipErrorInvalidValue);
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld,
-                       vocab, fparams, iparams, seen, seen_stride, out_tokens, last_tokens);
+                       vocab, fparams, iparams, seen, seen_stride, out_tokens, last_tokens, best, best_ld, best_parts,
+                       best_cols);
     return CELEG_LAUNCH_RESULT();
 }
 

@@ -163,6 +163,7 @@ class HipOps:
         out = json.loads(answer.decode())
         self.last_stat_blocks = out.get("last_stat_blocks", self.last_stat_blocks)
         self.last_best_parts = out.get("last_best_parts", 0)
+        self.last_best_cols = out.get("last_best_cols", 0)
         return out
 
     def paths(self) -> Dict[str, int]:
@@ -262,12 +263,13 @@ class HipOps:
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, fparams, iparams, seen, out_tokens, last_tokens=None, all_greedy=False, row_best=None,
-               row_best_parts=0):
+               row_best_parts=0, row_best_cols=0, penalised=False):
         """One token per row.  ``all_greedy``: the caller knows that every row takes its
         (penalised) largest logit; the rows are then cut into parts over many workgroups.
-        ``row_best`` [>= row_best_parts, >= rows] (int64): what the head's product left beside these
-        logits (``fused_linear(..., row_best=...)``); greedy rows without a penalty then take their
-        token from it."""
+        ``row_best`` [>= rows, >= row_best_parts] (int64): what the head's product left beside these
+        logits (``fused_linear(..., row_best=...)``, ``row_best_cols`` columns a part: ``last_best_cols``); greedy
+        rows without a penalty (``penalised`` false) then take their token from it, and sampled rows look for
+        their candidates in the columns of the parts it names instead of reading the row."""
         R, V = logits.shape
         if out_tokens.numel() != R or fparams.numel() < 4 * R or iparams.numel() < 3 * R:
             raise KernelError("sample: parameter arrays do not fit the rows")
@@ -278,7 +280,8 @@ class HipOps:
                    seen_stride=int(seen.stride(0)) if seen is not None else 0, out_tokens=_address(out_tokens, "out_tokens"),
                    last_tokens=_address(last_tokens, "last_tokens"), all_greedy=bool(all_greedy),
                    row_best=_address(row_best, "row_best", torch.int64),
-                   row_best_ld=int(row_best.stride(0)) if row_best is not None else 0, row_best_parts=int(row_best_parts))
+                   row_best_ld=int(row_best.stride(0)) if row_best is not None else 0, row_best_parts=int(row_best_parts),
+                   row_best_cols=int(row_best_cols), penalised=bool(penalised))
 
     def mark_seen(self, seen, token_ids, token_slot, n):
         if token_ids.numel() < n or token_slot.numel() < n:
@@ -343,7 +346,7 @@ class HipOps:
                      stat_blocks=0, rows=None, bias=None, stats_out=None, conv=None, n_rows=None,
                      out_bf16=None, row_best=None):
         """out = epilogue(prologue(a) w^T) for up to 64 rows, bfloat16 weights (``Ops::fused_linear``).
-        ``row_best`` (int64 [parts, >= rows], with "store_f32"): receives the best (logit, index) of every
+        ``row_best`` (int64 [>= rows, >= parts], with "store_f32"): receives the best (logit, index) of every
         share of a row's columns; ``last_best_parts`` says how many parts were written.
 
         ``a``: bfloat16 rows [M, K], or, with ``norm_weight``, the 32-bit residual stream,
@@ -369,7 +372,7 @@ class HipOps:
                    out_bf16=_tensor(out_bf16, "out_bf16"), packed=w.dim() == 3,
                    row_best=_address(row_best, "row_best", torch.int64),
                    row_best_ld=int(row_best.stride(0)) if row_best is not None else 0,
-                   row_best_parts=int(row_best.shape[0]) if row_best is not None else 0)
+                   row_best_rows=int(row_best.shape[0]) if row_best is not None else 0)
         return out
 
     # ------------------------------------------------------------------ fused products of many rows

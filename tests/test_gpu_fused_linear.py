@@ -120,7 +120,7 @@ def test_the_32bit_store_leaves_the_best_of_every_share_of_a_row(ops, M, N, K, f
         w[lo] = boost
         w[hi] = boost
     room = max((N + 15) // 16, min((N + 3) // 4, 4096))
-    best = torch.full((room, M + 3), -1, dtype=torch.int64, device=DEV)
+    best = torch.full((M + 3, room), -1, dtype=torch.int64, device=DEV)
     out = torch.empty(M, N, device=DEV)
     if form == "norm":
         ops.fused_linear(h, w, out, epilogue="store_f32", norm_weight=nw, eps=1e-5, row_best=best)
@@ -130,10 +130,10 @@ def test_the_32bit_store_leaves_the_best_of_every_share_of_a_row(ops, M, N, K, f
         ops.stream_prepare(h, xb, stats)
         ops.fused_linear(xb, ops.fold_weight(w, nw), out, epilogue="store_f32", eps=1e-5, stats=stats, stat_blocks=1,
                          row_best=best)
-    parts = ops.last_best_parts
-    assert 0 < parts <= room
-    assert bool((best[parts:] == -1).all()) and bool((best[:, M:] == -1).all())
-    top = best[:parts, :M].cpu().numpy().view("uint64").max(axis=0)
+    parts, part_cols = ops.last_best_parts, ops.last_best_cols
+    assert 0 < parts <= room and parts * part_cols >= N > (parts - 1) * part_cols
+    assert bool((best[M:] == -1).all()) and bool((best[:, parts:] == -1).all())
+    top = best[:M, :parts].cpu().numpy().view("uint64").max(axis=1)
     index = (0xffffffff - (top & 0xffffffff)).astype("int64")
     logits = out.cpu()
     want = [int((logits[m] == logits[m].max()).nonzero()[0]) for m in range(M)]
@@ -143,7 +143,8 @@ def test_the_32bit_store_leaves_the_best_of_every_share_of_a_row(ops, M, N, K, f
     f = torch.tensor([[0.0, 1.0, 1.0, 0.0]] * M, dtype=torch.float32, device=DEV).reshape(-1)
     i = torch.tensor([[1, -1, m + 1 if m % 2 else -1] for m in range(M)], dtype=torch.int32, device=DEV).reshape(-1)
     before = ops.paths().get("argmax_merged", 0)
-    ops.sample(out, f, i, None, tokens, last_tokens=last, all_greedy=True, row_best=best, row_best_parts=parts)
+    ops.sample(out, f, i, None, tokens, last_tokens=last, all_greedy=True, row_best=best, row_best_parts=parts,
+               row_best_cols=part_cols)
     assert ops.paths()["argmax_merged"] == before + 1
     assert tokens.tolist() == want
     assert last.tolist() == [-1] + [want[m] if m % 2 else -1 for m in range(M)]

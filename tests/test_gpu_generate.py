@@ -203,8 +203,25 @@ def sample_with_draw(logits, temperature, top_k, top_p, penalty, seen, u):
         plain.random_unit = generator
 
 
-def run_sample(ops, logits, rows, all_greedy=False):
-    """rows: list of (temperature, top_k, top_p, penalty, u, seen list or None)"""
+def parts_of(logits, cols):
+    """What an output head leaves beside its logits: the best (logit, index) of every ``cols`` columns,
+    [rows, parts], packed as the kernels pack it (the logit's ordered bits above the inverted index)."""
+    import numpy as np
+    x = (logits.float() + 0.0).numpy()
+    bits = x.view(np.uint32).astype(np.uint64)
+    key = np.where(bits & 0x80000000, ~bits & 0xffffffff, bits | 0x80000000)
+    R, V = x.shape
+    packed = (key << np.uint64(32)) | (np.uint64(0xffffffff) - np.arange(V, dtype=np.uint64))[None, :]
+    parts = (V + cols - 1) // cols
+    padded = np.zeros((R, parts * cols), dtype=np.uint64)
+    padded[:, :V] = packed
+    best = padded.reshape(R, parts, cols).max(axis=2).copy()
+    return torch.from_numpy(best.view(np.int64)).to(DEV)
+
+
+def run_sample(ops, logits, rows, all_greedy=False, part_cols=0):
+    """rows: list of (temperature, top_k, top_p, penalty, u, seen list or None); part_cols: the kernel also
+    gets what an output head would have left beside these logits, a part every part_cols columns"""
     R, V = logits.shape
     f = torch.tensor([[t, p, pen, u] for t, k, p, pen, u, s in rows], dtype=torch.float32)
     seen = torch.zeros(R, V, dtype=torch.uint8)
@@ -214,8 +231,10 @@ def run_sample(ops, logits, rows, all_greedy=False):
             seen[r, torch.tensor(s, dtype=torch.long)] = 1
         i.append([k, r if s is not None else -1, -1])
     out = torch.empty(R, dtype=torch.int32, device=DEV)
+    best = parts_of(logits, part_cols) if part_cols else None
     ops.sample(logits.to(DEV), f.reshape(-1).to(DEV), torch.tensor(i, dtype=torch.int32).reshape(-1).to(DEV),
-               seen.to(DEV), out, all_greedy=all_greedy)
+               seen.to(DEV), out, all_greedy=all_greedy, row_best=best, row_best_parts=best.shape[1] if part_cols else 0,
+               row_best_cols=part_cols, penalised=any(s is not None and pen > 1 for t, k, p, pen, u, s in rows))
     return out.tolist()
 
 
@@ -242,12 +261,45 @@ def test_sampling_kernel_equals_plain_sampler(ops, vocab):
             (0.5, 17, 0.5, 1.0, 0.999, None), (0.0, 50, 1.0, 1.7, 0.0, seen[3]),
             (2.0, 128, 0.95, 1.1, 0.05, seen[4]), (1.3, 2, 1.0, 1.0, 0.5, None)]
     got = run_sample(ops, logits, rows)
+    want = []
     for r, (t, k, p, pen, u, s) in enumerate(rows):
         flags = [False] * vocab
         for tok in (s or []):
             flags[tok] = True
-        want = sample_with_draw(logits[r].tolist(), t, k, p, pen, flags, u)
-        assert got[r] == want, f"row {r}"
+        want.append(sample_with_draw(logits[r].tolist(), t, k, p, pen, flags, u))
+        assert got[r] == want[r], f"row {r}"
+    # the same from what an output head leaves beside the logits (the best of every 16, 64 or 7 columns):
+    # the candidates are then looked for in the parts whose best logit is large enough, not in the whole row
+    for part_cols in (16, 64, 7):
+        assert run_sample(ops, logits, rows, part_cols=part_cols) == want, part_cols
+
+
+@pytest.mark.parametrize("vocab", [4096, 65536])
+def test_sampling_from_the_heads_parts_when_penalties_reorder_the_top(ops, vocab):
+    """The parts hold the best logit of their columns before any penalty.  Here the 300 largest logits of a
+    row have all been seen and a penalty of 3 throws them far down, so the tokens that win come from parts
+    whose best logit was nowhere near the top; in another row all logits are equal (nothing bounds anything:
+    the kernel reads the row after all); in a third the maximum of every part is the same value."""
+    g = torch.Generator().manual_seed(vocab + 7)
+    R = 4
+    logits = torch.randn(R, vocab, generator=g) * 2
+    top = torch.topk(logits[0], 300).indices.tolist()
+    logits[1] = 0.5
+    logits[2, ::16] = 9.0
+    logits[3] = -logits[3].abs() - 1.0              # all negative: a penalty makes seen ones smaller still
+    seen3 = torch.topk(logits[3], 100).indices.tolist()
+    rows = [(0.7, 50, 0.95, 3.0, 0.42, top), (1.0, 50, 1.0, 1.0, 0.77, None), (0.9, 128, 0.9, 1.2, 0.13, list(range(0, 4096, 32))),
+            (0.5, 20, 1.0, 1.5, 0.6, seen3)]
+    want = []
+    for r, (t, k, p, pen, u, s) in enumerate(rows):
+        flags = [False] * vocab
+        for tok in (s or []):
+            flags[tok] = True
+        want.append(sample_with_draw(logits[r].tolist(), t, k, p, pen, flags, u))
+    assert want[0] not in top[:50]
+    assert run_sample(ops, logits, rows) == want
+    for part_cols in (16, 64):
+        assert run_sample(ops, logits, rows, part_cols=part_cols) == want, part_cols
 
 
 @pytest.mark.parametrize("vocab", [5, 331, 4100, 65536, 70001])
