@@ -348,9 +348,13 @@ static RowsShape rows_shape(int M, int N, int K, int streams) {
     const bool forced = g_force_ct > 0 || g_force_mt > 0 || g_force_cols > 0;
     if (!forced) {
         const auto row_groups = [&](int mt) { return (M + 16 * mt - 1) / (16 * mt); };
-        // (a) compute units without a workgroup
+        // (a) compute units without a workgroup: half the columns a workgroup, and half again, while
+        // that still leaves no compute unit with a second one (36 to 48 rows by 1,024 columns are 3
+        // groups of rows and 192 workgroups of 16 columns: 8 columns would be 384, a round and a half,
+        // w2 8.4 to 9.2 us against 7.2 to 7.7; shares that are no power of two, 13 columns for 237
+        // workgroups, were slower too: 8.0 to 8.4)
         if (s.ct == 1)
-            while (s.cols > 4 && row_groups(s.mt) * ((N + s.cols - 1) / s.cols) < ROWS_COMPUTE_UNITS) s.cols >>= 1;
+            while (s.cols > 4 && row_groups(s.mt) * ((N + s.cols / 2 - 1) / (s.cols / 2)) <= ROWS_COMPUTE_UNITS) s.cols >>= 1;
         // (b) a last round of workgroups that is less than three quarters full
         const long long groups = static_cast<long long>(row_groups(s.mt)) * ((N + s.cols - 1) / s.cols);
         const long long rounds = (groups + ROWS_COMPUTE_UNITS - 1) / ROWS_COMPUTE_UNITS;
