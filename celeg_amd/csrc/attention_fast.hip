@@ -1020,9 +1020,10 @@ static int attention_decode(
     if (whole < 0) whole = kv_heads * chunks * n_rows >= 192 ? 1 : 0;
     if (whole) {
         // 16 wavefronts a workgroup (what the registers of a compute unit hold at this head size),
-        // 8 once there are two workgroups and more for every compute unit: their ends overlap
-        // (64 requests x 8 heads: 4 to 6 % faster at contexts of 1,000 to 4,000; equal at 32 requests)
-        if (head_dim == 64 && kv_heads * chunks * n_rows >= 512)
+        // 8 once there are more workgroups than compute units: two of them then share a compute unit
+        // where workgroups of 16 would take a second round (64 requests x 8 heads: 4 to 6 % faster at
+        // contexts of 1,000 to 4,000; 36 to 60 requests: 1.2 to 2 % of a decode step; equal at 32 requests)
+        if (head_dim == 64 && kv_heads * chunks * n_rows > 256)
             return launch_decode_heads<64, 8>(q, ldq, k_pool, v_pool, table, table_stride, token_slot, positions,
                                               out, ldo, n_rows, kv_heads, group, page_tokens, page_shift,
                                               n_layers, layer, scale, window, fresh, stream);
