@@ -431,6 +431,11 @@ extern "C" int celeg_gemm_rows_blocks(int M, int N, int K, int epi) {
     const RowsShape s = rows_shape(M, N, K, streams_of(epi));
     return (N + s.cols - 1) / s.cols;
 }
+// All workgroups of the launch: those shares of columns times the groups of rows.
+extern "C" int celeg_gemm_rows_workgroups(int M, int N, int K, int epi) {
+    const RowsShape s = rows_shape(M, N, K, streams_of(epi));
+    return ((N + s.cols - 1) / s.cols) * ((M + s.mt * 16 - 1) / (s.mt * 16));
+}
 
 // M <= 64 (made for 17 and more; fewer rows work too), K % 32 == 0, bfloat16 a and
 // w (in the layouts that the strides describe).  The fields of GemvParams that are read are

@@ -89,6 +89,7 @@ int celeg_embed_stream_prologue(const void* table, int* ids, float* out, void* x
                                 const int* updates, int capacity, const int* token_slot, const int* last_tokens,
                                 hipStream_t stream);
 int celeg_gemm_rows_blocks(int M, int N, int K, int epi);
+int celeg_gemm_rows_workgroups(int M, int N, int K, int epi);
 int celeg_gemm_rows_cols(int M, int N, int K, int epi);
 int celeg_gemm_rows(const GemvParams* params, int epi, hipStream_t stream);
 int celeg_gemv_fused(const GemvParams* params, int amode, int epi, int shape, hipStream_t stream);

@@ -78,3 +78,29 @@ def test_table_updates_travel_in_the_same_buffer_and_arrays_start_at_multiples_o
         build([StepEntry(1, 0, [4, 5, 6], [3])])
     with pytest.raises(HostError, match="padded"):
         build(entries, pad_to=4)
+
+
+def test_the_products_for_up_to_64_rows_share_out_their_columns():
+    """The products for 9 to 64 rows and for up to 16 say how many columns a workgroup owns and how
+    many workgroups that makes: together the shares cover every column once; a share never exceeds
+    the 64 columns a workgroup's tiles can hold; and where a share is smaller than a tile of 16
+    columns (few columns: the share is halved so that more compute units get a workgroup), the
+    workgroups of all row groups still fit the chip's 256 compute units at once."""
+    import ctypes
+    from celeg_amd.csrc import build as library
+    lib = ctypes.CDLL(library.ensure_built())
+    epilogues = {"store": 0, "store_f32": 1, "residual": 2, "swiglu": 3, "conv": 4}
+    for name, epi in epilogues.items():
+        for n in (24, 333, 1024, 2048, 3072, 4608, 7168, 65536):
+            for k in (64, 1024, 4608):
+                for m in range(1, 65):
+                    cols, blocks = lib.celeg_gemm_rows_cols(m, n, k, epi), lib.celeg_gemm_rows_blocks(m, n, k, epi)
+                    assert 1 <= cols <= 64 and (blocks - 1) * cols < n <= blocks * cols, (name, m, n, k, cols, blocks)
+                    groups = lib.celeg_gemm_rows_workgroups(m, n, k, epi)
+                    assert groups % blocks == 0 and 1 <= groups // blocks <= (m + 15) // 16
+                    if cols < 16:
+                        assert groups <= 256, (name, m, n, k, cols, blocks, groups)
+                if name != "conv" or k % 8 == 0:
+                    for m in range(1, 17):
+                        cols, blocks = lib.celeg_gemv_slices_cols(m, n, k), lib.celeg_gemv_slices_blocks(m, n, k)
+                        assert cols >= 1 and (blocks - 1) * cols < n <= blocks * cols, (m, n, k, cols, blocks)
