@@ -187,7 +187,7 @@ __device__ __forceinline__ void short_conv_state_vec(
 // request's rows, the only ones that read the old state, are all computed by the block that
 // holds the request's first row (also those that lie in the next block, which skips them), and
 // the same thread then writes the new state for its channels.
-#define CONV_BLOCK_TOKENS 2     // (2,048 tokens of 1,024 channels, with the state update: 9.2 us with 2, 10.0 with 4 a thread; more were slower)
+#define CONV_BLOCK_TOKENS 2     // (2,048 tokens of 1,024 channels, with the state update: 8.8 us with 2, 9.4 with 1 and 10.1 with 4 a thread; more were slower)
 template <typename T, int TAPS, int TT>
 __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
     const T* __restrict__ bcx, int ld_bcx, const float* __restrict__ w,
@@ -199,7 +199,13 @@ __global__ __launch_bounds__(256) void short_conv_fwd_block_kernel(
     typedef typename ConvVec<T>::raw raw;
     const int ch = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
     if (ch >= width) return;
-    const int t0 = blockIdx.x * TT;
+    // Workgroups go to the chip's 8 dies in turn, and each die has an L2 of its own: die d takes a
+    // run of tokens, so that the rows two neighbouring workgroups both read (the taps before a
+    // workgroup's first token) come from memory once, not once for each of two dies.  (The grid is
+    // 8 runs of gridDim.x / 8 workgroups; those beyond the last token have nothing to do.)
+    const int per_die = gridDim.x >> 3;
+    const int t0 = ((blockIdx.x & 7) * per_die + (blockIdx.x >> 3)) * TT;
+    if (t0 >= n_tokens) return;
     const int n = min(TT, n_tokens - t0);
     // (asked for ahead of the rows; what depends on it is asked for while the rows are on their way)
     const int s = token_seq[t0], s_end = token_seq[min(t0 + TT - 1, n_tokens - 1)];
@@ -305,7 +311,7 @@ extern "C" int celeg_short_conv(const void* bcx, int ld_bcx, int dtype, const fl
         dim3 vblock(threads), vgrid(n_tokens, (width / vec + threads - 1) / threads);
         if (taps >= 2 && taps <= 4) {      // (n_tokens >= 16 here)
             const int tt = g_force_block_tokens == 4 ? 4 : CONV_BLOCK_TOKENS;
-            dim3 bgrid((n_tokens + tt - 1) / tt, vgrid.y);
+            dim3 bgrid(((n_tokens + tt - 1) / tt + 7) / 8 * 8, vgrid.y);      // (8 runs of tokens, one a die)
 #define CELEG_CONV_BLOCK(T_, TAPS_)                                                                \
     if (tt == 4) CELEG_CONV_BLOCK_TT(T_, TAPS_, 4); else CELEG_CONV_BLOCK_TT(T_, TAPS_, CONV_BLOCK_TOKENS)
 #define CELEG_CONV_BLOCK_TT(T_, TAPS_, TT_)                                                        \
