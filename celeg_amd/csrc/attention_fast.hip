@@ -696,22 +696,31 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     const int* __restrict__ pages = table + static_cast<size_t>(token_slot[t]) * table_stride;
     const int page_mask = page_tokens - 1;
 
+    // The query heads as the product left them: norm and rotation here.  A workgroup of one
+    // wavefront (one round of keys) asks for what that needs now, does the arithmetic once its
+    // round's keys have been asked for, and asks for the new key and value ahead of the round
+    // too (LAZY).  In a workgroup of many wavefronts the first one (which starts first) prepares q
+    // for all and adds the new token, and takes the last turn at the rounds: the others ask for the
+    // keys and values of their first round at once, meet it at a barrier and take q from LDS, so
+    // that q's preparation and the keys' way from memory overlap (a decode step of one request
+    // 0.385 -> 0.374 ms, of four 0.417 -> 0.406, of 64 0.849 -> 0.843).  Parts of 16 wavefronts were
+    // 0.35 us a launch slower that way (8 requests): there every wavefront prepares q for itself.
+    constexpr bool LAZY = WAVES == 1;
+    constexpr bool SHARED_Q = FRESH && !LAZY && !(SPLIT && WAVES == 16);
+    const bool prepares_q = !SHARED_Q || wave == 0;
+    const int turn = SHARED_Q ? (wave + WAVES - 1) % WAVES : wave;     // which of the rounds are the wavefront's
+    bf16x8_t* const q_share = reinterpret_cast<bf16x8_t*>(smem_heads + static_cast<size_t>(WAVES) * gp * (HD + 2));   // [KS][64]
     bf16x8_t qf[KS];
-    {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[s] = bf16x8_t{};
+    if (prepares_q) {
         const bf16* qrow = q + static_cast<size_t>(t) * ldq + static_cast<size_t>(h0 + min(c, gp - 1)) * HD + qd * 8;
 #pragma unroll
         for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const bf16x8_t*>(qrow + s * 32);
     }
-    // The query heads as the product left them: norm and rotation here.  A workgroup of one
-    // wavefront (one round of keys) asks for what that needs now, does the arithmetic once its
-    // round's keys have been asked for, and asks for the new key and value ahead of the round
-    // too (LAZY).  Wavefronts with many rounds have no registers to hold all that meanwhile:
-    // they prepare q at once, each of them the same, which a compute unit that runs many such
-    // workgroups in turn pays every time (the host sends it launches of few workgroups only).
-    constexpr bool LAZY = WAVES == 1;
     const float* const fresh_cs = FRESH && fresh.cos_sin ? fresh.cos_sin + static_cast<size_t>(pos) * HD : nullptr;
     DecodeHeadOperands<KS> q_operands;
-    if (FRESH) decode_head_operands<KS>(q_operands, fresh.q_weight, fresh_cs, qd);
+    if (FRESH && prepares_q) decode_head_operands<KS>(q_operands, fresh.q_weight, fresh_cs, qd);
     bool q_ready = !FRESH;
     auto prepare_q = [&]() {
         float x[KS][8];
@@ -726,7 +735,6 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             for (int e = 0; e < 8; ++e) qf[s][e] = static_cast<__bf16>(x[s][e]);
         q_ready = true;
     };
-    if (FRESH && !LAZY) prepare_q();
     // (with a fresh token the rounds end at the position before it)
     const int last_key = FRESH ? pos - 1 : pos;
     float m_run = -INFINITY, l_run = 0.f;
@@ -764,7 +772,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
     // The new token as one more key: before the rounds where the wavefront has many (what it
     // needs from memory arrives with q), after its one round otherwise.
     auto add_fresh = [&]() {
-        if (!q_ready) prepare_q();            // (a part that holds no other key)
+        if (!SHARED_Q && !q_ready) prepare_q();    // (a part that holds no other key; where one wavefront prepares q for all it is ready by now)
         if (!LAZY) {
             const bf16* krow = fresh.k + static_cast<size_t>(t) * fresh.ldk + static_cast<size_t>(kvh) * HD + qd * 8;
 #pragma unroll
@@ -818,14 +826,15 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             }
         }
     };
-    // One round of 64 keys; after_loads runs once the round's keys and values have been asked for.
-    auto one_round = [&](const int r, auto&& after_loads) {
+    // One round of 64 keys in two steps: its keys and values asked for (false: the round holds no
+    // key: a window of one key with a fresh token), and the arithmetic.
+    bf16x8_t kf[4][KS], vf[DT][2];
+    auto round_loads = [&](const int r) {
         const int kb = r * DEC_KEYS;
         const int k_lo = max(lo, kb), k_hi = min(last_key, kb + DEC_KEYS - 1);
-        if (k_lo > k_hi) return;              // (a window of one key with a fresh token: no round holds a key)
+        if (k_lo > k_hi) return false;
         const int first_page = kb >> page_shift, last_page = k_hi >> page_shift;
         const int my_page = pages[min(first_page + lane, last_page)];
-        bf16x8_t kf[4][KS], vf[DT][2];
 #pragma unroll
         for (int T = 0; T < 4; ++T) {
             const int keyc = min(max(kb + 32 * (T >> 1) + 8 * (c >> 2) + 4 * (T & 1) + (c & 3), k_lo), k_hi);
@@ -846,7 +855,11 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
             for (int dt = 0; dt < DT; ++dt)
                 vf[dt][j] = *reinterpret_cast<const bf16x8_t*>(vbase + static_cast<size_t>(16 * dt + c) * page_tokens);
         }
-        after_loads();
+        return true;
+    };
+    auto round_arithmetic = [&](const int r) {
+        const int kb = r * DEC_KEYS;
+        const int k_lo = max(lo, kb), k_hi = min(last_key, kb + DEC_KEYS - 1);
         float sc[4][4];
         float mx = -INFINITY;
 #pragma unroll
@@ -894,10 +907,38 @@ __global__ __launch_bounds__(WAVES * 64) void attention_decode_heads_kernel(
                 o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt][j], pb, o[dt], 0, 0, 0);
         }
     };
-    if (adds_fresh && !LAZY) add_fresh();
-    if constexpr (SPLIT && WAVES == 1) {       // a part of one round (more, if the caller gave fewer parts than rounds)
+    // after_loads runs once the round's keys and values have been asked for
+    auto one_round = [&](const int r, auto&& after_loads) {
+        if (!round_loads(r)) return;
+        after_loads();
+        round_arithmetic(r);
+    };
+    if constexpr (SHARED_Q) {
+        int r = r_begin + turn;
+        bool asked = false;
+        if (!prepares_q && r <= r_end) asked = round_loads(r);       // on their way while q is prepared
+        if (prepares_q) {
+            prepare_q();
+#pragma unroll
+            for (int s = 0; s < KS; ++s) q_share[s * 64 + lane] = qf[s];
+        }
+        __syncthreads();
+        if (!prepares_q) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) qf[s] = q_share[s * 64 + lane];
+            q_ready = true;
+            if (r <= r_end) {
+                if (asked) round_arithmetic(r);
+                r += WAVES;
+            }
+        }
+        if (adds_fresh) add_fresh();
+        for (; r <= r_end; r += WAVES) one_round(r, []() {});
+    } else if constexpr (SPLIT && WAVES == 1) {       // a part of one round (more, if the caller gave fewer parts than rounds)
         for (int r = r_begin; r <= r_end; ++r) one_round(r, [&]() { if (FRESH && !q_ready) prepare_q(); });
     } else {
+        if (FRESH && !LAZY) prepare_q();               // (every wavefront for itself)
+        if (adds_fresh && !LAZY) add_fresh();
         for (int r = r_begin + wave; r <= r_end; r += WAVES) one_round(r, []() {});
     }
     if (adds_fresh && LAZY) add_fresh();
@@ -950,7 +991,8 @@ static int launch_decode_heads(const void* q, int ldq, const void* k_pool, const
                                int group, int page_tokens, int page_shift, int n_layers, int layer,
                                float scale, int window, const DecodeFresh& fresh, hipStream_t stream) {
     const int chunks = (group + 15) / 16;
-    const size_t lds = static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
+    // (the wavefronts' partial results, and the prepared q that one of them leaves for the others)
+    const size_t lds = static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float) + (fresh.k ? HD / 32 * 1024 : 0);
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, false, false>),
@@ -978,7 +1020,7 @@ static int launch_decode_parts(const void* q, int ldq, const void* k_pool, const
                                int page_shift, int n_layers, int layer, float scale, int window,
                                int split_rounds, int n_parts, const DecodeFresh& fresh, hipStream_t stream) {
     const int chunks = (group + 15) / 16;
-    const size_t lds = WAVES == 1 ? 0 : static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float);
+    const size_t lds = WAVES == 1 ? 0 : static_cast<size_t>(WAVES) * min(group, 16) * (HD + 2) * sizeof(float) + (fresh.k ? HD / 32 * 1024 : 0);
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_decode_heads_kernel<HD, WAVES, true, false>),
