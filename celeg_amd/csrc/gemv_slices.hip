@@ -272,6 +272,11 @@ static int launch_slices(const GemvParams& params, int chunks_per_wave, int cols
     else if (chunks_per_wave <= 4 || NS > 1)
         hipLaunchKernelGGL((gemv_slices_kernel<G, KW, 4, 1, EPI>), grid, block, 0, stream, p.a, p.w, p.rows, p.M, p.N, p.K, cols, p.lda, p.stream_rows,
                            static_cast<int>(p.w_row_stride), static_cast<int>(p.w_kb_stride), p);
+    else if (NS == 1 && chunks_per_wave > 6 && chunks_per_wave <= 8)
+        // (a long K, 7,168 or 8,192 values over two halves and eight wavefronts: all of a wavefront's
+        // chunks in one trip to memory instead of six and then one or two)
+        hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 8), 1, EPI>), grid, block, 0, stream, p.a, p.w, p.rows, p.M, p.N, p.K, cols, p.lda, p.stream_rows,
+                           static_cast<int>(p.w_row_stride), static_cast<int>(p.w_kb_stride), p);
     else
         hipLaunchKernelGGL((gemv_slices_kernel<G, KW, (NS > 1 ? 4 : 6), 1, EPI>), grid, block, 0, stream, p.a, p.w, p.rows, p.M, p.N, p.K, cols, p.lda, p.stream_rows,
                            static_cast<int>(p.w_row_stride), static_cast<int>(p.w_kb_stride), p);
