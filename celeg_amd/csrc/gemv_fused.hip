@@ -204,10 +204,16 @@ __global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvPara
 #pragma unroll
         for (int s = 0; s < NS; ++s) acc[mt][s] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
+    // element (n, k) of w lies at n * w_row_stride + (k / 32) * w_kb_stride + k % 32: rows one after
+    // the other (K, 32), or [K/32, rows, 32] (32, rows * 32), where the 16 weight rows of a tile are
+    // a kilobyte in a row for every block of 32 values of k: an output head of 65,536 rows then
+    // reads whole kilobytes instead of 64 bytes of each of 16 rows that lie kilobytes apart (rows
+    // of 2,048 values, 8 rows of A: 54.6 against 62.4 us; rows of 1,024 values: no difference)
+    const size_t w_row_stride = static_cast<size_t>(p.w_row_stride), w_kb_stride = static_cast<size_t>(p.w_kb_stride);
     const bf16* wrow[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s)
-        wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(tile * 16 + c16, p.N - 1)) * K;
+        wrow[s] = p.w + (static_cast<size_t>(s) * p.stream_rows + min(tile * 16 + c16, p.N - 1)) * w_row_stride;
 
     // K is cut in chunks of 64 which are dealt to the KW wavefronts of a tile.  Inside a
     // chunk, lane group q holds the k values {q*8..q*8+7} and {32+q*8..32+q*8+7}: each of
@@ -230,7 +236,8 @@ __global__ __launch_bounds__(TW * KW * 64) void gemv_fused_kernel(const GemvPara
                 const bool in = c0 + u < c_end && k + 8 <= K;    // K % 8 == 0
 #pragma unroll
                 for (int s = 0; s < NS; ++s)
-                    wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + k) : Frag2{};
+                    // (8 values from k on never leave a block of 32)
+                    wv[u][s][v] = in ? *reinterpret_cast<const Frag2*>(wrow[s] + static_cast<size_t>(k >> 5) * w_kb_stride + (k & 31)) : Frag2{};
             }
     };
     // ---- rows of A: 1/rms (A_NORM), and the rows themselves into LDS (ALDS); one wavefront
@@ -468,6 +475,10 @@ extern "C" int celeg_gemv_fused(const GemvParams* params, int amode, int epi, in
     if (p.M <= 0 || p.N <= 0) return 0;
     if (p.M > 64 || p.K <= 0 || (p.K % 8) || (p.lda % 8)) return static_cast<int>(hipErrorInvalidValue);
     if (epi == E_CONV && (p.taps < 1 || p.taps > CONV_PREFETCH_TAPS || p.stream_rows != p.N))
+        return static_cast<int>(hipErrorInvalidValue);
+    // (the weights' layout: rows one after the other, or blocks of 32 values of k with the rows side by side)
+    if (p.w_row_stride <= 0 || p.w_kb_stride <= 0 || (p.w_row_stride % 8) || (p.w_kb_stride % 8) ||
+        (p.w_kb_stride != 32 && (p.K % 32)))
         return static_cast<int>(hipErrorInvalidValue);
     const int tiles = (p.N + 15) / 16, chunks = (p.K + 63) / 64;
     if (p.row_best && (epi != E_STORE_F32 || p.row_best_rows < p.M || p.row_best_ld < tiles)) return static_cast<int>(hipErrorInvalidValue);

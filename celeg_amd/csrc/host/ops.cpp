@@ -680,7 +680,7 @@ void Ops::fused_linear(const Tensor& a, const Tensor& w, const Tensor& out, cons
     if ((a.ndim == 3 || out.ndim == 3 || (args.out_bf16.defined() && args.out_bf16.ndim == 3)) && !streamed)
         throw KernelError("fused_linear: operands with the rows side by side go with the kernel for 9 to 64 rows");
     need(!(out.ndim == 3 && out_dtype != DType::BF16), "fused_linear: a 32-bit output has its rows one after the other");
-    need(!packed || sliced || streamed, "fused_linear: packed weights go with bfloat16 rows");
+    need(!packed || sliced || streamed || K % 32 == 0, "fused_linear: a packed weight has an inner size that is a multiple of 32");
     prm.w_row_stride = packed ? 32 : K;
     prm.w_kb_stride = packed ? w_rows * 32 : 32;
     if (args.out_bf16.defined()) {

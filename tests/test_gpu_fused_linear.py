@@ -471,3 +471,25 @@ def test_output_head_at_the_real_vocabulary(tmp_path, R, K):
     # the last columns and rows are there
     assert_close_bf16(got[-1:, -64:], ref[-1:, -64:], "head, last columns")
     lm.close()
+
+
+@pytest.mark.parametrize("M,N,K,epilogue", [(1, 4100, 64, "store_f32"), (8, 70000, 2048, "store_f32"), (16, 333, 96, "store"),
+                                            (5, 24, 160, "store_f32"), (8, 200, 128, "swiglu"), (33, 1000, 96, "store_f32")])
+def test_the_staged_kernel_reads_weights_in_blocks_of_32_as_it_reads_rows(ops, M, N, K, epilogue):
+    """The kernel that normalises the rows itself takes its weights with the rows one after the other
+    or as [K/32, rows, 32] (what a wide model's output head is copied to): the same products in
+    the same order, so the same bits."""
+    streams = 2 if epilogue == "swiglu" else 1
+    h = randn(M, K, seed=41)
+    nw = 1 + randn(K, seed=42, scale=0.1)
+    w = randn(streams * N, K, seed=43, scale=0.1, dtype=BF)
+    dtype = torch.float32 if epilogue == "store_f32" else BF
+    a = torch.empty(M, N, dtype=dtype, device=DEV)
+    b = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.fused_linear(h, w, a, epilogue=epilogue, norm_weight=nw, eps=1e-5)
+    ops.fused_linear(h, ops.pack_weight(w), b, epilogue=epilogue, norm_weight=nw, eps=1e-5)
+    assert torch.equal(a, b)
+    x = h * torch.rsqrt((h * h).mean(dim=1, keepdim=True) + 1e-5) * nw
+    y = x.to(BF).float() @ w.float().T
+    want = torch.nn.functional.silu(y[:, :N]) * y[:, N:] if streams == 2 else y
+    assert torch.allclose(a.float(), want, rtol=2e-2, atol=2e-2 * float(want.abs().max()))
